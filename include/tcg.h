@@ -1,0 +1,234 @@
+/*
+ * tcg.h -- C ABI of the MI355X (gfx950) evaluation backend for tenncor
+ * operator graphs.
+ *
+ * The tenncor reference has no FFI on this path: its seam is the C++ pair
+ * `egen::typed_exec<T>(opcode, out, outshape, in, attrib)` (generated from
+ * cfg/ops.yml:6 by tools/egen/plugins/opcodes.py:36-46), which builds one
+ * Eigen closure per graph node, and `eigen::Device::calc`
+ * (internal/eigen/device.hpp:546-576), which runs it into a buffer borrowed
+ * from `eigen::iRuntimeMemory` (internal/eigen/memory.hpp:14-22).  Every entry
+ * point below is what one `stmt` of cfg/ops.yml binds to once the Eigen
+ * closure is replaced by a stream-ordered GPU launch; the comment on each
+ * names the statement and the Eigen call site it replaces.
+ *
+ * Conventions
+ *   - all functions return 0 (TCG_OK) or a tcg_status; no C++ exception
+ *     crosses this boundary; tcg_last_error() gives the message
+ *   - shapes are uint64_t[8] in tenncor order: dim 0 is the fastest-varying
+ *     dim, unused dims are 1 (internal/teq/shape.hpp:56-59)
+ *   - dtype codes follow cfg/mintype.yml:4-13: 1 double, 2 float, 3 int32
+ *   - opcodes are the values of egen::_GENERATED_OPCODE, i.e. the key order
+ *     of cfg/ops.yml with BAD_OP = 0 (tools/egen/plugins/opcodes.py:16-22)
+ *   - data pointers are DEVICE pointers (from tcg_alloc, or any HIP device
+ *     allocation of the same device); element offsets into them are allowed
+ *     (the reference aliases last-dim slices by pointer offset,
+ *     internal/eigen/operator.hpp:231-248)
+ *   - every launch is ordered on the context's single stream; one host thread
+ *     per context (the reference evaluates single-threaded)
+ *   - the library never falls back to the CPU: if no gfx950 device is present
+ *     tcg_ctx_create fails
+ */
+#ifndef TCG_H
+#define TCG_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TCG_RANK_CAP 8
+
+typedef struct tcg_ctx tcg_ctx;
+
+enum tcg_status
+{
+	TCG_OK = 0,
+	TCG_ERR_ARG = 1,         /* argument the reference would reject at node construction */
+	TCG_ERR_HIP = 2,         /* a HIP runtime call failed */
+	TCG_ERR_UNSUPPORTED = 3, /* opcode/dtype combination not implemented on the device */
+	TCG_ERR_OOM = 4
+};
+
+enum tcg_dtype { TCG_BAD_TYPE = 0, TCG_DOUBLE = 1, TCG_FLOAT = 2, TCG_INT32 = 3 };
+
+enum tcg_opcode
+{
+	TCG_BAD_OP = 0, TCG_IDENTITY, TCG_ABS, TCG_NEG, TCG_SIN, TCG_COS, TCG_TAN,
+	TCG_EXP, TCG_LOG, TCG_SQRT, TCG_ROUND, TCG_SIGMOID, TCG_TANH, TCG_SQUARE,
+	TCG_CUBE, TCG_RAND_UNIF, TCG_REVERSE, TCG_REDUCE_SUM, TCG_REDUCE_PROD,
+	TCG_REDUCE_MIN, TCG_REDUCE_MAX, TCG_ARGMAX, TCG_PERMUTE, TCG_EXTEND,
+	TCG_RESHAPE, TCG_SLICE, TCG_PAD, TCG_STRIDE, TCG_SCATTER, TCG_POW, TCG_ADD,
+	TCG_SUB, TCG_MUL, TCG_DIV, TCG_MIN, TCG_MAX, TCG_EQ, TCG_NEQ, TCG_LT,
+	TCG_GT, TCG_MATMUL, TCG_CONTRACT, TCG_CONV, TCG_SELECT, TCG_CONCAT,
+	TCG_ASSIGN, TCG_ASSIGN_ADD, TCG_ASSIGN_SUB, TCG_ASSIGN_MUL, TCG_ASSIGN_DIV,
+	TCG_CAST, TCG_N_OPCODES
+};
+
+/* ---- context, memory, transfers -------------------------------------- */
+
+/* Replaces: constructing an eigen::Device (internal/eigen/device.hpp:546-553).
+ * Fails with TCG_ERR_HIP when no GPU is visible. */
+int tcg_ctx_create (int device, tcg_ctx** out);
+int tcg_ctx_destroy (tcg_ctx* ctx);
+/* Message of the last failing call on this context ("" if none). With a NULL
+ * context: the message of the last failing tcg_ctx_create of this thread. */
+const char* tcg_last_error (const tcg_ctx* ctx);
+/* Name of the device the context runs on, e.g. "gfx950" */
+const char* tcg_device_arch (const tcg_ctx* ctx);
+
+/* Replaces: eigen::iRuntimeMemory::allocate / deallocate
+ * (internal/eigen/memory.hpp:14-22), bytes not elements, deallocate receives
+ * the original size.  Blocks are recycled in stream order without touching
+ * hipMalloc/hipFree on the steady state; 256-byte aligned. */
+int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr);
+int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes);
+/* Bytes currently handed out / held by the pool (for leak checks in tests) */
+int tcg_mem_stats (const tcg_ctx* ctx, uint64_t* in_use, uint64_t* pooled);
+
+/* Replaces: the memcpy in eigen::SrcRef<T>::assign (internal/eigen/device.hpp:
+ * 200-247) and host reads through iDeviceRef::data()
+ * (internal/teq/itensor.hpp:22-35).  h2d: the host buffer may be reused as
+ * soon as the call returns.  d2h: blocks until the bytes are in `dst`. */
+int tcg_h2d (tcg_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);
+int tcg_d2h (tcg_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);
+int tcg_d2d (tcg_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
+int tcg_fill_zero (tcg_ctx* ctx, void* dst_dev, size_t bytes);
+int tcg_sync (tcg_ctx* ctx);
+
+/* Timing on the context's stream with HIP events (for benchmarks):
+ * begin records an event, end records a second one, waits for it and returns
+ * the milliseconds between them. */
+int tcg_timer_begin (tcg_ctx* ctx);
+int tcg_timer_end (tcg_ctx* ctx, float* ms);
+
+/* ---- elementwise ------------------------------------------------------ */
+
+/* ABS..CUBE: `out = eigen::abs<T>(outshape, *in[0])` ... `eigen::cube<T>`
+ * (cfg/ops.yml:75-100; internal/eigen/operator.hpp:377-659) */
+int tcg_ew_unary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
+	const void* in, void* out);
+
+/* POW, SUB, DIV, MIN, MAX, EQ, NEQ, LT, GT and two-argument ADD/MUL
+ * (cfg/ops.yml:453-493; internal/eigen/operator.hpp:665-987) */
+int tcg_ew_binary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
+	const void* a, const void* b, void* out);
+
+/* ADD / MUL over nargs >= 2 operands, folded left to right
+ * (`eigen::add<T>(outshape, in)`, internal/eigen/operator.hpp:694-732,757-795) */
+int tcg_ew_nary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
+	const void* const* ins, void* out);
+
+/* SELECT (cfg/ops.yml:608-609; internal/eigen/operator.hpp:1050-1067) */
+int tcg_ew_select (tcg_ctx* ctx, int dtype, uint64_t n, const void* cond,
+	const void* then, const void* otherwise, void* out);
+
+/* CAST (cfg/ops.yml:681-711; internal/eigen/operator.hpp:1239-1260) */
+int tcg_cast (tcg_ctx* ctx, int out_dtype, int in_dtype, uint64_t n,
+	const void* in, void* out);
+
+/* ASSIGN, ASSIGN_ADD/SUB/MUL/DIV: target (op)= source in place
+ * (cfg/ops.yml:654-680; internal/eigen/operator.hpp:1190-1237) */
+int tcg_assign (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
+	void* target, const void* source);
+
+/* A chain of elementwise nodes evaluated in one pass over memory: what a run
+ * of consecutive MatOp/TensOp closures (internal/eigen/device.hpp:304-372)
+ * computes, without materialising the intermediates.
+ * Three registers (ACC, T0, T1); operands name a register, a leaf or the
+ * instruction's immediate. */
+enum tcg_ew_operand
+{
+	TCG_OPD_NONE = 0, TCG_OPD_ACC = 1, TCG_OPD_T0 = 2, TCG_OPD_T1 = 3,
+	TCG_OPD_IMM = 4,
+	TCG_OPD_LEAF0 = 8 /* TCG_OPD_LEAF0 + k = leaf k, k < TCG_EW_MAX_LEAVES */
+};
+#define TCG_EW_MAX_LEAVES 4
+#define TCG_EW_MAX_INSTRS 32
+typedef struct tcg_ew_instr
+{
+	uint8_t opcode; /* unary or binary tcg_opcode; TCG_IDENTITY copies `a` */
+	uint8_t a;      /* tcg_ew_operand */
+	uint8_t b;      /* tcg_ew_operand, TCG_OPD_NONE for unary opcodes */
+	uint8_t dst;    /* TCG_OPD_ACC, TCG_OPD_T0 or TCG_OPD_T1 */
+	uint32_t pad_;
+	double imm;     /* converted to the kernel's dtype */
+} tcg_ew_instr;
+/* The value of ACC after the last instruction is written to out. */
+int tcg_ew_fused (tcg_ctx* ctx, int dtype, uint64_t n, int nleaves,
+	const void* const* leaves, int ninstrs, const tcg_ew_instr* program, void* out);
+
+/* ---- reductions ------------------------------------------------------- */
+
+/* REDUCE_SUM / REDUCE_PROD / REDUCE_MIN / REDUCE_MAX
+ * (`eigen::reduce_sum<T>(outshape, *in[0], attrib)`, cfg/ops.yml:106-151;
+ * internal/eigen/operator.hpp:54-132).  Bit i of rankmask = dim i reduced. */
+int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
+	unsigned rankmask, const void* in, void* out);
+
+/* ARGMAX (cfg/ops.yml:152-186; internal/eigen/operator.hpp:134-155);
+ * return_dim >= 8 gives the flat index of the maximum */
+int tcg_argmax (tcg_ctx* ctx, int dtype, const uint64_t shape[8], int return_dim,
+	const void* in, void* out);
+
+/* ---- data movement ---------------------------------------------------- */
+
+/* EXTEND (cfg/ops.yml:239-283; internal/eigen/operator.hpp:157-173) */
+int tcg_extend (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t bcast[8], const void* in, void* out);
+/* PERMUTE (cfg/ops.yml:187-238; internal/eigen/operator.hpp:175-210);
+ * `order` is the completed 8-entry permutation: out dim i = in dim order[i] */
+int tcg_permute (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t order[8], const void* in, void* out);
+/* SLICE (cfg/ops.yml:319-371; internal/eigen/operator.hpp:212-255);
+ * offsets/extents are the clamped values of lines 225-230 */
+int tcg_slice (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t offsets[8], const uint64_t extents[8], const void* in, void* out);
+/* PAD (cfg/ops.yml:372-412; internal/eigen/operator.hpp:257-275) */
+int tcg_pad (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t before[8], const uint64_t after[8], const void* in, void* out);
+/* REVERSE (cfg/ops.yml:104-105; internal/eigen/operator.hpp:316-333) */
+int tcg_reverse (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
+	unsigned rankmask, const void* in, void* out);
+/* STRIDE (cfg/ops.yml:413-438; internal/eigen/operator.hpp:277-293) */
+int tcg_stride (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t incr[8], const uint64_t outshape[8], const void* in, void* out);
+/* SCATTER (cfg/ops.yml:439-452; internal/eigen/operator.hpp:295-314) */
+int tcg_scatter (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t incr[8], const uint64_t outshape[8], const void* in, void* out);
+/* CONCAT (cfg/ops.yml:610-653; internal/eigen/operator.hpp:335-368);
+ * shapes = nargs * 8 values */
+int tcg_concat (tcg_ctx* ctx, int dtype, int axis, int nargs,
+	const uint64_t* shapes, const void* const* ins, void* out);
+
+/* ---- contractions ----------------------------------------------------- */
+
+/* MATMUL (cfg/ops.yml:494-514; internal/eigen/operator.hpp:1107-1139):
+ * a{K,M,batch...}, b{N,K,batch...} -> out{N,M,batch...} */
+int tcg_matmul (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
+	const uint64_t bshape[8], const void* a, const void* b, void* out);
+/* CONTRACT (cfg/ops.yml:515-565; internal/eigen/operator.hpp:1069-1103);
+ * pairs = npairs * (a_dim, b_dim); out dims = b's free dims then a's */
+int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
+	const uint64_t bshape[8], int npairs, const uint64_t* pairs,
+	const void* a, const void* b, void* out);
+/* Strided row-major GEMM the two above lower to:
+ * C[b][m][n] = sum_k A[b][m][k] * B[b][k][n], element strides given;
+ * trans_a: A element (m,k) at m*1 + k*lda instead of m*lda + k, same for B */
+int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
+	uint64_t batch, const void* A, uint64_t lda, uint64_t stride_a, int trans_a,
+	const void* B, uint64_t ldb, uint64_t stride_b, int trans_b,
+	void* C, uint64_t ldc, uint64_t stride_c);
+/* CONV (cfg/ops.yml:566-607; internal/eigen/operator.hpp:1141-1187):
+ * valid cross-correlation, kernel dim i slides along image dim ranks[i] */
+int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const void* img, const void* kernel, void* out);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TCG_H */

@@ -1,0 +1,64 @@
+"""Builds the native libraries of this package in-tree.
+
+``python -m tenncor_amd.build`` compiles every ``csrc/*.hip`` for gfx950 into
+``tenncor_amd/libtcg.so``.  hipcc cross-compiles without a GPU.
+"""
+import glob
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIBTCG = os.path.join(PKG, "libtcg.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed fp32 forms are kept off on this pool
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_libtcg(jobs=8, verbose=False):
+    """Compile every csrc/*.hip to an object (in parallel) and link libtcg.so."""
+    from concurrent.futures import ThreadPoolExecutor
+    objdir = os.path.join(PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+    sources = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    if not sources:
+        raise RuntimeError("no HIP sources under %s" % CSRC)
+    objs = [os.path.join(objdir, os.path.basename(s)[:-4] + ".o") for s in sources]
+
+    def compile_one(pair):
+        src, obj = pair
+        out = _run([HIPCC] + HIP_FLAGS + ["-c", src, "-o", obj])
+        if verbose and out.strip():
+            print(out)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(compile_one, zip(sources, objs)))
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBTCG] + objs)
+    return LIBTCG
+
+
+def main():
+    path = build_libtcg(verbose=True)
+    print("built", path)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,340 @@
+"""ctypes binding of the C ABI in ``include/tcg.h`` (``libtcg.so``).
+
+Thin by design: one Python method per exported function, device buffers are
+plain integers (device addresses), shapes are tenncor shapes (dim 0 fastest).
+The library is loaded from the package folder; if it is missing this module
+raises -- there is no fallback path.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libtcg.so")
+
+RANK_CAP = 8
+DOUBLE, FLOAT, INT32 = 1, 2, 3
+NP_OF = {DOUBLE: np.float64, FLOAT: np.float32, INT32: np.int32}
+
+OPCODES = [
+    "BAD_OP", "IDENTITY", "ABS", "NEG", "SIN", "COS", "TAN", "EXP", "LOG", "SQRT", "ROUND",
+    "SIGMOID", "TANH", "SQUARE", "CUBE", "RAND_UNIF", "REVERSE", "REDUCE_SUM", "REDUCE_PROD",
+    "REDUCE_MIN", "REDUCE_MAX", "ARGMAX", "PERMUTE", "EXTEND", "RESHAPE", "SLICE", "PAD",
+    "STRIDE", "SCATTER", "POW", "ADD", "SUB", "MUL", "DIV", "MIN", "MAX", "EQ", "NEQ", "LT",
+    "GT", "MATMUL", "CONTRACT", "CONV", "SELECT", "CONCAT", "ASSIGN", "ASSIGN_ADD",
+    "ASSIGN_SUB", "ASSIGN_MUL", "ASSIGN_DIV", "CAST",
+]
+OP = {name: i for i, name in enumerate(OPCODES)}
+
+OPD_NONE, OPD_ACC, OPD_T0, OPD_T1, OPD_IMM, OPD_LEAF0 = 0, 1, 2, 3, 4, 8
+
+# every symbol include/tcg.h declares
+EXPORTS = [
+    "tcg_ctx_create", "tcg_ctx_destroy", "tcg_last_error", "tcg_device_arch", "tcg_alloc", "tcg_free",
+    "tcg_mem_stats", "tcg_h2d", "tcg_d2h", "tcg_d2d", "tcg_fill_zero", "tcg_sync", "tcg_timer_begin",
+    "tcg_timer_end", "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
+    "tcg_assign", "tcg_ew_fused", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
+    "tcg_pad", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
+    "tcg_gemm", "tcg_conv",
+]
+
+
+class TcgError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("tcg status %d: %s" % (status, message))
+        self.status = status
+
+
+class EwInstr(ctypes.Structure):
+    _fields_ = [("opcode", ctypes.c_uint8), ("a", ctypes.c_uint8), ("b", ctypes.c_uint8),
+                ("dst", ctypes.c_uint8), ("pad_", ctypes.c_uint32), ("imm", ctypes.c_double)]
+
+
+_lib = None
+
+
+def load():
+    """Load libtcg.so and declare the argument types of every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("%s is missing: build it with `python -m tenncor_amd.build` "
+                          "(there is no CPU fallback)" % LIB_PATH)
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, u64, i32, sz = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int, ctypes.c_size_t
+    u64p, vpp = ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_void_p)
+    sig = {
+        "tcg_ctx_create": [i32, ctypes.POINTER(vp)],
+        "tcg_ctx_destroy": [vp],
+        "tcg_alloc": [vp, sz, ctypes.POINTER(vp)],
+        "tcg_free": [vp, vp, sz],
+        "tcg_mem_stats": [vp, u64p, u64p],
+        "tcg_h2d": [vp, vp, vp, sz],
+        "tcg_d2h": [vp, vp, vp, sz],
+        "tcg_d2d": [vp, vp, vp, sz],
+        "tcg_fill_zero": [vp, vp, sz],
+        "tcg_sync": [vp],
+        "tcg_timer_begin": [vp],
+        "tcg_timer_end": [vp, ctypes.POINTER(ctypes.c_float)],
+        "tcg_ew_unary": [vp, i32, i32, u64, vp, vp],
+        "tcg_ew_binary": [vp, i32, i32, u64, vp, vp, vp],
+        "tcg_ew_nary": [vp, i32, i32, u64, i32, vpp, vp],
+        "tcg_ew_select": [vp, i32, u64, vp, vp, vp, vp],
+        "tcg_cast": [vp, i32, i32, u64, vp, vp],
+        "tcg_assign": [vp, i32, i32, u64, vp, vp],
+        "tcg_ew_fused": [vp, i32, u64, i32, vpp, i32, ctypes.POINTER(EwInstr), vp],
+        "tcg_reduce": [vp, i32, i32, u64p, ctypes.c_uint, vp, vp],
+        "tcg_argmax": [vp, i32, u64p, i32, vp, vp],
+        "tcg_extend": [vp, i32, u64p, u64p, vp, vp],
+        "tcg_permute": [vp, i32, u64p, u64p, vp, vp],
+        "tcg_slice": [vp, i32, u64p, u64p, u64p, vp, vp],
+        "tcg_pad": [vp, i32, u64p, u64p, u64p, vp, vp],
+        "tcg_reverse": [vp, i32, u64p, ctypes.c_uint, vp, vp],
+        "tcg_stride": [vp, i32, u64p, u64p, u64p, vp, vp],
+        "tcg_scatter": [vp, i32, u64p, u64p, u64p, vp, vp],
+        "tcg_concat": [vp, i32, i32, i32, u64p, vpp, vp],
+        "tcg_matmul": [vp, i32, u64p, u64p, vp, vp, vp],
+        "tcg_contract": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
+        "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
+        "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
+    }
+    for name, argtypes in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+    lib.tcg_last_error.argtypes = [vp]
+    lib.tcg_last_error.restype = ctypes.c_char_p
+    lib.tcg_device_arch.argtypes = [vp]
+    lib.tcg_device_arch.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def shape8(shape, fill=1):
+    s = [int(d) for d in shape] + [fill] * (RANK_CAP - len(shape))
+    return s[:RANK_CAP]
+
+
+def n_elems(shape):
+    n = 1
+    for d in shape8(shape):
+        n *= d
+    return n
+
+
+def _u64(vals):
+    return (ctypes.c_uint64 * len(vals))(*[int(v) for v in vals])
+
+
+def _mask(ranks):
+    m = 0
+    for r in ranks:
+        m |= 1 << int(r)
+    return m
+
+
+def dtype_code(np_dtype):
+    t = np.dtype(np_dtype)
+    for code, npt in NP_OF.items():
+        if t == npt:
+            return code
+    raise TypeError("unsupported dtype %s" % t)
+
+
+def _opcode(op):
+    return OP[op] if isinstance(op, str) else int(op)
+
+
+class Context:
+    """One device context (tcg_ctx): a stream, a memory pool, the launches."""
+
+    def __init__(self, device=0):
+        self.lib = load()
+        handle = ctypes.c_void_p()
+        rc = self.lib.tcg_ctx_create(device, ctypes.byref(handle))
+        if rc != 0:
+            raise TcgError(rc, self.lib.tcg_last_error(None).decode())
+        self.handle = handle
+
+    def close(self):
+        if self.handle:
+            self.lib.tcg_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def _check(self, rc):
+        if rc != 0:
+            raise TcgError(rc, self.lib.tcg_last_error(self.handle).decode())
+
+    @property
+    def arch(self):
+        return self.lib.tcg_device_arch(self.handle).decode()
+
+    # ---- memory ----
+    def alloc(self, nbytes):
+        p = ctypes.c_void_p()
+        self._check(self.lib.tcg_alloc(self.handle, nbytes, ctypes.byref(p)))
+        return p.value
+
+    def free(self, ptr, nbytes):
+        self._check(self.lib.tcg_free(self.handle, ptr, nbytes))
+
+    def mem_stats(self):
+        a, b = ctypes.c_uint64(), ctypes.c_uint64()
+        self._check(self.lib.tcg_mem_stats(self.handle, ctypes.byref(a), ctypes.byref(b)))
+        return a.value, b.value
+
+    def h2d(self, dst, host):
+        host = np.ascontiguousarray(host)
+        self._check(self.lib.tcg_h2d(self.handle, dst, host.ctypes.data, host.nbytes))
+
+    def d2h(self, src, n, np_dtype):
+        out = np.empty(int(n), dtype=np_dtype)
+        self._check(self.lib.tcg_d2h(self.handle, out.ctypes.data, src, out.nbytes))
+        return out
+
+    def d2d(self, dst, src, nbytes):
+        self._check(self.lib.tcg_d2d(self.handle, dst, src, nbytes))
+
+    def fill_zero(self, dst, nbytes):
+        self._check(self.lib.tcg_fill_zero(self.handle, dst, nbytes))
+
+    def upload(self, host):
+        """Allocate a device buffer holding ``host`` (flattened); returns a DevBuf."""
+        host = np.ascontiguousarray(host).reshape(-1)
+        buf = DevBuf(self, host.size, host.dtype)
+        self.h2d(buf.ptr, host)
+        return buf
+
+    def empty(self, n, np_dtype):
+        return DevBuf(self, n, np_dtype)
+
+    def sync(self):
+        self._check(self.lib.tcg_sync(self.handle))
+
+    def timer_begin(self):
+        self._check(self.lib.tcg_timer_begin(self.handle))
+
+    def timer_end(self):
+        ms = ctypes.c_float()
+        self._check(self.lib.tcg_timer_end(self.handle, ctypes.byref(ms)))
+        return ms.value
+
+    # ---- elementwise ----
+    def ew_unary(self, op, dtype, n, src, dst):
+        self._check(self.lib.tcg_ew_unary(self.handle, _opcode(op), dtype, n, src, dst))
+
+    def ew_binary(self, op, dtype, n, a, b, dst):
+        self._check(self.lib.tcg_ew_binary(self.handle, _opcode(op), dtype, n, a, b, dst))
+
+    def ew_nary(self, op, dtype, n, srcs, dst):
+        ptrs = (ctypes.c_void_p * len(srcs))(*srcs)
+        self._check(self.lib.tcg_ew_nary(self.handle, _opcode(op), dtype, n, len(srcs), ptrs, dst))
+
+    def ew_select(self, dtype, n, cond, then, otherwise, dst):
+        self._check(self.lib.tcg_ew_select(self.handle, dtype, n, cond, then, otherwise, dst))
+
+    def cast(self, out_dtype, in_dtype, n, src, dst):
+        self._check(self.lib.tcg_cast(self.handle, out_dtype, in_dtype, n, src, dst))
+
+    def assign(self, op, dtype, n, target, source):
+        self._check(self.lib.tcg_assign(self.handle, _opcode(op), dtype, n, target, source))
+
+    def ew_fused(self, dtype, n, leaves, program, dst):
+        """program: list of (opcode, a, b, dst[, imm])."""
+        instrs = (EwInstr * len(program))()
+        for i, ins in enumerate(program):
+            instrs[i].opcode = _opcode(ins[0])
+            instrs[i].a, instrs[i].b, instrs[i].dst = ins[1], ins[2], ins[3]
+            instrs[i].imm = float(ins[4]) if len(ins) > 4 else 0.0
+        ptrs = (ctypes.c_void_p * len(leaves))(*leaves)
+        self._check(self.lib.tcg_ew_fused(self.handle, dtype, n, len(leaves), ptrs, len(program), instrs, dst))
+
+    # ---- reductions ----
+    def reduce(self, op, dtype, shape, rank_set, src, dst):
+        self._check(self.lib.tcg_reduce(self.handle, _opcode(op), dtype, _u64(shape8(shape)), _mask(rank_set), src, dst))
+
+    def argmax(self, dtype, shape, return_dim, src, dst):
+        self._check(self.lib.tcg_argmax(self.handle, dtype, _u64(shape8(shape)), int(return_dim), src, dst))
+
+    # ---- data movement ----
+    def extend(self, dtype, inshape, bcast, src, dst):
+        self._check(self.lib.tcg_extend(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(bcast)), src, dst))
+
+    def permute(self, dtype, inshape, order8, src, dst):
+        self._check(self.lib.tcg_permute(self.handle, dtype, _u64(shape8(inshape)), _u64(order8), src, dst))
+
+    def slice(self, dtype, inshape, offsets, extents, src, dst):
+        self._check(self.lib.tcg_slice(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(offsets, 0)),
+                                       _u64(shape8(extents)), src, dst))
+
+    def pad(self, dtype, inshape, before, after, src, dst):
+        self._check(self.lib.tcg_pad(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(before, 0)),
+                                     _u64(shape8(after, 0)), src, dst))
+
+    def reverse(self, dtype, shape, rank_set, src, dst):
+        self._check(self.lib.tcg_reverse(self.handle, dtype, _u64(shape8(shape)), _mask(rank_set), src, dst))
+
+    def stride(self, dtype, inshape, incr, outshape, src, dst):
+        self._check(self.lib.tcg_stride(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(incr)),
+                                        _u64(shape8(outshape)), src, dst))
+
+    def scatter(self, dtype, inshape, incr, outshape, src, dst):
+        self._check(self.lib.tcg_scatter(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(incr)),
+                                         _u64(shape8(outshape)), src, dst))
+
+    def concat(self, dtype, axis, shapes, srcs, dst):
+        flat = [d for s in shapes for d in shape8(s)]
+        ptrs = (ctypes.c_void_p * len(srcs))(*srcs)
+        self._check(self.lib.tcg_concat(self.handle, dtype, int(axis), len(srcs), _u64(flat), ptrs, dst))
+
+    # ---- contractions ----
+    def matmul(self, dtype, ashape, bshape, a, b, dst):
+        self._check(self.lib.tcg_matmul(self.handle, dtype, _u64(shape8(ashape)), _u64(shape8(bshape)), a, b, dst))
+
+    def contract(self, dtype, ashape, bshape, pairs, a, b, dst):
+        flat = [int(v) for p in pairs for v in p]
+        self._check(self.lib.tcg_contract(self.handle, dtype, _u64(shape8(ashape)), _u64(shape8(bshape)),
+                                          len(pairs), _u64(flat), a, b, dst))
+
+    def gemm(self, dtype, M, N, K, batch, A, lda, stride_a, trans_a, B, ldb, stride_b, trans_b, C, ldc, stride_c):
+        self._check(self.lib.tcg_gemm(self.handle, dtype, M, N, K, batch, A, lda, stride_a, int(trans_a),
+                                      B, ldb, stride_b, int(trans_b), C, ldc, stride_c))
+
+    def conv(self, dtype, imgshape, kshape, ranks, img, kernel, dst):
+        r = [int(v) for v in ranks][:RANK_CAP]
+        self._check(self.lib.tcg_conv(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
+                                      len(r), _u64(r if r else [0]), img, kernel, dst))
+
+
+class DevBuf:
+    """A device buffer from the context's pool, returned to it on release."""
+
+    def __init__(self, ctx, n, np_dtype):
+        self.ctx = ctx
+        self.n = int(n)
+        self.np_dtype = np.dtype(np_dtype)
+        self.dtype = dtype_code(np_dtype)
+        self.nbytes = max(self.n, 1) * self.np_dtype.itemsize
+        self.ptr = ctx.alloc(self.nbytes)
+
+    def get(self):
+        return self.ctx.d2h(self.ptr, self.n, self.np_dtype)
+
+    def release(self):
+        if self.ptr is not None and self.ctx.handle:
+            self.ctx.free(self.ptr, self.nbytes)
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.release()
+        except Exception:
+            pass

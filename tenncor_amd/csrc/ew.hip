@@ -1,0 +1,707 @@
+// Elementwise kernels: unary, binary, n-ary, select, cast, in-place assign and
+// the fused chain interpreter.  All of them stream memory once with 128-bit
+// accesses per lane and are bound by HBM bandwidth.
+#include "tcg_internal.hpp"
+
+namespace
+{
+
+// ---- scalar semantics (internal/eigen/operator.hpp:377-987) --------------
+
+template <typename T> struct is_int { static constexpr bool value = false; };
+template <> struct is_int<int32_t> { static constexpr bool value = true; };
+
+template <typename T>
+__device__ __forceinline__ T wrap_add (T a, T b)
+{
+	if constexpr (is_int<T>::value) { return (T) ((uint32_t) a + (uint32_t) b); }
+	else { return a + b; }
+}
+
+template <typename T>
+__device__ __forceinline__ T wrap_sub (T a, T b)
+{
+	if constexpr (is_int<T>::value) { return (T) ((uint32_t) a - (uint32_t) b); }
+	else { return a - b; }
+}
+
+template <typename T>
+__device__ __forceinline__ T wrap_mul (T a, T b)
+{
+	if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b); }
+	else { return a * b; }
+}
+
+template <typename T>
+__device__ __forceinline__ T safe_div (T a, T b)
+{
+	if constexpr (is_int<T>::value)
+	{
+		// the CPU traps on these two; the device returns 0 instead
+		if (b == 0 || (a == INT32_MIN && b == -1)) { return 0; }
+		return a / b;
+	}
+	else { return a / b; }
+}
+
+// (int) std::pow(a, b) of the CPU path is exact whenever the power is an
+// integer that a double holds; the device pow() is not correctly rounded, so
+// integer powers are computed by squaring (wrapping like the other int ops)
+__device__ __forceinline__ int32_t int_pow (int32_t a, int32_t b)
+{
+	if (b < 0)
+	{
+		// |a| > 1: the fraction truncates to 0; a == 0 divides by zero on the CPU
+		if (a == 1) { return 1; }
+		if (a == -1) { return (b & 1) ? -1 : 1; }
+		return 0;
+	}
+	uint32_t base = (uint32_t) a, r = 1;
+	uint32_t e = (uint32_t) b;
+	while (e)
+	{
+		if (e & 1) { r *= base; }
+		base *= base;
+		e >>= 1;
+	}
+	return (int32_t) r;
+}
+
+// float: single-precision library routines (<= 1-2 ulp, far inside the 1e-5
+// budget); int32: through double and truncated, like std::sin(int) on the CPU
+template <typename T>
+__device__ __forceinline__ T apply_unary (int op, T x)
+{
+	switch (op)
+	{
+		case TCG_IDENTITY: return x;
+		case TCG_ABS:
+			if constexpr (is_int<T>::value) { return x < 0 ? (T) (0u - (uint32_t) x) : x; }
+			else if constexpr (sizeof(T) == 4) { return fabsf(x); }
+			else { return fabs(x); }
+		case TCG_NEG:
+			if constexpr (is_int<T>::value) { return (T) (0u - (uint32_t) x); }
+			else { return -x; }
+		case TCG_SIN:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return sinf(x); }
+			else { return (T) sin((double) x); }
+		case TCG_COS:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return cosf(x); }
+			else { return (T) cos((double) x); }
+		case TCG_TAN:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return tanf(x); }
+			else { return (T) tan((double) x); }
+		case TCG_EXP:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return expf(x); }
+			else { return (T) exp((double) x); }
+		case TCG_LOG:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return logf(x); }
+			else { return (T) log((double) x); }
+		case TCG_SQRT:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return sqrtf(x); }
+			else { return (T) sqrt((double) x); }
+		case TCG_ROUND:
+			if constexpr (is_int<T>::value) { return x; }
+			else if constexpr (sizeof(T) == 4) { return roundf(x); }
+			else { return round(x); }
+		case TCG_SIGMOID:
+			if constexpr (is_int<T>::value)
+			{
+				T e = (T) exp(-(double) x);
+				T d = (T) (1u + (uint32_t) e);
+				return d == 0 ? 0 : (T) (1 / d);
+			}
+			else if constexpr (sizeof(T) == 4) { return 1.0f / (1.0f + expf(-x)); }
+			else { return 1.0 / (1.0 + exp(-x)); }
+		case TCG_TANH:
+			if constexpr (sizeof(T) == 4 && !is_int<T>::value) { return tanhf(x); }
+			else { return (T) tanh((double) x); }
+		case TCG_SQUARE: return wrap_mul(x, x);
+		case TCG_CUBE: return wrap_mul(wrap_mul(x, x), x);
+		default: return x;
+	}
+}
+
+template <typename T>
+__device__ __forceinline__ T apply_binary (int op, T a, T b)
+{
+	switch (op)
+	{
+		case TCG_POW:
+			if constexpr (is_int<T>::value) { return int_pow(a, b); }
+			else if constexpr (sizeof(T) == 4) { return powf(a, b); }
+			else { return pow(a, b); }
+		case TCG_ADD: return wrap_add(a, b);
+		case TCG_SUB: return wrap_sub(a, b);
+		case TCG_MUL: return wrap_mul(a, b);
+		case TCG_DIV: return safe_div(a, b);
+		case TCG_MIN: return a < b ? a : b;
+		case TCG_MAX: return a > b ? a : b;
+		case TCG_EQ: return (T) (a == b);
+		case TCG_NEQ: return (T) (a != b);
+		case TCG_LT: return (T) (a < b);
+		case TCG_GT: return (T) (a > b);
+		default: return a;
+	}
+}
+
+bool is_unary_op (int op)
+{
+	return op >= TCG_ABS && op <= TCG_CUBE;
+}
+
+bool is_binary_op (int op)
+{
+	return op >= TCG_POW && op <= TCG_GT;
+}
+
+// ---- streaming kernels ---------------------------------------------------
+
+constexpr int EW_BLOCK = 256;
+constexpr int EW_UNROLL = 4;
+
+template <typename T>
+__device__ __forceinline__ typename Vec16<T>::type ldv (const T* p, uint64_t vidx)
+{
+	return __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(p) + vidx);
+}
+
+template <typename T>
+__device__ __forceinline__ void stv (T* p, uint64_t vidx, typename Vec16<T>::type v)
+{
+	__builtin_nontemporal_store(v, reinterpret_cast<typename Vec16<T>::type*>(p) + vidx);
+}
+
+// OP is a compile-time constant so that the switch in apply_* folds away
+template <typename T, int OP>
+__global__ __launch_bounds__(EW_BLOCK) void ew_unary_vec_k (
+	const T* __restrict__ in, T* __restrict__ out, uint64_t n)
+{
+	constexpr int N = Vec16<T>::N;
+	const uint64_t nvec = n / N;
+	const uint64_t tile = (uint64_t) EW_BLOCK * EW_UNROLL;
+	for (uint64_t base = (uint64_t) blockIdx.x * tile; base < nvec; base += (uint64_t) gridDim.x * tile)
+	{
+		VecU<T> r[EW_UNROLL];
+#pragma unroll
+		for (int u = 0; u < EW_UNROLL; ++u)
+		{
+			uint64_t idx = base + (uint64_t) u * EW_BLOCK + threadIdx.x;
+			if (idx < nvec) { r[u].v = ldv(in, idx); }
+		}
+#pragma unroll
+		for (int u = 0; u < EW_UNROLL; ++u)
+		{
+			uint64_t idx = base + (uint64_t) u * EW_BLOCK + threadIdx.x;
+			if (idx < nvec)
+			{
+#pragma unroll
+				for (int e = 0; e < N; ++e) { r[u].e[e] = apply_unary<T>(OP, r[u].e[e]); }
+				stv(out, idx, r[u].v);
+			}
+		}
+	}
+	if (blockIdx.x == 0)
+	{
+		uint64_t i = nvec * N + threadIdx.x;
+		if (i < n) { out[i] = apply_unary<T>(OP, in[i]); }
+	}
+}
+
+template <typename T, int OP>
+__global__ __launch_bounds__(EW_BLOCK) void ew_binary_vec_k (
+	const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out, uint64_t n)
+{
+	constexpr int N = Vec16<T>::N;
+	const uint64_t nvec = n / N;
+	const uint64_t tile = (uint64_t) EW_BLOCK * EW_UNROLL;
+	for (uint64_t base = (uint64_t) blockIdx.x * tile; base < nvec; base += (uint64_t) gridDim.x * tile)
+	{
+		VecU<T> ra[EW_UNROLL], rb[EW_UNROLL];
+#pragma unroll
+		for (int u = 0; u < EW_UNROLL; ++u)
+		{
+			uint64_t idx = base + (uint64_t) u * EW_BLOCK + threadIdx.x;
+			if (idx < nvec)
+			{
+				ra[u].v = ldv(a, idx);
+				rb[u].v = ldv(b, idx);
+			}
+		}
+#pragma unroll
+		for (int u = 0; u < EW_UNROLL; ++u)
+		{
+			uint64_t idx = base + (uint64_t) u * EW_BLOCK + threadIdx.x;
+			if (idx < nvec)
+			{
+#pragma unroll
+				for (int e = 0; e < N; ++e) { ra[u].e[e] = apply_binary<T>(OP, ra[u].e[e], rb[u].e[e]); }
+				stv(out, idx, ra[u].v);
+			}
+		}
+	}
+	if (blockIdx.x == 0)
+	{
+		uint64_t i = nvec * N + threadIdx.x;
+		if (i < n) { out[i] = apply_binary<T>(OP, a[i], b[i]); }
+	}
+}
+
+// fallbacks for pointers that are not 16-byte aligned (aliased slices)
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void ew_unary_scalar_k (int op, const T* in, T* out, uint64_t n)
+{
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < n; i += step) { out[i] = apply_unary<T>(op, in[i]); }
+}
+
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void ew_binary_scalar_k (int op, const T* a, const T* b, T* out, uint64_t n)
+{
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < n; i += step) { out[i] = apply_binary<T>(op, a[i], b[i]); }
+}
+
+constexpr int NARY_MAX = 8;
+template <typename T>
+struct NaryArgs
+{
+	const T* in[NARY_MAX];
+	int nargs;
+};
+
+// out = in0 (op) in1 (op) ... folded left to right, one pass over memory
+template <typename T, bool VEC>
+__global__ __launch_bounds__(EW_BLOCK) void ew_nary_k (int op, NaryArgs<T> args, T* __restrict__ out, uint64_t n)
+{
+	constexpr int N = VEC ? Vec16<T>::N : 1;
+	const uint64_t nvec = n / N;
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	const uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < nvec; i += step)
+	{
+		if constexpr (VEC)
+		{
+			VecU<T> acc, x;
+			acc.v = ldv(args.in[0], i);
+			for (int j = 1; j < args.nargs; ++j)
+			{
+				x.v = ldv(args.in[j], i);
+#pragma unroll
+				for (int e = 0; e < N; ++e) { acc.e[e] = apply_binary<T>(op, acc.e[e], x.e[e]); }
+			}
+			stv(out, i, acc.v);
+		}
+		else
+		{
+			T acc = args.in[0][i];
+			for (int j = 1; j < args.nargs; ++j) { acc = apply_binary<T>(op, acc, args.in[j][i]); }
+			out[i] = acc;
+		}
+	}
+	if (VEC && blockIdx.x == 0)
+	{
+		uint64_t t = nvec * N + threadIdx.x;
+		if (t < n)
+		{
+			T acc = args.in[0][t];
+			for (int j = 1; j < args.nargs; ++j) { acc = apply_binary<T>(op, acc, args.in[j][t]); }
+			out[t] = acc;
+		}
+	}
+}
+
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void ew_select_k (const T* c, const T* a, const T* b, T* out, uint64_t n)
+{
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < n; i += step) { out[i] = c[i] != 0 ? a[i] : b[i]; }
+}
+
+template <typename TO, typename TI>
+__global__ __launch_bounds__(EW_BLOCK) void ew_cast_k (const TI* in, TO* out, uint64_t n)
+{
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < n; i += step) { out[i] = static_cast<TO>(in[i]); }
+}
+
+template <typename T>
+__global__ __launch_bounds__(EW_BLOCK) void ew_assign_k (int op, T* target, const T* source, uint64_t n)
+{
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < n; i += step)
+	{
+		T t = target[i], s = source[i];
+		switch (op)
+		{
+			case TCG_ASSIGN: t = s; break;
+			case TCG_ASSIGN_ADD: t = wrap_add(t, s); break;
+			case TCG_ASSIGN_SUB: t = wrap_sub(t, s); break;
+			case TCG_ASSIGN_MUL: t = wrap_mul(t, s); break;
+			case TCG_ASSIGN_DIV: t = safe_div(t, s); break;
+		}
+		target[i] = t;
+	}
+}
+
+// ---- fused chain interpreter ---------------------------------------------
+
+struct FusedProgram
+{
+	int ninstrs;
+	uint8_t opcode[TCG_EW_MAX_INSTRS];
+	uint8_t a[TCG_EW_MAX_INSTRS];
+	uint8_t b[TCG_EW_MAX_INSTRS];
+	uint8_t dst[TCG_EW_MAX_INSTRS];
+	double imm[TCG_EW_MAX_INSTRS];
+};
+
+template <typename T, int NLEAF>
+struct FusedLeaves
+{
+	const T* p[NLEAF];
+};
+
+// Every index below is a compile-time constant or a wave-uniform value taken
+// from kernel arguments, so registers are never indexed dynamically and the
+// dispatch costs scalar branches only.
+template <typename T, int NLEAF, int N>
+__device__ __forceinline__ void fused_eval (const FusedProgram& prog,
+	const T (&leaf)[NLEAF][N], T (&acc)[N])
+{
+	T t0[N], t1[N];
+#pragma unroll
+	for (int e = 0; e < N; ++e) { acc[e] = 0; t0[e] = 0; t1[e] = 0; }
+	for (int pc = 0; pc < prog.ninstrs; ++pc)
+	{
+		const int op = prog.opcode[pc];
+		const int ka = prog.a[pc], kb = prog.b[pc], kd = prog.dst[pc];
+		const T imm = (T) prog.imm[pc];
+		T r[N];
+#pragma unroll
+		for (int e = 0; e < N; ++e)
+		{
+			T va = ka == TCG_OPD_ACC ? acc[e] : ka == TCG_OPD_T0 ? t0[e] : ka == TCG_OPD_T1 ? t1[e] : imm;
+			T vb = kb == TCG_OPD_ACC ? acc[e] : kb == TCG_OPD_T0 ? t0[e] : kb == TCG_OPD_T1 ? t1[e] : imm;
+#pragma unroll
+			for (int k = 0; k < NLEAF; ++k)
+			{
+				if (ka == TCG_OPD_LEAF0 + k) { va = leaf[k][e]; }
+				if (kb == TCG_OPD_LEAF0 + k) { vb = leaf[k][e]; }
+			}
+			r[e] = kb == TCG_OPD_NONE ? apply_unary<T>(op, va) : apply_binary<T>(op, va, vb);
+		}
+#pragma unroll
+		for (int e = 0; e < N; ++e)
+		{
+			if (kd == TCG_OPD_T0) { t0[e] = r[e]; }
+			else if (kd == TCG_OPD_T1) { t1[e] = r[e]; }
+			else { acc[e] = r[e]; }
+		}
+	}
+}
+
+template <typename T, int NLEAF, bool VEC>
+__global__ __launch_bounds__(EW_BLOCK) void ew_fused_k (FusedProgram prog,
+	FusedLeaves<T,NLEAF> leaves, T* __restrict__ out, uint64_t n)
+{
+	constexpr int N = VEC ? Vec16<T>::N : 1;
+	const uint64_t nvec = n / N;
+	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
+	const uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
+	for (; i < nvec; i += step)
+	{
+		T leaf[NLEAF][N];
+		T acc[N];
+#pragma unroll
+		for (int k = 0; k < NLEAF; ++k)
+		{
+			if constexpr (VEC)
+			{
+				VecU<T> x;
+				x.v = ldv(leaves.p[k], i);
+#pragma unroll
+				for (int e = 0; e < N; ++e) { leaf[k][e] = x.e[e]; }
+			}
+			else { leaf[k][0] = leaves.p[k][i]; }
+		}
+		fused_eval<T,NLEAF,N>(prog, leaf, acc);
+		if constexpr (VEC)
+		{
+			VecU<T> y;
+#pragma unroll
+			for (int e = 0; e < N; ++e) { y.e[e] = acc[e]; }
+			stv(out, i, y.v);
+		}
+		else { out[i] = acc[0]; }
+	}
+	if (VEC && blockIdx.x == 0)
+	{
+		uint64_t t = nvec * N + threadIdx.x;
+		if (t < n)
+		{
+			T leaf[NLEAF][1];
+			T acc[1];
+#pragma unroll
+			for (int k = 0; k < NLEAF; ++k) { leaf[k][0] = leaves.p[k][t]; }
+			fused_eval<T,NLEAF,1>(prog, leaf, acc);
+			out[t] = acc[0];
+		}
+	}
+}
+
+// ---- host-side launchers ---------------------------------------------------
+
+template <typename T, int OP>
+void launch_unary_vec (tcg_ctx* ctx, const T* in, T* out, uint64_t n)
+{
+	uint64_t nvec = n / Vec16<T>::N;
+	unsigned grid = tcg_grid(ctx, nvec, EW_BLOCK * EW_UNROLL, 16);
+	ew_unary_vec_k<T,OP><<<grid, EW_BLOCK, 0, ctx->stream>>>(in, out, n);
+}
+
+template <typename T, int OP>
+void launch_binary_vec (tcg_ctx* ctx, const T* a, const T* b, T* out, uint64_t n)
+{
+	uint64_t nvec = n / Vec16<T>::N;
+	unsigned grid = tcg_grid(ctx, nvec, EW_BLOCK * EW_UNROLL, 16);
+	ew_binary_vec_k<T,OP><<<grid, EW_BLOCK, 0, ctx->stream>>>(a, b, out, n);
+}
+
+#define UNARY_CASE(OPC) case OPC: launch_unary_vec<T,OPC>(ctx, in, out, n); break;
+#define BINARY_CASE(OPC) case OPC: launch_binary_vec<T,OPC>(ctx, a, b, out, n); break;
+
+template <typename T>
+int unary_impl (tcg_ctx* ctx, int op, uint64_t n, const T* in, T* out)
+{
+	if (tcg_aligned16(in) && tcg_aligned16(out))
+	{
+		switch (op)
+		{
+			UNARY_CASE(TCG_ABS) UNARY_CASE(TCG_NEG) UNARY_CASE(TCG_SIN) UNARY_CASE(TCG_COS)
+			UNARY_CASE(TCG_TAN) UNARY_CASE(TCG_EXP) UNARY_CASE(TCG_LOG) UNARY_CASE(TCG_SQRT)
+			UNARY_CASE(TCG_ROUND) UNARY_CASE(TCG_SIGMOID) UNARY_CASE(TCG_TANH)
+			UNARY_CASE(TCG_SQUARE) UNARY_CASE(TCG_CUBE)
+		}
+	}
+	else
+	{
+		unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
+		ew_unary_scalar_k<T><<<grid, EW_BLOCK, 0, ctx->stream>>>(op, in, out, n);
+	}
+	TCG_LAUNCH_CHECK(ctx, "ew_unary");
+	return TCG_OK;
+}
+
+template <typename T>
+int binary_impl (tcg_ctx* ctx, int op, uint64_t n, const T* a, const T* b, T* out)
+{
+	if (tcg_aligned16(a) && tcg_aligned16(b) && tcg_aligned16(out))
+	{
+		switch (op)
+		{
+			BINARY_CASE(TCG_POW) BINARY_CASE(TCG_ADD) BINARY_CASE(TCG_SUB) BINARY_CASE(TCG_MUL)
+			BINARY_CASE(TCG_DIV) BINARY_CASE(TCG_MIN) BINARY_CASE(TCG_MAX) BINARY_CASE(TCG_EQ)
+			BINARY_CASE(TCG_NEQ) BINARY_CASE(TCG_LT) BINARY_CASE(TCG_GT)
+		}
+	}
+	else
+	{
+		unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
+		ew_binary_scalar_k<T><<<grid, EW_BLOCK, 0, ctx->stream>>>(op, a, b, out, n);
+	}
+	TCG_LAUNCH_CHECK(ctx, "ew_binary");
+	return TCG_OK;
+}
+
+template <typename T>
+int nary_impl (tcg_ctx* ctx, int op, uint64_t n, int nargs, const void* const* ins, T* out)
+{
+	// more than NARY_MAX operands: fold the first NARY_MAX, then keep folding
+	// into `out`; the left-to-right order of the reference is preserved
+	int done = 0;
+	while (done < nargs)
+	{
+		NaryArgs<T> args;
+		int k = 0;
+		bool vec = tcg_aligned16(out);
+		if (done > 0) { args.in[k++] = out; }
+		while (k < NARY_MAX && done < nargs) { args.in[k++] = (const T*) ins[done++]; }
+		args.nargs = k;
+		for (int j = 0; j < k; ++j) { vec = vec && tcg_aligned16(args.in[j]); }
+		if (vec)
+		{
+			unsigned grid = tcg_grid(ctx, n / Vec16<T>::N, EW_BLOCK, 32);
+			ew_nary_k<T,true><<<grid, EW_BLOCK, 0, ctx->stream>>>(op, args, out, n);
+		}
+		else
+		{
+			unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 32);
+			ew_nary_k<T,false><<<grid, EW_BLOCK, 0, ctx->stream>>>(op, args, out, n);
+		}
+		TCG_LAUNCH_CHECK(ctx, "ew_nary");
+	}
+	return TCG_OK;
+}
+
+template <typename TO>
+int cast_impl (tcg_ctx* ctx, int in_dtype, uint64_t n, const void* in, TO* out)
+{
+	unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
+	switch (in_dtype)
+	{
+		case TCG_DOUBLE: ew_cast_k<TO,double><<<grid, EW_BLOCK, 0, ctx->stream>>>((const double*) in, out, n); break;
+		case TCG_FLOAT: ew_cast_k<TO,float><<<grid, EW_BLOCK, 0, ctx->stream>>>((const float*) in, out, n); break;
+		case TCG_INT32: ew_cast_k<TO,int32_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const int32_t*) in, out, n); break;
+		default: return tcg_fail(ctx, TCG_ERR_ARG, "tcg_cast: unknown input dtype %d", in_dtype);
+	}
+	TCG_LAUNCH_CHECK(ctx, "ew_cast");
+	return TCG_OK;
+}
+
+template <typename T, int NLEAF>
+int fused_launch (tcg_ctx* ctx, const FusedProgram& prog, const void* const* leaves, T* out, uint64_t n)
+{
+	FusedLeaves<T,NLEAF> lv;
+	bool vec = tcg_aligned16(out);
+	for (int k = 0; k < NLEAF; ++k)
+	{
+		lv.p[k] = (const T*) leaves[k];
+		vec = vec && tcg_aligned16(leaves[k]);
+	}
+	if (vec)
+	{
+		unsigned grid = tcg_grid(ctx, n / Vec16<T>::N, EW_BLOCK, 32);
+		ew_fused_k<T,NLEAF,true><<<grid, EW_BLOCK, 0, ctx->stream>>>(prog, lv, out, n);
+	}
+	else
+	{
+		unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 32);
+		ew_fused_k<T,NLEAF,false><<<grid, EW_BLOCK, 0, ctx->stream>>>(prog, lv, out, n);
+	}
+	TCG_LAUNCH_CHECK(ctx, "ew_fused");
+	return TCG_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int tcg_ew_unary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, const void* in, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, is_unary_op(opcode), "tcg_ew_unary: opcode %d is not a unary elementwise op", opcode);
+	if (n == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, in && out, "tcg_ew_unary: NULL pointer");
+	TCG_DISPATCH_TYPE(ctx, dtype, return unary_impl<T>(ctx, opcode, n, (const T*) in, (T*) out));
+	return TCG_OK;
+}
+
+int tcg_ew_binary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
+	const void* a, const void* b, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, is_binary_op(opcode), "tcg_ew_binary: opcode %d is not a binary elementwise op", opcode);
+	if (n == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, a && b && out, "tcg_ew_binary: NULL pointer");
+	TCG_DISPATCH_TYPE(ctx, dtype, return binary_impl<T>(ctx, opcode, n, (const T*) a, (const T*) b, (T*) out));
+	return TCG_OK;
+}
+
+int tcg_ew_nary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
+	const void* const* ins, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, opcode == TCG_ADD || opcode == TCG_MUL, "tcg_ew_nary: opcode %d is not ADD or MUL", opcode);
+	TCG_REQUIRE(ctx, nargs >= 2 && ins, "tcg_ew_nary: needs at least 2 operands, got %d", nargs);
+	if (n == 0) { return TCG_OK; }
+	for (int i = 0; i < nargs; ++i) { TCG_REQUIRE(ctx, ins[i], "tcg_ew_nary: operand %d is NULL", i); }
+	TCG_REQUIRE(ctx, out, "tcg_ew_nary: NULL output");
+	TCG_DISPATCH_TYPE(ctx, dtype, return nary_impl<T>(ctx, opcode, n, nargs, ins, (T*) out));
+	return TCG_OK;
+}
+
+int tcg_ew_select (tcg_ctx* ctx, int dtype, uint64_t n, const void* cond,
+	const void* then, const void* otherwise, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (n == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, cond && then && otherwise && out, "tcg_ew_select: NULL pointer");
+	unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
+	TCG_DISPATCH_TYPE(ctx, dtype, (ew_select_k<T><<<grid, EW_BLOCK, 0, ctx->stream>>>(
+		(const T*) cond, (const T*) then, (const T*) otherwise, (T*) out, n)));
+	TCG_LAUNCH_CHECK(ctx, "ew_select");
+	return TCG_OK;
+}
+
+int tcg_cast (tcg_ctx* ctx, int out_dtype, int in_dtype, uint64_t n, const void* in, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (n == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, in && out, "tcg_cast: NULL pointer");
+	TCG_DISPATCH_TYPE(ctx, out_dtype, return cast_impl<T>(ctx, in_dtype, n, in, (T*) out));
+	return TCG_OK;
+}
+
+int tcg_assign (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, void* target, const void* source)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, opcode >= TCG_ASSIGN && opcode <= TCG_ASSIGN_DIV, "tcg_assign: opcode %d is not an ASSIGN op", opcode);
+	if (n == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, target && source, "tcg_assign: NULL pointer");
+	unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
+	TCG_DISPATCH_TYPE(ctx, dtype, (ew_assign_k<T><<<grid, EW_BLOCK, 0, ctx->stream>>>(
+		opcode, (T*) target, (const T*) source, n)));
+	TCG_LAUNCH_CHECK(ctx, "ew_assign");
+	return TCG_OK;
+}
+
+int tcg_ew_fused (tcg_ctx* ctx, int dtype, uint64_t n, int nleaves,
+	const void* const* leaves, int ninstrs, const tcg_ew_instr* program, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, nleaves >= 1 && nleaves <= TCG_EW_MAX_LEAVES, "tcg_ew_fused: %d leaves (1..%d allowed)", nleaves, TCG_EW_MAX_LEAVES);
+	TCG_REQUIRE(ctx, ninstrs >= 1 && ninstrs <= TCG_EW_MAX_INSTRS, "tcg_ew_fused: %d instructions (1..%d allowed)", ninstrs, TCG_EW_MAX_INSTRS);
+	TCG_REQUIRE(ctx, leaves && program && out, "tcg_ew_fused: NULL pointer");
+	FusedProgram prog;
+	memset(&prog, 0, sizeof(prog));
+	prog.ninstrs = ninstrs;
+	auto operand_ok = [nleaves](int k, bool allow_none)
+	{
+		if (k == TCG_OPD_NONE) { return allow_none; }
+		if (k >= TCG_OPD_ACC && k <= TCG_OPD_IMM) { return true; }
+		return k >= TCG_OPD_LEAF0 && k < TCG_OPD_LEAF0 + nleaves;
+	};
+	for (int i = 0; i < ninstrs; ++i)
+	{
+		const tcg_ew_instr& ins = program[i];
+		bool unary = ins.opcode == TCG_IDENTITY || is_unary_op(ins.opcode);
+		TCG_REQUIRE(ctx, unary || is_binary_op(ins.opcode), "tcg_ew_fused: instruction %d has opcode %d", i, (int) ins.opcode);
+		TCG_REQUIRE(ctx, operand_ok(ins.a, false) && operand_ok(ins.b, unary) && (unary == (ins.b == TCG_OPD_NONE)),
+			"tcg_ew_fused: instruction %d has bad operands (%d, %d)", i, (int) ins.a, (int) ins.b);
+		TCG_REQUIRE(ctx, ins.dst >= TCG_OPD_ACC && ins.dst <= TCG_OPD_T1, "tcg_ew_fused: instruction %d has bad destination %d", i, (int) ins.dst);
+		prog.opcode[i] = ins.opcode;
+		prog.a[i] = ins.a;
+		prog.b[i] = ins.b;
+		prog.dst[i] = ins.dst;
+		prog.imm[i] = ins.imm;
+	}
+	if (n == 0) { return TCG_OK; }
+	for (int k = 0; k < nleaves; ++k) { TCG_REQUIRE(ctx, leaves[k], "tcg_ew_fused: leaf %d is NULL", k); }
+	TCG_DISPATCH_TYPE(ctx, dtype,
+		switch (nleaves)
+		{
+			case 1: return fused_launch<T,1>(ctx, prog, leaves, (T*) out, n);
+			case 2: return fused_launch<T,2>(ctx, prog, leaves, (T*) out, n);
+			case 3: return fused_launch<T,3>(ctx, prog, leaves, (T*) out, n);
+			default: return fused_launch<T,4>(ctx, prog, leaves, (T*) out, n);
+		});
+	return TCG_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,468 @@
+// REDUCE_SUM / PROD / MIN / MAX and ARGMAX.
+//
+// Any reduction over a set of dims of an 8-D tensor is decomposed on the host
+// into steps of the form [A, R, B] -> [A, B] (A = contiguous kept elements,
+// R = reduced extent, B = everything outside):
+//   A == 1: "inner" kernel, one workgroup (or S of them) per row of R
+//           contiguous elements, 128-bit loads, wave shuffle + LDS tree;
+//   A  > 1: "outer" kernel, a workgroup owns a strip of columns, lanes run
+//           along the contiguous dim, rows are split over the wave rows of
+//           the group and over S groups; LDS combines the wave rows.
+// When R is split over S workgroups the partial results go to a scratch
+// tensor [A, S, B] that a second launch of the same kernel reduces.
+// Both kernels read every input byte exactly once: HBM-bound.
+#include "tcg_internal.hpp"
+
+#include <limits>
+
+namespace
+{
+
+template <typename T> struct is_int { static constexpr bool value = false; };
+template <> struct is_int<int32_t> { static constexpr bool value = true; };
+
+template <typename T, int OP>
+struct Red
+{
+	static __device__ __forceinline__ T identity ()
+	{
+		if constexpr (OP == TCG_REDUCE_SUM) { return (T) 0; }
+		else if constexpr (OP == TCG_REDUCE_PROD) { return (T) 1; }
+		else if constexpr (OP == TCG_REDUCE_MIN)
+		{
+			if constexpr (is_int<T>::value) { return INT32_MAX; }
+			else { return (T) INFINITY; }
+		}
+		else
+		{
+			if constexpr (is_int<T>::value) { return INT32_MIN; }
+			else { return (T) -INFINITY; }
+		}
+	}
+
+	static __device__ __forceinline__ T combine (T a, T b)
+	{
+		if constexpr (OP == TCG_REDUCE_SUM)
+		{
+			if constexpr (is_int<T>::value) { return (T) ((uint32_t) a + (uint32_t) b); }
+			else { return a + b; }
+		}
+		else if constexpr (OP == TCG_REDUCE_PROD)
+		{
+			if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b); }
+			else { return a * b; }
+		}
+		else if constexpr (OP == TCG_REDUCE_MIN) { return b < a ? b : a; }
+		else { return b > a ? b : a; }
+	}
+};
+
+template <typename T>
+__device__ __forceinline__ T shfl_xor_t (T v, int mask)
+{
+	if constexpr (sizeof(T) == 8)
+	{
+		union { T t; int i[2]; } u;
+		u.t = v;
+		u.i[0] = __shfl_xor(u.i[0], mask, TCG_WAVE);
+		u.i[1] = __shfl_xor(u.i[1], mask, TCG_WAVE);
+		return u.t;
+	}
+	else { return __shfl_xor(v, mask, TCG_WAVE); }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ T wave_reduce (T v)
+{
+#pragma unroll
+	for (int m = TCG_WAVE / 2; m >= 1; m >>= 1)
+	{
+		v = Red<T,OP>::combine(v, shfl_xor_t(v, m));
+	}
+	return v;
+}
+
+constexpr int RED_BLOCK = 256;
+constexpr int RED_WAVES = RED_BLOCK / TCG_WAVE;
+
+// rows of R contiguous elements; block b reduces the part `b % S` of row
+// `b / S` and writes out[row * S + part]
+template <typename T, int OP, bool VEC>
+__global__ __launch_bounds__(RED_BLOCK) void reduce_inner_k (
+	const T* __restrict__ in, T* __restrict__ out, uint64_t R, uint32_t S, uint64_t chunk)
+{
+	constexpr int N = VEC ? Vec16<T>::N : 1;
+	const uint64_t row = blockIdx.x / S;
+	const uint32_t part = blockIdx.x % S;
+	const T* base = in + row * R;
+	const uint64_t lo = (uint64_t) part * chunk;
+	uint64_t hi = lo + chunk;
+	if (hi > R) { hi = R; }
+
+	T acc[4];
+#pragma unroll
+	for (int u = 0; u < 4; ++u) { acc[u] = Red<T,OP>::identity(); }
+	if constexpr (VEC)
+	{
+		// lo and chunk are multiples of N; the tail of the row is scalar
+		const uint64_t vlo = lo / N, vhi = hi / N;
+		uint64_t i = vlo + threadIdx.x;
+		for (; i + 3 * RED_BLOCK < vhi; i += 4 * RED_BLOCK)
+		{
+			VecU<T> x[4];
+#pragma unroll
+			for (int u = 0; u < 4; ++u)
+			{
+				x[u].v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base) + i + u * RED_BLOCK);
+			}
+#pragma unroll
+			for (int u = 0; u < 4; ++u)
+			{
+#pragma unroll
+				for (int e = 0; e < N; ++e) { acc[u] = Red<T,OP>::combine(acc[u], x[u].e[e]); }
+			}
+		}
+		for (; i < vhi; i += RED_BLOCK)
+		{
+			VecU<T> x;
+			x.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base) + i);
+#pragma unroll
+			for (int e = 0; e < N; ++e) { acc[0] = Red<T,OP>::combine(acc[0], x.e[e]); }
+		}
+		uint64_t t = vhi * N + threadIdx.x;
+		if (t < hi) { acc[1] = Red<T,OP>::combine(acc[1], base[t]); }
+	}
+	else
+	{
+		for (uint64_t i = lo + threadIdx.x; i < hi; i += RED_BLOCK)
+		{
+			acc[0] = Red<T,OP>::combine(acc[0], base[i]);
+		}
+	}
+	T v = Red<T,OP>::combine(Red<T,OP>::combine(acc[0], acc[1]), Red<T,OP>::combine(acc[2], acc[3]));
+	v = wave_reduce<T,OP>(v);
+	__shared__ T smem[RED_WAVES];
+	const int wave = threadIdx.x / TCG_WAVE, lane = threadIdx.x % TCG_WAVE;
+	if (lane == 0) { smem[wave] = v; }
+	__syncthreads();
+	if (threadIdx.x == 0)
+	{
+		T r = smem[0];
+#pragma unroll
+		for (int w = 1; w < RED_WAVES; ++w) { r = Red<T,OP>::combine(r, smem[w]); }
+		out[row * S + part] = r;
+	}
+}
+
+// in[a + r*A + b*A*R] -> out[a + s*A + b*A*S]; the group is TX lanes wide
+// (each lane N columns) and TY = 256 / TX rows tall
+template <typename T, int OP, bool VEC>
+__global__ __launch_bounds__(RED_BLOCK) void reduce_outer_k (
+	const T* __restrict__ in, T* __restrict__ out, uint64_t A, uint64_t R,
+	uint32_t S, uint64_t chunk, uint32_t txlog2, uint32_t col_tiles)
+{
+	constexpr int N = VEC ? Vec16<T>::N : 1;
+	const uint32_t TX = 1u << txlog2, TY = RED_BLOCK >> txlog2;
+	const uint32_t tx = threadIdx.x & (TX - 1), ty = threadIdx.x >> txlog2;
+	uint64_t bid = blockIdx.x;
+	const uint32_t ctile = bid % col_tiles;
+	bid /= col_tiles;
+	const uint32_t part = bid % S;
+	const uint64_t b = bid / S;
+	const uint64_t col = ((uint64_t) ctile * TX + tx) * N;
+	const uint64_t lo = (uint64_t) part * chunk;
+	uint64_t hi = lo + chunk;
+	if (hi > R) { hi = R; }
+
+	T acc[N], acc2[N];
+#pragma unroll
+	for (int e = 0; e < N; ++e) { acc[e] = Red<T,OP>::identity(); acc2[e] = Red<T,OP>::identity(); }
+	if (col < A)
+	{
+		const T* base = in + col + b * A * R;
+		uint64_t r = lo + ty;
+		if constexpr (VEC)
+		{
+			for (; r + TY < hi; r += 2 * TY)
+			{
+				VecU<T> x, y;
+				x.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base + r * A));
+				y.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base + (r + TY) * A));
+#pragma unroll
+				for (int e = 0; e < N; ++e)
+				{
+					acc[e] = Red<T,OP>::combine(acc[e], x.e[e]);
+					acc2[e] = Red<T,OP>::combine(acc2[e], y.e[e]);
+				}
+			}
+			for (; r < hi; r += TY)
+			{
+				VecU<T> x;
+				x.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base + r * A));
+#pragma unroll
+				for (int e = 0; e < N; ++e) { acc[e] = Red<T,OP>::combine(acc[e], x.e[e]); }
+			}
+		}
+		else
+		{
+			for (; r < hi; r += TY) { acc[0] = Red<T,OP>::combine(acc[0], base[r * A]); }
+		}
+	}
+#pragma unroll
+	for (int e = 0; e < N; ++e) { acc[e] = Red<T,OP>::combine(acc[e], acc2[e]); }
+
+	// combine the TY rows of the group through LDS; row stride padded by one
+	// element so that the column walk below is conflict-free
+	__shared__ T smem[RED_BLOCK * (VEC ? Vec16<T>::N : 1) + RED_BLOCK];
+	const uint32_t pitch = TX * N + 1;
+#pragma unroll
+	for (int e = 0; e < N; ++e) { smem[ty * pitch + tx * N + e] = acc[e]; }
+	__syncthreads();
+	const uint32_t ncols = TX * N;
+	for (uint32_t c = threadIdx.x; c < ncols; c += RED_BLOCK)
+	{
+		T r = smem[c];
+		for (uint32_t y = 1; y < TY; ++y) { r = Red<T,OP>::combine(r, smem[y * pitch + c]); }
+		uint64_t gcol = (uint64_t) ctile * TX * N + c;
+		if (gcol < A) { out[gcol + (uint64_t) part * A + b * A * S] = r; }
+	}
+}
+
+// block per output (a, b): value and index of the first maximum along R
+template <typename T>
+__global__ __launch_bounds__(RED_BLOCK) void argmax_k (
+	const T* __restrict__ in, T* __restrict__ out, uint64_t A, uint64_t R)
+{
+	const uint64_t a = blockIdx.x % A, b = blockIdx.x / A;
+	const T* base = in + a + b * A * R;
+	uint64_t best_i = ~(uint64_t) 0;
+	T best = 0;
+	for (uint64_t r = threadIdx.x; r < R; r += RED_BLOCK)
+	{
+		T v = base[r * A];
+		if (best_i == ~(uint64_t) 0 || v > best) { best = v; best_i = r; }
+	}
+	__shared__ T sval[RED_BLOCK];
+	__shared__ uint64_t sidx[RED_BLOCK];
+	sval[threadIdx.x] = best;
+	sidx[threadIdx.x] = best_i;
+	__syncthreads();
+	for (int s = RED_BLOCK / 2; s >= 1; s >>= 1)
+	{
+		if ((int) threadIdx.x < s)
+		{
+			T ov = sval[threadIdx.x + s];
+			uint64_t oi = sidx[threadIdx.x + s];
+			uint64_t mi = sidx[threadIdx.x];
+			if (oi != ~(uint64_t) 0 && (mi == ~(uint64_t) 0 || ov > sval[threadIdx.x] ||
+				(ov == sval[threadIdx.x] && oi < mi)))
+			{
+				sval[threadIdx.x] = ov;
+				sidx[threadIdx.x] = oi;
+			}
+		}
+		__syncthreads();
+	}
+	if (threadIdx.x == 0) { out[blockIdx.x] = (T) sidx[0]; }
+}
+
+uint32_t ilog2_floor (uint64_t v)
+{
+	uint32_t l = 0;
+	while (v > 1) { v >>= 1; ++l; }
+	return l;
+}
+
+template <typename T, int OP>
+int launch_inner (tcg_ctx* ctx, const T* in, T* out, uint64_t R, uint64_t K, uint32_t S, uint64_t chunk)
+{
+	bool vec = tcg_aligned16(in) && (R % Vec16<T>::N == 0);
+	uint64_t blocks = K * S;
+	TCG_REQUIRE(ctx, blocks < (1ull << 31), "tcg_reduce: %llu rows are too many for one launch", (unsigned long long) blocks);
+	if (vec) { reduce_inner_k<T,OP,true><<<(unsigned) blocks, RED_BLOCK, 0, ctx->stream>>>(in, out, R, S, chunk); }
+	else { reduce_inner_k<T,OP,false><<<(unsigned) blocks, RED_BLOCK, 0, ctx->stream>>>(in, out, R, S, chunk); }
+	TCG_LAUNCH_CHECK(ctx, "reduce_inner");
+	return TCG_OK;
+}
+
+template <typename T, int OP>
+int launch_outer (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint64_t B, uint32_t S, uint64_t chunk, uint32_t txlog2, bool vec)
+{
+	const uint32_t N = vec ? Vec16<T>::N : 1;
+	uint64_t col_tiles = (A + ((uint64_t) N << txlog2) - 1) / ((uint64_t) N << txlog2);
+	uint64_t blocks = col_tiles * S * B;
+	TCG_REQUIRE(ctx, blocks < (1ull << 31) && col_tiles < (1ull << 31), "tcg_reduce: %llu workgroups are too many for one launch", (unsigned long long) blocks);
+	if (vec) { reduce_outer_k<T,OP,true><<<(unsigned) blocks, RED_BLOCK, 0, ctx->stream>>>(in, out, A, R, S, chunk, txlog2, (uint32_t) col_tiles); }
+	else { reduce_outer_k<T,OP,false><<<(unsigned) blocks, RED_BLOCK, 0, ctx->stream>>>(in, out, A, R, S, chunk, txlog2, (uint32_t) col_tiles); }
+	TCG_LAUNCH_CHECK(ctx, "reduce_outer");
+	return TCG_OK;
+}
+
+// [A, R, B] -> [A, B]
+template <typename T, int OP>
+int reduce_step (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint64_t B)
+{
+	const uint64_t target_blocks = (uint64_t) ctx->num_cus * 8;
+	if (A == 1)
+	{
+		// split rows only when there are too few of them to fill the chip
+		constexpr uint64_t quantum = (uint64_t) RED_BLOCK * Vec16<T>::N * 4;
+		uint64_t S = 1;
+		if (B < target_blocks && R >= 4 * quantum)
+		{
+			S = (target_blocks + B - 1) / B;
+			uint64_t maxs = R / (2 * quantum);
+			if (S > maxs) { S = maxs; }
+			if (S < 1) { S = 1; }
+		}
+		uint64_t chunk = (R + S - 1) / S;
+		chunk = (chunk + quantum - 1) / quantum * quantum;
+		S = (R + chunk - 1) / chunk;
+		if (S == 1) { return launch_inner<T,OP>(ctx, in, out, R, B, 1, chunk); }
+		void* partial = nullptr;
+		int rc = tcg_alloc(ctx, sizeof(T) * B * S, &partial);
+		if (rc != TCG_OK) { return rc; }
+		rc = launch_inner<T,OP>(ctx, in, (T*) partial, R, B, (uint32_t) S, chunk);
+		if (rc == TCG_OK) { rc = launch_inner<T,OP>(ctx, (const T*) partial, out, S, B, 1, S); }
+		tcg_free(ctx, partial, sizeof(T) * B * S);
+		return rc;
+	}
+	bool vec = tcg_aligned16(in) && (A % Vec16<T>::N == 0);
+	const uint32_t N = vec ? Vec16<T>::N : 1;
+	uint64_t lanes = (A + N - 1) / N;
+	uint32_t txlog2 = lanes >= 64 ? 6 : ilog2_floor(lanes);
+	if (((uint64_t) 1 << txlog2) < lanes && txlog2 < 6) { ++txlog2; }
+	const uint32_t TY = RED_BLOCK >> txlog2;
+	uint64_t col_tiles = (lanes + ((uint64_t) 1 << txlog2) - 1) >> txlog2;
+	uint64_t base_blocks = col_tiles * B;
+	uint64_t S = 1;
+	if (base_blocks < target_blocks && R >= (uint64_t) TY * 16)
+	{
+		S = (target_blocks + base_blocks - 1) / base_blocks;
+		uint64_t maxs = R / ((uint64_t) TY * 8);
+		if (S > maxs) { S = maxs; }
+		if (S < 1) { S = 1; }
+	}
+	uint64_t chunk = (R + S - 1) / S;
+	S = (R + chunk - 1) / chunk;
+	if (S == 1) { return launch_outer<T,OP>(ctx, in, out, A, R, B, 1, chunk, txlog2, vec); }
+	void* partial = nullptr;
+	int rc = tcg_alloc(ctx, sizeof(T) * A * S * B, &partial);
+	if (rc != TCG_OK) { return rc; }
+	rc = launch_outer<T,OP>(ctx, in, (T*) partial, A, R, B, (uint32_t) S, chunk, txlog2, vec);
+	if (rc == TCG_OK) { rc = launch_outer<T,OP>(ctx, (const T*) partial, out, A, S, B, 1, S, txlog2, vec); }
+	tcg_free(ctx, partial, sizeof(T) * A * S * B);
+	return rc;
+}
+
+template <typename T, int OP>
+int reduce_impl (tcg_ctx* ctx, const uint64_t shape[8], unsigned mask, const T* in, T* out)
+{
+	// merge neighbouring dims of equal kind, dropping singular dims
+	uint64_t seg[8];
+	bool red[8];
+	int nseg = 0;
+	for (int d = 0; d < 8; ++d)
+	{
+		if (shape[d] == 1) { continue; }
+		bool r = (mask >> d) & 1;
+		if (nseg > 0 && red[nseg - 1] == r) { seg[nseg - 1] *= shape[d]; }
+		else { seg[nseg] = shape[d]; red[nseg] = r; ++nseg; }
+	}
+	int nred = 0;
+	uint64_t n = 1;
+	for (int i = 0; i < nseg; ++i) { nred += red[i]; n *= seg[i]; }
+	if (nred == 0)
+	{
+		TCG_HIP(ctx, hipMemcpyAsync(out, in, sizeof(T) * n, hipMemcpyDeviceToDevice, ctx->stream));
+		return TCG_OK;
+	}
+	// reduce the innermost reduced segment first; what is left of the tensor
+	// shrinks at every step
+	const T* cur = in;
+	void* tmp_prev = nullptr;
+	size_t tmp_prev_bytes = 0;
+	int rc = TCG_OK;
+	while (nred > 0 && rc == TCG_OK)
+	{
+		int i = 0;
+		while (!red[i]) { ++i; }
+		uint64_t A = 1, B = 1;
+		for (int j = 0; j < i; ++j) { A *= seg[j]; }
+		for (int j = i + 1; j < nseg; ++j) { B *= seg[j]; }
+		uint64_t R = seg[i];
+		T* dst = out;
+		void* tmp = nullptr;
+		size_t tmp_bytes = 0;
+		if (nred > 1)
+		{
+			tmp_bytes = sizeof(T) * A * B;
+			rc = tcg_alloc(ctx, tmp_bytes, &tmp);
+			if (rc != TCG_OK) { break; }
+			dst = (T*) tmp;
+		}
+		rc = reduce_step<T,OP>(ctx, cur, dst, A, R, B);
+		if (tmp_prev) { tcg_free(ctx, tmp_prev, tmp_prev_bytes); }
+		tmp_prev = tmp;
+		tmp_prev_bytes = tmp_bytes;
+		cur = dst;
+		// drop segment i and merge its (kept) neighbours
+		for (int j = i; j + 1 < nseg; ++j) { seg[j] = seg[j + 1]; red[j] = red[j + 1]; }
+		--nseg;
+		--nred;
+		if (i > 0 && i < nseg && red[i - 1] == red[i])
+		{
+			seg[i - 1] *= seg[i];
+			for (int j = i; j + 1 < nseg; ++j) { seg[j] = seg[j + 1]; red[j] = red[j + 1]; }
+			--nseg;
+		}
+	}
+	if (tmp_prev) { tcg_free(ctx, tmp_prev, tmp_prev_bytes); }
+	return rc;
+}
+
+} // namespace
+
+extern "C" {
+
+int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
+	unsigned rankmask, const void* in, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, opcode >= TCG_REDUCE_SUM && opcode <= TCG_REDUCE_MAX, "tcg_reduce: opcode %d is not a reduction", opcode);
+	TCG_REQUIRE(ctx, shape && in && out, "tcg_reduce: NULL pointer");
+	TCG_REQUIRE(ctx, rankmask < 256, "tcg_reduce: rank set 0x%x names a dim >= 8", rankmask);
+	if (tcg_n_elems(shape) == 0) { return TCG_OK; }
+	TCG_DISPATCH_TYPE(ctx, dtype,
+		switch (opcode)
+		{
+			case TCG_REDUCE_SUM: return reduce_impl<T,TCG_REDUCE_SUM>(ctx, shape, rankmask, (const T*) in, (T*) out);
+			case TCG_REDUCE_PROD: return reduce_impl<T,TCG_REDUCE_PROD>(ctx, shape, rankmask, (const T*) in, (T*) out);
+			case TCG_REDUCE_MIN: return reduce_impl<T,TCG_REDUCE_MIN>(ctx, shape, rankmask, (const T*) in, (T*) out);
+			default: return reduce_impl<T,TCG_REDUCE_MAX>(ctx, shape, rankmask, (const T*) in, (T*) out);
+		});
+	return TCG_OK;
+}
+
+int tcg_argmax (tcg_ctx* ctx, int dtype, const uint64_t shape[8], int return_dim,
+	const void* in, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, shape && in && out, "tcg_argmax: NULL pointer");
+	TCG_REQUIRE(ctx, return_dim >= 0, "tcg_argmax: negative return_dim");
+	uint64_t n = tcg_n_elems(shape);
+	if (n == 0) { return TCG_OK; }
+	uint64_t A = 1, R = n, B = 1;
+	if (return_dim < 8)
+	{
+		R = shape[return_dim];
+		for (int d = 0; d < return_dim; ++d) { A *= shape[d]; }
+		for (int d = return_dim + 1; d < 8; ++d) { B *= shape[d]; }
+	}
+	TCG_REQUIRE(ctx, A * B < (1ull << 31), "tcg_argmax: too many outputs for one launch");
+	TCG_DISPATCH_TYPE(ctx, dtype, (argmax_k<T><<<(unsigned) (A * B), RED_BLOCK, 0, ctx->stream>>>((const T*) in, (T*) out, A, R)));
+	TCG_LAUNCH_CHECK(ctx, "argmax");
+	return TCG_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,296 @@
+// Context, stream-ordered memory pool, host<->device transfers and stream
+// timers of the gfx950 backend.
+#include "tcg_internal.hpp"
+
+static thread_local std::string g_create_error;
+
+int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...)
+{
+	char buf[1024];
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(buf, sizeof(buf), fmt, ap);
+	va_end(ap);
+	if (ctx) { ctx->error = buf; }
+	else { g_create_error = buf; }
+	return status;
+}
+
+static __global__ void fill_zero_k (uint32_t* dst, uint64_t nwords)
+{
+	uint64_t i = (uint64_t) blockIdx.x * blockDim.x + threadIdx.x;
+	uint64_t step = (uint64_t) gridDim.x * blockDim.x;
+	for (; i < nwords; i += step) { dst[i] = 0u; }
+}
+
+static __global__ void fill_zero_bytes_k (uint8_t* dst, uint64_t n)
+{
+	uint64_t i = (uint64_t) blockIdx.x * blockDim.x + threadIdx.x;
+	if (i < n) { dst[i] = 0; }
+}
+
+extern "C" {
+
+int tcg_ctx_create (int device, tcg_ctx** out)
+{
+	if (!out) { return tcg_fail(nullptr, TCG_ERR_ARG, "tcg_ctx_create: out is NULL"); }
+	*out = nullptr;
+	int ndev = 0;
+	hipError_t err = hipGetDeviceCount(&ndev);
+	if (err != hipSuccess || ndev <= 0)
+	{
+		return tcg_fail(nullptr, TCG_ERR_HIP,
+			"tcg_ctx_create: no HIP device visible (%s); this backend has no CPU fallback",
+			err != hipSuccess ? hipGetErrorString(err) : "device count is 0");
+	}
+	if (device < 0 || device >= ndev)
+	{
+		return tcg_fail(nullptr, TCG_ERR_ARG, "tcg_ctx_create: device %d of %d", device, ndev);
+	}
+	tcg_ctx* ctx = new tcg_ctx();
+	ctx->device = device;
+	hipDeviceProp_t prop;
+	if ((err = hipSetDevice(device)) != hipSuccess ||
+		(err = hipGetDeviceProperties(&prop, device)) != hipSuccess ||
+		(err = hipStreamCreate(&ctx->stream)) != hipSuccess ||
+		(err = hipEventCreate(&ctx->ev_begin)) != hipSuccess ||
+		(err = hipEventCreate(&ctx->ev_end)) != hipSuccess)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: %s", hipGetErrorString(err));
+		delete ctx;
+		return rc;
+	}
+	ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+	ctx->arch = prop.gcnArchName;
+	size_t colon = ctx->arch.find(':');
+	if (colon != std::string::npos) { ctx->arch.resize(colon); }
+	ctx->staging_size = 8u << 20;
+	if ((err = hipHostMalloc((void**) &ctx->staging, ctx->staging_size, hipHostMallocDefault)) != hipSuccess)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: hipHostMalloc: %s", hipGetErrorString(err));
+		delete ctx;
+		return rc;
+	}
+	*out = ctx;
+	return TCG_OK;
+}
+
+int tcg_ctx_destroy (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_OK; }
+	(void) hipSetDevice(ctx->device);
+	(void) hipStreamSynchronize(ctx->stream);
+	for (auto& kv : ctx->block_size) { (void) hipFree(kv.first); }
+	if (ctx->scratch) { (void) hipFree(ctx->scratch); }
+	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
+	(void) hipEventDestroy(ctx->ev_begin);
+	(void) hipEventDestroy(ctx->ev_end);
+	(void) hipStreamDestroy(ctx->stream);
+	delete ctx;
+	return TCG_OK;
+}
+
+const char* tcg_last_error (const tcg_ctx* ctx)
+{
+	return ctx ? ctx->error.c_str() : g_create_error.c_str();
+}
+
+const char* tcg_device_arch (const tcg_ctx* ctx)
+{
+	return ctx ? ctx->arch.c_str() : "";
+}
+
+static size_t round_block (size_t bytes)
+{
+	// 256-byte granules up to 1 MiB, then 1/8-octave steps: bounded
+	// fragmentation with few distinct size classes
+	if (bytes == 0) { bytes = 1; }
+	if (bytes <= (1u << 20)) { return (bytes + 255) & ~(size_t) 255; }
+	size_t p = (size_t) 1 << 20;
+	while (p * 2 <= bytes) { p *= 2; }
+	size_t step = p / 8;
+	return (bytes + step - 1) / step * step;
+}
+
+int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr)
+{
+	if (!ctx || !devptr) { return TCG_ERR_ARG; }
+	size_t sz = round_block(bytes);
+	auto it = ctx->free_blocks.find(sz);
+	if (it != ctx->free_blocks.end() && !it->second.empty())
+	{
+		*devptr = it->second.back();
+		it->second.pop_back();
+		ctx->bytes_pooled -= sz;
+		ctx->bytes_in_use += sz;
+		return TCG_OK;
+	}
+	void* p = nullptr;
+	hipError_t err = hipMalloc(&p, sz);
+	if (err != hipSuccess)
+	{
+		// give cached blocks back to the driver and retry once
+		(void) hipStreamSynchronize(ctx->stream);
+		for (auto& kv : ctx->free_blocks)
+		{
+			for (void* q : kv.second)
+			{
+				(void) hipFree(q);
+				ctx->block_size.erase(q);
+			}
+			kv.second.clear();
+		}
+		ctx->bytes_pooled = 0;
+		err = hipMalloc(&p, sz);
+		if (err != hipSuccess)
+		{
+			(void) hipGetLastError();
+			return tcg_fail(ctx, TCG_ERR_OOM, "tcg_alloc: %zu bytes: %s", sz, hipGetErrorString(err));
+		}
+	}
+	ctx->block_size[p] = sz;
+	ctx->bytes_in_use += sz;
+	*devptr = p;
+	return TCG_OK;
+}
+
+int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (!devptr) { return TCG_OK; }
+	auto it = ctx->block_size.find(devptr);
+	TCG_REQUIRE(ctx, it != ctx->block_size.end(), "tcg_free: %p was not allocated by this context", devptr);
+	size_t sz = it->second;
+	TCG_REQUIRE(ctx, round_block(bytes) == sz,
+		"tcg_free: %p was allocated with another size (%zu bytes given)", devptr, bytes);
+	ctx->free_blocks[sz].push_back(devptr);
+	ctx->bytes_in_use -= sz;
+	ctx->bytes_pooled += sz;
+	return TCG_OK;
+}
+
+int tcg_mem_stats (const tcg_ctx* ctx, uint64_t* in_use, uint64_t* pooled)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (in_use) { *in_use = ctx->bytes_in_use; }
+	if (pooled) { *pooled = ctx->bytes_pooled; }
+	return TCG_OK;
+}
+
+int tcg_h2d (tcg_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (bytes == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, dst_dev && src_host, "tcg_h2d: NULL pointer");
+	if (bytes <= ctx->staging_size / 4)
+	{
+		// small: stage through pinned memory so that the call returns at once
+		size_t need = (bytes + 63) & ~(size_t) 63;
+		if (ctx->staging_head + need > ctx->staging_size)
+		{
+			TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
+			ctx->staging_head = 0;
+		}
+		char* slot = ctx->staging + ctx->staging_head;
+		memcpy(slot, src_host, bytes);
+		ctx->staging_head += need;
+		TCG_HIP(ctx, hipMemcpyAsync(dst_dev, slot, bytes, hipMemcpyHostToDevice, ctx->stream));
+		return TCG_OK;
+	}
+	TCG_HIP(ctx, hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_d2h (tcg_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (bytes == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, dst_host && src_dev, "tcg_d2h: NULL pointer");
+	TCG_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_d2d (tcg_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (bytes == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, dst_dev && src_dev, "tcg_d2d: NULL pointer");
+	TCG_HIP(ctx, hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_fill_zero (tcg_ctx* ctx, void* dst_dev, size_t bytes)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (bytes == 0) { return TCG_OK; }
+	TCG_REQUIRE(ctx, dst_dev, "tcg_fill_zero: NULL pointer");
+	// a fill kernel rather than hipMemsetAsync: callers may capture this
+	// stream into a graph
+	uint8_t* p = (uint8_t*) dst_dev;
+	size_t head = (4 - (reinterpret_cast<uintptr_t>(p) & 3)) & 3;
+	if (head > bytes) { head = bytes; }
+	if (head)
+	{
+		fill_zero_bytes_k<<<1, 64, 0, ctx->stream>>>(p, head);
+	}
+	size_t nwords = (bytes - head) / 4;
+	if (nwords)
+	{
+		unsigned grid = tcg_grid(ctx, nwords, 256 * 8, 8);
+		fill_zero_k<<<grid, 256, 0, ctx->stream>>>((uint32_t*) (p + head), nwords);
+	}
+	size_t tail = bytes - head - nwords * 4;
+	if (tail)
+	{
+		fill_zero_bytes_k<<<1, 64, 0, ctx->stream>>>(p + head + nwords * 4, tail);
+	}
+	TCG_LAUNCH_CHECK(ctx, "fill_zero");
+	return TCG_OK;
+}
+
+int tcg_sync (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_timer_begin (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_HIP(ctx, hipEventRecord(ctx->ev_begin, ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_timer_end (tcg_ctx* ctx, float* ms)
+{
+	if (!ctx || !ms) { return TCG_ERR_ARG; }
+	TCG_HIP(ctx, hipEventRecord(ctx->ev_end, ctx->stream));
+	TCG_HIP(ctx, hipEventSynchronize(ctx->ev_end));
+	TCG_HIP(ctx, hipEventElapsedTime(ms, ctx->ev_begin, ctx->ev_end));
+	return TCG_OK;
+}
+
+} // extern "C"
+
+int tcg_scratch (tcg_ctx* ctx, size_t bytes, void** out)
+{
+	if (bytes > ctx->scratch_size)
+	{
+		if (ctx->scratch)
+		{
+			// earlier launches may still read the old scratch
+			TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
+			TCG_HIP(ctx, hipFree(ctx->scratch));
+			ctx->scratch = nullptr;
+			ctx->scratch_size = 0;
+		}
+		size_t sz = (bytes + (1u << 20) - 1) & ~(size_t) ((1u << 20) - 1);
+		TCG_HIP(ctx, hipMalloc(&ctx->scratch, sz));
+		ctx->scratch_size = sz;
+	}
+	*out = ctx->scratch;
+	return TCG_OK;
+}

@@ -1,0 +1,128 @@
+// Shared declarations of the gfx950 backend: context layout, error helpers,
+// dtype dispatch and the small device utilities every kernel file uses.
+#ifndef TCG_INTERNAL_HPP
+#define TCG_INTERNAL_HPP
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "tcg.h"
+
+#define TCG_WAVE 64
+
+struct tcg_ctx
+{
+	int device = 0;
+	hipStream_t stream = nullptr;
+	hipEvent_t ev_begin = nullptr;
+	hipEvent_t ev_end = nullptr;
+	int num_cus = 256;
+	std::string arch;
+	std::string error;
+
+	// stream-ordered pool: freed blocks go back to a per-size free list and are
+	// handed out again without a device-wide synchronisation, which is safe
+	// because every launch of the context is ordered on `stream`
+	std::map<size_t,std::vector<void*>> free_blocks;
+	std::map<void*,size_t> block_size; // every block ever hipMalloc'ed
+	uint64_t bytes_in_use = 0;
+	uint64_t bytes_pooled = 0;
+
+	// pinned staging ring for small host->device copies
+	char* staging = nullptr;
+	size_t staging_size = 0;
+	size_t staging_head = 0;
+
+	// scratch for two-pass reductions and operand repacking; grown on demand
+	void* scratch = nullptr;
+	size_t scratch_size = 0;
+};
+
+int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);
+int tcg_scratch (tcg_ctx* ctx, size_t bytes, void** out);
+
+#define TCG_HIP(ctx, call) do {\
+	hipError_t err__ = (call);\
+	if (err__ != hipSuccess) {\
+		return tcg_fail(ctx, TCG_ERR_HIP, "%s failed: %s (%s:%d)", #call,\
+			hipGetErrorString(err__), __FILE__, __LINE__);\
+	} } while (0)
+
+#define TCG_LAUNCH_CHECK(ctx, what) do {\
+	hipError_t err__ = hipGetLastError();\
+	if (err__ != hipSuccess) {\
+		return tcg_fail(ctx, TCG_ERR_HIP, "launch of %s failed: %s", what,\
+			hipGetErrorString(err__));\
+	} } while (0)
+
+#define TCG_REQUIRE(ctx, cond, ...) do {\
+	if (!(cond)) { return tcg_fail(ctx, TCG_ERR_ARG, __VA_ARGS__); } } while (0)
+
+static inline size_t tcg_type_size (int dtype)
+{
+	switch (dtype)
+	{
+		case TCG_DOUBLE: return 8;
+		case TCG_FLOAT: return 4;
+		case TCG_INT32: return 4;
+		default: return 0;
+	}
+}
+
+static inline uint64_t tcg_n_elems (const uint64_t shape[8])
+{
+	uint64_t n = 1;
+	for (int i = 0; i < 8; ++i) { n *= shape[i]; }
+	return n;
+}
+
+static inline bool tcg_aligned16 (const void* p)
+{
+	return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+
+// Number of workgroups for a streaming kernel: enough to cover `work` items,
+// capped at a multiple of the CU count so that a grid-stride loop takes over
+static inline unsigned tcg_grid (const tcg_ctx* ctx, uint64_t work_items,
+	unsigned per_block, unsigned blocks_per_cu)
+{
+	uint64_t need = (work_items + per_block - 1) / per_block;
+	uint64_t cap = (uint64_t) ctx->num_cus * blocks_per_cu;
+	if (need < 1) { need = 1; }
+	return (unsigned) (need < cap ? need : cap);
+}
+
+// Runs `stmt` with `T` bound to the C++ type of `dtype`
+#define TCG_DISPATCH_TYPE(ctx, dtype, ...) do {\
+	switch (dtype) {\
+		case TCG_DOUBLE: { using T = double; __VA_ARGS__; } break;\
+		case TCG_FLOAT: { using T = float; __VA_ARGS__; } break;\
+		case TCG_INT32: { using T = int32_t; __VA_ARGS__; } break;\
+		default: return tcg_fail(ctx, TCG_ERR_ARG, "unknown dtype %d", (int) (dtype));\
+	} } while (0)
+
+// 16-byte vector of T (compiler vector types: the non-temporal load/store
+// builtins take these, not the HIP float4 structs)
+typedef float tcg_f32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t tcg_i32x4 __attribute__((ext_vector_type(4)));
+typedef double tcg_f64x2 __attribute__((ext_vector_type(2)));
+template <typename T> struct Vec16;
+template <> struct Vec16<float> { using type = tcg_f32x4; static constexpr int N = 4; };
+template <> struct Vec16<int32_t> { using type = tcg_i32x4; static constexpr int N = 4; };
+template <> struct Vec16<double> { using type = tcg_f64x2; static constexpr int N = 2; };
+
+template <typename T>
+union VecU
+{
+	typename Vec16<T>::type v;
+	T e[Vec16<T>::N];
+};
+
+#endif // TCG_INTERNAL_HPP

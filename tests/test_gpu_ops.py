@@ -1,0 +1,515 @@
+"""GPU parity: every entry point of the C ABI against the CPU oracle on the
+same seeded inputs, and against the reference's golden vectors.
+
+Bars (BASELINE north_star): bit-exact for int32 ops and PERMUTE / SLICE / EXTEND
+(and the other pure data movement), 1e-5 relative for fp32 elementwise, 1e-4
+relative for fp32 reductions and contractions.  fp32 reductions/contractions are
+compared with the oracle accumulating in fp64, relative to max(|ref|, floor)
+where floor = mean |ref| of the output (individual sums of signed values can be
+arbitrarily close to zero).
+"""
+import json
+import os
+import zlib
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+with open(os.path.join(GOLDEN, "operator_goldens.json")) as f:
+    OPG = json.load(f)
+with open(os.path.join(GOLDEN, "equation_vectors.json")) as f:
+    EQV = json.load(f)
+
+def seed_of(*parts):
+    """Deterministic per-case seed (hash() of str is salted per process)."""
+    return zlib.crc32(repr(parts).encode())
+
+
+EW_RTOL = 1e-5
+ACC_RTOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from tenncor_amd import capi
+    c = capi.Context(0)
+    assert c.arch.startswith("gfx9"), c.arch
+    yield c
+    c.close()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tenncor_amd import ops as o
+    return o
+
+
+def assert_acc_close(got, ref, rtol=ACC_RTOL):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    floor = np.mean(np.abs(ref)) if ref.size else 0.0
+    denom = np.maximum(np.abs(ref), floor)
+    denom[denom == 0] = 1.0
+    err = np.abs(got - ref) / denom
+    assert err.max() <= rtol, "max rel err %.3g at %d (got %r ref %r)" % (
+        err.max(), err.argmax(), got.flat[err.argmax()], ref.flat[err.argmax()])
+
+
+def gpu_case(ops, ctx, case, np_dtype=np.float64):
+    op = case["op"]
+    args = [ops.from_host(ctx, np.asarray(a["data"], dtype=np_dtype), a["shape"]) for a in case["args"]]
+    if op in ("REDUCE_SUM", "REDUCE_PROD", "REDUCE_MIN", "REDUCE_MAX"):
+        out = ops.reduce(op, args[0], case["rank_set"])
+    elif op == "ARGMAX":
+        out = ops.argmax(args[0], case["rank"])
+    elif op == "EXTEND":
+        out = ops.extend(args[0], case["dimensions"])
+    elif op == "PERMUTE":
+        out = ops.permute(args[0], case["ranks"])
+    elif op == "SLICE":
+        out = ops.slice_(args[0], case["dimension_pairs"])
+    elif op == "PAD":
+        out = ops.pad(args[0], case["dimension_pairs"])
+    elif op == "STRIDE":
+        out = ops.stride(args[0], case["dimensions"])
+    elif op == "SCATTER":
+        out = ops.scatter(args[0], case["dimensions"], case["outshape"])
+    elif op == "REVERSE":
+        out = ops.reverse(args[0], case["rank_set"])
+    elif op == "CONCAT":
+        out = ops.concat(args, case["rank"])
+    elif op == "SELECT":
+        out = ops.select(*args)
+    elif op == "CONTRACT":
+        out = ops.contract(args[0], args[1], case["rank_pairs"])
+    elif op == "CONV":
+        out = ops.convolution(args[0], args[1], case["ranks"])
+    elif op in ("ADD", "MUL"):
+        out = ops.nary(op, args)
+    else:
+        out = ops.binary(op, args[0], args[1])
+    return out.get(), out.shape
+
+
+@pytest.mark.parametrize("case", OPG["cases"], ids=[c["name"] for c in OPG["cases"]])
+def test_reference_goldens_on_gpu(ctx, ops, oracle, case):
+    """internal/eigen/test/test_operator.cpp vectors, evaluated in double."""
+    got, shape = gpu_case(ops, ctx, case)
+    assert list(shape) == oracle.shape8(case["outshape"])
+    expect = np.asarray(case["expect"], dtype=np.float64)
+    if "tol" in case or case["op"] in ("POW", "DIV"):
+        np.testing.assert_allclose(got, expect, rtol=1e-13, atol=0)
+    else:
+        np.testing.assert_array_equal(got, expect)
+
+
+UNARY = ["ABS", "NEG", "SIN", "COS", "TAN", "EXP", "LOG", "SQRT", "ROUND", "SIGMOID", "TANH", "SQUARE", "CUBE"]
+BINARY = ["POW", "ADD", "SUB", "MUL", "DIV", "MIN", "MAX", "EQ", "NEQ", "LT", "GT"]
+
+
+@pytest.mark.parametrize("op", UNARY)
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32])
+def test_unary_vs_oracle(ctx, ops, oracle, op, np_dtype):
+    rng = np.random.default_rng(seed_of(op, str(np_dtype)))
+    n = 1000003  # odd: exercises the vector body and the scalar tail
+    if np_dtype == np.int32:
+        x = rng.integers(-30, 30, n).astype(np.int32)
+        if op in ("LOG", "SQRT"):
+            x = np.abs(x) + 1
+        if op in ("EXP",):
+            x = rng.integers(-5, 20, n).astype(np.int32)
+    else:
+        x = rng.uniform(-4, 4, n).astype(np_dtype)
+        if op in ("LOG", "SQRT"):
+            x = np.abs(x) + np_dtype(0.01)
+        if op == "TAN":
+            x = rng.uniform(-1.4, 1.4, n).astype(np_dtype)
+    t = ops.from_host(ctx, x, [n])
+    got = ops.unary(op, t).get()
+    ref = oracle.unary(op, x)
+    if np_dtype == np.int32:
+        if op in ("SIN", "COS", "TAN", "EXP", "LOG", "SQRT", "TANH"):
+            # double-precision libm on both sides, truncated: the integer part can
+            # differ only when the value sits within an ulp of an integer
+            assert np.mean(got != ref) < 1e-4
+        else:
+            np.testing.assert_array_equal(got, ref)
+    elif op in ("ABS", "NEG", "ROUND", "SQUARE", "CUBE", "SQRT"):
+        np.testing.assert_array_equal(got, ref)  # exactly rounded operations
+    else:
+        rtol = EW_RTOL if np_dtype == np.float32 else 1e-13
+        np.testing.assert_allclose(got, ref, rtol=rtol, atol=0)
+
+
+@pytest.mark.parametrize("op", BINARY)
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32])
+def test_binary_vs_oracle(ctx, ops, oracle, op, np_dtype):
+    rng = np.random.default_rng(seed_of(op, str(np_dtype), 2))
+    n = 777777
+    if np_dtype == np.int32:
+        a = rng.integers(-1000, 1000, n).astype(np.int32)
+        b = rng.integers(-1000, 1000, n).astype(np.int32)
+        if op == "MUL":
+            a = rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)  # wraps
+        if op == "DIV":
+            b[b == 0] = 7
+        if op == "POW":
+            a = rng.integers(-9, 9, n).astype(np.int32)
+            b = rng.integers(0, 9, n).astype(np.int32)
+    else:
+        a = rng.uniform(-3, 3, n).astype(np_dtype)
+        b = rng.uniform(-3, 3, n).astype(np_dtype)
+        if op == "POW":
+            a = np.abs(a) + np_dtype(0.1)
+        b[::7] = a[::7]  # some equal pairs for EQ/NEQ/MIN/MAX
+    ta, tb = ops.from_host(ctx, a, [n]), ops.from_host(ctx, b, [n])
+    got = ops.binary(op, ta, tb).get()
+    ref = oracle.binary(op, a, b)
+    if np_dtype == np.int32 or op not in ("POW",):
+        np.testing.assert_array_equal(got, ref)
+    else:
+        np.testing.assert_allclose(got, ref, rtol=EW_RTOL if np_dtype == np.float32 else 1e-13, atol=0)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32])
+@pytest.mark.parametrize("nargs", [3, 8, 11])
+def test_nary_left_fold(ctx, ops, oracle, np_dtype, nargs):
+    rng = np.random.default_rng(nargs)
+    n = 300001
+    if np_dtype == np.int32:
+        xs = [rng.integers(-2 ** 30, 2 ** 30, n).astype(np.int32) for _ in range(nargs)]
+    else:
+        xs = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(nargs)]
+    ts = [ops.from_host(ctx, x, [n]) for x in xs]
+    for op in ("ADD", "MUL"):
+        got = ops.nary(op, ts).get()
+        np.testing.assert_array_equal(got, oracle.nary(op, xs))  # same fold order: bit-exact
+
+
+def test_select_cast_assign(ctx, ops, oracle):
+    from tenncor_amd import capi
+    rng = np.random.default_rng(5)
+    n = 100003
+    c = (rng.uniform(size=n) < 0.5).astype(np.float32)
+    a = rng.standard_normal(n).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    tc, ta, tb = (ops.from_host(ctx, v, [n]) for v in (c, a, b))
+    np.testing.assert_array_equal(ops.select(tc, ta, tb).get(), oracle.select(c, a, b))
+    x = (a * 100).astype(np.float32)
+    for out_dtype in (capi.INT32, capi.DOUBLE, capi.FLOAT):
+        np.testing.assert_array_equal(ops.cast(ops.from_host(ctx, x, [n]), out_dtype).get(), oracle.cast(x, out_dtype))
+    xi = rng.integers(-10 ** 6, 10 ** 6, n).astype(np.int32)
+    np.testing.assert_array_equal(ops.cast(ops.from_host(ctx, xi, [n]), capi.FLOAT).get(), oracle.cast(xi, capi.FLOAT))
+    for op in ("ASSIGN", "ASSIGN_ADD", "ASSIGN_SUB", "ASSIGN_MUL", "ASSIGN_DIV"):
+        t = ops.from_host(ctx, a, [n])
+        ops.assign(op, t, tb)
+        ref = oracle.assign(op, a.copy(), b)
+        np.testing.assert_array_equal(t.get(), ref)
+
+
+def test_unaligned_operands_take_the_scalar_path(ctx, ops, oracle):
+    """Aliased last-dim slices give pointers that are not 16-byte aligned
+    (internal/eigen/operator.hpp:231-248)."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(9)
+    n = 4099
+    a = rng.standard_normal(n + 3).astype(np.float32)
+    b = rng.standard_normal(n + 3).astype(np.float32)
+    da, db = ctx.upload(a), ctx.upload(b)
+    out = ctx.empty(n + 3, np.float32)
+    ctx.ew_binary("ADD", capi.FLOAT, n, da.ptr + 4, db.ptr + 8, out.ptr + 12)
+    np.testing.assert_array_equal(out.get()[3:], oracle.binary("ADD", a[1:n + 1], b[2:n + 2]))
+    ctx.ew_unary("EXP", capi.FLOAT, n, da.ptr + 4, out.ptr)
+    np.testing.assert_allclose(out.get()[:n], oracle.unary("EXP", a[1:n + 1]), rtol=EW_RTOL)
+    ctx.reduce("REDUCE_SUM", capi.FLOAT, [n], [0], da.ptr + 4, out.ptr)
+    assert_acc_close(out.get()[:1], oracle.reduce("REDUCE_SUM", a[1:n + 1], [n], [0], wide_acc=True)[0])
+
+
+def test_fused_chain_equals_node_by_node(ctx, ops, oracle):
+    """config 2's chain ADD, MUL, EXP, TANH, SIGMOID in one pass over memory."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(2)
+    n = 1 << 20
+    a, b, c = (rng.uniform(-1, 1, n).astype(np.float32) for _ in range(3))
+    ta, tb, tc = (ops.from_host(ctx, v, [n]) for v in (a, b, c))
+    L = capi.OPD_LEAF0
+    prog = [("ADD", L + 0, L + 1, capi.OPD_ACC), ("MUL", capi.OPD_ACC, L + 2, capi.OPD_ACC),
+            ("EXP", capi.OPD_ACC, 0, capi.OPD_ACC), ("TANH", capi.OPD_ACC, 0, capi.OPD_ACC),
+            ("SIGMOID", capi.OPD_ACC, 0, capi.OPD_ACC)]
+    out = ctx.empty(n, np.float32)
+    ctx.ew_fused(capi.FLOAT, n, [ta.ptr, tb.ptr, tc.ptr], prog, out.ptr)
+    unfused = ops.unary("SIGMOID", ops.unary("TANH", ops.unary("EXP", ops.binary("MUL", ops.binary("ADD", ta, tb), tc))))
+    np.testing.assert_array_equal(out.get(), unfused.get())
+    ref = oracle.unary("SIGMOID", oracle.unary("TANH", oracle.unary("EXP", oracle.binary("MUL", oracle.binary("ADD", a, b), c))))
+    np.testing.assert_allclose(out.get(), ref, rtol=EW_RTOL)
+    # registers and immediates: sigmoid gradient  s * (1 - s) * g  with s = sigmoid(a)
+    prog = [("SIGMOID", L + 0, 0, capi.OPD_T0), ("SUB", capi.OPD_IMM, capi.OPD_T0, capi.OPD_ACC, 1.0),
+            ("MUL", capi.OPD_T0, capi.OPD_ACC, capi.OPD_ACC), ("MUL", capi.OPD_ACC, L + 1, capi.OPD_ACC)]
+    ctx.ew_fused(capi.FLOAT, n, [ta.ptr, tb.ptr], prog, out.ptr)
+    s = oracle.unary("SIGMOID", a)
+    ref = oracle.binary("MUL", oracle.binary("MUL", s, oracle.binary("SUB", np.ones(n, np.float32), s)), b)
+    np.testing.assert_allclose(out.get(), ref, rtol=EW_RTOL, atol=1e-12)
+    # int32 chain is bit-exact
+    ai, bi = (rng.integers(-1000, 1000, n).astype(np.int32) for _ in range(2))
+    tai, tbi = ops.from_host(ctx, ai, [n]), ops.from_host(ctx, bi, [n])
+    outi = ctx.empty(n, np.int32)
+    ctx.ew_fused(capi.INT32, n, [tai.ptr, tbi.ptr], [("ADD", L, L + 1, capi.OPD_ACC), ("MUL", capi.OPD_ACC, L + 1, capi.OPD_ACC),
+                                                      ("CUBE", capi.OPD_ACC, 0, capi.OPD_ACC)], outi.ptr)
+    np.testing.assert_array_equal(outi.get(), oracle.unary("CUBE", oracle.binary("MUL", oracle.binary("ADD", ai, bi), bi)))
+
+
+REDUCE_CASES = [
+    ([2048, 512], [0]), ([2048, 512], [1]), ([2048, 512], [0, 1]),
+    ([64, 20, 20, 16], [1, 2]), ([5, 7, 3, 4], [0, 2]), ([5, 7, 3, 4], [1, 3]), ([5, 7, 3, 4], [0, 1, 2, 3]),
+    ([3, 100000], [1]), ([100003], [0]), ([9, 3], [1]), ([1, 1, 300, 1, 77], [2]), ([33, 1, 17], [0, 2]),
+    ([1 << 22], [0]), ([6, 5, 4, 3, 2, 2, 3, 2], [0, 2, 4, 6]), ([6, 5, 4, 3, 2, 2, 3, 2], [1, 3, 5, 7]),
+]
+
+
+@pytest.mark.parametrize("shape,ranks", REDUCE_CASES, ids=[str(c) for c in REDUCE_CASES])
+def test_reduce_vs_oracle(ctx, ops, oracle, shape, ranks):
+    rng = np.random.default_rng(seed_of(shape, ranks))
+    n = oracle.n_elems(shape)
+    xf = rng.uniform(-1, 1, n).astype(np.float32)
+    xi = rng.integers(-1000, 1000, n).astype(np.int32) * rng.integers(-1000, 1000, n).astype(np.int32)
+    tf, ti = ops.from_host(ctx, xf, shape), ops.from_host(ctx, xi, shape)
+    for op in ("REDUCE_SUM", "REDUCE_MAX", "REDUCE_MIN"):
+        out = ops.reduce(op, tf, ranks)
+        ref, oshape = oracle.reduce(op, xf, shape, ranks, wide_acc=True)
+        assert out.shape == oshape
+        if op == "REDUCE_SUM":
+            assert_acc_close(out.get(), ref)
+        else:
+            np.testing.assert_array_equal(out.get(), ref)
+        # int32: wrap-around sums are order independent, so bit-exact
+        np.testing.assert_array_equal(ops.reduce(op, ti, ranks).get(), oracle.reduce(op, xi, shape, ranks)[0])
+    xd = rng.uniform(0.999, 1.001, n)  # keeps products of millions of values in range
+    got = ops.reduce("REDUCE_PROD", ops.from_host(ctx, xd, shape), ranks).get()
+    np.testing.assert_allclose(got, oracle.reduce("REDUCE_PROD", xd, shape, ranks)[0], rtol=1e-9)
+
+
+def test_argmax_vs_oracle(ctx, ops, oracle):
+    rng = np.random.default_rng(4)
+    shape = [7, 50, 9]
+    x = rng.integers(-50, 50, oracle.n_elems(shape)).astype(np.float32)  # ties on purpose
+    t = ops.from_host(ctx, x, shape)
+    for rd in (0, 1, 2, 8):
+        np.testing.assert_array_equal(ops.argmax(t, rd).get(), oracle.argmax(x, shape, rd)[0])
+
+
+def movement_cases(oracle, ops, rng):
+    """(name, gpu thunk, oracle thunk) over int32 payloads: all bit-exact."""
+    cases = []
+
+    def add(name, shape, gfn, ofn):
+        cases.append((name, shape, gfn, ofn))
+
+    add("permute_2d", [300, 200], lambda t: ops.permute(t, [1, 0]), lambda x, s: oracle.permute(x, s, [1, 0]))
+    add("permute_batched", [70, 130, 5], lambda t: ops.permute(t, [1, 0, 2]), lambda x, s: oracle.permute(x, s, [1, 0, 2]))
+    add("permute_rot", [20, 30, 40], lambda t: ops.permute(t, [2, 0, 1]), lambda x, s: oracle.permute(x, s, [2, 0, 1]))
+    add("permute_inner_kept", [64, 5, 7, 3], lambda t: ops.permute(t, [0, 2, 1, 3]), lambda x, s: oracle.permute(x, s, [0, 2, 1, 3]))
+    add("permute_conv2d", [1, 20, 18, 6, 32], lambda t: ops.permute(t, [4, 1, 2, 3]), lambda x, s: oracle.permute(x, s, [4, 1, 2, 3]))
+    add("permute_small", [3, 4, 5], lambda t: ops.permute(t, [2, 1, 0]), lambda x, s: oracle.permute(x, s, [2, 1, 0]))
+    add("extend_bias", [9, 1], lambda t: ops.extend(t, [1, 300]), lambda x, s: oracle.extend(x, s, [1, 300]))
+    add("extend_scalar", [1], lambda t: ops.extend(t, [32, 24, 24, 8]), lambda x, s: oracle.extend(x, s, [32, 24, 24, 8]))
+    add("extend_mid", [16, 1, 5, 1], lambda t: ops.extend(t, [1, 33, 1, 4]), lambda x, s: oracle.extend(x, s, [1, 33, 1, 4]))
+    add("extend_inner", [1, 77], lambda t: ops.extend(t, [130]), lambda x, s: oracle.extend(x, s, [130]))
+    add("slice_seq", [256, 64, 16], lambda t: ops.slice_(t, [[0, 256], [5, 1]]), lambda x, s: oracle.slice_(x, s, [[0, 256], [5, 1]]))
+    add("slice_gate", [2048, 1, 16], lambda t: ops.slice_(t, [[512, 512]]), lambda x, s: oracle.slice_(x, s, [[512, 512]]))
+    add("slice_odd", [37, 11, 5], lambda t: ops.slice_(t, [[3, 30], [2, 100], [1, 3]]), lambda x, s: oracle.slice_(x, s, [[3, 30], [2, 100], [1, 3]]))
+    add("pad_dim4", [4, 10, 9, 2], lambda t: ops.pad(t, [[0, 0]] * 4 + [[2, 2]]), lambda x, s: oracle.pad(x, s, [[0, 0]] * 4 + [[2, 2]]))
+    add("pad_inner", [16, 7], lambda t: ops.pad(t, [[4, 8], [1, 0]]), lambda x, s: oracle.pad(x, s, [[4, 8], [1, 0]]))
+    add("pad_odd", [5, 6, 3], lambda t: ops.pad(t, [[1, 2], [0, 3], [2, 0]]), lambda x, s: oracle.pad(x, s, [[1, 2], [0, 3], [2, 0]]))
+    add("reverse_0", [32, 4, 5, 6], lambda t: ops.reverse(t, [0]), lambda x, s: oracle.reverse(x, s, [0]))
+    add("reverse_all", [8, 4, 5, 6], lambda t: ops.reverse(t, [0, 1, 2, 3]), lambda x, s: oracle.reverse(x, s, [0, 1, 2, 3]))
+    add("stride", [17, 9, 4], lambda t: ops.stride(t, [2, 3]), lambda x, s: oracle.stride(x, s, [2, 3]))
+    add("scatter", [9, 3, 4], lambda t: ops.scatter(t, [2, 3], [17, 9, 4]), lambda x, s: oracle.scatter(x, s, [2, 3], [17, 9, 4]))
+    return cases
+
+
+def test_data_movement_bit_exact(ctx, ops, oracle):
+    rng = np.random.default_rng(12)
+    for name, shape, gfn, ofn in movement_cases(oracle, ops, rng):
+        n = oracle.n_elems(shape)
+        for np_dtype in (np.int32, np.float64):
+            x = rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+            if np_dtype == np.float64:
+                x = rng.standard_normal(n)
+            out = gfn(ops.from_host(ctx, x, shape))
+            ref, oshape = ofn(x, shape)
+            assert out.shape == oracle.shape8(oshape), name
+            np.testing.assert_array_equal(out.get(), ref, err_msg=name)
+
+
+def test_concat_bit_exact(ctx, ops, oracle):
+    rng = np.random.default_rng(13)
+    sa, sb = [256, 1, 16], [512, 1, 16]
+    a = rng.standard_normal(oracle.n_elems(sa)).astype(np.float32)
+    b = rng.standard_normal(oracle.n_elems(sb)).astype(np.float32)
+    out = ops.concat([ops.from_host(ctx, a, sa), ops.from_host(ctx, b, sb)], 0)
+    ref, oshape = oracle.concat([a, b], [sa, sb], 0)
+    assert out.shape == oshape
+    np.testing.assert_array_equal(out.get(), ref)
+    # n-ary form along the sequence dim
+    shapes = [[48, 1, 5]] * 9
+    xs = [rng.integers(-99, 99, 240).astype(np.int32) for _ in shapes]
+    out = ops.concat([ops.from_host(ctx, x, s) for x, s in zip(xs, shapes)], 1)
+    ref, oshape = oracle.concat(xs, shapes, 1)
+    assert out.shape == oshape
+    np.testing.assert_array_equal(out.get(), ref)
+
+
+MATMUL_CASES = [
+    ([10, 3], [9, 10]), ([64, 64], [64, 64]), ([100, 37], [53, 100]), ([256, 128], [192, 256]),
+    ([768, 256], [2048, 768]), ([32, 48, 5], [40, 32, 5]), ([128, 128, 3, 2], [128, 128, 3, 2]),
+    ([513, 130], [259, 513]), ([1024, 512], [512, 1024]),
+]
+
+
+@pytest.mark.parametrize("ashape,bshape", MATMUL_CASES, ids=[str(c) for c in MATMUL_CASES])
+def test_matmul_vs_oracle(ctx, ops, oracle, ashape, bshape):
+    rng = np.random.default_rng(seed_of(ashape, bshape))
+    a = rng.standard_normal(oracle.n_elems(ashape)).astype(np.float32)
+    b = (rng.standard_normal(oracle.n_elems(bshape)) / np.sqrt(ashape[0])).astype(np.float32)
+    out = ops.matmul(ops.from_host(ctx, a, ashape), ops.from_host(ctx, b, bshape))
+    ref, oshape = oracle.matmul(a, ashape, b, bshape, wide_acc=True)
+    assert out.shape == oshape
+    assert_acc_close(out.get(), ref)
+    if oracle.n_elems(ashape) <= 1 << 16:
+        ai = rng.integers(-2 ** 15, 2 ** 15, oracle.n_elems(ashape)).astype(np.int32)
+        bi = rng.integers(-2 ** 15, 2 ** 15, oracle.n_elems(bshape)).astype(np.int32)
+        outi = ops.matmul(ops.from_host(ctx, ai, ashape), ops.from_host(ctx, bi, bshape))
+        np.testing.assert_array_equal(outi.get(), oracle.matmul(ai, ashape, bi, bshape)[0])  # wraps, exact
+        ad, bd = a.astype(np.float64), b.astype(np.float64)
+        outd = ops.matmul(ops.from_host(ctx, ad, ashape), ops.from_host(ctx, bd, bshape))
+        np.testing.assert_allclose(outd.get(), oracle.matmul(ad, ashape, bd, bshape)[0], rtol=1e-10, atol=1e-12)
+
+
+CONTRACT_CASES = [
+    ([10, 3], [9, 10], [[0, 1]]),                      # dense layer (config 1)
+    ([768, 1, 64], [512, 768], [[0, 1]]),              # LSTM gate product (config 4)
+    ([64, 1, 1, 32], [10, 64], [[0, 1]]),              # CNN dense head (config 5)
+    ([4, 2, 3], [2, 4, 2], [[0, 1], [1, 2]]),          # reference golden shape
+    ([12, 7], [12, 9], [[0, 0]]),                      # both contracted-inner
+    ([7, 12], [9, 12], [[1, 1]]),                      # both contracted-outer
+    ([7, 12], [12, 9], [[1, 0]]),
+    ([5, 6, 7], [6, 4], [[1, 0]]),                     # a needs repacking
+    ([5, 6, 7], [7, 3, 5], [[0, 2], [2, 0]]),          # b's order differs
+    ([3, 4, 5, 6], [5, 2, 3], [[0, 2], [2, 0]]),
+]
+
+
+@pytest.mark.parametrize("ashape,bshape,pairs", CONTRACT_CASES, ids=[str(c) for c in CONTRACT_CASES])
+def test_contract_vs_oracle(ctx, ops, oracle, ashape, bshape, pairs):
+    rng = np.random.default_rng(seed_of(ashape, bshape))
+    a = rng.standard_normal(oracle.n_elems(ashape)).astype(np.float32)
+    b = rng.standard_normal(oracle.n_elems(bshape)).astype(np.float32)
+    out = ops.contract(ops.from_host(ctx, a, ashape), ops.from_host(ctx, b, bshape), pairs)
+    ref, oshape = oracle.contract(a, ashape, b, bshape, pairs, wide_acc=True)
+    assert out.shape == oshape
+    assert_acc_close(out.get(), ref)
+    ai = rng.integers(-999, 999, a.size).astype(np.int32)
+    bi = rng.integers(-999, 999, b.size).astype(np.int32)
+    outi = ops.contract(ops.from_host(ctx, ai, ashape), ops.from_host(ctx, bi, bshape), pairs)
+    np.testing.assert_array_equal(outi.get(), oracle.contract(ai, ashape, bi, bshape, pairs)[0])
+
+
+CONV_CASES = [
+    ([3, 3], [2], [1]),
+    ([2, 4, 3, 3], [1, 2, 2, 1], list(range(8))),            # tenncor/test/test_api.cpp:2265
+    ([1, 12, 12, 4, 5], [3, 1, 5, 5], [4, 0, 1, 2]),          # conv2d idiom, small
+    ([4, 10, 9, 2, 5], [3, 4, 5, 6], [4, 0, 1, 2]),           # tenncor/test/test_api.cpp:2505 shapes
+    ([4, 10, 9, 2, 5], [1, 6, 4, 2, 3], list(range(8))),      # kernel-gradient form
+    ([20, 16], [5, 3], [0, 1]),
+]
+
+
+@pytest.mark.parametrize("ishape,kshape,ranks", CONV_CASES, ids=[str(c) for c in CONV_CASES])
+def test_conv_vs_oracle(ctx, ops, oracle, ishape, kshape, ranks):
+    rng = np.random.default_rng(seed_of(ishape, kshape))
+    img = rng.uniform(-1, 1, oracle.n_elems(ishape)).astype(np.float32)
+    ker = rng.uniform(-1, 1, oracle.n_elems(kshape)).astype(np.float32)
+    out = ops.convolution(ops.from_host(ctx, img, ishape), ops.from_host(ctx, ker, kshape), ranks)
+    ref, oshape = oracle.conv(img, ishape, ker, kshape, ranks, wide_acc=True)
+    assert out.shape == oshape
+    assert_acc_close(out.get(), ref)
+    ii = rng.integers(-99, 99, img.size).astype(np.int32)
+    ki = rng.integers(-99, 99, ker.size).astype(np.int32)
+    outi = ops.convolution(ops.from_host(ctx, ii, ishape), ops.from_host(ctx, ki, kshape), ranks)
+    np.testing.assert_array_equal(outi.get(), oracle.conv(ii, ishape, ki, kshape, ranks)[0])
+
+
+def test_api_convolution_golden_on_gpu(ctx, ops):
+    fx = EQV["api_convolution"]
+    out = ops.convolution(ops.from_host(ctx, np.array(fx["data"]), fx["alist"]),
+                          ops.from_host(ctx, np.array(fx["data2"]), fx["blist"]), list(range(8)))
+    assert out.shape == fx["expectslist"]
+    np.testing.assert_array_equal(out.get(), np.array(fx["expect_out"]))
+
+
+def test_matmul_chain_golden_on_gpu(ctx, ops):
+    """tenncor/test/test_equation.cpp:26-87 in double."""
+    fx = EQV["matmul_complex"]
+    a, b, c = (ops.from_host(ctx, np.array(fx[k]), fx[s]) for k, s in (("data", "alist"), ("data2", "blist"), ("data3", "clist")))
+    d = ops.matmul(a, b)
+    e = ops.matmul(c, d)
+    f = ops.matmul(ops.permute(d, [1, 0]), ops.permute(c, [1, 0]))
+    dest = ops.matmul(e, f)
+    np.testing.assert_allclose(dest.get(), np.array(fx["expect_dest"]), rtol=1e-14)
+
+
+def test_errors_are_reported_not_thrown_across_the_abi(ctx, ops):
+    from tenncor_amd import capi
+    a = ops.from_host(ctx, np.zeros(12, np.float32), [4, 3])
+    with pytest.raises(capi.TcgError) as info:
+        ctx.extend(capi.FLOAT, [4, 3], [2, 1], a.ptr, a.ptr)
+    assert "non-singular" in str(info.value)
+    with pytest.raises(capi.TcgError):
+        ctx.permute(capi.FLOAT, [4, 3], [0, 0, 2, 3, 4, 5, 6, 7], a.ptr, a.ptr)
+    with pytest.raises(capi.TcgError):
+        ctx.ew_unary("ADD", capi.FLOAT, 12, a.ptr, a.ptr)
+    with pytest.raises(capi.TcgError):
+        ctx.ew_unary("EXP", 9, 12, a.ptr, a.ptr)
+
+
+def test_pool_recycles_blocks(ctx):
+    in_use0, _ = ctx.mem_stats()
+    p = ctx.alloc(1 << 20)
+    ctx.free(p, 1 << 20)
+    q = ctx.alloc(1 << 20)
+    assert q == p  # stream-ordered reuse without going back to the driver
+    ctx.free(q, 1 << 20)
+    assert ctx.mem_stats()[0] == in_use0
+
+
+def test_full_size_properties_config2(ctx, ops):
+    """[4096,16384] tensors: properties that need no CPU pass over 256 MiB."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(2)
+    shape = [16384, 4096]
+    n = 16384 * 4096
+    xi = rng.integers(-1000, 1001, n, dtype=np.int32)
+    yi = rng.integers(-1000, 1001, n, dtype=np.int32)
+    tx, ty = ops.from_host(ctx, xi, shape), ops.from_host(ctx, yi, shape)
+    prod = ops.binary("MUL", ops.binary("ADD", tx, ty), ty)
+    # checksum of checksums: reducing dim 0 then dim 1 == reducing dim 1 then dim 0 == all at once
+    r0 = ops.reduce("REDUCE_SUM", ops.reduce("REDUCE_SUM", prod, [0]), [1]).get()
+    r1 = ops.reduce("REDUCE_SUM", ops.reduce("REDUCE_SUM", prod, [1]), [0]).get()
+    rall = ops.reduce("REDUCE_SUM", prod, [0, 1]).get()
+    want = np.int64(((xi.astype(np.int64) + yi) * yi).sum()).astype(np.int32)  # mod 2^32
+    assert r0[0] == r1[0] == rall[0] == want
+    m0 = ops.reduce("REDUCE_MAX", ops.reduce("REDUCE_MAX", prod, [0]), [1]).get()
+    assert m0[0] == ops.reduce("REDUCE_MAX", prod, [0, 1]).get()[0] == ((xi.astype(np.int64) + yi) * yi).max()
+    # row sums against numpy on the first and last rows
+    rows = ops.reduce("REDUCE_SUM", prod, [0]).get()
+    p_host = ((xi.astype(np.int64) + yi) * yi).astype(np.int32).reshape(4096, 16384)
+    np.testing.assert_array_equal(rows, p_host.sum(axis=1, dtype=np.int32))
+    cols = ops.reduce("REDUCE_SUM", prod, [1]).get()
+    np.testing.assert_array_equal(cols, p_host.sum(axis=0, dtype=np.int32))
+    # PERMUTE twice is the identity; a transposed row is a column
+    tt = ops.permute(ops.permute(prod, [1, 0]), [1, 0])
+    np.testing.assert_array_equal(tt.get(), p_host.reshape(-1))
+    np.testing.assert_array_equal(ops.permute(prod, [1, 0]).get().reshape(16384, 4096)[5], p_host[:, 5])
