@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the operator hot path on one MI355X.
+
+Workload (BASELINE.json configs[1], "elementwise+reduce microbench"): fp32 and
+int32 tensors np[4096,16384] (tenncor shape {16384,4096}).  One step evaluates,
+node by node as the reference does (every node materialises its output):
+  fp32 : t1=ADD(a,b) t2=MUL(t1,c) t3=EXP(t2) t4=TANH(t3) t5=SIGMOID(t4),
+         REDUCE_SUM and REDUCE_MAX of t5 over dim 0 and over dim 1
+  int32: u1=ADD(x,y) u2=MUL(u1,z), REDUCE_SUM and REDUCE_MAX of u2 over each dim
+`value` = algorithmic bytes of one step / time of one step, inputs resident in
+HBM before the timed region.  Per-kernel durations are taken with HIP events
+recorded on the launch stream inside the timed region.
+
+Prints ONE JSON line.  Everything runs on one GPU; --gpus > 1 is refused.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
+MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+
+ROWS, COLS = 4096, 16384
+N = ROWS * COLS
+SHAPE = [COLS, ROWS]  # tenncor order: dim 0 fastest
+
+# HBM bytes per launch of the dominant kernel from `rocprofv3 --pmc` runs
+# (FETCH_SIZE + WRITE_SIZE scaled by a plain copy kernel); None until measured.
+MEASURED_TRAFFIC = {}
+
+
+def algorithmic_bytes():
+    """Per-kernel algorithmic bytes of one step (4-byte elements)."""
+    e = 4
+    return {
+        "ew_binary_f32": 2 * 3 * e * N,                 # ADD, MUL
+        "ew_unary_f32": 3 * 2 * e * N,                  # EXP, TANH, SIGMOID
+        "reduce_dim0_f32": 2 * (e * N + e * ROWS),      # SUM, MAX -> {1,4096}
+        "reduce_dim1_f32": 2 * (e * N + e * COLS),      # SUM, MAX -> {16384,1}
+        "ew_binary_i32": 2 * 3 * e * N,
+        "reduce_dim0_i32": 2 * (e * N + e * ROWS),
+        "reduce_dim1_i32": 2 * (e * N + e * COLS),
+    }
+
+
+class Step:
+    """Device-resident inputs and outputs of the config-2 graph."""
+
+    def __init__(self, ctx, seed=2):
+        from tenncor_amd import capi
+        self.ctx, self.capi = ctx, capi
+        rng = np.random.default_rng(seed)
+        self.f = [ctx.upload(rng.uniform(-1, 1, N).astype(np.float32)) for _ in range(3)]
+        self.i = [ctx.upload(rng.integers(-1000, 1001, N, dtype=np.int32)) for _ in range(3)]
+        self.t = [ctx.empty(N, np.float32) for _ in range(5)]
+        self.u = [ctx.empty(N, np.int32) for _ in range(2)]
+        self.rf = [ctx.empty(ROWS, np.float32), ctx.empty(ROWS, np.float32),
+                   ctx.empty(COLS, np.float32), ctx.empty(COLS, np.float32)]
+        self.ri = [ctx.empty(ROWS, np.int32), ctx.empty(ROWS, np.int32),
+                   ctx.empty(COLS, np.int32), ctx.empty(COLS, np.int32)]
+
+    def launches(self):
+        """(kernel class, thunk) in evaluation order."""
+        c, F, I = self.ctx, self.capi.FLOAT, self.capi.INT32
+        f, t, rf, i, u, ri = self.f, self.t, self.rf, self.i, self.u, self.ri
+        return [
+            ("ew_binary_f32", lambda: c.ew_binary("ADD", F, N, f[0].ptr, f[1].ptr, t[0].ptr)),
+            ("ew_binary_f32", lambda: c.ew_binary("MUL", F, N, t[0].ptr, f[2].ptr, t[1].ptr)),
+            ("ew_unary_f32", lambda: c.ew_unary("EXP", F, N, t[1].ptr, t[2].ptr)),
+            ("ew_unary_f32", lambda: c.ew_unary("TANH", F, N, t[2].ptr, t[3].ptr)),
+            ("ew_unary_f32", lambda: c.ew_unary("SIGMOID", F, N, t[3].ptr, t[4].ptr)),
+            ("reduce_dim0_f32", lambda: c.reduce("REDUCE_SUM", F, SHAPE, [0], t[4].ptr, rf[0].ptr)),
+            ("reduce_dim0_f32", lambda: c.reduce("REDUCE_MAX", F, SHAPE, [0], t[4].ptr, rf[1].ptr)),
+            ("reduce_dim1_f32", lambda: c.reduce("REDUCE_SUM", F, SHAPE, [1], t[4].ptr, rf[2].ptr)),
+            ("reduce_dim1_f32", lambda: c.reduce("REDUCE_MAX", F, SHAPE, [1], t[4].ptr, rf[3].ptr)),
+            ("ew_binary_i32", lambda: c.ew_binary("ADD", I, N, i[0].ptr, i[1].ptr, u[0].ptr)),
+            ("ew_binary_i32", lambda: c.ew_binary("MUL", I, N, u[0].ptr, i[2].ptr, u[1].ptr)),
+            ("reduce_dim0_i32", lambda: c.reduce("REDUCE_SUM", I, SHAPE, [0], u[1].ptr, ri[0].ptr)),
+            ("reduce_dim0_i32", lambda: c.reduce("REDUCE_MAX", I, SHAPE, [0], u[1].ptr, ri[1].ptr)),
+            ("reduce_dim1_i32", lambda: c.reduce("REDUCE_SUM", I, SHAPE, [1], u[1].ptr, ri[2].ptr)),
+            ("reduce_dim1_i32", lambda: c.reduce("REDUCE_MAX", I, SHAPE, [1], u[1].ptr, ri[3].ptr)),
+        ]
+
+
+def run_gpu(steps, warmup):
+    from tenncor_amd import capi
+    ctx = capi.Context(0)
+    st = Step(ctx)
+    launches = st.launches()
+    for _ in range(warmup):
+        for _, fn in launches:
+            fn()
+    ctx.sync()
+    # one event before and after every launch, all on the launch stream
+    events = [[ctx.event() for _ in range(len(launches) + 1)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s in range(steps):
+        ctx.record(events[s][0])
+        for k, (_, fn) in enumerate(launches):
+            fn()
+            ctx.record(events[s][k + 1])
+    ctx.sync()
+    wall = time.perf_counter() - t0
+    per_class = {}
+    for s in range(steps):
+        for k, (name, _) in enumerate(launches):
+            per_class.setdefault(name, []).append(ctx.elapsed_ms(events[s][k], events[s][k + 1]))
+    for evs in events:
+        for ev in evs:
+            ctx.event_destroy(ev)
+    extra = run_extras(ctx, capi)
+    arch = ctx.arch
+    ctx.close()
+    return wall, per_class, extra, arch
+
+
+def run_extras(ctx, capi):
+    """Side metrics of BASELINE's metric triple: fused chain, fp32 MATMUL."""
+    extra = {}
+    # fused chain: 3 leaf reads + 1 write
+    rng = np.random.default_rng(22)
+    leaves = [ctx.upload(rng.uniform(-1, 1, N).astype(np.float32)) for _ in range(3)]
+    out = ctx.empty(N, np.float32)
+    L = capi.OPD_LEAF0
+    prog = [("ADD", L, L + 1, capi.OPD_ACC), ("MUL", capi.OPD_ACC, L + 2, capi.OPD_ACC),
+            ("EXP", capi.OPD_ACC, 0, capi.OPD_ACC), ("TANH", capi.OPD_ACC, 0, capi.OPD_ACC),
+            ("SIGMOID", capi.OPD_ACC, 0, capi.OPD_ACC)]
+    for _ in range(2):
+        ctx.ew_fused(capi.FLOAT, N, [b.ptr for b in leaves], prog, out.ptr)
+    ctx.timer_begin()
+    reps = 10
+    for _ in range(reps):
+        ctx.ew_fused(capi.FLOAT, N, [b.ptr for b in leaves], prog, out.ptr)
+    ms = ctx.timer_end() / reps
+    extra["fused_chain_GBps"] = round(4 * 4 * N / (ms * 1e-3) / 1e9, 1)
+    extra["fused_chain_ms"] = round(ms, 4)
+    for b in leaves + [out]:
+        b.release()
+    # 4096^3 fp32 MATMUL (configs[2])
+    M = 4096
+    a = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
+    b = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
+    c = ctx.empty(M * M, np.float32)
+    for _ in range(2):
+        ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
+    ctx.timer_begin()
+    reps = 5
+    for _ in range(reps):
+        ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
+    ms = ctx.timer_end() / reps
+    tf = 2.0 * M ** 3 / (ms * 1e-3) / 1e12
+    extra["matmul_4096_fp32_TFLOPs"] = round(tf, 2)
+    extra["matmul_4096_fp32_ms"] = round(ms, 4)
+    extra["matmul_4096_frac_of_fp32_mfma_peak"] = round(tf / MFMA_F32_PEAK_TFLOPS, 4)
+    # PERMUTE of the result (HBM-bound)
+    d = ctx.empty(M * M, np.float32)
+    order = [1, 0, 2, 3, 4, 5, 6, 7]
+    for _ in range(2):
+        ctx.permute(capi.FLOAT, [M, M], order, c.ptr, d.ptr)
+    ctx.timer_begin()
+    for _ in range(reps):
+        ctx.permute(capi.FLOAT, [M, M], order, c.ptr, d.ptr)
+    ms = ctx.timer_end() / reps
+    extra["permute_4096_GBps"] = round(2 * 4 * M * M / (ms * 1e-3) / 1e9, 1)
+    for buf in (a, b, c, d):
+        buf.release()
+    return extra
+
+
+def run_cpu_baseline():
+    """The oracle (a scalar C port of the reference semantics) on one host core,
+    on a row slab of the same workload sized for roughly 10-30 s."""
+    from oracle import oracle as orc
+    orc.build()
+    rows = ROWS  # the whole tensor: about 15 s on one core
+    n = rows * COLS
+    shape = [COLS, rows]
+    rng = np.random.default_rng(2)
+    f = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(3)]
+    i = [rng.integers(-1000, 1001, n, dtype=np.int32) for _ in range(3)]
+    e = 4
+    nbytes = (2 * 3 + 3 * 2) * e * n + 2 * (e * n + e * rows) + 2 * (e * n + e * COLS)
+    nbytes += 2 * 3 * e * n + 2 * (e * n + e * rows) + 2 * (e * n + e * COLS)
+    passes = 0
+    t0 = time.perf_counter()
+    while passes < 1 or (time.perf_counter() - t0 < 10.0 and passes < 16):
+        t = orc.binary("ADD", f[0], f[1])
+        t = orc.binary("MUL", t, f[2])
+        t = orc.unary("EXP", t)
+        t = orc.unary("TANH", t)
+        t = orc.unary("SIGMOID", t)
+        for op in ("REDUCE_SUM", "REDUCE_MAX"):
+            orc.reduce(op, t, shape, [0])
+            orc.reduce(op, t, shape, [1])
+        u = orc.binary("ADD", i[0], i[1])
+        u = orc.binary("MUL", u, i[2])
+        for op in ("REDUCE_SUM", "REDUCE_MAX"):
+            orc.reduce(op, u, shape, [0])
+            orc.reduce(op, u, shape, [1])
+        passes += 1
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(passes * nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": "the same graph on np[%d,%d] (the whole workload), %d passes, %.1f s single-thread"
+                  % (rows, COLS, passes, dt),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs on one GPU; --gpus %d is not supported "
+                 "(no collectives or sharding are part of this build)" % args.gpus)
+
+    wall, per_class, extra, arch = run_gpu(args.steps, args.warmup)
+    abytes = algorithmic_bytes()
+    launches_per_step = {"ew_binary_f32": 2, "ew_unary_f32": 3, "reduce_dim0_f32": 2, "reduce_dim1_f32": 2,
+                         "ew_binary_i32": 2, "reduce_dim0_i32": 2, "reduce_dim1_i32": 2}
+    total_bytes = sum(abytes.values())
+    ms_per_step = wall * 1e3 / args.steps
+    value = total_bytes / (wall / args.steps) / 1e9
+    kernels = {}
+    for name, times in per_class.items():
+        avg_ms = float(np.mean(times))
+        per_launch = abytes[name] / launches_per_step[name]
+        kernels[name] = {"avg_ms": round(avg_ms, 4), "GBps": round(per_launch / (avg_ms * 1e-3) / 1e9, 1),
+                         "frac": round(per_launch / (avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    dominant = max(kernels, key=lambda k: kernels[k]["avg_ms"] * launches_per_step[k])
+    dom = kernels[dominant]
+    result = {
+        "metric": "graph evals/sec; elementwise+reduce HBM GB/s; fp32 MATMUL TFLOP/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32+i32", "data": "synthetic",
+        "config": {"workload": "configs[1]: elementwise+reduce microbench, fp32 and int32 np[4096,16384], "
+                               "node-by-node (ADD,MUL,EXP,TANH,SIGMOID + REDUCE_SUM/MAX over each dim; "
+                               "int32 ADD,MUL + the same reductions)",
+                   "algorithmic_bytes_per_step": total_bytes, "device": arch},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get(dominant)},
+        "kernels": kernels,
+        "extra": extra,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = run_cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -103,6 +103,12 @@ int tcg_sync (tcg_ctx* ctx);
  * the milliseconds between them. */
 int tcg_timer_begin (tcg_ctx* ctx);
 int tcg_timer_end (tcg_ctx* ctx, float* ms);
+/* Non-blocking variant: events recorded on the context's stream between
+ * launches; tcg_event_elapsed waits for `stop` and returns stop - start. */
+int tcg_event_create (tcg_ctx* ctx, void** event);
+int tcg_event_destroy (tcg_ctx* ctx, void* event);
+int tcg_event_record (tcg_ctx* ctx, void* event);
+int tcg_event_elapsed (tcg_ctx* ctx, void* start, void* stop, float* ms);
 
 /* ---- elementwise ------------------------------------------------------ */
 

@@ -54,9 +54,14 @@ def build_libtcg(jobs=8, verbose=False):
     return LIBTCG
 
 
+def build_all(verbose=False):
+    """Everything native in this package."""
+    return [build_libtcg(verbose=verbose)]
+
+
 def main():
-    path = build_libtcg(verbose=True)
-    print("built", path)
+    for path in build_all(verbose=True):
+        print("built", path)
     return 0
 
 

@@ -33,7 +33,8 @@ OPD_NONE, OPD_ACC, OPD_T0, OPD_T1, OPD_IMM, OPD_LEAF0 = 0, 1, 2, 3, 4, 8
 EXPORTS = [
     "tcg_ctx_create", "tcg_ctx_destroy", "tcg_last_error", "tcg_device_arch", "tcg_alloc", "tcg_free",
     "tcg_mem_stats", "tcg_h2d", "tcg_d2h", "tcg_d2d", "tcg_fill_zero", "tcg_sync", "tcg_timer_begin",
-    "tcg_timer_end", "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
+    "tcg_timer_end", "tcg_event_create", "tcg_event_destroy", "tcg_event_record", "tcg_event_elapsed",
+    "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
     "tcg_gemm", "tcg_conv",
@@ -78,6 +79,10 @@ def load():
         "tcg_sync": [vp],
         "tcg_timer_begin": [vp],
         "tcg_timer_end": [vp, ctypes.POINTER(ctypes.c_float)],
+        "tcg_event_create": [vp, ctypes.POINTER(vp)],
+        "tcg_event_destroy": [vp, vp],
+        "tcg_event_record": [vp, vp],
+        "tcg_event_elapsed": [vp, vp, vp, ctypes.POINTER(ctypes.c_float)],
         "tcg_ew_unary": [vp, i32, i32, u64, vp, vp],
         "tcg_ew_binary": [vp, i32, i32, u64, vp, vp, vp],
         "tcg_ew_nary": [vp, i32, i32, u64, i32, vpp, vp],
@@ -225,6 +230,22 @@ class Context:
     def timer_end(self):
         ms = ctypes.c_float()
         self._check(self.lib.tcg_timer_end(self.handle, ctypes.byref(ms)))
+        return ms.value
+
+    def event(self):
+        ev = ctypes.c_void_p()
+        self._check(self.lib.tcg_event_create(self.handle, ctypes.byref(ev)))
+        return ev.value
+
+    def event_destroy(self, ev):
+        self._check(self.lib.tcg_event_destroy(self.handle, ev))
+
+    def record(self, ev):
+        self._check(self.lib.tcg_event_record(self.handle, ev))
+
+    def elapsed_ms(self, start, stop):
+        ms = ctypes.c_float()
+        self._check(self.lib.tcg_event_elapsed(self.handle, start, stop, ctypes.byref(ms)))
         return ms.value
 
     # ---- elementwise ----

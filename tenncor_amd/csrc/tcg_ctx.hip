@@ -273,6 +273,37 @@ int tcg_timer_end (tcg_ctx* ctx, float* ms)
 	return TCG_OK;
 }
 
+int tcg_event_create (tcg_ctx* ctx, void** event)
+{
+	if (!ctx || !event) { return TCG_ERR_ARG; }
+	hipEvent_t ev;
+	TCG_HIP(ctx, hipEventCreate(&ev));
+	*event = (void*) ev;
+	return TCG_OK;
+}
+
+int tcg_event_destroy (tcg_ctx* ctx, void* event)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (event) { TCG_HIP(ctx, hipEventDestroy((hipEvent_t) event)); }
+	return TCG_OK;
+}
+
+int tcg_event_record (tcg_ctx* ctx, void* event)
+{
+	if (!ctx || !event) { return TCG_ERR_ARG; }
+	TCG_HIP(ctx, hipEventRecord((hipEvent_t) event, ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_event_elapsed (tcg_ctx* ctx, void* start, void* stop, float* ms)
+{
+	if (!ctx || !start || !stop || !ms) { return TCG_ERR_ARG; }
+	TCG_HIP(ctx, hipEventSynchronize((hipEvent_t) stop));
+	TCG_HIP(ctx, hipEventElapsedTime(ms, (hipEvent_t) start, (hipEvent_t) stop));
+	return TCG_OK;
+}
+
 } // extern "C"
 
 int tcg_scratch (tcg_ctx* ctx, size_t bytes, void** out)
