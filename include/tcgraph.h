@@ -1,0 +1,79 @@
+/*
+ * tcgraph.h -- flat C binding of the host graph layer (libtenncor_host.so).
+ *
+ * The host layer keeps tenncor's C++ node API (eteq::make_functor, Variable,
+ * Constant, tcr::derive, teq::Evaluator + eigen::Device); this header exposes
+ * the same calls to languages without C++ linkage, the way the reference's
+ * pybind11 module does for Python (tenncor/python/eteq_ext.cpp:130-157 for
+ * evaluation and data access, tenncor/python/tenncor_ext.cpp for derive).
+ * Nodes are integers local to a tcr_graph; attributes use the nine keys of
+ * internal/eigen/packattr.hpp:60-363 with integer-list values.
+ *
+ * Every function returns 0 on success; tcr_last_error() gives the message of
+ * the last failure of the calling thread (the text the reference would have
+ * thrown).
+ */
+#ifndef TCGRAPH_H
+#define TCGRAPH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tcr_graph tcr_graph;
+
+const char* tcr_last_error (void);
+
+int tcr_graph_create (tcr_graph** out);
+int tcr_graph_destroy (tcr_graph* g);
+
+/* eteq::make_variable<T>(data, shape, label) -- tenncor/eteq/make.hpp:50-56.
+ * dtype: 1 double, 2 float, 3 int32; shape: 8 dims, dim 0 fastest */
+int tcr_variable (tcr_graph* g, int dtype, const uint64_t shape[8], const void* data,
+	const char* label, int* node);
+/* eteq::make_constant<T>(data, shape) -- tenncor/eteq/make.hpp:108-119 */
+int tcr_constant (tcr_graph* g, int dtype, const uint64_t shape[8], const void* data, int* node);
+/* Variable<T>::assign(data) -- tenncor/eteq/variable.hpp:72-90 */
+int tcr_assign (tcr_graph* g, int variable, const void* data);
+
+/* eteq::make_funcattr(opcode, children, attrs) -- tenncor/eteq/src/make.cpp:14-29.
+ * Attribute i has key keys[i] and the integer list vals[i][0..lens[i]);
+ * "rank" takes one value, "dtype" takes one dtype code, "tensor" takes one
+ * node id.  The result may be one of the children (build-time elision). */
+int tcr_functor (tcr_graph* g, int opcode, int nargs, const int* args, int nattrs,
+	const char* const* keys, const int64_t* const* vals, const int* lens, int* node);
+
+/* tcr::derive(root, targets) -- tenncor/src/eteq.cpp:40-76 */
+int tcr_derive (tcr_graph* g, int root, int ntargets, const int* targets, int* grads);
+
+/* teq::get_eval().evaluate(eigen::Device, targets) --
+ * tenncor/eteq/src/etens.cpp:46-62 */
+int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets);
+/* Block until the device has finished everything enqueued */
+int tcr_sync (tcr_graph* g);
+
+/* iTensor::shape / get_meta().type_code / device().data() */
+int tcr_shape (tcr_graph* g, int node, uint64_t shape[8]);
+int tcr_dtype (tcr_graph* g, int node, int* dtype);
+/* Copies the node's value (n_elems * type_size bytes) into out; fails when
+ * the node has no data (never evaluated or expired) */
+int tcr_data (tcr_graph* g, int node, void* out, size_t bytes);
+int tcr_version (tcr_graph* g, int node, uint64_t* version);
+
+/* Structure: opcode (0 for leaves), operands, and the indented dump used by
+ * the reference's graph-equality tests (testutil/tutil.hpp) */
+int tcr_opcode (tcr_graph* g, int node, int* opcode);
+int tcr_nargs (tcr_graph* g, int node, int* nargs);
+int tcr_args (tcr_graph* g, int node, int* args, int capacity);
+int tcr_to_string (tcr_graph* g, int node, char* out, size_t capacity);
+/* Number of distinct functors reachable from the given nodes */
+int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TCGRAPH_H */

@@ -54,9 +54,37 @@ def build_libtcg(jobs=8, verbose=False):
     return LIBTCG
 
 
+HOST = os.path.join(PKG, "host")
+LIBHOST = os.path.join(PKG, "libtenncor_host.so")
+CXX = os.environ.get("CXX", "g++")
+
+
+def build_libhost(jobs=8, verbose=False):
+    """Compile the C++ host graph layer (host/src/*.cpp) against libtcg.so."""
+    from concurrent.futures import ThreadPoolExecutor
+    objdir = os.path.join(PKG, "build")
+    os.makedirs(objdir, exist_ok=True)
+    sources = sorted(glob.glob(os.path.join(HOST, "src", "*.cpp")))
+    objs = [os.path.join(objdir, "host_" + os.path.basename(s)[:-4] + ".o") for s in sources]
+    flags = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra", "-I" + HOST, "-I" + os.path.join(ROOT, "include")]
+
+    def compile_one(pair):
+        src, obj = pair
+        out = _run([CXX] + flags + ["-c", src, "-o", obj])
+        if verbose and out.strip():
+            print(out)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(compile_one, zip(sources, objs)))
+    _run([CXX, "-shared", "-fPIC", "-o", LIBHOST] + objs +
+         ["-L" + PKG, "-ltcg", "-Wl,-rpath,$ORIGIN"])
+    return LIBHOST
+
+
 def build_all(verbose=False):
     """Everything native in this package."""
-    return [build_libtcg(verbose=verbose)]
+    return [build_libtcg(verbose=verbose), build_libhost(verbose=verbose)]
 
 
 def main():

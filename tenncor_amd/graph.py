@@ -1,0 +1,383 @@
+"""ctypes binding of ``include/tcgraph.h`` (``libtenncor_host.so``): the C++
+host graph layer -- Variable / Constant / Functor nodes, the gradient builder,
+the evaluator and the GPU device -- driven from Python the way the reference's
+pybind11 module drives tenncor (tenncor/python/*.cpp).
+
+``Graph`` owns nodes; ``Node`` is a handle with numpy-side shape bookkeeping.
+The composite helpers at the bottom restate the generated ``TenncorAPI`` methods
+the benchmark configurations are built from (cfg/tenncor/*.yml); they only
+compose primitive opcodes.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import capi
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libtenncor_host.so")
+
+OP = capi.OP
+DOUBLE, FLOAT, INT32 = capi.DOUBLE, capi.FLOAT, capi.INT32
+RANK_CAP = 8
+DIM_MAX = 65535  # std::numeric_limits<teq::DimT>::max()
+
+EXPORTS = [
+    "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
+    "tcr_functor", "tcr_derive", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
+    "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
+]
+
+_lib = None
+
+
+class GraphError(RuntimeError):
+    pass
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError("%s is missing: build it with `python -m tenncor_amd.build`" % LIB_PATH)
+    capi.load()  # libtcg.so first, so that the dependency resolves in-tree
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i32 = ctypes.c_void_p, ctypes.c_int
+    i32p, u64p = ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_uint64)
+    sig = {
+        "tcr_graph_create": [ctypes.POINTER(vp)],
+        "tcr_graph_destroy": [vp],
+        "tcr_variable": [vp, i32, u64p, vp, ctypes.c_char_p, i32p],
+        "tcr_constant": [vp, i32, u64p, vp, i32p],
+        "tcr_assign": [vp, i32, vp],
+        "tcr_functor": [vp, i32, i32, i32p, i32, ctypes.POINTER(ctypes.c_char_p),
+                        ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)), i32p, i32p],
+        "tcr_derive": [vp, i32, i32, i32p, i32p],
+        "tcr_evaluate": [vp, i32, i32p],
+        "tcr_sync": [vp],
+        "tcr_shape": [vp, i32, u64p],
+        "tcr_dtype": [vp, i32, i32p],
+        "tcr_data": [vp, i32, vp, ctypes.c_size_t],
+        "tcr_version": [vp, i32, u64p],
+        "tcr_opcode": [vp, i32, i32p],
+        "tcr_nargs": [vp, i32, i32p],
+        "tcr_args": [vp, i32, i32p, i32],
+        "tcr_to_string": [vp, i32, ctypes.c_char_p, ctypes.c_size_t],
+        "tcr_count_functors": [vp, i32, i32p, i32p],
+    }
+    for name, argtypes in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+    lib.tcr_last_error.argtypes = []
+    lib.tcr_last_error.restype = ctypes.c_char_p
+    _lib = lib
+    return lib
+
+
+def _ints(vals):
+    return (ctypes.c_int * len(vals))(*[int(v) for v in vals])
+
+
+class Node:
+    def __init__(self, graph, nid):
+        self.graph = graph
+        self.id = nid
+
+    @property
+    def shape(self):
+        return self.graph.shape(self)
+
+    @property
+    def dtype(self):
+        return self.graph.dtype(self)
+
+    def get(self):
+        return self.graph.data(self)
+
+    def __repr__(self):
+        return "Node(%d)" % self.id
+
+
+class Graph:
+    def __init__(self):
+        self.lib = load()
+        h = ctypes.c_void_p()
+        self._check(self.lib.tcr_graph_create(ctypes.byref(h)))
+        self.h = h
+
+    def close(self):
+        if self.h:
+            self.lib.tcr_graph_destroy(self.h)
+            self.h = None
+
+    def _check(self, rc):
+        if rc != 0:
+            raise GraphError(self.lib.tcr_last_error().decode())
+
+    # ---- leaves ----
+    def variable(self, data, shape, label=""):
+        data = np.ascontiguousarray(data).reshape(-1)
+        assert data.size == capi.n_elems(shape)
+        out = ctypes.c_int()
+        s = (ctypes.c_uint64 * 8)(*capi.shape8(shape))
+        self._check(self.lib.tcr_variable(self.h, capi.dtype_code(data.dtype), s, data.ctypes.data,
+                                          label.encode(), ctypes.byref(out)))
+        return Node(self, out.value)
+
+    def constant(self, data, shape):
+        data = np.ascontiguousarray(data).reshape(-1)
+        assert data.size == capi.n_elems(shape)
+        out = ctypes.c_int()
+        s = (ctypes.c_uint64 * 8)(*capi.shape8(shape))
+        self._check(self.lib.tcr_constant(self.h, capi.dtype_code(data.dtype), s, data.ctypes.data, ctypes.byref(out)))
+        return Node(self, out.value)
+
+    def scalar(self, value, np_dtype, shape=()):
+        return self.constant(np.full(capi.n_elems(shape), value, dtype=np_dtype), list(shape))
+
+    def assign(self, var, data):
+        data = np.ascontiguousarray(data, dtype=capi.NP_OF[var.dtype]).reshape(-1)
+        assert data.size == capi.n_elems(var.shape)
+        self._check(self.lib.tcr_assign(self.h, var.id, data.ctypes.data))
+
+    # ---- functors ----
+    def functor(self, op, args, **attrs):
+        """attrs: key -> list of ints (pairs flattened), a Node for `tensor`."""
+        opcode = OP[op] if isinstance(op, str) else int(op)
+        keys, arrays = [], []
+        for key, val in attrs.items():
+            if isinstance(val, Node):
+                val = [val.id]
+            elif np.isscalar(val):
+                val = [int(val)]
+            keys.append(key.encode())
+            arrays.append((ctypes.c_int64 * len(val))(*[int(v) for v in val]))
+        ckeys = (ctypes.c_char_p * len(keys))(*keys)
+        cvals = (ctypes.POINTER(ctypes.c_int64) * len(keys))(
+            *[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in arrays])
+        clens = _ints([len(a) for a in arrays])
+        out = ctypes.c_int()
+        self._check(self.lib.tcr_functor(self.h, opcode, len(args), _ints([a.id for a in args]), len(keys),
+                                         ckeys, cvals, clens, ctypes.byref(out)))
+        return Node(self, out.value)
+
+    def derive(self, root, targets):
+        out = (ctypes.c_int * len(targets))()
+        self._check(self.lib.tcr_derive(self.h, root.id, len(targets), _ints([t.id for t in targets]), out))
+        return [Node(self, out[i]) for i in range(len(targets))]
+
+    def evaluate(self, targets):
+        self._check(self.lib.tcr_evaluate(self.h, len(targets), _ints([t.id for t in targets])))
+
+    def sync(self):
+        self._check(self.lib.tcr_sync(self.h))
+
+    # ---- inspection ----
+    def shape(self, node):
+        s = (ctypes.c_uint64 * 8)()
+        self._check(self.lib.tcr_shape(self.h, node.id, s))
+        return list(s)
+
+    def dtype(self, node):
+        d = ctypes.c_int()
+        self._check(self.lib.tcr_dtype(self.h, node.id, ctypes.byref(d)))
+        return d.value
+
+    def data(self, node):
+        out = np.empty(capi.n_elems(self.shape(node)), dtype=capi.NP_OF[self.dtype(node)])
+        self._check(self.lib.tcr_data(self.h, node.id, out.ctypes.data, out.nbytes))
+        return out
+
+    def version(self, node):
+        v = ctypes.c_uint64()
+        self._check(self.lib.tcr_version(self.h, node.id, ctypes.byref(v)))
+        return v.value
+
+    def opcode(self, node):
+        o = ctypes.c_int()
+        self._check(self.lib.tcr_opcode(self.h, node.id, ctypes.byref(o)))
+        return capi.OPCODES[o.value]
+
+    def args(self, node):
+        n = ctypes.c_int()
+        self._check(self.lib.tcr_nargs(self.h, node.id, ctypes.byref(n)))
+        buf = (ctypes.c_int * max(n.value, 1))()
+        self._check(self.lib.tcr_args(self.h, node.id, buf, n.value))
+        return [Node(self, buf[i]) for i in range(n.value)]
+
+    def to_string(self, node):
+        buf = ctypes.create_string_buffer(1 << 20)
+        self._check(self.lib.tcr_to_string(self.h, node.id, buf, len(buf)))
+        return buf.value.decode()
+
+    def count_functors(self, nodes):
+        c = ctypes.c_int()
+        self._check(self.lib.tcr_count_functors(self.h, len(nodes), _ints([n.id for n in nodes]), ctypes.byref(c)))
+        return c.value
+
+
+class Api:
+    """The TenncorAPI methods the configurations use (cfg/tenncor/core.yml,
+    nn.yml, layer.yml, loss.yml), restated over Graph.functor."""
+
+    def __init__(self, graph):
+        self.g = graph
+
+    def _like(self, scalar, like):
+        """eteq::make_constant_like: scalar Constant + EXTEND to `like`
+        (tenncor/eteq/make.hpp:168-183)."""
+        cst = self.g.scalar(scalar, capi.NP_OF[like.dtype])
+        return self.g.functor("EXTEND", [cst], tensor=like)
+
+    def _operand(self, x, like):
+        return x if isinstance(x, Node) else self._like(x, like)
+
+    def unary(self, op, x):
+        return self.g.functor(op, [x])
+
+    def binary(self, op, a, b):
+        if not isinstance(a, Node):
+            a = self._like(a, b)
+        b = self._operand(b, a)
+        return self.g.functor(op, [a, b])
+
+    def add(self, a, b):
+        return self.binary("ADD", a, b)
+
+    def sub(self, a, b):
+        return self.binary("SUB", a, b)
+
+    def mul(self, a, b):
+        return self.binary("MUL", a, b)
+
+    def div(self, a, b):
+        return self.binary("DIV", a, b)
+
+    def pow(self, a, b):
+        return self.binary("POW", a, b)
+
+    def sigmoid(self, x):
+        return self.unary("SIGMOID", x)
+
+    def tanh(self, x):
+        return self.unary("TANH", x)
+
+    def exp(self, x):
+        return self.unary("EXP", x)
+
+    def log(self, x):
+        return self.unary("LOG", x)
+
+    def neg(self, x):
+        return self.unary("NEG", x)
+
+    def square(self, x):
+        return self.unary("SQUARE", x)
+
+    def identity(self, x):
+        return self.g.functor("IDENTITY", [x])
+
+    def relu(self, x):
+        """core.yml:1261-1267: max(arg, 0)."""
+        return self.binary("MAX", x, 0.0)
+
+    def matmul(self, a, b):
+        return self.g.functor("MATMUL", [a, b])
+
+    def contract(self, a, b, dims=((0, 1),)):
+        return self.g.functor("CONTRACT", [a, b], rank_pairs=[v for p in dims for v in p])
+
+    def transpose(self, x):
+        return self.permute(x, [1, 0])
+
+    def permute(self, x, order):
+        return self.g.functor("PERMUTE", [x], ranks=list(order))
+
+    def extend(self, x, offset, xlist):
+        """core.yml:679-693."""
+        return self.g.functor("EXTEND", [x], dimensions=[1] * offset + list(xlist))
+
+    def extend_like(self, x, like):
+        return self.g.functor("EXTEND", [x], tensor=like)
+
+    def reduce(self, op, x, offset=0, ndims=RANK_CAP):
+        """core.yml:773-800: dims offset .. offset+ndims-1."""
+        dims = list(range(offset, min(offset + ndims, RANK_CAP)))
+        return self.g.functor(op, [x], rank_set=dims)
+
+    def reduce_sum(self, x, offset=0, ndims=RANK_CAP):
+        return self.reduce("REDUCE_SUM", x, offset, ndims)
+
+    def reduce_max(self, x, offset=0, ndims=RANK_CAP):
+        return self.reduce("REDUCE_MAX", x, offset, ndims)
+
+    def slice(self, x, offset, extent, dimension):
+        """core.yml:909-927."""
+        ext = [0, DIM_MAX] * max(RANK_CAP, dimension)
+        ext[2 * dimension:2 * dimension + 2] = [offset, extent]
+        return self.g.functor("SLICE", [x], dimension_pairs=ext)
+
+    def pad(self, x, pairs):
+        return self.g.functor("PAD", [x], dimension_pairs=[v for p in pairs for v in p])
+
+    def reverse(self, x, dims):
+        return self.g.functor("REVERSE", [x], rank_set=list(dims))
+
+    def concat(self, args, axis):
+        return self.g.functor("CONCAT", list(args), rank=axis)
+
+    def convolution(self, img, kernel, dims):
+        return self.g.functor("CONV", [img, kernel], ranks=list(dims))
+
+    def dense(self, x, weight, bias=None, dims=((0, 1),)):
+        """nn.yml:14-47 fully_connect with one pair, wrapped in the IDENTITY the
+        layer tagging adds (tenncor/test/test_api.cpp:2433-2440)."""
+        out = self.contract(x, weight, dims)
+        if bias is not None:
+            out = self.add(out, self.extend_like(bias, out))
+        return self.identity(out)
+
+    def conv2d(self, image, kernel, bias=None):
+        """nn.yml:76-98 without explicit zero padding: image {in,w,h,batch},
+        kernel {out,in,kw,kh} -> {out,w',h',batch}."""
+        img_pad = kernel.shape[0] - 1
+        cimage = self.pad(image, [(0, 0)] * 4 + [(img_pad, img_pad)])
+        out = self.permute(self.convolution(cimage, self.reverse(kernel, [0]), [4, 0, 1, 2]), [4, 1, 2, 3])
+        if bias is not None:
+            out = self.add(out, self.extend_like(bias, out))
+        return out
+
+    def softmax(self, x, offset=0, ndims=RANK_CAP):
+        """core.yml:1232-1260."""
+        eps = float(np.finfo(np.float32).eps)
+        shifted = self.sub(x, self.extend_like(self.reduce_max(x, offset, ndims), x))
+        exarg = self.exp(shifted)
+        return self.div(exarg, self.extend_like(self.add(self.reduce_sum(exarg, offset, ndims), eps), exarg))
+
+    def cross_entropy(self, target, x):
+        """loss.yml:40-59."""
+        eps = float(np.finfo(np.float32).eps)
+        inp = self.add(x, eps)
+        not_in = self.sub(1.0, inp)
+        not_targ = self.sub(1.0, target)
+        return self.neg(self.add(self.mul(target, self.log(inp)), self.mul(not_targ, self.log(not_in))))
+
+    def lstm(self, x, init_state, init_hidden, gates, seq_dim=1):
+        """layer.yml:716-768.  gates = dict name -> callable(xc) for the g, i, f
+        and o gate layers (each a dense layer over concat(x_t, hidden))."""
+        nseq = x.shape[seq_dim]
+        state, hidden, states = init_state, init_hidden, []
+        for i in range(nseq):
+            inslice = self.slice(x, i, 1, seq_dim)
+            xc = self.concat([inslice, hidden], 0)
+            gate = self.tanh(gates["g"](xc))
+            inp = self.sigmoid(gates["i"](xc))
+            forget = self.sigmoid(gates["f"](xc))
+            output = self.sigmoid(gates["o"](xc))
+            state = self.add(self.mul(gate, inp), self.mul(state, forget))
+            hidden = self.mul(state, output)
+            states.append(hidden)
+        return self.identity(self.concat(states, seq_dim))

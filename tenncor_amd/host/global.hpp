@@ -1,0 +1,102 @@
+// Process-wide helpers of the host layer: error reporting in the style of
+// tenncor's global logger (internal/global/logs.hpp:11-81, where the `fatal`
+// and `throw_err` levels throw std::runtime_error, internal/global/g3logs.hpp:
+// 140-152), the graph-wide version clock and the seeded random generator
+// (internal/global/random.hpp:78-146).
+#ifndef TCH_GLOBAL_HPP
+#define TCH_GLOBAL_HPP
+
+#include <cstdarg>
+#include <cstdio>
+#include <functional>
+#include <random>
+#include <stdexcept>
+#include <string>
+
+namespace global
+{
+
+inline std::string vformat (const char* fmt, va_list ap)
+{
+	char buf[2048];
+	vsnprintf(buf, sizeof(buf), fmt, ap);
+	return std::string(buf);
+}
+
+[[noreturn]] inline void fatal (const std::string& msg)
+{
+	throw std::runtime_error(msg);
+}
+
+[[noreturn]] inline void throw_err (const std::string& msg)
+{
+	throw std::runtime_error(msg);
+}
+
+[[noreturn]] inline void fatalf (const char* fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	std::string msg = vformat(fmt, ap);
+	va_end(ap);
+	throw std::runtime_error(msg);
+}
+
+[[noreturn]] inline void throw_errf (const char* fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	std::string msg = vformat(fmt, ap);
+	va_end(ap);
+	throw std::runtime_error(msg);
+}
+
+// Diagnostics below `error` are routed to an optional sink (none by default)
+using LogSinkF = std::function<void(const std::string& level, const std::string& msg)>;
+LogSinkF& log_sink (void);
+
+inline void log (const char* level, const std::string& msg)
+{
+	if (auto& sink = log_sink()) { sink(level, msg); }
+}
+
+inline void debug (const std::string& msg) { log("debug", msg); }
+inline void warn (const std::string& msg) { log("warn", msg); }
+
+inline void debugf (const char* fmt, ...)
+{
+	if (!log_sink()) { return; }
+	va_list ap;
+	va_start(ap, fmt);
+	std::string msg = vformat(fmt, ap);
+	va_end(ap);
+	log("debug", msg);
+}
+
+inline void warnf (const char* fmt, ...)
+{
+	if (!log_sink()) { return; }
+	va_list ap;
+	va_start(ap, fmt);
+	std::string msg = vformat(fmt, ap);
+	va_end(ap);
+	log("warn", msg);
+}
+
+// Highest state version handed out so far; a Variable assignment takes the
+// next one so that every dependant recomputes (tenncor/eteq/variable.hpp:55-61)
+size_t& last_version (void);
+
+inline void note_version (size_t v)
+{
+	if (v > last_version()) { last_version() = v; }
+}
+
+// Seeded generator behind RAND_UNIF (host side, like the reference)
+using RandEngineT = std::default_random_engine;
+RandEngineT& get_generator (void);
+void seed (size_t s);
+
+}
+
+#endif // TCH_GLOBAL_HPP

@@ -1,0 +1,295 @@
+// Flat C binding of the host graph layer (include/tcgraph.h).
+#include "tcgraph.h"
+
+#include <sstream>
+
+#include "eteq.hpp"
+
+struct tcr_graph
+{
+	std::vector<teq::TensptrT> nodes;
+	std::unordered_map<teq::iTensor*,int> ids;
+
+	int add (teq::TensptrT tens)
+	{
+		auto it = ids.find(tens.get());
+		if (it != ids.end()) { return it->second; }
+		int id = (int) nodes.size();
+		nodes.push_back(tens);
+		ids.emplace(tens.get(), id);
+		return id;
+	}
+
+	teq::TensptrT at (int id) const
+	{
+		if (id < 0 || (size_t) id >= nodes.size()) { global::fatalf("unknown node %d", id); }
+		return nodes[id];
+	}
+};
+
+static thread_local std::string g_error;
+
+template <typename F>
+static int guarded (F fn)
+{
+	try
+	{
+		fn();
+		return 0;
+	}
+	catch (const std::exception& e)
+	{
+		g_error = e.what();
+		return 1;
+	}
+}
+
+static teq::Shape to_shape (const uint64_t shape[8])
+{
+	teq::DimsT dims;
+	for (int i = 0; i < 8; ++i)
+	{
+		if (shape[i] > 65535) { global::fatalf("dimension %d of extent %llu exceeds 65535", i, (unsigned long long) shape[i]); }
+		dims.push_back((teq::DimT) shape[i]);
+	}
+	return teq::Shape(dims);
+}
+
+// One node per line, children indented under their parent with "`--" branches
+// and "|" rails for parents that still have children to come
+static void print_tree (std::ostringstream& out, const teq::TensptrT& node,
+	const std::string& prefix, bool root, bool last)
+{
+	if (!root) { out << "\n" << prefix << "`--"; }
+	out << "(";
+	auto f = dynamic_cast<teq::iFunctor*>(node.get());
+	auto leaf = dynamic_cast<teq::iLeaf*>(node.get());
+	if (leaf && leaf->get_usage() == teq::IMMUTABLE) { out << "constant:"; }
+	else if (leaf) { out << "variable:"; }
+	out << node->to_string() << "<" << node->get_meta().type_label() << ">" << node->shape().to_string() << ")";
+	if (f)
+	{
+		std::string child_prefix = root ? "_" : prefix + (last ? "____" : "|___");
+		auto args = f->get_args();
+		for (size_t i = 0; i < args.size(); ++i)
+		{
+			print_tree(out, args[i], child_prefix, false, i + 1 == args.size());
+		}
+	}
+}
+
+extern "C" {
+
+const char* tcr_last_error (void) { return g_error.c_str(); }
+
+int tcr_graph_create (tcr_graph** out)
+{
+	return guarded([&] { *out = new tcr_graph(); });
+}
+
+int tcr_graph_destroy (tcr_graph* g)
+{
+	return guarded([&] { delete g; });
+}
+
+int tcr_variable (tcr_graph* g, int dtype, const uint64_t shape[8], const void* data, const char* label, int* node)
+{
+	return guarded([&]
+	{
+		teq::Shape s = to_shape(shape);
+		std::string lbl = label ? label : "";
+		teq::TensptrT out;
+#define TCH_VAR(T) out = eteq::make_variable<T>((const T*) data, s, lbl);
+		TYPE_LOOKUP(TCH_VAR, dtype)
+#undef TCH_VAR
+		*node = g->add(out);
+	});
+}
+
+int tcr_constant (tcr_graph* g, int dtype, const uint64_t shape[8], const void* data, int* node)
+{
+	return guarded([&]
+	{
+		teq::Shape s = to_shape(shape);
+		teq::TensptrT out;
+#define TCH_CST(T) out = eteq::make_constant_tensor<T>((const T*) data, s);
+		TYPE_LOOKUP(TCH_CST, dtype)
+#undef TCH_CST
+		*node = g->add(out);
+	});
+}
+
+int tcr_assign (tcr_graph* g, int variable, const void* data)
+{
+	return guarded([&]
+	{
+		teq::TensptrT tens = g->at(variable);
+		auto dtype = (egen::_GENERATED_DTYPE) tens->get_meta().type_code();
+#define TCH_ASSIGN(T) {\
+		auto var = dynamic_cast<eteq::Variable<T>*>(tens.get());\
+		if (nullptr == var) { global::fatalf("node %d is not a variable", variable); }\
+		var->assign((const T*) data, tens->shape()); }
+		TYPE_LOOKUP(TCH_ASSIGN, dtype)
+#undef TCH_ASSIGN
+	});
+}
+
+int tcr_functor (tcr_graph* g, int opcode, int nargs, const int* args, int nattrs,
+	const char* const* keys, const int64_t* const* vals, const int* lens, int* node)
+{
+	return guarded([&]
+	{
+		teq::TensptrsT children;
+		for (int i = 0; i < nargs; ++i) { children.push_back(g->at(args[i])); }
+		marsh::Maps attrs;
+		for (int i = 0; i < nattrs; ++i)
+		{
+			std::string key = keys[i];
+			std::vector<int64_t> v(vals[i], vals[i] + lens[i]);
+			if (key == "rank")
+			{
+				if (v.size() != 1) { global::fatal("`rank` takes one value"); }
+				attrs.add_attr(key, std::make_unique<marsh::Number<int64_t>>(v[0]));
+			}
+			else if (key == "dtype")
+			{
+				if (v.size() != 1) { global::fatal("`dtype` takes one value"); }
+				attrs.add_attr(key, std::make_unique<marsh::String>(egen::name_type((egen::_GENERATED_DTYPE) v[0])));
+			}
+			else if (key == "tensor")
+			{
+				if (v.size() != 1) { global::fatal("`tensor` takes one node"); }
+				attrs.add_attr(key, std::make_unique<teq::TensorObj>(g->at((int) v[0])));
+			}
+			else
+			{
+				attrs.add_attr(key, std::make_unique<marsh::NumArray<int64_t>>(v));
+			}
+		}
+		auto op = (egen::_GENERATED_OPCODE) opcode;
+		if (op <= egen::BAD_OP || op >= egen::_N_GENERATED_OPCODES) { global::fatal("unknown opcode"); }
+		*node = g->add(eteq::make_funcattr(op, children, attrs));
+	});
+}
+
+int tcr_derive (tcr_graph* g, int root, int ntargets, const int* targets, int* grads)
+{
+	return guarded([&]
+	{
+		teq::TensptrsT wrt;
+		for (int i = 0; i < ntargets; ++i) { wrt.push_back(g->at(targets[i])); }
+		auto ders = tcr::derive(g->at(root), wrt);
+		for (int i = 0; i < ntargets; ++i) { grads[i] = g->add(ders[i]); }
+	});
+}
+
+int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets)
+{
+	return guarded([&]
+	{
+		teq::TensptrsT roots;
+		for (int i = 0; i < ntargets; ++i) { roots.push_back(g->at(targets[i])); }
+		eteq::run(roots);
+	});
+}
+
+int tcr_sync (tcr_graph*)
+{
+	return guarded([&] { eigen::hip_check(tcg_sync(eigen::hip_context())); });
+}
+
+int tcr_shape (tcr_graph* g, int node, uint64_t shape[8])
+{
+	return guarded([&]
+	{
+		teq::Shape s = g->at(node)->shape();
+		std::copy(s.begin(), s.end(), shape);
+	});
+}
+
+int tcr_dtype (tcr_graph* g, int node, int* dtype)
+{
+	return guarded([&] { *dtype = (int) g->at(node)->get_meta().type_code(); });
+}
+
+int tcr_data (tcr_graph* g, int node, void* out, size_t bytes)
+{
+	return guarded([&]
+	{
+		teq::TensptrT tens = g->at(node);
+		size_t need = tens->shape().n_elems() * tens->get_meta().type_size();
+		if (bytes < need) { global::fatalf("buffer of %d bytes is too small for %d", (int) bytes, (int) need); }
+		const void* src = tens->device().data();
+		if (nullptr == src) { global::fatalf("node %s has no data", tens->to_string().c_str()); }
+		memcpy(out, src, need);
+	});
+}
+
+int tcr_version (tcr_graph* g, int node, uint64_t* version)
+{
+	return guarded([&] { *version = g->at(node)->get_meta().state_version(); });
+}
+
+int tcr_opcode (tcr_graph* g, int node, int* opcode)
+{
+	return guarded([&]
+	{
+		auto f = dynamic_cast<teq::iFunctor*>(g->at(node).get());
+		*opcode = f ? (int) f->get_opcode().code_ : 0;
+	});
+}
+
+int tcr_nargs (tcr_graph* g, int node, int* nargs)
+{
+	return guarded([&]
+	{
+		auto f = dynamic_cast<teq::iFunctor*>(g->at(node).get());
+		*nargs = f ? (int) f->get_args().size() : 0;
+	});
+}
+
+int tcr_args (tcr_graph* g, int node, int* args, int capacity)
+{
+	return guarded([&]
+	{
+		auto f = dynamic_cast<teq::iFunctor*>(g->at(node).get());
+		if (nullptr == f) { return; }
+		auto children = f->get_args();
+		if ((int) children.size() > capacity) { global::fatal("argument buffer is too small"); }
+		for (size_t i = 0; i < children.size(); ++i) { args[i] = g->add(children[i]); }
+	});
+}
+
+int tcr_to_string (tcr_graph* g, int node, char* out, size_t capacity)
+{
+	return guarded([&]
+	{
+		std::ostringstream ss;
+		print_tree(ss, g->at(node), "", true, true);
+		std::string s = ss.str();
+		if (s.size() + 1 > capacity) { global::fatal("string buffer is too small"); }
+		memcpy(out, s.c_str(), s.size() + 1);
+	});
+}
+
+int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count)
+{
+	return guarded([&]
+	{
+		struct Counter final : public teq::iOnceTraveler
+		{
+			size_t nfuncs = 0;
+			void visit_leaf (teq::iLeaf&) override {}
+			void visit_func (teq::iFunctor& f) override
+			{
+				++nfuncs;
+				auto args = f.get_args();
+				teq::multi_visit(*this, args);
+			}
+		} counter;
+		for (int i = 0; i < nnodes; ++i) { g->at(nodes[i])->accept(counter); }
+		*count = (int) counter.nfuncs;
+	});
+}
+
+} // extern "C"

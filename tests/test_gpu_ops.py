@@ -388,6 +388,34 @@ def test_matmul_vs_oracle(ctx, ops, oracle, ashape, bshape):
         np.testing.assert_allclose(outd.get(), oracle.matmul(ad, ashape, bd, bshape)[0], rtol=1e-10, atol=1e-12)
 
 
+GEMM_CASES = [
+    # (M, N, K, batch, trans_a, trans_b): sizes on the matrix-core path (multiples of 4, >= 32)
+    (128, 128, 64, 1, 0, 0), (128, 128, 64, 1, 1, 0), (128, 128, 64, 1, 0, 1), (128, 128, 64, 1, 1, 1),
+    (100, 36, 40, 1, 0, 0), (100, 36, 40, 3, 1, 1), (260, 132, 72, 2, 1, 0), (260, 132, 72, 2, 0, 1),
+    (512, 384, 200, 1, 0, 0), (2048, 256, 768, 1, 1, 0), (768, 2048, 256, 1, 0, 1),
+    # off the matrix-core path: odd extents
+    (33, 35, 17, 2, 0, 0), (33, 35, 17, 2, 1, 1),
+]
+
+
+@pytest.mark.parametrize("M,N,K,batch,ta,tb", GEMM_CASES, ids=[str(c) for c in GEMM_CASES])
+def test_gemm_transposed_operands_vs_oracle(ctx, oracle, M, N, K, batch, ta, tb):
+    """tcg_gemm with every operand layout a contraction can lower to."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of(M, N, K, batch, ta, tb))
+    a = rng.standard_normal(batch * M * K).astype(np.float32)
+    b = (rng.standard_normal(batch * K * N) / np.sqrt(K)).astype(np.float32)
+    # oracle works on the canonical layout a{K,M,batch}, b{N,K,batch}
+    a_can = a if not ta else oracle.permute(a, [M, K, batch], [1, 0, 2])[0]
+    b_can = b if not tb else oracle.permute(b, [K, N, batch], [1, 0, 2])[0]
+    ref, _ = oracle.matmul(a_can, [K, M, batch], b_can, [N, K, batch], wide_acc=True)
+    da, db = ctx.upload(a), ctx.upload(b)
+    dc = ctx.empty(batch * M * N, np.float32)
+    ctx.gemm(capi.FLOAT, M, N, K, batch, da.ptr, M if ta else K, M * K, ta,
+             db.ptr, K if tb else N, K * N, tb, dc.ptr, N, M * N)
+    assert_acc_close(dc.get(), ref)
+
+
 CONTRACT_CASES = [
     ([10, 3], [9, 10], [[0, 1]]),                      # dense layer (config 1)
     ([768, 1, 64], [512, 768], [[0, 1]]),              # LSTM gate product (config 4)

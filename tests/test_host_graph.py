@@ -1,0 +1,260 @@
+"""Host graph layer without a GPU: node construction, shape / type / elision
+rules (cfg/ops.yml), automatic casts, the gradient builder's output graphs and
+the reference's error messages.  Nothing here evaluates a node."""
+import numpy as np
+import pytest
+
+
+@pytest.fixture()
+def g():
+    from tenncor_amd import graph
+    gr = graph.Graph()
+    yield gr
+    gr.close()
+
+
+@pytest.fixture()
+def api(g):
+    from tenncor_amd import graph
+    return graph.Api(g)
+
+
+def var(g, shape, dtype=np.float32, label="x"):
+    n = int(np.prod(shape))
+    return g.variable(np.arange(n, dtype=dtype), shape, label)
+
+
+def test_library_exports_every_declared_symbol():
+    import ctypes
+    import os
+    import re
+    from tenncor_amd import graph
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(root, "include", "tcgraph.h")).read(), flags=re.S)
+    declared = sorted(set(re.findall(r"\b(tcr_[a-z0-9_]+)\s*\(", text)))
+    assert declared == sorted(graph.EXPORTS)
+    lib = ctypes.CDLL(graph.LIB_PATH)
+    assert not [s for s in declared if not hasattr(lib, s)]
+
+
+# internal/eigen/test/test_shaper.cpp:21-437 -- (op, arg shapes, attrs, expected shape)
+SHAPE_CASES = [
+    ("ADD", [[3, 2], [3, 2]], {}, [3, 2]),
+    ("REDUCE_SUM", [[3, 2, 4]], {"rank_set": [1]}, [3, 1, 4]),
+    ("REDUCE_MAX", [[3, 2, 4]], {"rank_set": [0, 2]}, [1, 2, 1]),
+    ("ARGMAX", [[3, 2, 4]], {"rank": 1}, [3, 1, 4]),
+    ("ARGMAX", [[3, 2, 4]], {"rank": 8}, [1]),
+    ("PERMUTE", [[3, 2, 4]], {"ranks": [2, 0, 1]}, [4, 3, 2]),
+    ("PERMUTE", [[3, 2, 4]], {"ranks": [1, 0]}, [2, 3, 4]),
+    ("EXTEND", [[3, 1, 2]], {"dimensions": [1, 4]}, [3, 4, 2]),
+    ("RESHAPE", [[3, 2, 4]], {"shape": [6, 4]}, [6, 4]),
+    ("SLICE", [[3, 2]], {"dimension_pairs": [1, 2, 1, 1]}, [2, 1]),
+    ("SLICE", [[3, 2]], {"dimension_pairs": [1, 200]}, [2, 2]),
+    ("PAD", [[2, 3]], {"dimension_pairs": [1, 1]}, [4, 3]),
+    ("STRIDE", [[2, 3]], {"dimensions": [1, 2]}, [2, 2]),
+    ("SCATTER", [[2, 2]], {"dimensions": [2, 2], "shape": [3, 3, 1, 1, 1, 1, 1, 1]}, [3, 3]),
+    ("MATMUL", [[4, 3], [2, 4]], {}, [2, 3]),
+    ("MATMUL", [[4, 3, 5], [2, 4, 5]], {}, [2, 3, 5]),
+    ("CONTRACT", [[4, 3], [2, 4]], {"rank_pairs": [0, 1]}, [2, 3]),
+    ("CONTRACT", [[4, 2, 3], [2, 4, 2]], {"rank_pairs": [0, 1, 1, 2]}, [2, 3]),
+    ("CONTRACT", [[768, 1, 256], [2048, 768]], {"rank_pairs": [0, 1]}, [2048, 1, 256]),
+    ("CONV", [[3, 3], [2]], {"ranks": [1]}, [3, 2]),
+    ("CONV", [[4, 10, 9, 2, 5], [3, 4, 5, 6]], {"ranks": [4, 0, 1, 2]}, [1, 6, 4, 2, 3]),
+    ("CONCAT", [[2, 3], [1, 3]], {"rank": 0}, [3, 3]),
+    ("CONCAT", [[1, 4], [1, 4], [1, 4]], {"rank": 0}, [3, 4]),
+    ("SELECT", [[2, 3], [2, 3], [2, 3]], {}, [2, 3]),
+]
+
+
+@pytest.mark.parametrize("op,shapes,attrs,expect", SHAPE_CASES, ids=[c[0] + str(c[1]) for c in SHAPE_CASES])
+def test_shape_rules(g, op, shapes, attrs, expect):
+    from tenncor_amd import capi
+    args = [var(g, s) for s in shapes]
+    out = g.functor(op, args, **attrs)
+    assert out.shape == capi.shape8(expect)
+
+
+ERROR_CASES = [
+    ("ADD", [[3, 2], [2, 3]], {}, "cannot ADD with incompatible shapes"),
+    ("PERMUTE", [[3, 2]], {"ranks": [1, 1]}, "permute does not support repeated orders"),
+    ("EXTEND", [[3, 2]], {"dimensions": [2]}, "cannot extend non-singular dimension 0"),
+    ("EXTEND", [[1, 2]], {"dimensions": [0]}, "cannot extend using zero dimensions"),
+    ("RESHAPE", [[3, 2]], {"shape": [5]}, "cannot RESHAPE with shapes of different sizes"),
+    ("SLICE", [[3, 2]], {"dimension_pairs": [0, 0]}, "cannot create slice with 0 dimensions"),
+    ("MATMUL", [[4, 3], [2, 5]], {}, "have mismatch common dimension 0,1"),
+    ("MATMUL", [[4, 3, 2], [2, 4, 3]], {}, "do not match for dimensions 2+"),
+    ("CONTRACT", [[4, 3], [2, 5]], {"rank_pairs": [0, 1]}, "do not match common dimensions"),
+    ("CONTRACT", [[4, 4], [4, 4]], {"rank_pairs": [0, 1, 0, 0]}, "must be unique for each side"),
+    ("CONV", [[3, 3], [2, 2]], {"ranks": [1]}, "cannot have ambiguous ranks not specified in kernelshape"),
+    ("CONV", [[3, 3], [5]], {"ranks": [1]}, "cannot convolve a kernel of shape"),
+    ("CONCAT", [[2, 3], [2, 4]], {"rank": 0}, "cannot group concat incompatible shapes"),
+    ("CONCAT", [[2, 3], [2, 3], [2, 3]], {"rank": 0}, "cannot group concat shapes with dimension that is not one"),
+    ("REDUCE_SUM", [[3, 2]], {}, "cannot find `rank_set` attribute"),
+]
+
+
+@pytest.mark.parametrize("op,shapes,attrs,message", ERROR_CASES, ids=[c[0] + ":" + c[3][:24] for c in ERROR_CASES])
+def test_construction_errors_carry_the_reference_messages(g, op, shapes, attrs, message):
+    from tenncor_amd import graph
+    args = [var(g, s) for s in shapes]
+    with pytest.raises(graph.GraphError) as info:
+        g.functor(op, args, **attrs)
+    assert message in str(info.value)
+
+
+def test_redundant_nodes_are_elided(g):
+    """cfg/ops.yml FuncOpt: the first child stands in for the node."""
+    x = var(g, [3, 2, 4])
+    assert g.functor("REDUCE_SUM", [x], rank_set=[]).id == x.id
+    assert g.functor("PERMUTE", [x], ranks=[0, 1, 2]).id == x.id
+    assert g.functor("PERMUTE", [x], ranks=[]).id == x.id
+    assert g.functor("EXTEND", [x], dimensions=[1, 1]).id == x.id
+    assert g.functor("RESHAPE", [x], shape=[3, 2, 4, 1, 1, 1, 1, 1]).id == x.id
+    assert g.functor("SLICE", [x], dimension_pairs=[0, 65535, 0, 65535]).id == x.id
+    assert g.functor("SLICE", [x], dimension_pairs=[0, 3]).id != x.id  # extent must exceed the dim
+    assert g.functor("PAD", [x], dimension_pairs=[0, 0, 0, 0]).id == x.id
+    assert g.functor("ADD", [x]).id == x.id
+    assert g.functor("ARGMAX", [var(g, [3, 1])], rank=1).id != x.id
+    y = var(g, [3, 1])
+    assert g.functor("ARGMAX", [y], rank=1).id == y.id
+    from tenncor_amd import capi
+    assert g.functor("CAST", [x], dtype=capi.FLOAT).id == x.id
+
+
+def test_type_rule_and_automatic_casts(g):
+    """cfg/ops.yml:44-62 + tenncor/eteq/caster.hpp: the node takes the most
+    precise child dtype; other children get a CAST in front."""
+    from tenncor_amd import capi
+    f = var(g, [2, 2], np.float32, "f")
+    i = var(g, [2, 2], np.int32, "i")
+    d = var(g, [2, 2], np.float64, "d")
+    out = g.functor("ADD", [i, f])
+    assert out.dtype == capi.FLOAT
+    a0, a1 = g.args(out)
+    assert g.opcode(a0) == "CAST" and a0.dtype == capi.FLOAT and g.args(a0)[0].id == i.id
+    assert a1.id == f.id
+    out = g.functor("MUL", [f, d, i])
+    assert out.dtype == capi.DOUBLE
+    assert [g.opcode(a) for a in g.args(out)] == ["CAST", "BAD_OP", "CAST"]
+    # ASSIGN takes the target's dtype (cfg/ops.yml:656-664)
+    out = g.functor("ASSIGN_SUB", [f, d])
+    assert out.dtype == capi.FLOAT and g.opcode(g.args(out)[1]) == "CAST"
+    c = g.functor("CAST", [f], dtype=capi.INT32)
+    assert c.dtype == capi.INT32
+
+
+def test_dense_and_conv2d_lower_like_the_reference(g, api):
+    """Graph dumps of tenncor/test/test_api.cpp:2433-2446 and :2519-2529."""
+    x = g.variable(np.zeros(12, np.float32), [6, 2], "x")
+    weight = g.variable(np.zeros(30, np.float32), [5, 6], "weight")
+    bias = g.variable(np.zeros(5, np.float32), [5], "bias")
+    y = api.dense(x, weight, bias)
+    assert g.to_string(y) == (
+        "(IDENTITY<FLOAT>[5\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_`--(ADD<FLOAT>[5\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_____`--(CONTRACT<FLOAT>[5\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_____|___`--(variable:x<FLOAT>[6\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_____|___`--(variable:weight<FLOAT>[5\\6\\1\\1\\1\\1\\1\\1])\n"
+        "_____`--(EXTEND<FLOAT>[5\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_________`--(variable:bias<FLOAT>[5\\1\\1\\1\\1\\1\\1\\1])")
+    x = g.variable(np.zeros(4 * 10 * 9 * 2, np.float32), [4, 10, 9, 2], "x")
+    weight = g.variable(np.zeros(3 * 4 * 5 * 6, np.float32), [3, 4, 5, 6], "weight")
+    bias = g.variable(np.zeros(3, np.float32), [3], "bias")
+    y = api.identity(api.conv2d(x, weight, bias))
+    assert g.to_string(y) == (
+        "(IDENTITY<FLOAT>[3\\6\\4\\2\\1\\1\\1\\1])\n"
+        "_`--(ADD<FLOAT>[3\\6\\4\\2\\1\\1\\1\\1])\n"
+        "_____`--(PERMUTE<FLOAT>[3\\6\\4\\2\\1\\1\\1\\1])\n"
+        "_____|___`--(CONV<FLOAT>[1\\6\\4\\2\\3\\1\\1\\1])\n"
+        "_____|_______`--(PAD<FLOAT>[4\\10\\9\\2\\5\\1\\1\\1])\n"
+        "_____|_______|___`--(variable:x<FLOAT>[4\\10\\9\\2\\1\\1\\1\\1])\n"
+        "_____|_______`--(REVERSE<FLOAT>[3\\4\\5\\6\\1\\1\\1\\1])\n"
+        "_____|___________`--(variable:weight<FLOAT>[3\\4\\5\\6\\1\\1\\1\\1])\n"
+        "_____`--(EXTEND<FLOAT>[3\\6\\4\\2\\1\\1\\1\\1])\n"
+        "_________`--(variable:bias<FLOAT>[3\\1\\1\\1\\1\\1\\1\\1])")
+
+
+S32 = "[3\\2\\1\\1\\1\\1\\1\\1]"
+
+
+def test_gradient_graphs_match_the_reference_structure(g, api):
+    """tenncor/eteq/test/test_backprop.cpp:201-228 (Sigmoid, Tanh), :435-459
+    (Contract) and :462-485 (Conv): the same trees with the upstream gradient
+    being the all-ones seed of teq::derive."""
+    arg = g.variable(np.arange(6, dtype=np.float64) + 1, [3, 2], "arg1")
+    op = api.sigmoid(arg)
+    (grad,) = g.derive(op, [arg])
+    assert g.to_string(grad) == (
+        "(MUL<DOUBLE>%s)\n"
+        "_`--(MUL<DOUBLE>%s)\n"
+        "_|___`--(SIGMOID<DOUBLE>%s)\n"
+        "_|___|___`--(variable:arg1<DOUBLE>%s)\n"
+        "_|___`--(SUB<DOUBLE>%s)\n"
+        "_|_______`--(EXTEND<DOUBLE>%s)\n"
+        "_|_______|___`--(constant:1<DOUBLE>[1\\1\\1\\1\\1\\1\\1\\1])\n"
+        "_|_______`--(SIGMOID<DOUBLE>%s)\n"
+        "_|___________`--(variable:arg1<DOUBLE>%s)\n"
+        "_`--(constant:1<DOUBLE>%s)") % ((S32,) * 9)
+    op = api.tanh(arg)
+    (grad,) = g.derive(op, [arg])
+    assert g.to_string(grad) == (
+        "(MUL<DOUBLE>%s)\n"
+        "_`--(SUB<DOUBLE>%s)\n"
+        "_|___`--(EXTEND<DOUBLE>%s)\n"
+        "_|___|___`--(constant:1<DOUBLE>[1\\1\\1\\1\\1\\1\\1\\1])\n"
+        "_|___`--(SQUARE<DOUBLE>%s)\n"
+        "_|_______`--(TANH<DOUBLE>%s)\n"
+        "_|___________`--(variable:arg1<DOUBLE>%s)\n"
+        "_`--(constant:1<DOUBLE>%s)") % ((S32,) * 7)
+    a1 = g.variable(np.arange(6, dtype=np.float64), [3, 2], "arg1")
+    a2 = g.variable(np.arange(6, dtype=np.float64), [2, 3], "arg2")
+    op = api.contract(a1, a2)
+    (grad,) = g.derive(op, [a2])
+    assert g.to_string(grad) == (
+        "(PERMUTE<DOUBLE>[2\\3\\1\\1\\1\\1\\1\\1])\n"
+        "_`--(CONTRACT<DOUBLE>[3\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_____`--(constant:1<DOUBLE>[2\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_____`--(variable:arg1<DOUBLE>[3\\2\\1\\1\\1\\1\\1\\1])")
+    img = g.variable(np.arange(6, dtype=np.float64), [3, 2], "arg1")
+    ker = g.variable(np.arange(4, dtype=np.float64), [2, 2], "arg2")
+    op = api.convolution(img, ker, [0, 1])
+    (grad,) = g.derive(op, [ker])
+    assert g.to_string(grad) == (
+        "(CONV<DOUBLE>[2\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_`--(variable:arg1<DOUBLE>[3\\2\\1\\1\\1\\1\\1\\1])\n"
+        "_`--(constant:1<DOUBLE>[2\\1\\1\\1\\1\\1\\1\\1])")
+
+
+def test_derive_of_unrelated_and_self(g, api):
+    x = var(g, [3, 2], np.float64, "x")
+    y = var(g, [3, 2], np.float64, "y")
+    op = api.exp(x)
+    gx, gy, gself = g.derive(op, [x, y, op])
+    assert g.opcode(gx) == "MUL"
+    assert g.opcode(gy) == "BAD_OP" and g.to_string(gy).startswith("(constant:0<DOUBLE>")
+    assert g.to_string(gself).startswith("(constant:1<DOUBLE>")
+    from tenncor_amd import graph
+    with pytest.raises(graph.GraphError) as info:
+        g.derive(g.functor("ARGMAX", [x], rank=0), [x])
+    assert "cannot derive ARGMAX" in str(info.value)
+
+
+def test_mlp_gradient_graph_only_uses_table_opcodes(g, api):
+    """config 1: the GradBuilder's output is an ordinary graph over ops.yml opcodes."""
+    rng = np.random.default_rng(1)
+    x = g.variable(rng.uniform(-1, 1, 30), [10, 3], "x")
+    w0 = g.variable(rng.uniform(-1, 1, 90), [9, 10], "w0")
+    b0 = g.variable(np.zeros(9), [9], "b0")
+    sig0 = api.sigmoid(api.add(api.matmul(x, w0), api.extend(b0, 1, [3])))
+    err = api.square(sig0)
+    grads = g.derive(err, [w0, b0])
+    seen, stack, ops = set(), list(grads), set()
+    while stack:
+        n = stack.pop()
+        if n.id in seen:
+            continue
+        seen.add(n.id)
+        ops.add(g.opcode(n))
+        stack.extend(g.args(n))
+    assert ops <= {"BAD_OP", "MUL", "SUB", "EXTEND", "SIGMOID", "ADD", "MATMUL", "PERMUTE", "REDUCE_SUM", "SQUARE"}
+    assert grads[0].shape[:2] == [9, 10] and grads[1].shape[:2] == [9, 1]
