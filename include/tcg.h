@@ -232,6 +232,17 @@ int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
 	const void* img, const void* kernel, void* out);
+/* The same correlation for the idioms tenncor builds convolutions from
+ * (cfg/tenncor/nn.yml:88-93 pads a singleton axis before CONV;
+ * tenncor/eteq/backprop.hpp:372-439 pads the upstream gradient and slices one
+ * index of the result): the caller promises that `img` is zero outside
+ * [img_lo, img_hi) and asks only for the outputs inside [out_lo, out_hi);
+ * the rest of `out` is left untouched.  NULL boxes mean "everything". */
+int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const uint64_t img_lo[8], const uint64_t img_hi[8],
+	const uint64_t out_lo[8], const uint64_t out_hi[8],
+	const void* img, const void* kernel, void* out);
 
 #ifdef __cplusplus
 }

@@ -37,7 +37,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
-    "tcg_gemm", "tcg_conv",
+    "tcg_gemm", "tcg_conv", "tcg_conv_boxed",
 ]
 
 
@@ -104,6 +104,7 @@ def load():
         "tcg_contract": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
+        "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -333,6 +334,14 @@ class Context:
         r = [int(v) for v in ranks][:RANK_CAP]
         self._check(self.lib.tcg_conv(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
                                       len(r), _u64(r if r else [0]), img, kernel, dst))
+
+    def conv_boxed(self, dtype, imgshape, kshape, ranks, img_box, out_box, img, kernel, dst):
+        """img_box / out_box: (lo[8], hi[8]) or None for the whole extent."""
+        r = [int(v) for v in ranks][:RANK_CAP]
+        ilo, ihi = (_u64(img_box[0]), _u64(img_box[1])) if img_box else (None, None)
+        olo, ohi = (_u64(out_box[0]), _u64(out_box[1])) if out_box else (None, None)
+        self._check(self.lib.tcg_conv_boxed(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
+                                            len(r), _u64(r if r else [0]), ilo, ihi, olo, ohi, img, kernel, dst))
 
 
 class DevBuf:

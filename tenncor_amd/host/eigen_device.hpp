@@ -146,7 +146,20 @@ struct iEigen : public teq::iDeviceRef
 	virtual const void* device_data (void) const = 0;
 	/// device_data() plus the guard odata() carries
 	virtual teq::Once<const void*> odevice (void) const = 0;
+	/// True when the last launch filled only the part of the buffer its
+	/// consumers read (see convolution); such a value is never reused
+	virtual bool is_partial (void) const { return false; }
 };
+
+/// Lifetime given to the node whose launch is being enqueued, and a flag the
+/// launch closure raises when it fills only part of its output
+struct LaunchScope final
+{
+	size_t ttl = 0;
+	bool partial = false;
+};
+
+LaunchScope& launch_scope (void);
 
 using EigenptrT = std::shared_ptr<iEigen>;
 
@@ -350,14 +363,21 @@ struct HipOp final : public iTmpEigen<T>
 			ptrs.push_back(argdata.get());
 			onces.push_back(std::move(argdata));
 		}
+		LaunchScope& scope = launch_scope();
+		scope.ttl = ttl;
+		scope.partial = false;
 		op_(hip_context(), this->data_.get(), ptrs);
+		partial_ = scope.partial;
 		// the guards die here: producers whose last reader this was hand their
 		// buffer back to the pool, after this launch in stream order
 	}
 
+	bool is_partial (void) const override { return partial_; }
+
 private:
 	OpF op_;
 	teq::CTensT args_;
+	bool partial_ = false;
 };
 
 /// An operator evaluated on the host (RAND_UNIF draws from the seeded host
@@ -573,7 +593,7 @@ struct Device final : public teq::iDevice
 		auto& obsdev = static_cast<iEigen&>(tens.device());
 		size_t valid_ttl = obs.nsubs() + cache_ttl;
 		// recompute when an operand moved on or when the value is gone
-		if (obs.prop_version(max_version_) || nullptr == obsdev.device_data())
+		if (obs.prop_version(max_version_) || nullptr == obsdev.device_data() || obsdev.is_partial())
 		{
 			obsdev.assign(std::max<size_t>(1, valid_ttl), memory_);
 		}

@@ -377,6 +377,63 @@ EigenptrT matmul (teq::Shape outshape, const teq::iTensor& a, const teq::iTensor
 	});
 }
 
+/// Where a node's value can be non-zero, known from how it was built: PAD
+/// nodes (and IDENTITY aliases of them) shift and keep their operand's box
+inline void nonzero_box (const teq::iTensor& tens, Shape8& lo, Shape8& hi)
+{
+	auto f = dynamic_cast<const teq::iFunctor*>(&tens);
+	if (nullptr != f && f->get_opcode().code_ == egen::PAD)
+	{
+		auto arg = f->get_args().front();
+		nonzero_box(*arg, lo, hi);
+		PairVecT<teq::DimT> paddings;
+		Packer<PairVecT<teq::DimT>>().unpack(paddings, *f);
+		for (size_t i = 0, n = std::min((size_t) teq::rank_cap, paddings.size()); i < n; ++i)
+		{
+			lo[i] += paddings[i].first;
+			hi[i] += paddings[i].first;
+		}
+		return;
+	}
+	if (nullptr != f && f->get_opcode().code_ == egen::IDENTITY)
+	{
+		nonzero_box(*f->get_args().front(), lo, hi);
+		return;
+	}
+	lo.fill(0);
+	hi = shape8(tens.shape());
+}
+
+/// The part of `self`'s value its consumers read: when every consumer is a
+/// SLICE of it and the node is no evaluation target, the bounding box of
+/// those slices; otherwise everything (false)
+inline bool consumed_window (const Observable* self, const teq::Shape& outshape, Shape8& lo, Shape8& hi)
+{
+	if (nullptr == self || self->nsubs() == 0 || launch_scope().ttl != self->nsubs()) { return false; }
+	bool first = true;
+	for (Observable* sub : self->get_observables())
+	{
+		if (sub->get_opcode().code_ != egen::SLICE) { return false; }
+		auto args = sub->get_args();
+		if (args.size() != 1 || args[0].get() != self) { return false; }
+		PairVecT<teq::DimT> encoding;
+		Packer<PairVecT<teq::DimT>>().unpack(encoding, *sub);
+		for (teq::RankT i = 0; i < teq::rank_cap; ++i)
+		{
+			uint64_t off = 0, ext = outshape.at(i);
+			if (i < encoding.size())
+			{
+				off = std::min(encoding[i].first, (teq::DimT) (outshape.at(i) - 1));
+				ext = std::min(encoding[i].second, (teq::DimT) (outshape.at(i) - off));
+			}
+			lo[i] = first ? off : std::min(lo[i], off);
+			hi[i] = first ? off + ext : std::max(hi[i], off + ext);
+		}
+		first = false;
+	}
+	return true;
+}
+
 template <typename T>
 EigenptrT convolution (teq::Shape outshape, const teq::iTensor& input,
 	const teq::iTensor& kernel, const marsh::iAttributed& attrib)
@@ -406,10 +463,19 @@ EigenptrT convolution (teq::Shape outshape, const teq::iTensor& input,
 	}
 	std::vector<uint64_t> ranks(order.begin(), order.begin() + n);
 	Shape8 ishape = shape8(input.shape()), ks = shape8(kshape);
-	return make_op<T>(outshape, {&input, &kernel}, [ranks, ishape, ks](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
+	// padding the image operand carries is skipped, not multiplied
+	Shape8 ilo, ihi;
+	nonzero_box(input, ilo, ihi);
+	auto self = dynamic_cast<const Observable*>(&attrib);
+	return make_op<T>(outshape, {&input, &kernel},
+	[ranks, ishape, ks, ilo, ihi, self, outshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_conv(ctx, egen::get_type<T>(), ishape.data(), ks.data(), (int) ranks.size(),
-			ranks.data(), args[0], args[1], out));
+		Shape8 olo, ohi;
+		bool windowed = consumed_window(self, outshape, olo, ohi);
+		launch_scope().partial = windowed;
+		hip_check(tcg_conv_boxed(ctx, egen::get_type<T>(), ishape.data(), ks.data(), (int) ranks.size(),
+			ranks.data(), ilo.data(), ihi.data(), windowed ? olo.data() : nullptr,
+			windowed ? ohi.data() : nullptr, args[0], args[1], out));
 	});
 }
 

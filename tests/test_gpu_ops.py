@@ -470,6 +470,50 @@ def test_conv_vs_oracle(ctx, ops, oracle, ishape, kshape, ranks):
     np.testing.assert_array_equal(outi.get(), oracle.conv(ii, ishape, ki, kshape, ranks)[0])
 
 
+def test_conv_boxed_skips_padding_and_unread_outputs(ctx, ops, oracle):
+    """The conv2d idiom and its image-gradient idiom: an image that is zero
+    outside a box, and an output of which only a window is read.  Inside the
+    window the result must equal the plain correlation bit for bit in int32
+    (skipped terms are exact zeros) and to 1e-4 in fp32."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(77)
+    C, W, H, B, O, KW, KH = 3, 7, 6, 2, 4, 3, 2
+    for np_dtype in (np.int32, np.float32):
+        if np_dtype == np.int32:
+            x = rng.integers(-50, 50, C * W * H * B).astype(np.int32)
+            k = rng.integers(-50, 50, O * C * KW * KH).astype(np.int32)
+        else:
+            x = rng.uniform(-1, 1, C * W * H * B).astype(np.float32)
+            k = rng.uniform(-1, 1, O * C * KW * KH).astype(np.float32)
+        dt = capi.dtype_code(np_dtype)
+        # forward idiom: PAD dim 4 by (O-1, O-1), kernel dims -> image dims {4,0,1,2}
+        padded, pshape = oracle.pad(x, [C, W, H, B], [[0, 0]] * 4 + [[O - 1, O - 1]])
+        ref, oshape = oracle.conv(padded, pshape, k, [O, C, KW, KH], [4, 0, 1, 2], wide_acc=np_dtype == np.float32)
+        dimg, dker = ctx.upload(padded), ctx.upload(k)
+        out = ctx.empty(oracle.n_elems(oshape), np_dtype)
+        lo = [0, 0, 0, 0, O - 1, 0, 0, 0]
+        hi = [C, W, H, B, O, 1, 1, 1]
+        ctx.conv_boxed(dt, pshape, [O, C, KW, KH], [4, 0, 1, 2], (lo, hi), None, dimg.ptr, dker.ptr, out.ptr)
+        if np_dtype == np.int32:
+            np.testing.assert_array_equal(out.get(), ref)
+        else:
+            assert_acc_close(out.get(), ref)
+        # output window: only index 1 of dim 4 is asked for; the rest stays as it was
+        sentinel = np.full(oracle.n_elems(oshape), 12345, dtype=np_dtype)
+        ctx.h2d(out.ptr, sentinel)
+        wlo = [0, 0, 0, 0, 1, 0, 0, 0]
+        whi = list(oshape)
+        whi[4] = 2
+        ctx.conv_boxed(dt, pshape, [O, C, KW, KH], [4, 0, 1, 2], (lo, hi), (wlo, whi), dimg.ptr, dker.ptr, out.ptr)
+        got = out.get().reshape(oshape[::-1])
+        want = ref.reshape(oshape[::-1])
+        if np_dtype == np.int32:
+            np.testing.assert_array_equal(got[:, :, :, 1], want[:, :, :, 1])
+        else:
+            assert_acc_close(got[:, :, :, 1], want[:, :, :, 1])
+        assert (got[:, :, :, 0] == 12345).all() and (got[:, :, :, 2:] == 12345).all()
+
+
 def test_api_convolution_golden_on_gpu(ctx, ops):
     fx = EQV["api_convolution"]
     out = ops.convolution(ops.from_host(ctx, np.array(fx["data"]), fx["alist"]),
