@@ -31,9 +31,19 @@ ROWS, COLS = 4096, 16384
 N = ROWS * COLS
 SHAPE = [COLS, ROWS]  # tenncor order: dim 0 fastest
 
-# HBM bytes per launch of the dominant kernel from `rocprofv3 --pmc` runs
-# (FETCH_SIZE + WRITE_SIZE scaled by a plain copy kernel); None until measured.
-MEASURED_TRAFFIC = {}
+# HBM bytes per launch from two `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
+# counter reads for the plain NEG copy of known size: FETCH_SIZE x 2.000,
+# WRITE_SIZE x 1.000.  Per kernel class of the step, bytes per launch.
+MEASURED_TRAFFIC = {
+    "ew_binary_f32": (2 * 262162 + 262144) * 1024,
+    "ew_binary_i32": (2 * 262162 + 262144) * 1024,
+    "ew_unary_f32": (2 * 131096 + 262144) * 1024,
+    "reduce_dim0_f32": (2 * 131089 + 134) * 1024,
+    "reduce_dim0_i32": (2 * 131089 + 134) * 1024,
+    "reduce_dim1_f32": (4 * 65685 + 576) * 1024,   # main launch + second pass
+    "reduce_dim1_i32": (4 * 65685 + 576) * 1024,
+}
 
 
 def algorithmic_bytes():
@@ -141,6 +151,15 @@ def run_extras(ctx, capi):
     ms = ctx.timer_end() / reps
     extra["fused_chain_GBps"] = round(4 * 4 * N / (ms * 1e-3) / 1e9, 1)
     extra["fused_chain_ms"] = round(ms, 4)
+    # plain streaming copy (NEG: N floats in, N floats out), the known-size kernel
+    # that hardware byte counters are scaled by
+    for _ in range(2):
+        ctx.ew_unary("NEG", capi.FLOAT, N, leaves[0].ptr, out.ptr)
+    ctx.timer_begin()
+    for _ in range(reps):
+        ctx.ew_unary("NEG", capi.FLOAT, N, leaves[0].ptr, out.ptr)
+    ms = ctx.timer_end() / reps
+    extra["copy_GBps"] = round(2 * 4 * N / (ms * 1e-3) / 1e9, 1)
     for b in leaves + [out]:
         b.release()
     # 4096^3 fp32 MATMUL (configs[2])

@@ -85,6 +85,32 @@ __device__ __forceinline__ T wave_reduce (T v)
 constexpr int RED_BLOCK = 256;
 constexpr int RED_WAVES = RED_BLOCK / TCG_WAVE;
 
+// launch shape of the column kernel: how many lanes (log2) run along the
+// contiguous dim at most, how many workgroups per CU a launch aims for when it
+// splits the reduced dim, and how many rows a lane keeps in flight.
+// Measured on config 2: 2 workgroups per CU (long row chunks, 8 partial rows)
+// beat 8 per CU by 25 % on the column reduction.
+#ifndef TCG_RED_TXMAX_LOG2
+#define TCG_RED_TXMAX_LOG2 6
+#endif
+#ifndef TCG_RED_BLOCKS_PER_CU
+#define TCG_RED_BLOCKS_PER_CU 2
+#endif
+#ifndef TCG_RED_OUTER_UNROLL
+#define TCG_RED_OUTER_UNROLL 2
+#endif
+// the operand of a reduction was usually written by the node before it, and
+// part of it is still in the last-level cache: plain loads hit there, the
+// non-temporal hint measured 4-15 % slower
+#ifndef TCG_RED_NONTEMPORAL
+#define TCG_RED_NONTEMPORAL 0
+#endif
+#if TCG_RED_NONTEMPORAL
+#define RED_LOAD(ptr) __builtin_nontemporal_load(ptr)
+#else
+#define RED_LOAD(ptr) (*(ptr))
+#endif
+
 // rows of R contiguous elements; block b reduces the part `b % S` of row
 // `b / S` and writes out[row * S + part]
 template <typename T, int OP, bool VEC>
@@ -113,7 +139,7 @@ __global__ __launch_bounds__(RED_BLOCK) void reduce_inner_k (
 #pragma unroll
 			for (int u = 0; u < 4; ++u)
 			{
-				x[u].v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base) + i + u * RED_BLOCK);
+				x[u].v = RED_LOAD(reinterpret_cast<const typename Vec16<T>::type*>(base) + i + u * RED_BLOCK);
 			}
 #pragma unroll
 			for (int u = 0; u < 4; ++u)
@@ -125,7 +151,7 @@ __global__ __launch_bounds__(RED_BLOCK) void reduce_inner_k (
 		for (; i < vhi; i += RED_BLOCK)
 		{
 			VecU<T> x;
-			x.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base) + i);
+			x.v = RED_LOAD(reinterpret_cast<const typename Vec16<T>::type*>(base) + i);
 #pragma unroll
 			for (int e = 0; e < N; ++e) { acc[0] = Red<T,OP>::combine(acc[0], x.e[e]); }
 		}
@@ -174,42 +200,56 @@ __global__ __launch_bounds__(RED_BLOCK) void reduce_outer_k (
 	uint64_t hi = lo + chunk;
 	if (hi > R) { hi = R; }
 
-	T acc[N], acc2[N];
+	constexpr int U = TCG_RED_OUTER_UNROLL; // rows in flight per lane
+	T accs[U][N];
 #pragma unroll
-	for (int e = 0; e < N; ++e) { acc[e] = Red<T,OP>::identity(); acc2[e] = Red<T,OP>::identity(); }
+	for (int u = 0; u < U; ++u)
+	{
+#pragma unroll
+		for (int e = 0; e < N; ++e) { accs[u][e] = Red<T,OP>::identity(); }
+	}
 	if (col < A)
 	{
 		const T* base = in + col + b * A * R;
 		uint64_t r = lo + ty;
 		if constexpr (VEC)
 		{
-			for (; r + TY < hi; r += 2 * TY)
+			for (; r + (U - 1) * TY < hi; r += U * TY)
 			{
-				VecU<T> x, y;
-				x.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base + r * A));
-				y.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base + (r + TY) * A));
+				VecU<T> x[U];
 #pragma unroll
-				for (int e = 0; e < N; ++e)
+				for (int u = 0; u < U; ++u)
 				{
-					acc[e] = Red<T,OP>::combine(acc[e], x.e[e]);
-					acc2[e] = Red<T,OP>::combine(acc2[e], y.e[e]);
+					x[u].v = RED_LOAD(reinterpret_cast<const typename Vec16<T>::type*>(base + (r + u * TY) * A));
+				}
+#pragma unroll
+				for (int u = 0; u < U; ++u)
+				{
+#pragma unroll
+					for (int e = 0; e < N; ++e) { accs[u][e] = Red<T,OP>::combine(accs[u][e], x[u].e[e]); }
 				}
 			}
 			for (; r < hi; r += TY)
 			{
 				VecU<T> x;
-				x.v = __builtin_nontemporal_load(reinterpret_cast<const typename Vec16<T>::type*>(base + r * A));
+				x.v = RED_LOAD(reinterpret_cast<const typename Vec16<T>::type*>(base + r * A));
 #pragma unroll
-				for (int e = 0; e < N; ++e) { acc[e] = Red<T,OP>::combine(acc[e], x.e[e]); }
+				for (int e = 0; e < N; ++e) { accs[0][e] = Red<T,OP>::combine(accs[0][e], x.e[e]); }
 			}
 		}
 		else
 		{
-			for (; r < hi; r += TY) { acc[0] = Red<T,OP>::combine(acc[0], base[r * A]); }
+			for (; r < hi; r += TY) { accs[0][0] = Red<T,OP>::combine(accs[0][0], base[r * A]); }
 		}
 	}
+	T acc[N];
 #pragma unroll
-	for (int e = 0; e < N; ++e) { acc[e] = Red<T,OP>::combine(acc[e], acc2[e]); }
+	for (int e = 0; e < N; ++e)
+	{
+		acc[e] = accs[0][e];
+#pragma unroll
+		for (int u = 1; u < U; ++u) { acc[e] = Red<T,OP>::combine(acc[e], accs[u][e]); }
+	}
 
 	// combine the TY rows of the group through LDS; row stride padded by one
 	// element so that the column walk below is conflict-free
@@ -302,7 +342,7 @@ int launch_outer (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uin
 template <typename T, int OP>
 int reduce_step (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint64_t B)
 {
-	const uint64_t target_blocks = (uint64_t) ctx->num_cus * 8;
+	const uint64_t target_blocks = (uint64_t) ctx->num_cus * TCG_RED_BLOCKS_PER_CU;
 	if (A == 1)
 	{
 		// split rows only when there are too few of them to fill the chip
@@ -330,8 +370,8 @@ int reduce_step (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint
 	bool vec = tcg_aligned16(in) && (A % Vec16<T>::N == 0);
 	const uint32_t N = vec ? Vec16<T>::N : 1;
 	uint64_t lanes = (A + N - 1) / N;
-	uint32_t txlog2 = lanes >= 64 ? 6 : ilog2_floor(lanes);
-	if (((uint64_t) 1 << txlog2) < lanes && txlog2 < 6) { ++txlog2; }
+	uint32_t txlog2 = lanes >= (1u << TCG_RED_TXMAX_LOG2) ? TCG_RED_TXMAX_LOG2 : ilog2_floor(lanes);
+	if (((uint64_t) 1 << txlog2) < lanes && txlog2 < TCG_RED_TXMAX_LOG2) { ++txlog2; }
 	const uint32_t TY = RED_BLOCK >> txlog2;
 	uint64_t col_tiles = (lanes + ((uint64_t) 1 << txlog2) - 1) >> txlog2;
 	uint64_t base_blocks = col_tiles * B;
