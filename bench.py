@@ -128,6 +128,7 @@ def run_gpu(steps, warmup):
     extra = run_extras(ctx, capi)
     arch = ctx.arch
     ctx.close()
+    extra.update(run_graph_configs())
     return wall, per_class, extra, arch
 
 
@@ -190,7 +191,79 @@ def run_extras(ctx, capi):
     extra["permute_4096_GBps"] = round(2 * 4 * M * M / (ms * 1e-3) / 1e9, 1)
     for buf in (a, b, c, d):
         buf.release()
+    # batched CONTRACT np[64,512,512] x np[64,512,512] + PERMUTE {1,0,2} (configs[2])
+    nb, m = 64, 512
+    a = ctx.upload((rng.standard_normal(nb * m * m) / np.sqrt(m)).astype(np.float32))
+    b = ctx.upload((rng.standard_normal(nb * m * m) / np.sqrt(m)).astype(np.float32))
+    c = ctx.empty(nb * m * m, np.float32)
+    d = ctx.empty(nb * m * m, np.float32)
+    for _ in range(2):
+        ctx.matmul(capi.FLOAT, [m, m, nb], [m, m, nb], a.ptr, b.ptr, c.ptr)
+    ctx.timer_begin()
+    for _ in range(reps):
+        ctx.matmul(capi.FLOAT, [m, m, nb], [m, m, nb], a.ptr, b.ptr, c.ptr)
+    ms = ctx.timer_end() / reps
+    extra["matmul_64x512_fp32_TFLOPs"] = round(nb * 2.0 * m ** 3 / (ms * 1e-3) / 1e12, 2)
+    order = [1, 0, 2, 3, 4, 5, 6, 7]
+    for _ in range(2):
+        ctx.permute(capi.FLOAT, [m, m, nb], order, c.ptr, d.ptr)
+    ctx.timer_begin()
+    for _ in range(reps):
+        ctx.permute(capi.FLOAT, [m, m, nb], order, c.ptr, d.ptr)
+    ms = ctx.timer_end() / reps
+    extra["permute_64x512_GBps"] = round(2 * 4 * nb * m * m / (ms * 1e-3) / 1e9, 1)
+    for buf in (a, b, c, d):
+        buf.release()
     return extra
+
+
+def run_graph_configs():
+    """configs[0], [3], [4] through the host graph layer (Functor nodes, the
+    gradient builder, teq::Evaluator + eigen::Device): wall time of
+    evaluate(targets) after re-assigning the input, which forces a full
+    recompute (the recipe of tenncor/bm/benchmark.cpp:377-391)."""
+    from tenncor_amd import graph as tg, configs
+    out = {}
+    rng = np.random.default_rng(0)
+
+    def timed(g, targets, x, fresh, reps):
+        g.evaluate(targets)
+        g.sync()
+        ts = []
+        for _ in range(reps):
+            g.assign(x, fresh())
+            t0 = time.perf_counter()
+            g.evaluate(targets)
+            g.sync()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    g = tg.Graph()
+    targets, x, _ = configs.config1_mlp(g)
+    t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
+    out["config1_mlp_evals_per_sec"] = round(1.0 / t, 1)
+    out["config1_mlp_us_per_eval"] = round(t * 1e6, 1)
+    out["config1_mlp_functors"] = g.count_functors(targets)
+    g.close()
+
+    g = tg.Graph()
+    targets, x, _, flops = configs.config4_lstm(g)
+    xs = rng.uniform(-1, 1, 256 * 64 * 256).astype(np.float32)
+    t = timed(g, targets, x, lambda: xs, 5)
+    out["config4_lstm_ms_per_step"] = round(t * 1e3, 3)
+    out["config4_lstm_gemm_TFLOPs"] = round(flops / t / 1e12, 2)
+    out["config4_lstm_functors"] = g.count_functors(targets)
+    g.close()
+
+    g = tg.Graph()
+    targets, x, _, flops = configs.config5_cnn(g)
+    xs = rng.uniform(0, 1, 128 * 28 * 28).astype(np.float32)
+    t = timed(g, targets, x, lambda: xs, 3)
+    out["config5_cnn_ms_per_step"] = round(t * 1e3, 3)
+    out["config5_cnn_useful_TFLOPs"] = round(flops / t / 1e12, 3)
+    out["config5_cnn_functors"] = g.count_functors(targets)
+    g.close()
+    return out
 
 
 def run_cpu_baseline():

@@ -195,7 +195,13 @@ int tcg_slice (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 /* PAD (cfg/ops.yml:372-412; internal/eigen/operator.hpp:257-275) */
 int tcg_pad (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	const uint64_t before[8], const uint64_t after[8], const void* in, void* out);
-/* REVERSE (cfg/ops.yml:104-105; internal/eigen/operator.hpp:316-333) */
+/* PAD without its zero border: copies `in` to its place inside `out` and
+ * leaves every other element of `out` as it was. For a padded image whose
+ * only readers are tcg_conv_boxed calls clipped to that place (the same
+ * reference operator as tcg_pad; the border is what its readers skip) */
+int tcg_pad_interior (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t before[8], const uint64_t after[8], const void* in, void* out);
+/* REVERSE(cfg/ops.yml:104-105; internal/eigen/operator.hpp:316-333) */
 int tcg_reverse (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 	unsigned rankmask, const void* in, void* out);
 /* STRIDE (cfg/ops.yml:413-438; internal/eigen/operator.hpp:277-293) */

@@ -36,7 +36,7 @@ EXPORTS = [
     "tcg_timer_end", "tcg_event_create", "tcg_event_destroy", "tcg_event_record", "tcg_event_elapsed",
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
-    "tcg_pad", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
+    "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
     "tcg_gemm", "tcg_conv", "tcg_conv_boxed",
 ]
 
@@ -96,6 +96,7 @@ def load():
         "tcg_permute": [vp, i32, u64p, u64p, vp, vp],
         "tcg_slice": [vp, i32, u64p, u64p, u64p, vp, vp],
         "tcg_pad": [vp, i32, u64p, u64p, u64p, vp, vp],
+        "tcg_pad_interior": [vp, i32, u64p, u64p, u64p, vp, vp],
         "tcg_reverse": [vp, i32, u64p, ctypes.c_uint, vp, vp],
         "tcg_stride": [vp, i32, u64p, u64p, u64p, vp, vp],
         "tcg_scatter": [vp, i32, u64p, u64p, u64p, vp, vp],
@@ -300,6 +301,10 @@ class Context:
     def pad(self, dtype, inshape, before, after, src, dst):
         self._check(self.lib.tcg_pad(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(before, 0)),
                                      _u64(shape8(after, 0)), src, dst))
+
+    def pad_interior(self, dtype, inshape, before, after, src, dst):
+        self._check(self.lib.tcg_pad_interior(self.handle, dtype, _u64(shape8(inshape)), _u64(shape8(before, 0)),
+                                              _u64(shape8(after, 0)), src, dst))
 
     def reverse(self, dtype, shape, rank_set, src, dst):
         self._check(self.lib.tcg_reverse(self.handle, dtype, _u64(shape8(shape)), _mask(rank_set), src, dst))

@@ -384,6 +384,25 @@ int tcg_pad (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	return TCG_OK;
 }
 
+int tcg_pad_interior (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
+	const uint64_t before[8], const uint64_t after[8], const void* in, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, inshape && before && after && in && out, "tcg_pad_interior: NULL pointer");
+	CHECK_DIMS(ctx, inshape, "tcg_pad_interior");
+	uint64_t oshape[8];
+	int64_t is[8], os[8];
+	contiguous_strides(inshape, is);
+	for (int d = 0; d < 8; ++d) { oshape[d] = inshape[d] + before[d] + after[d]; }
+	CHECK_DIMS(ctx, oshape, "tcg_pad_interior");
+	contiguous_strides(oshape, os);
+	CopyPlan p;
+	for (int d = 0; d < 8; ++d) { p.dbase += (int64_t) before[d] * os[d]; }
+	plan_finish(p, inshape, is, os, nullptr, nullptr);
+	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_pad_interior"));
+	return TCG_OK;
+}
+
 int tcg_reverse (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 	unsigned rankmask, const void* in, void* out)
 {

@@ -252,6 +252,20 @@ EigenptrT slice (teq::Shape outshape, const teq::TensptrT& in, const marsh::iAtt
 	});
 }
 
+/// True when the value being launched for `self` is read by CONV nodes only,
+/// each taking it as the image operand, and by no evaluation target
+inline bool only_convolved (const Observable* self)
+{
+	if (nullptr == self || self->nsubs() == 0 || launch_scope().ttl != self->nsubs()) { return false; }
+	for (Observable* sub : self->get_observables())
+	{
+		if (sub->get_opcode().code_ != egen::CONV) { return false; }
+		auto args = sub->get_args();
+		if (args.size() != 2 || args[0].get() != self || args[1].get() == self) { return false; }
+	}
+	return true;
+}
+
 template <typename T>
 EigenptrT pad (teq::Shape outshape, const teq::iTensor& in, const marsh::iAttributed& attrib)
 {
@@ -266,8 +280,18 @@ EigenptrT pad (teq::Shape outshape, const teq::iTensor& in, const marsh::iAttrib
 		after[i] = encoding[i].second;
 	}
 	Shape8 ishape = shape8(in.shape());
-	return make_op<T>(outshape, {&in}, [before, after, ishape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
+	auto self = dynamic_cast<const Observable*>(&attrib);
+	return make_op<T>(outshape, {&in}, [before, after, ishape, self](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
+		// convolutions read only the non-zero box of a padded image (see
+		// nonzero_box): when they are the only readers the zero border is
+		// never looked at and need not be written
+		if (only_convolved(self))
+		{
+			launch_scope().partial = true;
+			hip_check(tcg_pad_interior(ctx, egen::get_type<T>(), ishape.data(), before.data(), after.data(), args[0], out));
+			return;
+		}
 		hip_check(tcg_pad(ctx, egen::get_type<T>(), ishape.data(), before.data(), after.data(), args[0], out));
 	});
 }

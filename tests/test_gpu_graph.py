@@ -340,3 +340,36 @@ def test_aliases_casts_and_rand(g, api):
     assert first.min() > 0.25 and first.max() < 3.2
     g.evaluate([r])  # not idempotent: a new draw every evaluation
     assert not np.array_equal(first, r.get())
+
+
+def test_padded_image_read_by_convolutions_and_by_others(g, api, oracle):
+    """A PAD node whose only readers are CONV nodes has its border left
+    unwritten; as soon as anything else reads it (an evaluation target, another
+    operator) it must hold the zeros PAD defines (internal/eigen/operator.hpp:
+    257-275).  The buffer is dirtied first so that a missing border would show."""
+    rng = np.random.default_rng(5)
+    C, W, H, B, O, KW, KH = 2, 6, 5, 2, 3, 3, 2
+    xv = rng.integers(1, 9, C * W * H * B).astype(np.float32)
+    kv = rng.integers(-4, 5, O * C * KW * KH).astype(np.float32)
+    padded_ref, pshape = oracle.pad(xv, [C, W, H, B], [[0, 0]] * 4 + [[O - 1, O - 1]])
+    conv_ref, oshape = oracle.conv(padded_ref, pshape, kv, [O, C, KW, KH], [4, 0, 1, 2])
+    n_pad = oracle.n_elems(pshape)
+    # leave non-zero garbage of the padded size in the pool
+    junk = g.variable(np.full(n_pad, 7.0, np.float32), pshape[:5], "junk")
+    dirty = api.reduce_sum(api.add(junk, 1.0))
+    g.evaluate([dirty])
+    x = g.variable(xv, [C, W, H, B], "x")
+    k = g.variable(kv, [O, C, KW, KH], "k")
+    pad = api.pad(x, [[0, 0]] * 4 + [[O - 1, O - 1]])
+    conv = api.convolution(pad, k, [4, 0, 1, 2])
+    g.evaluate([conv])
+    np.testing.assert_array_equal(conv.get(), conv_ref)
+    # now the padded image itself is asked for too
+    total = api.reduce_sum(pad)
+    g.assign(junk, np.full(n_pad, 5.0, np.float32))
+    g.assign(x, xv)
+    g.evaluate([dirty])
+    g.evaluate([conv, pad, total])
+    np.testing.assert_array_equal(conv.get(), conv_ref)
+    np.testing.assert_array_equal(pad.get(), padded_ref)
+    np.testing.assert_array_equal(total.get(), [xv.sum()])

@@ -514,6 +514,32 @@ def test_conv_boxed_skips_padding_and_unread_outputs(ctx, ops, oracle):
         assert (got[:, :, :, 0] == 12345).all() and (got[:, :, :, 2:] == 12345).all()
 
 
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
+def test_pad_interior_writes_the_operand_and_nothing_else(ctx, oracle, np_dtype):
+    """tcg_pad_interior against PAD: equal to the oracle's padded tensor inside
+    the operand's box, the destination's earlier content everywhere else; a
+    convolution clipped to the box then gives the PAD + CONV result."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(1234)
+    dt = capi.dtype_code(np_dtype)
+    for shape, pads in (([8, 5, 3], [[4, 4], [0, 2], [1, 0]]), ([3, 7, 6, 2], [[0, 0]] * 4 + [[3, 3]]),
+                        ([5], [[2, 6]]), ([4, 4], [[0, 0], [0, 0]])):
+        n = oracle.n_elems(shape)
+        x = rng.integers(1, 90, n).astype(np_dtype)
+        ref, pshape = oracle.pad(x, shape, pads)
+        before = [p[0] for p in pads]
+        after = [p[1] for p in pads]
+        sentinel = np.full(oracle.n_elems(pshape), 77777, dtype=np_dtype)
+        out, src = ctx.upload(sentinel), ctx.upload(x)
+        ctx.pad_interior(dt, shape, before, after, src.ptr, out.ptr)
+        got = out.get()
+        # the oracle's padding is zero and the operand is >= 1: zeros mark the border
+        inside = ref != 0
+        np.testing.assert_array_equal(got[inside], ref[inside])
+        assert (got[~inside] == 77777).all()
+        assert inside.sum() == n
+
+
 def test_api_convolution_golden_on_gpu(ctx, ops):
     fx = EQV["api_convolution"]
     out = ops.convolution(ops.from_host(ctx, np.array(fx["data"]), fx["alist"]),
