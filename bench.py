@@ -227,7 +227,9 @@ def run_graph_configs():
     rng = np.random.default_rng(0)
 
     def timed(g, targets, x, fresh, reps):
-        g.evaluate(targets)
+        for _ in range(2):
+            g.assign(x, fresh())
+            g.evaluate(targets)
         g.sync()
         ts = []
         for _ in range(reps):
@@ -238,31 +240,38 @@ def run_graph_configs():
             ts.append(time.perf_counter() - t0)
         return float(np.median(ts))
 
-    g = tg.Graph()
-    targets, x, _ = configs.config1_mlp(g)
-    t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
-    out["config1_mlp_evals_per_sec"] = round(1.0 / t, 1)
-    out["config1_mlp_us_per_eval"] = round(t * 1e6, 1)
-    out["config1_mlp_functors"] = g.count_functors(targets)
-    g.close()
+    for kind, tag in (("plain", ""), ("replay", "_replay")):
+        # "replay": the evaluator that records a target set's launches on its
+        # second pass and enqueues the recording afterwards
+        tg.set_evaluator(kind)
+        g = tg.Graph()
+        targets, x, _ = configs.config1_mlp(g)
+        t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
+        out["config1_mlp%s_evals_per_sec" % tag] = round(1.0 / t, 1)
+        out["config1_mlp%s_us_per_eval" % tag] = round(t * 1e6, 1)
+        out["config1_mlp_functors"] = g.count_functors(targets)
+        g.close()
 
-    g = tg.Graph()
-    targets, x, _, flops = configs.config4_lstm(g)
-    xs = rng.uniform(-1, 1, 256 * 64 * 256).astype(np.float32)
-    t = timed(g, targets, x, lambda: xs, 5)
-    out["config4_lstm_ms_per_step"] = round(t * 1e3, 3)
-    out["config4_lstm_gemm_TFLOPs"] = round(flops / t / 1e12, 2)
-    out["config4_lstm_functors"] = g.count_functors(targets)
-    g.close()
+        g = tg.Graph()
+        targets, x, _, flops = configs.config4_lstm(g)
+        xs = rng.uniform(-1, 1, 256 * 64 * 256).astype(np.float32)
+        t = timed(g, targets, x, lambda: xs, 5)
+        out["config4_lstm%s_ms_per_step" % tag] = round(t * 1e3, 3)
+        out["config4_lstm%s_gemm_TFLOPs" % tag] = round(flops / t / 1e12, 2)
+        out["config4_lstm_functors"] = g.count_functors(targets)
+        g.close()
 
-    g = tg.Graph()
-    targets, x, _, flops = configs.config5_cnn(g)
-    xs = rng.uniform(0, 1, 128 * 28 * 28).astype(np.float32)
-    t = timed(g, targets, x, lambda: xs, 3)
-    out["config5_cnn_ms_per_step"] = round(t * 1e3, 3)
-    out["config5_cnn_useful_TFLOPs"] = round(flops / t / 1e12, 3)
-    out["config5_cnn_functors"] = g.count_functors(targets)
-    g.close()
+        g = tg.Graph()
+        targets, x, _, flops = configs.config5_cnn(g)
+        xs = rng.uniform(0, 1, 128 * 28 * 28).astype(np.float32)
+        t = timed(g, targets, x, lambda: xs, 3)
+        out["config5_cnn%s_ms_per_step" % tag] = round(t * 1e3, 3)
+        out["config5_cnn%s_useful_TFLOPs" % tag] = round(flops / t / 1e12, 3)
+        out["config5_cnn_functors"] = g.count_functors(targets)
+        if kind == "replay":
+            out["config5_cnn_replay_launches"] = tg.evaluator_stats()["launches"]
+        g.close()
+    tg.set_evaluator("plain")
     return out
 
 

@@ -110,6 +110,31 @@ int tcg_event_destroy (tcg_ctx* ctx, void* event);
 int tcg_event_record (tcg_ctx* ctx, void* event);
 int tcg_event_elapsed (tcg_ctx* ctx, void* start, void* stop, float* ms);
 
+/* ---- recorded launch sequences ---------------------------------------- */
+
+/* What one pass of teq::Evaluator::evaluate enqueues (internal/teq/
+ * evaluator.hpp:11-61: a post-order walk calling eigen::Device::calc, which
+ * runs one operator per functor) can be recorded once and launched again as
+ * a whole, without the host walking the graph: between tcg_capture_begin and
+ * tcg_capture_end every entry point of this header records its kernels
+ * instead of running them, and tcg_alloc hands out memory that belongs to
+ * the recording (tcg_free returns it to the recording, never to the pool), so
+ * that the addresses baked into the recorded launches stay valid for as long
+ * as the graph lives. tcg_h2d, tcg_d2h, tcg_sync and the timers are refused
+ * while recording. tcg_graph_launch enqueues the whole sequence on the
+ * context's stream; a buffer of the recording that the caller wants to own
+ * again afterwards (an output it reads) is taken with tcg_graph_claim and
+ * given back with tcg_free as usual. tcg_graph_destroy returns the memory to
+ * the pool, except blocks still claimed, which stay with their owner. */
+typedef struct tcg_graph tcg_graph;
+int tcg_capture_begin (tcg_ctx* ctx);
+int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out);
+int tcg_capture_abort (tcg_ctx* ctx);
+int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph);
+int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr);
+int tcg_graph_stats (const tcg_graph* graph, uint64_t* nodes, uint64_t* arena_bytes);
+int tcg_graph_destroy (tcg_ctx* ctx, tcg_graph* graph);
+
 /* ---- elementwise ------------------------------------------------------ */
 
 /* ABS..CUBE: `out = eigen::abs<T>(outshape, *in[0])` ... `eigen::cube<T>`
@@ -165,6 +190,48 @@ typedef struct tcg_ew_instr
 /* The value of ACC after the last instruction is written to out. */
 int tcg_ew_fused (tcg_ctx* ctx, int dtype, uint64_t n, int nleaves,
 	const void* const* leaves, int ninstrs, const tcg_ew_instr* program, void* out);
+
+/* A group of elementwise nodes of one shape evaluated in one launch, reading
+ * its operands through views and storing several results: what the closures
+ * of the group's nodes (internal/eigen/device.hpp:304-372), together with the
+ * EXTEND / SLICE / PAD / PERMUTE nodes that only feed them
+ * (internal/eigen/operator.hpp:157-275), compute one node at a time.
+ * A leaf is addressed as ptr[offset + sum_d c[d] * stride[d]] for the output
+ * coordinate c (strides in elements; 0 broadcasts, as EXTEND does); where c[d]
+ * lies outside [lo[d], hi[d]) the leaf reads as zero and memory is not
+ * touched (PAD). Registers hold one value per element; TCG_FX_STORE writes
+ * operand `a` to outs[dst] at the element's position (outputs are dense, of
+ * the given shape). TCG_SELECT takes three operands: a != 0 ? b : c. */
+enum tcg_fx_operand
+{
+	TCG_FX_NONE = 0, TCG_FX_IMM = 1,
+	TCG_FX_LEAF0 = 8,  /* + k, k < TCG_FX_MAX_LEAVES */
+	TCG_FX_REG0 = 32   /* + r, r < TCG_FX_MAX_REGS */
+};
+#define TCG_FX_MAX_LEAVES 8
+#define TCG_FX_MAX_REGS 16
+#define TCG_FX_MAX_INSTRS 64
+#define TCG_FX_MAX_OUTS 4
+#define TCG_FX_STORE 255 /* opcode */
+typedef struct tcg_fx_leaf
+{
+	const void* ptr;
+	int64_t offset;
+	int64_t stride[8];
+	uint64_t lo[8];
+	uint64_t hi[8];
+} tcg_fx_leaf;
+typedef struct tcg_fx_instr
+{
+	uint8_t opcode; /* tcg_opcode (unary, binary, TCG_IDENTITY, TCG_SELECT) or TCG_FX_STORE */
+	uint8_t a, b, c; /* tcg_fx_operand; unused ones TCG_FX_NONE */
+	uint8_t dst;    /* TCG_FX_REG0 + r, or the output index of a store */
+	uint8_t pad_[3];
+	double imm;     /* value of TCG_FX_IMM operands, converted to the dtype */
+} tcg_fx_instr;
+int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
+	int nleaves, const tcg_fx_leaf* leaves, int ninstrs, const tcg_fx_instr* program,
+	int nouts, void* const* outs);
 
 /* ---- reductions ------------------------------------------------------- */
 

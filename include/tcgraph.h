@@ -55,6 +55,19 @@ int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets);
 /* Block until the device has finished everything enqueued */
 int tcr_sync (tcr_graph* g);
 
+/* teq::set_eval (internal/teq/src/evaluator.cpp:9-20): which evaluator the
+ * process uses from now on. TCR_EVAL_PLAIN is teq::Evaluator, the node-by-node
+ * walk; TCR_EVAL_REPLAY records the launches of a set of targets the second
+ * time it is evaluated and enqueues the recording as a whole afterwards. */
+#define TCR_EVAL_PLAIN 0
+#define TCR_EVAL_REPLAY 1
+int tcr_set_evaluator (int kind);
+/* Counters of the replaying evaluator (zeros under TCR_EVAL_PLAIN):
+ * out[0] passes walked node by node, out[1] recordings made, out[2] passes
+ * served by a recording, out[3] passes with nothing to do, out[4] launches in
+ * the latest recording, out[5] device bytes reserved by live recordings */
+int tcr_evaluator_stats (uint64_t out[6]);
+
 /* iTensor::shape / get_meta().type_code / device().data() */
 int tcr_shape (tcr_graph* g, int node, uint64_t shape[8]);
 int tcr_dtype (tcr_graph* g, int node, int* dtype);

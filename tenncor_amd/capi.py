@@ -35,9 +35,10 @@ EXPORTS = [
     "tcg_mem_stats", "tcg_h2d", "tcg_d2h", "tcg_d2d", "tcg_fill_zero", "tcg_sync", "tcg_timer_begin",
     "tcg_timer_end", "tcg_event_create", "tcg_event_destroy", "tcg_event_record", "tcg_event_elapsed",
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
-    "tcg_assign", "tcg_ew_fused", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
+    "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
-    "tcg_gemm", "tcg_conv", "tcg_conv_boxed",
+    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_capture_begin", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
 ]
 
 
@@ -51,6 +52,18 @@ class EwInstr(ctypes.Structure):
     _fields_ = [("opcode", ctypes.c_uint8), ("a", ctypes.c_uint8), ("b", ctypes.c_uint8),
                 ("dst", ctypes.c_uint8), ("pad_", ctypes.c_uint32), ("imm", ctypes.c_double)]
 
+
+class FxLeaf(ctypes.Structure):
+    _fields_ = [("ptr", ctypes.c_void_p), ("offset", ctypes.c_int64), ("stride", ctypes.c_int64 * 8),
+                ("lo", ctypes.c_uint64 * 8), ("hi", ctypes.c_uint64 * 8)]
+
+
+class FxInstr(ctypes.Structure):
+    _fields_ = [("opcode", ctypes.c_uint8), ("a", ctypes.c_uint8), ("b", ctypes.c_uint8), ("c", ctypes.c_uint8),
+                ("dst", ctypes.c_uint8), ("pad_", ctypes.c_uint8 * 3), ("imm", ctypes.c_double)]
+
+
+FX_NONE, FX_IMM, FX_LEAF0, FX_REG0, FX_STORE = 0, 1, 8, 32, 255
 
 _lib = None
 
@@ -90,6 +103,7 @@ def load():
         "tcg_cast": [vp, i32, i32, u64, vp, vp],
         "tcg_assign": [vp, i32, i32, u64, vp, vp],
         "tcg_ew_fused": [vp, i32, u64, i32, vpp, i32, ctypes.POINTER(EwInstr), vp],
+        "tcg_ew_fusedx": [vp, i32, u64p, i32, ctypes.POINTER(FxLeaf), i32, ctypes.POINTER(FxInstr), i32, vpp],
         "tcg_reduce": [vp, i32, i32, u64p, ctypes.c_uint, vp, vp],
         "tcg_argmax": [vp, i32, u64p, i32, vp, vp],
         "tcg_extend": [vp, i32, u64p, u64p, vp, vp],
@@ -106,6 +120,13 @@ def load():
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
+        "tcg_capture_begin": [vp],
+        "tcg_capture_end": [vp, ctypes.POINTER(vp)],
+        "tcg_capture_abort": [vp],
+        "tcg_graph_launch": [vp, vp],
+        "tcg_graph_claim": [vp, vp, vp],
+        "tcg_graph_stats": [vp, u64p, u64p],
+        "tcg_graph_destroy": [vp, vp],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -280,6 +301,31 @@ class Context:
         ptrs = (ctypes.c_void_p * len(leaves))(*leaves)
         self._check(self.lib.tcg_ew_fused(self.handle, dtype, n, len(leaves), ptrs, len(program), instrs, dst))
 
+    def ew_fusedx(self, dtype, shape, leaves, program, outs):
+        """leaves: dicts with ptr, and optionally offset, stride (8 element
+        strides; default: dense over `shape`), lo, hi (default: everything).
+        program: tuples (opcode | "STORE", a, b, c, dst[, imm])."""
+        shp = shape8(shape)
+        dense = [1] * RANK_CAP
+        for d in range(1, RANK_CAP):
+            dense[d] = dense[d - 1] * shp[d - 1]
+        lv = (FxLeaf * len(leaves))()
+        for k, leaf in enumerate(leaves):
+            lv[k].ptr = leaf["ptr"]
+            lv[k].offset = int(leaf.get("offset", 0))
+            for d in range(RANK_CAP):
+                lv[k].stride[d] = int(leaf.get("stride", dense)[d])
+                lv[k].lo[d] = int(leaf.get("lo", [0] * RANK_CAP)[d])
+                lv[k].hi[d] = int(leaf.get("hi", shp)[d])
+        instrs = (FxInstr * len(program))()
+        for i, ins in enumerate(program):
+            instrs[i].opcode = FX_STORE if ins[0] == "STORE" else _opcode(ins[0])
+            instrs[i].a, instrs[i].b, instrs[i].c, instrs[i].dst = ins[1], ins[2], ins[3], ins[4]
+            instrs[i].imm = float(ins[5]) if len(ins) > 5 else 0.0
+        ptrs = (ctypes.c_void_p * len(outs))(*outs)
+        self._check(self.lib.tcg_ew_fusedx(self.handle, dtype, _u64(shp), len(leaves), lv, len(program), instrs,
+                                           len(outs), ptrs))
+
     # ---- reductions ----
     def reduce(self, op, dtype, shape, rank_set, src, dst):
         self._check(self.lib.tcg_reduce(self.handle, _opcode(op), dtype, _u64(shape8(shape)), _mask(rank_set), src, dst))
@@ -347,6 +393,33 @@ class Context:
         olo, ohi = (_u64(out_box[0]), _u64(out_box[1])) if out_box else (None, None)
         self._check(self.lib.tcg_conv_boxed(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
                                             len(r), _u64(r if r else [0]), ilo, ihi, olo, ohi, img, kernel, dst))
+
+
+    # ---- recorded launch sequences ----
+    def capture_begin(self):
+        self._check(self.lib.tcg_capture_begin(self.handle))
+
+    def capture_end(self):
+        g = ctypes.c_void_p()
+        self._check(self.lib.tcg_capture_end(self.handle, ctypes.byref(g)))
+        return g
+
+    def capture_abort(self):
+        self._check(self.lib.tcg_capture_abort(self.handle))
+
+    def graph_launch(self, graph):
+        self._check(self.lib.tcg_graph_launch(self.handle, graph))
+
+    def graph_claim(self, graph, ptr):
+        self._check(self.lib.tcg_graph_claim(self.handle, graph, ptr))
+
+    def graph_stats(self, graph):
+        nodes, nbytes = ctypes.c_uint64(), ctypes.c_uint64()
+        self._check(self.lib.tcg_graph_stats(graph, ctypes.byref(nodes), ctypes.byref(nbytes)))
+        return nodes.value, nbytes.value
+
+    def graph_destroy(self, graph):
+        self._check(self.lib.tcg_graph_destroy(self.handle, graph))
 
 
 class DevBuf:

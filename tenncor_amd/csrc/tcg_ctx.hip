@@ -81,7 +81,6 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	(void) hipSetDevice(ctx->device);
 	(void) hipStreamSynchronize(ctx->stream);
 	for (auto& kv : ctx->block_size) { (void) hipFree(kv.first); }
-	if (ctx->scratch) { (void) hipFree(ctx->scratch); }
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
 	(void) hipEventDestroy(ctx->ev_begin);
 	(void) hipEventDestroy(ctx->ev_end);
@@ -112,10 +111,32 @@ static size_t round_block (size_t bytes)
 	return (bytes + step - 1) / step * step;
 }
 
+static void graph_adopt_block (tcg_ctx* ctx, tcg_graph* g, void* p, size_t sz)
+{
+	g->blocks[p] = sz;
+	g->held.insert(p);
+	g->bytes += sz;
+	ctx->graph_blocks[p] = g;
+}
+
 int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr)
 {
 	if (!ctx || !devptr) { return TCG_ERR_ARG; }
 	size_t sz = round_block(bytes);
+	tcg_graph* cap = ctx->capturing;
+	if (cap)
+	{
+		// blocks the captured sequence has already given back are reused first:
+		// the recorded launches run in the order they were recorded
+		auto git = cap->free_blocks.find(sz);
+		if (git != cap->free_blocks.end() && !git->second.empty())
+		{
+			*devptr = git->second.back();
+			git->second.pop_back();
+			cap->held.insert(*devptr);
+			return TCG_OK;
+		}
+	}
 	auto it = ctx->free_blocks.find(sz);
 	if (it != ctx->free_blocks.end() && !it->second.empty())
 	{
@@ -123,10 +144,16 @@ int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr)
 		it->second.pop_back();
 		ctx->bytes_pooled -= sz;
 		ctx->bytes_in_use += sz;
+		if (cap) { graph_adopt_block(ctx, cap, *devptr, sz); }
 		return TCG_OK;
 	}
 	void* p = nullptr;
 	hipError_t err = hipMalloc(&p, sz);
+	if (err != hipSuccess && cap)
+	{
+		(void) hipGetLastError();
+		return tcg_fail(ctx, TCG_ERR_OOM, "tcg_alloc: %zu bytes while capturing: %s", sz, hipGetErrorString(err));
+	}
 	if (err != hipSuccess)
 	{
 		// give cached blocks back to the driver and retry once
@@ -150,6 +177,7 @@ int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr)
 	}
 	ctx->block_size[p] = sz;
 	ctx->bytes_in_use += sz;
+	if (cap) { graph_adopt_block(ctx, cap, p, sz); }
 	*devptr = p;
 	return TCG_OK;
 }
@@ -163,6 +191,15 @@ int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes)
 	size_t sz = it->second;
 	TCG_REQUIRE(ctx, round_block(bytes) == sz,
 		"tcg_free: %p was allocated with another size (%zu bytes given)", devptr, bytes);
+	auto owner = ctx->graph_blocks.find(devptr);
+	if (owner != ctx->graph_blocks.end())
+	{
+		// stays with its graph; reusable only by the sequence being recorded
+		tcg_graph* g = owner->second;
+		g->held.erase(devptr);
+		if (g == ctx->capturing) { g->free_blocks[sz].push_back(devptr); }
+		return TCG_OK;
+	}
 	ctx->free_blocks[sz].push_back(devptr);
 	ctx->bytes_in_use -= sz;
 	ctx->bytes_pooled += sz;
@@ -182,6 +219,7 @@ int tcg_h2d (tcg_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes)
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (bytes == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, dst_dev && src_host, "tcg_h2d: NULL pointer");
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_h2d: host transfers cannot be part of a captured sequence");
 	if (bytes <= ctx->staging_size / 4)
 	{
 		// small: stage through pinned memory so that the call returns at once
@@ -207,6 +245,7 @@ int tcg_d2h (tcg_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes)
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (bytes == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, dst_host && src_dev, "tcg_d2h: NULL pointer");
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_d2h: host transfers cannot be part of a captured sequence");
 	TCG_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
 	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
 	return TCG_OK;
@@ -253,6 +292,7 @@ int tcg_fill_zero (tcg_ctx* ctx, void* dst_dev, size_t bytes)
 int tcg_sync (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_sync: cannot wait while a sequence is being captured");
 	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
 	return TCG_OK;
 }
@@ -260,6 +300,7 @@ int tcg_sync (tcg_ctx* ctx)
 int tcg_timer_begin (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_timer_begin: timers cannot be part of a captured sequence");
 	TCG_HIP(ctx, hipEventRecord(ctx->ev_begin, ctx->stream));
 	return TCG_OK;
 }
@@ -267,6 +308,7 @@ int tcg_timer_begin (tcg_ctx* ctx)
 int tcg_timer_end (tcg_ctx* ctx, float* ms)
 {
 	if (!ctx || !ms) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_timer_end: timers cannot be part of a captured sequence");
 	TCG_HIP(ctx, hipEventRecord(ctx->ev_end, ctx->stream));
 	TCG_HIP(ctx, hipEventSynchronize(ctx->ev_end));
 	TCG_HIP(ctx, hipEventElapsedTime(ms, ctx->ev_begin, ctx->ev_end));
@@ -292,6 +334,7 @@ int tcg_event_destroy (tcg_ctx* ctx, void* event)
 int tcg_event_record (tcg_ctx* ctx, void* event)
 {
 	if (!ctx || !event) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_event_record: timers cannot be part of a captured sequence");
 	TCG_HIP(ctx, hipEventRecord((hipEvent_t) event, ctx->stream));
 	return TCG_OK;
 }
@@ -304,24 +347,101 @@ int tcg_event_elapsed (tcg_ctx* ctx, void* start, void* stop, float* ms)
 	return TCG_OK;
 }
 
-} // extern "C"
+// ---- captured launch sequences -------------------------------------------
 
-int tcg_scratch (tcg_ctx* ctx, size_t bytes, void** out)
+int tcg_capture_begin (tcg_ctx* ctx)
 {
-	if (bytes > ctx->scratch_size)
-	{
-		if (ctx->scratch)
-		{
-			// earlier launches may still read the old scratch
-			TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
-			TCG_HIP(ctx, hipFree(ctx->scratch));
-			ctx->scratch = nullptr;
-			ctx->scratch_size = 0;
-		}
-		size_t sz = (bytes + (1u << 20) - 1) & ~(size_t) ((1u << 20) - 1);
-		TCG_HIP(ctx, hipMalloc(&ctx->scratch, sz));
-		ctx->scratch_size = sz;
-	}
-	*out = ctx->scratch;
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_capture_begin: a capture is already in progress");
+	// relaxed mode: the pool may still call hipMalloc for a size it has not seen
+	TCG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+	ctx->capturing = new tcg_graph();
 	return TCG_OK;
 }
+
+static void graph_release (tcg_ctx* ctx, tcg_graph* g)
+{
+	if (g->exec) { (void) hipGraphExecDestroy(g->exec); }
+	if (g->graph) { (void) hipGraphDestroy(g->graph); }
+	for (auto& kv : g->blocks)
+	{
+		ctx->graph_blocks.erase(kv.first);
+		if (g->held.count(kv.first)) { continue; } // its owner frees it the ordinary way
+		ctx->free_blocks[kv.second].push_back(kv.first);
+		ctx->bytes_in_use -= kv.second;
+		ctx->bytes_pooled += kv.second;
+	}
+	delete g;
+}
+
+int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out)
+{
+	if (!ctx || !out) { return TCG_ERR_ARG; }
+	*out = nullptr;
+	TCG_REQUIRE(ctx, ctx->capturing, "tcg_capture_end: no capture in progress");
+	tcg_graph* g = ctx->capturing;
+	ctx->capturing = nullptr;
+	g->free_blocks.clear();
+	hipError_t err = hipStreamEndCapture(ctx->stream, &g->graph);
+	if (err == hipSuccess) { err = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0); }
+	size_t nodes = 0;
+	if (err == hipSuccess) { err = hipGraphGetNodes(g->graph, nullptr, &nodes); }
+	if (err != hipSuccess)
+	{
+		(void) hipGetLastError();
+		graph_release(ctx, g);
+		return tcg_fail(ctx, TCG_ERR_HIP, "tcg_capture_end: %s", hipGetErrorString(err));
+	}
+	g->kernels = nodes;
+	*out = g;
+	return TCG_OK;
+}
+
+int tcg_capture_abort (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (!ctx->capturing) { return TCG_OK; }
+	tcg_graph* g = ctx->capturing;
+	ctx->capturing = nullptr;
+	(void) hipStreamEndCapture(ctx->stream, &g->graph);
+	(void) hipGetLastError();
+	graph_release(ctx, g);
+	return TCG_OK;
+}
+
+int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph)
+{
+	if (!ctx || !graph) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_graph_launch: cannot launch while capturing");
+	TCG_HIP(ctx, hipGraphLaunch(graph->exec, ctx->stream));
+	return TCG_OK;
+}
+
+int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr)
+{
+	if (!ctx || !graph) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, graph->blocks.count(devptr), "tcg_graph_claim: %p does not belong to this graph", devptr);
+	graph->held.insert(devptr);
+	return TCG_OK;
+}
+
+int tcg_graph_stats (const tcg_graph* graph, uint64_t* nodes, uint64_t* arena_bytes)
+{
+	if (!graph) { return TCG_ERR_ARG; }
+	if (nodes) { *nodes = graph->kernels; }
+	if (arena_bytes) { *arena_bytes = graph->bytes; }
+	return TCG_OK;
+}
+
+int tcg_graph_destroy (tcg_ctx* ctx, tcg_graph* graph)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (!graph) { return TCG_OK; }
+	TCG_REQUIRE(ctx, graph != ctx->capturing, "tcg_graph_destroy: the graph is still being captured");
+	// a launch of it may still be in flight
+	if (!ctx->capturing) { TCG_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+	graph_release(ctx, graph);
+	return TCG_OK;
+}
+
+} // extern "C"

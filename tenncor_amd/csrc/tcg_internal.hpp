@@ -10,12 +10,28 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <set>
 #include <string>
 #include <vector>
 
 #include "tcg.h"
 
 #define TCG_WAVE 64
+
+// One captured launch sequence and the device memory it owns: every block
+// handed out while it was being captured stays with it (never returns to the
+// context's pool) until the graph is destroyed, because the recorded launches
+// keep addressing it
+struct tcg_graph
+{
+	hipGraph_t graph = nullptr;
+	hipGraphExec_t exec = nullptr;
+	std::map<void*,size_t> blocks;                      // block -> rounded size
+	std::set<void*> held;                               // blocks a caller currently owns
+	std::map<size_t,std::vector<void*>> free_blocks;    // reuse while capturing
+	uint64_t bytes = 0;
+	uint64_t kernels = 0;
+};
 
 struct tcg_ctx
 {
@@ -40,13 +56,13 @@ struct tcg_ctx
 	size_t staging_size = 0;
 	size_t staging_head = 0;
 
-	// scratch for two-pass reductions and operand repacking; grown on demand
-	void* scratch = nullptr;
-	size_t scratch_size = 0;
+	// launch capture: the graph being recorded and, for every block that
+	// belongs to some graph, its owner
+	tcg_graph* capturing = nullptr;
+	std::map<void*,tcg_graph*> graph_blocks;
 };
 
 int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);
-int tcg_scratch (tcg_ctx* ctx, size_t bytes, void** out);
 
 #define TCG_HIP(ctx, call) do {\
 	hipError_t err__ = (call);\

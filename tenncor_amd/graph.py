@@ -27,7 +27,10 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
+    "tcr_set_evaluator", "tcr_evaluator_stats",
 ]
+
+EVAL_PLAIN, EVAL_REPLAY = 0, 1
 
 _lib = None
 
@@ -66,6 +69,8 @@ def load():
         "tcr_args": [vp, i32, i32p, i32],
         "tcr_to_string": [vp, i32, ctypes.c_char_p, ctypes.c_size_t],
         "tcr_count_functors": [vp, i32, i32p, i32p],
+        "tcr_set_evaluator": [i32],
+        "tcr_evaluator_stats": [u64p],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -75,6 +80,26 @@ def load():
     lib.tcr_last_error.restype = ctypes.c_char_p
     _lib = lib
     return lib
+
+
+def set_evaluator(kind):
+    """teq::set_eval: "plain" (node-by-node walk, the default) or "replay"
+    (record a target set's launches on its second evaluation, enqueue the
+    recording afterwards).  Process-wide, like the reference's evaluator slot."""
+    lib = load()
+    code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY}[kind]
+    if lib.tcr_set_evaluator(code) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+
+
+def evaluator_stats():
+    """Counters of the replaying evaluator as a dict (zeros under "plain")."""
+    lib = load()
+    out = (ctypes.c_uint64 * 6)()
+    if lib.tcr_evaluator_stats(out) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+    keys = ("plain", "recorded", "replayed", "skipped", "launches", "reserved_bytes")
+    return dict(zip(keys, [int(v) for v in out]))
 
 
 def _ints(vals):

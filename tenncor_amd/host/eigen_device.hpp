@@ -110,6 +110,25 @@ struct Expirable final
 		if (ttl_ < ttl) { ttl_ = ttl; }
 	}
 
+	/// Become the owner of `ptr` (a buffer a replayed launch sequence has just
+	/// filled) with `ttl` reads left; whatever was held before is returned
+	void adopt (RTMemptrT& memory, T* ptr, size_t nelems, size_t ttl)
+	{
+		if (nullptr == ptr || 0 == ttl)
+		{
+			expire();
+			return;
+		}
+		if (ptr_ != ptr)
+		{
+			expire();
+			ptr_ = ptr;
+			size_ = sizeof(T) * nelems;
+			allocator_ = memory;
+		}
+		ttl_ = ttl;
+	}
+
 private:
 	size_t ttl_ = 0;
 	T* ptr_ = nullptr;
@@ -149,6 +168,24 @@ struct iEigen : public teq::iDeviceRef
 	/// True when the last launch filled only the part of the buffer its
 	/// consumers read (see convolution); such a value is never reused
 	virtual bool is_partial (void) const { return false; }
+
+	// what recording an evaluation and replaying it needs (ReplayEvaluator)
+	/// Buffer and reads left, as an evaluation pass leaves them
+	struct LifeState final
+	{
+		void* ptr = nullptr;
+		size_t ttl = 0;
+	};
+	/// False for values produced on the host, which a recording cannot hold
+	virtual bool replayable (void) const { return true; }
+	/// Forget the current value without counting as a read
+	virtual void drop (void) {}
+	virtual LifeState save_life (void) const { return LifeState(); }
+	/// Put back the state save_life() saw after the recorded launches have
+	/// been enqueued again; `graph` owns state.ptr
+	virtual void restore_life (const LifeState&, RTMemptrT&, tcg_graph*) {}
+	/// Host-side effects of a launch that was replayed rather than issued
+	virtual void replayed (void) {}
 };
 
 /// Lifetime given to the node whose launch is being enqueued, and a flag the
@@ -189,6 +226,15 @@ struct CacheEigen final : public iPermEigen
 	void assign (size_t ttl, RTMemptrT& runtime) override { data_->assign(ttl, runtime); }
 	const void* device_data (void) const override { return data_->device_data(); }
 	teq::Once<const void*> odevice (void) const override { return teq::Once<const void*>(device_data()); }
+	bool is_partial (void) const override { return data_->is_partial(); }
+	bool replayable (void) const override { return data_->replayable(); }
+	void drop (void) override { data_->drop(); }
+	LifeState save_life (void) const override { return data_->save_life(); }
+	void restore_life (const LifeState& state, RTMemptrT& memory, tcg_graph* graph) override
+	{
+		data_->restore_life(state, memory, graph);
+	}
+	void replayed (void) override { data_->replayed(); }
 private:
 	EigenptrT data_;
 };
@@ -204,6 +250,7 @@ struct SrcRef final : public iPermEigen
 
 	~SrcRef (void)
 	{
+		global::note_structure_change();
 		if (dev_) { tcg_free(hip_context(), dev_, host_.size() * sizeof(T)); }
 	}
 
@@ -313,6 +360,26 @@ struct iTmpEigen : public iEigen
 		return teq::Once<const void*>(data_.get(), [this] { data_.tick(); });
 	}
 
+	void drop (void) override { data_.expire(); }
+
+	iEigen::LifeState save_life (void) const override
+	{
+		iEigen::LifeState out;
+		out.ptr = data_.get();
+		out.ttl = data_.get_ttl();
+		return out;
+	}
+
+	void restore_life (const iEigen::LifeState& state, RTMemptrT& memory, tcg_graph* graph) override
+	{
+		if (nullptr != state.ptr && state.ttl > 0)
+		{
+			hip_check(tcg_graph_claim(hip_context(), graph, state.ptr));
+		}
+		data_.adopt(memory, (T*) state.ptr, nelems_, state.ttl);
+		mirror_valid_ = false;
+	}
+
 protected:
 	T* sync_mirror (void) const
 	{
@@ -408,6 +475,8 @@ struct HostOp final : public iTmpEigen<T>
 		this->mirror_valid_ = true;
 	}
 
+	bool replayable (void) const override { return false; }
+
 private:
 	OpF op_;
 	teq::CTensT args_;
@@ -441,6 +510,17 @@ struct iRefEigen : public iEigen
 	{
 		if (ref_ttl_ < ttl) { ref_ttl_ = ttl; }
 	}
+
+	void drop (void) override { ref_ttl_ = 0; }
+
+	LifeState save_life (void) const override
+	{
+		LifeState out;
+		out.ttl = ref_ttl_;
+		return out;
+	}
+
+	void restore_life (const LifeState& state, RTMemptrT&, tcg_graph*) override { ref_ttl_ = state.ttl; }
 
 protected:
 	teq::iTensor* ref_;
@@ -523,6 +603,12 @@ struct TensAssign final : public iRefEigen
 		void* dst = static_cast<SrcRef<T>&>(ref_->device()).device_data_mut();
 		hip_check(tcg_assign(hip_context(), opcode_, egen::get_type<T>(), ref_->shape().n_elems(), dst, src));
 	}
+	void replayed (void) override
+	{
+		// the recorded kernel has updated the leaf's device copy again
+		static_cast<iMutableLeaf*>(ref_)->upversion(arg_->get_meta().state_version() + 1);
+		static_cast<SrcRef<T>&>(ref_->device()).device_data_mut();
+	}
 private:
 	const teq::iTensor* arg_;
 	int opcode_;
@@ -603,8 +689,19 @@ struct Device final : public teq::iDevice
 		}
 	}
 
+	/// calc() without the freshness test: always launches
+	void calc_forced (teq::iTensor& tens, size_t cache_ttl)
+	{
+		auto& obs = static_cast<Observable&>(tens);
+		auto& obsdev = static_cast<iEigen&>(tens.device());
+		obs.prop_version(max_version_);
+		obsdev.assign(std::max<size_t>(1, obs.nsubs() + cache_ttl), memory_);
+	}
+
 	/// Block until everything enqueued so far has run
 	void sync (void) { hip_check(tcg_sync(hip_context())); }
+
+	RTMemptrT& memory (void) { return memory_; }
 
 	size_t max_version_;
 

@@ -147,6 +147,7 @@ struct Functor final : public eigen::Observable
 
 	~Functor (void)
 	{
+		global::note_structure_change();
 		for (teq::TensptrT child : args_)
 		{
 			if (auto f = dynamic_cast<eigen::Observable*>(child.get())) { f->unsubscribe(this); }
@@ -168,6 +169,7 @@ struct Functor final : public eigen::Observable
 			global::throw_errf("cannot replace argument %d when only there are only %d available",
 				(int) index, (int) args_.size());
 		}
+		global::note_structure_change();
 		uninitialize();
 		teq::Shape nexshape = arg->shape();
 		teq::Shape curshape = args_[index]->shape();
@@ -242,6 +244,7 @@ struct Functor final : public eigen::Observable
 	void cache_init (void) override
 	{
 		if (cache_data_) { return; }
+		global::note_structure_change();
 		cache_data_ = true;
 		ref_ = nullptr;
 		must_initialize();

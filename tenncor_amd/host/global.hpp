@@ -92,6 +92,17 @@ inline void note_version (size_t v)
 	if (v > last_version()) { last_version() = v; }
 }
 
+// Counts events that make remembered node pointers unsafe (a node destroyed,
+// an operand replaced, a launch closure rebuilt); whoever caches anything per
+// node compares it with the value seen when the cache was filled
+size_t& structure_epoch (void);
+
+inline void note_structure_change (void) { ++structure_epoch(); }
+
+// True once the process has begun to exit: device resources are then left to
+// the driver rather than released one by one
+bool& process_exiting (void);
+
 // Seeded generator behind RAND_UNIF (host side, like the reference)
 using RandEngineT = std::default_random_engine;
 RandEngineT& get_generator (void);

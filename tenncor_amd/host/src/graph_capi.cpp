@@ -4,6 +4,7 @@
 #include <sstream>
 
 #include "eteq.hpp"
+#include "replay_eval.hpp"
 
 struct tcr_graph
 {
@@ -196,6 +197,37 @@ int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets)
 int tcr_sync (tcr_graph*)
 {
 	return guarded([&] { eigen::hip_check(tcg_sync(eigen::hip_context())); });
+}
+
+int tcr_set_evaluator (int kind)
+{
+	return guarded([&]
+	{
+		switch (kind)
+		{
+			case TCR_EVAL_PLAIN: teq::set_eval(new teq::Evaluator()); break;
+			case TCR_EVAL_REPLAY: teq::set_eval(new eigen::ReplayEvaluator()); break;
+			default: global::fatalf("unknown evaluator kind %d", kind);
+		}
+	});
+}
+
+int tcr_evaluator_stats (uint64_t out[6])
+{
+	return guarded([&]
+	{
+		std::fill(out, out + 6, 0);
+		if (auto replay = dynamic_cast<eigen::ReplayEvaluator*>(&teq::get_eval()))
+		{
+			auto& st = replay->stats();
+			out[0] = st.plain;
+			out[1] = st.recorded;
+			out[2] = st.replayed;
+			out[3] = st.skipped;
+			out[4] = st.launches;
+			out[5] = st.reserved_bytes;
+		}
+	});
 }
 
 int tcr_shape (tcr_graph* g, int node, uint64_t shape[8])

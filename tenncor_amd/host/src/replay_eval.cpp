@@ -1,0 +1,258 @@
+// Recording and replaying whole evaluation passes (see replay_eval.hpp).
+#include "replay_eval.hpp"
+
+#include <algorithm>
+
+namespace eigen
+{
+
+namespace
+{
+
+/// Functors under the targets in the order the plain evaluator computes them
+/// (children first, internal/teq/evaluator.hpp:33-45), and the leaves
+struct Collector final : public teq::iOnceTraveler
+{
+	std::vector<Observable*> funcs_;
+	std::vector<teq::iLeaf*> leaves_;
+
+private:
+	void visit_leaf (teq::iLeaf& leaf) override { leaves_.push_back(&leaf); }
+
+	void visit_func (teq::iFunctor& func) override
+	{
+		auto dependencies = func.get_args();
+		teq::multi_visit(*this, dependencies);
+		funcs_.push_back(static_cast<Observable*>(&func));
+	}
+};
+
+}
+
+struct ReplayEvaluator::Plan final
+{
+	std::vector<Observable*> funcs;
+	std::vector<iEigen*> devs;
+	std::vector<iEigen::LifeState> after;
+	std::vector<iEigen*> effects; // launches with host-side effects (ASSIGN*)
+	std::vector<iEigen*> targets;
+	std::vector<teq::iLeaf*> leaves;
+	std::vector<const void*> leaf_ptrs;
+	std::vector<size_t> leaf_versions;
+	tcg_graph* graph = nullptr;
+	uint64_t bytes = 0;
+	bool fresh = true;
+};
+
+ReplayEvaluator::ReplayEvaluator (size_t warm_passes, size_t max_plans) :
+	warm_passes_(warm_passes), max_plans_(std::max<size_t>(1, max_plans)),
+	epoch_(global::structure_epoch()) {}
+
+ReplayEvaluator::~ReplayEvaluator (void)
+{
+	clear();
+}
+
+void ReplayEvaluator::release (Plan& plan)
+{
+	if (nullptr != plan.graph && false == global::process_exiting())
+	{
+		tcg_graph_destroy(hip_context(), plan.graph);
+	}
+	plan.graph = nullptr;
+}
+
+void ReplayEvaluator::clear (void)
+{
+	for (auto& kv : slots_)
+	{
+		if (kv.second.plan) { release(*kv.second.plan); }
+	}
+	slots_.clear();
+	stats_.reserved_bytes = 0;
+}
+
+void ReplayEvaluator::plain (teq::iDevice& device, const teq::TensSetT& targets, const teq::TensSetT& ignored)
+{
+	++stats_.plain;
+	plain_.evaluate(device, targets, ignored);
+}
+
+void ReplayEvaluator::evict (void)
+{
+	size_t live = 0;
+	for (auto& kv : slots_) { live += (nullptr != kv.second.plan); }
+	while (live > max_plans_)
+	{
+		Slot* oldest = nullptr;
+		for (auto& kv : slots_)
+		{
+			if (kv.second.plan && (nullptr == oldest || kv.second.last_used < oldest->last_used))
+			{
+				oldest = &kv.second;
+			}
+		}
+		stats_.reserved_bytes -= oldest->plan->bytes;
+		release(*oldest->plan);
+		oldest->plan = nullptr;
+		oldest->seen = 0;
+		--live;
+	}
+}
+
+void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targets, const teq::TensSetT& ignored)
+{
+	auto gpu = dynamic_cast<Device*>(&device);
+	if (nullptr == gpu || false == ignored.empty() || targets.empty())
+	{
+		plain(device, targets, ignored);
+		return;
+	}
+	if (epoch_ != global::structure_epoch())
+	{
+		// some node went away or was rewired: remembered pointers may dangle
+		clear();
+		epoch_ = global::structure_epoch();
+	}
+	KeyT key;
+	key.reserve(targets.size());
+	for (teq::iTensor* t : targets)
+	{
+		if (nullptr != t) { key.push_back(t); }
+	}
+	std::sort(key.begin(), key.end());
+	Slot& slot = slots_[key];
+	slot.last_used = ++clock_;
+	if (slot.unplannable)
+	{
+		plain(device, targets, ignored);
+		return;
+	}
+	if (nullptr == slot.plan)
+	{
+		if (slot.seen++ < warm_passes_)
+		{
+			plain(device, targets, ignored);
+			return;
+		}
+		slot.plan = record(*gpu, key, targets);
+		if (nullptr == slot.plan)
+		{
+			slot.unplannable = true;
+			plain(device, targets, ignored);
+			return;
+		}
+		stats_.reserved_bytes += slot.plan->bytes;
+		evict();
+	}
+	if (false == replay(*gpu, *slot.plan))
+	{
+		stats_.reserved_bytes -= slot.plan->bytes;
+		release(*slot.plan);
+		slot.plan = nullptr;
+		slot.unplannable = true;
+		plain(device, targets, ignored);
+	}
+}
+
+std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, const KeyT& key, const teq::TensSetT& targets)
+{
+	Collector collector;
+	teq::multi_visit(collector, key);
+	if (collector.funcs_.empty()) { return nullptr; }
+	auto plan = std::make_unique<Plan>();
+	plan->funcs = collector.funcs_;
+	plan->leaves = collector.leaves_;
+	for (Observable* f : plan->funcs)
+	{
+		// device() builds the launch closure of a functor that has none yet
+		auto dev = &static_cast<iEigen&>(f->device());
+		if (false == dev->replayable()) { return nullptr; }
+		plan->devs.push_back(dev);
+		if (false == egen::is_idempotent((egen::_GENERATED_OPCODE) f->get_opcode().code_))
+		{
+			plan->effects.push_back(dev);
+		}
+		if (targets.count(f)) { plan->targets.push_back(dev); }
+	}
+	// leaves reach the device before recording starts: uploads are not recorded
+	for (teq::iLeaf* leaf : plan->leaves)
+	{
+		plan->leaf_ptrs.push_back(eigen_ref(*leaf).device_data());
+		plan->leaf_versions.push_back(leaf->get_meta().state_version());
+	}
+	// every value under the targets is recomputed into memory of the recording
+	for (iEigen* dev : plan->devs) { dev->drop(); }
+	tcg_ctx* ctx = hip_context();
+	hip_check(tcg_capture_begin(ctx));
+	bool ok = true;
+	try
+	{
+		for (Observable* f : plan->funcs)
+		{
+			device.calc_forced(*f, (size_t) (targets.count(f) > 0));
+		}
+	}
+	catch (...)
+	{
+		// the node-by-node pass that follows reports whatever went wrong
+		ok = false;
+	}
+	if (ok)
+	{
+		ok = TCG_OK == tcg_capture_end(ctx, &plan->graph);
+	}
+	else
+	{
+		tcg_capture_abort(ctx);
+	}
+	if (false == ok)
+	{
+		for (iEigen* dev : plan->devs) { dev->drop(); }
+		return nullptr;
+	}
+	plan->after.reserve(plan->devs.size());
+	for (iEigen* dev : plan->devs) { plan->after.push_back(dev->save_life()); }
+	uint64_t launches = 0;
+	tcg_graph_stats(plan->graph, &launches, &plan->bytes);
+	++stats_.recorded;
+	stats_.launches = launches;
+	return plan;
+}
+
+bool ReplayEvaluator::replay (Device& device, Plan& plan)
+{
+	bool stale = plan.fresh || false == plan.effects.empty();
+	for (size_t i = 0, n = plan.leaves.size(); i < n; ++i)
+	{
+		// uploads a leaf whose host copy moved on
+		if (eigen_ref(*plan.leaves[i]).device_data() != plan.leaf_ptrs[i]) { return false; }
+		size_t version = plan.leaves[i]->get_meta().state_version();
+		if (version != plan.leaf_versions[i])
+		{
+			plan.leaf_versions[i] = version;
+			stale = true;
+		}
+	}
+	for (size_t i = 0, n = plan.targets.size(); i < n && false == stale; ++i)
+	{
+		stale = nullptr == plan.targets[i]->device_data();
+	}
+	if (false == stale)
+	{
+		++stats_.skipped;
+		return true;
+	}
+	for (Observable* f : plan.funcs) { f->prop_version(device.max_version_); }
+	hip_check(tcg_graph_launch(hip_context(), plan.graph));
+	for (size_t i = 0, n = plan.devs.size(); i < n; ++i)
+	{
+		plan.devs[i]->restore_life(plan.after[i], device.memory(), plan.graph);
+	}
+	for (iEigen* dev : plan.effects) { dev->replayed(); }
+	plan.fresh = false;
+	++stats_.replayed;
+	return true;
+}
+
+}

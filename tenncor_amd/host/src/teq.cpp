@@ -2,6 +2,7 @@
 // internal/teq/src/derive.cpp).
 #include "teq.hpp"
 
+#include <cstdlib>
 #include <list>
 
 namespace global
@@ -17,6 +18,18 @@ size_t& last_version (void)
 {
 	static size_t version = 0;
 	return version;
+}
+
+size_t& structure_epoch (void)
+{
+	static size_t epoch = 0;
+	return epoch;
+}
+
+bool& process_exiting (void)
+{
+	static bool exiting = false;
+	return exiting;
 }
 
 RandEngineT& get_generator (void)
@@ -50,6 +63,9 @@ TravEvaluator::TravEvaluator (iDevice& device, const TensSetT& targets, const Te
 static std::unique_ptr<iEvaluator>& eval_slot (void)
 {
 	static std::unique_ptr<iEvaluator> slot;
+	// registered after the slot exists, so it runs before the slot is destroyed
+	static bool registered = (std::atexit([] { global::process_exiting() = true; }), true);
+	(void) registered;
 	return slot;
 }
 

@@ -1,0 +1,287 @@
+"""Recorded launch sequences (tcg_capture_* / tcg_graph_*) and the evaluator
+built on them (eigen::ReplayEvaluator, the replacement for the node-by-node
+walk of internal/teq/evaluator.hpp:11-61).
+
+A replay must give what issuing the same calls one by one gives, bit for bit:
+the same kernels run with the same arguments.  Every test replays several
+times, with ordinary launches and synchronisations of the same context between
+the replays, and checks every replay against the eagerly computed result.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+with open(os.path.join(GOLDEN, "equation_vectors.json")) as f:
+    EQV = json.load(f)
+
+
+@pytest.fixture()
+def ctx():
+    from tenncor_amd import capi
+    c = capi.Context(0)
+    yield c
+    c.close()
+
+
+def chain(ctx, capi, M, K, N, a, b, bias, work, out_sum, out_max):
+    """matmul -> + bias row -> tanh -> reductions; uses pool temporaries inside
+    tcg_reduce and tcg_extend targets allocated by the caller."""
+    ctx.matmul(capi.FLOAT, [K, M], [N, K], a, b, work[0])
+    ctx.extend(capi.FLOAT, [N], [1, M], bias, work[1])
+    ctx.ew_binary("ADD", capi.FLOAT, M * N, work[0], work[1], work[2])
+    ctx.ew_unary("TANH", capi.FLOAT, M * N, work[2], work[0])
+    ctx.reduce("REDUCE_SUM", capi.FLOAT, [N, M], [1], work[0], out_sum)
+    ctx.reduce("REDUCE_MAX", capi.FLOAT, [N, M], [0, 1], work[0], out_max)
+
+
+def test_recorded_sequence_replays_bit_exact(ctx):
+    from tenncor_amd import capi
+    rng = np.random.default_rng(11)
+    M, K, N = 96, 200, 160
+    av = rng.uniform(-1, 1, M * K).astype(np.float32)
+    bv = rng.uniform(-1, 1, K * N).astype(np.float32)
+    cv = rng.uniform(-1, 1, N).astype(np.float32)
+    a, b, bias = ctx.upload(av), ctx.upload(bv), ctx.upload(cv)
+    # eager pass, ordinary pool memory
+    work = [ctx.empty(M * N, np.float32) for _ in range(3)]
+    s_eager, m_eager = ctx.empty(N, np.float32), ctx.empty(1, np.float32)
+    chain(ctx, capi, M, K, N, a.ptr, b.ptr, bias.ptr, [w.ptr for w in work], s_eager.ptr, m_eager.ptr)
+    want_s, want_m = s_eager.get(), m_eager.get()
+    in_use_before, _ = ctx.mem_stats()
+
+    # recorded pass: buffers allocated while recording belong to the recording
+    ctx.capture_begin()
+    rwork = [ctx.alloc(M * N * 4) for _ in range(3)]
+    rs, rm = ctx.alloc(N * 4), ctx.alloc(4)
+    chain(ctx, capi, M, K, N, a.ptr, b.ptr, bias.ptr, rwork, rs, rm)
+    for p in rwork:
+        ctx.free(p, M * N * 4)
+    with pytest.raises(capi.TcgError):
+        ctx.sync()              # refused while recording
+    with pytest.raises(capi.TcgError):
+        ctx.d2h(rs, N, np.float32)
+    graph = ctx.capture_end()
+    nodes, nbytes = ctx.graph_stats(graph)
+    assert nodes >= 6 and nbytes >= 3 * M * N * 4
+    # recording runs nothing
+    for rep in range(4):
+        ctx.graph_launch(graph)
+        np.testing.assert_array_equal(ctx.d2h(rs, N, np.float32), want_s)
+        np.testing.assert_array_equal(ctx.d2h(rm, 1, np.float32), want_m)
+        # ordinary work and a new input between replays
+        av = rng.uniform(-1, 1, M * K).astype(np.float32)
+        ctx.h2d(a.ptr, av)
+        scratch = ctx.empty(M * N, np.float32)
+        ctx.ew_unary("NEG", capi.FLOAT, M * N, work[0].ptr, scratch.ptr)
+        chain(ctx, capi, M, K, N, a.ptr, b.ptr, bias.ptr, [w.ptr for w in work], s_eager.ptr, m_eager.ptr)
+        ctx.sync()
+        want_s, want_m = s_eager.get(), m_eager.get()
+        scratch.release()
+    # memory of the recording returns to the pool with it, claimed blocks stay
+    ctx.graph_claim(graph, rs)
+    ctx.graph_destroy(graph)
+    ctx.free(rs, N * 4)
+    ctx.free(rm, 4)  # given back after its graph is gone: ordinary pool block by now
+    in_use_after, _ = ctx.mem_stats()
+    assert in_use_after == in_use_before
+
+
+def test_capture_abort_and_errors(ctx):
+    from tenncor_amd import capi
+    x = ctx.upload(np.ones(64, np.float32))
+    ctx.capture_begin()
+    with pytest.raises(capi.TcgError):
+        ctx.capture_begin()
+    tmp = ctx.alloc(256)
+    ctx.ew_unary("NEG", capi.FLOAT, 64, x.ptr, tmp)
+    ctx.capture_abort()
+    # nothing ran, nothing leaked, the context still works
+    y = ctx.empty(64, np.float32)
+    ctx.ew_unary("NEG", capi.FLOAT, 64, x.ptr, y.ptr)
+    np.testing.assert_array_equal(y.get(), -np.ones(64, np.float32))
+    with pytest.raises(capi.TcgError):
+        ctx.capture_end()
+
+
+# ---- the evaluator ---------------------------------------------------------
+
+@pytest.fixture()
+def replay_graph():
+    from tenncor_amd import graph
+    graph.set_evaluator("replay")
+    g = graph.Graph()
+    try:
+        yield g, graph.Api(g), graph
+    finally:
+        g.close()
+        graph.set_evaluator("plain")
+
+
+def mlp(g, api, fx, np_dtype):
+    x = g.variable(np.array(fx["in_data"], np_dtype), [10, 3], "in")
+    w0 = g.variable(np.array(fx["w0_data"], np_dtype), [9, 10], "w0")
+    b0 = g.variable(np.array(fx["b0_data"], np_dtype), [9], "b0")
+    w1 = g.variable(np.array(fx["w1_data"], np_dtype), [5, 9], "w1")
+    b1 = g.variable(np.array(fx["b1_data"], np_dtype), [5], "b1")
+    out = g.variable(np.array(fx["out_data"], np_dtype), [5, 3], "out")
+    l0 = api.sigmoid(api.add(api.matmul(x, w0), api.extend(b0, 1, [3])))
+    l1 = api.sigmoid(api.add(api.matmul(l0, w1), api.extend(b1, 1, [3])))
+    err = api.pow(api.sub(out, l1), 2.0)
+    grads = g.derive(err, [w0, b0, w1, b1])
+    return x, [w0, b0, w1, b1], err, grads
+
+
+def test_replayed_mlp_matches_golden_and_plain_walk(replay_graph):
+    """tenncor/test/test_equation.cpp:482-706 evaluated five times with new
+    inputs: passes 1 walks node by node, pass 2 records, later ones replay."""
+    g, api, graph = replay_graph
+    fx = EQV["sigmoid_mlp_fast"]
+    x, leaves, err, grads = mlp(g, api, fx, np.float64)
+    targets = [err] + grads
+    rng = np.random.default_rng(3)
+    x0 = np.array(fx["in_data"], np.float64)
+    inputs = [x0, rng.uniform(-1, 1, 30), rng.uniform(-1, 1, 30), x0, rng.uniform(-1, 1, 30), x0]
+    got = []
+    for xv in inputs:
+        g.assign(x, xv)
+        g.evaluate(targets)
+        got.append([t.get().copy() for t in targets])
+    st = graph.evaluator_stats()
+    assert st["plain"] == 1 and st["recorded"] == 1 and st["replayed"] == 5 and st["launches"] > 20
+    for key, val in zip(("expect_gw0", "expect_gb0", "expect_gw1", "expect_gb1"), got[0][1:]):
+        np.testing.assert_allclose(val, np.array(fx[key]), rtol=1e-12)
+    # same inputs, same launches: identical bits whether walked or replayed
+    for i in (3, 5):
+        for a, b in zip(got[0], got[i]):
+            np.testing.assert_array_equal(a, b)
+    # nothing moved: nothing to do
+    g.evaluate(targets)
+    assert graph.evaluator_stats()["skipped"] == 1
+    for a, t in zip(got[5], targets):
+        np.testing.assert_array_equal(a, t.get())
+    # the other inputs against the plain evaluator on a second graph
+    graph.set_evaluator("plain")
+    g2 = graph.Graph()
+    api2 = graph.Api(g2)
+    x2, _, err2, grads2 = mlp(g2, api2, fx, np.float64)
+    for i in (1, 2, 4):
+        g2.assign(x2, inputs[i])
+        g2.evaluate([err2] + grads2)
+        for a, t in zip(got[i], [err2] + grads2):
+            np.testing.assert_array_equal(a, t.get())
+    g2.close()
+
+
+def test_replayed_training_loop_updates_leaves_in_place(replay_graph):
+    """sgd (cfg/tenncor/approx.yml:52) through ASSIGN_SUB nodes: the recorded
+    step must keep moving the weights, and the host view must follow."""
+    g, api, graph = replay_graph
+    rng = np.random.default_rng(8)
+    wv = rng.uniform(-1, 1, 12).astype(np.float32)
+    xs = [rng.uniform(-1, 1, 8).astype(np.float32) for _ in range(6)]
+    def build(gr, ap):
+        w = gr.variable(wv, [3, 4], "w")
+        x = gr.variable(xs[0], [4, 2], "x")
+        loss = ap.reduce_sum(ap.square(ap.tanh(ap.matmul(x, w))))
+        (dw,) = gr.derive(loss, [w])
+        step = gr.functor("ASSIGN_SUB", [w, ap.mul(0.05, dw)])
+        return w, x, loss, step
+    w, x, loss, step = build(g, api)
+    seen = []
+    for xv in xs:
+        g.assign(x, xv)
+        g.evaluate([step])
+        seen.append(w.get().copy())
+    st = graph.evaluator_stats()
+    assert st["replayed"] >= 4
+    graph.set_evaluator("plain")
+    g2 = graph.Graph()
+    w2, x2, loss2, step2 = build(g2, graph.Api(g2))
+    for i, xv in enumerate(xs):
+        g2.assign(x2, xv)
+        g2.evaluate([step2])
+        np.testing.assert_array_equal(seen[i], w2.get())
+    g2.close()
+    graph.set_evaluator("replay")
+    # a different target set afterwards sees the updated weights
+    g.evaluate([loss])
+    g2 = None
+    ref = np.sum(np.tanh(xs[-1].reshape(2, 4).astype(np.float64) @ seen[-1].reshape(4, 3).astype(np.float64)) ** 2)
+    np.testing.assert_allclose(loss.get(), [ref], rtol=1e-5)
+
+
+def test_replay_mixes_with_other_target_sets_and_aliases(replay_graph):
+    """Recorded and walked passes interleaved on one graph: targets that are
+    aliases, a padded image read only by a convolution, and a node read by a
+    later, different target set."""
+    g, api, graph = replay_graph
+    rng = np.random.default_rng(21)
+    C, W, H, B, O = 2, 6, 5, 2, 3
+    xv = rng.integers(1, 9, C * W * H * B).astype(np.float32)
+    kv = rng.integers(-4, 5, O * C * 3 * 2).astype(np.float32)
+    x = g.variable(xv, [C, W, H, B], "x")
+    k = g.variable(kv, [O, C, 3, 2], "k")
+    conv = api.conv2d(x, k)
+    act = api.relu(conv)
+    alias = api.identity(act)
+    total = api.reduce_sum(act)
+    results = []
+    for i in range(5):
+        g.assign(x, xv + i)
+        g.evaluate([alias, total])
+        results.append((alias.get().copy(), total.get().copy()))
+        if i == 2:
+            # another target set in between, walked node by node
+            g.evaluate([conv])
+            mid = conv.get().copy()
+    assert graph.evaluator_stats()["replayed"] >= 3
+    graph.set_evaluator("plain")
+    g2 = graph.Graph()
+    api2 = graph.Api(g2)
+    x2 = g2.variable(xv, [C, W, H, B], "x")
+    k2 = g2.variable(kv, [O, C, 3, 2], "k")
+    conv2 = api2.conv2d(x2, k2)
+    act2 = api2.relu(conv2)
+    tot2 = api2.reduce_sum(act2)
+    for i in range(5):
+        g2.assign(x2, xv + i)
+        g2.evaluate([act2, tot2, conv2])
+        np.testing.assert_array_equal(results[i][0], act2.get())
+        np.testing.assert_array_equal(results[i][1], tot2.get())
+        if i == 2:
+            np.testing.assert_array_equal(mid, conv2.get())
+    g2.close()
+    graph.set_evaluator("replay")
+
+
+def test_recordings_are_dropped_when_nodes_go_away():
+    from tenncor_amd import graph
+    graph.set_evaluator("replay")
+    try:
+        g = graph.Graph()
+        api = graph.Api(g)
+        x = g.variable(np.arange(6, dtype=np.float32), [3, 2], "x")
+        y = api.exp(api.neg(x))
+        for i in range(3):
+            g.assign(x, np.arange(6, dtype=np.float32) + i)
+            g.evaluate([y])
+        assert graph.evaluator_stats()["reserved_bytes"] > 0
+        np.testing.assert_allclose(y.get(), np.exp(-(np.arange(6) + 2.0)), rtol=1e-6)
+        g.close()
+        # a new graph may reuse the node addresses: nothing of the old one may be replayed
+        g = graph.Graph()
+        api = graph.Api(g)
+        x = g.variable(np.arange(6, dtype=np.float32), [3, 2], "x")
+        y = api.square(x)
+        for i in range(3):
+            g.assign(x, np.arange(6, dtype=np.float32) + i)
+            g.evaluate([y])
+            np.testing.assert_array_equal(y.get(), (np.arange(6, dtype=np.float32) + i) ** 2)
+        g.close()
+    finally:
+        graph.set_evaluator("plain")
