@@ -58,9 +58,12 @@ int tcr_sync (tcr_graph* g);
 /* teq::set_eval (internal/teq/src/evaluator.cpp:9-20): which evaluator the
  * process uses from now on. TCR_EVAL_PLAIN is teq::Evaluator, the node-by-node
  * walk; TCR_EVAL_REPLAY records the launches of a set of targets the second
- * time it is evaluated and enqueues the recording as a whole afterwards. */
+ * time it is evaluated and enqueues the recording as a whole afterwards, with
+ * elementwise functors that feed one another computed in shared launches;
+ * TCR_EVAL_REPLAY_UNFUSED records one launch per functor, as the walk issues. */
 #define TCR_EVAL_PLAIN 0
 #define TCR_EVAL_REPLAY 1
+#define TCR_EVAL_REPLAY_UNFUSED 2
 int tcr_set_evaluator (int kind);
 /* Counters of the replaying evaluator (zeros under TCR_EVAL_PLAIN):
  * out[0] passes walked node by node, out[1] recordings made, out[2] passes

@@ -30,7 +30,7 @@ EXPORTS = [
     "tcr_set_evaluator", "tcr_evaluator_stats",
 ]
 
-EVAL_PLAIN, EVAL_REPLAY = 0, 1
+EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED = 0, 1, 2
 
 _lib = None
 
@@ -83,11 +83,13 @@ def load():
 
 
 def set_evaluator(kind):
-    """teq::set_eval: "plain" (node-by-node walk, the default) or "replay"
-    (record a target set's launches on its second evaluation, enqueue the
-    recording afterwards).  Process-wide, like the reference's evaluator slot."""
+    """teq::set_eval: "plain" (node-by-node walk, the default), "replay"
+    (record a target set's launches on its second evaluation, with elementwise
+    functors sharing launches, and enqueue the recording afterwards) or
+    "replay_unfused" (the same with one launch per functor).  Process-wide,
+    like the reference's evaluator slot."""
     lib = load()
-    code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY}[kind]
+    code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY, "replay_unfused": EVAL_REPLAY_UNFUSED}[kind]
     if lib.tcr_set_evaluator(code) != 0:
         raise GraphError(lib.tcr_last_error().decode())
 

@@ -186,6 +186,9 @@ struct iEigen : public teq::iDeviceRef
 	virtual void restore_life (const LifeState&, RTMemptrT&, tcg_graph*) {}
 	/// Host-side effects of a launch that was replayed rather than issued
 	virtual void replayed (void) {}
+	/// The buffer a launch issued by someone else (a fused group) fills for
+	/// this node, with `ttl` reads to live; nullptr when the node cannot take one
+	virtual void* borrow_output (size_t, RTMemptrT&) { return nullptr; }
 };
 
 /// Lifetime given to the node whose launch is being enqueued, and a flag the
@@ -235,6 +238,7 @@ struct CacheEigen final : public iPermEigen
 		data_->restore_life(state, memory, graph);
 	}
 	void replayed (void) override { data_->replayed(); }
+	void* borrow_output (size_t ttl, RTMemptrT& memory) override { return data_->borrow_output(ttl, memory); }
 private:
 	EigenptrT data_;
 };
@@ -440,6 +444,15 @@ struct HipOp final : public iTmpEigen<T>
 	}
 
 	bool is_partial (void) const override { return partial_; }
+
+	void* borrow_output (size_t ttl, RTMemptrT& runtime) override
+	{
+		if (this->data_.is_expired()) { this->data_.borrow(runtime, this->nelems_, ttl); }
+		else { this->data_.extend_life(ttl); }
+		this->mirror_valid_ = false;
+		partial_ = false;
+		return this->data_.get();
+	}
 
 private:
 	OpF op_;

@@ -1,0 +1,60 @@
+// Grouping of elementwise functors for the replaying evaluator: which nodes
+// of an evaluation pass are computed together in one tcg_ew_fusedx launch,
+// which EXTEND / SLICE / PAD / PERMUTE / IDENTITY nodes are never materialised
+// because elementwise groups read straight through them, and in which order
+// the remaining launches run.  The reference evaluates one node at a time
+// (internal/teq/evaluator.hpp:33-45 calling internal/eigen/device.hpp:555-570);
+// Eigen fuses only inside one node's expression.
+#ifndef TCH_FUSE_PLAN_HPP
+#define TCH_FUSE_PLAN_HPP
+
+#include "eigen_device.hpp"
+
+namespace eigen
+{
+
+/// One launch computing several elementwise nodes
+struct FusedGroup final
+{
+	struct Leaf final
+	{
+		teq::iTensor* base = nullptr; ///< materialised tensor the view starts from
+		tcg_fx_leaf view;             ///< ptr is filled in at launch
+	};
+
+	int dtype = 0;
+	std::array<uint64_t,8> shape;
+	std::vector<Observable*> members;  ///< in evaluation order
+	std::vector<Observable*> outputs;  ///< members whose value is stored, by output index
+	std::vector<Leaf> leaves;
+	std::vector<tcg_fx_instr> program;
+	/// materialised tensors that count one read when this group has launched:
+	/// what the members and the views folded into them would have read
+	std::vector<teq::iTensor*> reads;
+};
+
+struct FusionPlan final
+{
+	struct Step final
+	{
+		Observable* node = nullptr; ///< launched through its own closure, or
+		int group = -1;             ///< index into groups
+	};
+
+	std::vector<FusedGroup> groups;
+	std::vector<Step> steps;
+	/// functors that are computed inside a group or folded into operand views
+	/// and therefore never hold a value of their own
+	std::vector<Observable*> absorbed;
+};
+
+/// `funcs`: every functor under the targets, children first
+FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSetT& targets);
+
+/// Enqueue one group: borrows the outputs' buffers (lifetimes as
+/// eigen::Device::calc gives them), launches, counts the reads
+void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory);
+
+}
+
+#endif // TCH_FUSE_PLAN_HPP

@@ -39,7 +39,9 @@ struct ReplayEvaluator final : public teq::iEvaluator
 
 	/// A set of targets is recorded when it is asked for the
 	/// (`warm_passes` + 1)-th time; at most `max_plans` recordings are kept
-	ReplayEvaluator (size_t warm_passes = 1, size_t max_plans = 16);
+	/// With `fuse`, elementwise functors that feed one another are computed
+	/// in shared launches (fuse_plan.hpp)
+	ReplayEvaluator (size_t warm_passes = 1, size_t max_plans = 16, bool fuse = true);
 
 	~ReplayEvaluator (void);
 
@@ -79,6 +81,7 @@ private:
 	Stats stats_;
 	size_t warm_passes_;
 	size_t max_plans_;
+	bool fuse_;
 	size_t epoch_ = 0;
 	size_t clock_ = 0;
 };

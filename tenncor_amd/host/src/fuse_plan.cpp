@@ -1,0 +1,676 @@
+// Which functors of an evaluation pass share a launch (see fuse_plan.hpp).
+#include "fuse_plan.hpp"
+
+#include <algorithm>
+#include <functional>
+#include <map>
+#include <set>
+
+#include "eigen_ops.hpp"
+
+namespace eigen
+{
+
+namespace
+{
+
+enum Kind { OTHER = 0, EW, VIEW };
+
+constexpr size_t max_members = 48;
+
+struct View final
+{
+	teq::iTensor* base = nullptr;
+	int64_t off = 0;
+	int64_t stride[8];
+	uint64_t lo[8];
+	uint64_t hi[8];
+
+	bool operator < (const View& o) const
+	{
+		if (base != o.base) { return base < o.base; }
+		if (off != o.off) { return off < o.off; }
+		int c = memcmp(stride, o.stride, sizeof(stride));
+		if (c != 0) { return c < 0; }
+		c = memcmp(lo, o.lo, sizeof(lo));
+		if (c != 0) { return c < 0; }
+		return memcmp(hi, o.hi, sizeof(hi)) < 0;
+	}
+};
+
+struct Node final
+{
+	Observable* f = nullptr;
+	Kind kind = OTHER;
+	int op = 0;
+	int dtype = 0;
+	bool target = false;
+	bool absorbed = false;      // a VIEW no launch of its own computes
+	std::vector<int> args;      // index of the functor operand, -1 for a leaf
+	teq::TensptrsT arg_tens;
+	std::vector<int> consumers; // functors of this pass reading the node
+	Shape8 shape;
+};
+
+bool is_unary (int op)
+{
+	return op >= egen::ABS && op <= egen::CUBE;
+}
+
+bool is_binary (int op)
+{
+	return op >= egen::POW && op <= egen::GT;
+}
+
+View dense_view (teq::iTensor* tens, const Shape8& shape)
+{
+	View v;
+	v.base = tens;
+	int64_t s = 1;
+	for (int d = 0; d < 8; ++d)
+	{
+		v.stride[d] = s;
+		s *= (int64_t) shape[d];
+		v.lo[d] = 0;
+		v.hi[d] = shape[d];
+	}
+	return v;
+}
+
+bool scalar_constant (const teq::iTensor* tens, double& value)
+{
+	auto leaf = dynamic_cast<const teq::iLeaf*>(tens);
+	if (nullptr == leaf || leaf->get_usage() != teq::IMMUTABLE || leaf->shape().n_elems() != 1)
+	{
+		return false;
+	}
+	const void* data = leaf->device().data();
+	switch (leaf->get_meta().type_code())
+	{
+		case egen::DOUBLE: value = *(const double*) data; return true;
+		case egen::FLOAT: value = *(const float*) data; return true;
+		case egen::INT32: value = *(const int32_t*) data; return true;
+		default: return false;
+	}
+}
+
+struct Planner final
+{
+	Planner (const std::vector<Observable*>& funcs, const teq::TensSetT& targets)
+	{
+		nodes_.resize(funcs.size());
+		for (size_t i = 0; i < funcs.size(); ++i) { index_.emplace(funcs[i], (int) i); }
+		for (size_t i = 0; i < funcs.size(); ++i)
+		{
+			Node& n = nodes_[i];
+			n.f = funcs[i];
+			n.op = (int) n.f->get_opcode().code_;
+			n.dtype = (int) n.f->get_meta().type_code();
+			n.target = targets.count(n.f) > 0;
+			n.shape = shape8(n.f->shape());
+			n.arg_tens = n.f->get_args();
+			for (auto& arg : n.arg_tens)
+			{
+				auto it = index_.find(arg.get());
+				int a = it == index_.end() ? -1 : it->second;
+				n.args.push_back(a);
+				if (a >= 0 && (nodes_[a].consumers.empty() || nodes_[a].consumers.back() != (int) i))
+				{
+					nodes_[a].consumers.push_back((int) i);
+				}
+			}
+			n.kind = classify(n);
+		}
+		// a view is folded away when everything that reads it can read through it
+		for (size_t i = nodes_.size(); i-- > 0;)
+		{
+			Node& n = nodes_[i];
+			if (n.kind != VIEW || n.target || n.consumers.empty()) { continue; }
+			n.absorbed = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
+			{
+				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed);
+			});
+		}
+		uf_.resize(nodes_.size());
+		for (size_t i = 0; i < uf_.size(); ++i) { uf_[i] = (int) i; }
+		minpos_.resize(nodes_.size());
+		maxpos_.resize(nodes_.size());
+		members_.resize(nodes_.size());
+		deps_.resize(nodes_.size());
+		stamp_.assign(nodes_.size(), 0);
+	}
+
+	Kind classify (const Node& n) const
+	{
+		size_t nargs = n.args.size();
+		bool ew = (is_unary(n.op) && nargs == 1) ||
+			(is_binary(n.op) && (nargs == 2 || ((n.op == egen::ADD || n.op == egen::MUL) && nargs > 2))) ||
+			(n.op == egen::SELECT && nargs == 3);
+		if (ew)
+		{
+			if (nargs > TCG_FX_MAX_LEAVES) { return OTHER; }
+			for (auto& arg : n.arg_tens)
+			{
+				if (shape8(arg->shape()) != n.shape || (int) arg->get_meta().type_code() != n.dtype) { return OTHER; }
+			}
+			return EW;
+		}
+		if (nargs != 1) { return OTHER; }
+		switch (n.op)
+		{
+			case egen::IDENTITY: case egen::EXTEND: case egen::SLICE: case egen::PAD:
+				return VIEW;
+			case egen::PERMUTE:
+			{
+				// reading through a permutation that moves the fastest dim is
+				// uncoalesced: worth it only while the tensor is small
+				teq::RanksT order;
+				Packer<teq::RanksT>().unpack(order, *n.f);
+				bool keeps_dim0 = order.empty() || order[0] == 0;
+				return keeps_dim0 || n.f->shape().n_elems() <= (1u << 16) ? VIEW : OTHER;
+			}
+			default: return OTHER;
+		}
+	}
+
+	// ---- views ----
+
+	/// How consumer `c` sees its operand `argpos`, in c's operand coordinates
+	View view_of_arg (int c, size_t argpos, std::vector<int>* through = nullptr)
+	{
+		int a = nodes_[c].args[argpos];
+		if (a >= 0 && nodes_[a].kind == VIEW && nodes_[a].absorbed)
+		{
+			return view_through(a, through);
+		}
+		teq::iTensor* tens = nodes_[c].arg_tens[argpos].get();
+		return dense_view(tens, shape8(tens->shape()));
+	}
+
+	View view_through (int v, std::vector<int>* through)
+	{
+		if (through) { through->push_back(v); }
+		const Node& n = nodes_[v];
+		View in = view_of_arg(v, 0, through);
+		Shape8 inshape = shape8(n.arg_tens[0]->shape());
+		View out = in;
+		switch (n.op)
+		{
+			case egen::IDENTITY: break;
+			case egen::EXTEND:
+			{
+				auto bopt = unpack_extend(n.arg_tens[0]->shape(), *n.f);
+				if (!bopt) { global::fatal("cannot find extend attributes"); }
+				for (size_t d = 0, m = std::min((size_t) 8, bopt->size()); d < m; ++d)
+				{
+					if ((*bopt)[d] > 1)
+					{
+						out.stride[d] = 0;
+						bool whole = in.lo[d] == 0 && in.hi[d] >= 1;
+						out.lo[d] = 0;
+						out.hi[d] = whole ? n.shape[d] : 0;
+					}
+				}
+			}
+				break;
+			case egen::SLICE:
+			{
+				PairVecT<teq::DimT> encoding;
+				Packer<PairVecT<teq::DimT>>().unpack(encoding, *n.f);
+				for (size_t d = 0, m = std::min(encoding.size(), (size_t) 8); d < m; ++d)
+				{
+					uint64_t offset = std::min<uint64_t>(encoding[d].first, inshape[d] - 1);
+					uint64_t extent = std::min<uint64_t>(encoding[d].second, inshape[d] - offset);
+					out.off += (int64_t) offset * in.stride[d];
+					out.lo[d] = in.lo[d] > offset ? in.lo[d] - offset : 0;
+					out.hi[d] = in.hi[d] > offset ? std::min(in.hi[d] - offset, extent) : 0;
+				}
+			}
+				break;
+			case egen::PAD:
+			{
+				PairVecT<teq::DimT> encoding;
+				Packer<PairVecT<teq::DimT>>().unpack(encoding, *n.f);
+				for (size_t d = 0, m = std::min(encoding.size(), (size_t) 8); d < m; ++d)
+				{
+					uint64_t before = encoding[d].first;
+					out.off -= (int64_t) before * in.stride[d];
+					out.lo[d] = in.lo[d] + before;
+					out.hi[d] = in.hi[d] + before;
+				}
+			}
+				break;
+			case egen::PERMUTE:
+			{
+				teq::RanksT order;
+				Packer<teq::RanksT>().unpack(order, *n.f);
+				if (order.size() > 8) { order.resize(8); }
+				bool visited[8] = {false};
+				for (teq::RankT r : order) { visited[r] = true; }
+				for (teq::RankT d = 0; d < 8; ++d)
+				{
+					if (false == visited[d]) { order.push_back(d); }
+				}
+				for (int d = 0; d < 8; ++d)
+				{
+					out.stride[d] = in.stride[order[d]];
+					out.lo[d] = in.lo[order[d]];
+					out.hi[d] = in.hi[order[d]];
+				}
+			}
+				break;
+			default: global::fatal("not a view");
+		}
+		return out;
+	}
+
+	// ---- units: what is launched as one thing ----
+
+	int find (int i)
+	{
+		while (uf_[i] != i)
+		{
+			uf_[i] = uf_[uf_[i]];
+			i = uf_[i];
+		}
+		return i;
+	}
+
+	/// Units whose results node i reads (through folded views)
+	void inputs_of (int i, std::vector<int>& out)
+	{
+		for (int a : nodes_[i].args)
+		{
+			if (a < 0) { continue; }
+			if (nodes_[a].kind == VIEW && nodes_[a].absorbed) { inputs_of(a, out); }
+			else { out.push_back(find(a)); }
+		}
+	}
+
+	/// Does unit u depend, directly or not, on unit g?
+	bool reaches (int u, int g)
+	{
+		++clock_;
+		return reaches_rec(find(u), find(g));
+	}
+
+	bool reaches_rec (int u, int g)
+	{
+		if (u == g) { return true; }
+		if (maxpos_[u] < minpos_[g] || stamp_[u] == clock_) { return false; }
+		stamp_[u] = clock_;
+		for (int d : deps_[u])
+		{
+			if (reaches_rec(find(d), g)) { return true; }
+		}
+		return false;
+	}
+
+	void group_all (void)
+	{
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			Node& n = nodes_[i];
+			minpos_[i] = maxpos_[i] = (int) i;
+			if (n.kind == VIEW && n.absorbed) { continue; }
+			std::vector<int> ins;
+			inputs_of((int) i, ins);
+			deps_[i].insert(ins.begin(), ins.end());
+			if (n.kind != EW) { continue; }
+			members_[i].push_back((int) i);
+			std::vector<int> cands;
+			for (int a : n.args)
+			{
+				if (a >= 0 && nodes_[a].kind == EW) { cands.push_back(find(a)); }
+			}
+			std::sort(cands.begin(), cands.end(), [&](int x, int y) { return maxpos_[x] > maxpos_[y]; });
+			cands.erase(std::unique(cands.begin(), cands.end()), cands.end());
+			int self = (int) i;
+			for (int cand : cands)
+			{
+				cand = find(cand);
+				self = find(self);
+				if (cand == self || members_[self].size() + members_[cand].size() > max_members) { continue; }
+				if (mergeable(self, cand)) { self = merge(self, cand); }
+			}
+		}
+	}
+
+	/// No launch outside the two units may sit between them
+	bool mergeable (int g, int cand)
+	{
+		for (int d : deps_[g])
+		{
+			d = find(d);
+			if (d != cand && d != g && reaches(d, cand)) { return false; }
+		}
+		for (int d : deps_[cand])
+		{
+			d = find(d);
+			if (d != cand && d != g && reaches(d, g)) { return false; }
+		}
+		return true;
+	}
+
+	int merge (int g, int cand)
+	{
+		// the earlier unit stays the root: positions order the members
+		int root = std::min(g, cand), other = std::max(g, cand);
+		uf_[other] = root;
+		std::vector<int> merged;
+		std::merge(members_[root].begin(), members_[root].end(),
+			members_[other].begin(), members_[other].end(), std::back_inserter(merged));
+		members_[root] = merged;
+		members_[other].clear();
+		std::set<int> deps;
+		for (int d : deps_[root]) { if (find(d) != root) { deps.insert(find(d)); } }
+		for (int d : deps_[other]) { if (find(d) != root) { deps.insert(find(d)); } }
+		deps_[root] = deps;
+		deps_[other].clear();
+		minpos_[root] = std::min(minpos_[root], minpos_[other]);
+		maxpos_[root] = std::max(maxpos_[root], maxpos_[other]);
+		return root;
+	}
+
+	// ---- emission ----
+
+	/// members [lo, hi) of unit g as one launch; false when it does not fit
+	bool build (const std::vector<int>& members, size_t lo, size_t hi, FusedGroup& out, std::vector<int>& views)
+	{
+		out = FusedGroup();
+		views.clear();
+		const Node& first = nodes_[members[lo]];
+		out.dtype = first.dtype;
+		out.shape = first.shape;
+		std::map<int,size_t> pos; // member -> position in the launch
+		for (size_t p = lo; p < hi; ++p) { pos.emplace(members[p], p - lo); }
+		auto inside = [&](int a) { return a >= 0 && pos.count(a) > 0; };
+		std::vector<size_t> last_use(hi - lo, 0);
+		std::vector<bool> stored(hi - lo, false);
+		for (size_t p = lo; p < hi; ++p)
+		{
+			const Node& n = nodes_[members[p]];
+			for (int a : n.args)
+			{
+				if (inside(a)) { last_use[pos[a]] = p - lo; }
+			}
+			stored[p - lo] = n.target || std::any_of(n.consumers.begin(), n.consumers.end(),
+				[&](int c) { return false == inside(c); });
+		}
+		std::map<View,int> leaf_of;
+		std::vector<int> reg_of(hi - lo, -1);
+		std::vector<bool> busy(TCG_FX_MAX_REGS, false);
+		auto take_reg = [&]() -> int
+		{
+			for (int r = 0; r < TCG_FX_MAX_REGS; ++r)
+			{
+				if (false == busy[r])
+				{
+					busy[r] = true;
+					return r;
+				}
+			}
+			return -1;
+		};
+		for (size_t p = lo; p < hi; ++p)
+		{
+			const Node& n = nodes_[members[p]];
+			size_t here = p - lo;
+			// operands: a register of this launch, an immediate or a leaf
+			bool fold = n.args.size() > 2 && n.op != egen::SELECT;
+			std::vector<uint8_t> codes;
+			std::vector<double> vals;
+			for (size_t k = 0; k < n.args.size(); ++k)
+			{
+				int a = n.args[k];
+				if (inside(a))
+				{
+					codes.push_back((uint8_t) (TCG_FX_REG0 + reg_of[pos[a]]));
+					vals.push_back(0);
+					continue;
+				}
+				View v = view_of_arg(members[p], k, &views);
+				double value;
+				if (scalar_constant(v.base, value))
+				{
+					// an instruction carries one immediate: operands sharing an
+					// instruction (all of them unless the node is an n-ary fold,
+					// where only the first two do) must agree on it
+					bool clash = false;
+					for (size_t j = fold ? (k == 1 ? 0 : k) : 0; j < k; ++j)
+					{
+						clash = clash || (codes[j] == TCG_FX_IMM && vals[j] != value);
+					}
+					if (false == clash)
+					{
+						codes.push_back(TCG_FX_IMM);
+						vals.push_back(value);
+						continue;
+					}
+				}
+				auto it = leaf_of.find(v);
+				if (it == leaf_of.end())
+				{
+					if (out.leaves.size() >= TCG_FX_MAX_LEAVES) { return false; }
+					FusedGroup::Leaf leaf;
+					leaf.base = v.base;
+					leaf.view.ptr = nullptr;
+					leaf.view.offset = v.off;
+					std::copy(v.stride, v.stride + 8, leaf.view.stride);
+					std::copy(v.lo, v.lo + 8, leaf.view.lo);
+					std::copy(v.hi, v.hi + 8, leaf.view.hi);
+					it = leaf_of.emplace(v, (int) out.leaves.size()).first;
+					out.leaves.push_back(leaf);
+				}
+				codes.push_back((uint8_t) (TCG_FX_LEAF0 + it->second));
+				vals.push_back(0);
+			}
+			auto imm_of = [&](size_t j, size_t k)
+			{
+				return codes[j] == TCG_FX_IMM ? vals[j] : codes[k] == TCG_FX_IMM ? vals[k] : 0.0;
+			};
+			// registers: a one-instruction node may overwrite an operand that
+			// dies here; a fold keeps its accumulator apart from its operands
+			auto release_dead = [&]()
+			{
+				for (int a : n.args)
+				{
+					if (inside(a) && last_use[pos[a]] == here) { busy[reg_of[pos[a]]] = false; }
+				}
+			};
+			if (false == fold) { release_dead(); }
+			int dst = take_reg();
+			if (dst < 0) { return false; }
+			reg_of[here] = dst;
+			tcg_fx_instr ins;
+			memset(&ins, 0, sizeof(ins));
+			ins.dst = (uint8_t) (TCG_FX_REG0 + dst);
+			ins.opcode = (uint8_t) n.op;
+			if (fold)
+			{
+				// ((a0 op a1) op a2) ... like the n-ary kernel
+				ins.a = codes[0];
+				ins.b = codes[1];
+				ins.imm = imm_of(0, 1);
+				out.program.push_back(ins);
+				for (size_t k = 2; k < codes.size(); ++k)
+				{
+					ins.a = (uint8_t) (TCG_FX_REG0 + dst);
+					ins.b = codes[k];
+					ins.imm = imm_of(k, k);
+					out.program.push_back(ins);
+				}
+				release_dead();
+			}
+			else
+			{
+				ins.a = codes[0];
+				ins.b = codes.size() > 1 ? codes[1] : (uint8_t) TCG_FX_NONE;
+				ins.c = codes.size() > 2 ? codes[2] : (uint8_t) TCG_FX_NONE;
+				for (size_t k = 0; k < codes.size(); ++k)
+				{
+					if (codes[k] == TCG_FX_IMM) { ins.imm = vals[k]; }
+				}
+				out.program.push_back(ins);
+			}
+			if (stored[here])
+			{
+				if (out.outputs.size() >= TCG_FX_MAX_OUTS) { return false; }
+				tcg_fx_instr st;
+				memset(&st, 0, sizeof(st));
+				st.opcode = TCG_FX_STORE;
+				st.a = (uint8_t) (TCG_FX_REG0 + dst);
+				st.dst = (uint8_t) out.outputs.size();
+				out.program.push_back(st);
+				out.outputs.push_back(n.f);
+			}
+			if (false == std::any_of(n.consumers.begin(), n.consumers.end(), inside))
+			{
+				busy[dst] = false; // nothing in this launch reads it
+			}
+			if (out.program.size() > TCG_FX_MAX_INSTRS) { return false; }
+			out.members.push_back(n.f);
+			// reads the plain pass would have counted
+			for (size_t k = 0; k < n.args.size(); ++k)
+			{
+				int a = n.args[k];
+				if (a < 0) { continue; }
+				bool materialised = inside(a) ? stored[pos[a]] : false == (nodes_[a].kind == VIEW && nodes_[a].absorbed);
+				if (materialised) { out.reads.push_back(n.arg_tens[k].get()); }
+			}
+		}
+		return true;
+	}
+
+	FusionPlan finish (void)
+	{
+		FusionPlan plan;
+		std::vector<bool> done(nodes_.size(), false);
+		std::map<int,int> last_user; // folded view -> last group reading through it
+		std::function<void(int)> visit = [&](int u)
+		{
+			u = find(u);
+			if (done[u]) { return; }
+			done[u] = true;
+			std::vector<int> deps;
+			for (int d : deps_[u]) { deps.push_back(find(d)); }
+			std::sort(deps.begin(), deps.end(), [&](int x, int y) { return minpos_[x] < minpos_[y]; });
+			for (int d : deps)
+			{
+				if (d != u) { visit(d); }
+			}
+			if (nodes_[u].kind != EW)
+			{
+				FusionPlan::Step step;
+				step.node = nodes_[u].f;
+				plan.steps.push_back(step);
+				return;
+			}
+			const std::vector<int>& members = members_[u];
+			for (size_t lo = 0; lo < members.size();)
+			{
+				FusedGroup group, next;
+				std::vector<int> views, next_views;
+				size_t hi = lo + 1;
+				if (false == build(members, lo, hi, group, views))
+				{
+					global::fatalf("cannot plan a launch for %s", nodes_[members[lo]].f->to_string().c_str());
+				}
+				while (hi < members.size() && build(members, lo, hi + 1, next, next_views))
+				{
+					group = next;
+					views = next_views;
+					++hi;
+				}
+				FusionPlan::Step step;
+				if (hi == lo + 1 && views.empty() && false == uses_immediate(group))
+				{
+					step.node = nodes_[members[lo]].f; // nothing to gain: its own kernel
+				}
+				else
+				{
+					step.group = (int) plan.groups.size();
+					for (int v : views) { last_user[v] = step.group; }
+					for (size_t p = lo; p < hi; ++p)
+					{
+						const Node& n = nodes_[members[p]];
+						if (std::find(group.outputs.begin(), group.outputs.end(), n.f) == group.outputs.end())
+						{
+							plan.absorbed.push_back(n.f);
+						}
+					}
+					plan.groups.push_back(group);
+				}
+				plan.steps.push_back(step);
+				lo = hi;
+			}
+		};
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			if (nodes_[i].target) { visit((int) i); }
+		}
+		// a folded view counts one read of its operand, when the last launch
+		// that looks through it has been enqueued
+		for (auto& kv : last_user)
+		{
+			const Node& v = nodes_[kv.first];
+			plan.absorbed.push_back(v.f);
+			int a = v.args[0];
+			if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+			{
+				plan.groups[kv.second].reads.push_back(v.arg_tens[0].get());
+			}
+		}
+		return plan;
+	}
+
+	static bool uses_immediate (const FusedGroup& group)
+	{
+		return std::any_of(group.program.begin(), group.program.end(), [](const tcg_fx_instr& ins)
+		{
+			return ins.a == TCG_FX_IMM || ins.b == TCG_FX_IMM || ins.c == TCG_FX_IMM;
+		});
+	}
+
+	std::vector<Node> nodes_;
+	std::unordered_map<teq::iTensor*,int> index_;
+	std::vector<int> uf_, minpos_, maxpos_;
+	std::vector<std::vector<int>> members_;
+	std::vector<std::set<int>> deps_;
+	std::vector<size_t> stamp_;
+	size_t clock_ = 0;
+};
+
+}
+
+FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSetT& targets)
+{
+	Planner planner(funcs, targets);
+	planner.group_all();
+	return planner.finish();
+}
+
+void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory)
+{
+	std::vector<void*> outs;
+	for (Observable* out : group.outputs)
+	{
+		size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
+		void* ptr = static_cast<iEigen&>(out->device()).borrow_output(ttl, memory);
+		if (nullptr == ptr) { global::fatalf("%s cannot take a fused result", out->to_string().c_str()); }
+		outs.push_back(ptr);
+	}
+	std::vector<tcg_fx_leaf> leaves;
+	for (auto& leaf : group.leaves)
+	{
+		tcg_fx_leaf view = leaf.view;
+		view.ptr = eigen_ref(*leaf.base).device_data();
+		if (nullptr == view.ptr) { global::fatalf("operand %s has no data", leaf.base->to_string().c_str()); }
+		leaves.push_back(view);
+	}
+	hip_check(tcg_ew_fusedx(hip_context(), group.dtype, group.shape.data(), (int) leaves.size(), leaves.data(),
+		(int) group.program.size(), group.program.data(), (int) outs.size(), outs.data()));
+	for (teq::iTensor* tens : group.reads) { eigen_ref(*tens).odevice(); }
+}
+
+}

@@ -1,5 +1,6 @@
 // Recording and replaying whole evaluation passes (see replay_eval.hpp).
 #include "replay_eval.hpp"
+#include "fuse_plan.hpp"
 
 #include <algorithm>
 
@@ -44,8 +45,8 @@ struct ReplayEvaluator::Plan final
 	bool fresh = true;
 };
 
-ReplayEvaluator::ReplayEvaluator (size_t warm_passes, size_t max_plans) :
-	warm_passes_(warm_passes), max_plans_(std::max<size_t>(1, max_plans)),
+ReplayEvaluator::ReplayEvaluator (size_t warm_passes, size_t max_plans, bool fuse) :
+	warm_passes_(warm_passes), max_plans_(std::max<size_t>(1, max_plans)), fuse_(fuse),
 	epoch_(global::structure_epoch()) {}
 
 ReplayEvaluator::~ReplayEvaluator (void)
@@ -181,16 +182,37 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		plan->leaf_ptrs.push_back(eigen_ref(*leaf).device_data());
 		plan->leaf_versions.push_back(leaf->get_meta().state_version());
 	}
+	// which launches the pass needs: elementwise nodes share launches and read
+	// through the views in front of them
+	FusionPlan fusion;
+	if (fuse_) { fusion = plan_fusion(plan->funcs, targets); }
+	else
+	{
+		for (Observable* f : plan->funcs)
+		{
+			FusionPlan::Step step;
+			step.node = f;
+			fusion.steps.push_back(step);
+		}
+	}
 	// every value under the targets is recomputed into memory of the recording
 	for (iEigen* dev : plan->devs) { dev->drop(); }
+	for (Observable* f : plan->funcs) { f->prop_version(device.max_version_); }
 	tcg_ctx* ctx = hip_context();
 	hip_check(tcg_capture_begin(ctx));
 	bool ok = true;
 	try
 	{
-		for (Observable* f : plan->funcs)
+		for (auto& step : fusion.steps)
 		{
-			device.calc_forced(*f, (size_t) (targets.count(f) > 0));
+			if (nullptr != step.node)
+			{
+				device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0));
+			}
+			else
+			{
+				launch_group(fusion.groups[step.group], targets, device.memory());
+			}
 		}
 	}
 	catch (...)

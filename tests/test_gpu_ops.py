@@ -611,3 +611,86 @@ def test_full_size_properties_config2(ctx, ops):
     tt = ops.permute(ops.permute(prod, [1, 0]), [1, 0])
     np.testing.assert_array_equal(tt.get(), p_host.reshape(-1))
     np.testing.assert_array_equal(ops.permute(prod, [1, 0]).get().reshape(16384, 4096)[5], p_host[:, 5])
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
+def test_fused_group_with_views_and_several_outputs(ctx, oracle, np_dtype):
+    """tcg_ew_fusedx against the same nodes evaluated one by one by the oracle:
+    an LSTM-cell shaped group reading four SLICE views of one matrix, an
+    EXTEND view of a bias row and a PAD view, storing three results.  The
+    fused kernel uses the scalar routines of the one-node kernels, so fp32
+    results are held to the elementwise bar and int32 ones to bit equality."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of("fusedx", str(np_dtype)))
+    dt = capi.dtype_code(np_dtype)
+    for H, B in ((8, 5), (7, 3), (64, 12)):
+        if np_dtype == np.int32:
+            draw = lambda n: rng.integers(-9, 10, n).astype(np.int32)
+        else:
+            draw = lambda n: rng.uniform(-1, 1, n).astype(np_dtype)
+        gates = draw(4 * H * B)          # teq shape [4H, B]
+        state = draw(H * B)              # [H, B]
+        bias = draw(H)                   # [H] extended over B
+        small = draw((H - 2) * B)        # [H-2, B] padded by (1, 1) along dim 0
+        # the graph, node by node on the oracle
+        sl = [oracle.slice_(gates, [4 * H, B], [[k * H, H]])[0] for k in range(4)]
+        bext = oracle.extend(bias, [H], [1, B])[0]
+        padded = oracle.pad(small, [H - 2, B], [[1, 1]])[0]
+        g = oracle.unary("TANH", oracle.binary("ADD", sl[0], bext))
+        i = oracle.unary("SIGMOID", sl[1])
+        f = oracle.unary("SIGMOID", sl[2])
+        o = oracle.unary("ABS", sl[3])
+        new_state = oracle.nary("ADD", [oracle.binary("MUL", g, i), oracle.binary("MUL", state, f), padded])
+        hidden = oracle.binary("MUL", new_state, o)
+        picked = oracle.select(oracle.binary("GT", hidden, np.full(H * B, 0.25).astype(np_dtype)), hidden,
+                               oracle.binary("MUL", hidden, np.full(H * B, 2).astype(np_dtype)))
+        dg, ds, db, dp = ctx.upload(gates), ctx.upload(state), ctx.upload(bias), ctx.upload(small)
+        L, R = capi.FX_LEAF0, capi.FX_REG0
+        leaves = [{"ptr": dg.ptr, "offset": k * H, "stride": [1, 4 * H] + [4 * H * B] * 6} for k in range(4)]
+        leaves.append({"ptr": ds.ptr})
+        leaves.append({"ptr": db.ptr, "stride": [1, 0, 0, 0, 0, 0, 0, 0]})
+        leaves.append({"ptr": dp.ptr, "offset": -1, "stride": [1, H - 2] + [(H - 2) * B] * 6,
+                       "lo": [1, 0, 0, 0, 0, 0, 0, 0], "hi": [H - 1, B, 1, 1, 1, 1, 1, 1]})
+        N = capi.FX_NONE
+        prog = [
+            ("ADD", L + 0, L + 5, N, R + 0),
+            ("TANH", R + 0, N, N, R + 0),
+            ("SIGMOID", L + 1, N, N, R + 1),
+            ("SIGMOID", L + 2, N, N, R + 2),
+            ("ABS", L + 3, N, N, R + 3),
+            ("MUL", R + 0, R + 1, N, R + 4),
+            ("MUL", L + 4, R + 2, N, R + 5),
+            ("ADD", R + 4, R + 5, N, R + 6),
+            ("ADD", R + 6, L + 6, N, R + 6),
+            ("STORE", R + 6, N, N, 0),
+            ("MUL", R + 6, R + 3, N, R + 7),
+            ("STORE", R + 7, N, N, 1),
+            ("GT", R + 7, capi.FX_IMM, N, R + 8, 0.25),
+            ("MUL", R + 7, capi.FX_IMM, N, R + 9, 2.0),
+            ("SELECT", R + 8, R + 7, R + 9, R + 10),
+            ("STORE", R + 10, N, N, 2),
+        ]
+        outs = [ctx.empty(H * B, np_dtype) for _ in range(3)]
+        ctx.ew_fusedx(dt, [H, B], leaves, prog, [o_.ptr for o_ in outs])
+        for got, want in zip(outs, (new_state, hidden, picked)):
+            if np_dtype == np.int32:
+                np.testing.assert_array_equal(got.get(), want)
+            else:
+                np.testing.assert_allclose(got.get(), want, rtol=EW_RTOL, atol=1e-7)
+
+
+def test_fused_group_rejects_malformed_programs(ctx):
+    from tenncor_amd import capi
+    x = ctx.upload(np.ones(16, np.float32))
+    out = ctx.empty(16, np.float32)
+    L, R, N = capi.FX_LEAF0, capi.FX_REG0, capi.FX_NONE
+    bad = [
+        [("NEG", L + 1, N, N, R + 0), ("STORE", R + 0, N, N, 0)],      # leaf that does not exist
+        [("NEG", R + 3, N, N, R + 0), ("STORE", R + 0, N, N, 0)],      # register never written
+        [("NEG", L + 0, N, N, R + 0)],                                 # output never stored
+        [("MATMUL", L + 0, L + 0, N, R + 0), ("STORE", R + 0, N, N, 0)],
+        [("NEG", L + 0, N, N, R + 16), ("STORE", R + 0, N, N, 0)],
+    ]
+    for prog in bad:
+        with pytest.raises(capi.TcgError):
+            ctx.ew_fusedx(capi.FLOAT, [16], [{"ptr": x.ptr}], prog, [out.ptr])
