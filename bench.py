@@ -139,19 +139,29 @@ def run_extras(ctx, capi):
     rng = np.random.default_rng(22)
     leaves = [ctx.upload(rng.uniform(-1, 1, N).astype(np.float32)) for _ in range(3)]
     out = ctx.empty(N, np.float32)
-    L = capi.OPD_LEAF0
-    prog = [("ADD", L, L + 1, capi.OPD_ACC), ("MUL", capi.OPD_ACC, L + 2, capi.OPD_ACC),
+    # the chain as one group launch (the kernel is compiled for the program on
+    # first use) and through the three-register interpreter
+    L, R, NONE = capi.FX_LEAF0, capi.FX_REG0, capi.FX_NONE
+    group = [("ADD", L, L + 1, NONE, R), ("MUL", R, L + 2, NONE, R), ("EXP", R, NONE, NONE, R),
+             ("TANH", R, NONE, NONE, R), ("SIGMOID", R, NONE, NONE, R), ("STORE", R, NONE, NONE, 0)]
+    O = capi.OPD_LEAF0
+    prog = [("ADD", O, O + 1, capi.OPD_ACC), ("MUL", capi.OPD_ACC, O + 2, capi.OPD_ACC),
             ("EXP", capi.OPD_ACC, 0, capi.OPD_ACC), ("TANH", capi.OPD_ACC, 0, capi.OPD_ACC),
             ("SIGMOID", capi.OPD_ACC, 0, capi.OPD_ACC)]
-    for _ in range(2):
-        ctx.ew_fused(capi.FLOAT, N, [b.ptr for b in leaves], prog, out.ptr)
-    ctx.timer_begin()
     reps = 10
-    for _ in range(reps):
-        ctx.ew_fused(capi.FLOAT, N, [b.ptr for b in leaves], prog, out.ptr)
-    ms = ctx.timer_end() / reps
-    extra["fused_chain_GBps"] = round(4 * 4 * N / (ms * 1e-3) / 1e9, 1)
-    extra["fused_chain_ms"] = round(ms, 4)
+    runs = {
+        "fused_chain": lambda: ctx.ew_fusedx(capi.FLOAT, [COLS, ROWS], [{"ptr": b.ptr} for b in leaves], group, [out.ptr]),
+        "fused_chain_interpreted": lambda: ctx.ew_fused(capi.FLOAT, N, [b.ptr for b in leaves], prog, out.ptr),
+    }
+    for key, fn in runs.items():
+        for _ in range(2):
+            fn()
+        ctx.timer_begin()
+        for _ in range(reps):
+            fn()
+        ms = ctx.timer_end() / reps
+        extra[key + "_GBps"] = round(4 * 4 * N / (ms * 1e-3) / 1e9, 1)
+        extra[key + "_ms"] = round(ms, 4)
     # plain streaming copy (NEG: N floats in, N floats out), the known-size kernel
     # that hardware byte counters are scaled by
     for _ in range(2):

@@ -211,7 +211,7 @@ enum tcg_fx_operand
 #define TCG_FX_MAX_LEAVES 8
 #define TCG_FX_MAX_REGS 16
 #define TCG_FX_MAX_INSTRS 64
-#define TCG_FX_MAX_OUTS 4
+#define TCG_FX_MAX_OUTS 8
 #define TCG_FX_STORE 255 /* opcode */
 typedef struct tcg_fx_leaf
 {

@@ -50,7 +50,7 @@ def build_libtcg(jobs=8, verbose=False):
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(compile_one, zip(sources, objs)))
-    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBTCG] + objs)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIBTCG] + objs + ["-lhiprtc"])
     return LIBTCG
 
 

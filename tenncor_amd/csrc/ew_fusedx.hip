@@ -12,21 +12,27 @@
 // one-node kernels: results are bit-identical to the unfused evaluation.
 #include "ew_scalar.hpp"
 
+#include <hip/hiprtc.h>
+
+#include <cstdlib>
+#include <mutex>
+#include <sstream>
+#include <unordered_map>
+
 namespace
 {
 
 constexpr int FX_BLOCK = 256;
-constexpr int FX_MAXD = 8;
+#define FX_MAXD 8
 constexpr int FX_SLOTS = TCG_FX_MAX_LEAVES + TCG_FX_MAX_REGS;
 
-struct FxDiv
-{
-	uint32_t d = 1, m = 0, s1 = 0, s2 = 0;
-};
+#define TCG_CORE(...) __VA_ARGS__
+#include "ew_fusedx_args.inc"
+#undef TCG_CORE
 
 FxDiv fx_make_div (uint32_t d)
 {
-	FxDiv f;
+	FxDiv f = {1, 0, 0, 0};
 	f.d = d;
 	uint32_t l = 0;
 	while (((uint64_t) 1 << l) < d) { ++l; }
@@ -36,39 +42,90 @@ FxDiv fx_make_div (uint32_t d)
 	return f;
 }
 
-__device__ __forceinline__ uint32_t fx_div (uint32_t n, const FxDiv& f)
+// The register file of one lane: leaves first, then registers.  It is only
+// ever indexed by constants, so it lives in VGPRs; the slot an instruction
+// names is wave-uniform, so picking it is a scalar branch, not a memory access
+// (an array indexed by the slot number would be placed in scratch memory).
+static_assert(FX_SLOTS == 24, "fx_get / fx_put enumerate the slots");
+
+// ends every case of the slot switches: without it the optimiser merges the
+// cases into one access through a selected address, which forces the file
+// into memory
+#define FX_KEEP_APART asm volatile("")
+
+// one statement per element of the lane's vector, without a loop: every index
+// must be a constant before the optimiser decides where the file lives
+#define FX_EACH(stmt)\
+	{ if constexpr (N > 0) { constexpr int e_ = 0; stmt; }\
+	if constexpr (N > 1) { constexpr int e_ = 1; stmt; }\
+	if constexpr (N > 2) { constexpr int e_ = 2; stmt; }\
+	if constexpr (N > 3) { constexpr int e_ = 3; stmt; } }
+
+template <typename T, int N>
+__device__ __forceinline__ void fx_get (const T (&file)[FX_SLOTS][N], int s, T (&v)[N])
 {
-	uint32_t t = __umulhi(f.m, n);
-	return (t + ((n - t) >> f.s1)) >> f.s2;
+	switch (s)
+	{
+		case 0: FX_EACH(v[e_] = file[0][e_]) FX_KEEP_APART; break;
+		case 1: FX_EACH(v[e_] = file[1][e_]) FX_KEEP_APART; break;
+		case 2: FX_EACH(v[e_] = file[2][e_]) FX_KEEP_APART; break;
+		case 3: FX_EACH(v[e_] = file[3][e_]) FX_KEEP_APART; break;
+		case 4: FX_EACH(v[e_] = file[4][e_]) FX_KEEP_APART; break;
+		case 5: FX_EACH(v[e_] = file[5][e_]) FX_KEEP_APART; break;
+		case 6: FX_EACH(v[e_] = file[6][e_]) FX_KEEP_APART; break;
+		case 7: FX_EACH(v[e_] = file[7][e_]) FX_KEEP_APART; break;
+		case 8: FX_EACH(v[e_] = file[8][e_]) FX_KEEP_APART; break;
+		case 9: FX_EACH(v[e_] = file[9][e_]) FX_KEEP_APART; break;
+		case 10: FX_EACH(v[e_] = file[10][e_]) FX_KEEP_APART; break;
+		case 11: FX_EACH(v[e_] = file[11][e_]) FX_KEEP_APART; break;
+		case 12: FX_EACH(v[e_] = file[12][e_]) FX_KEEP_APART; break;
+		case 13: FX_EACH(v[e_] = file[13][e_]) FX_KEEP_APART; break;
+		case 14: FX_EACH(v[e_] = file[14][e_]) FX_KEEP_APART; break;
+		case 15: FX_EACH(v[e_] = file[15][e_]) FX_KEEP_APART; break;
+		case 16: FX_EACH(v[e_] = file[16][e_]) FX_KEEP_APART; break;
+		case 17: FX_EACH(v[e_] = file[17][e_]) FX_KEEP_APART; break;
+		case 18: FX_EACH(v[e_] = file[18][e_]) FX_KEEP_APART; break;
+		case 19: FX_EACH(v[e_] = file[19][e_]) FX_KEEP_APART; break;
+		case 20: FX_EACH(v[e_] = file[20][e_]) FX_KEEP_APART; break;
+		case 21: FX_EACH(v[e_] = file[21][e_]) FX_KEEP_APART; break;
+		case 22: FX_EACH(v[e_] = file[22][e_]) FX_KEEP_APART; break;
+		case 23: FX_EACH(v[e_] = file[23][e_]) FX_KEEP_APART; break;
+		default: break;
+	}
 }
 
-struct FxLeaf
+template <typename T, int N>
+__device__ __forceinline__ void fx_put (T (&file)[FX_SLOTS][N], int s, const T (&v)[N])
 {
-	const void* ptr;
-	int64_t off;               // elements
-	int64_t stride[FX_MAXD];   // elements per iteration dim; 0 = broadcast
-	uint32_t lo[FX_MAXD];      // with `boxed`: outside [lo, hi) the operand
-	uint32_t hi[FX_MAXD];      // reads as zero and memory is not touched
-	uint32_t boxed;
-	uint32_t bcast0;           // stride[0] == 0
-};
-
-struct FxInstr
-{
-	uint8_t opcode, a, b, c, dst, pad_[3];
-};
-
-struct FxArgs
-{
-	uint32_t nd, nleaf, ninstr, nout;
-	uint32_t size[FX_MAXD];    // iteration extents in elements, dim 0 innermost
-	FxDiv div[FX_MAXD];        // div[0] divides by size[0] / N
-	uint64_t total;            // elements
-	FxLeaf leaf[TCG_FX_MAX_LEAVES];
-	FxInstr prog[TCG_FX_MAX_INSTRS];
-	double imm[TCG_FX_MAX_INSTRS];
-	void* out[TCG_FX_MAX_OUTS];
-};
+	switch (s)
+	{
+		case 0: FX_EACH(file[0][e_] = v[e_]) FX_KEEP_APART; break;
+		case 1: FX_EACH(file[1][e_] = v[e_]) FX_KEEP_APART; break;
+		case 2: FX_EACH(file[2][e_] = v[e_]) FX_KEEP_APART; break;
+		case 3: FX_EACH(file[3][e_] = v[e_]) FX_KEEP_APART; break;
+		case 4: FX_EACH(file[4][e_] = v[e_]) FX_KEEP_APART; break;
+		case 5: FX_EACH(file[5][e_] = v[e_]) FX_KEEP_APART; break;
+		case 6: FX_EACH(file[6][e_] = v[e_]) FX_KEEP_APART; break;
+		case 7: FX_EACH(file[7][e_] = v[e_]) FX_KEEP_APART; break;
+		case 8: FX_EACH(file[8][e_] = v[e_]) FX_KEEP_APART; break;
+		case 9: FX_EACH(file[9][e_] = v[e_]) FX_KEEP_APART; break;
+		case 10: FX_EACH(file[10][e_] = v[e_]) FX_KEEP_APART; break;
+		case 11: FX_EACH(file[11][e_] = v[e_]) FX_KEEP_APART; break;
+		case 12: FX_EACH(file[12][e_] = v[e_]) FX_KEEP_APART; break;
+		case 13: FX_EACH(file[13][e_] = v[e_]) FX_KEEP_APART; break;
+		case 14: FX_EACH(file[14][e_] = v[e_]) FX_KEEP_APART; break;
+		case 15: FX_EACH(file[15][e_] = v[e_]) FX_KEEP_APART; break;
+		case 16: FX_EACH(file[16][e_] = v[e_]) FX_KEEP_APART; break;
+		case 17: FX_EACH(file[17][e_] = v[e_]) FX_KEEP_APART; break;
+		case 18: FX_EACH(file[18][e_] = v[e_]) FX_KEEP_APART; break;
+		case 19: FX_EACH(file[19][e_] = v[e_]) FX_KEEP_APART; break;
+		case 20: FX_EACH(file[20][e_] = v[e_]) FX_KEEP_APART; break;
+		case 21: FX_EACH(file[21][e_] = v[e_]) FX_KEEP_APART; break;
+		case 22: FX_EACH(file[22][e_] = v[e_]) FX_KEEP_APART; break;
+		case 23: FX_EACH(file[23][e_] = v[e_]) FX_KEEP_APART; break;
+		default: break;
+	}
+}
 
 // operand code -> slot of the register file (leaves first)
 __device__ __forceinline__ int fx_slot (int code)
@@ -118,7 +175,7 @@ __global__ __launch_bounds__(FX_BLOCK) void ew_fusedx_k (FxArgs p)
 				}
 			}
 		}
-		T slot[FX_SLOTS][N];
+		T file[FX_SLOTS][N];
 #pragma unroll
 		for (int k = 0; k < TCG_FX_MAX_LEAVES; ++k)
 		{
@@ -127,21 +184,18 @@ __global__ __launch_bounds__(FX_BLOCK) void ew_fusedx_k (FxArgs p)
 				const T* src = (const T*) p.leaf[k].ptr + off[k];
 				if (!inside[k])
 				{
-#pragma unroll
-					for (int e = 0; e < N; ++e) { slot[k][e] = (T) 0; }
+					FX_EACH(file[k][e_] = (T) 0)
 				}
 				else if (N > 1 && !p.leaf[k].bcast0)
 				{
 					VecU<T> v;
 					v.v = *reinterpret_cast<const typename Vec16<T>::type*>(src);
-#pragma unroll
-					for (int e = 0; e < N; ++e) { slot[k][e] = v.e[e]; }
+					FX_EACH(file[k][e_] = v.e[e_])
 				}
 				else
 				{
 					T s = *src;
-#pragma unroll
-					for (int e = 0; e < N; ++e) { slot[k][e] = s; }
+					FX_EACH(file[k][e_] = s)
 				}
 			}
 		}
@@ -149,12 +203,13 @@ __global__ __launch_bounds__(FX_BLOCK) void ew_fusedx_k (FxArgs p)
 		{
 			const FxInstr ins = p.prog[i];
 			const T imm = (T) p.imm[i];
-			T va[N], vb[N], vc[N];
+			T va[N], vb[N], vc[N], vr[N];
+			if (ins.a == TCG_FX_IMM)
 			{
-				const int sa = fx_slot(ins.a);
 #pragma unroll
-				for (int e = 0; e < N; ++e) { va[e] = ins.a == TCG_FX_IMM ? imm : slot[sa][e]; }
+				for (int e = 0; e < N; ++e) { va[e] = imm; }
 			}
+			else { fx_get<T,N>(file, fx_slot(ins.a), va); }
 			if (ins.opcode == TCG_FX_STORE)
 			{
 				T* dst = (T*) p.out[ins.dst] + (uint64_t) idx * N;
@@ -172,26 +227,38 @@ __global__ __launch_bounds__(FX_BLOCK) void ew_fusedx_k (FxArgs p)
 			const bool has_c = ins.c != TCG_FX_NONE;
 			if (has_b)
 			{
-				const int sb = fx_slot(ins.b);
+				if (ins.b == TCG_FX_IMM)
+				{
 #pragma unroll
-				for (int e = 0; e < N; ++e) { vb[e] = ins.b == TCG_FX_IMM ? imm : slot[sb][e]; }
+					for (int e = 0; e < N; ++e) { vb[e] = imm; }
+				}
+				else { fx_get<T,N>(file, fx_slot(ins.b), vb); }
 			}
 			if (has_c)
 			{
-				const int sc = fx_slot(ins.c);
+				if (ins.c == TCG_FX_IMM)
+				{
 #pragma unroll
-				for (int e = 0; e < N; ++e) { vc[e] = ins.c == TCG_FX_IMM ? imm : slot[sc][e]; }
+					for (int e = 0; e < N; ++e) { vc[e] = imm; }
+				}
+				else { fx_get<T,N>(file, fx_slot(ins.c), vc); }
 			}
-			const int sd = fx_slot(ins.dst);
-#pragma unroll
-			for (int e = 0; e < N; ++e)
+			if (has_c)
 			{
-				T r;
-				if (has_c) { r = va[e] != (T) 0 ? vb[e] : vc[e]; } // SELECT
-				else if (has_b) { r = apply_binary<T>(ins.opcode, va[e], vb[e]); }
-				else { r = apply_unary<T>(ins.opcode, va[e]); }
-				slot[sd][e] = r;
+#pragma unroll
+				for (int e = 0; e < N; ++e) { vr[e] = va[e] != (T) 0 ? vb[e] : vc[e]; } // SELECT
 			}
+			else if (has_b)
+			{
+#pragma unroll
+				for (int e = 0; e < N; ++e) { vr[e] = apply_binary<T>(ins.opcode, va[e], vb[e]); }
+			}
+			else
+			{
+#pragma unroll
+				for (int e = 0; e < N; ++e) { vr[e] = apply_unary<T>(ins.opcode, va[e]); }
+			}
+			fx_put<T,N>(file, fx_slot(ins.dst), vr);
 		}
 	}
 }
@@ -212,6 +279,267 @@ int fusedx_launch (tcg_ctx* ctx, FxArgs& p, bool vec)
 		ew_fusedx_k<T,1><<<grid, FX_BLOCK, 0, ctx->stream>>>(p);
 	}
 	TCG_LAUNCH_CHECK(ctx, "ew_fusedx");
+	return TCG_OK;
+}
+
+// ---- kernels compiled at run time ------------------------------------------
+//
+// The interpreter above pays for decoding the program in every wave.  A group
+// that is evaluated again and again (every step of an unrolled recurrent
+// graph, every replay of a recording) is better served by a kernel written
+// for it: the program becomes straight-line code over named registers, the
+// number of dims and the way each leaf is addressed are fixed in the source.
+// Extents, strides, offsets, bounds, immediates and pointers stay launch
+// arguments, so one kernel serves every launch of the same program shape.
+// The source is built from the same scalar routines (ew_scalar_core.inc) and
+// compiled by the runtime compiler with the flags the library is built with.
+
+#define TCG_CORE(...) #__VA_ARGS__
+const char* const fx_scalar_src =
+#include "ew_scalar_core.inc"
+;
+const char* const fx_args_src =
+#include "ew_fusedx_args.inc"
+;
+#undef TCG_CORE
+
+struct FxJit
+{
+	std::mutex mu;
+	std::unordered_map<std::string,hipFunction_t> kernels;
+};
+
+FxJit& fx_jit (void)
+{
+	// never destroyed: loaded code may be launched until the process ends
+	static FxJit* jit = new FxJit();
+	return *jit;
+}
+
+bool fx_jit_enabled (void)
+{
+	static const bool on = []
+	{
+		const char* env = getenv("TCG_FX_JIT");
+		return !(env && env[0] == '0');
+	}();
+	return on;
+}
+
+// dense: the leaf is addressed like the output (offset + linear index)
+std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
+{
+	const char* tname = dtype == TCG_DOUBLE ? "double" : dtype == TCG_FLOAT ? "float" : "int";
+	std::ostringstream o;
+	o << "typedef signed char int8_t; typedef unsigned char uint8_t; typedef int int32_t;\n"
+		"typedef unsigned int uint32_t; typedef long int64_t; typedef unsigned long uint64_t;\n"
+		"#ifndef INT32_MIN\n#define INT32_MIN (-2147483647 - 1)\n#endif\n"
+		"#define FX_MAXD " << FX_MAXD << "\n"
+		"#define TCG_FX_MAX_LEAVES " << TCG_FX_MAX_LEAVES << "\n"
+		"#define TCG_FX_MAX_INSTRS " << TCG_FX_MAX_INSTRS << "\n"
+		"#define TCG_FX_MAX_OUTS " << TCG_FX_MAX_OUTS << "\n";
+	static const struct { const char* name; int value; } opcodes[] = {
+#define FX_OP(n) {#n, n}
+		FX_OP(TCG_IDENTITY), FX_OP(TCG_ABS), FX_OP(TCG_NEG), FX_OP(TCG_SIN), FX_OP(TCG_COS), FX_OP(TCG_TAN),
+		FX_OP(TCG_EXP), FX_OP(TCG_LOG), FX_OP(TCG_SQRT), FX_OP(TCG_ROUND), FX_OP(TCG_SIGMOID), FX_OP(TCG_TANH),
+		FX_OP(TCG_SQUARE), FX_OP(TCG_CUBE), FX_OP(TCG_POW), FX_OP(TCG_ADD), FX_OP(TCG_SUB), FX_OP(TCG_MUL),
+		FX_OP(TCG_DIV), FX_OP(TCG_MIN), FX_OP(TCG_MAX), FX_OP(TCG_EQ), FX_OP(TCG_NEQ), FX_OP(TCG_LT), FX_OP(TCG_GT),
+#undef FX_OP
+	};
+	o << "enum {";
+	for (auto& op : opcodes) { o << op.name << " = " << op.value << ", "; }
+	o << "};\n" << fx_scalar_src << "\n" << fx_args_src << "\n";
+	o << "typedef " << tname << " T;\n";
+	if (N > 1)
+	{
+		o << "typedef T VT __attribute__((ext_vector_type(" << N << ")));\n"
+			"union VU { VT v; T e[" << N << "]; };\n";
+	}
+	o << "extern \"C\" __global__ __launch_bounds__(" << FX_BLOCK << ") void fx (FxArgs p)\n{\n"
+		"const uint32_t nvec = (uint32_t) (p.total / " << N << ");\n"
+		"const uint32_t step = gridDim.x * " << FX_BLOCK << ";\n"
+		"for (uint32_t idx = blockIdx.x * " << FX_BLOCK << " + threadIdx.x; idx < nvec; idx += step)\n{\n";
+	bool need_coords = false;
+	for (uint32_t k = 0; k < p.nleaf; ++k) { need_coords = need_coords || !dense[k]; }
+	if (need_coords)
+	{
+		o << "uint32_t rem = idx;\n";
+		for (uint32_t d = 0; d + 1 < p.nd; ++d)
+		{
+			o << "const uint32_t q" << d << " = fx_div(rem, p.div[" << d << "]);\n"
+				"uint32_t c" << d << " = rem - q" << d << " * p.div[" << d << "].d;\nrem = q" << d << ";\n";
+		}
+		o << "uint32_t c" << p.nd - 1 << " = rem;\n";
+		if (N > 1) { o << "c0 *= " << N << ";\n"; }
+	}
+	for (uint32_t k = 0; k < p.nleaf; ++k)
+	{
+		const FxLeaf& L = p.leaf[k];
+		o << "T l" << k << "[" << N << "];\n{\n";
+		if (dense[k])
+		{
+			o << "const T* src = (const T*) p.leaf[" << k << "].ptr + (p.leaf[" << k << "].off + (int64_t) idx * " << N << ");\n";
+		}
+		else
+		{
+			o << "int64_t off = p.leaf[" << k << "].off";
+			for (uint32_t d = 0; d < p.nd; ++d)
+			{
+				if (d == 0 && L.bcast0) { continue; }
+				o << " + (int64_t) c" << d << " * p.leaf[" << k << "].stride[" << d << "]";
+			}
+			o << ";\nconst T* src = (const T*) p.leaf[" << k << "].ptr + off;\n";
+		}
+		if (L.boxed)
+		{
+			o << "bool inside = true";
+			for (uint32_t d = 0; d < p.nd; ++d)
+			{
+				o << " && c" << d << " >= p.leaf[" << k << "].lo[" << d << "] && c" << d << " < p.leaf[" << k << "].hi[" << d << "]";
+			}
+			o << ";\nif (inside)\n";
+		}
+		o << "{\n";
+		if (N > 1 && !L.bcast0)
+		{
+			o << "VU v; v.v = *(const VT*) src;\n";
+			for (int e = 0; e < N; ++e) { o << "l" << k << "[" << e << "] = v.e[" << e << "];\n"; }
+		}
+		else
+		{
+			o << "const T s = *src;\n";
+			for (int e = 0; e < N; ++e) { o << "l" << k << "[" << e << "] = s;\n"; }
+		}
+		o << "}\n";
+		if (L.boxed)
+		{
+			o << "else\n{\n";
+			for (int e = 0; e < N; ++e) { o << "l" << k << "[" << e << "] = (T) 0;\n"; }
+			o << "}\n";
+		}
+		o << "}\n";
+	}
+	// straight-line program: every write of a register gets a name of its own
+	std::string reg_name[TCG_FX_MAX_REGS];
+	auto operand = [&](int code, uint32_t i, int e) -> std::string
+	{
+		if (code == TCG_FX_IMM) { return "imm" + std::to_string(i); }
+		if (code >= TCG_FX_REG0) { return reg_name[code - TCG_FX_REG0] + "[" + std::to_string(e) + "]"; }
+		return "l" + std::to_string(code - TCG_FX_LEAF0) + "[" + std::to_string(e) + "]";
+	};
+	for (uint32_t i = 0; i < p.ninstr; ++i)
+	{
+		const FxInstr& ins = p.prog[i];
+		bool uses_imm = ins.a == TCG_FX_IMM || ins.b == TCG_FX_IMM || ins.c == TCG_FX_IMM;
+		if (uses_imm) { o << "const T imm" << i << " = (T) p.imm[" << i << "];\n"; }
+		if (ins.opcode == TCG_FX_STORE)
+		{
+			o << "{\nT* dst = (T*) p.out[" << (int) ins.dst << "] + (uint64_t) idx * " << N << ";\n";
+			if (N > 1)
+			{
+				o << "VU v;\n";
+				for (int e = 0; e < N; ++e) { o << "v.e[" << e << "] = " << operand(ins.a, i, e) << ";\n"; }
+				o << "*(VT*) dst = v.v;\n";
+			}
+			else { o << "*dst = " << operand(ins.a, i, 0) << ";\n"; }
+			o << "}\n";
+			continue;
+		}
+		std::string name = "v" + std::to_string(i);
+		o << "T " << name << "[" << N << "];\n";
+		for (int e = 0; e < N; ++e)
+		{
+			o << name << "[" << e << "] = ";
+			if (ins.c != TCG_FX_NONE)
+			{
+				o << operand(ins.a, i, e) << " != (T) 0 ? " << operand(ins.b, i, e) << " : " << operand(ins.c, i, e);
+			}
+			else if (ins.b != TCG_FX_NONE)
+			{
+				o << "apply_binary<T>(" << (int) ins.opcode << ", " << operand(ins.a, i, e) << ", " << operand(ins.b, i, e) << ")";
+			}
+			else
+			{
+				o << "apply_unary<T>(" << (int) ins.opcode << ", " << operand(ins.a, i, e) << ")";
+			}
+			o << ";\n";
+		}
+		reg_name[ins.dst - TCG_FX_REG0] = name;
+	}
+	o << "}\n}\n";
+	return o.str();
+}
+
+int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out)
+{
+	hiprtcProgram prog;
+	hiprtcResult rc = hiprtcCreateProgram(&prog, source.c_str(), "fused_group.hip", 0, nullptr, nullptr);
+	if (rc != HIPRTC_SUCCESS)
+	{
+		return tcg_fail(ctx, TCG_ERR_HIP, "tcg_ew_fusedx: hiprtcCreateProgram: %s", hiprtcGetErrorString(rc));
+	}
+	std::string arch = "--offload-arch=" + ctx->arch;
+	// the flags libtcg itself is built with (packed fp32 forms stay off), and
+	// no contraction: a multiply node feeding an add node must round twice, as
+	// it does when the two nodes run as separate kernels
+	const char* opts[] = {arch.c_str(), "-O3", "-std=c++17", "-ffp-contract=off",
+		"-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+	rc = hiprtcCompileProgram(prog, (int) (sizeof(opts) / sizeof(opts[0])), opts);
+	if (rc != HIPRTC_SUCCESS)
+	{
+		size_t n = 0;
+		hiprtcGetProgramLogSize(prog, &n);
+		std::string log(n, '\0');
+		if (n) { hiprtcGetProgramLog(prog, &log[0]); }
+		hiprtcDestroyProgram(&prog);
+		if (log.size() > 800) { log.resize(800); }
+		return tcg_fail(ctx, TCG_ERR_HIP, "tcg_ew_fusedx: run-time compilation failed: %s", log.c_str());
+	}
+	size_t size = 0;
+	hiprtcGetCodeSize(prog, &size);
+	std::vector<char> code(size);
+	hiprtcGetCode(prog, code.data());
+	hiprtcDestroyProgram(&prog);
+	hipModule_t module;
+	TCG_HIP(ctx, hipModuleLoadData(&module, code.data()));
+	TCG_HIP(ctx, hipModuleGetFunction(out, module, "fx"));
+	return TCG_OK;
+}
+
+int fusedx_jit_launch (tcg_ctx* ctx, int dtype, FxArgs& p, bool vec)
+{
+	const int N = vec ? (int) (16 / tcg_type_size(dtype)) : 1;
+	if (vec) { p.div[0] = fx_make_div(p.size[0] / N); }
+	bool dense[TCG_FX_MAX_LEAVES];
+	for (uint32_t k = 0; k < p.nleaf; ++k)
+	{
+		const FxLeaf& L = p.leaf[k];
+		dense[k] = !L.boxed;
+		int64_t run = 1;
+		for (uint32_t d = 0; d < p.nd && dense[k]; ++d)
+		{
+			dense[k] = L.stride[d] == run;
+			run *= (int64_t) p.size[d];
+		}
+	}
+	std::string source = fx_source(dtype, N, p, dense);
+	FxJit& jit = fx_jit();
+	hipFunction_t fn = nullptr;
+	{
+		std::lock_guard<std::mutex> lock(jit.mu);
+		auto it = jit.kernels.find(source);
+		if (it == jit.kernels.end())
+		{
+			int rc = fx_compile(ctx, source, &fn);
+			if (rc != TCG_OK) { return rc; }
+			jit.kernels.emplace(source, fn);
+		}
+		else { fn = it->second; }
+	}
+	unsigned grid = tcg_grid(ctx, p.total / N, FX_BLOCK, 16);
+	size_t size = sizeof(FxArgs);
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &p, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+	TCG_HIP(ctx, hipModuleLaunchKernel(fn, grid, 1, 1, FX_BLOCK, 1, 1, 0, ctx->stream, nullptr, config));
 	return TCG_OK;
 }
 
@@ -359,6 +687,7 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		}
 		if (L.boxed) { vec = vec && L.lo[0] % N == 0 && L.hi[0] % N == 0; }
 	}
+	if (fx_jit_enabled()) { return fusedx_jit_launch(ctx, dtype, p, vec); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return fusedx_launch<T>(ctx, p, vec));
 	return TCG_OK;
 }
