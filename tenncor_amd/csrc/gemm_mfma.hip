@@ -29,6 +29,10 @@ struct GemmArgs
 	int64_t lda, ldb, ldc;
 	int64_t batch_a, batch_b, batch_c;
 	uint32_t tiles_m, tiles_n, tiles_per_batch, total_tiles;
+	// split K: block id / total_tiles picks a K range of k_per_split columns;
+	// with more than one range the C tile goes to partial[range][batch][M][N]
+	uint32_t k_per_split;
+	float* partial;
 };
 
 // TA: A(m,k) at m + k*lda (M contiguous) instead of m*lda + k.
@@ -46,7 +50,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 	__shared__ __attribute__((aligned(16))) float Bs[2][BK * BP];
 
 	// ---- which tile: XCD-aware, grouped order --------------------------------
-	uint32_t id = blockIdx.x;
+	const uint32_t split = blockIdx.x / g.total_tiles;
+	uint32_t id = blockIdx.x - split * g.total_tiles;
+	const uint32_t k_begin = split * g.k_per_split;
+	const uint32_t k_end = g.K - k_begin < g.k_per_split ? g.K : k_begin + g.k_per_split;
 	if (g.total_tiles % NXCD == 0)
 	{
 		id = (id % NXCD) * (g.total_tiles / NXCD) + id / NXCD;
@@ -63,7 +70,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 	const uint32_t m0 = tm * BM, n0 = tn * BN;
 	const float* __restrict__ A = g.A + (int64_t) bz * g.batch_a;
 	const float* __restrict__ B = g.B + (int64_t) bz * g.batch_b;
-	float* __restrict__ C = g.C + (int64_t) bz * g.batch_c;
+	float* __restrict__ C = g.partial ?
+		g.partial + ((int64_t) split * (g.total_tiles / g.tiles_per_batch) + bz) * ((int64_t) g.M * g.N) :
+		g.C + (int64_t) bz * g.batch_c;
+	const int64_t ldc = g.partial ? (int64_t) g.N : g.ldc;
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63, wave = tid >> 6;
@@ -96,14 +106,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 				// K contiguous: BK/4 lanes per row
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t m = m0 + mm, k = k0 + kq * 4;
-				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * g.lda + k) : zero4;
+				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * g.lda + k) : zero4;
 			}
 			else
 			{
 				// M contiguous: BM/4 lanes per k
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
 				uint32_t m = m0 + mq * 4, k = k0 + kk;
-				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) k * g.lda + m) : zero4;
+				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) k * g.lda + m) : zero4;
 			}
 		}
 #pragma unroll
@@ -115,14 +125,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 				// N contiguous: BN/4 lanes per k
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
 				uint32_t n = n0 + nq * 4, k = k0 + kk;
-				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) k * g.ldb + n) : zero4;
+				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) k * g.ldb + n) : zero4;
 			}
 			else
 			{
 				// K contiguous: BK/4 lanes per n
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t n = n0 + nn, k = k0 + kq * 4;
-				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * g.ldb + k) : zero4;
+				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * g.ldb + k) : zero4;
 			}
 		}
 	};
@@ -166,14 +176,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 		}
 	};
 
-	const uint32_t nslabs = (g.K + BK - 1) / BK;
-	load_slab(0);
+	const uint32_t nslabs = (k_end - k_begin + BK - 1) / BK;
+	load_slab(k_begin);
 	store_slab(0);
 	__syncthreads();
 	for (uint32_t s = 0; s < nslabs; ++s)
 	{
 		const int buf = s & 1;
-		if (s + 1 < nslabs) { load_slab((s + 1) * BK); }
+		if (s + 1 < nslabs) { load_slab(k_begin + (s + 1) * BK); }
 		const float* as = As[buf] + (wm * WM + l32) * AP + lh;
 		const float* bs = Bs[buf] + lh * BP + wn * WN + l32;
 #pragma unroll
@@ -211,14 +221,32 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 			for (int r = 0; r < 16; ++r)
 			{
 				const uint32_t m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-				if (m < g.M) { C[(int64_t) m * g.ldc + n] = acc[i][j][r]; }
+				if (m < g.M) { C[(int64_t) m * ldc + n] = acc[i][j][r]; }
 			}
 		}
 	}
 }
 
+// C[b][m][n] = partial[0][b][m][n] + partial[1][b][m][n] + ... in that order
+__global__ __launch_bounds__(256) void gemm_split_sum_k (const float* __restrict__ partial, float* __restrict__ C,
+	uint32_t splits, uint32_t M, uint32_t N, uint32_t batch, int64_t ldc, int64_t batch_c)
+{
+	const uint64_t per_split = (uint64_t) batch * M * N;
+	const uint64_t step = (uint64_t) gridDim.x * 256;
+	for (uint64_t i = (uint64_t) blockIdx.x * 256 + threadIdx.x; i < per_split; i += step)
+	{
+		float acc = partial[i];
+		for (uint32_t s = 1; s < splits; ++s) { acc += partial[s * per_split + i]; }
+		const uint32_t n = (uint32_t) (i % N);
+		const uint64_t bm = i / N;
+		const uint32_t m = (uint32_t) (bm % M);
+		const uint64_t b = bm / M;
+		C[b * batch_c + (int64_t) m * ldc + n] = acc;
+	}
+}
+
 template <int BM, int BN>
-int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b)
+int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1)
 {
 	GemmArgs g = base;
 	uint64_t tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
@@ -228,10 +256,37 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	g.tiles_n = (uint32_t) tiles_n;
 	g.tiles_per_batch = (uint32_t) (tiles_m * tiles_n);
 	g.total_tiles = (uint32_t) total;
-	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,false,false><<<g.total_tiles, 256, 0, ctx->stream>>>(g); }
-	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,true,false><<<g.total_tiles, 256, 0, ctx->stream>>>(g); }
-	else if (!trans_a && trans_b) { gemm_mfma_k<BM,BN,false,true><<<g.total_tiles, 256, 0, ctx->stream>>>(g); }
-	else { gemm_mfma_k<BM,BN,true,true><<<g.total_tiles, 256, 0, ctx->stream>>>(g); }
+	g.k_per_split = g.K;
+	g.partial = nullptr;
+	size_t partial_bytes = 0;
+	if (splits > 1)
+	{
+		// ranges are whole slabs; the last one may be shorter
+		g.k_per_split = ((g.K + splits - 1) / splits + BK - 1) / BK * BK;
+		splits = (g.K + g.k_per_split - 1) / g.k_per_split;
+	}
+	if (splits > 1)
+	{
+		TCG_REQUIRE(ctx, total * splits < (1ull << 31), "tcg_gemm: too many tiles for one launch");
+		partial_bytes = sizeof(float) * splits * batch * g.M * g.N;
+		void* buf = nullptr;
+		int rc = tcg_alloc(ctx, partial_bytes, &buf);
+		if (rc != TCG_OK) { return rc; }
+		g.partial = (float*) buf;
+	}
+	else { splits = 1; }
+	const unsigned grid = g.total_tiles * splits;
+	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (!trans_a && trans_b) { gemm_mfma_k<BM,BN,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	else { gemm_mfma_k<BM,BN,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	if (g.partial)
+	{
+		uint64_t n = batch * g.M * g.N;
+		unsigned rgrid = tcg_grid(ctx, n, 256, 8);
+		gemm_split_sum_k<<<rgrid, 256, 0, ctx->stream>>>(g.partial, g.C, splits, g.M, g.N, (uint32_t) batch, g.ldc, g.batch_c);
+		tcg_free(ctx, g.partial, partial_bytes);
+	}
 	TCG_LAUNCH_CHECK(ctx, "gemm_mfma");
 	return TCG_OK;
 }
@@ -262,5 +317,13 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	// small problems: smaller tiles so that the grid still covers the chip
 	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
 	if (big_tiles >= (uint64_t) ctx->num_cus) { return launch<128,128>(ctx, g, batch, trans_a, trans_b); }
-	return launch<64,64>(ctx, g, batch, trans_a, trans_b);
+	// still too few tiles for the chip and a long K: several workgroups share a
+	// tile, each summing a range of K, and a second kernel adds the ranges up
+	// in a fixed order (so that results do not depend on scheduling)
+	uint64_t tiles = ((M + 63) / 64) * ((N + 63) / 64) * batch;
+	uint64_t splits = 2 * (uint64_t) ctx->num_cus / tiles;
+	if (splits > K / 64) { splits = K / 64; }
+	if (splits > 32) { splits = 32; }
+	if (splits < 2 || batch >= (1ull << 16)) { splits = 1; }
+	return launch<64,64>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
 }

@@ -393,6 +393,8 @@ GEMM_CASES = [
     (128, 128, 64, 1, 0, 0), (128, 128, 64, 1, 1, 0), (128, 128, 64, 1, 0, 1), (128, 128, 64, 1, 1, 1),
     (100, 36, 40, 1, 0, 0), (100, 36, 40, 3, 1, 1), (260, 132, 72, 2, 1, 0), (260, 132, 72, 2, 0, 1),
     (512, 384, 200, 1, 0, 0), (2048, 256, 768, 1, 1, 0), (768, 2048, 256, 1, 0, 1),
+    # few tiles, long K: several workgroups share a tile (K split in ranges, last one ragged)
+    (256, 768, 2048, 1, 0, 1), (256, 2048, 768, 1, 0, 0), (64, 96, 1000, 2, 1, 0), (36, 44, 4100, 1, 0, 0),
     # off the matrix-core path: odd extents
     (33, 35, 17, 2, 0, 0), (33, 35, 17, 2, 1, 1),
 ]
