@@ -143,6 +143,402 @@ __global__ __launch_bounds__(CV_BLOCK) void conv_boxed_k (ConvPlan p,
 	}
 }
 
+// ---- lowering to a matrix product ------------------------------------------
+//
+// Per image dim d (kernel extent K_d, image non-zero box [lo, hi), output
+// window W_d) the correlation does one of three things:
+//   K_d == 1            the output coordinate indexes the image directly:
+//                       a row dim of the product (batch-like);
+//   hi - lo == 1        only one kernel index per output coordinate meets the
+//                       box (w = lo - x): no sum, the output coordinate picks
+//                       the kernel slice: a column dim (this is how conv2d
+//                       spells "output channels": a singleton axis padded to
+//                       2*O - 1 and correlated with the O filters);
+//   otherwise           the output coordinate is a row dim and the kernel
+//                       coordinate a summed dim (spatial dims; a dim whose
+//                       output extent is 1 is a plain summed channel dim).
+// So out[rows, cols] = A[rows, sums] * B[sums, cols] with A gathered from the
+// image (zero outside its box) and B gathered from the kernel.  A and B are
+// materialised (A in row chunks of bounded size), the product runs on the GEMM
+// path (matrix cores for fp32), and the result is scattered to the window.
+// Reads of A are the dominant traffic: rows*sums elements written and read once.
+
+struct ConvDiv
+{
+	uint32_t d, m, s1, s2;
+};
+
+ConvDiv conv_make_div (uint32_t d)
+{
+	ConvDiv f = {d, 0, 0, 0};
+	uint32_t l = 0;
+	while (((uint64_t) 1 << l) < d) { ++l; }
+	f.m = (uint32_t) ((((uint64_t) 1 << 32) * (((uint64_t) 1 << l) - d)) / d + 1);
+	f.s1 = l < 1 ? l : 1;
+	f.s2 = l == 0 ? 0 : l - 1;
+	return f;
+}
+
+__device__ __forceinline__ uint32_t conv_div (uint32_t n, const ConvDiv& f)
+{
+	uint32_t t = __umulhi(f.m, n);
+	return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
+struct ConvGemmPlan
+{
+	// per image dim: extents of its row, summed and column component (1 = none)
+	uint32_t msize[8], ssize[8], nsize[8];
+	ConvDiv mdiv[8], sdiv[8], ndiv[8];
+	int32_t xlo[8];     // first output coordinate of the window, in image coordinates
+	int32_t oxlo[8];    // the same in output coordinates (they differ when the
+	                    // image has been cut down to its non-zero box)
+	int32_t slo[8];     // first summed kernel coordinate
+	uint32_t is_col[8]; // column dim: image coordinate fixed at ilo, kernel index ilo - x
+	int32_t ilo[8], ihi[8];
+	uint32_t ksize[8];
+	int64_t istr[8], ostr[8], kstr[8];
+	uint32_t M, N, S;   // rows, columns, summed
+	uint32_t Sp, Np;    // padded to multiples of 4 (leading dims of A / B and C)
+	// dims where a row coordinate and a summed coordinate (or the box) decide
+	// together whether the image element exists; -1 pads the list
+	int32_t check_dim[4];
+	uint32_t check_ext[4];
+	int32_t ncheck;     // -1: more than four, the general gather handles them
+};
+
+// Per row / per summed index: image offset and, for the checked dims, the
+// coordinate relative to the box start (row part and summed part add up)
+struct ConvTabEntry
+{
+	int64_t off;
+	int32_t c[4];
+};
+
+constexpr int CG_BLOCK = 256;
+
+// A[m - m0][s] for m in [m0, m0 + rows)
+template <typename T>
+__global__ __launch_bounds__(CG_BLOCK) void conv_gather_image_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
+	const T* __restrict__ img, T* __restrict__ A)
+{
+	const uint64_t total = (uint64_t) rows * p.Sp;
+	const uint64_t step = (uint64_t) gridDim.x * CG_BLOCK;
+	for (uint64_t i = (uint64_t) blockIdx.x * CG_BLOCK + threadIdx.x; i < total; i += step)
+	{
+		uint32_t r = (uint32_t) (i / p.Sp);
+		uint32_t s = (uint32_t) (i - (uint64_t) r * p.Sp);
+		T v = 0;
+		if (s < p.S)
+		{
+			uint32_t rm = m0 + r, rs = s;
+			int64_t off = 0;
+			bool inside = true;
+#pragma unroll
+			for (int d = 0; d < 8; ++d)
+			{
+				uint32_t qm = conv_div(rm, p.mdiv[d]);
+				int32_t x = (int32_t) (rm - qm * p.msize[d]);
+				rm = qm;
+				uint32_t qs = conv_div(rs, p.sdiv[d]);
+				int32_t w = (int32_t) (rs - qs * p.ssize[d]);
+				rs = qs;
+				int32_t c = p.is_col[d] ? p.ilo[d] : p.xlo[d] + x + p.slo[d] + w;
+				inside = inside && c >= p.ilo[d] && c < p.ihi[d];
+				off += (int64_t) c * p.istr[d];
+			}
+			if (inside) { v = img[off]; }
+		}
+		A[i] = v;
+	}
+}
+
+// rows: entry m describes output row m; sums: entry s describes summed index s
+__global__ __launch_bounds__(CG_BLOCK) void conv_tables_k (ConvGemmPlan p, ConvTabEntry* __restrict__ rows,
+	ConvTabEntry* __restrict__ sums)
+{
+	const uint32_t i = blockIdx.x * CG_BLOCK + threadIdx.x;
+	if (i < p.M)
+	{
+		uint32_t rm = i;
+		ConvTabEntry e;
+		e.off = 0;
+		e.c[0] = e.c[1] = e.c[2] = e.c[3] = 0;
+#pragma unroll
+		for (int d = 0; d < 8; ++d)
+		{
+			uint32_t qm = conv_div(rm, p.mdiv[d]);
+			int32_t x = (int32_t) (rm - qm * p.msize[d]);
+			rm = qm;
+			int32_t c = p.is_col[d] ? p.ilo[d] : p.xlo[d] + x;
+			e.off += (int64_t) c * p.istr[d];
+#pragma unroll
+			for (int j = 0; j < 4; ++j)
+			{
+				if (p.check_dim[j] == d) { e.c[j] = c - p.ilo[d]; }
+			}
+		}
+		rows[i] = e;
+	}
+	if (i < p.Sp)
+	{
+		uint32_t rs = i;
+		ConvTabEntry e;
+		e.off = 0;
+		e.c[0] = e.c[1] = e.c[2] = e.c[3] = 0;
+#pragma unroll
+		for (int d = 0; d < 8; ++d)
+		{
+			uint32_t qs = conv_div(rs, p.sdiv[d]);
+			int32_t w = (int32_t) (rs - qs * p.ssize[d]) + p.slo[d];
+			rs = qs;
+			e.off += (int64_t) w * p.istr[d];
+#pragma unroll
+			for (int j = 0; j < 4; ++j)
+			{
+				if (p.check_dim[j] == d) { e.c[j] = w; }
+			}
+		}
+		// padding columns of A: a coordinate no row can complete into the box
+		if (i >= p.S) { e.c[0] = INT32_MIN / 2; }
+		sums[i] = e;
+	}
+}
+
+constexpr int CG_ROWS = 16;
+
+// A[m - m0][s] from the two tables: one summed index per lane, CG_ROWS rows per workgroup
+template <typename T, int NCHECK>
+__global__ __launch_bounds__(CG_BLOCK) void conv_gather_tab_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
+	const ConvTabEntry* __restrict__ rowtab, const ConvTabEntry* __restrict__ sumtab,
+	const T* __restrict__ img, T* __restrict__ A)
+{
+	const uint32_t s = blockIdx.x * CG_BLOCK + threadIdx.x;
+	if (s >= p.Sp) { return; }
+	const ConvTabEntry col = sumtab[s];
+	const bool pad_col = s >= p.S;
+	const uint32_t r0 = blockIdx.y * CG_ROWS;
+#pragma unroll 4
+	for (uint32_t r = r0; r < r0 + CG_ROWS && r < rows; ++r)
+	{
+		const ConvTabEntry row = rowtab[m0 + r];
+		bool inside = !pad_col;
+#pragma unroll
+		for (int j = 0; j < NCHECK; ++j)
+		{
+			inside = inside && (uint32_t) (row.c[j] + col.c[j]) < p.check_ext[j];
+		}
+		T v = 0;
+		if (inside) { v = img[row.off + col.off]; }
+		A[(uint64_t) r * p.Sp + s] = v;
+	}
+}
+
+// B[s][n]
+template <typename T>
+__global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_k (ConvGemmPlan p,
+	const T* __restrict__ ker, T* __restrict__ B)
+{
+	const uint64_t total = (uint64_t) p.Sp * p.Np;
+	const uint64_t step = (uint64_t) gridDim.x * CG_BLOCK;
+	for (uint64_t i = (uint64_t) blockIdx.x * CG_BLOCK + threadIdx.x; i < total; i += step)
+	{
+		uint32_t s = (uint32_t) (i / p.Np);
+		uint32_t n = (uint32_t) (i - (uint64_t) s * p.Np);
+		T v = 0;
+		if (s < p.S && n < p.N)
+		{
+			uint32_t rs = s, rn = n;
+			int64_t off = 0;
+			bool valid = true;
+#pragma unroll
+			for (int d = 0; d < 8; ++d)
+			{
+				uint32_t qs = conv_div(rs, p.sdiv[d]);
+				int32_t w = (int32_t) (rs - qs * p.ssize[d]) + p.slo[d];
+				rs = qs;
+				uint32_t qn = conv_div(rn, p.ndiv[d]);
+				int32_t x = (int32_t) (rn - qn * p.nsize[d]) + p.xlo[d];
+				rn = qn;
+				if (p.is_col[d]) { w = p.ilo[d] - x; }
+				valid = valid && w >= 0 && w < (int32_t) p.ksize[d];
+				off += (int64_t) w * p.kstr[d];
+			}
+			if (valid) { v = ker[off]; }
+		}
+		B[i] = v;
+	}
+}
+
+// out[window coordinate of (m, n)] = C[m - m0][n]
+template <typename T>
+__global__ __launch_bounds__(CG_BLOCK) void conv_scatter_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
+	const T* __restrict__ C, T* __restrict__ out)
+{
+	const uint64_t total = (uint64_t) rows * p.N;
+	const uint64_t step = (uint64_t) gridDim.x * CG_BLOCK;
+	for (uint64_t i = (uint64_t) blockIdx.x * CG_BLOCK + threadIdx.x; i < total; i += step)
+	{
+		uint32_t r = (uint32_t) (i / p.N);
+		uint32_t n = (uint32_t) (i - (uint64_t) r * p.N);
+		uint32_t rm = m0 + r, rn = n;
+		int64_t off = 0;
+#pragma unroll
+		for (int d = 0; d < 8; ++d)
+		{
+			uint32_t qm = conv_div(rm, p.mdiv[d]);
+			int32_t xm = (int32_t) (rm - qm * p.msize[d]);
+			rm = qm;
+			uint32_t qn = conv_div(rn, p.ndiv[d]);
+			int32_t xn = (int32_t) (rn - qn * p.nsize[d]);
+			rn = qn;
+			off += (int64_t) (p.oxlo[d] + xm + xn) * p.ostr[d];
+		}
+		out[off] = C[(uint64_t) r * p.Np + n];
+	}
+}
+
+// Whether the product form pays: enough columns to fill matrix tiles and
+// enough work to amortise materialising the operands
+bool conv_gemm_plan (const ConvPlan& c, ConvGemmPlan& g)
+{
+	uint64_t M = 1, N = 1, S = 1;
+	for (int d = 0; d < 8; ++d)
+	{
+		g.msize[d] = g.ssize[d] = g.nsize[d] = 1;
+		g.xlo[d] = (int32_t) c.wlo[d];
+		g.oxlo[d] = (int32_t) c.wlo[d];
+		g.slo[d] = 0;
+		g.is_col[d] = 0;
+		g.ilo[d] = c.ilo[d];
+		g.ihi[d] = c.ihi[d];
+		g.ksize[d] = c.ksize[d];
+		g.istr[d] = c.istr[d];
+		g.ostr[d] = c.ostr[d];
+		g.kstr[d] = c.kstr[d];
+		if (c.ksize[d] == 1) { g.msize[d] = c.wsize[d]; }
+		else if (c.ihi[d] - c.ilo[d] == 1)
+		{
+			g.nsize[d] = c.wsize[d];
+			g.is_col[d] = 1;
+		}
+		else
+		{
+			g.msize[d] = c.wsize[d];
+			// kernel coordinates that meet the box for some output of the window
+			int32_t first = c.ilo[d] - (int32_t) (c.wlo[d] + c.wsize[d] - 1);
+			int32_t last = c.ihi[d] - (int32_t) c.wlo[d]; // exclusive
+			if (first < 0) { first = 0; }
+			if (last > (int32_t) c.ksize[d]) { last = (int32_t) c.ksize[d]; }
+			if (last <= first) { return false; } // nothing to sum: the direct kernel writes the zeros
+			g.slo[d] = first;
+			g.ssize[d] = (uint32_t) (last - first);
+		}
+		g.mdiv[d] = conv_make_div(g.msize[d]);
+		g.sdiv[d] = conv_make_div(g.ssize[d]);
+		g.ndiv[d] = conv_make_div(g.nsize[d]);
+		M *= g.msize[d];
+		N *= g.nsize[d];
+		S *= g.ssize[d];
+	}
+	if (N < 8 || S < 8 || M < 32 || M >= (1ull << 31) || N >= (1ull << 31) || S >= (1ull << 31)) { return false; }
+	if (M * N * S < (1ull << 22)) { return false; }
+	g.M = (uint32_t) M;
+	g.N = (uint32_t) N;
+	g.S = (uint32_t) S;
+	g.Sp = (g.S + 3) & ~3u;
+	g.Np = (g.N + 3) & ~3u;
+	g.ncheck = 0;
+	for (int j = 0; j < 4; ++j)
+	{
+		g.check_dim[j] = -1;
+		g.check_ext[j] = 0;
+	}
+	for (int d = 0; d < 8; ++d)
+	{
+		if (g.is_col[d]) { continue; }
+		// coordinates this dim can take against the box
+		int64_t first = (int64_t) g.xlo[d] + g.slo[d];
+		int64_t last = first + (g.msize[d] - 1) + (g.ssize[d] - 1);
+		if (first >= g.ilo[d] && last < g.ihi[d]) { continue; } // always inside
+		if (g.ncheck >= 0 && g.ncheck < 4)
+		{
+			g.check_dim[g.ncheck] = d;
+			g.check_ext[g.ncheck] = (uint32_t) (g.ihi[d] - g.ilo[d]);
+			++g.ncheck;
+		}
+		else { g.ncheck = -1; }
+	}
+	return true;
+}
+
+template <typename T>
+int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img, const T* ker, T* out)
+{
+	// rows of A per pass: at most 512 MiB of gathered image at a time
+	uint64_t max_rows = ((512ull << 20) / sizeof(T)) / g.Sp;
+	if (max_rows < 64) { max_rows = 64; }
+	max_rows &= ~(uint64_t) 63;
+	uint32_t chunk = (uint32_t) (g.M < max_rows ? g.M : max_rows);
+	size_t a_bytes = sizeof(T) * (size_t) chunk * g.Sp;
+	size_t b_bytes = sizeof(T) * (size_t) g.Sp * g.Np;
+	size_t c_bytes = sizeof(T) * (size_t) chunk * g.Np;
+	size_t rt_bytes = sizeof(ConvTabEntry) * (size_t) g.M, st_bytes = sizeof(ConvTabEntry) * (size_t) g.Sp;
+	void *A = nullptr, *B = nullptr, *C = nullptr, *RT = nullptr, *ST = nullptr;
+	const bool tables = g.ncheck >= 0;
+	int rc = tcg_alloc(ctx, a_bytes, &A);
+	if (rc == TCG_OK) { rc = tcg_alloc(ctx, b_bytes, &B); }
+	if (rc == TCG_OK) { rc = tcg_alloc(ctx, c_bytes, &C); }
+	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, rt_bytes, &RT); }
+	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, st_bytes, &ST); }
+	if (rc == TCG_OK)
+	{
+		unsigned grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
+		conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
+		if (tables)
+		{
+			uint32_t longest = g.M > g.Sp ? g.M : g.Sp;
+			conv_tables_k<<<(longest + CG_BLOCK - 1) / CG_BLOCK, CG_BLOCK, 0, ctx->stream>>>(g,
+				(ConvTabEntry*) RT, (ConvTabEntry*) ST);
+		}
+		for (uint32_t m0 = 0; m0 < g.M && rc == TCG_OK; m0 += chunk)
+		{
+			uint32_t rows = g.M - m0 < chunk ? g.M - m0 : chunk;
+			if (tables)
+			{
+				dim3 tgrid((g.Sp + CG_BLOCK - 1) / CG_BLOCK, (rows + CG_ROWS - 1) / CG_ROWS);
+				const ConvTabEntry* rt = (const ConvTabEntry*) RT;
+				const ConvTabEntry* st = (const ConvTabEntry*) ST;
+				switch (g.ncheck)
+				{
+					case 0: conv_gather_tab_k<T,0><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
+					case 1: conv_gather_tab_k<T,1><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
+					case 2: conv_gather_tab_k<T,2><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
+					case 3: conv_gather_tab_k<T,3><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
+					default: conv_gather_tab_k<T,4><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
+				}
+			}
+			else
+			{
+				grid = tcg_grid(ctx, (uint64_t) rows * g.Sp, CG_BLOCK, 32);
+				conv_gather_image_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, img, (T*) A);
+			}
+			rc = tcg_gemm(ctx, dtype, rows, g.Np, g.Sp, 1, A, g.Sp, 0, 0, B, g.Np, 0, 0, C, g.Np, 0);
+			if (rc != TCG_OK) { break; }
+			grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
+			conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+		}
+	}
+	if (A) { tcg_free(ctx, A, a_bytes); }
+	if (B) { tcg_free(ctx, B, b_bytes); }
+	if (C) { tcg_free(ctx, C, c_bytes); }
+	if (RT) { tcg_free(ctx, RT, rt_bytes); }
+	if (ST) { tcg_free(ctx, ST, st_bytes); }
+	if (rc != TCG_OK) { return rc; }
+	TCG_LAUNCH_CHECK(ctx, "conv_gemm");
+	return TCG_OK;
+}
+
 } // namespace
 
 extern "C" {
@@ -215,6 +611,53 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 		p.nwin *= p.wsize[d];
 		uint64_t span = ihi - ilo < p.ksize[d] ? ihi - ilo : p.ksize[d];
 		max_terms *= span;
+	}
+	ConvGemmPlan gp;
+	if (conv_gemm_plan(p, gp))
+	{
+		// An image that is mostly padding (conv2d's image gradient pads the
+		// fastest dim from 1 to 2*C - 1) scatters its non-zero elements over
+		// memory: cut the box out into a dense buffer first, unless the box is
+		// one contiguous slab already (only the slowest dim is cut)
+		uint64_t box[8], lo[8], box_elems = 1, img_elems = 1;
+		int last_sig = 0, first_cut = 8;
+		for (int d = 0; d < 8; ++d)
+		{
+			lo[d] = (uint64_t) p.ilo[d];
+			box[d] = (uint64_t) (p.ihi[d] - p.ilo[d]);
+			box_elems *= box[d];
+			img_elems *= imgshape[d];
+			if (imgshape[d] > 1) { last_sig = d; }
+			if (box[d] < imgshape[d] && d < first_cut) { first_cut = d; }
+		}
+		size_t esz = tcg_type_size(dtype);
+		bool compact = esz && box_elems > 0 && first_cut < last_sig && box_elems * 2 <= img_elems &&
+			box_elems * esz <= (1ull << 30);
+		void* dense = nullptr;
+		if (compact)
+		{
+			int rc = tcg_alloc(ctx, box_elems * esz, &dense);
+			if (rc == TCG_OK) { rc = tcg_slice(ctx, dtype, imgshape, lo, box, img, dense); }
+			if (rc != TCG_OK)
+			{
+				if (dense) { tcg_free(ctx, dense, box_elems * esz); }
+				return rc;
+			}
+			int64_t run = 1;
+			for (int d = 0; d < 8; ++d)
+			{
+				gp.xlo[d] -= p.ilo[d];
+				gp.ilo[d] = 0;
+				gp.ihi[d] = (int32_t) box[d];
+				gp.istr[d] = run;
+				run *= (int64_t) box[d];
+			}
+			img = dense;
+		}
+		int rc = TCG_OK;
+		TCG_DISPATCH_TYPE(ctx, dtype, rc = conv_gemm_run<T>(ctx, dtype, gp, (const T*) img, (const T*) kernel, (T*) out));
+		if (dense) { tcg_free(ctx, dense, box_elems * esz); }
+		return rc;
 	}
 	// few outputs with long sums: give each output a whole workgroup
 	bool group = p.nwin < (uint64_t) ctx->num_cus * 64 * 16 && max_terms >= 2048;
