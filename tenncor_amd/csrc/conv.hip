@@ -16,6 +16,8 @@
 // an LDS tree at the end (few outputs, long sums: kernel gradients).
 #include "tcg_internal.hpp"
 
+#include <cstdlib>
+
 namespace
 {
 
@@ -477,6 +479,11 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 {
 	// rows of A per pass: at most 512 MiB of gathered image at a time
 	uint64_t max_rows = ((512ull << 20) / sizeof(T)) / g.Sp;
+	if (const char* env = getenv("TCG_CONV_CHUNK_ROWS")) // for tests of the chunked path
+	{
+		uint64_t forced = strtoull(env, nullptr, 10);
+		if (forced) { max_rows = forced; }
+	}
 	if (max_rows < 64) { max_rows = 64; }
 	max_rows &= ~(uint64_t) 63;
 	uint32_t chunk = (uint32_t) (g.M < max_rows ? g.M : max_rows);
@@ -613,7 +620,8 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 		max_terms *= span;
 	}
 	ConvGemmPlan gp;
-	if (conv_gemm_plan(p, gp))
+	const char* gemm_env = getenv("TCG_CONV_GEMM"); // "0": direct kernels only (the parity reference)
+	if (!(gemm_env && gemm_env[0] == '0') && conv_gemm_plan(p, gp))
 	{
 		// An image that is mostly padding (conv2d's image gradient pads the
 		// fastest dim from 1 to 2*C - 1) scatters its non-zero elements over

@@ -516,6 +516,77 @@ def test_conv_boxed_skips_padding_and_unread_outputs(ctx, ops, oracle):
         assert (got[:, :, :, 0] == 12345).all() and (got[:, :, :, 2:] == 12345).all()
 
 
+def conv2d_idiom_cases(C, W, H, B, O, KW, KH):
+    """(image shape, kernel shape, ranks, image box, output window) of conv2d's
+    forward, image-gradient and kernel-gradient convolutions
+    (cfg/tenncor/nn.yml:48-98 and the CONV rules of tenncor/eteq/backprop.hpp)."""
+    OW, OH = W - KW + 1, H - KH + 1
+    one = [1, 1, 1]
+    fwd = ([C, W, H, B, 2 * O - 1] + one, [O, C, KW, KH], [4, 0, 1, 2],
+           ([0, 0, 0, 0, O - 1, 0, 0, 0], [C, W, H, B, O] + one), None)
+    # gradient of the padded image: supgrad {1,OW,OH,B,O} padded by K-1 on every kernel dim
+    gshape = [2 * C - 1, OW + 2 * (KW - 1), OH + 2 * (KH - 1), B, 3 * O - 2] + one
+    dgrad = (gshape, [O, C, KW, KH], [4, 0, 1, 2],
+             ([C - 1, KW - 1, KH - 1, 0, O - 1, 0, 0, 0], [C, KW - 1 + OW, KH - 1 + OH, B, 2 * O - 1] + one),
+             ([0, 0, 0, 0, O - 1, 0, 0, 0], [C, W, H, B, O] + one))
+    # gradient of the kernel: the padded image correlated with supgrad as the kernel
+    wgrad = ([C, W, H, B, 2 * O - 1] + one, [1, OW, OH, B, O], list(range(8)),
+             ([0, 0, 0, 0, O - 1, 0, 0, 0], [C, W, H, B, O] + one), None)
+    return {"forward": fwd, "image_gradient": dgrad, "kernel_gradient": wgrad}
+
+
+@pytest.mark.parametrize("which", ["forward", "image_gradient", "kernel_gradient"])
+def test_conv_as_matrix_product_equals_direct_kernels(ctx, oracle, which):
+    """The three convolutions of a conv2d layer at a size where tcg_conv_boxed
+    takes the matrix-product route (with a small row chunk, so that several
+    passes are made), against the direct kernels: equal bit for bit in int32
+    (both sum exact products, the skipped terms are zeros), 1e-4 in fp32."""
+    from tenncor_amd import capi
+    ishape, kshape, ranks, ibox, obox = conv2d_idiom_cases(C=12, W=15, H=13, B=12, O=24, KW=3, KH=4)[which]
+    rng = np.random.default_rng(seed_of("convgemm", which))
+    n_img, n_ker = oracle.n_elems(ishape), oracle.n_elems(kshape)
+    oshape = oracle.conv_shape(ishape, kshape, ranks)
+    n_out = oracle.n_elems(oshape)
+    lo, hi = ibox
+    # zero outside the box, as PAD leaves it... except where nothing may look
+    inside = np.ones(ishape[::-1], dtype=bool)
+    for d in range(8):
+        idx = np.arange(ishape[d])
+        keep = (idx >= lo[d]) & (idx < hi[d])
+        shape = [1] * 8
+        shape[7 - d] = ishape[d]
+        inside &= keep.reshape(shape)
+    inside = inside.reshape(-1)
+    for np_dtype in (np.int32, np.float32):
+        if np_dtype == np.int32:
+            img = rng.integers(-40, 41, n_img).astype(np.int32)
+            ker = rng.integers(-40, 41, n_ker).astype(np.int32)
+        else:
+            img = rng.uniform(-1, 1, n_img).astype(np.float32)
+            ker = rng.uniform(-1, 1, n_ker).astype(np.float32)
+        img[~inside] = 12345  # garbage outside the box must never be read
+        dt = capi.dtype_code(np_dtype)
+        dimg, dker = ctx.upload(img), ctx.upload(ker)
+        results = {}
+        for route, env in (("direct", {"TCG_CONV_GEMM": "0"}), ("product", {"TCG_CONV_GEMM": "1", "TCG_CONV_CHUNK_ROWS": "128"})):
+            os.environ.update(env)
+            try:
+                out = ctx.upload(np.full(n_out, 777, dtype=np_dtype))
+                ctx.conv_boxed(dt, ishape, kshape, ranks, ibox, obox, dimg.ptr, dker.ptr, out.ptr)
+                results[route] = out.get()
+            finally:
+                for key in env:
+                    os.environ.pop(key, None)
+        if np_dtype == np.int32:
+            np.testing.assert_array_equal(results["product"], results["direct"])
+        else:
+            assert_acc_close(results["product"], results["direct"])
+        if obox is not None:
+            # outside the window the destination keeps what it held
+            untouched = results["direct"] == 777
+            assert untouched.any() and (results["product"][untouched] == 777).all()
+
+
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
 def test_pad_interior_writes_the_operand_and_nothing_else(ctx, oracle, np_dtype):
     """tcg_pad_interior against PAD: equal to the oracle's padded tensor inside
