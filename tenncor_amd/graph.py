@@ -304,8 +304,22 @@ class Api:
     def square(self, x):
         return self.unary("SQUARE", x)
 
-    def identity(self, x):
-        return self.g.functor("IDENTITY", [x])
+    def identity(self, x, execute_in_parallel=()):
+        """core.yml:171-187: the value of `x`; further arguments are only
+        dependencies, evaluated along with it."""
+        return self.g.functor("IDENTITY", [x] + list(execute_in_parallel))
+
+    def sqrt(self, x):
+        return self.unary("SQRT", x)
+
+    def assign(self, target, source):
+        return self.g.functor("ASSIGN", [target, source])
+
+    def assign_add(self, target, source):
+        return self.g.functor("ASSIGN_ADD", [target, source])
+
+    def assign_sub(self, target, source):
+        return self.g.functor("ASSIGN_SUB", [target, source])
 
     def relu(self, x):
         """core.yml:1261-1267: max(arg, 0)."""
@@ -408,3 +422,87 @@ class Api:
             hidden = self.mul(state, output)
             states.append(hidden)
         return self.identity(self.concat(states, seq_dim))
+
+
+class Approx:
+    """The update rules of cfg/tenncor/approx.yml (ApproxAPI): for every
+    variable an assignment node that applies one optimisation step in place on
+    the device copy of the variable.  Each method returns [(variable, assign
+    node)], the reference's layr::VarErrsT."""
+
+    def __init__(self, api):
+        self.api = api
+        self.g = api.g
+
+    def _variable_like(self, scalar, like, label):
+        """eteq::make_variable_like (tenncor/eteq/make.hpp:185-200)."""
+        np_dtype = capi.NP_OF[like.dtype]
+        return self.g.variable(np.full(capi.n_elems(like.shape), scalar, np_dtype), like.shape, label)
+
+    def sgd(self, error, variables, learning_rate=0.5):
+        """approx.yml:12-52: x -= learning_rate * f'(x)."""
+        a = self.api
+        ders = self.g.derive(error, variables)
+        return [(x, a.assign_sub(x, a.mul(der, learning_rate))) for x, der in zip(variables, ders)]
+
+    def adagrad(self, error, variables, learning_rate=0.5, epsilon=float(np.finfo(np.float32).eps)):
+        """approx.yml:53-94: momentum += f'(x)^2; x -= lr f'(x) / (sqrt(momentum) + eps)."""
+        a = self.api
+        out = []
+        for x, der in zip(variables, self.g.derive(error, variables)):
+            momentum = self._variable_like(1, der, "momentum")
+            update = a.assign_add(momentum, a.square(der))
+            out.append((x, a.assign_sub(x, a.div(a.mul(der, learning_rate), a.add(a.sqrt(update), epsilon)))))
+        return out
+
+    def adam(self, error, variables, step_rate=0.001, decay1=0.9, decay2=0.999,
+             epsilon=float(np.finfo(np.float32).eps)):
+        """approx.yml:95-176."""
+        a = self.api
+        out = []
+        for x, der in zip(variables, self.g.derive(error, variables)):
+            m = self._variable_like(0, der, "moment1")
+            v = self._variable_like(0, der, "moment2")
+            t = self._variable_like(0, der, "t")
+            one_t = a._like(1, der)
+            next_m = a.assign(m, a.add(a.mul(decay1, m), a.mul(1.0 - decay1, der)))
+            next_v = a.assign(v, a.add(a.mul(decay2, v), a.mul(1.0 - decay2, a.square(der))))
+            incr = a.assign_add(t, one_t)
+            m_corr = a.div(next_m, a.sub(one_t, a.pow(decay1, incr)))
+            v_corr = a.div(next_v, a.sub(one_t, a.pow(decay2, incr)))
+            delta = a.mul(step_rate, a.div(m_corr, a.add(a.sqrt(v_corr), epsilon)))
+            out.append((x, a.assign_sub(x, delta)))
+        return out
+
+    def adadelta(self, error, variables, step_rate=1.0, decay=0.9, offset=0.0001,
+                 epsilon=float(np.finfo(np.float32).eps)):
+        """approx.yml:177-247."""
+        a = self.api
+        out = []
+        for x, der in zip(variables, self.g.derive(error, variables)):
+            msg = self._variable_like(0, der, "ex_sqr_grad")
+            msd = self._variable_like(0, der, "ex_sqr_delx")
+            msg_next = a.assign(msg, a.add(a.mul(decay, msg), a.mul(1.0 - decay, a.square(der))))
+            delta = a.mul(a.mul(step_rate, a.div(a.sqrt(a.add(msd, offset)),
+                                                 a.add(a.sqrt(a.add(msg_next, offset)), epsilon))), der)
+            msd_next = a.assign(msd, a.add(a.mul(decay, msd), a.mul(1.0 - decay, a.square(delta))))
+            out.append((x, a.assign_sub(x, a.identity(delta, [msd_next]))))
+        return out
+
+    def rms_momentum(self, error, variables, learning_rate=0.5, discount_factor=0.99,
+                     epsilon=float(np.finfo(np.float32).eps)):
+        """approx.yml:248-304."""
+        a = self.api
+        out = []
+        for x, der in zip(variables, self.g.derive(error, variables)):
+            momentum = self._variable_like(1, der, "momentum")
+            update = a.assign(momentum, a.add(a.mul(discount_factor, momentum),
+                                              a.mul(1.0 - discount_factor, a.square(der))))
+            out.append((x, a.assign_sub(x, a.div(a.mul(der, learning_rate), a.add(a.sqrt(update), epsilon)))))
+        return out
+
+    def apply_update(self, error, updates):
+        """tenncor/trainer/apply_update.hpp:13-41 without the re-trailing of the
+        error through the assignments: one node that yields the error (at the
+        weights the step started from) and depends on every assignment."""
+        return self.api.identity(error, [assign for _, assign in updates])

@@ -378,3 +378,82 @@ def test_padded_image_read_by_convolutions_and_by_others(g, api, oracle):
     np.testing.assert_array_equal(conv.get(), conv_ref)
     np.testing.assert_array_equal(pad.get(), padded_ref)
     np.testing.assert_array_equal(total.get(), [xv.sum()])
+
+
+# ---- optimiser steps on the device (cfg/tenncor/approx.yml) -------------------
+
+def numpy_optimisers(rule, w, grad_fn, steps, **kw):
+    """The update rules restated in numpy (fp64), one trajectory of `steps`."""
+    eps = float(np.finfo(np.float32).eps)
+    state = {}
+    traj = []
+    w = w.astype(np.float64).copy()
+    for _ in range(steps):
+        g = grad_fn(w)
+        if rule == "sgd":
+            w = w - kw.get("learning_rate", 0.5) * g
+        elif rule == "adagrad":
+            state["m"] = state.get("m", np.ones_like(w)) + g * g
+            w = w - kw.get("learning_rate", 0.5) * g / (np.sqrt(state["m"]) + eps)
+        elif rule == "rms_momentum":
+            d = kw.get("discount_factor", 0.99)
+            state["m"] = d * state.get("m", np.ones_like(w)) + (1 - d) * g * g
+            w = w - kw.get("learning_rate", 0.5) * g / (np.sqrt(state["m"]) + eps)
+        elif rule == "adam":
+            b1, b2, lr = kw.get("decay1", 0.9), kw.get("decay2", 0.999), kw.get("step_rate", 0.001)
+            state["m"] = b1 * state.get("m", np.zeros_like(w)) + (1 - b1) * g
+            state["v"] = b2 * state.get("v", np.zeros_like(w)) + (1 - b2) * g * g
+            state["t"] = state.get("t", 0) + 1
+            mc = state["m"] / (1 - b1 ** state["t"])
+            vc = state["v"] / (1 - b2 ** state["t"])
+            w = w - lr * mc / (np.sqrt(vc) + eps)
+        elif rule == "adadelta":
+            d, off, lr = kw.get("decay", 0.9), kw.get("offset", 0.0001), kw.get("step_rate", 1.0)
+            state["msg"] = d * state.get("msg", np.zeros_like(w)) + (1 - d) * g * g
+            delta = lr * np.sqrt(state.get("msd", np.zeros_like(w)) + off) / (np.sqrt(state["msg"] + off) + eps) * g
+            state["msd"] = d * state.get("msd", np.zeros_like(w)) + (1 - d) * delta * delta
+            w = w - delta
+        traj.append(w.copy())
+    return traj
+
+
+@pytest.mark.parametrize("evaluator", ["plain", "replay"])
+@pytest.mark.parametrize("rule,kw", [("sgd", {"learning_rate": 0.05}), ("adagrad", {"learning_rate": 0.1}),
+                                     ("rms_momentum", {"learning_rate": 0.01}), ("adam", {"step_rate": 0.01}),
+                                     ("adadelta", {})])
+def test_optimiser_steps_stay_on_the_device(rule, kw, evaluator):
+    """Five steps of every ApproxAPI rule on a least-squares problem: the
+    variable (and the rule's state variables) are updated in place by ASSIGN*
+    nodes; the host view of the weights after each step follows numpy's
+    trajectory of the same rule to fp32 accuracy."""
+    from tenncor_amd import graph
+    rng = np.random.default_rng(31)
+    xv = rng.uniform(-1, 1, (6, 4)).astype(np.float32)     # np[batch, in]
+    yv = rng.uniform(-1, 1, (6, 3)).astype(np.float32)
+    w0 = rng.uniform(-0.5, 0.5, (4, 3)).astype(np.float32)
+
+    def grad_fn(w):
+        r = xv.astype(np.float64) @ w - yv
+        return 2 * xv.astype(np.float64).T @ r
+
+    want = numpy_optimisers(rule, w0, grad_fn, 5, **kw)
+    graph.set_evaluator(evaluator)
+    g = graph.Graph()
+    try:
+        api = graph.Api(g)
+        x = g.variable(xv, [4, 6], "x")
+        y = g.variable(yv, [3, 6], "y")
+        w = g.variable(w0, [3, 4], "w")
+        err = api.reduce_sum(api.square(api.sub(api.matmul(x, w), y)))
+        updates = getattr(graph.Approx(api), rule)(err, [w], **kw)
+        step = graph.Approx(api).apply_update(err, updates)
+        for i in range(5):
+            g.evaluate([step])
+            np.testing.assert_allclose(w.get().reshape(4, 3), want[i], rtol=2e-4, atol=2e-6)
+        r = xv.astype(np.float64) @ want[3] - yv
+        np.testing.assert_allclose(step.get(), [np.sum(r * r)], rtol=1e-4)   # error at the weights the step began with
+        if evaluator == "replay":
+            assert graph.evaluator_stats()["replayed"] >= 3
+    finally:
+        g.close()
+        graph.set_evaluator("plain")
