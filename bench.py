@@ -99,7 +99,7 @@ class Step:
         ]
 
 
-def run_gpu(steps, warmup):
+def run_gpu(steps, warmup, graphs=True):
     from tenncor_amd import capi
     ctx = capi.Context(0)
     st = Step(ctx)
@@ -128,7 +128,8 @@ def run_gpu(steps, warmup):
     extra = run_extras(ctx, capi)
     arch = ctx.arch
     ctx.close()
-    extra.update(run_graph_configs())
+    if graphs:
+        extra.update(run_graph_configs())
     return wall, per_class, extra, arch
 
 
@@ -227,7 +228,7 @@ def run_extras(ctx, capi):
     return extra
 
 
-def run_graph_configs():
+def run_graph_configs(only=None, evaluator=None, reps=20):
     """configs[0], [3], [4] through the host graph layer (Functor nodes, the
     gradient builder, teq::Evaluator + eigen::Device): wall time of
     evaluate(targets) after re-assigning the input, which forces a full
@@ -250,10 +251,29 @@ def run_graph_configs():
             ts.append(time.perf_counter() - t0)
         return float(np.median(ts))
 
-    for kind, tag in (("plain", ""), ("replay", "_replay")):
+    kinds = (("plain", ""), ("replay", "_replay")) if evaluator is None else ((evaluator, ""),)
+    for kind, tag in kinds:
         # "replay": the evaluator that records a target set's launches on its
         # second pass and enqueues the recording afterwards
         tg.set_evaluator(kind)
+        if only is not None:
+            # one configuration under one evaluator (the form profiles are taken in)
+            g = tg.Graph()
+            if only == 1:
+                targets, x, _ = configs.config1_mlp(g)
+                t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
+            elif only == 4:
+                targets, x, _, flops = configs.config4_lstm(g)
+                xs = rng.uniform(-1, 1, 256 * 64 * 256).astype(np.float32)
+                t = timed(g, targets, x, lambda: xs, reps)
+            else:
+                targets, x, _, flops = configs.config5_cnn(g)
+                xs = rng.uniform(0, 1, 128 * 28 * 28).astype(np.float32)
+                t = timed(g, targets, x, lambda: xs, reps)
+            out = {"graph_config": only, "evaluator": kind, "ms_per_eval": round(t * 1e3, 4),
+                   "functors": g.count_functors(targets), "evaluator_stats": tg.evaluator_stats()}
+            tg.set_evaluator("plain")
+            return out
         g = tg.Graph()
         targets, x, _ = configs.config1_mlp(g)
         t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
@@ -330,12 +350,20 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graphs", action="store_true", help="skip the whole-graph side metrics (configs 1, 4, 5)")
+    ap.add_argument("--graph-config", type=int, choices=[1, 4, 5], default=None,
+                    help="time only this whole-graph configuration and print its line (for profiling)")
+    ap.add_argument("--evaluator", choices=["plain", "replay", "replay_unfused"], default="replay")
+    ap.add_argument("--reps", type=int, default=20, help="timed evaluations with --graph-config 4 or 5")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU; --gpus %d is not supported "
                  "(no collectives or sharding are part of this build)" % args.gpus)
 
-    wall, per_class, extra, arch = run_gpu(args.steps, args.warmup)
+    if args.graph_config is not None:
+        print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps)))
+        return
+    wall, per_class, extra, arch = run_gpu(args.steps, args.warmup, graphs=not args.no_graphs)
     abytes = algorithmic_bytes()
     launches_per_step = {"ew_binary_f32": 2, "ew_unary_f32": 3, "reduce_dim0_f32": 2, "reduce_dim1_f32": 2,
                          "ew_binary_i32": 2, "reduce_dim0_i32": 2, "reduce_dim1_i32": 2}
