@@ -87,6 +87,13 @@ int tcr_args (tcr_graph* g, int node, int* args, int capacity);
 int tcr_to_string (tcr_graph* g, int node, char* out, size_t capacity);
 /* Number of distinct functors reachable from the given nodes */
 int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count);
+/* How the replaying evaluator would launch one pass over these targets, as
+ * text, one launch per line in launch order (needs no GPU): "node OPCODE" for
+ * a functor launched through its own operator, or
+ * "group OP+OP+... leaves=L stores=S instrs=I" for elementwise functors sharing
+ * a launch; a last line "folded N" counts the functors that never hold a value
+ * of their own. Returns the length the text needs (it is cut to `capacity`). */
+int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, size_t capacity, size_t* needed);
 
 #ifdef __cplusplus
 }

@@ -27,7 +27,7 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
-    "tcr_set_evaluator", "tcr_evaluator_stats",
+    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan",
 ]
 
 EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED = 0, 1, 2
@@ -71,6 +71,7 @@ def load():
         "tcr_count_functors": [vp, i32, i32p, i32p],
         "tcr_set_evaluator": [i32],
         "tcr_evaluator_stats": [u64p],
+        "tcr_launch_plan": [vp, i32, i32p, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -239,6 +240,17 @@ class Graph:
         buf = ctypes.create_string_buffer(1 << 20)
         self._check(self.lib.tcr_to_string(self.h, node.id, buf, len(buf)))
         return buf.value.decode()
+
+    def launch_plan(self, targets):
+        """The launches one recorded pass over `targets` would consist of: a list
+        of lines, "node OP" or "group OP+OP... leaves=L stores=S instrs=I", and a
+        final "folded N".  Pure host logic: works without a GPU."""
+        ids = _ints([t.id for t in targets])
+        need = ctypes.c_size_t()
+        self._check(self.lib.tcr_launch_plan(self.h, len(targets), ids, None, 0, ctypes.byref(need)))
+        buf = ctypes.create_string_buffer(need.value + 1)
+        self._check(self.lib.tcr_launch_plan(self.h, len(targets), ids, buf, need.value + 1, ctypes.byref(need)))
+        return buf.value.decode().splitlines()
 
     def count_functors(self, nodes):
         c = ctypes.c_int()

@@ -49,6 +49,11 @@ struct Node final
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
 	teq::TensptrsT arg_tens;
 	std::vector<int> consumers; // functors of this pass reading the node
+	// args with folded single-operand IDENTITY nodes looked through (an alias
+	// of an elementwise node must not keep that node out of its reader's
+	// group), and the aliases skipped on the way
+	std::vector<int> direct;
+	std::vector<std::vector<int>> aliases;
 	Shape8 shape;
 };
 
@@ -131,6 +136,20 @@ struct Planner final
 				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed);
 			});
 		}
+		for (Node& n : nodes_)
+		{
+			for (int a : n.args)
+			{
+				std::vector<int> skipped;
+				while (a >= 0 && is_alias(a))
+				{
+					skipped.push_back(a);
+					a = nodes_[a].args[0];
+				}
+				n.direct.push_back(a);
+				n.aliases.push_back(skipped);
+			}
+		}
 		uf_.resize(nodes_.size());
 		for (size_t i = 0; i < uf_.size(); ++i) { uf_[i] = (int) i; }
 		minpos_.resize(nodes_.size());
@@ -138,6 +157,33 @@ struct Planner final
 		members_.resize(nodes_.size());
 		deps_.resize(nodes_.size());
 		stamp_.assign(nodes_.size(), 0);
+	}
+
+	bool is_alias (int i) const
+	{
+		const Node& n = nodes_[i];
+		return n.kind == VIEW && n.absorbed && n.op == egen::IDENTITY;
+	}
+
+	/// Does anything other than the launch described by `inside` read node i?
+	template <typename F>
+	bool read_elsewhere (int i, F inside) const
+	{
+		for (int c : nodes_[i].consumers)
+		{
+			if (is_alias(c) ? read_elsewhere(c, inside) : false == inside(c)) { return true; }
+		}
+		return false;
+	}
+
+	template <typename F>
+	bool read_by (int i, F inside) const
+	{
+		for (int c : nodes_[i].consumers)
+		{
+			if (is_alias(c) ? read_by(c, inside) : inside(c)) { return true; }
+		}
+		return false;
 	}
 
 	Kind classify (const Node& n) const
@@ -319,7 +365,7 @@ struct Planner final
 			if (n.kind != EW) { continue; }
 			members_[i].push_back((int) i);
 			std::vector<int> cands;
-			for (int a : n.args)
+			for (int a : n.direct)
 			{
 				if (a >= 0 && nodes_[a].kind == EW) { cands.push_back(find(a)); }
 			}
@@ -390,12 +436,11 @@ struct Planner final
 		for (size_t p = lo; p < hi; ++p)
 		{
 			const Node& n = nodes_[members[p]];
-			for (int a : n.args)
+			for (int a : n.direct)
 			{
 				if (inside(a)) { last_use[pos[a]] = p - lo; }
 			}
-			stored[p - lo] = n.target || std::any_of(n.consumers.begin(), n.consumers.end(),
-				[&](int c) { return false == inside(c); });
+			stored[p - lo] = n.target || read_elsewhere(members[p], inside);
 		}
 		std::map<View,int> leaf_of;
 		std::vector<int> reg_of(hi - lo, -1);
@@ -422,11 +467,12 @@ struct Planner final
 			std::vector<double> vals;
 			for (size_t k = 0; k < n.args.size(); ++k)
 			{
-				int a = n.args[k];
+				int a = n.direct[k];
 				if (inside(a))
 				{
 					codes.push_back((uint8_t) (TCG_FX_REG0 + reg_of[pos[a]]));
 					vals.push_back(0);
+					views.insert(views.end(), n.aliases[k].begin(), n.aliases[k].end());
 					continue;
 				}
 				View v = view_of_arg(members[p], k, &views);
@@ -473,7 +519,7 @@ struct Planner final
 			// dies here; a fold keeps its accumulator apart from its operands
 			auto release_dead = [&]()
 			{
-				for (int a : n.args)
+				for (int a : n.direct)
 				{
 					if (inside(a) && last_use[pos[a]] == here) { busy[reg_of[pos[a]]] = false; }
 				}
@@ -524,7 +570,7 @@ struct Planner final
 				out.program.push_back(st);
 				out.outputs.push_back(n.f);
 			}
-			if (false == std::any_of(n.consumers.begin(), n.consumers.end(), inside))
+			if (false == read_by(members[p], inside))
 			{
 				busy[dst] = false; // nothing in this launch reads it
 			}

@@ -1,10 +1,13 @@
 // Flat C binding of the host graph layer (include/tcgraph.h).
 #include "tcgraph.h"
 
+#include <algorithm>
+#include <cstring>
 #include <sstream>
 
 #include "eteq.hpp"
 #include "replay_eval.hpp"
+#include "fuse_plan.hpp"
 
 struct tcr_graph
 {
@@ -322,6 +325,57 @@ int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count)
 		} counter;
 		for (int i = 0; i < nnodes; ++i) { g->at(nodes[i])->accept(counter); }
 		*count = (int) counter.nfuncs;
+	});
+}
+
+int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, size_t capacity, size_t* needed)
+{
+	return guarded([&]
+	{
+		struct Collector final : public teq::iOnceTraveler
+		{
+			std::vector<eigen::Observable*> funcs;
+			void visit_leaf (teq::iLeaf&) override {}
+			void visit_func (teq::iFunctor& f) override
+			{
+				auto args = f.get_args();
+				teq::multi_visit(*this, args);
+				funcs.push_back(static_cast<eigen::Observable*>(&f));
+			}
+		} collector;
+		teq::TensSetT tset;
+		std::vector<teq::iTensor*> key;
+		for (int i = 0; i < ntargets; ++i) { key.push_back(g->at(targets[i]).get()); }
+		tset.insert(key.begin(), key.end());
+		std::sort(key.begin(), key.end());
+		teq::multi_visit(collector, key);
+		eigen::FusionPlan plan = eigen::plan_fusion(collector.funcs, tset);
+		std::stringstream ss;
+		for (auto& step : plan.steps)
+		{
+			if (nullptr != step.node)
+			{
+				ss << "node " << step.node->get_opcode().name_ << "\n";
+				continue;
+			}
+			auto& group = plan.groups[step.group];
+			ss << "group ";
+			for (size_t i = 0; i < group.members.size(); ++i)
+			{
+				ss << (i ? "+" : "") << group.members[i]->get_opcode().name_;
+			}
+			ss << " leaves=" << group.leaves.size() << " stores=" << group.outputs.size()
+				<< " instrs=" << group.program.size() << "\n";
+		}
+		ss << "folded " << plan.absorbed.size() << "\n";
+		std::string text = ss.str();
+		if (needed) { *needed = text.size(); }
+		if (out && capacity)
+		{
+			size_t n = std::min(text.size(), capacity - 1);
+			memcpy(out, text.data(), n);
+			out[n] = '\0';
+		}
 	});
 }
 

@@ -258,3 +258,88 @@ def test_mlp_gradient_graph_only_uses_table_opcodes(g, api):
         stack.extend(g.args(n))
     assert ops <= {"BAD_OP", "MUL", "SUB", "EXTEND", "SIGMOID", "ADD", "MATMUL", "PERMUTE", "REDUCE_SUM", "SQUARE"}
     assert grads[0].shape[:2] == [9, 10] and grads[1].shape[:2] == [9, 1]
+
+
+# ---- launch planning of the replaying evaluator (host logic only) -------------
+
+def parse_plan(lines):
+    steps = []
+    for line in lines:
+        kind, _, rest = line.partition(" ")
+        if kind == "node":
+            steps.append(("node", [rest], {}))
+        elif kind == "group":
+            ops, *fields = rest.split(" ")
+            steps.append(("group", ops.split("+"), {k: int(v) for k, v in (f.split("=") for f in fields)}))
+        else:
+            steps.append(("folded", [], {"n": int(rest)}))
+    return steps
+
+
+def test_launch_plan_groups_the_elementwise_nodes_of_an_mlp(g):
+    from tenncor_amd import configs
+    targets, _, _ = configs.config1_mlp(g)
+    steps = parse_plan(g.launch_plan(targets))
+    launches = [s for s in steps if s[0] != "folded"]
+    folded = steps[-1][2]["n"]
+    nfunc = g.count_functors(targets)
+    # every functor is launched on its own, computed inside a group, or folded into operand views
+    in_groups = sum(len(s[1]) for s in launches if s[0] == "group")
+    stores = sum(s[2]["stores"] for s in launches if s[0] == "group")
+    alone = sum(1 for s in launches if s[0] == "node")
+    assert alone + stores + folded == nfunc
+    assert len(launches) < nfunc // 2
+    assert any(s[0] == "group" and "SIGMOID" in s[1] and len(s[1]) >= 3 for s in launches)
+    # the matrix products and reductions keep their own kernels
+    assert sum(1 for s in launches if s[0] == "node" and s[1][0] in ("CONTRACT", "MATMUL")) == 5
+    for s in launches:
+        if s[0] == "group":
+            assert s[2]["leaves"] <= 8 and s[2]["stores"] <= 8 and s[2]["instrs"] <= 64
+
+
+def test_launch_plan_keeps_a_launch_between_two_groups_in_order(g, api):
+    """t feeds a matmul whose result comes back into elementwise nodes that also
+    read t: the two elementwise parts cannot share a launch."""
+    x = var(g, [6, 4], np.float32, "x")
+    w = var(g, [6, 6], np.float32, "w")
+    s = api.add(x, 1.0)
+    t = api.mul(api.square(s), api.neg(s))
+    m = api.matmul(t, w)
+    u = api.sub(api.add(t, m), api.mul(s, 2.0))
+    steps = [st for st in parse_plan(g.launch_plan([u])) if st[0] != "folded"]
+    kinds = [(k, ops) for k, ops, _ in steps]
+    mm = next(i for i, (k, ops) in enumerate(kinds) if k == "node" and ops == ["MATMUL"])
+    before = [ops for k, ops in kinds[:mm] if k == "group"]
+    after = [ops for k, ops in kinds[mm + 1:] if k == "group"]
+    assert any("SQUARE" in ops and "NEG" in ops for ops in before)
+    assert any("SUB" in ops for ops in after)
+    assert all("SUB" not in ops for ops in before)
+    # s and t are read on both sides of the product: both are stored by the first group
+    first = next(st for st in steps if st[0] == "group")
+    assert first[2]["stores"] == 2
+
+
+def test_launch_plan_folds_views_and_splits_oversized_groups(g, api):
+    x = var(g, [8, 4], np.float32, "x")
+    b = var(g, [8], np.float32, "b")
+    wide = var(g, [16, 4], np.float32, "wide")
+    # EXTEND, SLICE and PAD in front of elementwise nodes never get a launch
+    y = api.add(api.mul(x, api.extend(b, 1, [4])), api.slice(wide, 4, 8, 0))
+    z = api.add(api.pad(api.slice(y, 1, 6, 0), [[1, 1]]), x)
+    lines = g.launch_plan([z])
+    assert all(not l.startswith("node") for l in lines[:-1]), lines
+    assert parse_plan(lines)[-1][2]["n"] >= 4
+    # ... but a view read by a matrix product is materialised
+    m = api.matmul(api.slice(wide, 4, 8, 0), var(g, [3, 8], np.float32, "w"))
+    assert "node SLICE" in g.launch_plan([m])
+    # a chain longer than one launch's program is cut into several launches
+    deep = x
+    for k in range(150):
+        deep = api.add(api.mul(deep, x), float(k + 1))
+    steps = [s for s in parse_plan(g.launch_plan([deep])) if s[0] == "group"]
+    assert len(steps) >= 5 and sum(len(s[1]) for s in steps) == 300
+    assert all(s[2]["instrs"] <= 64 for s in steps)
+    # ten results of one group: more than one launch stores
+    outs = [api.mul(z, float(k + 2)) for k in range(10)]
+    steps = [s for s in parse_plan(g.launch_plan(outs)) if s[0] == "group"]
+    assert sum(s[2]["stores"] for s in steps) >= 10 and all(s[2]["stores"] <= 8 for s in steps)
