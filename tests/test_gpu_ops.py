@@ -312,6 +312,9 @@ def movement_cases(oracle, ops, rng):
     add("permute_rot", [20, 30, 40], lambda t: ops.permute(t, [2, 0, 1]), lambda x, s: oracle.permute(x, s, [2, 0, 1]))
     add("permute_inner_kept", [64, 5, 7, 3], lambda t: ops.permute(t, [0, 2, 1, 3]), lambda x, s: oracle.permute(x, s, [0, 2, 1, 3]))
     add("permute_conv2d", [1, 20, 18, 6, 32], lambda t: ops.permute(t, [4, 1, 2, 3]), lambda x, s: oracle.permute(x, s, [4, 1, 2, 3]))
+    add("permute_wide_tiles", [132, 68, 3], lambda t: ops.permute(t, [1, 0, 2]), lambda x, s: oracle.permute(x, s, [1, 0, 2]))
+    add("permute_wide_batched", [64, 6, 128], lambda t: ops.permute(t, [2, 1, 0]), lambda x, s: oracle.permute(x, s, [2, 1, 0]))
+    add("permute_narrow_odd", [66, 35], lambda t: ops.permute(t, [1, 0]), lambda x, s: oracle.permute(x, s, [1, 0]))
     add("permute_small", [3, 4, 5], lambda t: ops.permute(t, [2, 1, 0]), lambda x, s: oracle.permute(x, s, [2, 1, 0]))
     add("extend_bias", [9, 1], lambda t: ops.extend(t, [1, 300]), lambda x, s: oracle.extend(x, s, [1, 300]))
     add("extend_scalar", [1], lambda t: ops.extend(t, [32, 24, 24, 8]), lambda x, s: oracle.extend(x, s, [32, 24, 24, 8]))
