@@ -560,13 +560,13 @@ def test_conv_as_matrix_product_equals_direct_kernels(ctx, oracle, which):
         shape[7 - d] = ishape[d]
         inside &= keep.reshape(shape)
     inside = inside.reshape(-1)
-    for np_dtype in (np.int32, np.float32):
+    for np_dtype in (np.int32, np.float32, np.float64):
         if np_dtype == np.int32:
             img = rng.integers(-40, 41, n_img).astype(np.int32)
             ker = rng.integers(-40, 41, n_ker).astype(np.int32)
         else:
-            img = rng.uniform(-1, 1, n_img).astype(np.float32)
-            ker = rng.uniform(-1, 1, n_ker).astype(np.float32)
+            img = rng.uniform(-1, 1, n_img).astype(np_dtype)
+            ker = rng.uniform(-1, 1, n_ker).astype(np_dtype)
         img[~inside] = 12345  # garbage outside the box must never be read
         dt = capi.dtype_code(np_dtype)
         dimg, dker = ctx.upload(img), ctx.upload(ker)
@@ -583,7 +583,7 @@ def test_conv_as_matrix_product_equals_direct_kernels(ctx, oracle, which):
         if np_dtype == np.int32:
             np.testing.assert_array_equal(results["product"], results["direct"])
         else:
-            assert_acc_close(results["product"], results["direct"])
+            assert_acc_close(results["product"], results["direct"], ACC_RTOL if np_dtype == np.float32 else 1e-12)
         if obox is not None:
             # outside the window the destination keeps what it held
             untouched = results["direct"] == 777
@@ -770,3 +770,20 @@ def test_fused_group_rejects_malformed_programs(ctx):
     for prog in bad:
         with pytest.raises(capi.TcgError):
             ctx.ew_fusedx(capi.FLOAT, [16], [{"ptr": x.ptr}], prog, [out.ptr])
+
+
+def test_interpreted_groups_match_too():
+    """TCG_FX_JIT=0 sends fused groups to the interpreting kernel instead of a
+    kernel compiled for the program; the switch is read once per process, so the
+    group tests and the LSTM replay test are run again in a child process."""
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    env = dict(os.environ, TCG_FX_JIT="0")
+    cmd = [sys.executable, "-m", "pytest", "-x", "-q", "-p", "no:cacheprovider",
+           os.path.join(here, "test_gpu_ops.py"), os.path.join(here, "test_gpu_replay.py"),
+           "-k", "fused_group_with_views or fused_lstm or fused_views"]
+    done = subprocess.run(cmd, env=env, cwd=os.path.dirname(here), stdout=subprocess.PIPE, stderr=subprocess.STDOUT,
+                          text=True, timeout=300)
+    assert done.returncode == 0, done.stdout[-3000:]
+    assert " passed" in done.stdout
