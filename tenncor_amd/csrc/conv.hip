@@ -443,7 +443,7 @@ bool conv_gemm_plan (const ConvPlan& c, ConvGemmPlan& g)
 		N *= g.nsize[d];
 		S *= g.ssize[d];
 	}
-	if (N < 8 || S < 8 || M < 32 || M >= (1ull << 31) || N >= (1ull << 31) || S >= (1ull << 31)) { return false; }
+	if (N < 8 || S < 8 || M < 8 || M >= (1ull << 31) || N >= (1ull << 31) || S >= (1ull << 31)) { return false; }
 	if (M * N * S < (1ull << 22)) { return false; }
 	g.M = (uint32_t) M;
 	g.N = (uint32_t) N;

@@ -301,7 +301,8 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	*handled = false;
 	// 128-bit operand loads: every row start and every slab offset must be
 	// 16-byte aligned; anything else goes to the generic kernel
-	bool ok = M >= 32 && N >= 32 && K >= 8 &&
+	// (a sliver of a tile still pays when K is long: the K ranges spread it over the chip)
+	bool ok = M >= 8 && N >= 8 && K >= 8 && ((M >= 32 && N >= 32) || K >= 512) &&
 		M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31) &&
 		tcg_aligned16(A) && tcg_aligned16(B) &&
 		lda % 4 == 0 && ldb % 4 == 0 && stride_a % 4 == 0 && stride_b % 4 == 0 &&

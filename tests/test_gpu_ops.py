@@ -398,6 +398,7 @@ GEMM_CASES = [
     (512, 384, 200, 1, 0, 0), (2048, 256, 768, 1, 1, 0), (768, 2048, 256, 1, 0, 1),
     # few tiles, long K: several workgroups share a tile (K split in ranges, last one ragged)
     (256, 768, 2048, 1, 0, 1), (256, 2048, 768, 1, 0, 0), (64, 96, 1000, 2, 1, 0), (36, 44, 4100, 1, 0, 0),
+    (12, 32, 2048, 1, 0, 0), (24, 8, 1024, 1, 1, 0), (8, 20, 600, 3, 0, 1),
     # off the matrix-core path: odd extents
     (33, 35, 17, 2, 0, 0), (33, 35, 17, 2, 1, 1),
 ]
