@@ -208,7 +208,7 @@ enum tcg_fx_operand
 	TCG_FX_LEAF0 = 8,  /* + k, k < TCG_FX_MAX_LEAVES */
 	TCG_FX_REG0 = 32   /* + r, r < TCG_FX_MAX_REGS */
 };
-#define TCG_FX_MAX_LEAVES 8
+#define TCG_FX_MAX_LEAVES 16
 #define TCG_FX_MAX_REGS 16
 #define TCG_FX_MAX_INSTRS 64
 #define TCG_FX_MAX_OUTS 8

@@ -30,6 +30,8 @@ constexpr int FX_SLOTS = TCG_FX_MAX_LEAVES + TCG_FX_MAX_REGS;
 #include "ew_fusedx_args.inc"
 #undef TCG_CORE
 
+static_assert(sizeof(FxArgs) <= 4096, "launch arguments must fit the kernel argument segment");
+
 FxDiv fx_make_div (uint32_t d)
 {
 	FxDiv f = {1, 0, 0, 0};
@@ -46,7 +48,7 @@ FxDiv fx_make_div (uint32_t d)
 // ever indexed by constants, so it lives in VGPRs; the slot an instruction
 // names is wave-uniform, so picking it is a scalar branch, not a memory access
 // (an array indexed by the slot number would be placed in scratch memory).
-static_assert(FX_SLOTS == 24, "fx_get / fx_put enumerate the slots");
+static_assert(FX_SLOTS == 32, "fx_get / fx_put enumerate the slots");
 
 // ends every case of the slot switches: without it the optimiser merges the
 // cases into one access through a selected address, which forces the file
@@ -90,6 +92,14 @@ __device__ __forceinline__ void fx_get (const T (&file)[FX_SLOTS][N], int s, T (
 		case 21: FX_EACH(v[e_] = file[21][e_]) FX_KEEP_APART; break;
 		case 22: FX_EACH(v[e_] = file[22][e_]) FX_KEEP_APART; break;
 		case 23: FX_EACH(v[e_] = file[23][e_]) FX_KEEP_APART; break;
+		case 24: FX_EACH(v[e_] = file[24][e_]) FX_KEEP_APART; break;
+		case 25: FX_EACH(v[e_] = file[25][e_]) FX_KEEP_APART; break;
+		case 26: FX_EACH(v[e_] = file[26][e_]) FX_KEEP_APART; break;
+		case 27: FX_EACH(v[e_] = file[27][e_]) FX_KEEP_APART; break;
+		case 28: FX_EACH(v[e_] = file[28][e_]) FX_KEEP_APART; break;
+		case 29: FX_EACH(v[e_] = file[29][e_]) FX_KEEP_APART; break;
+		case 30: FX_EACH(v[e_] = file[30][e_]) FX_KEEP_APART; break;
+		case 31: FX_EACH(v[e_] = file[31][e_]) FX_KEEP_APART; break;
 		default: break;
 	}
 }
@@ -123,6 +133,14 @@ __device__ __forceinline__ void fx_put (T (&file)[FX_SLOTS][N], int s, const T (
 		case 21: FX_EACH(file[21][e_] = v[e_]) FX_KEEP_APART; break;
 		case 22: FX_EACH(file[22][e_] = v[e_]) FX_KEEP_APART; break;
 		case 23: FX_EACH(file[23][e_] = v[e_]) FX_KEEP_APART; break;
+		case 24: FX_EACH(file[24][e_] = v[e_]) FX_KEEP_APART; break;
+		case 25: FX_EACH(file[25][e_] = v[e_]) FX_KEEP_APART; break;
+		case 26: FX_EACH(file[26][e_] = v[e_]) FX_KEEP_APART; break;
+		case 27: FX_EACH(file[27][e_] = v[e_]) FX_KEEP_APART; break;
+		case 28: FX_EACH(file[28][e_] = v[e_]) FX_KEEP_APART; break;
+		case 29: FX_EACH(file[29][e_] = v[e_]) FX_KEEP_APART; break;
+		case 30: FX_EACH(file[30][e_] = v[e_]) FX_KEEP_APART; break;
+		case 31: FX_EACH(file[31][e_] = v[e_]) FX_KEEP_APART; break;
 		default: break;
 	}
 }
