@@ -213,6 +213,10 @@ enum tcg_fx_operand
 #define TCG_FX_MAX_INSTRS 64
 #define TCG_FX_MAX_OUTS 8
 #define TCG_FX_STORE 255 /* opcode */
+/* opcode: bitwise OR of the two operands' representations. Zero-bordered
+ * leaves whose boxes tile the output, OR-ed together, are CONCAT
+ * (internal/eigen/operator.hpp:335-368) with every bit kept. */
+#define TCG_FX_BITOR 254
 typedef struct tcg_fx_leaf
 {
 	const void* ptr;
@@ -223,7 +227,7 @@ typedef struct tcg_fx_leaf
 } tcg_fx_leaf;
 typedef struct tcg_fx_instr
 {
-	uint8_t opcode; /* tcg_opcode (unary, binary, TCG_IDENTITY, TCG_SELECT) or TCG_FX_STORE */
+	uint8_t opcode; /* tcg_opcode (unary, binary, TCG_IDENTITY, TCG_SELECT), TCG_FX_BITOR or TCG_FX_STORE */
 	uint8_t a, b, c; /* tcg_fx_operand; unused ones TCG_FX_NONE */
 	uint8_t dst;    /* TCG_FX_REG0 + r, or the output index of a store */
 	uint8_t pad_[3];

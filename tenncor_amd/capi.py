@@ -63,7 +63,7 @@ class FxInstr(ctypes.Structure):
                 ("dst", ctypes.c_uint8), ("pad_", ctypes.c_uint8 * 3), ("imm", ctypes.c_double)]
 
 
-FX_NONE, FX_IMM, FX_LEAF0, FX_REG0, FX_STORE = 0, 1, 8, 32, 255
+FX_NONE, FX_IMM, FX_LEAF0, FX_REG0, FX_STORE, FX_BITOR = 0, 1, 8, 32, 255, 254
 
 _lib = None
 
@@ -319,7 +319,7 @@ class Context:
                 lv[k].hi[d] = int(leaf.get("hi", shp)[d])
         instrs = (FxInstr * len(program))()
         for i, ins in enumerate(program):
-            instrs[i].opcode = FX_STORE if ins[0] == "STORE" else _opcode(ins[0])
+            instrs[i].opcode = {"STORE": FX_STORE, "BITOR": FX_BITOR}.get(ins[0]) or _opcode(ins[0])
             instrs[i].a, instrs[i].b, instrs[i].c, instrs[i].dst = ins[1], ins[2], ins[3], ins[4]
             instrs[i].imm = float(ins[5]) if len(ins) > 5 else 0.0
         ptrs = (ctypes.c_void_p * len(outs))(*outs)

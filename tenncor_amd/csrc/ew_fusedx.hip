@@ -269,7 +269,10 @@ __global__ __launch_bounds__(FX_BLOCK) void ew_fusedx_k (FxArgs p)
 			else if (has_b)
 			{
 #pragma unroll
-				for (int e = 0; e < N; ++e) { vr[e] = apply_binary<T>(ins.opcode, va[e], vb[e]); }
+				for (int e = 0; e < N; ++e)
+				{
+					vr[e] = ins.opcode == TCG_FX_BITOR ? bit_or<T>(va[e], vb[e]) : apply_binary<T>(ins.opcode, va[e], vb[e]);
+				}
 			}
 			else
 			{
@@ -472,6 +475,10 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
 			{
 				o << operand(ins.a, i, e) << " != (T) 0 ? " << operand(ins.b, i, e) << " : " << operand(ins.c, i, e);
 			}
+			else if (ins.opcode == TCG_FX_BITOR)
+			{
+				o << "bit_or<T>(" << operand(ins.a, i, e) << ", " << operand(ins.b, i, e) << ")";
+			}
 			else if (ins.b != TCG_FX_NONE)
 			{
 				o << "apply_binary<T>(" << (int) ins.opcode << ", " << operand(ins.a, i, e) << ", " << operand(ins.b, i, e) << ")";
@@ -612,7 +619,7 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		else
 		{
 			bool unary = ins.opcode == TCG_IDENTITY || is_unary_op(ins.opcode);
-			bool binary = is_binary_op(ins.opcode);
+			bool binary = is_binary_op(ins.opcode) || ins.opcode == TCG_FX_BITOR;
 			bool select = ins.opcode == TCG_SELECT;
 			TCG_REQUIRE(ctx, unary || binary || select, "tcg_ew_fusedx: instruction %d has opcode %d", i, (int) ins.opcode);
 			TCG_REQUIRE(ctx, (unary && ins.b == TCG_FX_NONE && ins.c == TCG_FX_NONE) ||

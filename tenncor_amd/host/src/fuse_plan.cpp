@@ -192,6 +192,17 @@ struct Planner final
 		bool ew = (is_unary(n.op) && nargs == 1) ||
 			(is_binary(n.op) && (nargs == 2 || ((n.op == egen::ADD || n.op == egen::MUL) && nargs > 2))) ||
 			(n.op == egen::SELECT && nargs == 3);
+		if (n.op == egen::CONCAT)
+		{
+			// every element comes from exactly one operand: the operands become
+			// zero-bordered leaves whose boxes tile the output, OR-ed together
+			if (nargs < 2 || nargs > TCG_FX_MAX_LEAVES) { return OTHER; }
+			for (auto& arg : n.arg_tens)
+			{
+				if ((int) arg->get_meta().type_code() != n.dtype) { return OTHER; }
+			}
+			return EW;
+		}
 		if (ew)
 		{
 			if (nargs > TCG_FX_MAX_LEAVES) { return OTHER; }
@@ -367,7 +378,10 @@ struct Planner final
 			std::vector<int> cands;
 			for (int a : n.direct)
 			{
-				if (a >= 0 && nodes_[a].kind == EW) { cands.push_back(find(a)); }
+				if (a >= 0 && nodes_[a].kind == EW && nodes_[a].shape == n.shape && n.op != egen::CONCAT)
+				{
+					cands.push_back(find(a));
+				}
 			}
 			std::sort(cands.begin(), cands.end(), [&](int x, int y) { return maxpos_[x] > maxpos_[y]; });
 			cands.erase(std::unique(cands.begin(), cands.end()), cands.end());
@@ -463,12 +477,16 @@ struct Planner final
 			size_t here = p - lo;
 			// operands: a register of this launch, an immediate or a leaf
 			bool fold = n.args.size() > 2 && n.op != egen::SELECT;
+			const bool concat = n.op == egen::CONCAT;
+			teq::RankT axis = 0;
+			uint64_t before = 0; // extent of the operands already placed along `axis`
+			if (concat) { Packer<teq::RankT>().unpack(axis, *n.f); }
 			std::vector<uint8_t> codes;
 			std::vector<double> vals;
 			for (size_t k = 0; k < n.args.size(); ++k)
 			{
 				int a = n.direct[k];
-				if (inside(a))
+				if (false == concat && inside(a))
 				{
 					codes.push_back((uint8_t) (TCG_FX_REG0 + reg_of[pos[a]]));
 					vals.push_back(0);
@@ -476,8 +494,18 @@ struct Planner final
 					continue;
 				}
 				View v = view_of_arg(members[p], k, &views);
+				if (concat)
+				{
+					// operand k occupies [before, before + extent) of the axis
+					// and reads as zero elsewhere, like a PAD of it would
+					uint64_t extent = shape8(n.arg_tens[k]->shape())[axis];
+					v.off -= (int64_t) before * v.stride[axis];
+					v.lo[axis] += before;
+					v.hi[axis] += before;
+					before += extent;
+				}
 				double value;
-				if (scalar_constant(v.base, value))
+				if (false == concat && scalar_constant(v.base, value))
 				{
 					// an instruction carries one immediate: operands sharing an
 					// instruction (all of them unless the node is an n-ary fold,
@@ -531,7 +559,7 @@ struct Planner final
 			tcg_fx_instr ins;
 			memset(&ins, 0, sizeof(ins));
 			ins.dst = (uint8_t) (TCG_FX_REG0 + dst);
-			ins.opcode = (uint8_t) n.op;
+			ins.opcode = (uint8_t) (concat ? TCG_FX_BITOR : n.op);
 			if (fold)
 			{
 				// ((a0 op a1) op a2) ... like the n-ary kernel
@@ -629,7 +657,8 @@ struct Planner final
 					++hi;
 				}
 				FusionPlan::Step step;
-				if (hi == lo + 1 && views.empty() && false == uses_immediate(group))
+				if (hi == lo + 1 && views.empty() && false == uses_immediate(group) &&
+					nodes_[members[lo]].op != egen::CONCAT)
 				{
 					step.node = nodes_[members[lo]].f; // nothing to gain: its own kernel
 				}

@@ -406,3 +406,37 @@ def test_fused_views_diamonds_and_wide_groups(np_dtype):
     results, stats = run_both(build, feeds, kinds=("plain", "replay"))
     assert_same_bits(results)
     assert stats["replay"]["replayed"] == 3
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
+def test_fused_concat_keeps_every_bit(np_dtype):
+    """CONCAT inside a group is an OR of zero-bordered operands: signed zeros,
+    NaN payloads and every integer bit pattern must come through, also when the
+    operands are seen through SLICE views and feed further elementwise nodes."""
+    rng = np.random.default_rng(41)
+    if np_dtype == np.int32:
+        draw = lambda n: rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+    else:
+        def draw(n):
+            v = rng.uniform(-1, 1, n).astype(np_dtype)
+            v[::7] = -0.0
+            v[3::11] = np.nan
+            return v
+    feeds = [draw(5 * 4 * 3) for _ in range(4)]
+    other = draw(7 * 3)
+
+    def build(g, api):
+        x = g.variable(feeds[0], [5, 4, 3], "x")
+        y = g.variable(other, [7, 1, 3], "y")
+        first = api.slice(x, 1, 1, 1)                    # [5, 1, 3] views of x
+        last = api.slice(x, 3, 1, 1)
+        along0 = api.concat([api.concat([first, y], 0), last], 0)   # [17, 1, 3], nested two-operand forms
+        along1 = api.concat([first, last, api.slice(x, 0, 1, 1)], 1)   # [5, 3, 3]
+        doubled = api.neg(api.neg(along0))               # elementwise readers in the same launch
+        return [along0, along1, doubled, api.neg(along1)], x
+
+    results, stats = run_both(build, feeds, kinds=("plain", "replay"))
+    for row, ref in zip(results["replay"], results["plain"]):
+        for a, b in zip(row, ref):
+            assert a.tobytes() == b.tobytes()
+    assert stats["replay"]["replayed"] == 3
