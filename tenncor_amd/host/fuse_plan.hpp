@@ -33,15 +33,32 @@ struct FusedGroup final
 	std::vector<teq::iTensor*> reads;
 };
 
+/// PERMUTE{1,0}(CONTRACT(a, b)) with a matrix result is CONTRACT(b, a) with
+/// the pairs swapped: one product written straight into the PERMUTE node's
+/// buffer, no transposition pass (the shape every matrix-product gradient
+/// takes, tenncor/eteq/backprop.hpp:269-359)
+struct SwappedContract final
+{
+	Observable* node = nullptr;      ///< the PERMUTE node that receives the result
+	teq::iTensor* a = nullptr;       ///< first operand of the product that is launched
+	teq::iTensor* b = nullptr;
+	std::array<uint64_t,8> ashape, bshape;
+	std::vector<uint64_t> pairs;     ///< flattened (dim of a, dim of b)
+	int dtype = 0;
+	std::vector<teq::iTensor*> reads;
+};
+
 struct FusionPlan final
 {
 	struct Step final
 	{
 		Observable* node = nullptr; ///< launched through its own closure, or
-		int group = -1;             ///< index into groups
+		int group = -1;             ///< index into groups, or
+		int contract = -1;          ///< index into contracts
 	};
 
 	std::vector<FusedGroup> groups;
+	std::vector<SwappedContract> contracts;
 	std::vector<Step> steps;
 	/// functors that are computed inside a group or folded into operand views
 	/// and therefore never hold a value of their own
@@ -54,6 +71,8 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 /// Enqueue one group: borrows the outputs' buffers (lifetimes as
 /// eigen::Device::calc gives them), launches, counts the reads
 void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory);
+
+void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 }
 

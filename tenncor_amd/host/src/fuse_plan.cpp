@@ -46,6 +46,7 @@ struct Node final
 	int dtype = 0;
 	bool target = false;
 	bool absorbed = false;      // a VIEW no launch of its own computes
+	int swapped_from = -1;      // PERMUTE launched as the swapped product of this CONTRACT node
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
 	teq::TensptrsT arg_tens;
 	std::vector<int> consumers; // functors of this pass reading the node
@@ -126,11 +127,48 @@ struct Planner final
 			}
 			n.kind = classify(n);
 		}
+		// PERMUTE{1,0} of a matrix-valued CONTRACT nothing else reads: launch the
+		// swapped product instead; the CONTRACT node is looked through like a view
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			Node& n = nodes_[i];
+			if (n.op != egen::PERMUTE || n.args.size() != 1 || n.args[0] < 0) { continue; }
+			Node& c = nodes_[n.args[0]];
+			if (c.op != egen::CONTRACT || c.target || c.consumers.size() != 1 || c.args.size() != 2) { continue; }
+			teq::RanksT order;
+			Packer<teq::RanksT>().unpack(order, *n.f);
+			bool swaps = order.size() >= 2 && order[0] == 1 && order[1] == 0;
+			for (size_t d = 2; d < order.size() && swaps; ++d) { swaps = order[d] == d; }
+			for (int d = 2; d < 8 && swaps; ++d) { swaps = c.shape[d] == 1; }
+			if (false == swaps || c.shape[0] == 1 || c.shape[1] == 1) { continue; }
+			// one surviving dim from each operand: only then is the transpose
+			// of the result the product with the operands exchanged
+			PairVecT<teq::RankT> dims;
+			Packer<PairVecT<teq::RankT>>().unpack(dims, *c.f);
+			size_t free_dims[2] = {0, 0};
+			for (size_t k = 0; k < 2; ++k)
+			{
+				Shape8 shape = shape8(c.arg_tens[k]->shape());
+				for (teq::RankT d = 0; d < 8; ++d)
+				{
+					bool contracted = std::any_of(dims.begin(), dims.end(), [&](const std::pair<teq::RankT,teq::RankT>& pr)
+					{
+						return (k == 0 ? pr.first : pr.second) == d;
+					});
+					free_dims[k] += shape[d] > 1 && false == contracted;
+				}
+			}
+			if (free_dims[0] != 1 || free_dims[1] != 1) { continue; }
+			n.kind = OTHER;
+			n.swapped_from = n.args[0];
+			c.kind = VIEW;
+			c.absorbed = true;
+		}
 		// a view is folded away when everything that reads it can read through it
 		for (size_t i = nodes_.size(); i-- > 0;)
 		{
 			Node& n = nodes_[i];
-			if (n.kind != VIEW || n.target || n.consumers.empty()) { continue; }
+			if (n.kind != VIEW || n.target || n.consumers.empty() || n.op == egen::CONTRACT) { continue; }
 			n.absorbed = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
 			{
 				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed);
@@ -633,6 +671,39 @@ struct Planner final
 			{
 				if (d != u) { visit(d); }
 			}
+			if (nodes_[u].kind != EW && nodes_[u].swapped_from >= 0)
+			{
+				const Node& c = nodes_[nodes_[u].swapped_from];
+				SwappedContract call;
+				call.node = nodes_[u].f;
+				call.dtype = c.dtype;
+				call.a = c.arg_tens[1].get();
+				call.b = c.arg_tens[0].get();
+				call.ashape = shape8(call.a->shape());
+				call.bshape = shape8(call.b->shape());
+				PairVecT<teq::RankT> dims;
+				Packer<PairVecT<teq::RankT>>().unpack(dims, *c.f);
+				for (auto& d : dims)
+				{
+					call.pairs.push_back(d.second);
+					call.pairs.push_back(d.first);
+				}
+				// the reads the two nodes would have counted: the product's operands
+				for (size_t k = 0; k < 2; ++k)
+				{
+					int a = c.args[k];
+					if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+					{
+						call.reads.push_back(c.arg_tens[k].get());
+					}
+				}
+				FusionPlan::Step step;
+				step.contract = (int) plan.contracts.size();
+				plan.contracts.push_back(call);
+				plan.absorbed.push_back(c.f);
+				plan.steps.push_back(step);
+				return;
+			}
 			if (nodes_[u].kind != EW)
 			{
 				FusionPlan::Step step;
@@ -723,6 +794,20 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 	Planner planner(funcs, targets);
 	planner.group_all();
 	return planner.finish();
+}
+
+void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory)
+{
+	Observable* out = call.node;
+	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
+	void* dst = static_cast<iEigen&>(out->device()).borrow_output(ttl, memory);
+	if (nullptr == dst) { global::fatalf("%s cannot take a product", out->to_string().c_str()); }
+	const void* a = eigen_ref(*call.a).device_data();
+	const void* b = eigen_ref(*call.b).device_data();
+	if (nullptr == a || nullptr == b) { global::fatal("operand of a matrix product has no data"); }
+	hip_check(tcg_contract(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
+		(int) (call.pairs.size() / 2), call.pairs.data(), a, b, dst));
+	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
 void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory)

@@ -358,6 +358,11 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 				ss << "node " << step.node->get_opcode().name_ << "\n";
 				continue;
 			}
+			if (step.contract >= 0)
+			{
+				ss << "swapped CONTRACT+PERMUTE\n";
+				continue;
+			}
 			auto& group = plan.groups[step.group];
 			ss << "group ";
 			for (size_t i = 0; i < group.members.size(); ++i)

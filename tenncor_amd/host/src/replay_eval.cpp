@@ -209,6 +209,10 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 			{
 				device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0));
 			}
+			else if (step.contract >= 0)
+			{
+				launch_contract(fusion.contracts[step.contract], targets, device.memory());
+			}
 			else
 			{
 				launch_group(fusion.groups[step.group], targets, device.memory());

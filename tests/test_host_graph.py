@@ -271,6 +271,8 @@ def parse_plan(lines):
         elif kind == "group":
             ops, *fields = rest.split(" ")
             steps.append(("group", ops.split("+"), {k: int(v) for k, v in (f.split("=") for f in fields)}))
+        elif kind == "swapped":
+            steps.append(("swapped", rest.split("+"), {}))
         else:
             steps.append(("folded", [], {"n": int(rest)}))
     return steps
@@ -286,12 +288,14 @@ def test_launch_plan_groups_the_elementwise_nodes_of_an_mlp(g):
     # every functor is launched on its own, computed inside a group, or folded into operand views
     in_groups = sum(len(s[1]) for s in launches if s[0] == "group")
     stores = sum(s[2]["stores"] for s in launches if s[0] == "group")
-    alone = sum(1 for s in launches if s[0] == "node")
+    alone = sum(1 for s in launches if s[0] in ("node", "swapped"))
     assert alone + stores + folded == nfunc
     assert len(launches) < nfunc // 2
     assert any(s[0] == "group" and "SIGMOID" in s[1] and len(s[1]) >= 3 for s in launches)
     # the matrix products and reductions keep their own kernels
-    assert sum(1 for s in launches if s[0] == "node" and s[1][0] in ("CONTRACT", "MATMUL")) == 5
+    # ... except that the transposed products of the weight gradients are launched as one product
+    assert sum(1 for s in launches if s[0] == "node" and s[1][0] in ("CONTRACT", "MATMUL")) == 3
+    assert sum(1 for s in launches if s[0] == "swapped") == 2 and "node PERMUTE" not in g.launch_plan(targets)
     for s in launches:
         if s[0] == "group":
             assert s[2]["leaves"] <= 8 and s[2]["stores"] <= 8 and s[2]["instrs"] <= 64
