@@ -228,7 +228,7 @@ def run_extras(ctx, capi):
     return extra
 
 
-def run_graph_configs(only=None, evaluator=None, reps=20):
+def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
     """configs[0], [3], [4] through the host graph layer (Functor nodes, the
     gradient builder, teq::Evaluator + eigen::Device): wall time of
     evaluate(targets) after re-assigning the input, which forces a full
@@ -261,17 +261,26 @@ def run_graph_configs(only=None, evaluator=None, reps=20):
             g = tg.Graph()
             if only == 1:
                 targets, x, _ = configs.config1_mlp(g)
-                t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
             elif only == 4:
                 targets, x, _, flops = configs.config4_lstm(g)
                 xs = rng.uniform(-1, 1, 256 * 64 * 256).astype(np.float32)
-                t = timed(g, targets, x, lambda: xs, reps)
+                fresh = lambda: xs
             else:
                 targets, x, _, flops = configs.config5_cnn(g)
                 xs = rng.uniform(0, 1, 128 * 28 * 28).astype(np.float32)
-                t = timed(g, targets, x, lambda: xs, reps)
+                fresh = lambda: xs
+            if only == 1:
+                fresh, reps = (lambda: rng.uniform(-1, 1, 30).astype(np.float32)), 300
+            cleanup = None
+            if optimize:
+                # hone::optimize first: equal subgraphs merged, constants folded,
+                # the shipped conversions applied
+                targets, cleanup = g.optimize(targets)
+            t = timed(g, targets, x, fresh, reps)
             out = {"graph_config": only, "evaluator": kind, "ms_per_eval": round(t * 1e3, 4),
                    "functors": g.count_functors(targets), "evaluator_stats": tg.evaluator_stats()}
+            if cleanup is not None:
+                out["optimize"] = cleanup
             tg.set_evaluator("plain")
             return out
         g = tg.Graph()
@@ -376,13 +385,15 @@ def main():
                     help="time only this whole-graph configuration and print its line (for profiling)")
     ap.add_argument("--evaluator", choices=["plain", "replay", "replay_unfused"], default="replay")
     ap.add_argument("--reps", type=int, default=20, help="timed evaluations with --graph-config 4 or 5")
+    ap.add_argument("--optimize", action="store_true",
+                    help="with --graph-config: clean the graph up first (duplicates merged, constants folded, conversions)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU; --gpus %d is not supported "
                  "(no collectives or sharding are part of this build)" % args.gpus)
 
     if args.graph_config is not None:
-        print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps)))
+        print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps, optimize=args.optimize)))
         return
     wall, per_class, extra, arch = run_gpu(args.steps, args.warmup, graphs=not args.no_graphs)
     abytes = algorithmic_bytes()

@@ -96,6 +96,20 @@ int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count);
  * of their own. Returns the length the text needs (it is cut to `capacity`). */
 int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, size_t capacity, size_t* needed);
 
+/* ---- graph clean-up (tenncor/hone/optimize.hpp:19-38: `hone::optimize(roots, rulestream)`) ----
+ * Merges equal subgraphs (tenncor/hone/duplicates.hpp:97-101), then repeats, until
+ * nothing changes (50 rounds at most, tenncor/hone/src/optimize.cpp:11,27-31):
+ * functors other than IDENTITY whose operands are all constants are evaluated
+ * on the GPU and replaced by constants (tenncor/hone/cstrules.hpp:48-65), and the
+ * conversions of `rules_json` are applied ({"conversions": [{"srcs": [pattern...],
+ * "dest": target}]}, the schema of internal/opt/optimize.proto:7-35 over
+ * internal/query/query.proto:7-79; NULL = no conversions). Readers of replaced
+ * nodes are rewired in place. out_roots[i] is the node that replaces roots[i].
+ * fold = 0 skips the evaluation of constant functors (needs no GPU then).
+ * stats = {nodes merged, functors folded, matches converted, rounds}. */
+int tcr_optimize (tcr_graph* g, int nroots, const int* roots, const char* rules_json, int fold,
+	int* out_roots, uint64_t stats[4]);
+
 #ifdef __cplusplus
 }
 #endif

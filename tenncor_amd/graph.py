@@ -27,10 +27,14 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
-    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan",
+    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan", "tcr_optimize",
 ]
 
 EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED = 0, 1, 2
+
+# conversions shipped with the package (the reference's cfg/optimizations.json
+# is a git-lfs pointer without content)
+DEFAULT_RULES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "host", "cfg", "optimizations.json")
 
 _lib = None
 
@@ -72,6 +76,7 @@ def load():
         "tcr_set_evaluator": [i32],
         "tcr_evaluator_stats": [u64p],
         "tcr_launch_plan": [vp, i32, i32p, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
+        "tcr_optimize": [vp, i32, i32p, ctypes.c_char_p, i32, i32p, u64p],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -251,6 +256,26 @@ class Graph:
         buf = ctypes.create_string_buffer(need.value + 1)
         self._check(self.lib.tcr_launch_plan(self.h, len(targets), ids, buf, need.value + 1, ctypes.byref(need)))
         return buf.value.decode().splitlines()
+
+    def optimize(self, roots, rules=DEFAULT_RULES, fold=True):
+        """hone::optimize (tenncor/hone/optimize.hpp:19-38): merge equal
+        subgraphs, fold functors of constants into constants (evaluated on the
+        GPU unless fold=False) and apply the conversions of `rules`: JSON text,
+        a path to a JSON file, or None for no conversions.  Readers of replaced
+        nodes are rewired in place.  Returns (new roots, stats)."""
+        text = None
+        if rules is not None:
+            text = rules
+            if os.path.exists(rules):
+                with open(rules) as f:
+                    text = f.read()
+            text = text.encode()
+        ids = _ints([r.id for r in roots])
+        out = (ctypes.c_int * len(roots))()
+        stats = (ctypes.c_uint64 * 4)()
+        self._check(self.lib.tcr_optimize(self.h, len(roots), ids, text, int(bool(fold)), out, stats))
+        keys = ("merged", "folded", "converted", "rounds")
+        return [Node(self, out[i]) for i in range(len(roots))], dict(zip(keys, [int(v) for v in stats]))
 
     def count_functors(self, nodes):
         c = ctypes.c_int()

@@ -8,6 +8,7 @@
 #include "eteq.hpp"
 #include "replay_eval.hpp"
 #include "fuse_plan.hpp"
+#include "hone.hpp"
 
 struct tcr_graph
 {
@@ -380,6 +381,28 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 			size_t n = std::min(text.size(), capacity - 1);
 			memcpy(out, text.data(), n);
 			out[n] = '\0';
+		}
+	});
+}
+
+int tcr_optimize (tcr_graph* g, int nroots, const int* roots, const char* rules_json, int fold,
+	int* out_roots, uint64_t stats[4])
+{
+	return guarded([&]
+	{
+		hone::RulesT rules;
+		if (nullptr != rules_json) { rules = hone::parse_rules(rules_json); }
+		teq::TensptrsT in;
+		for (int i = 0; i < nroots; ++i) { in.push_back(g->at(roots[i])); }
+		hone::Stats st;
+		teq::TensptrsT out = hone::optimize(in, rules, 0 != fold, &st);
+		for (int i = 0; i < nroots; ++i) { out_roots[i] = g->add(out[i]); }
+		if (nullptr != stats)
+		{
+			stats[0] = st.merged;
+			stats[1] = st.folded;
+			stats[2] = st.converted;
+			stats[3] = st.rounds;
 		}
 	});
 }

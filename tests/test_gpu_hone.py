@@ -1,0 +1,150 @@
+"""Graph clean-up with constant folding on the GPU: the reference's own
+expected graphs for hone::optimize (tenncor/hone/test/test_cstrules.cpp:20-147,
+tenncor/test/test_opt.cpp:25-112) -- their inputs and the printed graphs they
+expect are restated below -- and value equality of the benchmark graphs before
+and after the clean-up.  The reference's tests read cfg/optimizations.json,
+which is a git-lfs pointer without content; none of the expected graphs
+contains a pattern a conversion could match, so they pin merging and folding.
+
+Tolerance: the folded constants are integers computed in double (exact); the
+cleaned-up configuration graphs are compared at 1e-5 relative to max |ref|
+(conversions such as -(-x) -> x change no value, but merged operands change
+the order in which a gradient's n-ary ADD sums them).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+DATA = [59, 10, 28, 10, 67, 62, 23, 4, 55, 77, 28, 16, 82, 52, 47, 16, 7, 85, 37, 2, 8, 52, 62, 43]
+DATA2 = [22, 15, 74, 38, 61, 95, 62, 81, 99, 76, 7, 22, 56, 50, 19, 13, 12, 10, 31, 40, 60, 54, 6, 83]
+SHAPE = [2, 3, 4]
+S = "[2\\3\\4\\1\\1\\1\\1\\1]"
+
+
+@pytest.fixture()
+def g():
+    from tenncor_amd import graph
+    gr = graph.Graph()
+    yield gr
+    gr.close()
+
+
+def cst(g, values):
+    return g.constant(np.array(values, np.float64), SHAPE)
+
+
+def test_functors_of_constants_fold_into_one_constant(g):
+    # CSTRULES.Typical
+    a, b, c = cst(g, DATA), cst(g, DATA2), g.scalar(4.0, np.float64, SHAPE)
+    lhs = g.functor("ADD", [b, c])
+    rhs = g.functor("ADD", [a, b])
+    (out,), stats = g.optimize([g.functor("ADD", [lhs, rhs])])
+    assert g.to_string(out) == "(constant:[107\\44\\180\\90\\193\\...]<DOUBLE>%s)" % S
+    assert stats["folded"] == 3
+    expect = np.array(DATA, np.float64) + 2 * np.array(DATA2, np.float64) + 4
+    np.testing.assert_array_equal(g.data(out), expect)
+
+
+def test_folding_stops_at_a_variable(g):
+    # CSTRULES.StopAtVar
+    a = g.variable(np.array(DATA, np.float64), SHAPE, "a")
+    b, c = cst(g, DATA2), g.scalar(4.0, np.float64, SHAPE)
+    lhs = g.functor("ADD", [b, c])
+    rhs = g.functor("ADD", [a, b])
+    (out,), _ = g.optimize([g.functor("ADD", [lhs, rhs])])
+    assert g.to_string(out) == (
+        "(ADD<DOUBLE>%s)\n"
+        "_`--(constant:[26\\19\\78\\42\\65\\...]<DOUBLE>%s)\n"
+        "_`--(ADD<DOUBLE>%s)\n"
+        "_____`--(variable:a<DOUBLE>%s)\n"
+        "_____`--(constant:[22\\15\\74\\38\\61\\...]<DOUBLE>%s)" % (S, S, S, S, S))
+
+
+def test_identity_keeps_its_dependencies(g):
+    # CSTRULES.IdentityDependency
+    a, b, c = cst(g, DATA), cst(g, DATA2), g.scalar(4.0, np.float64, SHAPE)
+    lhs = g.functor("ADD", [b, c])
+    rhs = g.functor("ADD", [a, b])
+    (out,), _ = g.optimize([g.functor("IDENTITY", [lhs, rhs])])
+    assert g.to_string(out) == (
+        "(IDENTITY<DOUBLE>%s)\n"
+        "_`--(constant:[26\\19\\78\\42\\65\\...]<DOUBLE>%s)\n"
+        "_`--(constant:[81\\25\\102\\48\\128\\...]<DOUBLE>%s)" % (S, S, S))
+
+
+DEPENDS = (
+    "(%s<DOUBLE>" + S + ")\n"
+    "_`--(variable:<DOUBLE>" + S + ")\n"
+    "_`--(IDENTITY<DOUBLE>" + S + ")\n"
+    "_____`--(constant:[88\\60\\296\\152\\244\\...]<DOUBLE>" + S + ")\n"
+    "_____`--(constant:[81\\25\\102\\48\\128\\...]<DOUBLE>" + S + ")")
+
+
+def test_assignment_of_an_identity_with_dependencies(g):
+    # OPTIMIZE.Depends
+    target = g.variable(np.array(DATA, np.float64), SHAPE, "")
+    a, b, d = cst(g, DATA), cst(g, DATA2), g.scalar(4.0, np.float64, SHAPE)
+    c = g.functor("ADD", [a, b])
+    ident = g.functor("IDENTITY", [g.functor("MUL", [b, d]), c])
+    (out,), _ = g.optimize([g.functor("ASSIGN", [target, ident])])
+    assert g.to_string(out) == DEPENDS % "ASSIGN"
+
+
+def test_dependencies_are_not_taken_for_operands_of_a_sum(g):
+    # OPTIMIZE.DependsNnary: same values before and after
+    target = g.variable(np.array(DATA, np.float64), SHAPE, "")
+    a, b, d = cst(g, DATA), cst(g, DATA2), g.scalar(4.0, np.float64, SHAPE)
+    c = g.functor("ADD", [a, b])
+    ident = g.functor("IDENTITY", [g.functor("MUL", [b, d]), c])
+    add = g.functor("ADD", [target, ident])
+    g.evaluate([add])
+    before = g.data(add).copy()
+    (out,), _ = g.optimize([add])
+    assert g.to_string(out) == DEPENDS % "ADD"
+    g.evaluate([out])
+    np.testing.assert_array_equal(g.data(out), before)
+    np.testing.assert_array_equal(before, np.array(DATA, np.float64) + 4 * np.array(DATA2, np.float64))
+
+
+def test_scalar_constants_fold_through_extend_and_meet_the_conversions(g):
+    from tenncor_amd import graph
+    api = graph.Api(g)
+    x = g.variable(np.arange(6, dtype=np.float32) - 2.5, [3, 2], "x")
+    # mul(x, 1) and add(., 0) as the TenncorAPI builds them: EXTEND(scalar constant)
+    root = api.add(api.mul(x, 1.0), 0.0)
+    assert g.count_functors([root]) == 4
+    (out,), stats = g.optimize([root])
+    assert out.id == x.id
+    assert stats["folded"] == 2 and stats["converted"] == 2
+
+
+@pytest.mark.parametrize("evaluator", ["plain", "replay"])
+@pytest.mark.parametrize("config", ["mlp", "lstm", "cnn"])
+def test_configuration_graphs_keep_their_values(config, evaluator):
+    from tenncor_amd import graph, configs
+    graph.set_evaluator(evaluator)
+    try:
+        results = []
+        for optimize in (False, True):
+            g = graph.Graph()
+            if config == "mlp":
+                targets = configs.config1_mlp(g)[0]
+            elif config == "lstm":
+                targets = configs.config4_lstm(g, seq=6, batch=8, nin=16, hid=32)[0]
+            else:
+                targets = configs.config5_cnn(g, batch=4, hw=12, c1=4, c2=8)[0]
+            before = g.count_functors(targets)
+            if optimize:
+                targets, stats = g.optimize(targets)
+                assert g.count_functors(targets) < before
+                assert stats["merged"] > 0 and stats["rounds"] < 50
+            for _ in range(3):  # walked, recorded, replayed
+                g.evaluate(targets)
+            results.append([g.data(t).copy() for t in targets])
+            g.close()
+        for raw, cleaned in zip(*results):
+            scale = np.abs(raw).max() + 1e-30
+            assert np.abs(raw - cleaned).max() <= 1e-5 * scale
+    finally:
+        graph.set_evaluator("plain")
