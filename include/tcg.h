@@ -165,6 +165,26 @@ int tcg_cast (tcg_ctx* ctx, int out_dtype, int in_dtype, uint64_t n,
 int tcg_assign (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
 	void* target, const void* source);
 
+/* RAND_UNIF on the device: out[i] uniform between lo[i] and hi[i]
+ * (cfg/ops.yml:101-103; internal/eigen/operator.hpp:989-1044). The reference
+ * draws on the host from std::default_random_engine
+ * (internal/global/random.hpp:87-99, 143); this generator is Philox4x32-10
+ * keyed by `seed`, so the streams differ while the distributions agree: real
+ * types lo + u*(hi-lo) with u in [0,1) of 24 (float) or 53 (double) random
+ * bits, int32 uniform on the inclusive range lo..hi (multiply-shift of a
+ * 32-bit word). Generator block b of the context's stream is
+ * philox(counter = {b, 0}, key = seed); a draw of n elements consumes
+ * ceil(n/4) blocks (ceil(n/2) for double), element i taking word i%4 of block
+ * i/4 (words 2(i%2), 2(i%2)+1 of block i/2). Key and block count live in
+ * device memory and are advanced by kernels: a recorded sequence draws new
+ * values at every launch. tcg_rand_seed(seed) restarts the stream at block 0
+ * (the counterpart of global::seed, internal/global/random.hpp:79);
+ * tcg_rand_state returns {seed, blocks drawn} after a synchronisation. */
+int tcg_rand_seed (tcg_ctx* ctx, uint64_t seed);
+int tcg_rand_state (tcg_ctx* ctx, uint64_t out[2]);
+int tcg_rand_uniform (tcg_ctx* ctx, int dtype, uint64_t n, const void* lo,
+	const void* hi, void* out);
+
 /* A chain of elementwise nodes evaluated in one pass over memory: what a run
  * of consecutive MatOp/TensOp closures (internal/eigen/device.hpp:304-372)
  * computes, without materialising the intermediates.

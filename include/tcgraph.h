@@ -71,6 +71,20 @@ int tcr_set_evaluator (int kind);
  * the latest recording, out[5] device bytes reserved by live recordings */
 int tcr_evaluator_stats (uint64_t out[6]);
 
+/* Where RAND_UNIF nodes whose operator is built from now on draw their values.
+ * TCR_RANDOM_HOST (default): on the host from the seeded std::default_random_engine,
+ * as the reference does (internal/eigen/operator.hpp:989-1044,
+ * internal/global/random.hpp:87-99,143); such nodes make the replaying evaluator
+ * fall back to the node-by-node walk. TCR_RANDOM_DEVICE: on the GPU with the
+ * counter-based generator of tcg_rand_uniform (another stream, same
+ * distributions); recorded passes then draw new values at every replay. */
+#define TCR_RANDOM_HOST 0
+#define TCR_RANDOM_DEVICE 1
+int tcr_set_random (int where);
+/* global::seed (internal/global/random.hpp:79): seeds the host generator and
+ * restarts the device generator's stream under the same seed */
+int tcr_seed (uint64_t seed);
+
 /* iTensor::shape / get_meta().type_code / device().data() */
 int tcr_shape (tcr_graph* g, int node, uint64_t shape[8]);
 int tcr_dtype (tcr_graph* g, int node, int* dtype);

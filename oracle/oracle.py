@@ -319,3 +319,22 @@ def conv(img, imgshape, kernel, kshape, ranks, wide_acc=False):
     _check(lib().orc_conv(dtype_code(img), _u64(si), _u64(sk), len(r), _u64(r if r else [0]), int(wide_acc),
                           _p(img), _p(kernel), _p(out)), "CONV")
     return out, oshape
+
+
+def philox4x32_10(counter, key):
+    """Philox4x32-10 of four counter words under two key words."""
+    c = (ctypes.c_uint32 * 4)(*[int(v) for v in counter])
+    k = (ctypes.c_uint32 * 2)(*[int(v) for v in key])
+    out = (ctypes.c_uint32 * 4)()
+    lib().orc_philox4x32_10(c, k, out)
+    return [int(v) for v in out]
+
+
+def rand_uniform(lo, hi, seed, first_block=0):
+    """The device RAND_UNIF stream for bounds `lo`, `hi` (same dtype)."""
+    lo, hi = _flat(lo), _flat(hi)
+    assert lo.dtype == hi.dtype and lo.size == hi.size
+    out = np.empty(lo.size, dtype=lo.dtype)
+    _check(lib().orc_rand_uniform(dtype_code(lo), ctypes.c_uint64(lo.size), ctypes.c_uint64(seed),
+                                  ctypes.c_uint64(first_block), _p(lo), _p(hi), _p(out)), "RAND_UNIF")
+    return out

@@ -325,3 +325,60 @@ int orc_conv (int dtype, const uint64_t imgshape[8], const uint64_t kshape[8],
 		conv_f32(imgshape, kshape, nranks, ranks, wide_acc, (const float*) img, (const float*) kernel, (float*) out),
 		conv_i32(imgshape, kshape, nranks, ranks, 0, (const int32_t*) img, (const int32_t*) kernel, (int32_t*) out))
 }
+
+/* ---- device RAND_UNIF stream ------------------------------------------- */
+
+void orc_philox4x32_10 (const uint32_t counter[4], const uint32_t key[2], uint32_t out[4])
+{
+	uint32_t c[4] = {counter[0], counter[1], counter[2], counter[3]};
+	uint32_t k0 = key[0], k1 = key[1];
+	for (int round = 0; round < 10; ++round)
+	{
+		uint64_t p0 = (uint64_t) 0xD2511F53u * c[0];
+		uint64_t p1 = (uint64_t) 0xCD9E8D57u * c[2];
+		uint32_t n0 = (uint32_t) (p1 >> 32) ^ c[1] ^ k0;
+		uint32_t n1 = (uint32_t) p1;
+		uint32_t n2 = (uint32_t) (p0 >> 32) ^ c[3] ^ k1;
+		uint32_t n3 = (uint32_t) p0;
+		c[0] = n0; c[1] = n1; c[2] = n2; c[3] = n3;
+		k0 += 0x9E3779B9u;
+		k1 += 0xBB67AE85u;
+	}
+	memcpy(out, c, sizeof(c));
+}
+
+int orc_rand_uniform (int dtype, uint64_t n, uint64_t seed, uint64_t first_block,
+	const void* lo, const void* hi, void* out)
+{
+	const uint32_t key[2] = {(uint32_t) seed, (uint32_t) (seed >> 32)};
+	const uint64_t per = dtype == 1 ? 2 : 4;
+	if (dtype < 1 || dtype > 3) { return 1; }
+	for (uint64_t i = 0; i < n; ++i)
+	{
+		uint64_t block = first_block + i / per;
+		uint32_t ctr[4] = {(uint32_t) block, (uint32_t) (block >> 32), 0, 0}, r[4];
+		orc_philox4x32_10(ctr, key, r);
+		unsigned k = (unsigned) (i % per);
+		if (dtype == 2)
+		{
+			float a = ((const float*) lo)[i], b = ((const float*) hi)[i];
+			float u = (float) (r[k] >> 8) * 0x1p-24f;
+			((float*) out)[i] = fmaf(u, b - a, a);
+		}
+		else if (dtype == 1)
+		{
+			double a = ((const double*) lo)[i], b = ((const double*) hi)[i];
+			uint64_t bits = ((uint64_t) r[2 * k + 1] << 32) | r[2 * k];
+			double u = (double) (bits >> 11) * 0x1p-53;
+			((double*) out)[i] = fma(u, b - a, a);
+		}
+		else
+		{
+			int32_t a = ((const int32_t*) lo)[i], b = ((const int32_t*) hi)[i];
+			if (b < a) { ((int32_t*) out)[i] = a; continue; }
+			uint64_t range = (uint64_t) ((int64_t) b - (int64_t) a) + 1;
+			((int32_t*) out)[i] = (int32_t) ((int64_t) a + (int64_t) (((uint64_t) r[k] * range) >> 32));
+		}
+	}
+	return 0;
+}

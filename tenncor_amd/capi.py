@@ -39,6 +39,7 @@ EXPORTS = [
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
     "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_capture_begin", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
+    "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
 
 
@@ -102,6 +103,9 @@ def load():
         "tcg_ew_select": [vp, i32, u64, vp, vp, vp, vp],
         "tcg_cast": [vp, i32, i32, u64, vp, vp],
         "tcg_assign": [vp, i32, i32, u64, vp, vp],
+        "tcg_rand_seed": [vp, u64],
+        "tcg_rand_state": [vp, ctypes.POINTER(ctypes.c_uint64)],
+        "tcg_rand_uniform": [vp, i32, u64, vp, vp, vp],
         "tcg_ew_fused": [vp, i32, u64, i32, vpp, i32, ctypes.POINTER(EwInstr), vp],
         "tcg_ew_fusedx": [vp, i32, u64p, i32, ctypes.POINTER(FxLeaf), i32, ctypes.POINTER(FxInstr), i32, vpp],
         "tcg_reduce": [vp, i32, i32, u64p, ctypes.c_uint, vp, vp],
@@ -290,6 +294,18 @@ class Context:
 
     def assign(self, op, dtype, n, target, source):
         self._check(self.lib.tcg_assign(self.handle, _opcode(op), dtype, n, target, source))
+
+    def rand_seed(self, seed):
+        self._check(self.lib.tcg_rand_seed(self.handle, int(seed)))
+
+    def rand_state(self):
+        """(seed, generator blocks drawn so far)."""
+        out = (ctypes.c_uint64 * 2)()
+        self._check(self.lib.tcg_rand_state(self.handle, out))
+        return int(out[0]), int(out[1])
+
+    def rand_uniform(self, dtype, n, lo, hi, dst):
+        self._check(self.lib.tcg_rand_uniform(self.handle, dtype, n, lo, hi, dst))
 
     def ew_fused(self, dtype, n, leaves, program, dst):
         """program: list of (opcode, a, b, dst[, imm])."""

@@ -71,6 +71,14 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		delete ctx;
 		return rc;
 	}
+	const uint64_t rng_init[2] = {0, 0};
+	if ((err = hipMalloc((void**) &ctx->rng_state, sizeof(rng_init))) != hipSuccess ||
+		(err = hipMemcpy(ctx->rng_state, rng_init, sizeof(rng_init), hipMemcpyHostToDevice)) != hipSuccess)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: generator state: %s", hipGetErrorString(err));
+		delete ctx;
+		return rc;
+	}
 	*out = ctx;
 	return TCG_OK;
 }
@@ -82,6 +90,7 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	(void) hipStreamSynchronize(ctx->stream);
 	for (auto& kv : ctx->block_size) { (void) hipFree(kv.first); }
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
+	if (ctx->rng_state) { (void) hipFree(ctx->rng_state); }
 	(void) hipEventDestroy(ctx->ev_begin);
 	(void) hipEventDestroy(ctx->ev_end);
 	(void) hipStreamDestroy(ctx->stream);

@@ -56,6 +56,10 @@ struct tcg_ctx
 	size_t staging_size = 0;
 	size_t staging_head = 0;
 
+	// device generator: {key, blocks drawn so far}, read and advanced by
+	// kernels only so that recorded launches draw fresh values at every replay
+	uint64_t* rng_state = nullptr;
+
 	// launch capture: the graph being recorded and, for every block that
 	// belongs to some graph, its owner
 	tcg_graph* capturing = nullptr;

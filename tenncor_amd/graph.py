@@ -28,6 +28,7 @@ EXPORTS = [
     "tcr_functor", "tcr_derive", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
     "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan", "tcr_optimize",
+    "tcr_set_random", "tcr_seed",
 ]
 
 EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED = 0, 1, 2
@@ -77,6 +78,8 @@ def load():
         "tcr_evaluator_stats": [u64p],
         "tcr_launch_plan": [vp, i32, i32p, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
         "tcr_optimize": [vp, i32, i32p, ctypes.c_char_p, i32, i32p, u64p],
+        "tcr_set_random": [i32],
+        "tcr_seed": [ctypes.c_uint64],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -97,6 +100,22 @@ def set_evaluator(kind):
     lib = load()
     code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY, "replay_unfused": EVAL_REPLAY_UNFUSED}[kind]
     if lib.tcr_set_evaluator(code) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+
+
+def set_random(where):
+    """Where RAND_UNIF nodes built from now on draw: "host" (the reference's
+    std::default_random_engine, the default) or "device" (counter-based
+    generator on the GPU; another stream, the same distributions)."""
+    lib = load()
+    if lib.tcr_set_random({"host": 0, "device": 1}[where]) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+
+
+def seed(value):
+    """global::seed: seeds the host generator and restarts the device stream."""
+    lib = load()
+    if lib.tcr_seed(int(value)) != 0:
         raise GraphError(lib.tcr_last_error().decode())
 
 

@@ -113,6 +113,14 @@ EigenptrT select (teq::Shape outshape, const teq::iTensor& condition,
 template <typename T>
 EigenptrT rand_uniform (teq::Shape outshape, const teq::iTensor& a, const teq::iTensor& b)
 {
+	if (global::device_random())
+	{
+		uint64_t n = outshape.n_elems();
+		return make_op<T>(outshape, {&a, &b}, [n](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
+		{
+			hip_check(tcg_rand_uniform(ctx, egen::get_type<T>(), n, args[0], args[1], out));
+		});
+	}
 	return std::make_shared<HostOp<T>>(outshape, teq::CTensT{&a, &b},
 	[](T* out, const std::vector<const void*>& args, size_t n)
 	{

@@ -108,6 +108,12 @@ using RandEngineT = std::default_random_engine;
 RandEngineT& get_generator (void);
 void seed (size_t s);
 
+// Where RAND_UNIF closures built from now on draw: false = on the host from
+// get_generator() (the reference's behaviour and stream family), true = on the
+// device (a counter-based generator with its own stream; such nodes can be
+// part of a recorded launch sequence)
+bool& device_random (void);
+
 }
 
 #endif // TCH_GLOBAL_HPP

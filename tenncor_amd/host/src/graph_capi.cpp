@@ -385,6 +385,24 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 	});
 }
 
+int tcr_set_random (int where)
+{
+	return guarded([&]
+	{
+		if (TCR_RANDOM_HOST != where && TCR_RANDOM_DEVICE != where) { global::fatalf("unknown generator %d", where); }
+		global::device_random() = TCR_RANDOM_DEVICE == where;
+	});
+}
+
+int tcr_seed (uint64_t seed)
+{
+	return guarded([&]
+	{
+		global::seed(seed);
+		eigen::hip_check(tcg_rand_seed(eigen::hip_context(), seed));
+	});
+}
+
 int tcr_optimize (tcr_graph* g, int nroots, const int* roots, const char* rules_json, int fold,
 	int* out_roots, uint64_t stats[4])
 {

@@ -43,6 +43,12 @@ void seed (size_t s)
 	get_generator().seed(s);
 }
 
+bool& device_random (void)
+{
+	static bool on_device = false;
+	return on_device;
+}
+
 }
 
 namespace teq

@@ -788,3 +788,59 @@ def test_interpreted_groups_match_too():
                           text=True, timeout=300)
     assert done.returncode == 0, done.stdout[-3000:]
     assert " passed" in done.stdout
+
+
+# ---- device RAND_UNIF --------------------------------------------------------
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32])
+def test_device_generator_is_bit_exact_with_the_restated_stream(ctx, oracle, np_dtype):
+    """Bit-exact against the CPU restatement of Philox4x32-10 (itself pinned by
+    the published known-answer vectors): ragged sizes, consecutive draws that
+    continue one stream, a restart under a new seed."""
+    rng = np.random.default_rng(11)
+    seed = 0x5eed0000cafe
+    ctx.rand_seed(seed)
+    assert ctx.rand_state() == (seed, 0)
+    per = 2 if np_dtype == np.float64 else 4
+    drawn = 0
+    for n in (1, 3, 5, 64, 1000003):
+        if np_dtype == np.int32:
+            lo = rng.integers(-1000, 1000, n).astype(np.int32)
+            hi = (lo + rng.integers(0, 5000, n)).astype(np.int32)
+            if n > 4:
+                lo[1], hi[1] = -2 ** 31, 2 ** 31 - 1
+                lo[2], hi[2] = 9, 3
+        else:
+            lo = rng.uniform(-3, 1, n).astype(np_dtype)
+            hi = (lo + rng.uniform(0, 4, n)).astype(np_dtype)
+        dlo, dhi, out = ctx.upload(lo), ctx.upload(hi), ctx.empty(n, np_dtype)
+        ctx.rand_uniform(out.dtype, n, dlo.ptr, dhi.ptr, out.ptr)
+        got = out.get()
+        np.testing.assert_array_equal(got, oracle.rand_uniform(lo, hi, seed, first_block=drawn))
+        drawn += (n + per - 1) // per
+        assert ctx.rand_state() == (seed, drawn)
+        if np_dtype != np.int32:
+            assert np.all(got >= lo) and np.all(got <= hi)
+        for buf in (dlo, dhi, out):
+            buf.release()
+    ctx.rand_seed(77)
+    lo, hi = np.zeros(10, np_dtype), np.full(10, 100, np_dtype)
+    dlo, dhi, out = ctx.upload(lo), ctx.upload(hi), ctx.empty(10, np_dtype)
+    ctx.rand_uniform(out.dtype, 10, dlo.ptr, dhi.ptr, out.ptr)
+    np.testing.assert_array_equal(out.get(), oracle.rand_uniform(lo, hi, 77))
+
+
+def test_device_generator_draws_anew_at_every_launch_of_a_recording(ctx, oracle):
+    n, seed = 1000, 2024
+    lo, hi = np.full(n, -1, np.float32), np.full(n, 1, np.float32)
+    dlo, dhi, out = ctx.upload(lo), ctx.upload(hi), ctx.empty(n, np.float32)
+    ctx.rand_seed(seed)
+    ctx.sync()
+    ctx.capture_begin()
+    ctx.rand_uniform(out.dtype, n, dlo.ptr, dhi.ptr, out.ptr)
+    graph = ctx.capture_end()
+    for launch in range(4):
+        ctx.graph_launch(graph)
+        np.testing.assert_array_equal(out.get(), oracle.rand_uniform(lo, hi, seed, first_block=launch * 250))
+    assert ctx.rand_state() == (seed, 1000)
+    ctx.graph_destroy(graph)

@@ -237,3 +237,83 @@ def test_cast_and_assign(oracle):
     t = np.array([1., 2., 3.], dtype=np.float32)
     oracle.assign("ASSIGN_SUB", t, np.array([.5, .5, 4.], np.float32))
     np.testing.assert_array_equal(t, np.array([.5, 1.5, -1.], np.float32))
+
+
+# ---- the device RAND_UNIF stream -------------------------------------------
+
+# Known-answer vectors of the Random123 distribution (kat_vectors, philox4x32
+# with 10 rounds): counter words, key words, expected output words
+PHILOX_KAT = [
+    ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+    ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+    ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+     [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+]
+
+
+@pytest.mark.parametrize("counter,key,expect", PHILOX_KAT, ids=["zeros", "ones", "pi"])
+def test_philox_known_answers(oracle, counter, key, expect):
+    assert oracle.philox4x32_10(counter, key) == expect
+
+
+def test_rand_uniform_is_the_documented_function_of_the_generator_words(oracle):
+    """Element i takes word i%4 of block first+i/4 (double: two words of block
+    first+i/2); real results are the correctly rounded lo + u*(hi-lo); int32
+    results lo + ((word*(hi-lo+1)) >> 32).  Worked in exact rational /
+    integer arithmetic from the generator words."""
+    from fractions import Fraction
+    seed, first, n = 0x0123456789abcdef, (1 << 32) - 2, 23  # the block counter carries into its high word
+    key = [seed & 0xffffffff, seed >> 32]
+    rng = np.random.default_rng(0)
+
+    def words(block):
+        return oracle.philox4x32_10([block & 0xffffffff, block >> 32, 0, 0], key)
+
+    lo = rng.uniform(-3, 1, n).astype(np.float32)
+    hi = (lo + rng.uniform(0.5, 4, n)).astype(np.float32)
+    got = oracle.rand_uniform(lo, hi, seed, first)
+    for i in range(n):
+        u = Fraction(words(first + i // 4)[i % 4] >> 8, 1 << 24)
+        # fl(hi-lo) is what the multiply-add sees
+        exact = Fraction(float(lo[i])) + u * Fraction(float(np.float32(hi[i] - lo[i])))
+        assert abs(Fraction(float(got[i])) - exact) <= Fraction(float(np.spacing(np.abs(got[i])))) / 2
+
+    lo64 = rng.uniform(-3, 1, n)
+    hi64 = lo64 + rng.uniform(0.5, 4, n)
+    got = oracle.rand_uniform(lo64, hi64, seed, first)
+    for i in range(n):
+        w = words(first + i // 2)
+        u = Fraction(((w[2 * (i % 2) + 1] << 32) | w[2 * (i % 2)]) >> 11, 1 << 53)
+        exact = Fraction(float(lo64[i])) + u * Fraction(float(hi64[i] - lo64[i]))
+        assert abs(Fraction(float(got[i])) - exact) <= Fraction(float(np.spacing(np.abs(got[i])))) / 2
+
+    ilo = rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+    ihi = np.maximum(ilo, rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32))
+    ilo[0], ihi[0] = -2 ** 31, 2 ** 31 - 1   # the whole range
+    ilo[1], ihi[1] = 7, 7                    # one value
+    ilo[2], ihi[2] = 5, 4                    # empty range: lo
+    got = oracle.rand_uniform(ilo, ihi, seed, first)
+    for i in range(n):
+        if ihi[i] < ilo[i]:
+            assert got[i] == ilo[i]
+            continue
+        span = int(ihi[i]) - int(ilo[i]) + 1
+        assert int(got[i]) == int(ilo[i]) + ((words(first + i // 4)[i % 4] * span) >> 32)
+
+
+def test_rand_uniform_stream_properties(oracle):
+    n = 200000
+    lo, hi = np.full(n, -2.0, np.float32), np.full(n, 6.0, np.float32)
+    x = oracle.rand_uniform(lo, hi, 42)
+    assert x.min() >= -2.0 and x.max() < 6.0
+    # uniform on [-2, 6): mean 2, variance 64/12; 5 sigma of the estimators
+    assert abs(x.mean() - 2.0) < 5 * np.sqrt(64 / 12 / n)
+    assert abs(x.var() - 64 / 12) < 5 * np.sqrt(0.8 * (64 / 12) ** 2 / n)
+    # a later start continues the same stream; another seed is another stream
+    tail = oracle.rand_uniform(lo[:4000], hi[:4000], 42, first_block=1000)
+    np.testing.assert_array_equal(tail, x[4000:8000])
+    assert not np.array_equal(oracle.rand_uniform(lo, hi, 43), x)
+    dice = oracle.rand_uniform(np.full(n, 1, np.int32), np.full(n, 6, np.int32), 7)
+    counts = np.bincount(dice, minlength=7)
+    assert counts[0] == 0 and counts[1:].sum() == n
+    assert np.all(np.abs(counts[1:] - n / 6) < 5 * np.sqrt(n * 5 / 36))
