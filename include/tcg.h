@@ -340,6 +340,17 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const uint64_t img_lo[8], const uint64_t img_hi[8],
 	const uint64_t out_lo[8], const uint64_t out_hi[8],
 	const void* img, const void* kernel, void* out);
+/* tcg_conv_boxed for an image that was never laid out with its zero border:
+ * `box` holds only the elements inside [img_lo, img_hi), densely, in the same
+ * dim order. This is CONV(PAD(x), kernel) (cfg/tenncor/nn.yml:88-93,
+ * tenncor/eteq/backprop.hpp:372-399) computed from x itself: box = x,
+ * img_lo = the paddings before, img_hi = img_lo + shape of x. Results are
+ * those of tcg_conv_boxed on the padded image, bit for bit. */
+int tcg_conv_dense_box (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const uint64_t img_lo[8], const uint64_t img_hi[8],
+	const uint64_t out_lo[8], const uint64_t out_hi[8],
+	const void* box, const void* kernel, void* out);
 
 #ifdef __cplusplus
 }

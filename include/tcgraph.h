@@ -106,7 +106,9 @@ int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count);
  * a functor launched through its own operator, or
  * "group OP+OP+... leaves=L stores=S instrs=I" for elementwise functors sharing
  * a launch, or "swapped CONTRACT+PERMUTE" for a transposed matrix product
- * launched as the product with its operands exchanged; a last line "folded N" counts the functors that never hold a value
+ * launched as the product with its operands exchanged, or "padded PAD+CONV"
+ * ("padded PAD+CONV+SLICE" when only slices read the result) for a convolution
+ * computed from the operand of its PAD node; a last line "folded N" counts the functors that never hold a value
  * of their own. Returns the length the text needs (it is cut to `capacity`). */
 int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, size_t capacity, size_t* needed);
 

@@ -37,7 +37,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
-    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_capture_begin", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -124,6 +124,7 @@ def load():
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
+        "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_capture_begin": [vp],
         "tcg_capture_end": [vp, ctypes.POINTER(vp)],
         "tcg_capture_abort": [vp],
@@ -410,6 +411,13 @@ class Context:
         self._check(self.lib.tcg_conv_boxed(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
                                             len(r), _u64(r if r else [0]), ilo, ihi, olo, ohi, img, kernel, dst))
 
+    def conv_dense_box(self, dtype, imgshape, kshape, ranks, img_box, out_box, box, kernel, dst):
+        """conv_boxed with `box` holding only the elements inside img_box."""
+        r = [int(v) for v in ranks][:RANK_CAP]
+        olo, ohi = (_u64(out_box[0]), _u64(out_box[1])) if out_box else (None, None)
+        self._check(self.lib.tcg_conv_dense_box(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
+                                                len(r), _u64(r if r else [0]), _u64(img_box[0]), _u64(img_box[1]),
+                                                olo, ohi, box, kernel, dst))
 
     # ---- recorded launch sequences ----
     def capture_begin(self):

@@ -44,6 +44,7 @@ struct ConvPlan
 	int32_t ilo[8];      // image non-zero box
 	int32_t ihi[8];
 	uint64_t nwin = 1;   // outputs in the window
+	int64_t ioff0 = 0;   // image offset of coordinate 0 (negative when `img` holds the box only)
 };
 
 constexpr int CV_BLOCK = 256;
@@ -55,7 +56,7 @@ __global__ __launch_bounds__(CV_BLOCK) void conv_boxed_k (ConvPlan p,
 	uint64_t o = GROUP_PER_OUTPUT ? (uint64_t) blockIdx.x : (uint64_t) blockIdx.x * CV_BLOCK + threadIdx.x;
 	if (o >= p.nwin) { return; }
 	// output coordinate, and per image dim the clipped kernel range [k0, k0 + kr)
-	int64_t ibase = 0, obase = 0, kbase = 0;
+	int64_t ibase = p.ioff0, obase = 0, kbase = 0;
 	uint32_t kr[8];
 	uint64_t nterms = 1;
 	uint32_t rem = (uint32_t) o; // the host keeps nwin below 2^32
@@ -550,11 +551,12 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 
 extern "C" {
 
-int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+// dense_box: `img` holds only the elements inside [img_lo, img_hi), densely
+static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
 	const uint64_t img_lo[8], const uint64_t img_hi[8],
 	const uint64_t out_lo[8], const uint64_t out_hi[8],
-	const void* img, const void* kernel, void* out)
+	const void* img, const void* kernel, void* out, bool dense_box)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, imgshape && kshape && img && kernel && out && (ranks || nranks == 0), "tcg_conv: NULL pointer");
@@ -639,8 +641,8 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 			if (box[d] < imgshape[d] && d < first_cut) { first_cut = d; }
 		}
 		size_t esz = tcg_type_size(dtype);
-		bool compact = esz && box_elems > 0 && first_cut < last_sig && box_elems * 2 <= img_elems &&
-			box_elems * esz <= (1ull << 30);
+		bool compact = false == dense_box && esz && box_elems > 0 && first_cut < last_sig &&
+			box_elems * 2 <= img_elems && box_elems * esz <= (1ull << 30);
 		void* dense = nullptr;
 		if (compact)
 		{
@@ -651,6 +653,10 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 				if (dense) { tcg_free(ctx, dense, box_elems * esz); }
 				return rc;
 			}
+			img = dense;
+		}
+		if (compact || dense_box)
+		{
 			int64_t run = 1;
 			for (int d = 0; d < 8; ++d)
 			{
@@ -660,12 +666,21 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 				gp.istr[d] = run;
 				run *= (int64_t) box[d];
 			}
-			img = dense;
 		}
 		int rc = TCG_OK;
 		TCG_DISPATCH_TYPE(ctx, dtype, rc = conv_gemm_run<T>(ctx, dtype, gp, (const T*) img, (const T*) kernel, (T*) out));
 		if (dense) { tcg_free(ctx, dense, box_elems * esz); }
 		return rc;
+	}
+	if (dense_box)
+	{
+		int64_t run = 1;
+		for (int d = 0; d < 8; ++d)
+		{
+			p.istr[d] = run;
+			p.ioff0 -= (int64_t) p.ilo[d] * run;
+			run *= (int64_t) (p.ihi[d] - p.ilo[d]);
+		}
 	}
 	// few outputs with long sums: give each output a whole workgroup
 	bool group = p.nwin < (uint64_t) ctx->num_cus * 64 * 16 && max_terms >= 2048;
@@ -683,6 +698,28 @@ int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	}
 	TCG_LAUNCH_CHECK(ctx, "conv_boxed");
 	return TCG_OK;
+}
+
+int tcg_conv_boxed (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const uint64_t img_lo[8], const uint64_t img_hi[8],
+	const uint64_t out_lo[8], const uint64_t out_hi[8],
+	const void* img, const void* kernel, void* out)
+{
+	return conv_boxed_impl(ctx, dtype, imgshape, kshape, nranks, ranks, img_lo, img_hi, out_lo, out_hi,
+		img, kernel, out, false);
+}
+
+int tcg_conv_dense_box (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const uint64_t img_lo[8], const uint64_t img_hi[8],
+	const uint64_t out_lo[8], const uint64_t out_hi[8],
+	const void* box, const void* kernel, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, img_lo && img_hi, "tcg_conv_dense_box: the box is required");
+	return conv_boxed_impl(ctx, dtype, imgshape, kshape, nranks, ranks, img_lo, img_hi, out_lo, out_hi,
+		box, kernel, out, true);
 }
 
 int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],

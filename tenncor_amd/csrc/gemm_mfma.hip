@@ -37,17 +37,34 @@ struct GemmArgs
 
 // TA: A(m,k) at m + k*lda (M contiguous) instead of m*lda + k.
 // TB: B(k,n) at k + n*ldb (K contiguous) instead of k*ldb + n.
-template <int BM, int BN, bool TA, bool TB>
+// WGM: waves along M (2: waves 2x2, 4: waves 4x1 for narrow N).
+//
+// LDS layouts: an operand whose K runs contiguously in memory is kept
+// [row][k] with a pitch of BK+4 floats and read four k at a time (one 128-bit
+// read per four matrix instructions); an operand whose rows run contiguously
+// is kept [k][row] and read one float at a time, consecutive lanes on
+// consecutive banks.  Both are written with 128-bit stores straight from the
+// 128-bit global loads.  To make the four-at-a-time reads possible the two
+// lane halves of a matrix instruction (which supply k and k+1 of its K=2) take
+// k = 8*(j/4) + 4*half + j%4 in step j of a slab instead of 2j + half: the
+// order in which a slab's sixteen k are summed is a fixed permutation, the
+// same for every element.
+template <int BM, int BN, int WGM, bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 {
-	constexpr int WM = BM / 2, WN = BN / 2;   // wave tile
-	constexpr int TM = WM / 32, TN = WN / 32; // 32x32 accumulators per wave
-	constexpr int AP = BK + 1;                // As[m][k], odd pitch: conflict-free reads
-	constexpr int BP = BN + 4;                // Bs[k][n], 16-byte aligned rows
-	constexpr int A_VEC = BM * BK / 4 / 256;  // float4 per lane per slab
-	constexpr int B_VEC = BN * BK / 4 / 256;
-	__shared__ float As[2][BM * AP];
-	__shared__ __attribute__((aligned(16))) float Bs[2][BK * BP];
+	constexpr int WGN = 4 / WGM;
+	constexpr int WM = BM / WGM, WN = BN / WGN; // wave tile
+	constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 accumulators per wave
+	static_assert(WM % 32 == 0 && WN % 32 == 0 && TM >= 1 && TN >= 1, "wave tiles are made of 32x32 blocks");
+	constexpr int KP = BK + 4;                  // pitch of a [row][k] tile
+	constexpr int AP = TA ? BM + 4 : KP;
+	constexpr int BP = TB ? KP : BN + 4;
+	constexpr int A_SIZE = TA ? BK * AP : BM * AP;
+	constexpr int B_SIZE = TB ? BN * BP : BK * BP;
+	constexpr int A_CHUNKS = BM * BK / 4, B_CHUNKS = BN * BK / 4; // float4 per slab
+	constexpr int A_VEC = (A_CHUNKS + 255) / 256, B_VEC = (B_CHUNKS + 255) / 256;
+	__shared__ __attribute__((aligned(16))) float As[2][A_SIZE];
+	__shared__ __attribute__((aligned(16))) float Bs[2][B_SIZE];
 
 	// ---- which tile: XCD-aware, grouped order --------------------------------
 	const uint32_t split = blockIdx.x / g.total_tiles;
@@ -77,7 +94,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63, wave = tid >> 6;
-	const int wm = wave >> 1, wn = wave & 1;
+	const int wm = wave / WGN, wn = wave % WGN;
 	const int l32 = lane & 31, lh = lane >> 5;
 
 	f32x16 acc[TM][TN];
@@ -101,6 +118,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 		for (int v = 0; v < A_VEC; ++v)
 		{
 			int idx = tid + v * 256;
+			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
 			if constexpr (!TA)
 			{
 				// K contiguous: BK/4 lanes per row
@@ -120,6 +138,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 		for (int v = 0; v < B_VEC; ++v)
 		{
 			int idx = tid + v * 256;
+			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
 			if constexpr (!TB)
 			{
 				// N contiguous: BN/4 lanes per k
@@ -145,23 +164,23 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 		for (int v = 0; v < A_VEC; ++v)
 		{
 			int idx = tid + v * 256;
+			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
 			if constexpr (!TA)
 			{
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
-#pragma unroll
-				for (int e = 0; e < 4; ++e) { as[mm * AP + kq * 4 + e] = ra[v][e]; }
+				*reinterpret_cast<f32x4v*>(as + mm * AP + kq * 4) = ra[v];
 			}
 			else
 			{
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
-#pragma unroll
-				for (int e = 0; e < 4; ++e) { as[(mq * 4 + e) * AP + kk] = ra[v][e]; }
+				*reinterpret_cast<f32x4v*>(as + kk * AP + mq * 4) = ra[v];
 			}
 		}
 #pragma unroll
 		for (int v = 0; v < B_VEC; ++v)
 		{
 			int idx = tid + v * 256;
+			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
 			if constexpr (!TB)
 			{
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
@@ -170,8 +189,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 			else
 			{
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
-#pragma unroll
-				for (int e = 0; e < 4; ++e) { bs[(kq * 4 + e) * BP + nn] = rb[v][e]; }
+				*reinterpret_cast<f32x4v*>(bs + nn * BP + kq * 4) = rb[v];
 			}
 		}
 	};
@@ -184,23 +202,46 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 	{
 		const int buf = s & 1;
 		if (s + 1 < nslabs) { load_slab(k_begin + (s + 1) * BK); }
-		const float* as = As[buf] + (wm * WM + l32) * AP + lh;
-		const float* bs = Bs[buf] + lh * BP + wn * WN + l32;
+		const float* as = As[buf];
+		const float* bs = Bs[buf];
 #pragma unroll
-		for (int ks = 0; ks < BK / 2; ++ks)
+		for (int half = 0; half < BK / 8; ++half)
 		{
-			float a[TM], b[TN];
-#pragma unroll
-			for (int i = 0; i < TM; ++i) { a[i] = as[i * 32 * AP + ks * 2]; }
-#pragma unroll
-			for (int j = 0; j < TN; ++j) { b[j] = bs[ks * 2 * BP + j * 32]; }
+			const int kb = half * 8 + lh * 4; // this lane's four k of the half slab
+			f32x4v a[TM], b[TN];
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 			{
-#pragma unroll
-				for (int j = 0; j < TN; ++j)
+				const int row = wm * WM + i * 32 + l32;
+				if constexpr (!TA) { a[i] = *reinterpret_cast<const f32x4v*>(as + row * AP + kb); }
+				else
 				{
-					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+					for (int e = 0; e < 4; ++e) { a[i][e] = as[(kb + e) * AP + row]; }
+				}
+			}
+#pragma unroll
+			for (int j = 0; j < TN; ++j)
+			{
+				const int col = wn * WN + j * 32 + l32;
+				if constexpr (TB) { b[j] = *reinterpret_cast<const f32x4v*>(bs + col * BP + kb); }
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; ++e) { b[j][e] = bs[(kb + e) * BP + col]; }
+				}
+			}
+#pragma unroll
+			for (int e = 0; e < 4; ++e)
+			{
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+				{
+#pragma unroll
+					for (int j = 0; j < TN; ++j)
+					{
+						acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
+					}
 				}
 			}
 		}
@@ -245,7 +286,20 @@ __global__ __launch_bounds__(256) void gemm_split_sum_k (const float* __restrict
 	}
 }
 
-template <int BM, int BN>
+// the same sums for a densely stored C, four elements per lane
+__global__ __launch_bounds__(256) void gemm_split_sum_vec_k (const f32x4v* __restrict__ partial,
+	f32x4v* __restrict__ C, uint32_t splits, uint64_t per_split_vec)
+{
+	const uint64_t step = (uint64_t) gridDim.x * 256;
+	for (uint64_t i = (uint64_t) blockIdx.x * 256 + threadIdx.x; i < per_split_vec; i += step)
+	{
+		f32x4v acc = partial[i];
+		for (uint32_t s = 1; s < splits; ++s) { acc += partial[s * per_split_vec + i]; }
+		C[i] = acc;
+	}
+}
+
+template <int BM, int BN, int WGM = 2>
 int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1)
 {
 	GemmArgs g = base;
@@ -276,15 +330,24 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	}
 	else { splits = 1; }
 	const unsigned grid = g.total_tiles * splits;
-	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (!trans_a && trans_b) { gemm_mfma_k<BM,BN,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
-	else { gemm_mfma_k<BM,BN,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (!trans_a && trans_b) { gemm_mfma_k<BM,BN,WGM,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	else { gemm_mfma_k<BM,BN,WGM,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
 	if (g.partial)
 	{
 		uint64_t n = batch * g.M * g.N;
-		unsigned rgrid = tcg_grid(ctx, n, 256, 8);
-		gemm_split_sum_k<<<rgrid, 256, 0, ctx->stream>>>(g.partial, g.C, splits, g.M, g.N, (uint32_t) batch, g.ldc, g.batch_c);
+		bool dense = g.ldc == (int64_t) g.N && (batch == 1 || g.batch_c == (int64_t) g.M * g.N);
+		if (dense && n % 4 == 0 && tcg_aligned16(g.C))
+		{
+			unsigned rgrid = tcg_grid(ctx, n / 4, 256, 8);
+			gemm_split_sum_vec_k<<<rgrid, 256, 0, ctx->stream>>>((const f32x4v*) g.partial, (f32x4v*) g.C, splits, n / 4);
+		}
+		else
+		{
+			unsigned rgrid = tcg_grid(ctx, n, 256, 8);
+			gemm_split_sum_k<<<rgrid, 256, 0, ctx->stream>>>(g.partial, g.C, splits, g.M, g.N, (uint32_t) batch, g.ldc, g.batch_c);
+		}
 		tcg_free(ctx, g.partial, partial_bytes);
 	}
 	TCG_LAUNCH_CHECK(ctx, "gemm_mfma");
@@ -315,9 +378,18 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	g.batch_a = (int64_t) stride_a; g.batch_b = (int64_t) stride_b; g.batch_c = (int64_t) stride_c;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	*handled = true;
+	// narrow results (the column count of a convolution lowered to a product is
+	// its channel count): tiles as wide as N, so that no lane multiplies padding
+	const uint64_t cus = (uint64_t) ctx->num_cus;
+	if (N <= 32 && (M + 127) / 128 * batch >= cus)
+	{
+		if ((M + 255) / 256 * batch >= 2 * cus) { return launch<256,32,4>(ctx, g, batch, trans_a, trans_b); }
+		return launch<128,32,4>(ctx, g, batch, trans_a, trans_b);
+	}
+	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2>(ctx, g, batch, trans_a, trans_b); }
 	// small problems: smaller tiles so that the grid still covers the chip
 	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
-	if (big_tiles >= (uint64_t) ctx->num_cus) { return launch<128,128>(ctx, g, batch, trans_a, trans_b); }
+	if (big_tiles >= cus) { return launch<128,128>(ctx, g, batch, trans_a, trans_b); }
 	// still too few tiles for the chip and a long K: several workgroups share a
 	// tile, each summing a range of K, and a second kernel adds the ranges up
 	// in a fixed order (so that results do not depend on scheduling)

@@ -189,6 +189,8 @@ struct iEigen : public teq::iDeviceRef
 	/// The buffer a launch issued by someone else (a fused group) fills for
 	/// this node, with `ttl` reads to live; nullptr when the node cannot take one
 	virtual void* borrow_output (size_t, RTMemptrT&) { return nullptr; }
+	/// After borrow_output: the launch fills only part of the buffer
+	virtual void mark_partial (void) {}
 };
 
 /// Lifetime given to the node whose launch is being enqueued, and a flag the
@@ -239,6 +241,7 @@ struct CacheEigen final : public iPermEigen
 	}
 	void replayed (void) override { data_->replayed(); }
 	void* borrow_output (size_t ttl, RTMemptrT& memory) override { return data_->borrow_output(ttl, memory); }
+	void mark_partial (void) override { data_->mark_partial(); }
 private:
 	EigenptrT data_;
 };
@@ -453,6 +456,8 @@ struct HipOp final : public iTmpEigen<T>
 		partial_ = false;
 		return this->data_.get();
 	}
+
+	void mark_partial (void) override { partial_ = true; }
 
 private:
 	OpF op_;

@@ -436,12 +436,10 @@ inline void nonzero_box (const teq::iTensor& tens, Shape8& lo, Shape8& hi)
 	hi = shape8(tens.shape());
 }
 
-/// The part of `self`'s value its consumers read: when every consumer is a
-/// SLICE of it and the node is no evaluation target, the bounding box of
-/// those slices; otherwise everything (false)
-inline bool consumed_window (const Observable* self, const teq::Shape& outshape, Shape8& lo, Shape8& hi)
+/// The bounding box of the SLICEs reading `self`, false when anything else reads it
+inline bool slices_window (const Observable* self, const teq::Shape& outshape, Shape8& lo, Shape8& hi)
 {
-	if (nullptr == self || self->nsubs() == 0 || launch_scope().ttl != self->nsubs()) { return false; }
+	if (nullptr == self || self->nsubs() == 0) { return false; }
 	bool first = true;
 	for (Observable* sub : self->get_observables())
 	{
@@ -464,6 +462,16 @@ inline bool consumed_window (const Observable* self, const teq::Shape& outshape,
 		first = false;
 	}
 	return true;
+}
+
+/// The part of `self`'s value its consumers read: when every consumer is a
+/// SLICE of it and the node is no evaluation target, the bounding box of
+/// those slices; otherwise everything (false)
+inline bool consumed_window (const Observable* self, const teq::Shape& outshape, Shape8& lo, Shape8& hi)
+{
+	// a target is read in full
+	if (nullptr == self || launch_scope().ttl != self->nsubs()) { return false; }
+	return slices_window(self, outshape, lo, hi);
 }
 
 template <typename T>

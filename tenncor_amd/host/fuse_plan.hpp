@@ -48,17 +48,38 @@ struct SwappedContract final
 	std::vector<teq::iTensor*> reads;
 };
 
+/// CONV(PAD(x), kernel) where convolutions are all that read the PAD node:
+/// the correlation is computed from x itself, told where it sits inside the
+/// zero border, and the padded image is never laid out (conv2d and its
+/// gradients pad a singleton axis to 2n-1 before correlating,
+/// cfg/tenncor/nn.yml:88-93, tenncor/eteq/backprop.hpp:372-399)
+struct PaddedConv final
+{
+	Observable* node = nullptr;      ///< the CONV node
+	teq::iTensor* image = nullptr;   ///< operand of the PAD node
+	teq::iTensor* kernel = nullptr;
+	std::array<uint64_t,8> imgshape, kshape; ///< imgshape: the PAD node's
+	std::array<uint64_t,8> ilo, ihi; ///< where the operand sits in the padded image
+	bool windowed = false;           ///< only SLICEs read the result:
+	std::array<uint64_t,8> olo, ohi; ///< their bounding box
+	std::vector<uint64_t> ranks;
+	int dtype = 0;
+	std::vector<teq::iTensor*> reads;
+};
+
 struct FusionPlan final
 {
 	struct Step final
 	{
 		Observable* node = nullptr; ///< launched through its own closure, or
 		int group = -1;             ///< index into groups, or
-		int contract = -1;          ///< index into contracts
+		int contract = -1;          ///< index into contracts, or
+		int conv = -1;              ///< index into convs
 	};
 
 	std::vector<FusedGroup> groups;
 	std::vector<SwappedContract> contracts;
+	std::vector<PaddedConv> convs;
 	std::vector<Step> steps;
 	/// functors that are computed inside a group or folded into operand views
 	/// and therefore never hold a value of their own
@@ -73,6 +94,8 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory);
 
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
+
+void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 }
 

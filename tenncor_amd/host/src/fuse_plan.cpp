@@ -47,6 +47,8 @@ struct Node final
 	bool target = false;
 	bool absorbed = false;      // a VIEW no launch of its own computes
 	int swapped_from = -1;      // PERMUTE launched as the swapped product of this CONTRACT node
+	int padded_from = -1;       // CONV reading the operand of this PAD node in place of the padded image
+	bool through_conv = false;  // PAD that only such convolutions read
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
 	teq::TensptrsT arg_tens;
 	std::vector<int> consumers; // functors of this pass reading the node
@@ -164,14 +166,34 @@ struct Planner final
 			c.kind = VIEW;
 			c.absorbed = true;
 		}
+		// PAD of a plain value read by convolutions only, as their image: they
+		// read the value itself
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			Node& n = nodes_[i];
+			if (n.op != egen::PAD || n.kind != VIEW || n.target || n.consumers.empty()) { continue; }
+			bool convolved = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
+			{
+				const Node& conv = nodes_[c];
+				return conv.op == egen::CONV && conv.args.size() == 2 && conv.args[0] == (int) i &&
+					conv.args[1] != (int) i && conv.dtype == n.dtype;
+			});
+			Shape8 lo, hi, inner = shape8(n.arg_tens[0]->shape());
+			nonzero_box(*n.arg_tens[0], lo, hi);
+			bool plain = hi == inner && std::all_of(lo.begin(), lo.end(), [](uint64_t v) { return v == 0; });
+			if (false == convolved || false == plain) { continue; }
+			n.absorbed = true;
+			n.through_conv = true;
+			for (int c : n.consumers) { nodes_[c].padded_from = (int) i; }
+		}
 		// a view is folded away when everything that reads it can read through it
 		for (size_t i = nodes_.size(); i-- > 0;)
 		{
 			Node& n = nodes_[i];
-			if (n.kind != VIEW || n.target || n.consumers.empty() || n.op == egen::CONTRACT) { continue; }
+			if (n.kind != VIEW || n.target || n.consumers.empty() || n.op == egen::CONTRACT || n.through_conv) { continue; }
 			n.absorbed = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
 			{
-				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed);
+				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed && false == nodes_[c].through_conv);
 			});
 		}
 		for (Node& n : nodes_)
@@ -659,6 +681,7 @@ struct Planner final
 		FusionPlan plan;
 		std::vector<bool> done(nodes_.size(), false);
 		std::map<int,int> last_user; // folded view -> last group reading through it
+		std::map<int,int> last_conv; // PAD read in place -> last convolution of its operand
 		std::function<void(int)> visit = [&](int u)
 		{
 			u = find(u);
@@ -701,6 +724,33 @@ struct Planner final
 				step.contract = (int) plan.contracts.size();
 				plan.contracts.push_back(call);
 				plan.absorbed.push_back(c.f);
+				plan.steps.push_back(step);
+				return;
+			}
+			if (nodes_[u].kind != EW && nodes_[u].padded_from >= 0)
+			{
+				const Node& n = nodes_[u];
+				const Node& pad = nodes_[n.padded_from];
+				PaddedConv call;
+				call.node = n.f;
+				call.dtype = n.dtype;
+				call.image = pad.arg_tens[0].get();
+				call.kernel = n.arg_tens[1].get();
+				call.imgshape = pad.shape;
+				call.kshape = shape8(call.kernel->shape());
+				teq::RanksT order;
+				Packer<teq::RanksT>().unpack(order, *n.f);
+				for (size_t k = 0; k < std::min(order.size(), (size_t) teq::rank_cap); ++k) { call.ranks.push_back(order[k]); }
+				nonzero_box(*pad.f, call.ilo, call.ihi);
+				call.windowed = false == n.target && slices_window(n.f, n.f->shape(), call.olo, call.ohi);
+				if (n.args[1] >= 0 && false == (nodes_[n.args[1]].kind == VIEW && nodes_[n.args[1]].absorbed))
+				{
+					call.reads.push_back(call.kernel);
+				}
+				FusionPlan::Step step;
+				step.conv = (int) plan.convs.size();
+				last_conv[n.padded_from] = step.conv;
+				plan.convs.push_back(call);
 				plan.steps.push_back(step);
 				return;
 			}
@@ -757,6 +807,12 @@ struct Planner final
 		}
 		// a folded view counts one read of its operand, when the last launch
 		// that looks through it has been enqueued
+		for (auto& kv : last_conv)
+		{
+			const Node& pad = nodes_[kv.first];
+			plan.absorbed.push_back(pad.f);
+			if (pad.args[0] >= 0) { plan.convs[kv.second].reads.push_back(pad.arg_tens[0].get()); }
+		}
 		for (auto& kv : last_user)
 		{
 			const Node& v = nodes_[kv.first];
@@ -807,6 +863,23 @@ void launch_contract (const SwappedContract& call, const teq::TensSetT& targets,
 	if (nullptr == a || nullptr == b) { global::fatal("operand of a matrix product has no data"); }
 	hip_check(tcg_contract(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
 		(int) (call.pairs.size() / 2), call.pairs.data(), a, b, dst));
+	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
+}
+
+void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptrT& memory)
+{
+	Observable* out = call.node;
+	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
+	auto& ref = static_cast<iEigen&>(out->device());
+	void* dst = ref.borrow_output(ttl, memory);
+	if (nullptr == dst) { global::fatalf("%s cannot take a convolution", out->to_string().c_str()); }
+	const void* image = eigen_ref(*call.image).device_data();
+	const void* kernel = eigen_ref(*call.kernel).device_data();
+	if (nullptr == image || nullptr == kernel) { global::fatal("operand of a convolution has no data"); }
+	if (call.windowed) { ref.mark_partial(); }
+	hip_check(tcg_conv_dense_box(hip_context(), call.dtype, call.imgshape.data(), call.kshape.data(),
+		(int) call.ranks.size(), call.ranks.data(), call.ilo.data(), call.ihi.data(),
+		call.windowed ? call.olo.data() : nullptr, call.windowed ? call.ohi.data() : nullptr, image, kernel, dst));
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 

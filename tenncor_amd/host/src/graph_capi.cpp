@@ -364,6 +364,11 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 				ss << "swapped CONTRACT+PERMUTE\n";
 				continue;
 			}
+			if (step.conv >= 0)
+			{
+				ss << "padded PAD+CONV" << (plan.convs[step.conv].windowed ? "+SLICE" : "") << "\n";
+				continue;
+			}
 			auto& group = plan.groups[step.group];
 			ss << "group ";
 			for (size_t i = 0; i < group.members.size(); ++i)

@@ -209,6 +209,10 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 			{
 				device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0));
 			}
+			else if (step.conv >= 0)
+			{
+				launch_conv(fusion.convs[step.conv], targets, device.memory());
+			}
 			else if (step.contract >= 0)
 			{
 				launch_contract(fusion.contracts[step.contract], targets, device.memory());

@@ -399,6 +399,9 @@ GEMM_CASES = [
     # few tiles, long K: several workgroups share a tile (K split in ranges, last one ragged)
     (256, 768, 2048, 1, 0, 1), (256, 2048, 768, 1, 0, 0), (64, 96, 1000, 2, 1, 0), (36, 44, 4100, 1, 0, 0),
     (12, 32, 2048, 1, 0, 0), (24, 8, 1024, 1, 1, 0), (8, 20, 600, 3, 0, 1),
+    # tall with few columns (a convolution lowered to a product): tiles 32 or 64 columns wide
+    (33000, 32, 40, 1, 0, 0), (33000, 24, 40, 1, 1, 0), (131300, 32, 24, 1, 0, 1), (2100, 28, 52, 16, 1, 1),
+    (33000, 64, 40, 1, 0, 0), (33000, 40, 36, 1, 1, 1), (4200, 64, 72, 8, 0, 1),
     # off the matrix-core path: odd extents
     (33, 35, 17, 2, 0, 0), (33, 35, 17, 2, 1, 1),
 ]
@@ -589,6 +592,19 @@ def test_conv_as_matrix_product_equals_direct_kernels(ctx, oracle, which):
             # outside the window the destination keeps what it held
             untouched = results["direct"] == 777
             assert untouched.any() and (results["product"][untouched] == 777).all()
+        # the same correlations from the box alone (the image never laid out
+        # with its border): the same bits as from the padded image, by either route
+        box, _ = oracle.slice_(img, ishape, [[lo[d], hi[d] - lo[d]] for d in range(8)])
+        dbox = ctx.upload(box)
+        for route, env in (("direct", {"TCG_CONV_GEMM": "0"}), ("product", {"TCG_CONV_GEMM": "1", "TCG_CONV_CHUNK_ROWS": "128"})):
+            os.environ.update(env)
+            try:
+                out = ctx.upload(np.full(n_out, 777, dtype=np_dtype))
+                ctx.conv_dense_box(dt, ishape, kshape, ranks, ibox, obox, dbox.ptr, dker.ptr, out.ptr)
+                np.testing.assert_array_equal(out.get(), results[route])
+            finally:
+                for key in env:
+                    os.environ.pop(key, None)
 
 
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])

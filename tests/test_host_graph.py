@@ -271,8 +271,8 @@ def parse_plan(lines):
         elif kind == "group":
             ops, *fields = rest.split(" ")
             steps.append(("group", ops.split("+"), {k: int(v) for k, v in (f.split("=") for f in fields)}))
-        elif kind == "swapped":
-            steps.append(("swapped", rest.split("+"), {}))
+        elif kind in ("swapped", "padded"):
+            steps.append((kind, rest.split("+"), {}))
         else:
             steps.append(("folded", [], {"n": int(rest)}))
     return steps
@@ -347,3 +347,25 @@ def test_launch_plan_folds_views_and_splits_oversized_groups(g, api):
     outs = [api.mul(z, float(k + 2)) for k in range(10)]
     steps = [s for s in parse_plan(g.launch_plan(outs)) if s[0] == "group"]
     assert sum(s[2]["stores"] for s in steps) >= 10 and all(s[2]["stores"] <= 8 for s in steps)
+
+
+def test_launch_plan_reads_the_operand_of_a_pad_that_only_convolutions_read(g, api):
+    x = var(g, [2, 6, 5, 3], np.float32, "x")        # {C, W, H, B}
+    k = var(g, [4, 2, 3, 2], np.float32, "k")        # {O, C, KW, KH}
+    y = api.conv2d(x, k)
+    loss = api.reduce_sum(api.square(y))
+    dx, dk = g.derive(loss, [x, k])
+    lines = g.launch_plan([loss, dx, dk])
+    # forward, kernel gradient (both read PAD(x)) and image gradient (reads PAD of the
+    # upstream gradient; only one index of its result is sliced back out)
+    assert lines.count("padded PAD+CONV") == 2 and lines.count("padded PAD+CONV+SLICE") == 1
+    assert "node PAD" not in lines and "node CONV" not in lines
+    steps = parse_plan(lines)
+    alone = sum(1 for s in steps if s[0] in ("node", "swapped", "padded"))
+    stores = sum(s[2]["stores"] for s in steps if s[0] == "group")
+    assert alone + stores + steps[-1][2]["n"] == g.count_functors([loss, dx, dk])
+    # a padded image somebody else reads, or asks for, is laid out as before
+    padded = g.args(g.args(y)[0])[0]
+    assert g.opcode(padded) == "PAD"
+    lines = g.launch_plan([y, padded])
+    assert "node PAD" in lines and "node CONV" in lines and not any(l.startswith("padded") for l in lines)
