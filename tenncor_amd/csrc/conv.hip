@@ -17,6 +17,7 @@
 #include "tcg_internal.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace
 {
@@ -212,11 +213,7 @@ struct ConvGemmPlan
 
 // Per row / per summed index: image offset and, for the checked dims, the
 // coordinate relative to the box start (row part and summed part add up)
-struct ConvTabEntry
-{
-	int64_t off;
-	int32_t c[4];
-};
+using ConvTabEntry = tcg_conv_tab;
 
 constexpr int CG_BLOCK = 256;
 
@@ -475,6 +472,36 @@ bool conv_gemm_plan (const ConvPlan& c, ConvGemmPlan& g)
 	return true;
 }
 
+// How the matrix-core kernel can read A straight from the image: along which
+// index memory runs, and whether aligned groups of four along it are
+// contiguous, 16-byte aligned and inside or outside the box together
+void conv_operand_mode (const ConvGemmPlan& g, tcg_conv_operand& op)
+{
+	op.ncheck = g.ncheck;
+	for (int j = 0; j < 4; ++j) { op.check_ext[j] = j < g.ncheck ? g.check_ext[j] : 0; }
+	op.along_m = false;
+	op.vec4 = false;
+	int f = -1;
+	for (int d = 0; d < 8 && f < 0; ++d)
+	{
+		if (g.msize[d] > 1 || g.ssize[d] > 1) { f = d; }
+	}
+	if (f < 0 || g.istr[f] != 1 || g.is_col[f]) { return; }
+	op.along_m = g.msize[f] > 1;
+	bool checked = false;
+	for (int j = 0; j < g.ncheck; ++j) { checked = checked || g.check_dim[j] == f; }
+	uint32_t run = op.along_m ? g.msize[f] : g.ssize[f], other = op.along_m ? g.ssize[f] : g.msize[f];
+	bool vec = false == checked && run % 4 == 0 && other == 1 && (g.xlo[f] + g.slo[f]) % 4 == 0;
+	for (int d = 0; d < 8 && vec; ++d)
+	{
+		if (d == f || g.istr[d] % 4 == 0) { continue; }
+		// a dim with an odd stride may only add a constant multiple of four
+		int64_t fixed = g.is_col[d] ? g.ilo[d] : g.xlo[d] + g.slo[d];
+		vec = g.msize[d] == 1 && g.ssize[d] == 1 && (fixed * g.istr[d]) % 4 == 0;
+	}
+	op.vec4 = vec;
+}
+
 template <typename T>
 int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img, const T* ker, T* out)
 {
@@ -494,8 +521,10 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 	size_t rt_bytes = sizeof(ConvTabEntry) * (size_t) g.M, st_bytes = sizeof(ConvTabEntry) * (size_t) g.Sp;
 	void *A = nullptr, *B = nullptr, *C = nullptr, *RT = nullptr, *ST = nullptr;
 	const bool tables = g.ncheck >= 0;
-	int rc = tcg_alloc(ctx, a_bytes, &A);
-	if (rc == TCG_OK) { rc = tcg_alloc(ctx, b_bytes, &B); }
+	// fp32: the product reads A through the tables, nothing is gathered
+	const char* impl_env = getenv("TCG_CONV_IMPLICIT"); // "0": always materialise A (the parity reference)
+	bool implicit = std::is_same<T,float>::value && tables && !(impl_env && impl_env[0] == '0');
+	int rc = tcg_alloc(ctx, b_bytes, &B);
 	if (rc == TCG_OK) { rc = tcg_alloc(ctx, c_bytes, &C); }
 	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, rt_bytes, &RT); }
 	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, st_bytes, &ST); }
@@ -509,9 +538,44 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			conv_tables_k<<<(longest + CG_BLOCK - 1) / CG_BLOCK, CG_BLOCK, 0, ctx->stream>>>(g,
 				(ConvTabEntry*) RT, (ConvTabEntry*) ST);
 		}
+		tcg_conv_operand operand;
+		if (implicit)
+		{
+			conv_operand_mode(g, operand);
+			// gathering element by element inside the product is slower than
+			// materialising A with the coalesced gather kernel (measured on the
+			// image gradient of a 5x5 convolution: 285 vs 300 us, and 214 vs 76 us
+			// on a kernel gradient with 25 rows): only the 128-bit form is used
+			const char* scalar_env = getenv("TCG_CONV_IMPLICIT_SCALAR"); // "1": use it all the same (tests)
+			implicit = operand.vec4 || (scalar_env && scalar_env[0] == '1');
+		}
 		for (uint32_t m0 = 0; m0 < g.M && rc == TCG_OK; m0 += chunk)
 		{
 			uint32_t rows = g.M - m0 < chunk ? g.M - m0 : chunk;
+			if constexpr (std::is_same<T,float>::value)
+			{
+				if (implicit)
+				{
+					operand.rows = (const ConvTabEntry*) RT + m0;
+					operand.sums = (const ConvTabEntry*) ST;
+					bool handled = false;
+					rc = tcg_gemm_f32_mfma_conv(ctx, rows, g.Np, g.S, img, operand, (const float*) B, g.Np,
+						(float*) C, g.Np, &handled);
+					if (rc != TCG_OK) { break; }
+					if (handled)
+					{
+						grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
+						conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+						continue;
+					}
+					implicit = false; // shapes the matrix-core kernel does not take: gather as below
+				}
+			}
+			if (nullptr == A)
+			{
+				rc = tcg_alloc(ctx, a_bytes, &A);
+				if (rc != TCG_OK) { break; }
+			}
 			if (tables)
 			{
 				dim3 tgrid((g.Sp + CG_BLOCK - 1) / CG_BLOCK, (rows + CG_ROWS - 1) / CG_ROWS);

@@ -33,7 +33,23 @@ struct GemmArgs
 	// with more than one range the C tile goes to partial[range][batch][M][N]
 	uint32_t k_per_split;
 	float* partial;
+	// A read through a convolution's tables (IMPL != 0): A is the image
+	const tcg_conv_tab* rows;
+	const tcg_conv_tab* sums;
+	uint32_t check_ext[4];
+	int ncheck;
 };
+
+__device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_tab& row, const tcg_conv_tab& col)
+{
+	bool inside = true;
+#pragma unroll
+	for (int j = 0; j < 4; ++j)
+	{
+		if (j < g.ncheck) { inside = inside && (uint32_t) (row.c[j] + col.c[j]) < g.check_ext[j]; }
+	}
+	return inside;
+}
 
 // TA: A(m,k) at m + k*lda (M contiguous) instead of m*lda + k.
 // TB: B(k,n) at k + n*ldb (K contiguous) instead of k*ldb + n.
@@ -49,7 +65,13 @@ struct GemmArgs
 // k = 8*(j/4) + 4*half + j%4 in step j of a slab instead of 2j + half: the
 // order in which a slab's sixteen k are summed is a fixed permutation, the
 // same for every element.
-template <int BM, int BN, int WGM, bool TA, bool TB>
+//
+// IMPL: 0 = A is a matrix in memory.  1, 2 = A[m][k] = image[rows[m].off +
+// sums[k].off] or zero (a convolution's operand, never materialised); TA then
+// says which index runs along memory (consecutive m, or consecutive k).
+// 1: aligned groups of four along that index are contiguous and exist or not
+// together (one 128-bit load); 2: element by element.
+template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL>
 __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 {
 	constexpr int WGN = 4 / WGM;
@@ -112,6 +134,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 	f32x4v ra[A_VEC], rb[B_VEC];
 	const f32x4v zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
+	// the table rows a lane gathers from stay the same for every slab
+	constexpr int ROW_ENTS = IMPL == 0 ? 1 : (!TA ? A_VEC : (IMPL == 1 ? 1 : 4));
+	tcg_conv_tab rowent[ROW_ENTS];
+	if constexpr (IMPL != 0)
+	{
+		static_assert(256 % (BM / 4) == 0, "a lane keeps its rows from slab to slab");
+#pragma unroll
+		for (int e = 0; e < ROW_ENTS; ++e)
+		{
+			uint32_t m = !TA ? m0 + (tid + e * 256) / (BK / 4) : m0 + (tid % (BM / 4)) * 4 + e;
+			rowent[e] = g.rows[m < g.M ? m : g.M - 1];
+		}
+	}
+
 	auto load_slab = [&] (uint32_t k0)
 	{
 #pragma unroll
@@ -119,7 +155,65 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 		{
 			int idx = tid + v * 256;
 			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
-			if constexpr (!TA)
+			if constexpr (IMPL != 0 && !TA)
+			{
+				// one row, four consecutive k
+				int mm = idx / (BK / 4), kq = idx % (BK / 4);
+				uint32_t m = m0 + mm, k = k0 + kq * 4;
+				f32x4v val = zero4;
+				if (m < g.M && k < k_end)
+				{
+					if constexpr (IMPL == 1)
+					{
+						const tcg_conv_tab col = g.sums[k];
+						if (conv_inside(g, rowent[v], col))
+						{
+							val = *reinterpret_cast<const f32x4v*>(A + rowent[v].off + col.off);
+						}
+					}
+					else
+					{
+#pragma unroll
+						for (int e = 0; e < 4; ++e)
+						{
+							if (k + e < k_end)
+							{
+								const tcg_conv_tab col = g.sums[k + e];
+								if (conv_inside(g, rowent[v], col)) { val[e] = A[rowent[v].off + col.off]; }
+							}
+						}
+					}
+				}
+				ra[v] = val;
+			}
+			else if constexpr (IMPL != 0)
+			{
+				// one k, four consecutive rows
+				int kk = idx / (BM / 4), mq = idx % (BM / 4);
+				uint32_t m = m0 + mq * 4, k = k0 + kk;
+				f32x4v val = zero4;
+				if (m < g.M && k < k_end)
+				{
+					const tcg_conv_tab col = g.sums[k];
+					if constexpr (IMPL == 1)
+					{
+						if (conv_inside(g, rowent[0], col))
+						{
+							val = *reinterpret_cast<const f32x4v*>(A + rowent[0].off + col.off);
+						}
+					}
+					else
+					{
+#pragma unroll
+						for (int e = 0; e < 4; ++e)
+						{
+							if (m + e < g.M && conv_inside(g, rowent[e], col)) { val[e] = A[rowent[e].off + col.off]; }
+						}
+					}
+				}
+				ra[v] = val;
+			}
+			else if constexpr (!TA)
 			{
 				// K contiguous: BK/4 lanes per row
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
@@ -299,7 +393,7 @@ __global__ __launch_bounds__(256) void gemm_split_sum_vec_k (const f32x4v* __res
 	}
 }
 
-template <int BM, int BN, int WGM = 2>
+template <int BM, int BN, int WGM, int IMPL>
 int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1)
 {
 	GemmArgs g = base;
@@ -330,10 +424,14 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	}
 	else { splits = 1; }
 	const unsigned grid = g.total_tiles * splits;
-	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (!trans_a && trans_b) { gemm_mfma_k<BM,BN,WGM,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
-	else { gemm_mfma_k<BM,BN,WGM,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if constexpr (IMPL == 0)
+	{
+		if (!trans_a) { gemm_mfma_k<BM,BN,WGM,false,true,0><<<grid, 256, 0, ctx->stream>>>(g); }
+		else { gemm_mfma_k<BM,BN,WGM,true,true,0><<<grid, 256, 0, ctx->stream>>>(g); }
+	}
+	else { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
 	if (g.partial)
 	{
 		uint64_t n = batch * g.M * g.N;
@@ -352,6 +450,34 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	}
 	TCG_LAUNCH_CHECK(ctx, "gemm_mfma");
 	return TCG_OK;
+}
+
+// Tile shapes by problem shape
+template <int IMPL>
+int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int trans_b)
+{
+	const uint64_t M = g.M, N = g.N, K = g.K;
+	// narrow results (the column count of a convolution lowered to a product is
+	// its channel count): tiles as wide as N, so that no lane multiplies padding
+	const uint64_t cus = (uint64_t) ctx->num_cus;
+	if (N <= 32 && (M + 127) / 128 * batch >= cus)
+	{
+		if ((M + 255) / 256 * batch >= 2 * cus) { return launch<256,32,4,IMPL>(ctx, g, batch, trans_a, trans_b); }
+		return launch<128,32,4,IMPL>(ctx, g, batch, trans_a, trans_b);
+	}
+	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
+	// small problems: smaller tiles so that the grid still covers the chip
+	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
+	if (big_tiles >= cus) { return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
+	// still too few tiles for the chip and a long K: several workgroups share a
+	// tile, each summing a range of K, and a second kernel adds the ranges up
+	// in a fixed order (so that results do not depend on scheduling)
+	uint64_t tiles = ((M + 63) / 64) * ((N + 63) / 64) * batch;
+	uint64_t splits = 2 * (uint64_t) ctx->num_cus / tiles;
+	if (splits > K / 64) { splits = K / 64; }
+	if (splits > 32) { splits = 32; }
+	if (splits < 2 || batch >= (1ull << 16)) { splits = 1; }
+	return launch<64,64,2,IMPL>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
 }
 
 } // namespace
@@ -377,26 +503,32 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	g.lda = (int64_t) lda; g.ldb = (int64_t) ldb; g.ldc = (int64_t) ldc;
 	g.batch_a = (int64_t) stride_a; g.batch_b = (int64_t) stride_b; g.batch_c = (int64_t) stride_c;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
+	g.rows = g.sums = nullptr;
+	g.ncheck = 0;
 	*handled = true;
-	// narrow results (the column count of a convolution lowered to a product is
-	// its channel count): tiles as wide as N, so that no lane multiplies padding
-	const uint64_t cus = (uint64_t) ctx->num_cus;
-	if (N <= 32 && (M + 127) / 128 * batch >= cus)
-	{
-		if ((M + 255) / 256 * batch >= 2 * cus) { return launch<256,32,4>(ctx, g, batch, trans_a, trans_b); }
-		return launch<128,32,4>(ctx, g, batch, trans_a, trans_b);
-	}
-	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2>(ctx, g, batch, trans_a, trans_b); }
-	// small problems: smaller tiles so that the grid still covers the chip
-	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
-	if (big_tiles >= cus) { return launch<128,128>(ctx, g, batch, trans_a, trans_b); }
-	// still too few tiles for the chip and a long K: several workgroups share a
-	// tile, each summing a range of K, and a second kernel adds the ranges up
-	// in a fixed order (so that results do not depend on scheduling)
-	uint64_t tiles = ((M + 63) / 64) * ((N + 63) / 64) * batch;
-	uint64_t splits = 2 * (uint64_t) ctx->num_cus / tiles;
-	if (splits > K / 64) { splits = K / 64; }
-	if (splits > 32) { splits = 32; }
-	if (splits < 2 || batch >= (1ull << 16)) { splits = 1; }
-	return launch<64,64>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
+	return dispatch<0>(ctx, g, batch, trans_a, trans_b);
+}
+
+int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
+	const float* image, const tcg_conv_operand& op, const float* B, uint64_t ldb,
+	float* C, uint64_t ldc, bool* handled)
+{
+	*handled = false;
+	bool ok = M >= 8 && N >= 8 && S >= 8 && ((M >= 32 && N >= 32) || S >= 512) &&
+		M < (1ull << 31) && N < (1ull << 31) && S < (1ull << 31) &&
+		tcg_aligned16(B) && ldb % 4 == 0 && N % 4 == 0 && op.rows && op.sums && op.ncheck >= 0 && op.ncheck <= 4 &&
+		(false == op.vec4 || (tcg_aligned16(image) && (op.along_m ? M : S) % 4 == 0));
+	if (!ok) { return TCG_OK; }
+	GemmArgs g;
+	g.A = image; g.B = B; g.C = C;
+	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) S;
+	g.lda = 0; g.ldb = (int64_t) ldb; g.ldc = (int64_t) ldc;
+	g.batch_a = g.batch_b = g.batch_c = 0;
+	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
+	g.rows = op.rows;
+	g.sums = op.sums;
+	g.ncheck = op.ncheck;
+	for (int j = 0; j < 4; ++j) { g.check_ext[j] = op.check_ext[j]; }
+	*handled = true;
+	return op.vec4 ? dispatch<1>(ctx, g, 1, op.along_m, 0) : dispatch<2>(ctx, g, 1, op.along_m, 0);
 }

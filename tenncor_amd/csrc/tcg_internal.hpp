@@ -108,6 +108,33 @@ static inline bool tcg_aligned16 (const void* p)
 	return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
 
+// A convolution lowered to a matrix product reads A[m][s] = image[rows[m].off +
+// sums[s].off], or zero when, for some j < ncheck, rows[m].c[j] + sums[s].c[j]
+// falls outside [0, check_ext[j]) (the element lies in the zero border)
+struct tcg_conv_tab
+{
+	int64_t off;
+	int32_t c[4];
+};
+
+struct tcg_conv_operand
+{
+	const tcg_conv_tab* rows = nullptr;
+	const tcg_conv_tab* sums = nullptr;
+	uint32_t check_ext[4] = {0, 0, 0, 0};
+	int ncheck = 0;
+	// which index runs along memory (consecutive m, or consecutive s), and whether
+	// aligned groups of four of them are contiguous and inside or outside together
+	bool along_m = false;
+	bool vec4 = false;
+};
+
+// C[m][n] = sum_s A[m][s] B[s][n] with A read through `op` (never materialised);
+// *handled = false when the shapes do not fit the matrix-core kernel
+int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
+	const float* image, const tcg_conv_operand& op, const float* B, uint64_t ldb,
+	float* C, uint64_t ldc, bool* handled);
+
 // Number of workgroups for a streaming kernel: enough to cover `work` items,
 // capped at a multiple of the CU count so that a grid-stride loop takes over
 static inline unsigned tcg_grid (const tcg_ctx* ctx, uint64_t work_items,

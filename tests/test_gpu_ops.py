@@ -607,6 +607,53 @@ def test_conv_as_matrix_product_equals_direct_kernels(ctx, oracle, which):
                     os.environ.pop(key, None)
 
 
+@pytest.mark.parametrize("which", ["forward", "image_gradient", "kernel_gradient"])
+@pytest.mark.parametrize("channels", [(8, 32), (6, 36)], ids=["groups_of_four", "element_by_element"])
+def test_conv_product_reading_the_image_in_place(ctx, oracle, which, channels):
+    """fp32 convolutions whose matrix product gathers its left operand from the
+    image while multiplying (nothing materialised), with channel counts that
+    allow 128-bit gathers and ones that do not, against the same product with
+    the operand materialised first and against the direct kernels (1e-4).
+    Elements outside the box hold garbage that must never be read."""
+    from tenncor_amd import capi
+    C, O = channels
+    ishape, kshape, ranks, ibox, obox = conv2d_idiom_cases(C=C, W=15, H=13, B=12, O=O, KW=3, KH=4)[which]
+    rng = np.random.default_rng(seed_of("convimplicit", which, C))
+    n_img, n_ker = oracle.n_elems(ishape), oracle.n_elems(kshape)
+    n_out = oracle.n_elems(oracle.conv_shape(ishape, kshape, ranks))
+    lo, hi = ibox
+    img = rng.uniform(-1, 1, n_img).astype(np.float32)
+    ker = rng.uniform(-1, 1, n_ker).astype(np.float32)
+    box, _ = oracle.slice_(img, ishape, [[lo[d], hi[d] - lo[d]] for d in range(8)])
+    inside = np.ones(ishape[::-1], dtype=bool)
+    for d in range(8):
+        idx = np.arange(ishape[d])
+        shape = [1] * 8
+        shape[7 - d] = ishape[d]
+        inside &= ((idx >= lo[d]) & (idx < hi[d])).reshape(shape)
+    img[~inside.reshape(-1)] = 12345
+    dimg, dbox, dker = ctx.upload(img), ctx.upload(box), ctx.upload(ker)
+    results = {}
+    # gathers that cannot be 128 bits wide are only taken on request (they are slower than materialising)
+    routes = (("direct", {"TCG_CONV_GEMM": "0"}), ("materialised", {"TCG_CONV_IMPLICIT": "0"}),
+              ("in_place", {"TCG_CONV_IMPLICIT_SCALAR": "1"}),
+              ("in_place_chunked", {"TCG_CONV_IMPLICIT_SCALAR": "1", "TCG_CONV_CHUNK_ROWS": "192"}))
+    for route, env in routes:
+        os.environ.update(env)
+        try:
+            out = ctx.upload(np.full(n_out, 777, dtype=np.float32))
+            ctx.conv_boxed(capi.FLOAT, ishape, kshape, ranks, ibox, obox, dimg.ptr, dker.ptr, out.ptr)
+            results[route] = out.get()
+            out = ctx.upload(np.full(n_out, 777, dtype=np.float32))
+            ctx.conv_dense_box(capi.FLOAT, ishape, kshape, ranks, ibox, obox, dbox.ptr, dker.ptr, out.ptr)
+            np.testing.assert_array_equal(out.get(), results[route])
+        finally:
+            for key in env:
+                os.environ.pop(key, None)
+    for route in ("materialised", "in_place", "in_place_chunked"):
+        assert_acc_close(results[route], results["direct"])
+
+
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
 def test_pad_interior_writes_the_operand_and_nothing_else(ctx, oracle, np_dtype):
     """tcg_pad_interior against PAD: equal to the oracle's padded tensor inside
