@@ -388,7 +388,21 @@ __global__ __launch_bounds__(256) void gemm_split_sum_vec_k (const f32x4v* __res
 	for (uint64_t i = (uint64_t) blockIdx.x * 256 + threadIdx.x; i < per_split_vec; i += step)
 	{
 		f32x4v acc = partial[i];
-		for (uint32_t s = 1; s < splits; ++s) { acc += partial[s * per_split_vec + i]; }
+		// eight loads in flight, added in range order
+		for (uint32_t s0 = 1; s0 < splits; s0 += 8)
+		{
+			f32x4v v[8];
+#pragma unroll
+			for (uint32_t j = 0; j < 8; ++j)
+			{
+				if (s0 + j < splits) { v[j] = partial[(s0 + j) * per_split_vec + i]; }
+			}
+#pragma unroll
+			for (uint32_t j = 0; j < 8; ++j)
+			{
+				if (s0 + j < splits) { acc += v[j]; }
+			}
+		}
 		C[i] = acc;
 	}
 }
