@@ -383,7 +383,7 @@ def main():
     ap.add_argument("--no-graphs", action="store_true", help="skip the whole-graph side metrics (configs 1, 4, 5)")
     ap.add_argument("--graph-config", type=int, choices=[1, 4, 5], default=None,
                     help="time only this whole-graph configuration and print its line (for profiling)")
-    ap.add_argument("--evaluator", choices=["plain", "replay", "replay_unfused"], default="replay")
+    ap.add_argument("--evaluator", choices=["plain", "replay", "replay_launches", "replay_unfused"], default="replay")
     ap.add_argument("--reps", type=int, default=20, help="timed evaluations with --graph-config 4 or 5")
     ap.add_argument("--optimize", action="store_true",
                     help="with --graph-config: clean the graph up first (duplicates merged, constants folded, conversions)")

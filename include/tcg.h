@@ -130,6 +130,21 @@ typedef struct tcg_graph tcg_graph;
 int tcg_capture_begin (tcg_ctx* ctx);
 int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out);
 int tcg_capture_abort (tcg_ctx* ctx);
+/* The same for a pass over a SMALL graph (a dense layer on a batch of three:
+ * tensors of a few dozen elements), whose cost is being launched at all: the
+ * sequence is recorded as the steps of ONE kernel, run by a single workgroup
+ * with a barrier between steps, and tcg_graph_launch enqueues that one kernel.
+ * Entry points that can be steps: tcg_ew_fusedx, tcg_ew_unary/binary/nary/
+ * select, tcg_assign, tcg_reduce, tcg_contract, tcg_matmul without batch, and
+ * tcg_extend/permute/slice/pad/reverse/stride (gathers into a dense result).
+ * Elementwise steps compute exactly what their own launch computes;
+ * contractions sum each output in ascending order of the summed index with a
+ * fused multiply-add (the order of the generic product kernel), reductions
+ * fold each output in ascending index order. Anything else, or more work than
+ * one workgroup does in microseconds, fails with TCG_ERR_UNSUPPORTED (at the
+ * call or at tcg_capture_end): the caller aborts and records with
+ * tcg_capture_begin instead. */
+int tcg_capture_begin_small (tcg_ctx* ctx);
 int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph);
 int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr);
 int tcg_graph_stats (const tcg_graph* graph, uint64_t* nodes, uint64_t* arena_bytes);

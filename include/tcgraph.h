@@ -59,11 +59,18 @@ int tcr_sync (tcr_graph* g);
  * process uses from now on. TCR_EVAL_PLAIN is teq::Evaluator, the node-by-node
  * walk; TCR_EVAL_REPLAY records the launches of a set of targets the second
  * time it is evaluated and enqueues the recording as a whole afterwards, with
- * elementwise functors that feed one another computed in shared launches;
+ * elementwise functors that feed one another computed in shared launches, and
+ * the whole pass of a graph of small tensors (4096 elements at most each) as
+ * the steps of one kernel (tcg_capture_begin_small: sums then run in index
+ * order, equal to the walk's within the tolerance of reductions and
+ * contractions rather than bit for bit);
+ * TCR_EVAL_REPLAY_LAUNCHES is the same without such single-kernel passes:
+ * every value equals the walk's bit for bit;
  * TCR_EVAL_REPLAY_UNFUSED records one launch per functor, as the walk issues. */
 #define TCR_EVAL_PLAIN 0
 #define TCR_EVAL_REPLAY 1
 #define TCR_EVAL_REPLAY_UNFUSED 2
+#define TCR_EVAL_REPLAY_LAUNCHES 3
 int tcr_set_evaluator (int kind);
 /* Counters of the replaying evaluator (zeros under TCR_EVAL_PLAIN):
  * out[0] passes walked node by node, out[1] recordings made, out[2] passes

@@ -37,7 +37,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
-    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -128,6 +128,7 @@ def load():
         "tcg_capture_begin": [vp],
         "tcg_capture_end": [vp, ctypes.POINTER(vp)],
         "tcg_capture_abort": [vp],
+        "tcg_capture_begin_small": [vp],
         "tcg_graph_launch": [vp, vp],
         "tcg_graph_claim": [vp, vp, vp],
         "tcg_graph_stats": [vp, u64p, u64p],
@@ -420,8 +421,12 @@ class Context:
                                                 olo, ohi, box, kernel, dst))
 
     # ---- recorded launch sequences ----
-    def capture_begin(self):
-        self._check(self.lib.tcg_capture_begin(self.handle))
+    def capture_begin(self, small=False):
+        """small: record the sequence as the steps of one kernel."""
+        if small:
+            self._check(self.lib.tcg_capture_begin_small(self.handle))
+        else:
+            self._check(self.lib.tcg_capture_begin(self.handle))
 
     def capture_end(self):
         g = ctypes.c_void_p()

@@ -467,12 +467,56 @@ int fused_launch (tcg_ctx* ctx, const FusedProgram& prog, const void* const* lea
 
 extern "C" {
 
+// While a sequence is recorded as one kernel, an elementwise node is a group of one
+static int small_elementwise (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
+	const void* const* ins, void* out)
+{
+	if (nargs > TCG_FX_MAX_LEAVES) { return tcg_small_unsupported(ctx, "an elementwise node with that many operands"); }
+	uint64_t shape[8] = {n, 1, 1, 1, 1, 1, 1, 1};
+	tcg_fx_leaf leaves[TCG_FX_MAX_LEAVES];
+	memset(leaves, 0, sizeof(leaves));
+	for (int k = 0; k < nargs; ++k)
+	{
+		leaves[k].ptr = ins[k];
+		leaves[k].stride[0] = 1;
+		for (int d = 0; d < 8; ++d) { leaves[k].hi[d] = shape[d]; }
+	}
+	tcg_fx_instr program[TCG_FX_MAX_LEAVES + 1];
+	memset(program, 0, sizeof(program));
+	int ninstrs = 0;
+	auto emit = [&](int op, int a, int b, int c)
+	{
+		tcg_fx_instr& ins = program[ninstrs++];
+		ins.opcode = (uint8_t) op;
+		ins.a = (uint8_t) a;
+		ins.b = (uint8_t) b;
+		ins.c = (uint8_t) c;
+		ins.dst = TCG_FX_REG0;
+	};
+	if (opcode == TCG_SELECT) { emit(opcode, TCG_FX_LEAF0, TCG_FX_LEAF0 + 1, TCG_FX_LEAF0 + 2); }
+	else if (opcode == TCG_ASSIGN) { ninstrs = 0; } // the source is stored as it is
+	else if (nargs == 1) { emit(opcode, TCG_FX_LEAF0, TCG_FX_NONE, TCG_FX_NONE); }
+	else
+	{
+		emit(opcode, TCG_FX_LEAF0, TCG_FX_LEAF0 + 1, TCG_FX_NONE);
+		for (int k = 2; k < nargs; ++k) { emit(opcode, TCG_FX_REG0, TCG_FX_LEAF0 + k, TCG_FX_NONE); }
+	}
+	tcg_fx_instr& store = program[ninstrs++];
+	store.opcode = TCG_FX_STORE;
+	store.a = (uint8_t) (opcode == TCG_ASSIGN ? TCG_FX_LEAF0 : TCG_FX_REG0);
+	store.b = store.c = TCG_FX_NONE;
+	store.dst = 0;
+	void* outs[1] = {out};
+	return tcg_ew_fusedx(ctx, dtype, shape, nargs, leaves, ninstrs, program, 1, outs);
+}
+
 int tcg_ew_unary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, const void* in, void* out)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, is_unary_op(opcode), "tcg_ew_unary: opcode %d is not a unary elementwise op", opcode);
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, in && out, "tcg_ew_unary: NULL pointer");
+	if (tcg_small_mode(ctx)) { return small_elementwise(ctx, opcode, dtype, n, 1, &in, out); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return unary_impl<T>(ctx, opcode, n, (const T*) in, (T*) out));
 	return TCG_OK;
 }
@@ -484,6 +528,11 @@ int tcg_ew_binary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
 	TCG_REQUIRE(ctx, is_binary_op(opcode), "tcg_ew_binary: opcode %d is not a binary elementwise op", opcode);
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, a && b && out, "tcg_ew_binary: NULL pointer");
+	if (tcg_small_mode(ctx))
+	{
+		const void* ins[2] = {a, b};
+		return small_elementwise(ctx, opcode, dtype, n, 2, ins, out);
+	}
 	TCG_DISPATCH_TYPE(ctx, dtype, return binary_impl<T>(ctx, opcode, n, (const T*) a, (const T*) b, (T*) out));
 	return TCG_OK;
 }
@@ -497,6 +546,7 @@ int tcg_ew_nary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
 	if (n == 0) { return TCG_OK; }
 	for (int i = 0; i < nargs; ++i) { TCG_REQUIRE(ctx, ins[i], "tcg_ew_nary: operand %d is NULL", i); }
 	TCG_REQUIRE(ctx, out, "tcg_ew_nary: NULL output");
+	if (tcg_small_mode(ctx)) { return small_elementwise(ctx, opcode, dtype, n, nargs, ins, out); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return nary_impl<T>(ctx, opcode, n, nargs, ins, (T*) out));
 	return TCG_OK;
 }
@@ -507,6 +557,11 @@ int tcg_ew_select (tcg_ctx* ctx, int dtype, uint64_t n, const void* cond,
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, cond && then && otherwise && out, "tcg_ew_select: NULL pointer");
+	if (tcg_small_mode(ctx))
+	{
+		const void* ins[3] = {cond, then, otherwise};
+		return small_elementwise(ctx, TCG_SELECT, dtype, n, 3, ins, out);
+	}
 	unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
 	TCG_DISPATCH_TYPE(ctx, dtype, (ew_select_k<T><<<grid, EW_BLOCK, 0, ctx->stream>>>(
 		(const T*) cond, (const T*) then, (const T*) otherwise, (T*) out, n)));
@@ -529,6 +584,13 @@ int tcg_assign (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, void* target, c
 	TCG_REQUIRE(ctx, opcode >= TCG_ASSIGN && opcode <= TCG_ASSIGN_DIV, "tcg_assign: opcode %d is not an ASSIGN op", opcode);
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, target && source, "tcg_assign: NULL pointer");
+	if (tcg_small_mode(ctx))
+	{
+		if (opcode == TCG_ASSIGN) { return small_elementwise(ctx, TCG_ASSIGN, dtype, n, 1, &source, target); }
+		const int fold[] = {TCG_ADD, TCG_SUB, TCG_MUL, TCG_DIV};
+		const void* ins[2] = {target, source};
+		return small_elementwise(ctx, fold[opcode - TCG_ASSIGN_ADD], dtype, n, 2, ins, target);
+	}
 	unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 16);
 	TCG_DISPATCH_TYPE(ctx, dtype, (ew_assign_k<T><<<grid, EW_BLOCK, 0, ctx->stream>>>(
 		opcode, (T*) target, (const T*) source, n)));

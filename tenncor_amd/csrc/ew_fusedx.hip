@@ -28,6 +28,7 @@ constexpr int FX_SLOTS = TCG_FX_MAX_LEAVES + TCG_FX_MAX_REGS;
 
 #define TCG_CORE(...) __VA_ARGS__
 #include "ew_fusedx_args.inc"
+#include "pass_args.inc"
 #undef TCG_CORE
 
 static_assert(sizeof(FxArgs) <= 4096, "launch arguments must fit the kernel argument segment");
@@ -347,11 +348,9 @@ bool fx_jit_enabled (void)
 	return on;
 }
 
-// dense: the leaf is addressed like the output (offset + linear index)
-std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
+// typedefs, opcode names, the scalar routines and the argument structs
+void fx_emit_prelude (std::ostringstream& o)
 {
-	const char* tname = dtype == TCG_DOUBLE ? "double" : dtype == TCG_FLOAT ? "float" : "int";
-	std::ostringstream o;
 	o << "typedef signed char int8_t; typedef unsigned char uint8_t; typedef int int32_t;\n"
 		"typedef unsigned int uint32_t; typedef long int64_t; typedef unsigned long uint64_t;\n"
 		"#ifndef INT32_MIN\n#define INT32_MIN (-2147483647 - 1)\n#endif\n"
@@ -370,16 +369,50 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
 	o << "enum {";
 	for (auto& op : opcodes) { o << op.name << " = " << op.value << ", "; }
 	o << "};\n" << fx_scalar_src << "\n" << fx_args_src << "\n";
-	o << "typedef " << tname << " T;\n";
-	if (N > 1)
+}
+
+// What one index `idx` of the iteration space computes: operand loads, the
+// program as straight-line code, the stores.  Expects `p` (an FxArgs), `idx`
+// and the element type `T` (with N > 1 also VT and VU) in scope.
+// dense: the leaf is addressed like the output (offset + linear index)
+// Baked launch arguments: the generated code holds extents, strides, offsets,
+// bounds and immediates as literals and takes its pointers from these expressions
+struct FxBake
+{
+	std::string leaf_ptr[TCG_FX_MAX_LEAVES];
+	std::string out_ptr[TCG_FX_MAX_OUTS];
+};
+
+void fx_emit_body (std::ostringstream& o, int N, const FxArgs& p, const bool* dense, const FxBake* bake = nullptr)
+{
+	// how the generated code names a launch argument: a field of `p`, or (baked)
+	// the value itself and a pointer expression
+	auto num = [](int64_t v) { return "((int64_t) " + std::to_string(v) + "ll)"; };
+	auto r_off = [&](uint32_t k) { return bake ? num(p.leaf[k].off) : "p.leaf[" + std::to_string(k) + "].off"; };
+	auto r_stride = [&](uint32_t k, uint32_t d)
 	{
-		o << "typedef T VT __attribute__((ext_vector_type(" << N << ")));\n"
-			"union VU { VT v; T e[" << N << "]; };\n";
-	}
-	o << "extern \"C\" __global__ __launch_bounds__(" << FX_BLOCK << ") void fx (FxArgs p)\n{\n"
-		"const uint32_t nvec = (uint32_t) (p.total / " << N << ");\n"
-		"const uint32_t step = gridDim.x * " << FX_BLOCK << ";\n"
-		"for (uint32_t idx = blockIdx.x * " << FX_BLOCK << " + threadIdx.x; idx < nvec; idx += step)\n{\n";
+		return bake ? num(p.leaf[k].stride[d]) : "p.leaf[" + std::to_string(k) + "].stride[" + std::to_string(d) + "]";
+	};
+	auto r_lo = [&](uint32_t k, uint32_t d)
+	{
+		return bake ? std::to_string(p.leaf[k].lo[d]) + "u" : "p.leaf[" + std::to_string(k) + "].lo[" + std::to_string(d) + "]";
+	};
+	auto r_hi = [&](uint32_t k, uint32_t d)
+	{
+		return bake ? std::to_string(p.leaf[k].hi[d]) + "u" : "p.leaf[" + std::to_string(k) + "].hi[" + std::to_string(d) + "]";
+	};
+	auto r_leaf = [&](uint32_t k) { return bake ? bake->leaf_ptr[k] : "p.leaf[" + std::to_string(k) + "].ptr"; };
+	auto r_out = [&](uint32_t k) { return bake ? bake->out_ptr[k] : "p.out[" + std::to_string(k) + "]"; };
+	auto r_imm = [&](uint32_t i) -> std::string
+	{
+		if (!bake) { return "p.imm[" + std::to_string(i) + "]"; }
+		double v = p.imm[i];
+		if (v != v) { return "__builtin_nan(\"\")"; }
+		if (v - v != 0.0) { return v > 0 ? "__builtin_inf()" : "(-__builtin_inf())"; }
+		char text[64];
+		snprintf(text, sizeof(text), "%a", v);
+		return std::string("(") + text + ")";
+	};
 	bool need_coords = false;
 	for (uint32_t k = 0; k < p.nleaf; ++k) { need_coords = need_coords || !dense[k]; }
 	if (need_coords)
@@ -387,6 +420,12 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
 		o << "uint32_t rem = idx;\n";
 		for (uint32_t d = 0; d + 1 < p.nd; ++d)
 		{
+			if (bake)
+			{
+				o << "const uint32_t q" << d << " = rem / " << p.div[d].d << "u;\n"
+					"uint32_t c" << d << " = rem - q" << d << " * " << p.div[d].d << "u;\nrem = q" << d << ";\n";
+				continue;
+			}
 			o << "const uint32_t q" << d << " = fx_div(rem, p.div[" << d << "]);\n"
 				"uint32_t c" << d << " = rem - q" << d << " * p.div[" << d << "].d;\nrem = q" << d << ";\n";
 		}
@@ -399,24 +438,24 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
 		o << "T l" << k << "[" << N << "];\n{\n";
 		if (dense[k])
 		{
-			o << "const T* src = (const T*) p.leaf[" << k << "].ptr + (p.leaf[" << k << "].off + (int64_t) idx * " << N << ");\n";
+			o << "const T* src = (const T*) " << r_leaf(k) << " + (" << r_off(k) << " + (int64_t) idx * " << N << ");\n";
 		}
 		else
 		{
-			o << "int64_t off = p.leaf[" << k << "].off";
+			o << "int64_t off = " << r_off(k);
 			for (uint32_t d = 0; d < p.nd; ++d)
 			{
 				if (d == 0 && L.bcast0) { continue; }
-				o << " + (int64_t) c" << d << " * p.leaf[" << k << "].stride[" << d << "]";
+				o << " + (int64_t) c" << d << " * " << r_stride(k, d);
 			}
-			o << ";\nconst T* src = (const T*) p.leaf[" << k << "].ptr + off;\n";
+			o << ";\nconst T* src = (const T*) " << r_leaf(k) << " + off;\n";
 		}
 		if (L.boxed)
 		{
 			o << "bool inside = true";
 			for (uint32_t d = 0; d < p.nd; ++d)
 			{
-				o << " && c" << d << " >= p.leaf[" << k << "].lo[" << d << "] && c" << d << " < p.leaf[" << k << "].hi[" << d << "]";
+				o << " && c" << d << " >= " << r_lo(k, d) << " && c" << d << " < " << r_hi(k, d);
 			}
 			o << ";\nif (inside)\n";
 		}
@@ -452,10 +491,10 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
 	{
 		const FxInstr& ins = p.prog[i];
 		bool uses_imm = ins.a == TCG_FX_IMM || ins.b == TCG_FX_IMM || ins.c == TCG_FX_IMM;
-		if (uses_imm) { o << "const T imm" << i << " = (T) p.imm[" << i << "];\n"; }
+		if (uses_imm) { o << "const T imm" << i << " = (T) " << r_imm(i) << ";\n"; }
 		if (ins.opcode == TCG_FX_STORE)
 		{
-			o << "{\nT* dst = (T*) p.out[" << (int) ins.dst << "] + (uint64_t) idx * " << N << ";\n";
+			o << "{\nT* dst = (T*) " << r_out(ins.dst) << " + (uint64_t) idx * " << N << ";\n";
 			if (N > 1)
 			{
 				o << "VU v;\n";
@@ -491,6 +530,28 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
 		}
 		reg_name[ins.dst - TCG_FX_REG0] = name;
 	}
+}
+
+const char* fx_type_name (int dtype)
+{
+	return dtype == TCG_DOUBLE ? "double" : dtype == TCG_FLOAT ? "float" : "int";
+}
+
+std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense)
+{
+	std::ostringstream o;
+	fx_emit_prelude(o);
+	o << "typedef " << fx_type_name(dtype) << " T;\n";
+	if (N > 1)
+	{
+		o << "typedef T VT __attribute__((ext_vector_type(" << N << ")));\n"
+			"union VU { VT v; T e[" << N << "]; };\n";
+	}
+	o << "extern \"C\" __global__ __launch_bounds__(" << FX_BLOCK << ") void fx (FxArgs p)\n{\n"
+		"const uint32_t nvec = (uint32_t) (p.total / " << N << ");\n"
+		"const uint32_t step = gridDim.x * " << FX_BLOCK << ";\n"
+		"for (uint32_t idx = blockIdx.x * " << FX_BLOCK << " + threadIdx.x; idx < nvec; idx += step)\n{\n";
+	fx_emit_body(o, N, p, dense);
 	o << "}\n}\n";
 	return o.str();
 }
@@ -531,11 +592,8 @@ int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out)
 	return TCG_OK;
 }
 
-int fusedx_jit_launch (tcg_ctx* ctx, int dtype, FxArgs& p, bool vec)
+void fx_dense_leaves (const FxArgs& p, bool* dense)
 {
-	const int N = vec ? (int) (16 / tcg_type_size(dtype)) : 1;
-	if (vec) { p.div[0] = fx_make_div(p.size[0] / N); }
-	bool dense[TCG_FX_MAX_LEAVES];
 	for (uint32_t k = 0; k < p.nleaf; ++k)
 	{
 		const FxLeaf& L = p.leaf[k];
@@ -547,6 +605,14 @@ int fusedx_jit_launch (tcg_ctx* ctx, int dtype, FxArgs& p, bool vec)
 			run *= (int64_t) p.size[d];
 		}
 	}
+}
+
+int fusedx_jit_launch (tcg_ctx* ctx, int dtype, FxArgs& p, bool vec)
+{
+	const int N = vec ? (int) (16 / tcg_type_size(dtype)) : 1;
+	if (vec) { p.div[0] = fx_make_div(p.size[0] / N); }
+	bool dense[TCG_FX_MAX_LEAVES];
+	fx_dense_leaves(p, dense);
 	std::string source = fx_source(dtype, N, p, dense);
 	FxJit& jit = fx_jit();
 	hipFunction_t fn = nullptr;
@@ -568,6 +634,368 @@ int fusedx_jit_launch (tcg_ctx* ctx, int dtype, FxArgs& p, bool vec)
 	return TCG_OK;
 }
 
+// ---- a whole pass of a small graph as one kernel ------------------------------
+//
+// A graph of a few dozen functors over tensors of a few dozen elements (a
+// dense layer on a batch of three) spends its time being launched: a recorded
+// sequence of 13 kernels takes 37 us to enqueue and drain, one kernel 12 us.
+// Such a pass is recorded as the steps of ONE kernel: a single workgroup runs
+// the steps in order with a barrier between them.  Three kinds of steps:
+// elementwise groups (the code a fused group compiles to, so they are bit-exact
+// with tcg_ew_fusedx), contractions (each output summed in ascending order of
+// the summed index, fused multiply-add: what the generic product kernel does)
+// and reductions (each output folded in ascending order).  Work is bounded so
+// that one workgroup finishes in microseconds; anything else refuses the
+// recording and the caller records the sequence launch by launch.
+
+constexpr int PASS_BLOCK = 256;
+constexpr uint64_t PASS_MAX_WORK = 4096;  // iterations of the busiest lane, all steps together
+constexpr size_t PASS_MAX_STEPS = 256;
+
+struct PassStep
+{
+	int kind;  // 0 elementwise, 1 contraction, 2 reduction
+	int dtype;
+	int opcode;
+	FxArgs fx;
+	bool dense[TCG_FX_MAX_LEAVES];
+	PassContract ct;
+	PassReduce rd;
+};
+
+} // namespace
+
+struct tcg_small_pass
+{
+	std::vector<PassStep> steps;
+	uint64_t work = 0;
+	hipFunction_t fn = nullptr;
+	std::vector<void*> ptrs; // the kernel's argument block
+};
+
+namespace
+{
+
+int small_charge (tcg_ctx* ctx, uint64_t items, uint64_t per_item)
+{
+	tcg_small_pass* pass = ctx->capturing->pass;
+	uint64_t cost = (items + PASS_BLOCK - 1) / PASS_BLOCK * (per_item ? per_item : 1);
+	if (pass->steps.size() >= PASS_MAX_STEPS || pass->work + cost > PASS_MAX_WORK)
+	{
+		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "the sequence is too long for a single-launch pass");
+	}
+	pass->work += cost;
+	return TCG_OK;
+}
+
+int small_append_fx (tcg_ctx* ctx, int dtype, const FxArgs& p)
+{
+	int rc = small_charge(ctx, p.total, p.ninstr);
+	if (rc != TCG_OK) { return rc; }
+	PassStep step;
+	memset(&step, 0, sizeof(step));
+	step.kind = 0;
+	step.dtype = dtype;
+	step.fx = p;
+	fx_dense_leaves(p, step.dense);
+	ctx->capturing->pass->steps.push_back(step);
+	return TCG_OK;
+}
+
+// resolve: the expression the kernel uses for a device pointer of the recording
+template <typename Resolve>
+std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_t lds_bytes, Resolve resolve)
+{
+	std::ostringstream o;
+	fx_emit_prelude(o);
+	o << "struct PassPtrs { void* p[" << std::max<size_t>(1, nptrs) << "]; };\n"
+		"template <typename T> __device__ __forceinline__ T pass_mac (T a, T b, T acc)\n{\n"
+		"if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b + (uint32_t) acc); }\n"
+		"else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, acc); }\n"
+		"else { return __builtin_fma(a, b, acc); }\n}\n"
+		"extern \"C\" __global__ __launch_bounds__(" << PASS_BLOCK << ") void fx (PassPtrs P)\n{\n";
+	if (lds_bytes) { o << "__shared__ __attribute__((aligned(256))) char lds[" << lds_bytes << "];\n"; }
+	auto lit = [](int64_t v) { return "((int64_t) " + std::to_string(v) + "ll)"; };
+	// index -> coordinates over `n` dims with literal extents, accumulating offsets
+	auto decompose = [&](const char* index, uint32_t n, const uint32_t* size,
+		std::initializer_list<std::pair<const char*,const int64_t*>> sums)
+	{
+		for (uint32_t d = 0; d < n; ++d)
+		{
+			o << "{ const uint32_t q = " << index << " / " << size[d] << "u; const int64_t x = " << index << " - q * "
+				<< size[d] << "u; " << index << " = q;";
+			for (auto& sum : sums) { o << " " << sum.first << " += x * " << lit(sum.second[d]) << ";"; }
+			o << " }\n";
+		}
+	};
+	for (size_t i = 0; i < steps.size(); ++i)
+	{
+		const PassStep& s = steps[i];
+		if (i > 0) { o << "__syncthreads();\n"; }
+		o << "{\ntypedef " << fx_type_name(s.dtype) << " T;\n";
+		if (s.kind == 0)
+		{
+			FxBake bake;
+			for (uint32_t k = 0; k < s.fx.nleaf; ++k) { bake.leaf_ptr[k] = resolve(s.fx.leaf[k].ptr); }
+			for (uint32_t k = 0; k < s.fx.nout; ++k) { bake.out_ptr[k] = resolve(s.fx.out[k]); }
+			o << "for (uint32_t idx = threadIdx.x; idx < " << s.fx.total << "u; idx += " << PASS_BLOCK << ")\n{\n";
+			fx_emit_body(o, 1, s.fx, s.dense, &bake);
+			o << "}\n";
+		}
+		else if (s.kind == 1)
+		{
+			const PassContract& c = s.ct;
+			o << "const T* a = (const T*) " << resolve(c.a) << "; const T* b = (const T*) " << resolve(c.b)
+				<< "; T* out = (T*) " << resolve(c.out) << ";\n"
+				"for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << PASS_BLOCK << ")\n{\n"
+				"uint32_t rem = o; int64_t ao = 0, bo = 0;\n";
+			decompose("rem", c.nod, c.osize, {{"ao", c.oastr}, {"bo", c.obstr}});
+			o << "T acc = (T) 0;\n"
+				"for (uint32_t k = 0; k < " << c.K << "u; ++k)\n{\n"
+				"uint32_t r = k; int64_t ak = ao, bk = bo;\n";
+			decompose("r", c.nkd, c.ksize, {{"ak", c.kastr}, {"bk", c.kbstr}});
+			o << "acc = pass_mac<T>(a[ak], b[bk], acc);\n}\n"
+				"out[o] = acc;\n}\n";
+		}
+		else
+		{
+			const PassReduce& c = s.rd;
+			o << "const T* in = (const T*) " << resolve(c.in) << "; T* out = (T*) " << resolve(c.out) << ";\n"
+				"for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << PASS_BLOCK << ")\n{\n"
+				"uint32_t rem = o; int64_t base = 0;\n";
+			decompose("rem", c.nod, c.osize, {{"base", c.oistr}});
+			o << "T acc = in[base];\n"
+				"for (uint32_t k = 1; k < " << c.R << "u; ++k)\n{\n"
+				"uint32_t r = k; int64_t off = base;\n";
+			decompose("r", c.nrd, c.rsize, {{"off", c.ristr}});
+			o << "acc = apply_binary<T>(" << s.opcode << ", acc, in[off]);\n}\n"
+				"out[o] = acc;\n}\n";
+		}
+		o << "}\n";
+	}
+	o << "}\n";
+	return o.str();
+}
+
+} // namespace
+
+int tcg_small_unsupported (tcg_ctx* ctx, const char* what)
+{
+	return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "%s cannot be a step of a single-launch pass", what);
+}
+
+int tcg_small_begin (tcg_ctx*, tcg_graph* g)
+{
+	g->small = true;
+	g->pass = new tcg_small_pass();
+	return TCG_OK;
+}
+
+void tcg_small_release (tcg_graph* g)
+{
+	if (nullptr == g->pass) { return; }
+	delete g->pass;
+	g->pass = nullptr;
+}
+
+int tcg_small_finish (tcg_ctx* ctx, tcg_graph* g)
+{
+	tcg_small_pass* pass = g->pass;
+	if (pass->steps.empty()) { return TCG_OK; } // nothing to launch
+	// A buffer that the recording handed out and took back again is read and
+	// written by these steps only: it lives in LDS.  Everything else (leaves,
+	// results somebody holds on to) is reached through a pointer argument.
+	constexpr size_t lds_cap = 48u << 10;
+	std::map<void*,size_t> lds_offset;
+	size_t lds_bytes = 0;
+	std::map<const void*,size_t> slot;
+	auto resolve = [&](const void* ptr) -> std::string
+	{
+		auto it = g->blocks.upper_bound(const_cast<void*>(ptr));
+		if (it != g->blocks.begin())
+		{
+			--it;
+			const char* begin = (const char*) it->first;
+			if ((const char*) ptr < begin + it->second && 0 == g->held.count(it->first))
+			{
+				auto at = lds_offset.find(it->first);
+				if (at == lds_offset.end() && lds_bytes + it->second <= lds_cap)
+				{
+					at = lds_offset.emplace(it->first, lds_bytes).first;
+					lds_bytes += it->second;
+				}
+				if (at != lds_offset.end())
+				{
+					return "((void*) (lds + " + std::to_string(at->second + (size_t) ((const char*) ptr - begin)) + "))";
+				}
+			}
+		}
+		auto at = slot.find(ptr);
+		if (at == slot.end()) { at = slot.emplace(ptr, slot.size()).first; }
+		return "P.p[" + std::to_string(at->second) + "]";
+	};
+	// two passes: the first finds out how much LDS and how many pointers there are
+	(void) pass_source(pass->steps, 1, 0, resolve);
+	TCG_REQUIRE(ctx, slot.size() <= 480, "tcg_capture_end: %zu buffers are too many for a single-launch pass", slot.size());
+	std::string source = pass_source(pass->steps, slot.size(), lds_bytes, resolve);
+	pass->ptrs.assign(std::max<size_t>(1, slot.size()), nullptr);
+	for (auto& kv : slot) { pass->ptrs[kv.second] = const_cast<void*>(kv.first); }
+	FxJit& jit = fx_jit();
+	{
+		std::lock_guard<std::mutex> lock(jit.mu);
+		auto it = jit.kernels.find(source);
+		if (it == jit.kernels.end())
+		{
+			int rc = fx_compile(ctx, source, &pass->fn);
+			if (rc != TCG_OK) { return rc; }
+			jit.kernels.emplace(source, pass->fn);
+		}
+		else { pass->fn = it->second; }
+	}
+	g->kernels = 1;
+	return TCG_OK;
+}
+
+int tcg_small_launch (tcg_ctx* ctx, tcg_graph* g)
+{
+	tcg_small_pass* pass = g->pass;
+	if (nullptr == pass || nullptr == pass->fn) { return TCG_OK; }
+	size_t size = pass->ptrs.size() * sizeof(void*);
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, pass->ptrs.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+	TCG_HIP(ctx, hipModuleLaunchKernel(pass->fn, 1, 1, 1, PASS_BLOCK, 1, 1, 0, ctx->stream, nullptr, config));
+	return TCG_OK;
+}
+
+int tcg_small_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8], const uint64_t bshape[8],
+	int npairs, const uint64_t* pairs, const void* a, const void* b, void* out)
+{
+	TCG_REQUIRE(ctx, tcg_type_size(dtype) && a && b && out && npairs >= 0 && npairs <= 8 && (pairs || npairs == 0),
+		"tcg_contract: bad arguments");
+	PassStep step;
+	memset(&step, 0, sizeof(step));
+	step.kind = 1;
+	step.dtype = dtype;
+	PassContract& c = step.ct;
+	c.a = a; c.b = b; c.out = out;
+	int64_t astr[8], bstr[8];
+	astr[0] = bstr[0] = 1;
+	for (int d = 1; d < 8; ++d)
+	{
+		astr[d] = astr[d - 1] * (int64_t) ashape[d - 1];
+		bstr[d] = bstr[d - 1] * (int64_t) bshape[d - 1];
+	}
+	bool acon[8] = {false}, bcon[8] = {false};
+	uint64_t K = 1, nout = 1;
+	for (int i = 0; i < npairs; ++i)
+	{
+		uint64_t pa = pairs[2 * i], pb = pairs[2 * i + 1];
+		TCG_REQUIRE(ctx, pa < 8 && pb < 8 && !acon[pa] && !bcon[pb] && ashape[pa] == bshape[pb],
+			"tcg_contract: invalid shapes or contraction pairs");
+		acon[pa] = bcon[pb] = true;
+		if (ashape[pa] == 1) { continue; }
+		c.ksize[c.nkd] = (uint32_t) ashape[pa];
+		c.kastr[c.nkd] = astr[pa];
+		c.kbstr[c.nkd] = bstr[pb];
+		++c.nkd;
+		K *= ashape[pa];
+	}
+	// output dims: what is left of b, then what is left of a (internal/eigen/operator.hpp:1069-1103)
+	for (int side = 0; side < 2; ++side)
+	{
+		const uint64_t* shape = side == 0 ? bshape : ashape;
+		const bool* con = side == 0 ? bcon : acon;
+		for (int d = 0; d < 8; ++d)
+		{
+			if (con[d] || shape[d] == 1) { continue; }
+			TCG_REQUIRE(ctx, c.nod < 8, "tcg_contract: the result has more than 8 dims");
+			c.osize[c.nod] = (uint32_t) shape[d];
+			c.oastr[c.nod] = side == 0 ? 0 : astr[d];
+			c.obstr[c.nod] = side == 0 ? bstr[d] : 0;
+			++c.nod;
+			nout *= shape[d];
+		}
+	}
+	TCG_REQUIRE(ctx, nout < (1ull << 31) && K < (1ull << 31), "tcg_contract: too large");
+	c.nout = (uint32_t) nout;
+	c.K = (uint32_t) K;
+	int rc = small_charge(ctx, nout, K);
+	if (rc != TCG_OK) { return rc; }
+	ctx->capturing->pass->steps.push_back(step);
+	return TCG_OK;
+}
+
+int tcg_small_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8], unsigned rankmask,
+	const void* in, void* out)
+{
+	TCG_REQUIRE(ctx, tcg_type_size(dtype) && in && out, "tcg_reduce: bad arguments");
+	int fold = opcode == TCG_REDUCE_SUM ? TCG_ADD : opcode == TCG_REDUCE_PROD ? TCG_MUL :
+		opcode == TCG_REDUCE_MIN ? TCG_MIN : opcode == TCG_REDUCE_MAX ? TCG_MAX : 0;
+	TCG_REQUIRE(ctx, fold, "tcg_reduce: opcode %d is not a reduction", opcode);
+	PassStep step;
+	memset(&step, 0, sizeof(step));
+	step.kind = 2;
+	step.dtype = dtype;
+	step.opcode = fold;
+	PassReduce& c = step.rd;
+	c.in = in; c.out = out;
+	uint64_t nout = 1, R = 1;
+	int64_t stride = 1;
+	for (int d = 0; d < 8; ++d)
+	{
+		if (shape[d] > 1)
+		{
+			if (rankmask & (1u << d))
+			{
+				c.rsize[c.nrd] = (uint32_t) shape[d];
+				c.ristr[c.nrd] = stride;
+				++c.nrd;
+				R *= shape[d];
+			}
+			else
+			{
+				c.osize[c.nod] = (uint32_t) shape[d];
+				c.oistr[c.nod] = stride;
+				++c.nod;
+				nout *= shape[d];
+			}
+		}
+		stride *= (int64_t) shape[d];
+	}
+	TCG_REQUIRE(ctx, nout < (1ull << 31) && R < (1ull << 31), "tcg_reduce: too large");
+	c.nout = (uint32_t) nout;
+	c.R = (uint32_t) R;
+	int rc = small_charge(ctx, nout, R);
+	if (rc != TCG_OK) { return rc; }
+	ctx->capturing->pass->steps.push_back(step);
+	return TCG_OK;
+}
+
+int tcg_small_copy (tcg_ctx* ctx, int dtype, int nd, const uint64_t* shape, const int64_t* stride, int64_t offset,
+	const uint64_t* lo, const uint64_t* hi, const void* in, void* out)
+{
+	uint64_t full[8];
+	tcg_fx_leaf leaf;
+	memset(&leaf, 0, sizeof(leaf));
+	leaf.ptr = in;
+	leaf.offset = offset;
+	for (int d = 0; d < 8; ++d)
+	{
+		full[d] = d < nd ? shape[d] : 1;
+		leaf.stride[d] = d < nd ? stride[d] : 0;
+		leaf.lo[d] = (lo && d < nd) ? lo[d] : 0;
+		leaf.hi[d] = (hi && d < nd) ? hi[d] : full[d];
+	}
+	tcg_fx_instr store;
+	memset(&store, 0, sizeof(store));
+	store.opcode = TCG_FX_STORE;
+	store.a = TCG_FX_LEAF0;
+	store.dst = 0;
+	void* outs[1] = {out};
+	return tcg_ew_fusedx(ctx, dtype, full, 1, &leaf, 1, &store, 1, outs);
+}
+
+namespace
+{
 } // namespace
 
 extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
@@ -712,6 +1140,7 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		}
 		if (L.boxed) { vec = vec && L.lo[0] % N == 0 && L.hi[0] % N == 0; }
 	}
+	if (tcg_small_mode(ctx)) { return small_append_fx(ctx, dtype, p); }
 	if (fx_jit_enabled()) { return fusedx_jit_launch(ctx, dtype, p, vec); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return fusedx_launch<T>(ctx, p, vec));
 	return TCG_OK;

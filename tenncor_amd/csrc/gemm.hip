@@ -21,7 +21,8 @@ template <typename T>
 __device__ __forceinline__ T fma_wrap (T a, T b, T c)
 {
 	if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b + (uint32_t) c); }
-	else { return a * b + c; }
+	else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, c); }
+	else { return __builtin_fma(a, b, c); }
 }
 
 constexpr int GT = 64;  // tile of C per workgroup
@@ -189,6 +190,12 @@ int tcg_matmul (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 		TCG_REQUIRE(ctx, ashape[d] == bshape[d], "tcg_matmul: invalid shapes do not match for dimensions 2+ (dim %d)", d);
 		batch *= ashape[d];
 	}
+	if (tcg_small_mode(ctx))
+	{
+		if (batch != 1) { return tcg_small_unsupported(ctx, "a batched matrix product"); }
+		const uint64_t pair[2] = {0, 1};
+		return tcg_small_contract(ctx, dtype, ashape, bshape, 1, pair, a, b, out);
+	}
 	return tcg_gemm(ctx, dtype, M, N, K, batch, a, K, M * K, 0, b, N, K * N, 0, out, N, M * N);
 }
 
@@ -215,6 +222,16 @@ int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 		pa[q] = ad;
 		pb[q] = bd;
 		K *= ashape[ad];
+	}
+	if (tcg_small_mode(ctx))
+	{
+		uint64_t sorted[16];
+		for (int p = 0; p < npairs; ++p)
+		{
+			sorted[2 * p] = pa[p];
+			sorted[2 * p + 1] = pb[p];
+		}
+		return tcg_small_contract(ctx, dtype, ashape, bshape, npairs, sorted, a, b, out);
 	}
 	for (int d = 0; d < 8; ++d)
 	{

@@ -10,6 +10,7 @@
 //                   a 64x64 tile goes through LDS so that both the reads and
 //                   the writes are coalesced.
 // All of them move each byte once: HBM-bound.
+#include <type_traits>
 #include "tcg_internal.hpp"
 
 namespace
@@ -221,6 +222,24 @@ int run_plan (tcg_ctx* ctx, CopyPlan& p, const T* src, T* dst, const char* what)
 	if (p.total >= (1ull << 32))
 	{
 		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "%s: %llu elements exceed the 2^32 limit of one launch", what, (unsigned long long) p.total);
+	}
+	if (tcg_small_mode(ctx))
+	{
+		// a step of a sequence recorded as one kernel: a gather into a dense destination
+		int64_t run = 1;
+		bool dense_dst = p.dbase == 0;
+		uint64_t size[8], lo[8], hi[8];
+		for (int d = 0; d < p.nd; ++d)
+		{
+			dense_dst = dense_dst && p.dstride[d] == run;
+			run *= (int64_t) p.size[d];
+			size[d] = p.size[d];
+			lo[d] = p.box ? p.lo[d] : 0;
+			hi[d] = p.box ? p.hi[d] : p.size[d];
+		}
+		if (false == dense_dst) { return tcg_small_unsupported(ctx, "a copy into a strided destination"); }
+		int dtype = std::is_same<T,double>::value ? TCG_DOUBLE : std::is_same<T,float>::value ? TCG_FLOAT : TCG_INT32;
+		return tcg_small_copy(ctx, dtype, p.nd, size, p.sstride, p.sbase, lo, hi, src, dst);
 	}
 	constexpr int N = Vec16<T>::N;
 	// transpose path: destination contiguous along dim 0, source along dim j

@@ -473,6 +473,7 @@ int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
 	TCG_REQUIRE(ctx, shape && in && out, "tcg_reduce: NULL pointer");
 	TCG_REQUIRE(ctx, rankmask < 256, "tcg_reduce: rank set 0x%x names a dim >= 8", rankmask);
 	if (tcg_n_elems(shape) == 0) { return TCG_OK; }
+	if (tcg_small_mode(ctx)) { return tcg_small_reduce(ctx, opcode, dtype, shape, rankmask, in, out); }
 	TCG_DISPATCH_TYPE(ctx, dtype,
 		switch (opcode)
 		{

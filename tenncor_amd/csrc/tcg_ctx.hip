@@ -368,8 +368,20 @@ int tcg_capture_begin (tcg_ctx* ctx)
 	return TCG_OK;
 }
 
+int tcg_capture_begin_small (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_capture_begin_small: a capture is already in progress");
+	// the stream captures as well: a launch that is not handed over as a step
+	// is caught there (and fails tcg_capture_end) instead of running out of turn
+	TCG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+	ctx->capturing = new tcg_graph();
+	return tcg_small_begin(ctx, ctx->capturing);
+}
+
 static void graph_release (tcg_ctx* ctx, tcg_graph* g)
 {
+	tcg_small_release(g);
 	if (g->exec) { (void) hipGraphExecDestroy(g->exec); }
 	if (g->graph) { (void) hipGraphDestroy(g->graph); }
 	for (auto& kv : g->blocks)
@@ -392,9 +404,21 @@ int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out)
 	ctx->capturing = nullptr;
 	g->free_blocks.clear();
 	hipError_t err = hipStreamEndCapture(ctx->stream, &g->graph);
-	if (err == hipSuccess) { err = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0); }
 	size_t nodes = 0;
 	if (err == hipSuccess) { err = hipGraphGetNodes(g->graph, nullptr, &nodes); }
+	if (err == hipSuccess && g->small)
+	{
+		int rc = nodes == 0 ? tcg_small_finish(ctx, g) :
+			tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_capture_end: %zu launches were not steps of the single-launch pass", nodes);
+		if (rc != TCG_OK)
+		{
+			graph_release(ctx, g);
+			return rc;
+		}
+		*out = g;
+		return TCG_OK;
+	}
+	if (err == hipSuccess) { err = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0); }
 	if (err != hipSuccess)
 	{
 		(void) hipGetLastError();
@@ -422,6 +446,7 @@ int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph)
 {
 	if (!ctx || !graph) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_graph_launch: cannot launch while capturing");
+	if (graph->small) { return tcg_small_launch(ctx, graph); }
 	TCG_HIP(ctx, hipGraphLaunch(graph->exec, ctx->stream));
 	return TCG_OK;
 }

@@ -31,6 +31,9 @@ struct tcg_graph
 	std::map<size_t,std::vector<void*>> free_blocks;    // reuse while capturing
 	uint64_t bytes = 0;
 	uint64_t kernels = 0;
+	// a sequence recorded as the steps of ONE kernel (tcg_capture_begin_small)
+	bool small = false;
+	struct tcg_small_pass* pass = nullptr;
 };
 
 struct tcg_ctx
@@ -107,6 +110,26 @@ static inline bool tcg_aligned16 (const void* p)
 {
 	return (reinterpret_cast<uintptr_t>(p) & 15) == 0;
 }
+
+// ---- sequences recorded as one kernel (ew_fusedx.hip) ------------------------
+// While such a recording is open, entry points hand their work over as a step
+// instead of launching; anything that cannot be a step fails the recording.
+static inline bool tcg_small_mode (const tcg_ctx* ctx)
+{
+	return ctx->capturing && ctx->capturing->small;
+}
+int tcg_small_begin (tcg_ctx* ctx, tcg_graph* g);
+int tcg_small_finish (tcg_ctx* ctx, tcg_graph* g);   // compiles; the recording is closed
+int tcg_small_launch (tcg_ctx* ctx, tcg_graph* g);
+void tcg_small_release (tcg_graph* g);
+int tcg_small_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8], const uint64_t bshape[8],
+	int npairs, const uint64_t* pairs, const void* a, const void* b, void* out);
+int tcg_small_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8], unsigned rankmask,
+	const void* in, void* out);
+// out[i] = in[offset + sum_d c_d * stride[d]] over `shape` (zero outside [lo, hi) when given)
+int tcg_small_copy (tcg_ctx* ctx, int dtype, int nd, const uint64_t* shape, const int64_t* stride, int64_t offset,
+	const uint64_t* lo, const uint64_t* hi, const void* in, void* out);
+int tcg_small_unsupported (tcg_ctx* ctx, const char* what);
 
 // A convolution lowered to a matrix product reads A[m][s] = image[rows[m].off +
 // sums[s].off], or zero when, for some j < ncheck, rows[m].c[j] + sums[s].c[j]

@@ -31,7 +31,7 @@ EXPORTS = [
     "tcr_set_random", "tcr_seed",
 ]
 
-EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED = 0, 1, 2
+EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED, EVAL_REPLAY_LAUNCHES = 0, 1, 2, 3
 
 # conversions shipped with the package (the reference's cfg/optimizations.json
 # is a git-lfs pointer without content)
@@ -94,11 +94,14 @@ def load():
 def set_evaluator(kind):
     """teq::set_eval: "plain" (node-by-node walk, the default), "replay"
     (record a target set's launches on its second evaluation, with elementwise
-    functors sharing launches, and enqueue the recording afterwards) or
-    "replay_unfused" (the same with one launch per functor).  Process-wide,
-    like the reference's evaluator slot."""
+    functors sharing launches and the pass of a graph of small tensors as one
+    kernel, and enqueue the recording afterwards), "replay_launches" (the same
+    without single-kernel passes: bit-identical to the walk) or
+    "replay_unfused" (one launch per functor).  Process-wide, like the
+    reference's evaluator slot."""
     lib = load()
-    code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY, "replay_unfused": EVAL_REPLAY_UNFUSED}[kind]
+    code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY, "replay_unfused": EVAL_REPLAY_UNFUSED,
+            "replay_launches": EVAL_REPLAY_LAUNCHES}[kind]
     if lib.tcr_set_evaluator(code) != 0:
         raise GraphError(lib.tcr_last_error().decode())
 

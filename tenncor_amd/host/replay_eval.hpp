@@ -40,8 +40,11 @@ struct ReplayEvaluator final : public teq::iEvaluator
 	/// A set of targets is recorded when it is asked for the
 	/// (`warm_passes` + 1)-th time; at most `max_plans` recordings are kept
 	/// With `fuse`, elementwise functors that feed one another are computed
-	/// in shared launches (fuse_plan.hpp)
-	ReplayEvaluator (size_t warm_passes = 1, size_t max_plans = 16, bool fuse = true);
+	/// in shared launches (fuse_plan.hpp); with `small_passes` as well, the
+	/// pass over a graph of small tensors is recorded as the steps of one
+	/// kernel (sums then run in index order: equal to the walk within the
+	/// tolerance of reductions and contractions, not bit for bit)
+	ReplayEvaluator (size_t warm_passes = 1, size_t max_plans = 16, bool fuse = true, bool small_passes = true);
 
 	~ReplayEvaluator (void);
 
@@ -82,6 +85,7 @@ private:
 	size_t warm_passes_;
 	size_t max_plans_;
 	bool fuse_;
+	bool small_passes_ = true;
 	size_t epoch_ = 0;
 	size_t clock_ = 0;
 };

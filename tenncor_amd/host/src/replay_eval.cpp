@@ -3,6 +3,7 @@
 #include "fuse_plan.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 
 namespace eigen
 {
@@ -45,9 +46,9 @@ struct ReplayEvaluator::Plan final
 	bool fresh = true;
 };
 
-ReplayEvaluator::ReplayEvaluator (size_t warm_passes, size_t max_plans, bool fuse) :
+ReplayEvaluator::ReplayEvaluator (size_t warm_passes, size_t max_plans, bool fuse, bool small_passes) :
 	warm_passes_(warm_passes), max_plans_(std::max<size_t>(1, max_plans)), fuse_(fuse),
-	epoch_(global::structure_epoch()) {}
+	small_passes_(fuse && small_passes), epoch_(global::structure_epoch()) {}
 
 ReplayEvaluator::~ReplayEvaluator (void)
 {
@@ -196,46 +197,56 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		}
 	}
 	// every value under the targets is recomputed into memory of the recording
-	for (iEigen* dev : plan->devs) { dev->drop(); }
-	for (Observable* f : plan->funcs) { f->prop_version(device.max_version_); }
 	tcg_ctx* ctx = hip_context();
-	hip_check(tcg_capture_begin(ctx));
-	bool ok = true;
-	try
+	auto attempt = [&](bool as_one_kernel)
 	{
-		for (auto& step : fusion.steps)
+		for (iEigen* dev : plan->devs) { dev->drop(); }
+		for (Observable* f : plan->funcs) { f->prop_version(device.max_version_); }
+		hip_check(as_one_kernel ? tcg_capture_begin_small(ctx) : tcg_capture_begin(ctx));
+		bool ok = true;
+		try
 		{
-			if (nullptr != step.node)
+			for (auto& step : fusion.steps)
 			{
-				device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0));
-			}
-			else if (step.conv >= 0)
-			{
-				launch_conv(fusion.convs[step.conv], targets, device.memory());
-			}
-			else if (step.contract >= 0)
-			{
-				launch_contract(fusion.contracts[step.contract], targets, device.memory());
-			}
-			else
-			{
-				launch_group(fusion.groups[step.group], targets, device.memory());
+				if (nullptr != step.node)
+				{
+					device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0));
+				}
+				else if (step.conv >= 0)
+				{
+					launch_conv(fusion.convs[step.conv], targets, device.memory());
+				}
+				else if (step.contract >= 0)
+				{
+					launch_contract(fusion.contracts[step.contract], targets, device.memory());
+				}
+				else
+				{
+					launch_group(fusion.groups[step.group], targets, device.memory());
+				}
 			}
 		}
-	}
-	catch (...)
-	{
-		// the node-by-node pass that follows reports whatever went wrong
-		ok = false;
-	}
-	if (ok)
-	{
-		ok = TCG_OK == tcg_capture_end(ctx, &plan->graph);
-	}
-	else
-	{
-		tcg_capture_abort(ctx);
-	}
+		catch (...)
+		{
+			// the node-by-node pass that follows reports whatever went wrong
+			ok = false;
+		}
+		if (ok)
+		{
+			ok = TCG_OK == tcg_capture_end(ctx, &plan->graph);
+		}
+		else
+		{
+			tcg_capture_abort(ctx);
+		}
+		return ok;
+	};
+	// a graph of small tensors costs what its launches cost: its pass is
+	// recorded as the steps of one kernel when every launch can be a step
+	bool small = fuse_ && small_passes_ && plan->funcs.size() <= 256 &&
+		std::all_of(plan->funcs.begin(), plan->funcs.end(), [](Observable* f) { return f->shape().n_elems() <= 4096; });
+	bool ok = small && attempt(true);
+	if (false == ok) { ok = attempt(false); }
 	if (false == ok)
 	{
 		for (iEigen* dev : plan->devs) { dev->drop(); }

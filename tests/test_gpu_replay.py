@@ -3,7 +3,10 @@ built on them (eigen::ReplayEvaluator, the replacement for the node-by-node
 walk of internal/teq/evaluator.hpp:11-61).
 
 A replay must give what issuing the same calls one by one gives, bit for bit:
-the same kernels run with the same arguments.  Every test replays several
+the same kernels run with the same arguments ("replay_launches").  The default
+kind ("replay") also records the pass of a graph of small tensors as ONE
+kernel whose sums run in index order: those are checked at the tolerance of
+reductions and contractions.  Every test replays several
 times, with ordinary launches and synchronisations of the same context between
 the replays, and checks every replay against the eagerly computed result.
 """
@@ -113,7 +116,7 @@ def test_capture_abort_and_errors(ctx):
 @pytest.fixture()
 def replay_graph():
     from tenncor_amd import graph
-    graph.set_evaluator("replay")
+    graph.set_evaluator("replay_launches")
     g = graph.Graph()
     try:
         yield g, graph.Api(g), graph
@@ -207,7 +210,7 @@ def test_replayed_training_loop_updates_leaves_in_place(replay_graph):
         g2.evaluate([step2])
         np.testing.assert_array_equal(seen[i], w2.get())
     g2.close()
-    graph.set_evaluator("replay")
+    graph.set_evaluator("replay_launches")
     # a different target set afterwards sees the updated weights
     g.evaluate([loss])
     g2 = None
@@ -256,12 +259,12 @@ def test_replay_mixes_with_other_target_sets_and_aliases(replay_graph):
         if i == 2:
             np.testing.assert_array_equal(mid, conv2.get())
     g2.close()
-    graph.set_evaluator("replay")
+    graph.set_evaluator("replay_launches")
 
 
 def test_recordings_are_dropped_when_nodes_go_away():
     from tenncor_amd import graph
-    graph.set_evaluator("replay")
+    graph.set_evaluator("replay_launches")
     try:
         g = graph.Graph()
         api = graph.Api(g)
@@ -289,7 +292,7 @@ def test_recordings_are_dropped_when_nodes_go_away():
 
 # ---- shared launches ---------------------------------------------------------
 
-def run_both(build, feeds, kinds=("plain", "replay", "replay_unfused")):
+def run_both(build, feeds, kinds=("plain", "replay_launches", "replay_unfused")):
     """Evaluate the same graph under each evaluator over the same sequence of
     inputs; returns {kind: [[target values per pass]]} and the stats of each."""
     from tenncor_amd import graph
@@ -338,8 +341,8 @@ def test_fused_lstm_matches_the_walk_bit_for_bit():
 
     results, stats = run_both(build, feeds)
     assert_same_bits(results)
-    assert stats["replay"]["replayed"] == 3 and stats["replay_unfused"]["replayed"] == 3
-    assert stats["replay"]["launches"] < 0.5 * stats["replay_unfused"]["launches"]
+    assert stats["replay_launches"]["replayed"] == 3 and stats["replay_unfused"]["replayed"] == 3
+    assert stats["replay_launches"]["launches"] < 0.5 * stats["replay_unfused"]["launches"]
 
 
 def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
@@ -353,7 +356,7 @@ def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
 
     results, stats = run_both(cnn, feeds)
     assert_same_bits(results)
-    assert stats["replay"]["launches"] < stats["replay_unfused"]["launches"]
+    assert stats["replay_launches"]["launches"] < stats["replay_unfused"]["launches"]
 
     def mlp_cfg(g, api):
         targets, x, _ = configs.config1_mlp(g)
@@ -362,7 +365,7 @@ def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
     feeds = [rng.uniform(-1, 1, 30).astype(np.float32) for _ in range(4)]
     results, stats = run_both(mlp_cfg, feeds)
     assert_same_bits(results)
-    assert stats["replay"]["launches"] < stats["replay_unfused"]["launches"]
+    assert stats["replay_launches"]["launches"] < stats["replay_unfused"]["launches"]
 
 
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
@@ -403,9 +406,9 @@ def test_fused_views_diamonds_and_wide_groups(np_dtype):
         neg = api.neg(api.unary("ABS", tall))
         return [u, wide, tall, neg, padded] + outs, x
 
-    results, stats = run_both(build, feeds, kinds=("plain", "replay"))
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches"))
     assert_same_bits(results)
-    assert stats["replay"]["replayed"] == 3
+    assert stats["replay_launches"]["replayed"] == 3
 
 
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
@@ -435,11 +438,11 @@ def test_fused_concat_keeps_every_bit(np_dtype):
         doubled = api.neg(api.neg(along0))               # elementwise readers in the same launch
         return [along0, along1, doubled, api.neg(along1)], x
 
-    results, stats = run_both(build, feeds, kinds=("plain", "replay"))
-    for row, ref in zip(results["replay"], results["plain"]):
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches"))
+    for row, ref in zip(results["replay_launches"], results["plain"]):
         for a, b in zip(row, ref):
             assert a.tobytes() == b.tobytes()
-    assert stats["replay"]["replayed"] == 3
+    assert stats["replay_launches"]["replayed"] == 3
 
 
 @pytest.mark.parametrize("evaluator", ["plain", "replay"])
@@ -477,3 +480,204 @@ def test_rand_unif_on_the_device_under_both_evaluators(evaluator):
     finally:
         graph.set_random("host")
         graph.set_evaluator("plain")
+
+
+# ---- a whole pass recorded as one kernel ---------------------------------------
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32])
+def test_small_sequence_recorded_as_one_kernel(ctx, np_dtype):
+    """tcg_capture_begin_small: elementwise, data-movement, contraction,
+    reduction and in-place steps in one launch against the same calls issued
+    one by one.  Elementwise and data-movement results are bit-identical;
+    sums are compared at 1e-5 (fp32) / 1e-13 (fp64) relative to the largest
+    value, exactly in int32 (ascending order here, a tree there)."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(5)
+    dt = capi.dtype_code(np_dtype)
+    M, K, N = 6, 10, 9
+    if np_dtype == np.int32:
+        draw = lambda n: rng.integers(-50, 50, n).astype(np.int32)
+    else:
+        draw = lambda n: rng.uniform(-1, 1, n).astype(np_dtype)
+    av, bv, cv, tv = draw(M * K), draw(K * N), draw(N), draw(M * N)
+    a, b, bias = ctx.upload(av), ctx.upload(bv), ctx.upload(cv)
+    targets = [ctx.upload(tv), ctx.upload(tv)]
+
+    def sequence(alloc, target):
+        prod, ext, summed, act, perm, cut = (alloc(M * N) for _ in range(6))
+        s0, s1, mx, outer = alloc(N), alloc(M), alloc(1), alloc(M * M)
+        ctx.matmul(dt, [K, M], [N, K], a.ptr, b.ptr, prod)
+        ctx.extend(dt, [N], [1, M], bias.ptr, ext)
+        ctx.ew_binary("ADD", dt, M * N, prod, ext, summed)
+        ctx.ew_unary("ABS", dt, M * N, summed, act)
+        ctx.ew_nary("MUL", dt, M * N, [act, ext, summed], ext)
+        ctx.permute(dt, [N, M], [1, 0, 2, 3, 4, 5, 6, 7], act, perm)                    # {M, N}
+        ctx.slice(dt, [M, N], [1, 2], [4, 5], perm, cut)                # {4, 5}
+        ctx.reduce("REDUCE_SUM", dt, [N, M], [1], act, s0)
+        ctx.reduce("REDUCE_SUM", dt, [N, M], [0], act, s1)
+        ctx.reduce("REDUCE_MAX", dt, [N, M], [0, 1], act, mx)
+        ctx.contract(dt, [N, M], [N, M], [[0, 0]], act, summed, outer)  # act . summed^T -> {M, M}
+        ctx.assign("ASSIGN_ADD", dt, M * N, target, ext)
+        return {"act": (act, M * N), "ext": (ext, M * N), "perm": (perm, M * N), "cut": (cut, 20), "s0": (s0, N),
+                "s1": (s1, M), "mx": (mx, 1), "outer": (outer, M * M), "target": (target, M * N)}
+
+    esz = np.dtype(np_dtype).itemsize
+    eager = sequence(lambda n: ctx.alloc(n * esz), targets[0].ptr)
+    want = {k: ctx.d2h(p, n, np_dtype) for k, (p, n) in eager.items()}
+    ctx.capture_begin(small=True)
+    recorded = sequence(lambda n: ctx.alloc(n * esz), targets[1].ptr)
+    graph = ctx.capture_end()
+    assert ctx.graph_stats(graph)[0] == 1
+    updated = tv.copy()
+    for launch in range(3):
+        ctx.graph_launch(graph)
+        updated = updated + want["ext"]
+        got = {k: ctx.d2h(p, n, np_dtype) for k, (p, n) in recorded.items() if k != "target"}
+        for k in ("act", "ext", "perm", "cut", "mx"):
+            np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+        for k in ("s0", "s1", "outer"):
+            if np_dtype == np.int32:
+                np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+            else:
+                tol = (1e-5 if np_dtype == np.float32 else 1e-13) * np.abs(want[k]).max()
+                assert np.abs(got[k] - want[k]).max() <= tol, k
+        # the in-place update is applied once per launch
+        np.testing.assert_array_equal(targets[1].get(), updated)
+    ctx.graph_destroy(graph)
+
+
+def test_small_recording_refuses_what_one_workgroup_should_not_do(ctx):
+    from tenncor_amd import capi
+    n = 1 << 20
+    x, y = ctx.upload(np.ones(n, np.float32)), ctx.empty(n, np.float32)
+    ctx.capture_begin(small=True)
+    with pytest.raises(capi.TcgError) as err:
+        for _ in range(8):
+            ctx.ew_unary("EXP", capi.FLOAT, n, x.ptr, y.ptr)
+    assert err.value.status == 3 and "single-launch pass" in str(err.value)
+    ctx.capture_abort()
+    # a launch that cannot be a step is caught when the recording ends
+    img, ker = ctx.upload(np.ones(64, np.float32)), ctx.upload(np.ones(4, np.float32))
+    out = ctx.empty(49, np.float32)
+    ctx.capture_begin(small=True)
+    ctx.conv(capi.FLOAT, [8, 8], [2, 2], [0, 1], img.ptr, ker.ptr, out.ptr)
+    with pytest.raises(capi.TcgError) as err:
+        ctx.capture_end()
+    assert err.value.status == 3
+    # the context is usable afterwards
+    ctx.ew_unary("EXP", capi.FLOAT, 64, img.ptr, out.ptr)
+    np.testing.assert_allclose(ctx.d2h(out.ptr, 49, np.float32), np.e, rtol=1e-6)
+
+
+# ---- graphs of small tensors: the pass as one kernel -----------------------------
+
+def close_to(got, ref, rtol):
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    scale = max(np.abs(ref).max(), 1e-300)
+    assert np.abs(got - ref).max() <= rtol * scale
+
+
+def test_small_graph_pass_is_one_launch_and_matches_golden_and_walk():
+    """tenncor/test/test_equation.cpp:482-706 (the shapes of configs[0]) under
+    the default replaying evaluator: one launch per evaluation, the reference's
+    gradients at 1e-12 (double), new inputs against the walk at 1e-12."""
+    from tenncor_amd import graph
+    fx = EQV["sigmoid_mlp_fast"]
+    rng = np.random.default_rng(3)
+    x0 = np.array(fx["in_data"], np.float64)
+    inputs = [x0, rng.uniform(-1, 1, 30), rng.uniform(-1, 1, 30), x0]
+    rows = {}
+    for kind in ("plain", "replay"):
+        graph.set_evaluator(kind)
+        g = graph.Graph()
+        try:
+            x, leaves, err, grads = mlp(g, graph.Api(g), fx, np.float64)
+            rows[kind] = []
+            for xv in inputs:
+                g.assign(x, xv)
+                g.evaluate([err] + grads)
+                rows[kind].append([t.get().copy() for t in [err] + grads])
+            if kind == "replay":
+                st = graph.evaluator_stats()
+                assert st["plain"] == 1 and st["recorded"] == 1 and st["replayed"] == 3 and st["launches"] == 1
+        finally:
+            g.close()
+            graph.set_evaluator("plain")
+    for key, val in zip(("expect_gw0", "expect_gb0", "expect_gw1", "expect_gb1"), rows["replay"][3][1:]):
+        np.testing.assert_allclose(val, np.array(fx[key]), rtol=1e-12)
+    for got, ref in zip(rows["replay"], rows["plain"]):
+        for a, b in zip(got, ref):
+            close_to(a, b, 1e-12)
+
+
+@pytest.mark.parametrize("config", ["mlp", "lstm", "training"])
+def test_small_graph_passes_follow_the_walk(config):
+    """fp32 graphs whose tensors are small (configs[0]; configs[3] at reduced
+    size; an sgd step through ASSIGN_SUB) as one launch per evaluation, against
+    the walk at 1e-5 of the largest value (sums run in another order)."""
+    from tenncor_amd import graph, configs
+    rng = np.random.default_rng(23)
+    rows = {}
+    for kind in ("plain", "replay"):
+        graph.set_evaluator(kind)
+        g = graph.Graph()
+        try:
+            if config == "mlp":
+                targets, x, _ = configs.config1_mlp(g)
+                feeds = [rng.uniform(-1, 1, 30).astype(np.float32) for _ in range(4)] if kind == "plain" else feeds
+            elif config == "lstm":
+                targets, x, _, _ = configs.config4_lstm(g, seq=4, batch=3, nin=5, hid=6)
+                feeds = [rng.uniform(-1, 1, 3 * 4 * 5).astype(np.float32) for _ in range(4)] if kind == "plain" else feeds
+            else:
+                api = graph.Api(g)
+                w = g.variable(np.linspace(-1, 1, 12).astype(np.float32), [3, 4], "w")
+                x = g.variable(np.zeros(8, np.float32), [4, 2], "x")
+                loss = api.reduce_sum(api.square(api.tanh(api.matmul(x, w))))
+                (dw,) = g.derive(loss, [w])
+                targets = [g.functor("ASSIGN_SUB", [w, api.mul(0.05, dw)]), loss]
+                feeds = [rng.uniform(-1, 1, 8).astype(np.float32) for _ in range(5)] if kind == "plain" else feeds
+            rows[kind] = []
+            for feed in feeds:
+                g.assign(x, feed)
+                g.evaluate(targets)
+                rows[kind].append([t.get().copy() for t in targets])
+            if kind == "replay":
+                st = graph.evaluator_stats()
+                assert st["recorded"] == 1 and st["replayed"] == len(feeds) - 1 and st["launches"] == 1
+        finally:
+            g.close()
+            graph.set_evaluator("plain")
+    for got, ref in zip(rows["replay"], rows["plain"]):
+        for a, b in zip(got, ref):
+            close_to(a, b, 1e-5)
+
+
+def test_graphs_with_steps_one_kernel_cannot_take_are_recorded_launch_by_launch():
+    """A convolution among small tensors: the single-kernel recording is
+    refused, the pass is recorded launch by launch and equals the walk bit for bit."""
+    from tenncor_amd import graph
+    rng = np.random.default_rng(2)
+    xv = rng.integers(1, 9, 2 * 6 * 5 * 2).astype(np.float32)
+    kv = rng.integers(-4, 5, 3 * 2 * 3 * 2).astype(np.float32)
+    rows = {}
+    for kind in ("plain", "replay"):
+        graph.set_evaluator(kind)
+        g = graph.Graph()
+        try:
+            api = graph.Api(g)
+            x = g.variable(xv, [2, 6, 5, 2], "x")
+            k = g.variable(kv, [3, 2, 3, 2], "k")
+            total = api.reduce_sum(api.relu(api.conv2d(x, k)))
+            rows[kind] = []
+            for i in range(4):
+                g.assign(x, xv + i)
+                g.evaluate([total])
+                rows[kind].append(total.get().copy())
+            if kind == "replay":
+                st = graph.evaluator_stats()
+                assert st["recorded"] == 1 and st["replayed"] == 3 and st["launches"] > 1
+        finally:
+            g.close()
+            graph.set_evaluator("plain")
+    for a, b in zip(rows["replay"], rows["plain"]):
+        np.testing.assert_array_equal(a, b)
