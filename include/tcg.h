@@ -145,6 +145,16 @@ int tcg_capture_abort (tcg_ctx* ctx);
  * call or at tcg_capture_end): the caller aborts and records with
  * tcg_capture_begin instead. */
 int tcg_capture_begin_small (tcg_ctx* ctx);
+/* For such a recording, an input the host rewrites between launches (a leaf
+ * of a few dozen elements) can travel with the launch instead of being copied
+ * to the device by a launch of its own: tcg_capture_feed, called before
+ * tcg_capture_end, says that the `bytes` at device address `devptr` are
+ * supplied by the launch (1024 bytes at most in all, no step may write them;
+ * `host` is their first content). tcg_graph_feed replaces the content for the
+ * launches that follow; it is copied at the call. The device memory at
+ * `devptr` is neither read nor written by the recording. */
+int tcg_capture_feed (tcg_ctx* ctx, const void* devptr, size_t bytes, const void* host);
+int tcg_graph_feed (tcg_ctx* ctx, tcg_graph* graph, const void* devptr, const void* host, size_t bytes);
 int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph);
 int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr);
 int tcg_graph_stats (const tcg_graph* graph, uint64_t* nodes, uint64_t* arena_bytes);

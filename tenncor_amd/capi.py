@@ -37,7 +37,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
-    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -129,6 +129,8 @@ def load():
         "tcg_capture_end": [vp, ctypes.POINTER(vp)],
         "tcg_capture_abort": [vp],
         "tcg_capture_begin_small": [vp],
+        "tcg_capture_feed": [vp, vp, sz, vp],
+        "tcg_graph_feed": [vp, vp, vp, vp, sz],
         "tcg_graph_launch": [vp, vp],
         "tcg_graph_claim": [vp, vp, vp],
         "tcg_graph_stats": [vp, u64p, u64p],
@@ -427,6 +429,15 @@ class Context:
             self._check(self.lib.tcg_capture_begin_small(self.handle))
         else:
             self._check(self.lib.tcg_capture_begin(self.handle))
+
+    def capture_feed(self, devptr, host):
+        """The launch supplies the content of `devptr` (single-launch recordings)."""
+        host = np.ascontiguousarray(host)
+        self._check(self.lib.tcg_capture_feed(self.handle, devptr, host.nbytes, host.ctypes.data))
+
+    def graph_feed(self, graph, devptr, host):
+        host = np.ascontiguousarray(host)
+        self._check(self.lib.tcg_graph_feed(self.handle, graph, devptr, host.ctypes.data, host.nbytes))
 
     def capture_end(self):
         g = ctypes.c_void_p()

@@ -15,6 +15,7 @@
 #include <hip/hiprtc.h>
 
 #include <cstdlib>
+#include <map>
 #include <mutex>
 #include <sstream>
 #include <unordered_map>
@@ -670,7 +671,12 @@ struct tcg_small_pass
 	std::vector<PassStep> steps;
 	uint64_t work = 0;
 	hipFunction_t fn = nullptr;
-	std::vector<void*> ptrs; // the kernel's argument block
+	// the kernel's argument block: pointers, then the bytes of the buffers whose
+	// content the caller supplies with every launch
+	std::vector<void*> ptrs;
+	std::map<const void*,std::pair<size_t,size_t>> feeds; // device address -> (offset, bytes) in feed_data
+	std::vector<char> feed_data;
+	std::vector<char> kernarg;
 };
 
 namespace
@@ -704,17 +710,19 @@ int small_append_fx (tcg_ctx* ctx, int dtype, const FxArgs& p)
 
 // resolve: the expression the kernel uses for a device pointer of the recording
 template <typename Resolve>
-std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_t lds_bytes, Resolve resolve)
+std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_t feed_bytes, size_t lds_bytes, Resolve resolve)
 {
 	std::ostringstream o;
 	fx_emit_prelude(o);
-	o << "struct PassPtrs { void* p[" << std::max<size_t>(1, nptrs) << "]; };\n"
+	o << "struct PassPtrs { void* p[" << std::max<size_t>(1, nptrs) << "]; char feed[" << std::max<size_t>(16, feed_bytes) << "]; };\n"
 		"template <typename T> __device__ __forceinline__ T pass_mac (T a, T b, T acc)\n{\n"
 		"if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b + (uint32_t) acc); }\n"
 		"else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, acc); }\n"
 		"else { return __builtin_fma(a, b, acc); }\n}\n"
 		"extern \"C\" __global__ __launch_bounds__(" << PASS_BLOCK << ") void fx (PassPtrs P)\n{\n";
 	if (lds_bytes) { o << "__shared__ __attribute__((aligned(256))) char lds[" << lds_bytes << "];\n"; }
+	// fed buffers are read where the launch put them: in the argument block
+	o << "const char* feed = (const char*) __builtin_amdgcn_kernarg_segment_ptr() + " << std::max<size_t>(1, nptrs) * sizeof(void*) << ";\n";
 	auto lit = [](int64_t v) { return "((int64_t) " + std::to_string(v) + "ll)"; };
 	// index -> coordinates over `n` dims with literal extents, accumulating offsets
 	auto decompose = [&](const char* index, uint32_t n, const uint32_t* size,
@@ -811,6 +819,16 @@ int tcg_small_finish (tcg_ctx* ctx, tcg_graph* g)
 	std::map<const void*,size_t> slot;
 	auto resolve = [&](const void* ptr) -> std::string
 	{
+		auto fed = pass->feeds.upper_bound(ptr);
+		if (fed != pass->feeds.begin())
+		{
+			--fed;
+			const char* begin = (const char*) fed->first;
+			if ((const char*) ptr < begin + fed->second.second)
+			{
+				return "((void*) (feed + " + std::to_string(fed->second.first + (size_t) ((const char*) ptr - begin)) + "))";
+			}
+		}
 		auto it = g->blocks.upper_bound(const_cast<void*>(ptr));
 		if (it != g->blocks.begin())
 		{
@@ -835,11 +853,28 @@ int tcg_small_finish (tcg_ctx* ctx, tcg_graph* g)
 		return "P.p[" + std::to_string(at->second) + "]";
 	};
 	// two passes: the first finds out how much LDS and how many pointers there are
-	(void) pass_source(pass->steps, 1, 0, resolve);
-	TCG_REQUIRE(ctx, slot.size() <= 480, "tcg_capture_end: %zu buffers are too many for a single-launch pass", slot.size());
-	std::string source = pass_source(pass->steps, slot.size(), lds_bytes, resolve);
+	// what the launch supplies is never written by a step
+	for (auto& step : pass->steps)
+	{
+		std::vector<const void*> written;
+		if (step.kind == 0) { written.assign(step.fx.out, step.fx.out + step.fx.nout); }
+		else { written.push_back(step.kind == 1 ? step.ct.out : step.rd.out); }
+		for (const void* w : written)
+		{
+			auto fed = pass->feeds.upper_bound(w);
+			bool hit = fed != pass->feeds.begin() && (const char*) w < (const char*) std::prev(fed)->first + std::prev(fed)->second.second;
+			TCG_REQUIRE(ctx, !hit, "tcg_capture_end: a buffer fed by the launch is written by a step");
+		}
+	}
+	(void) pass_source(pass->steps, 1, 0, 0, resolve);
+	size_t feed_bytes = (pass->feed_data.size() + 15) & ~(size_t) 15;
+	TCG_REQUIRE(ctx, slot.size() * sizeof(void*) + feed_bytes <= 3840,
+		"tcg_capture_end: %zu buffers are too many for a single-launch pass", slot.size());
+	std::string source = pass_source(pass->steps, slot.size(), feed_bytes, lds_bytes, resolve);
 	pass->ptrs.assign(std::max<size_t>(1, slot.size()), nullptr);
 	for (auto& kv : slot) { pass->ptrs[kv.second] = const_cast<void*>(kv.first); }
+	pass->feed_data.resize(std::max<size_t>(16, feed_bytes), 0);
+	pass->kernarg.resize(pass->ptrs.size() * sizeof(void*) + pass->feed_data.size());
 	FxJit& jit = fx_jit();
 	{
 		std::lock_guard<std::mutex> lock(jit.mu);
@@ -860,9 +895,38 @@ int tcg_small_launch (tcg_ctx* ctx, tcg_graph* g)
 {
 	tcg_small_pass* pass = g->pass;
 	if (nullptr == pass || nullptr == pass->fn) { return TCG_OK; }
-	size_t size = pass->ptrs.size() * sizeof(void*);
-	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, pass->ptrs.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+	size_t size = pass->kernarg.size(), ptr_bytes = pass->ptrs.size() * sizeof(void*);
+	memcpy(pass->kernarg.data(), pass->ptrs.data(), ptr_bytes);
+	memcpy(pass->kernarg.data() + ptr_bytes, pass->feed_data.data(), pass->feed_data.size());
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, pass->kernarg.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
 	TCG_HIP(ctx, hipModuleLaunchKernel(pass->fn, 1, 1, 1, PASS_BLOCK, 1, 1, 0, ctx->stream, nullptr, config));
+	return TCG_OK;
+}
+
+int tcg_small_declare_feed (tcg_ctx* ctx, const void* devptr, size_t bytes, const void* host)
+{
+	tcg_small_pass* pass = ctx->capturing->pass;
+	TCG_REQUIRE(ctx, devptr && host && bytes > 0, "tcg_capture_feed: NULL pointer or no bytes");
+	if (pass->feeds.count(devptr)) { return TCG_OK; }
+	size_t offset = (pass->feed_data.size() + 15) & ~(size_t) 15;
+	if (offset + bytes > 1024)
+	{
+		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_capture_feed: more than 1024 bytes fed by the launch");
+	}
+	pass->feed_data.resize(offset + bytes);
+	memcpy(pass->feed_data.data() + offset, host, bytes);
+	pass->feeds.emplace(devptr, std::make_pair(offset, bytes));
+	return TCG_OK;
+}
+
+int tcg_small_feed (tcg_ctx* ctx, tcg_graph* g, const void* devptr, const void* host, size_t bytes)
+{
+	tcg_small_pass* pass = g->pass;
+	TCG_REQUIRE(ctx, pass && host, "tcg_graph_feed: not a single-launch recording");
+	auto it = pass->feeds.find(devptr);
+	TCG_REQUIRE(ctx, it != pass->feeds.end() && it->second.second == bytes,
+		"tcg_graph_feed: %p was not declared with %zu bytes while recording", devptr, bytes);
+	memcpy(pass->feed_data.data() + it->second.first, host, bytes);
 	return TCG_OK;
 }
 

@@ -379,6 +379,20 @@ int tcg_capture_begin_small (tcg_ctx* ctx)
 	return tcg_small_begin(ctx, ctx->capturing);
 }
 
+int tcg_capture_feed (tcg_ctx* ctx, const void* devptr, size_t bytes, const void* host)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, ctx->capturing && ctx->capturing->small, "tcg_capture_feed: no single-launch recording in progress");
+	return tcg_small_declare_feed(ctx, devptr, bytes, host);
+}
+
+int tcg_graph_feed (tcg_ctx* ctx, tcg_graph* graph, const void* devptr, const void* host, size_t bytes)
+{
+	if (!ctx || !graph) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, graph->small, "tcg_graph_feed: not a single-launch recording");
+	return tcg_small_feed(ctx, graph, devptr, host, bytes);
+}
+
 static void graph_release (tcg_ctx* ctx, tcg_graph* g)
 {
 	tcg_small_release(g);

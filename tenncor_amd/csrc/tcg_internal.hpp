@@ -130,6 +130,8 @@ int tcg_small_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[
 int tcg_small_copy (tcg_ctx* ctx, int dtype, int nd, const uint64_t* shape, const int64_t* stride, int64_t offset,
 	const uint64_t* lo, const uint64_t* hi, const void* in, void* out);
 int tcg_small_unsupported (tcg_ctx* ctx, const char* what);
+int tcg_small_declare_feed (tcg_ctx* ctx, const void* devptr, size_t bytes, const void* host);
+int tcg_small_feed (tcg_ctx* ctx, tcg_graph* g, const void* devptr, const void* host, size_t bytes);
 
 // A convolution lowered to a matrix product reads A[m][s] = image[rows[m].off +
 // sums[s].off], or zero when, for some j < ncheck, rows[m].c[j] + sums[s].c[j]

@@ -191,6 +191,9 @@ struct iEigen : public teq::iDeviceRef
 	virtual void* borrow_output (size_t, RTMemptrT&) { return nullptr; }
 	/// After borrow_output: the launch fills only part of the buffer
 	virtual void mark_partial (void) {}
+	/// Leaf storage: where the device copy lives, without bringing it up to
+	/// date (nullptr for anything that is not a leaf or has no device copy yet)
+	virtual const void* device_address (void) const { return nullptr; }
 };
 
 /// Lifetime given to the node whose launch is being enqueued, and a flag the
@@ -305,6 +308,8 @@ struct SrcRef final : public iPermEigen
 	}
 
 	teq::Once<const void*> odevice (void) const override { return teq::Once<const void*>(device_data()); }
+
+	const void* device_address (void) const override { return dev_; }
 
 	/// A kernel wrote the device copy in place (ASSIGN*)
 	void* device_data_mut (void)

@@ -41,6 +41,7 @@ struct ReplayEvaluator::Plan final
 	std::vector<teq::iLeaf*> leaves;
 	std::vector<const void*> leaf_ptrs;
 	std::vector<size_t> leaf_versions;
+	std::vector<size_t> leaf_fed; // bytes the launch carries for the leaf (0: read from device memory)
 	tcg_graph* graph = nullptr;
 	uint64_t bytes = 0;
 	bool fresh = true;
@@ -231,6 +232,29 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 			// the node-by-node pass that follows reports whatever went wrong
 			ok = false;
 		}
+		plan->leaf_fed.assign(plan->leaves.size(), 0);
+		if (ok && as_one_kernel)
+		{
+			// small leaves that no node of the pass updates in place travel with
+			// the launch: a new value costs no copy launch of its own
+			teq::TensSetT updated;
+			for (Observable* f : plan->funcs)
+			{
+				auto op = (egen::_GENERATED_OPCODE) f->get_opcode().code_;
+				if (op >= egen::ASSIGN && op <= egen::ASSIGN_DIV) { updated.emplace(f->get_args().front().get()); }
+			}
+			size_t total = 0;
+			for (size_t i = 0, n = plan->leaves.size(); i < n && ok; ++i)
+			{
+				teq::iLeaf* leaf = plan->leaves[i];
+				size_t bytes = leaf->shape().n_elems() * leaf->get_meta().type_size();
+				if (teq::IMMUTABLE == leaf->get_usage() || updated.count(leaf) || bytes > 256 || total + bytes > 960) { continue; }
+				const void* host = static_cast<const teq::iTensor*>(leaf)->device().data();
+				ok = TCG_OK == tcg_capture_feed(ctx, plan->leaf_ptrs[i], bytes, host);
+				plan->leaf_fed[i] = bytes;
+				total += (bytes + 15) & ~(size_t) 15;
+			}
+		}
 		if (ok)
 		{
 			ok = TCG_OK == tcg_capture_end(ctx, &plan->graph);
@@ -266,10 +290,21 @@ bool ReplayEvaluator::replay (Device& device, Plan& plan)
 	bool stale = plan.fresh || false == plan.effects.empty();
 	for (size_t i = 0, n = plan.leaves.size(); i < n; ++i)
 	{
-		// uploads a leaf whose host copy moved on
-		if (eigen_ref(*plan.leaves[i]).device_data() != plan.leaf_ptrs[i]) { return false; }
 		size_t version = plan.leaves[i]->get_meta().state_version();
-		if (version != plan.leaf_versions[i])
+		bool moved = version != plan.leaf_versions[i];
+		if (plan.leaf_fed[i] > 0)
+		{
+			// the launch carries the value: the device copy stays as it is
+			if (eigen_ref(*plan.leaves[i]).device_address() != plan.leaf_ptrs[i]) { return false; }
+			if (moved)
+			{
+				const void* host = static_cast<const teq::iTensor*>(plan.leaves[i])->device().data();
+				hip_check(tcg_graph_feed(hip_context(), plan.graph, plan.leaf_ptrs[i], host, plan.leaf_fed[i]));
+			}
+		}
+		// uploads a leaf whose host copy moved on
+		else if (eigen_ref(*plan.leaves[i]).device_data() != plan.leaf_ptrs[i]) { return false; }
+		if (moved)
 		{
 			plan.leaf_versions[i] = version;
 			stale = true;

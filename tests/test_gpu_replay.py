@@ -681,3 +681,35 @@ def test_graphs_with_steps_one_kernel_cannot_take_are_recorded_launch_by_launch(
             graph.set_evaluator("plain")
     for a, b in zip(rows["replay"], rows["plain"]):
         np.testing.assert_array_equal(a, b)
+
+
+def test_inputs_that_travel_with_the_launch(ctx):
+    """tcg_capture_feed / tcg_graph_feed: the recorded kernel reads a fed input
+    from its launch arguments; the device memory behind the address is neither
+    read nor written, and feeding a buffer that a step writes is refused."""
+    from tenncor_amd import capi
+    n = 24
+    xs = [np.arange(n, dtype=np.float32) * (k + 1) for k in range(3)]
+    x = ctx.upload(np.full(n, -1, np.float32))   # what the device copy holds is never looked at
+    w = ctx.upload(np.full(n, 2, np.float32))
+    ctx.capture_begin(small=True)
+    prod, total = ctx.alloc(n * 4), ctx.alloc(4)
+    ctx.ew_binary("MUL", capi.FLOAT, n, x.ptr, w.ptr, prod)
+    ctx.reduce("REDUCE_SUM", capi.FLOAT, [n], [0], prod, total)
+    ctx.capture_feed(x.ptr, xs[0])
+    graph = ctx.capture_end()
+    for k, xv in enumerate(xs):
+        if k > 0:
+            ctx.graph_feed(graph, x.ptr, xv)
+        ctx.graph_launch(graph)
+        ctx.graph_launch(graph)
+        np.testing.assert_array_equal(ctx.d2h(total, 1, np.float32), [2 * xv.sum()])
+    np.testing.assert_array_equal(x.get(), np.full(n, -1, np.float32))
+    with pytest.raises(capi.TcgError):
+        ctx.graph_feed(graph, w.ptr, xs[0])      # never declared
+    ctx.graph_destroy(graph)
+    ctx.capture_begin(small=True)
+    ctx.ew_unary("NEG", capi.FLOAT, n, w.ptr, x.ptr)
+    ctx.capture_feed(x.ptr, xs[0])
+    with pytest.raises(capi.TcgError, match="written by a step"):
+        ctx.capture_end()
