@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the operator hot path on one MI355X.
 
-Workload (BASELINE.json configs[1], "elementwise+reduce microbench"): fp32 and
+Workload (the elementwise+reduce microbenchmark, second of the five configurations): fp32 and
 int32 tensors np[4096,16384] (tenncor shape {16384,4096}).  One step evaluates,
 node by node as the reference does (every node materialises its output):
   fp32 : t1=ADD(a,b) t2=MUL(t1,c) t3=EXP(t2) t4=TANH(t3) t5=SIGMOID(t4),
@@ -134,7 +134,7 @@ def run_gpu(steps, warmup, graphs=True):
 
 
 def run_extras(ctx, capi):
-    """Side metrics of BASELINE's metric triple: fused chain, fp32 MATMUL."""
+    """The other parts of the metric triple: fused chain, fp32 MATMUL, PERMUTE."""
     extra = {}
     # fused chain: 3 leaf reads + 1 write
     rng = np.random.default_rng(22)

@@ -1,7 +1,7 @@
 """GPU parity: every entry point of the C ABI against the CPU oracle on the
 same seeded inputs, and against the reference's golden vectors.
 
-Bars (BASELINE north_star): bit-exact for int32 ops and PERMUTE / SLICE / EXTEND
+Bars: bit-exact for int32 ops and PERMUTE / SLICE / EXTEND
 (and the other pure data movement), 1e-5 relative for fp32 elementwise, 1e-4
 relative for fp32 reductions and contractions.  fp32 reductions/contractions are
 compared with the oracle accumulating in fp64, relative to max(|ref|, floor)
@@ -142,6 +142,32 @@ def test_unary_vs_oracle(ctx, ops, oracle, op, np_dtype):
     else:
         rtol = EW_RTOL if np_dtype == np.float32 else 1e-13
         np.testing.assert_allclose(got, ref, rtol=rtol, atol=0)
+
+
+@pytest.mark.parametrize("op", ["TANH", "SIGMOID"])
+def test_fp32_tanh_and_sigmoid_over_their_whole_range(ctx, ops, oracle, op):
+    """fp32 TANH is the rational approximation the reference itself computes
+    with (Eigen 3.3.7's generic_fast_tanh_float) and SIGMOID ends in a 1-ulp
+    reciprocal: against the libm oracle at 1e-5 relative from 1e-30 to
+    saturation, exactly at 0, the limits at infinity, NaN stays NaN."""
+    mags = np.logspace(-30, 2, 40001).astype(np.float32)
+    x = np.concatenate([mags, -mags, np.linspace(-12, 12, 200001).astype(np.float32)])
+    got = ops.unary(op, ops.from_host(ctx, x, [x.size])).get()
+    ref = oracle.unary(op, x)
+    tiny = np.abs(ref) < 1e-30   # sigmoid of large negative arguments underflows: compare absolutely there
+    np.testing.assert_allclose(got[~tiny], ref[~tiny], rtol=EW_RTOL, atol=0)
+    assert np.all(np.abs(got[tiny]) < 1e-30)
+    assert np.all(np.abs(got) <= 1)
+    edge = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 9.0, -9.0, 88.0, -88.0, 104.0, -104.0], np.float32)
+    got = ops.unary(op, ops.from_host(ctx, edge, [edge.size])).get()
+    want = np.tanh(edge.astype(np.float64)) if op == "TANH" else 1 / (1 + np.exp(-edge.astype(np.float64)))
+    assert np.isnan(got[4])
+    np.testing.assert_allclose(np.delete(got, 4), np.delete(want, 4), rtol=EW_RTOL, atol=1e-37)
+    if op == "TANH":
+        # saturation is the value of the approximation at its clamp, one ulp inside (-1, 1)
+        assert got[0] == 0 and got[1] == 0 and np.signbit(got[1]) and got[2] == -got[3] and 1 - 1e-7 <= got[2] <= 1
+    else:
+        assert got[0] == 0.5 and got[2] == 1 and got[3] == 0
 
 
 @pytest.mark.parametrize("op", BINARY)
