@@ -487,7 +487,9 @@ void conv_operand_mode (const ConvGemmPlan& g, tcg_conv_operand& op)
 		if (g.msize[d] > 1 || g.ssize[d] > 1) { f = d; }
 	}
 	if (f < 0 || g.istr[f] != 1 || g.is_col[f]) { return; }
-	op.along_m = g.msize[f] > 1;
+	// both indices may step along the contiguous dim (a spatial dim carries an
+	// output coordinate and a kernel coordinate): the longer run wins
+	op.along_m = g.msize[f] >= g.ssize[f];
 	bool checked = false;
 	for (int j = 0; j < g.ncheck; ++j) { checked = checked || g.check_dim[j] == f; }
 	uint32_t run = op.along_m ? g.msize[f] : g.ssize[f], other = op.along_m ? g.ssize[f] : g.msize[f];
@@ -542,12 +544,12 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 		if (implicit)
 		{
 			conv_operand_mode(g, operand);
-			// gathering element by element inside the product is slower than
-			// materialising A with the coalesced gather kernel (measured on the
-			// image gradient of a 5x5 convolution: 285 vs 300 us, and 214 vs 76 us
-			// on a kernel gradient with 25 rows): only the 128-bit form is used
-			const char* scalar_env = getenv("TCG_CONV_IMPLICIT_SCALAR"); // "1": use it all the same (tests)
-			implicit = operand.vec4 || (scalar_env && scalar_env[0] == '1');
+			// only where the gathers can be 128 bits wide: gathering element by
+			// element inside the product measured slower than materialising A with
+			// the coalesced gather kernel (image gradient of a 5x5 convolution:
+			// 285 vs 300 us for both steps, but 214-253 vs 76 us on a kernel gradient
+			// with 25 rows, whichever index ran along the lanes)
+			implicit = operand.vec4;
 		}
 		for (uint32_t m0 = 0; m0 < g.M && rc == TCG_OK; m0 += chunk)
 		{

@@ -66,11 +66,13 @@ __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_t
 // order in which a slab's sixteen k are summed is a fixed permutation, the
 // same for every element.
 //
-// IMPL: 0 = A is a matrix in memory.  1, 2 = A[m][k] = image[rows[m].off +
+// IMPL: 0 = A is a matrix in memory.  1 = A[m][k] = image[rows[m].off +
 // sums[k].off] or zero (a convolution's operand, never materialised); TA then
-// says which index runs along memory (consecutive m, or consecutive k).
-// 1: aligned groups of four along that index are contiguous and exist or not
-// together (one 128-bit load); 2: element by element.
+// says which index runs along memory (consecutive m, or consecutive k), and
+// aligned groups of four along that index are contiguous and exist or not
+// together: one table lookup and one 128-bit load per group.  A lane's row
+// entries stay in registers; the entry of the summed index is fetched one slab
+// ahead of the load that needs it.
 template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL>
 __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 {
@@ -135,16 +137,28 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 	const f32x4v zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
 	// the table rows a lane gathers from stay the same for every slab
-	constexpr int ROW_ENTS = IMPL == 0 ? 1 : (!TA ? A_VEC : (IMPL == 1 ? 1 : 4));
-	tcg_conv_tab rowent[ROW_ENTS];
+	constexpr int ROW_ENTS = IMPL == 0 ? 1 : (!TA ? A_VEC : 1);
+	tcg_conv_tab rowent[ROW_ENTS], colent[A_VEC];
+	// summed index of chunk v in the slab that starts at k0
+	auto chunk_k = [&] (uint32_t k0, int v) -> uint32_t
+	{
+		int idx = tid + v * 256;
+		return !TA ? k0 + (idx % (BK / 4)) * 4 : k0 + idx / (BM / 4);
+	};
 	if constexpr (IMPL != 0)
 	{
 		static_assert(256 % (BM / 4) == 0, "a lane keeps its rows from slab to slab");
 #pragma unroll
 		for (int e = 0; e < ROW_ENTS; ++e)
 		{
-			uint32_t m = !TA ? m0 + (tid + e * 256) / (BK / 4) : m0 + (tid % (BM / 4)) * 4 + e;
+			uint32_t m = !TA ? m0 + (tid + e * 256) / (BK / 4) : m0 + (tid % (BM / 4)) * 4;
 			rowent[e] = g.rows[m < g.M ? m : g.M - 1];
+		}
+#pragma unroll
+		for (int v = 0; v < A_VEC; ++v)
+		{
+			uint32_t k = chunk_k(k_begin, v);
+			colent[v] = g.sums[k < g.K ? k : g.K - 1];
 		}
 	}
 
@@ -155,63 +169,21 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 		{
 			int idx = tid + v * 256;
 			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
-			if constexpr (IMPL != 0 && !TA)
+			if constexpr (IMPL != 0)
 			{
-				// one row, four consecutive k
-				int mm = idx / (BK / 4), kq = idx % (BK / 4);
-				uint32_t m = m0 + mm, k = k0 + kq * 4;
+				// four consecutive k of one row, or four consecutive rows at one k
+				uint32_t m = !TA ? m0 + idx / (BK / 4) : m0 + (idx % (BM / 4)) * 4;
+				uint32_t k = chunk_k(k0, v);
+				const tcg_conv_tab& row = rowent[!TA ? v : 0];
 				f32x4v val = zero4;
-				if (m < g.M && k < k_end)
+				if (m < g.M && k < k_end && conv_inside(g, row, colent[v]))
 				{
-					if constexpr (IMPL == 1)
-					{
-						const tcg_conv_tab col = g.sums[k];
-						if (conv_inside(g, rowent[v], col))
-						{
-							val = *reinterpret_cast<const f32x4v*>(A + rowent[v].off + col.off);
-						}
-					}
-					else
-					{
-#pragma unroll
-						for (int e = 0; e < 4; ++e)
-						{
-							if (k + e < k_end)
-							{
-								const tcg_conv_tab col = g.sums[k + e];
-								if (conv_inside(g, rowent[v], col)) { val[e] = A[rowent[v].off + col.off]; }
-							}
-						}
-					}
+					val = *reinterpret_cast<const f32x4v*>(A + row.off + colent[v].off);
 				}
 				ra[v] = val;
-			}
-			else if constexpr (IMPL != 0)
-			{
-				// one k, four consecutive rows
-				int kk = idx / (BM / 4), mq = idx % (BM / 4);
-				uint32_t m = m0 + mq * 4, k = k0 + kk;
-				f32x4v val = zero4;
-				if (m < g.M && k < k_end)
-				{
-					const tcg_conv_tab col = g.sums[k];
-					if constexpr (IMPL == 1)
-					{
-						if (conv_inside(g, rowent[0], col))
-						{
-							val = *reinterpret_cast<const f32x4v*>(A + rowent[0].off + col.off);
-						}
-					}
-					else
-					{
-#pragma unroll
-						for (int e = 0; e < 4; ++e)
-						{
-							if (m + e < g.M && conv_inside(g, rowent[e], col)) { val[e] = A[rowent[e].off + col.off]; }
-						}
-					}
-				}
-				ra[v] = val;
+				// the entry the next slab needs is on its way while this one is multiplied
+				uint32_t kn = k + BK;
+				colent[v] = g.sums[kn < g.K ? kn : g.K - 1];
 			}
 			else if constexpr (!TA)
 			{
@@ -531,7 +503,7 @@ int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
 	bool ok = M >= 8 && N >= 8 && S >= 8 && ((M >= 32 && N >= 32) || S >= 512) &&
 		M < (1ull << 31) && N < (1ull << 31) && S < (1ull << 31) &&
 		tcg_aligned16(B) && ldb % 4 == 0 && N % 4 == 0 && op.rows && op.sums && op.ncheck >= 0 && op.ncheck <= 4 &&
-		(false == op.vec4 || (tcg_aligned16(image) && (op.along_m ? M : S) % 4 == 0));
+		op.vec4 && tcg_aligned16(image) && (op.along_m ? M : S) % 4 == 0;
 	if (!ok) { return TCG_OK; }
 	GemmArgs g;
 	g.A = image; g.B = B; g.C = C;
@@ -544,5 +516,5 @@ int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
 	g.ncheck = op.ncheck;
 	for (int j = 0; j < 4; ++j) { g.check_ext[j] = op.check_ext[j]; }
 	*handled = true;
-	return op.vec4 ? dispatch<1>(ctx, g, 1, op.along_m, 0) : dispatch<2>(ctx, g, 1, op.along_m, 0);
+	return dispatch<1>(ctx, g, 1, op.along_m, 0);
 }

@@ -150,6 +150,7 @@ struct tcg_conv_operand
 	int ncheck = 0;
 	// which index runs along memory (consecutive m, or consecutive s), and whether
 	// aligned groups of four of them are contiguous and inside or outside together
+	// (only then can the product read the image itself)
 	bool along_m = false;
 	bool vec4 = false;
 };
