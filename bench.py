@@ -289,7 +289,18 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
         out["config1_mlp%s_evals_per_sec" % tag] = round(1.0 / t, 1)
         out["config1_mlp%s_us_per_eval" % tag] = round(t * 1e6, 1)
         out["config1_mlp_functors"] = g.count_functors(targets)
+        if kind == "replay":
+            out["config1_mlp_replay_launches_per_eval"] = tg.evaluator_stats()["launches"]
         g.close()
+        if kind == "replay":
+            # the same recording kept launch by launch (bit-identical to the walk)
+            tg.set_evaluator("replay_launches")
+            g = tg.Graph()
+            targets, x, _ = configs.config1_mlp(g)
+            t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
+            out["config1_mlp_replay_launch_by_launch_us_per_eval"] = round(t * 1e6, 1)
+            g.close()
+            tg.set_evaluator(kind)
 
         g = tg.Graph()
         targets, x, _, flops = configs.config4_lstm(g)
