@@ -778,6 +778,75 @@ def test_full_size_properties_config2(ctx, ops):
     np.testing.assert_array_equal(ops.permute(prod, [1, 0]).get().reshape(16384, 4096)[5], p_host[:, 5])
 
 
+def test_full_size_properties_config3(ctx, ops):
+    """4096^3 fp32 MATMUL and the batched [64,512,512] product at full size,
+    checked without a CPU product: C r against A (B r) in fp64 for a random
+    vector r (Freivalds), at the 1e-4 bar relative to the largest entry; the
+    int32 product of the same shape exactly (mod 2^32); PERMUTE of the result
+    is an involution and moves rows to columns."""
+    rng = np.random.default_rng(3)
+    n = 4096
+    a = (rng.standard_normal(n * n) / 64).astype(np.float32)
+    b = (rng.standard_normal(n * n) / 64).astype(np.float32)
+    ta, tb = ops.from_host(ctx, a, [n, n]), ops.from_host(ctx, b, [n, n])
+    c = ops.matmul(ta, tb)
+    got = c.get().reshape(n, n).astype(np.float64)
+    r = rng.standard_normal(n)
+    want = a.reshape(n, n).astype(np.float64) @ (b.reshape(n, n).astype(np.float64) @ r)
+    assert np.abs(got @ r - want).max() <= ACC_RTOL * np.abs(want).max()
+    rt = rng.standard_normal(n)   # and from the left: r^T C = (r^T A) B
+    want = (rt @ a.reshape(n, n).astype(np.float64)) @ b.reshape(n, n).astype(np.float64)
+    assert np.abs(rt @ got - want).max() <= ACC_RTOL * np.abs(want).max()
+    ct = ops.permute(c, [1, 0])
+    np.testing.assert_array_equal(ops.permute(ct, [1, 0]).get(), c.get())
+    np.testing.assert_array_equal(ct.get().reshape(n, n)[7], c.get().reshape(n, n)[:, 7])
+    # int32: exact modulo 2^32 whatever the order of summation
+    ai = rng.integers(-1000, 1001, n * n, dtype=np.int32)
+    bi = rng.integers(-1000, 1001, n * n, dtype=np.int32)
+    ci = ops.matmul(ops.from_host(ctx, ai, [n, n]), ops.from_host(ctx, bi, [n, n])).get().reshape(n, n)
+    ri = rng.integers(-3, 4, n).astype(np.int64)
+    want = ai.reshape(n, n).astype(np.int64) @ (bi.reshape(n, n).astype(np.int64) @ ri)
+    np.testing.assert_array_equal((ci.astype(np.int64) @ ri).astype(np.int32), want.astype(np.int32))
+    # batched: np[64,512,512] x np[64,512,512], every batch by Freivalds
+    m, nb = 512, 64
+    a3 = (rng.standard_normal(nb * m * m) / 22).astype(np.float32)
+    b3 = (rng.standard_normal(nb * m * m) / 22).astype(np.float32)
+    c3 = ops.matmul(ops.from_host(ctx, a3, [m, m, nb]), ops.from_host(ctx, b3, [m, m, nb]))
+    got = c3.get().reshape(nb, m, m).astype(np.float64)
+    r = rng.standard_normal(m)
+    want = np.einsum("bij,bj->bi", a3.reshape(nb, m, m).astype(np.float64),
+                     np.einsum("bij,j->bi", b3.reshape(nb, m, m).astype(np.float64), r))
+    assert np.abs(got @ r - want).max() <= ACC_RTOL * np.abs(want).max()
+    swapped = ops.permute(c3, [1, 0, 2]).get().reshape(nb, m, m)
+    np.testing.assert_array_equal(swapped, got.astype(np.float32).transpose(0, 2, 1))
+
+
+@pytest.mark.parametrize("config", ["lstm", "cnn"])
+def test_full_size_recordings_equal_the_walk(config):
+    """configs[3] and configs[4] at their full sizes: the recorded pass (shared
+    launches, exchanged products, convolutions reading their operands in
+    place) against the node-by-node walk on the same input, bit for bit."""
+    from tenncor_amd import graph, configs
+    results = {}
+    for kind in ("plain", "replay_launches"):
+        graph.set_evaluator(kind)
+        g = graph.Graph()
+        try:
+            targets = (configs.config4_lstm if config == "lstm" else configs.config5_cnn)(g)[0]
+            for _ in range(3):  # walked, recorded, replayed
+                g.evaluate(targets)
+            results[kind] = [t.get().copy() for t in targets]
+            if kind != "plain":
+                st = graph.evaluator_stats()
+                assert st["recorded"] == 1 and st["launches"] < 0.4 * g.count_functors(targets) + 40
+        finally:
+            g.close()
+            graph.set_evaluator("plain")
+    for a, b in zip(results["plain"], results["replay_launches"]):
+        assert np.isfinite(a).all()
+        np.testing.assert_array_equal(a, b)
+
+
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
 def test_fused_group_with_views_and_several_outputs(ctx, oracle, np_dtype):
     """tcg_ew_fusedx against the same nodes evaluated one by one by the oracle:
