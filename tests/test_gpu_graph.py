@@ -199,12 +199,15 @@ def torch_or_skip():
     return torch
 
 
-def test_config4_lstm_forward_and_gradient(g, api):
-    """config 4 at reduced size (seq 6, batch 5, in 7, hidden 8): the layer.yml
-    lstm recipe with one fused gate weight {4h, in+h} cut by SLICEs, loss =
-    sum(h^2) over the concatenated hidden outputs, against torch autograd."""
+@pytest.mark.parametrize("seq,batch,nin,hid", [(6, 5, 7, 8), (64, 256, 256, 512)], ids=["reduced", "full_size"])
+def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid):
+    """config 4 at reduced size (seq 6, batch 5, in 7, hidden 8) and at its
+    full size: the layer.yml lstm recipe with one fused gate weight {4h, in+h}
+    cut by SLICEs, loss = sum(h^2) over the concatenated hidden outputs,
+    against torch autograd in fp64."""
     torch = torch_or_skip()
-    seq, batch, nin, hid = 6, 5, 7, 8
+    if batch > 16:
+        torch.set_num_threads(16)
     rng = np.random.default_rng(4)
     w_np = rng.normal(0, 0.05, (nin + hid, 4 * hid)).astype(np.float32)   # np[768,2048] in the config
     x_np = rng.uniform(-1, 1, (batch, seq, nin)).astype(np.float32)       # np[batch,seq,in]
@@ -246,8 +249,8 @@ def test_config4_lstm_forward_and_gradient(g, api):
     close(dw.get(), wt.grad.numpy().reshape(-1), 1e-4)
 
 
-@pytest.mark.parametrize("batch,hw,c1,c2,ncls", [(3, 12, 4, 6, 5), (16, 20, 8, 32, 10)],
-                         ids=["direct_kernels", "matrix_products"])
+@pytest.mark.parametrize("batch,hw,c1,c2,ncls", [(3, 12, 4, 6, 5), (16, 20, 8, 32, 10), (128, 28, 32, 64, 10)],
+                         ids=["direct_kernels", "matrix_products", "full_size"])
 def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls):
     """config 5 at reduced size (5x5 kernels 1->c1->c2, dense c2->ncls): the
     nn.yml conv2d idiom and its gradient idioms (PAD / REVERSE / CONV / PERMUTE
@@ -255,6 +258,8 @@ def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls):
     the direct convolution kernels; at the second the second layer's forward,
     image-gradient and kernel-gradient convolutions run as matrix products."""
     torch = torch_or_skip()
+    if batch > 16:
+        torch.set_num_threads(16)
     F = torch.nn.functional
     rng = np.random.default_rng(5)
     x_np = rng.uniform(0, 1, (batch, hw, hw, 1)).astype(np.float32)
