@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_F32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+MFMA_F64_PEAK_TFLOPS = 78.6  # MI355X dense fp64 matrix, published
 
 ROWS, COLS = 4096, 16384
 N = ROWS * COLS
@@ -190,6 +191,22 @@ def run_extras(ctx, capi):
     extra["matmul_4096_fp32_TFLOPs"] = round(tf, 2)
     extra["matmul_4096_fp32_ms"] = round(ms, 4)
     extra["matmul_4096_frac_of_fp32_mfma_peak"] = round(tf / MFMA_F32_PEAK_TFLOPS, 4)
+    # the same product in double (v_mfma_f64_16x16x4_f64)
+    M2 = 4096
+    a64 = ctx.upload(rng.standard_normal(M2 * M2) / 64)
+    b64 = ctx.upload(rng.standard_normal(M2 * M2) / 64)
+    c64 = ctx.empty(M2 * M2, np.float64)
+    for _ in range(2):
+        ctx.matmul(capi.DOUBLE, [M2, M2], [M2, M2], a64.ptr, b64.ptr, c64.ptr)
+    ctx.timer_begin()
+    for _ in range(reps):
+        ctx.matmul(capi.DOUBLE, [M2, M2], [M2, M2], a64.ptr, b64.ptr, c64.ptr)
+    ms = ctx.timer_end() / reps
+    tf = 2.0 * M2 ** 3 / (ms * 1e-3) / 1e12
+    extra["matmul_4096_fp64_TFLOPs"] = round(tf, 2)
+    extra["matmul_4096_frac_of_fp64_mfma_peak"] = round(tf / MFMA_F64_PEAK_TFLOPS, 4)
+    for buf in (a64, b64, c64):
+        buf.release()
     # PERMUTE of the result (HBM-bound)
     d = ctx.empty(M * M, np.float32)
     order = [1, 0, 2, 3, 4, 5, 6, 7]

@@ -2,14 +2,20 @@
 //
 // tcg_matmul and tcg_contract reduce to batched row-major GEMMs
 // C[b][m][n] = sum_k A[b][m][k] B[b][k][n].  fp32 problems whose operands are
-// 16-byte aligned go to the MFMA kernel (gemm_mfma.hip); everything else
-// (double, int32, odd strides) runs the LDS-tiled kernel below.
+// 16-byte aligned go to the MFMA kernel (gemm_mfma.hip), such fp64 problems to
+// gemm_mfma_f64.hip; everything else (int32, odd strides, small problems) runs
+// the LDS-tiled kernel below.
 #include "tcg_internal.hpp"
 
 int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
 	const float* A, uint64_t lda, uint64_t stride_a, int trans_a,
 	const float* B, uint64_t ldb, uint64_t stride_b, int trans_b,
 	float* C, uint64_t ldc, uint64_t stride_c, bool* handled);
+
+int tcg_gemm_f64_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
+	const double* A, uint64_t lda, uint64_t stride_a, int trans_a,
+	const double* B, uint64_t ldb, uint64_t stride_b, int trans_b,
+	double* C, uint64_t ldc, uint64_t stride_c, bool* handled);
 
 namespace
 {
@@ -170,6 +176,13 @@ int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 		bool handled = false;
 		int rc = tcg_gemm_f32_mfma(ctx, M, N, K, batch, (const float*) A, lda, stride_a, trans_a,
 			(const float*) B, ldb, stride_b, trans_b, (float*) C, ldc, stride_c, &handled);
+		if (rc != TCG_OK || handled) { return rc; }
+	}
+	else if (dtype == TCG_DOUBLE)
+	{
+		bool handled = false;
+		int rc = tcg_gemm_f64_mfma(ctx, M, N, K, batch, (const double*) A, lda, stride_a, trans_a,
+			(const double*) B, ldb, stride_b, trans_b, (double*) C, ldc, stride_c, &handled);
 		if (rc != TCG_OK || handled) { return rc; }
 	}
 	TCG_DISPATCH_TYPE(ctx, dtype, return gemm_generic<T>(ctx, M, N, K, batch,

@@ -1,0 +1,255 @@
+// fp64 GEMM on the matrix cores: C[b][m][n] = sum_k A[b][m][k] B[b][k][n].
+//
+// tenncor's goldens and many of its graphs are double (DOUBLE is the widest
+// dtype of cfg/mintype.yml); the products behind MATMUL / CONTRACT
+// (internal/eigen/operator.hpp:1069-1139) then run here.  One workgroup of 256
+// lanes (4 waves, 2x2) owns a BM x BN tile of C, each wave a quarter of it built
+// from 16x16 accumulators fed by v_mfma_f64_16x16x4_f64 (lane i + 16 k supplies
+// A[i][k] and B[k][i]; a lane holds C[4 r + lane / 16][lane % 16], r = 0..3).
+// A and B slabs of BK = 8 columns go global -> registers -> LDS (double
+// buffered, one barrier per slab), both kept [k][row] so that the sixteen lanes
+// of a k read sixteen consecutive doubles.  Sums run over k in ascending order.
+// MFMA-bound: 2*M*N*K flops against 78.6 TFLOP/s.
+#include "tcg_internal.hpp"
+
+namespace
+{
+
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+constexpr int DBK = 8;
+
+struct DGemmArgs
+{
+	const double* A;
+	const double* B;
+	double* C;
+	uint32_t M, N, K;
+	int64_t lda, ldb, ldc;
+	int64_t batch_a, batch_b, batch_c;
+	uint32_t tiles_m, tiles_n, tiles_per_batch;
+};
+
+// TA: A(m,k) at m + k*lda (M contiguous) instead of m*lda + k.
+// TB: B(k,n) at k + n*ldb (K contiguous) instead of k*ldb + n.
+template <int BM, int BN, bool TA, bool TB>
+__global__ __launch_bounds__(256) void dgemm_mfma_k (DGemmArgs g)
+{
+	constexpr int WM = BM / 2, WN = BN / 2;   // wave tile
+	constexpr int TM = WM / 16, TN = WN / 16; // 16x16 accumulators per wave
+	// pitches of the [k][row] tiles: a 64-bit read goes out in two halves of 32
+	// lanes (two k, sixteen rows each), which land on disjoint banks when the
+	// pitch is 32 dwords past a multiple of 64
+	constexpr int AP = BM + 16, BP = BN + 16;
+	constexpr int A_CHUNKS = BM * DBK / 2, B_CHUNKS = BN * DBK / 2; // double2 per slab
+	constexpr int A_VEC = (A_CHUNKS + 255) / 256, B_VEC = (B_CHUNKS + 255) / 256;
+	__shared__ __attribute__((aligned(16))) double As[2][DBK * AP];
+	__shared__ __attribute__((aligned(16))) double Bs[2][DBK * BP];
+
+	const uint32_t bz = blockIdx.x / g.tiles_per_batch;
+	const uint32_t t = blockIdx.x - bz * g.tiles_per_batch;
+	// neighbouring workgroups share a panel of B
+	const uint32_t tm = t % g.tiles_m, tn = t / g.tiles_m;
+	const uint32_t m0 = tm * BM, n0 = tn * BN;
+	const double* __restrict__ A = g.A + (int64_t) bz * g.batch_a;
+	const double* __restrict__ B = g.B + (int64_t) bz * g.batch_b;
+	double* __restrict__ C = g.C + (int64_t) bz * g.batch_c;
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63, wave = tid >> 6;
+	const int wm = wave >> 1, wn = wave & 1;
+	const int l16 = lane & 15, lk = lane >> 4;
+
+	f64x4 acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+	{
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+		{
+#pragma unroll
+			for (int r = 0; r < 4; ++r) { acc[i][j][r] = 0.0; }
+		}
+	}
+
+	f64x2 ra[A_VEC], rb[B_VEC];
+	const f64x2 zero2 = {0.0, 0.0};
+
+	auto load_slab = [&] (uint32_t k0)
+	{
+#pragma unroll
+		for (int v = 0; v < A_VEC; ++v)
+		{
+			int idx = tid + v * 256;
+			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			if constexpr (!TA)
+			{
+				int mm = idx / (DBK / 2), kq = idx % (DBK / 2);
+				uint32_t m = m0 + mm, k = k0 + kq * 2;
+				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f64x2*>(A + (int64_t) m * g.lda + k) : zero2;
+			}
+			else
+			{
+				int kk = idx / (BM / 2), mq = idx % (BM / 2);
+				uint32_t m = m0 + mq * 2, k = k0 + kk;
+				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f64x2*>(A + (int64_t) k * g.lda + m) : zero2;
+			}
+		}
+#pragma unroll
+		for (int v = 0; v < B_VEC; ++v)
+		{
+			int idx = tid + v * 256;
+			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			if constexpr (!TB)
+			{
+				int kk = idx / (BN / 2), nq = idx % (BN / 2);
+				uint32_t n = n0 + nq * 2, k = k0 + kk;
+				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f64x2*>(B + (int64_t) k * g.ldb + n) : zero2;
+			}
+			else
+			{
+				int nn = idx / (DBK / 2), kq = idx % (DBK / 2);
+				uint32_t n = n0 + nn, k = k0 + kq * 2;
+				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f64x2*>(B + (int64_t) n * g.ldb + k) : zero2;
+			}
+		}
+	};
+
+	auto store_slab = [&] (int buf)
+	{
+		double* as = As[buf];
+		double* bs = Bs[buf];
+#pragma unroll
+		for (int v = 0; v < A_VEC; ++v)
+		{
+			int idx = tid + v * 256;
+			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			if constexpr (!TA)
+			{
+				int mm = idx / (DBK / 2), kq = idx % (DBK / 2);
+				as[(kq * 2) * AP + mm] = ra[v][0];
+				as[(kq * 2 + 1) * AP + mm] = ra[v][1];
+			}
+			else
+			{
+				int kk = idx / (BM / 2), mq = idx % (BM / 2);
+				*reinterpret_cast<f64x2*>(as + kk * AP + mq * 2) = ra[v];
+			}
+		}
+#pragma unroll
+		for (int v = 0; v < B_VEC; ++v)
+		{
+			int idx = tid + v * 256;
+			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			if constexpr (!TB)
+			{
+				int kk = idx / (BN / 2), nq = idx % (BN / 2);
+				*reinterpret_cast<f64x2*>(bs + kk * BP + nq * 2) = rb[v];
+			}
+			else
+			{
+				int nn = idx / (DBK / 2), kq = idx % (DBK / 2);
+				bs[(kq * 2) * BP + nn] = rb[v][0];
+				bs[(kq * 2 + 1) * BP + nn] = rb[v][1];
+			}
+		}
+	};
+
+	const uint32_t nslabs = (g.K + DBK - 1) / DBK;
+	load_slab(0);
+	store_slab(0);
+	__syncthreads();
+	for (uint32_t s = 0; s < nslabs; ++s)
+	{
+		const int buf = s & 1;
+		if (s + 1 < nslabs) { load_slab((s + 1) * DBK); }
+		const double* as = As[buf] + lk * AP + wm * WM + l16;
+		const double* bs = Bs[buf] + lk * BP + wn * WN + l16;
+#pragma unroll
+		for (int ks = 0; ks < DBK / 4; ++ks)
+		{
+			double a[TM], b[TN];
+#pragma unroll
+			for (int i = 0; i < TM; ++i) { a[i] = as[ks * 4 * AP + i * 16]; }
+#pragma unroll
+			for (int j = 0; j < TN; ++j) { b[j] = bs[ks * 4 * BP + j * 16]; }
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+			{
+#pragma unroll
+				for (int j = 0; j < TN; ++j)
+				{
+					acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+				}
+			}
+		}
+		if (s + 1 < nslabs) { store_slab(buf ^ 1); }
+		__syncthreads();
+	}
+
+	// lane holds column l16; register r is row 4*r + lk of the 16x16 block
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+	{
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+		{
+			const uint32_t n = n0 + wn * WN + j * 16 + l16;
+			if (n >= g.N) { continue; }
+#pragma unroll
+			for (int r = 0; r < 4; ++r)
+			{
+				const uint32_t m = m0 + wm * WM + i * 16 + 4 * r + lk;
+				if (m < g.M) { C[(int64_t) m * g.ldc + n] = acc[i][j][r]; }
+			}
+		}
+	}
+}
+
+template <int BM, int BN>
+int dlaunch (tcg_ctx* ctx, DGemmArgs g, uint64_t batch, int trans_a, int trans_b)
+{
+	uint64_t tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+	uint64_t total = tiles_m * tiles_n * batch;
+	TCG_REQUIRE(ctx, total < (1ull << 31), "tcg_gemm: too many tiles for one launch");
+	g.tiles_m = (uint32_t) tiles_m;
+	g.tiles_n = (uint32_t) tiles_n;
+	g.tiles_per_batch = (uint32_t) (tiles_m * tiles_n);
+	const unsigned grid = (unsigned) total;
+	if (!trans_a && !trans_b) { dgemm_mfma_k<BM,BN,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (trans_a && !trans_b) { dgemm_mfma_k<BM,BN,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
+	else if (!trans_a && trans_b) { dgemm_mfma_k<BM,BN,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	else { dgemm_mfma_k<BM,BN,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	TCG_LAUNCH_CHECK(ctx, "dgemm_mfma");
+	return TCG_OK;
+}
+
+} // namespace
+
+int tcg_gemm_f64_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
+	const double* A, uint64_t lda, uint64_t stride_a, int trans_a,
+	const double* B, uint64_t ldb, uint64_t stride_b, int trans_b,
+	double* C, uint64_t ldc, uint64_t stride_c, bool* handled)
+{
+	*handled = false;
+	// 128-bit operand loads: every row start and every slab offset 16-byte aligned;
+	// problems too small to fill the chip with 64x64 tiles stay on the generic kernel
+	bool ok = M >= 32 && N >= 32 && K >= 8 &&
+		M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31) &&
+		((M + 63) / 64) * ((N + 63) / 64) * batch >= (uint64_t) ctx->num_cus / 2 &&
+		tcg_aligned16(A) && tcg_aligned16(B) &&
+		lda % 2 == 0 && ldb % 2 == 0 && stride_a % 2 == 0 && stride_b % 2 == 0 &&
+		((trans_a ? M : K) % 2 == 0) && ((trans_b ? K : N) % 2 == 0);
+	if (!ok) { return TCG_OK; }
+	DGemmArgs g;
+	g.A = A; g.B = B; g.C = C;
+	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) K;
+	g.lda = (int64_t) lda; g.ldb = (int64_t) ldb; g.ldc = (int64_t) ldc;
+	g.batch_a = (int64_t) stride_a; g.batch_b = (int64_t) stride_b; g.batch_c = (int64_t) stride_c;
+	g.tiles_m = g.tiles_n = g.tiles_per_batch = 0;
+	*handled = true;
+	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
+	if (big_tiles >= (uint64_t) ctx->num_cus) { return dlaunch<128,128>(ctx, g, batch, trans_a, trans_b); }
+	return dlaunch<64,64>(ctx, g, batch, trans_a, trans_b);
+}

@@ -451,6 +451,33 @@ def test_gemm_transposed_operands_vs_oracle(ctx, oracle, M, N, K, batch, ta, tb)
     assert_acc_close(dc.get(), ref)
 
 
+GEMM_F64_CASES = [
+    # on the fp64 matrix-core path: even extents, enough tiles to fill the chip
+    (1024, 1024, 64, 1, 0, 0), (1024, 1024, 64, 1, 1, 0), (1024, 1024, 64, 1, 0, 1), (1024, 1024, 64, 1, 1, 1),
+    (1500, 1100, 42, 1, 0, 0), (1500, 1100, 42, 1, 1, 1), (2048, 2050, 130, 1, 1, 0), (2050, 2048, 130, 1, 0, 1),
+    (260, 132, 72, 24, 0, 0), (260, 132, 72, 24, 1, 0), (132, 260, 10, 24, 0, 1), (100, 36, 40, 80, 1, 1),
+    # off it: odd extents, few tiles
+    (1025, 1023, 33, 1, 0, 0), (128, 128, 64, 1, 0, 0), (33, 35, 17, 2, 1, 1),
+]
+
+
+@pytest.mark.parametrize("M,N,K,batch,ta,tb", GEMM_F64_CASES, ids=[str(c) for c in GEMM_F64_CASES])
+def test_gemm_f64_transposed_operands_vs_oracle(ctx, oracle, M, N, K, batch, ta, tb):
+    """tcg_gemm in double: the matrix-core kernel and the generic one sum over k in ascending order."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of(M, N, K, batch, ta, tb, 64))
+    a = rng.standard_normal(batch * M * K)
+    b = rng.standard_normal(batch * K * N) / np.sqrt(K)
+    a_can = a if not ta else oracle.permute(a, [M, K, batch], [1, 0, 2])[0]
+    b_can = b if not tb else oracle.permute(b, [K, N, batch], [1, 0, 2])[0]
+    ref, _ = oracle.matmul(a_can, [K, M, batch], b_can, [N, K, batch])
+    da, db = ctx.upload(a), ctx.upload(b)
+    dc = ctx.empty(batch * M * N, np.float64)
+    ctx.gemm(capi.DOUBLE, M, N, K, batch, da.ptr, M if ta else K, M * K, ta,
+             db.ptr, K if tb else N, K * N, tb, dc.ptr, N, M * N)
+    assert_acc_close(dc.get(), ref, rtol=1e-12)
+
+
 CONTRACT_CASES = [
     ([10, 3], [9, 10], [[0, 1]]),                      # dense layer (config 1)
     ([768, 1, 64], [512, 768], [[0, 1]]),              # LSTM gate product (config 4)
