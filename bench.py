@@ -180,10 +180,12 @@ def run_extras(ctx, capi):
     a = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
     b = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
     c = ctx.empty(M * M, np.float32)
-    for _ in range(2):
+    # the matrix clock takes some 30 ms of matrix work to settle after the
+    # streaming kernels above: the timed launches start once it has
+    for _ in range(40):
         ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
     ctx.timer_begin()
-    reps = 5
+    reps = 20
     for _ in range(reps):
         ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
     ms = ctx.timer_end() / reps
@@ -196,7 +198,7 @@ def run_extras(ctx, capi):
     a64 = ctx.upload(rng.standard_normal(M2 * M2) / 64)
     b64 = ctx.upload(rng.standard_normal(M2 * M2) / 64)
     c64 = ctx.empty(M2 * M2, np.float64)
-    for _ in range(2):
+    for _ in range(10):
         ctx.matmul(capi.DOUBLE, [M2, M2], [M2, M2], a64.ptr, b64.ptr, c64.ptr)
     ctx.timer_begin()
     for _ in range(reps):
@@ -225,7 +227,7 @@ def run_extras(ctx, capi):
     b = ctx.upload((rng.standard_normal(nb * m * m) / np.sqrt(m)).astype(np.float32))
     c = ctx.empty(nb * m * m, np.float32)
     d = ctx.empty(nb * m * m, np.float32)
-    for _ in range(2):
+    for _ in range(40):
         ctx.matmul(capi.FLOAT, [m, m, nb], [m, m, nb], a.ptr, b.ptr, c.ptr)
     ctx.timer_begin()
     for _ in range(reps):
