@@ -19,6 +19,8 @@ typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 
 constexpr int DBK = 8;
+constexpr int DNXCD = 8;
+constexpr int DGROUP_M = 8;
 
 struct DGemmArgs
 {
@@ -28,7 +30,7 @@ struct DGemmArgs
 	uint32_t M, N, K;
 	int64_t lda, ldb, ldc;
 	int64_t batch_a, batch_b, batch_c;
-	uint32_t tiles_m, tiles_n, tiles_per_batch;
+	uint32_t tiles_m, tiles_n, tiles_per_batch, total_tiles;
 };
 
 // TA: A(m,k) at m + k*lda (M contiguous) instead of m*lda + k.
@@ -47,10 +49,23 @@ __global__ __launch_bounds__(256) void dgemm_mfma_k (DGemmArgs g)
 	__shared__ __attribute__((aligned(16))) double As[2][DBK * AP];
 	__shared__ __attribute__((aligned(16))) double Bs[2][DBK * BP];
 
-	const uint32_t bz = blockIdx.x / g.tiles_per_batch;
-	const uint32_t t = blockIdx.x - bz * g.tiles_per_batch;
-	// neighbouring workgroups share a panel of B
-	const uint32_t tm = t % g.tiles_m, tn = t / g.tiles_m;
+	// workgroups resident on one XCD (ids congruent mod 8) take consecutive
+	// tiles, and consecutive tiles walk down groups of eight tile rows: what an
+	// XCD works on at a time is a compact patch of C whose panels its L2 holds
+	uint32_t id = blockIdx.x;
+	if (g.total_tiles % DNXCD == 0)
+	{
+		id = (id % DNXCD) * (g.total_tiles / DNXCD) + id / DNXCD;
+	}
+	const uint32_t bz = id / g.tiles_per_batch;
+	const uint32_t t = id - bz * g.tiles_per_batch;
+	const uint32_t group_size = DGROUP_M * g.tiles_n;
+	const uint32_t group = t / group_size;
+	const uint32_t first_m = group * DGROUP_M;
+	const uint32_t rows_in_group = g.tiles_m - first_m < (uint32_t) DGROUP_M ? g.tiles_m - first_m : DGROUP_M;
+	const uint32_t in_group = t - group * group_size;
+	const uint32_t tm = first_m + in_group % rows_in_group;
+	const uint32_t tn = in_group / rows_in_group;
 	const uint32_t m0 = tm * BM, n0 = tn * BN;
 	const double* __restrict__ A = g.A + (int64_t) bz * g.batch_a;
 	const double* __restrict__ B = g.B + (int64_t) bz * g.batch_b;
@@ -216,6 +231,7 @@ int dlaunch (tcg_ctx* ctx, DGemmArgs g, uint64_t batch, int trans_a, int trans_b
 	g.tiles_m = (uint32_t) tiles_m;
 	g.tiles_n = (uint32_t) tiles_n;
 	g.tiles_per_batch = (uint32_t) (tiles_m * tiles_n);
+	g.total_tiles = (uint32_t) total;
 	const unsigned grid = (unsigned) total;
 	if (!trans_a && !trans_b) { dgemm_mfma_k<BM,BN,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
 	else if (trans_a && !trans_b) { dgemm_mfma_k<BM,BN,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
@@ -247,7 +263,7 @@ int tcg_gemm_f64_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) K;
 	g.lda = (int64_t) lda; g.ldb = (int64_t) ldb; g.ldc = (int64_t) ldc;
 	g.batch_a = (int64_t) stride_a; g.batch_b = (int64_t) stride_b; g.batch_c = (int64_t) stride_c;
-	g.tiles_m = g.tiles_n = g.tiles_per_batch = 0;
+	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	*handled = true;
 	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
 	if (big_tiles >= (uint64_t) ctx->num_cus) { return dlaunch<128,128>(ctx, g, batch, trans_a, trans_b); }

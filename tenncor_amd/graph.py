@@ -440,11 +440,15 @@ class Api:
             out = self.add(out, self.extend_like(bias, out))
         return self.identity(out)
 
-    def conv2d(self, image, kernel, bias=None):
-        """nn.yml:76-98 without explicit zero padding: image {in,w,h,batch},
-        kernel {out,in,kw,kh} -> {out,w',h',batch}."""
+    def conv2d(self, image, kernel, bias=None, zero_padding=((0, 0), (0, 0))):
+        """nn.yml:48-98: image {in,w,h,batch}, kernel {out,in,kw,kh} ->
+        {out,w',h',batch}; zero_padding = ((before, after) along the width,
+        (before, after) along the height)."""
+        cimage = image
+        if any(p > 0 for pair in zero_padding for p in pair):
+            cimage = self.pad(cimage, [(0, 0), tuple(zero_padding[0]), tuple(zero_padding[1])])
         img_pad = kernel.shape[0] - 1
-        cimage = self.pad(image, [(0, 0)] * 4 + [(img_pad, img_pad)])
+        cimage = self.pad(cimage, [(0, 0)] * 4 + [(img_pad, img_pad)])
         out = self.permute(self.convolution(cimage, self.reverse(kernel, [0]), [4, 0, 1, 2]), [4, 1, 2, 3])
         if bias is not None:
             out = self.add(out, self.extend_like(bias, out))
@@ -492,11 +496,27 @@ class Approx:
     def __init__(self, api):
         self.api = api
         self.g = api.g
+        self.slots = {}  # label -> the state variables created under it, in order
+
+    def _typed(self, like, *values):
+        """Scalars in the dtype of the variables, as the reference's templates
+        hold them (``T nodecay = 1. - decay``): 1 - 0.999f is 0.000999987."""
+        np_dtype = capi.NP_OF[like.dtype]
+        return [np_dtype(v) for v in values]
+
+    def _epsilon(self, like, epsilon):
+        """std::numeric_limits<T>::epsilon(), the default of every rule's epsilon."""
+        if epsilon is not None:
+            return epsilon
+        np_dtype = capi.NP_OF[like.dtype]
+        return float(np.finfo(np_dtype).eps) if np.issubdtype(np_dtype, np.floating) else 0
 
     def _variable_like(self, scalar, like, label):
         """eteq::make_variable_like (tenncor/eteq/make.hpp:185-200)."""
         np_dtype = capi.NP_OF[like.dtype]
-        return self.g.variable(np.full(capi.n_elems(like.shape), scalar, np_dtype), like.shape, label)
+        var = self.g.variable(np.full(capi.n_elems(like.shape), scalar, np_dtype), like.shape, label)
+        self.slots.setdefault(label, []).append(var)
+        return var
 
     def sgd(self, error, variables, learning_rate=0.5):
         """approx.yml:12-52: x -= learning_rate * f'(x)."""
@@ -504,60 +524,67 @@ class Approx:
         ders = self.g.derive(error, variables)
         return [(x, a.assign_sub(x, a.mul(der, learning_rate))) for x, der in zip(variables, ders)]
 
-    def adagrad(self, error, variables, learning_rate=0.5, epsilon=float(np.finfo(np.float32).eps)):
+    def adagrad(self, error, variables, learning_rate=0.5, epsilon=None):
         """approx.yml:53-94: momentum += f'(x)^2; x -= lr f'(x) / (sqrt(momentum) + eps)."""
         a = self.api
         out = []
         for x, der in zip(variables, self.g.derive(error, variables)):
             momentum = self._variable_like(1, der, "momentum")
             update = a.assign_add(momentum, a.square(der))
-            out.append((x, a.assign_sub(x, a.div(a.mul(der, learning_rate), a.add(a.sqrt(update), epsilon)))))
+            out.append((x, a.assign_sub(x, a.div(a.mul(der, learning_rate), a.add(a.sqrt(update), self._epsilon(der, epsilon))))))
         return out
 
     def adam(self, error, variables, step_rate=0.001, decay1=0.9, decay2=0.999,
-             epsilon=float(np.finfo(np.float32).eps)):
+             epsilon=None):
         """approx.yml:95-176."""
         a = self.api
         out = []
         for x, der in zip(variables, self.g.derive(error, variables)):
+            decay1, decay2 = self._typed(der, decay1, decay2)
+            nodecay1, nodecay2 = float(1 - decay1), float(1 - decay2)
+            decay1, decay2 = float(decay1), float(decay2)
             m = self._variable_like(0, der, "moment1")
             v = self._variable_like(0, der, "moment2")
             t = self._variable_like(0, der, "t")
             one_t = a._like(1, der)
-            next_m = a.assign(m, a.add(a.mul(decay1, m), a.mul(1.0 - decay1, der)))
-            next_v = a.assign(v, a.add(a.mul(decay2, v), a.mul(1.0 - decay2, a.square(der))))
+            next_m = a.assign(m, a.add(a.mul(decay1, m), a.mul(nodecay1, der)))
+            next_v = a.assign(v, a.add(a.mul(decay2, v), a.mul(nodecay2, a.square(der))))
             incr = a.assign_add(t, one_t)
             m_corr = a.div(next_m, a.sub(one_t, a.pow(decay1, incr)))
             v_corr = a.div(next_v, a.sub(one_t, a.pow(decay2, incr)))
-            delta = a.mul(step_rate, a.div(m_corr, a.add(a.sqrt(v_corr), epsilon)))
+            delta = a.mul(step_rate, a.div(m_corr, a.add(a.sqrt(v_corr), self._epsilon(der, epsilon))))
             out.append((x, a.assign_sub(x, delta)))
         return out
 
     def adadelta(self, error, variables, step_rate=1.0, decay=0.9, offset=0.0001,
-                 epsilon=float(np.finfo(np.float32).eps)):
+                 epsilon=None):
         """approx.yml:177-247."""
         a = self.api
         out = []
         for x, der in zip(variables, self.g.derive(error, variables)):
+            (decay,) = self._typed(der, decay)
+            nodecay, decay = float(1 - decay), float(decay)
             msg = self._variable_like(0, der, "ex_sqr_grad")
             msd = self._variable_like(0, der, "ex_sqr_delx")
-            msg_next = a.assign(msg, a.add(a.mul(decay, msg), a.mul(1.0 - decay, a.square(der))))
+            msg_next = a.assign(msg, a.add(a.mul(decay, msg), a.mul(nodecay, a.square(der))))
             delta = a.mul(a.mul(step_rate, a.div(a.sqrt(a.add(msd, offset)),
-                                                 a.add(a.sqrt(a.add(msg_next, offset)), epsilon))), der)
-            msd_next = a.assign(msd, a.add(a.mul(decay, msd), a.mul(1.0 - decay, a.square(delta))))
+                                                 a.add(a.sqrt(a.add(msg_next, offset)), self._epsilon(der, epsilon)))), der)
+            msd_next = a.assign(msd, a.add(a.mul(decay, msd), a.mul(nodecay, a.square(delta))))
             out.append((x, a.assign_sub(x, a.identity(delta, [msd_next]))))
         return out
 
     def rms_momentum(self, error, variables, learning_rate=0.5, discount_factor=0.99,
-                     epsilon=float(np.finfo(np.float32).eps)):
+                     epsilon=None):
         """approx.yml:248-304."""
         a = self.api
         out = []
         for x, der in zip(variables, self.g.derive(error, variables)):
+            (discount_factor,) = self._typed(der, discount_factor)
+            nodiscount, discount_factor = float(1 - discount_factor), float(discount_factor)
             momentum = self._variable_like(1, der, "momentum")
             update = a.assign(momentum, a.add(a.mul(discount_factor, momentum),
-                                              a.mul(1.0 - discount_factor, a.square(der))))
-            out.append((x, a.assign_sub(x, a.div(a.mul(der, learning_rate), a.add(a.sqrt(update), epsilon)))))
+                                              a.mul(nodiscount, a.square(der))))
+            out.append((x, a.assign_sub(x, a.div(a.mul(der, learning_rate), a.add(a.sqrt(update), self._epsilon(der, epsilon))))))
         return out
 
     def apply_update(self, error, updates):

@@ -7,6 +7,8 @@
 #ifndef TCH_ETEQ_HPP
 #define TCH_ETEQ_HPP
 
+#include <sstream>
+
 #include "eigen_ops.hpp"
 #include "oprules.hpp"
 
@@ -87,15 +89,13 @@ struct Constant final : public teq::iLeaf
 	{
 		const T* data = (const T*) static_cast<const eigen::iEigen&>(ref_).data();
 		size_t n = shape_.n_elems();
+		// stream formatting, six significant digits: the labels the reference's
+		// tests expect (tenncor/test/test_approx.cpp:85 "1.19209e-07", :462 "0.000999987")
 		auto fmt = [](T v)
 		{
-			std::string s = std::to_string(v);
-			if (s.find('.') != std::string::npos)
-			{
-				while (s.back() == '0') { s.pop_back(); }
-				if (s.back() == '.') { s.pop_back(); }
-			}
-			return s;
+			std::ostringstream s;
+			s << v;
+			return s.str();
 		};
 		if (std::all_of(data + 1, data + n, [&](const T& e) { return e == data[0]; })) { return fmt(data[0]); }
 		std::string out = "[";

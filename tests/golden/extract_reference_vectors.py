@@ -4,8 +4,10 @@ reference's own C++ tests hold.
 Run once in the authoring container (the reference tree is not available where
 the GPU tests run): ``python tests/golden/extract_reference_vectors.py``.
 It only reads the test sources as text: every ``std::vector<T> name = {...};``
-(or ``name{...}``) inside a given line range becomes ``name -> list`` and the
-result is committed as data.  Nothing of the reference is executed and no
+(or ``name{...}``) inside a given line range becomes ``name -> list``, every
+``double name = literal;`` becomes ``name -> number``, every printed graph a
+test expects (the adjacent string literals of an ``EXPECT_GRAPHEQ``) becomes
+one string, and the result is committed as data.  Nothing of the reference is executed and no
 source text is kept.
 """
 import ast
@@ -21,6 +23,8 @@ VEC_RE = re.compile(
     r"std::vector<\s*(double|float|int32_t)\s*>\s*(\w+)\s*(?:=\s*)?\{(.*?)\}\s*;", re.S)
 DIMS_RE = re.compile(r"teq::DimsT\s+(\w+)\s*=\s*\{(.*?)\}\s*;", re.S)
 SHAPE_RE = re.compile(r"teq::Shape\s+(\w+)\s*\(\s*\{(.*?)\}\s*\)\s*;", re.S)
+SCALAR_RE = re.compile(r"\b(?:double|float)\s+(\w+)\s*=\s*([0-9eE+\-.]+)f?\s*;")
+LITERAL_LINE_RE = re.compile(r'^\s*"((?:[^"\\]|\\.)*)"[^"]*$')
 
 
 def _strip_comments(text):
@@ -68,7 +72,29 @@ def read_block(relpath, first, last):
         out[name] = [int(v) for v in _numbers(body)]
     for name, body in SHAPE_RE.findall(text):
         out[name] = [int(v) for v in _numbers(body)]
+    for name, literal in SCALAR_RE.findall(text):
+        out[name] = float(literal)
     return out
+
+
+def _unescape(body):
+    return re.sub(r"\\(.)", lambda m: {"n": "\n", "t": "\t"}.get(m.group(1), m.group(1)), body)
+
+
+def read_expected_graphs(relpath, first, last):
+    """The printed graphs of the EXPECT_GRAPHEQ calls in a line range, in order:
+    runs of lines that hold nothing but a string literal."""
+    with open(os.path.join(REF, relpath)) as f:
+        lines = f.readlines()[first - 1:last]
+    graphs, run = [], []
+    for line in lines + [""]:
+        m = LITERAL_LINE_RE.match(line)
+        if m and ("`--" in m.group(1) or m.group(1).startswith("(")):
+            run.append(_unescape(m.group(1)))
+        elif run:
+            graphs.append("".join(run))
+            run = []
+    return graphs
 
 
 BLOCKS = {
@@ -85,7 +111,32 @@ BLOCKS = {
 }
 
 
+GRAPH_BLOCKS = {
+    # optimiser update rules: the graph each builds and the values one step leaves
+    "approx_sgd": ("tenncor/test/test_approx.cpp", 21, 45),
+    "approx_adagrad": ("tenncor/test/test_approx.cpp", 48, 86),
+    "approx_adadelta": ("tenncor/test/test_approx.cpp", 89, 286),
+    "approx_rms_momentum": ("tenncor/test/test_approx.cpp", 289, 385),
+    "approx_adam": ("tenncor/test/test_approx.cpp", 388, 512),
+    # a convolution layer trained one adadelta step: inputs and the error after the step
+    "opt_cnn_layer": ("tenncor/test/test_opt.cpp", 261, 408),
+}
+
+
+def write_graph_fixtures():
+    fixtures = {}
+    for key, (path, first, last) in GRAPH_BLOCKS.items():
+        fixtures[key] = read_block(path, first, last)
+        if key.startswith("approx_"):
+            fixtures[key]["expected_graphs"] = read_expected_graphs(path, first, last)
+        names = [k for k in fixtures[key] if not k.startswith("_")]
+        print("%-22s %s" % (key, ", ".join(names)))
+    with open(os.path.join(HERE, "approx_goldens.json"), "w") as f:
+        json.dump(fixtures, f, indent=0, separators=(",", ":"))
+
+
 def main():
+    write_graph_fixtures()
     fixtures = {}
     for key, (path, first, last) in BLOCKS.items():
         fixtures[key] = read_block(path, first, last)

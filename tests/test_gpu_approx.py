@@ -1,0 +1,117 @@
+"""One optimisation step of the update rules on the GPU against the values the
+reference's own tests expect (tenncor/test/test_approx.cpp:142-285 adadelta,
+:329-385 rms_momentum, :480-512 adam) and the error a convolution layer has
+after one adadelta step (tenncor/test/test_opt.cpp:261-408, in double), from
+tests/golden/approx_goldens.json.  The expected values depend on the order in
+which the assignments inside a rule run (the reference's comments work the
+alternatives out): the state of a rule is updated before the variable.
+
+Tolerances: those of the reference's assertions (1e-3 relative for the states
+and the variable, exact for the rms momentum); 1e-9 relative for the layer
+error, whose reference value was computed from a graph rewritten by
+conversions this build does not have (cfg/optimizations.json is absent).
+Every case runs under the node-by-node walk and under both replaying
+evaluators.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "approx_goldens.json")) as _f:
+    GOLD = json.load(_f)
+
+EVALUATORS = ["plain", "replay_launches", "replay"]
+
+
+@pytest.fixture(params=EVALUATORS)
+def env(request):
+    from tenncor_amd import graph
+    graph.set_evaluator(request.param)
+    g = graph.Graph()
+    api = graph.Api(g)
+    try:
+        yield g, api, graph.Approx(api)
+    finally:
+        g.close()
+        graph.set_evaluator("plain")
+
+
+def assert_rel(got, expected, rtol):
+    got = np.asarray(got, np.float64)
+    assert np.all(np.abs((expected - got) / expected) < rtol), "expect %r, got %r" % (expected, got[:4])
+
+
+def test_adadelta_step_runs_its_assignments_in_order(env):
+    g, api, approx = env
+    gold = GOLD["approx_adadelta"]
+    leaf = g.variable(np.zeros(18 * 9 * 3, np.float32), gold["slist"], "leaf")
+    groups = approx.adadelta(api.unary("SIN", leaf), [leaf], gold["step_rate"], gold["decay"], gold["offset"])
+    g.evaluate([groups[0][1]])
+    assert_rel(approx.slots["ex_sqr_grad"][0].get(), gold["exog"], 1e-3)
+    assert_rel(approx.slots["ex_sqr_delx"][0].get(), gold["exod"], 1e-3)
+    assert_rel(leaf.get(), gold["exdval"], 1e-3)
+    assert_rel(groups[0][1].get(), gold["exdval"], 1e-3)
+
+
+def test_rms_momentum_step(env):
+    g, api, approx = env
+    gold = GOLD["approx_rms_momentum"]
+    leaf = g.variable(np.zeros(5, np.float32), gold["shape"], "leaf")
+    err = api.div(api.unary("SIN", leaf), 2.0)
+    groups = approx.rms_momentum(err, [leaf], gold["learning_rate"], gold["discount_rate"],
+                                 float(np.finfo(np.float32).eps))
+    g.evaluate([groups[0][1]])
+    # momentum = 0.52 * 1 + 0.48 * 0.5^2: the reference compares with == 0.64f
+    np.testing.assert_array_equal(approx.slots["momentum"][0].get(), np.full(5, 0.64, np.float32))
+    assert_rel(leaf.get(), gold["exdval"], 1e-3)
+
+
+def test_adam_converges_and_counts_its_steps(env):
+    g, api, approx = env
+    x = g.variable(np.zeros(1, np.float32), [], "x")
+    loss = api.add(api.sub(api.square(x), api.mul(2.0, x)), 1.0)
+    step = approx.adam(loss, [x], 0.01, 0.9, 0.999, 1e-8)[0][1]
+    limit = 1000
+    i = 0
+    while i < limit:
+        before = x.get()[0]
+        g.evaluate([step])
+        if before == x.get()[0]:
+            break
+        i += 1
+    assert i < limit
+    assert abs(1 - x.get()[0]) < 1e-4
+    assert approx.slots["t"][0].get()[0] == i + 1
+
+
+def test_convolution_layer_error_after_one_adadelta_step(env):
+    g, api, approx = env
+    gold = GOLD["opt_cnn_layer"]
+    invar = g.variable(np.array(gold["in_data"]), gold["in_shape"], "invar")
+    outvar = g.variable(np.array(gold["out_data"]), gold["out_shape"], "outvar")
+    # conv2d<double>({3, 3}, 2, 2, ...): the weight {out 2, in 2, 3, 3} takes the
+    # first 36 of the 54 values the test holds
+    weight = g.variable(np.array(gold["cweight_data"][:36]), [2, 2, 3, 3], "weight")
+    bias = g.variable(np.array(gold["cbias_data"]), [2], "bias")
+    eps = float(np.finfo(np.float64).eps)
+    normalized = api.sub(api.div(invar, 255.0), 0.5)
+
+    def error_of(w, b):
+        out = api.relu(api.conv2d(normalized, w, b, zero_padding=((1, 1), (1, 1))))
+        return api.neg(api.reduce_sum(api.mul(outvar, api.log(api.add(out, eps)))))
+
+    error = error_of(weight, bias)
+    updates = approx.adadelta(error, [weight, bias], gold["learning_rate"], gold["l2_decay"])
+    # layr::trail (tenncor/layr/layer.hpp:57-118): the error again, reading the
+    # variables through their assignments, i.e. after the step
+    trailed = error_of(updates[0][1], updates[1][1])
+    err = api.identity(trailed, [assign for _, assign in updates])
+    g.evaluate([err])
+    got = err.get()
+    assert got.shape == (1,)
+    assert abs(got[0] - gold["evdata"]) <= 1e-9 * gold["evdata"], got[0]

@@ -1,0 +1,92 @@
+"""The graphs the optimiser update rules build, line by line against the
+printed graphs the reference's own tests expect
+(tenncor/test/test_approx.cpp:21-45 sgd, :48-86 adagrad, :89-193 adadelta,
+:289-327 rms_momentum, :388-478 adam), held in tests/golden/approx_goldens.json.
+The rules are those of cfg/tenncor/approx.yml; the derivative subgraphs inside
+them come from the gradient builder (tenncor/eteq/backprop.hpp).  Lines are
+compared as the reference compares them: leading and trailing '_' and blanks
+stripped, empty lines dropped (testutil/src/graph_comp.cpp:29-52).  Host logic
+only: no GPU.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+with open(os.path.join(HERE, "golden", "approx_goldens.json")) as _f:
+    GOLD = json.load(_f)
+
+EPS32 = "1.19209e-07"  # std::numeric_limits<float>::epsilon() through a stream
+
+
+def lines_of(text):
+    out = [line.strip("_ \t") for line in text.split("\n")]
+    return [line for line in out if line]
+
+
+@pytest.fixture()
+def env():
+    from tenncor_amd import graph
+    g = graph.Graph()
+    api = graph.Api(g)
+    yield g, api, graph.Approx(api)
+    g.close()
+
+
+def expect_graph(g, node, key, fill=()):
+    expected = GOLD[key]["expected_graphs"][0]
+    if fill:
+        expected = expected % fill
+    assert lines_of(g.to_string(node)) == lines_of(expected)
+
+
+def test_sgd_graph(env):
+    g, api, approx = env
+    leaf = g.variable(np.zeros(18 * 9 * 3, np.float32), GOLD["approx_sgd"]["slist"], "leaf")
+    groups = approx.sgd(api.unary("ABS", leaf), [leaf], 0.67)
+    assert len(groups) == 1
+    expect_graph(g, groups[0][1], "approx_sgd")
+
+
+def test_adagrad_graph(env):
+    g, api, approx = env
+    leaf = g.variable(np.zeros(18 * 9 * 3, np.float32), GOLD["approx_adagrad"]["slist"], "leaf")
+    groups = approx.adagrad(api.unary("ABS", leaf), [leaf], 0.67)
+    expect_graph(g, groups[0][1], "approx_adagrad")
+
+
+def test_adadelta_graph(env):
+    g, api, approx = env
+    gold = GOLD["approx_adadelta"]
+    leaf = g.variable(np.zeros(18 * 9 * 3, np.float32), gold["slist"], "leaf")
+    groups = approx.adadelta(api.unary("SIN", leaf), [leaf], gold["step_rate"], gold["decay"], gold["offset"])
+    expect_graph(g, groups[0][1], "approx_adadelta", (EPS32, EPS32))
+
+
+def test_rms_momentum_graph(env):
+    g, api, approx = env
+    gold = GOLD["approx_rms_momentum"]
+    leaf = g.variable(np.zeros(5, np.float32), gold["shape"], "leaf")
+    err = api.div(api.unary("SIN", leaf), 2.0)
+    groups = approx.rms_momentum(err, [leaf], gold["learning_rate"], gold["discount_rate"],
+                                 float(np.finfo(np.float32).eps))
+    expect_graph(g, groups[0][1], "approx_rms_momentum")
+
+
+def test_adam_graph(env):
+    g, api, approx = env
+    x = g.variable(np.zeros(1, np.float32), [], "x")
+    loss = api.add(api.sub(api.square(x), api.mul(2.0, x)), 1.0)
+    step = approx.adam(loss, [x], 0.01, 0.9, 0.999, 1e-8)[0][1]
+    # 1 - 0.999f is 0.000999987 in float: the label the reference expects
+    assert "constant:0.000999987<FLOAT>" in g.to_string(step)
+    expect_graph(g, step, "approx_adam")
+
+
+def test_default_epsilon_follows_the_dtype(env):
+    g, api, approx = env
+    x = g.variable(np.ones(4, np.float64), [4], "x")
+    step = approx.adagrad(api.square(x), [x], 0.5)[0][1]
+    assert "constant:2.22045e-16<DOUBLE>" in g.to_string(step)
