@@ -469,6 +469,21 @@ class Api:
         not_targ = self.sub(1.0, target)
         return self.neg(self.add(self.mul(target, self.log(inp)), self.mul(not_targ, self.log(not_in))))
 
+    def reduce_mean(self, x):
+        """core.yml:1096: the sum over every dim divided by the element count."""
+        return self.div(self.reduce_sum(x), float(capi.n_elems(x.shape)))
+
+    def rnn(self, x, init_state, cell, activation, seq_dim=1):
+        """layer.yml:694-715.  cell = callable(concat(x_t, state)) (a dense layer
+        over both); init_state has the shape of one slice with the hidden size
+        in dim 0 (layer.yml:291-292 extends a {hidden} variable like a slice)."""
+        state, states = init_state, []
+        for i in range(x.shape[seq_dim]):
+            inslice = self.slice(x, i, 1, seq_dim)
+            state = activation(cell(self.concat([inslice, state], 0)))
+            states.append(state)
+        return self.identity(self.concat(states, seq_dim))
+
     def lstm(self, x, init_state, init_hidden, gates, seq_dim=1):
         """layer.yml:716-768.  gates = dict name -> callable(xc) for the g, i, f
         and o gate layers (each a dense layer over concat(x_t, hidden))."""

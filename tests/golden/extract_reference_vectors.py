@@ -23,6 +23,9 @@ VEC_RE = re.compile(
     r"std::vector<\s*(double|float|int32_t)\s*>\s*(\w+)\s*(?:=\s*)?\{(.*?)\}\s*;", re.S)
 DIMS_RE = re.compile(r"teq::DimsT\s+(\w+)\s*=\s*\{(.*?)\}\s*;", re.S)
 SHAPE_RE = re.compile(r"teq::Shape\s+(\w+)\s*\(\s*\{(.*?)\}\s*\)\s*;", re.S)
+NESTED_RE = re.compile(
+    r"std::vector<\s*std::vector<\s*double\s*>\s*>\s*(\w+)\s*(?:=\s*)?\{((?:\s*\{[^{}]*\}\s*,?)*)\s*\}\s*;", re.S)
+DIM_RE = re.compile(r"teq::(?:DimT|RankT)\s+(\w+)\s*=\s*(\d+)\s*;")
 SCALAR_RE = re.compile(r"\b(?:double|float)\s+(\w+)\s*=\s*([0-9eE+\-.]+)f?\s*;")
 LITERAL_LINE_RE = re.compile(r'^\s*"((?:[^"\\]|\\.)*)"[^"]*$')
 
@@ -68,10 +71,16 @@ def read_block(relpath, first, last):
         else:
             vals = [float(v) for v in vals]
         out[name] = vals
-    for name, body in DIMS_RE.findall(text):
-        out[name] = [int(v) for v in _numbers(body)]
-    for name, body in SHAPE_RE.findall(text):
-        out[name] = [int(v) for v in _numbers(body)]
+    for name, body in NESTED_RE.findall(text):
+        out[name] = [[float(v) for v in _numbers(inner)] for inner in re.findall(r"\{([^{}]*)\}", body)]
+    for name, literal in DIM_RE.findall(text):
+        out[name] = int(literal)
+    for regex in (DIMS_RE, SHAPE_RE):
+        for name, body in regex.findall(text):
+            try:
+                out[name] = [int(v) for v in _numbers(body)]
+            except ValueError:
+                pass  # spelled with named dims: the test restates it from those
     for name, literal in SCALAR_RE.findall(text):
         out[name] = float(literal)
     return out
@@ -111,6 +120,32 @@ BLOCKS = {
 }
 
 
+LAYER_BLOCKS = {
+    # recurrent layers built through the layer API: gradients, and three groups
+    # of assignments of a hand-written rms-momentum training step
+    "equation_tanh_rnn_layer": ("tenncor/test/test_equation.cpp", 842, 969),
+    "equation_tanh_rnn_layer_connect": ("tenncor/test/test_equation.cpp", 972, 1101),
+    "connect_tanh_rnn": ("tenncor/test/test_layer.cpp", 264, 387),
+    "connect_dense_tanh_rnn": ("tenncor/test/test_layer.cpp", 390, 571),
+    "connect_tanh_rnn_full": ("tenncor/test/test_layer.cpp", 574, 813),
+    "connect_tanh_rnn_cross_entropy": ("tenncor/test/test_layer.cpp", 816, 1058),
+    "connect_tanh_rnn_training": ("tenncor/test/test_layer.cpp", 1061, 1593),
+    "bind_softmax": ("tenncor/test/test_layer.cpp", 199, 261),
+}
+
+
+def write_layer_fixtures():
+    fixtures = {}
+    for key, (path, first, last) in LAYER_BLOCKS.items():
+        fixtures[key] = read_block(path, first, last)
+        if key == "bind_softmax":
+            fixtures[key]["expected_graphs"] = read_expected_graphs(path, first, last)
+        names = [k for k in fixtures[key] if not k.startswith("_")]
+        print("%-32s %s" % (key, ", ".join(names)))
+    with open(os.path.join(HERE, "layer_goldens.json"), "w") as f:
+        json.dump(fixtures, f, indent=0, separators=(",", ":"))
+
+
 GRAPH_BLOCKS = {
     # optimiser update rules: the graph each builds and the values one step leaves
     "approx_sgd": ("tenncor/test/test_approx.cpp", 21, 45),
@@ -137,11 +172,12 @@ def write_graph_fixtures():
 
 def main():
     write_graph_fixtures()
+    write_layer_fixtures()
     fixtures = {}
     for key, (path, first, last) in BLOCKS.items():
         fixtures[key] = read_block(path, first, last)
         names = [k for k in fixtures[key] if not k.startswith("_")]
-        print("%-22s %s" % (key, ", ".join("%s[%d]" % (n, len(fixtures[key][n])) for n in names)))
+        print("%-22s %s" % (key, ", ".join(names)))
     with open(os.path.join(HERE, "equation_vectors.json"), "w") as f:
         json.dump(fixtures, f, indent=0, separators=(",", ":"))
     return 0

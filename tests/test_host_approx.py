@@ -90,3 +90,18 @@ def test_default_epsilon_follows_the_dtype(env):
     x = g.variable(np.ones(4, np.float64), [4], "x")
     step = approx.adagrad(api.square(x), [x], 0.5)[0][1]
     assert "constant:2.22045e-16<DOUBLE>" in g.to_string(step)
+
+
+def test_softmax_graphs():
+    # BIND.Softmax (tenncor/test/test_layer.cpp:199-261): softmax over dim 0 and
+    # over dim 1 behind the IDENTITY a bound layer ends in
+    from tenncor_amd import graph
+    with open(os.path.join(HERE, "golden", "layer_goldens.json")) as f:
+        expected = json.load(f)["bind_softmax"]["expected_graphs"]
+    g = graph.Graph()
+    api = graph.Api(g)
+    x = g.variable(np.zeros(12, np.float32), [6, 2], "x")
+    for dim, text in zip((0, 1), expected):
+        root = api.identity(api.softmax(x, dim, 1))
+        assert lines_of(g.to_string(root)) == lines_of(text % EPS32)
+    g.close()
