@@ -49,6 +49,11 @@ int tcr_functor (tcr_graph* g, int opcode, int nargs, const int* args, int nattr
 /* tcr::derive(root, targets) -- tenncor/src/eteq.cpp:40-76 */
 int tcr_derive (tcr_graph* g, int root, int ntargets, const int* targets, int* grads);
 
+/* eteq::DerivativeFuncs::lderive(op, supgrad, arg_idx) --
+ * tenncor/eteq/backprop.hpp:58-560: the gradient that functor `op` passes to its
+ * argument arg_idx when `supgrad` arrives at it. */
+int tcr_local_derivative (tcr_graph* g, int op, int supgrad, int arg_idx, int* grad);
+
 /* teq::get_eval().evaluate(eigen::Device, targets) --
  * tenncor/eteq/src/etens.cpp:46-62 */
 int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets);

@@ -25,7 +25,7 @@ DIM_MAX = 65535  # std::numeric_limits<teq::DimT>::max()
 
 EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
-    "tcr_functor", "tcr_derive", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
+    "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
     "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan", "tcr_optimize",
     "tcr_set_random", "tcr_seed",
@@ -63,6 +63,7 @@ def load():
         "tcr_functor": [vp, i32, i32, i32p, i32, ctypes.POINTER(ctypes.c_char_p),
                         ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)), i32p, i32p],
         "tcr_derive": [vp, i32, i32, i32p, i32p],
+        "tcr_local_derivative": [vp, i32, i32, i32, i32p],
         "tcr_evaluate": [vp, i32, i32p],
         "tcr_sync": [vp],
         "tcr_shape": [vp, i32, u64p],
@@ -223,6 +224,13 @@ class Graph:
         out = (ctypes.c_int * len(targets))()
         self._check(self.lib.tcr_derive(self.h, root.id, len(targets), _ints([t.id for t in targets]), out))
         return [Node(self, out[i]) for i in range(len(targets))]
+
+    def local_derivative(self, op, supgrad, arg_idx):
+        """eteq::DerivativeFuncs::lderive: what functor `op` passes to its
+        argument arg_idx when the gradient `supgrad` arrives at it."""
+        out = ctypes.c_int()
+        self._check(self.lib.tcr_local_derivative(self.h, op.id, supgrad.id, int(arg_idx), ctypes.byref(out)))
+        return Node(self, out.value)
 
     def evaluate(self, targets):
         self._check(self.lib.tcr_evaluate(self.h, len(targets), _ints([t.id for t in targets])))

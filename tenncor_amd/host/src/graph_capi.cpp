@@ -188,6 +188,18 @@ int tcr_derive (tcr_graph* g, int root, int ntargets, const int* targets, int* g
 	});
 }
 
+int tcr_local_derivative (tcr_graph* g, int op, int supgrad, int arg_idx, int* grad)
+{
+	return guarded([&]
+	{
+		auto func = std::dynamic_pointer_cast<teq::iFunctor>(g->at(op));
+		if (nullptr == func) { global::fatal("local derivative of a leaf"); }
+		if (arg_idx < 0 || (size_t) arg_idx >= func->get_args().size()) { global::fatalf("no argument %d", arg_idx); }
+		eteq::DerivativeFuncs funcs;
+		*grad = g->add(funcs.lderive(func, g->at(supgrad), (size_t) arg_idx));
+	});
+}
+
 int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets)
 {
 	return guarded([&]

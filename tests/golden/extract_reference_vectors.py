@@ -146,6 +146,28 @@ def write_layer_fixtures():
         json.dump(fixtures, f, indent=0, separators=(",", ":"))
 
 
+def write_backprop_fixtures():
+    """tenncor/eteq/test/test_backprop.cpp: per TEST, the opcodes handed to the
+    unary/binary helpers (if any) and the printed gradient graphs it expects."""
+    path = "tenncor/eteq/test/test_backprop.cpp"
+    with open(os.path.join(REF, path)) as f:
+        lines = f.readlines()
+    starts = [(i + 1, re.match(r"TEST\(BACKPROP,\s*(\w+)\)", line).group(1))
+              for i, line in enumerate(lines) if line.startswith("TEST(BACKPROP")]
+    fixtures = {"_source": path}
+    for idx, (first, name) in enumerate(starts):
+        last = starts[idx + 1][0] - 1 if idx + 1 < len(starts) else len(lines)
+        text = "".join(lines[first - 1:last])
+        fixtures[name] = {
+            "lines": "%d-%d" % (first, last),
+            "helper_opcodes": re.findall(r"(unary|binary)_derivative\(egen::(\w+)", text),
+            "expected_graphs": read_expected_graphs(path, first, last),
+        }
+        print("%-14s %s %d graph(s)" % (name, fixtures[name]["helper_opcodes"], len(fixtures[name]["expected_graphs"])))
+    with open(os.path.join(HERE, "backprop_goldens.json"), "w") as f:
+        json.dump(fixtures, f, indent=0, separators=(",", ":"))
+
+
 GRAPH_BLOCKS = {
     # optimiser update rules: the graph each builds and the values one step leaves
     "approx_sgd": ("tenncor/test/test_approx.cpp", 21, 45),
@@ -173,6 +195,7 @@ def write_graph_fixtures():
 def main():
     write_graph_fixtures()
     write_layer_fixtures()
+    write_backprop_fixtures()
     fixtures = {}
     for key, (path, first, last) in BLOCKS.items():
         fixtures[key] = read_block(path, first, last)
