@@ -57,6 +57,11 @@ int tcr_local_derivative (tcr_graph* g, int op, int supgrad, int arg_idx, int* g
 /* teq::get_eval().evaluate(eigen::Device, targets) --
  * tenncor/eteq/src/etens.cpp:46-62 */
 int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets);
+/* The same with the third argument of iEvaluator::evaluate
+ * (internal/teq/ievaluator.hpp:17-25): the walk does not enter the `ignored`
+ * nodes, whose readers use the value they already hold
+ * (internal/teq/evaluator.hpp:20-24; internal/teq/test/test_evaluator.cpp:75-207) */
+int tcr_evaluate_ignoring (tcr_graph* g, int ntargets, const int* targets, int nignored, const int* ignored);
 /* Block until the device has finished everything enqueued */
 int tcr_sync (tcr_graph* g);
 

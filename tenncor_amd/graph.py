@@ -25,7 +25,7 @@ DIM_MAX = 65535  # std::numeric_limits<teq::DimT>::max()
 
 EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
-    "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
+    "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_evaluate_ignoring", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
     "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan", "tcr_optimize",
     "tcr_set_random", "tcr_seed",
@@ -64,6 +64,7 @@ def load():
                         ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)), i32p, i32p],
         "tcr_derive": [vp, i32, i32, i32p, i32p],
         "tcr_local_derivative": [vp, i32, i32, i32, i32p],
+        "tcr_evaluate_ignoring": [vp, i32, i32p, i32, i32p],
         "tcr_evaluate": [vp, i32, i32p],
         "tcr_sync": [vp],
         "tcr_shape": [vp, i32, u64p],
@@ -234,6 +235,12 @@ class Graph:
 
     def evaluate(self, targets):
         self._check(self.lib.tcr_evaluate(self.h, len(targets), _ints([t.id for t in targets])))
+
+    def evaluate_ignoring(self, targets, ignored):
+        """iEvaluator::evaluate(device, targets, ignored): the walk stops at the
+        ignored nodes, whose readers use the values they already hold."""
+        self._check(self.lib.tcr_evaluate_ignoring(self.h, len(targets), _ints([t.id for t in targets]),
+                                                   len(ignored), _ints([t.id for t in ignored])))
 
     def sync(self):
         self._check(self.lib.tcr_sync(self.h))

@@ -399,7 +399,7 @@ struct DerivativeFuncs final : public teq::iDerivativeFuncs
 };
 
 /// Evaluate `targets` with the registered evaluator on a GPU device
-void run (const teq::TensptrsT& targets);
+void run (const teq::TensptrsT& targets, const teq::TensptrsT& ignored = {});
 
 }
 

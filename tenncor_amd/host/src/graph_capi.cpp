@@ -210,6 +210,17 @@ int tcr_evaluate (tcr_graph* g, int ntargets, const int* targets)
 	});
 }
 
+int tcr_evaluate_ignoring (tcr_graph* g, int ntargets, const int* targets, int nignored, const int* ignored)
+{
+	return guarded([&]
+	{
+		teq::TensptrsT roots, skip;
+		for (int i = 0; i < ntargets; ++i) { roots.push_back(g->at(targets[i])); }
+		for (int i = 0; i < nignored; ++i) { skip.push_back(g->at(ignored[i])); }
+		eteq::run(roots, skip);
+	});
+}
+
 int tcr_sync (tcr_graph*)
 {
 	return guarded([&] { eigen::hip_check(tcg_sync(eigen::hip_context())); });

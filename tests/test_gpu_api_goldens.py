@@ -125,3 +125,43 @@ def test_identity_runs_its_dependencies(env):
         np.testing.assert_array_equal(target.get(), np.array(DATA2, np.float64))
         np.testing.assert_array_equal(ass.get(), np.array(DATA2, np.float64))
         np.testing.assert_array_equal(c.get(), np.array(DATA, np.float64) + np.array(DATA2, np.float64))
+
+
+def test_ignored_nodes_keep_their_values(env):
+    # EVALUATOR.UpdateIgnore (internal/teq/test/test_evaluator.cpp:75-144): the
+    # walk does not enter an ignored node; its reader takes the value it holds
+    g, api, graph = env
+    one = np.ones(6)
+    a, b, c, d = (g.variable(one * k, [3, 2], n) for k, n in ((1, "a"), (2, "b"), (3, "c"), (4, "d")))
+    x = api.add(a, b)
+    y = api.add(x, c)
+    target = api.add(y, d)
+    g.evaluate([target, y, x])
+    np.testing.assert_array_equal(target.get(), one * 10)
+    g.assign(a, one * 101)
+    g.assign(c, one * 1003)
+    y_version = g.version(y)
+    g.evaluate_ignoring([target], [y])
+    assert g.version(y) == y_version
+    np.testing.assert_array_equal(target.get(), one * 10)   # stale y (6) + d
+    g.assign(d, one * 10004)
+    g.evaluate_ignoring([target], [x])
+    np.testing.assert_array_equal(target.get(), one * (3 + 1003 + 10004))  # stale x (3)
+
+
+def test_ignored_node_with_a_shared_operand(env):
+    # EVALUATOR.UpdateIgnoreCommonDesc (test_evaluator.cpp:147-207): u is read by
+    # the ignored y and by x; u and x are computed, y is not
+    g, api, graph = env
+    one = np.ones(6)
+    a, b, c = (g.variable(one * k, [3, 2], n) for k, n in ((1, "a"), (20, "b"), (300, "c")))
+    u = api.neg(a)
+    x = api.add(u, b)
+    y = api.add(c, u)
+    target = api.add(y, x)
+    g.evaluate([target, y, x, u])
+    np.testing.assert_array_equal(target.get(), one * (299 + 19))
+    g.assign(a, one * 5)
+    g.evaluate_ignoring([target], [y])
+    np.testing.assert_array_equal(target.get(), one * (299 + 15))
+    np.testing.assert_array_equal(u.get(), one * -5)
