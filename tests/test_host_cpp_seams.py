@@ -1,0 +1,31 @@
+"""Compiles tests/cpp/functor_seams.cpp against the host layer's C++ headers
+and runs it: the node API (Functor::get / update_child / prop_version /
+cache_init, teq::set_eval) used from C++ exactly as a tenncor checkout would,
+with the expectations of the reference's own unit tests
+(tenncor/eteq/test/test_functor.cpp:22-302,
+internal/teq/test/test_evaluator.cpp:20-30).  Builds graphs only: no GPU.
+"""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "tenncor_amd")
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="no host C++ compiler")
+def test_node_api_from_cpp(tmp_path):
+    if not os.path.exists(os.path.join(PKG, "libtenncor_host.so")):
+        from tenncor_amd import build
+        build.build_all()
+    exe = str(tmp_path / "functor_seams")
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(PKG, "host"), "-I" + os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cpp", "functor_seams.cpp"), "-o", exe,
+           "-L" + PKG, "-ltenncor_host", "-ltcg", "-Wl,-rpath," + PKG]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr[-4000:]
+    ran = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert ran.returncode == 0, ran.stdout[-4000:] + ran.stderr[-2000:]
+    assert "0 failure(s)" in ran.stdout
