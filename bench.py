@@ -395,7 +395,26 @@ def run_cpu_baseline():
             list(pool.map(lambda k: one_pass(bounds[k], bounds[k + 1]), range(cores)))
             mpasses += 1
     mdt = time.perf_counter() - t1
+    # the product part of the metric: the port's triple loop on one core, and the
+    # host's BLAS (numpy) on the same operands as the figure an optimised CPU
+    # library reaches (the reference multiplies through Eigen's blocked kernel)
+    m = 1024
+    a = (rng.standard_normal(m * m) / 32).astype(np.float32)
+    b = (rng.standard_normal(m * m) / 32).astype(np.float32)
+    t2 = time.perf_counter()
+    orc.matmul(a, [m, m], b, [m, m])
+    port_dt = time.perf_counter() - t2
+    a2, b2 = a.reshape(m, m), b.reshape(m, m)
+    a2 @ b2
+    t3 = time.perf_counter()
+    for _ in range(10):
+        a2 @ b2
+    blas_dt = (time.perf_counter() - t3) / 10
+    matmul = {"port_GFLOPs": round(2.0 * m ** 3 / port_dt / 1e9, 2), "cores": 1,
+              "host_blas_GFLOPs": round(2.0 * m ** 3 / blas_dt / 1e9, 1), "host_blas_cores": cores,
+              "sample": "fp32 %d^3 (the metric's product is 4096^3)" % m}
     return {
+        "matmul": matmul,
         "value": round(passes * nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": "the same graph on np[%d,%d] (the whole workload), %d passes, %.1f s single-thread"
                   % (rows, COLS, passes, dt),
