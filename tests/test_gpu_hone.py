@@ -3,8 +3,11 @@ expected graphs for hone::optimize (tenncor/hone/test/test_cstrules.cpp:20-147,
 tenncor/test/test_opt.cpp:25-112) -- their inputs and the printed graphs they
 expect are restated below -- and value equality of the benchmark graphs before
 and after the clean-up.  The reference's tests read cfg/optimizations.json,
-which is a git-lfs pointer without content; none of the expected graphs
+which is a git-lfs pointer without content; none of those expected graphs
 contains a pattern a conversion could match, so they pin merging and folding.
+The two layer cases at the end of this file (test_opt.cpp:115-408) do contain
+such patterns: their expected graphs, real files of 684, 633, 311, 71 and 1273
+lines, pin the conversions shipped here as well.
 
 Tolerance: the folded constants are integers computed in double (exact); the
 cleaned-up configuration graphs are compared at 1e-5 relative to max |ref|
@@ -148,3 +151,85 @@ def test_configuration_graphs_keep_their_values(config, evaluator):
             assert np.abs(raw - cleaned).max() <= 1e-5 * scale
     finally:
         graph.set_evaluator("plain")
+
+
+# ---- the reference's expected optimised graphs --------------------------------
+# OPTIMIZE.RNNLayer and OPTIMIZE.CNNLayer (tenncor/test/test_opt.cpp:115-258,
+# :261-408) optimise a recurrent layer's gradients and a convolution layer's
+# training step with cfg/optimizations.json and compare the printed results with
+# models/test/opt0..3.txt and models/test/cnn_opt.txt.  The rule file is a
+# git-lfs pointer without content; the expected graphs are real files and are
+# kept under tests/golden/optimized/.  The conversions shipped here
+# (host/cfg/optimizations.json) must turn the same inputs into the same graphs,
+# line for line.
+
+def _lines(text):
+    out = [line.strip("_ \t") for line in text.split("\n")]
+    return [line for line in out if line]
+
+
+def _expected(name):
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "optimized", name)) as f:
+        return _lines(f.read())
+
+
+def test_optimised_rnn_layer_equals_the_reference_graphs(g):
+    import json
+    import os
+    from tenncor_amd import graph
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "layer_goldens.json")) as f:
+        gold = json.load(f)["equation_tanh_rnn_layer"]
+    api = graph.Api(g)
+    x = g.variable(np.array(gold["in_data"]), [5, 3], "in")
+    weight = g.variable(np.array(gold["weight_data"]), [5, 10], "weight")
+    bias = g.variable(np.array(gold["bias_data"]), [5], "bias")
+    istate = g.variable(np.array(gold["state_data"]), [5], "state")
+    out = g.variable(np.array(gold["out_data"]), [5, 3], "out")
+    state = api.extend_like(istate, api.slice(x, 0, 1, 1))
+    output = api.rnn(x, state, lambda xc: api.dense(xc, weight, bias), api.tanh, 1)
+    err = api.pow(api.sub(out, output), 2.0)
+    roots = g.derive(err, [weight, bias, istate]) + [err]
+    roots, stats = g.optimize(roots)
+    assert stats["converted"] >= 1 and stats["folded"] >= 1
+    for i, root in enumerate(roots):
+        assert _lines(g.to_string(root)) == _expected("rnn_layer_root%d.txt" % i), "root %d" % i
+    # and the optimised gradients still carry the reference's values
+    g.evaluate(roots[:3])
+    for root, name in zip(roots, ("expect_gw", "expect_gb", "expect_gstate")):
+        np.testing.assert_allclose(root.get(), gold[name], rtol=1e-9, atol=1e-11 * np.abs(gold[name]).max())
+
+
+def test_optimised_cnn_training_step_equals_the_reference_graph(g):
+    import json
+    import os
+    from tenncor_amd import graph
+    here = os.path.dirname(os.path.abspath(__file__))
+    with open(os.path.join(here, "golden", "approx_goldens.json")) as f:
+        gold = json.load(f)["opt_cnn_layer"]
+    api = graph.Api(g)
+    approx = graph.Approx(api)
+    invar = g.variable(np.array(gold["in_data"]), gold["in_shape"], "invar")
+    outvar = g.variable(np.array(gold["out_data"]), gold["out_shape"], "outvar")
+    weight = g.variable(np.array(gold["cweight_data"][:36]), [2, 2, 3, 3], "weight")
+    bias = g.variable(np.array(gold["cbias_data"]), [2], "bias")
+    eps = float(np.finfo(np.float64).eps)
+    normalized = api.sub(api.div(invar, 255.0), 0.5)
+
+    def error_of(w, b):
+        # link(IDENTITY) of bind(IDENTITY of relu) of the conv2d layer (IDENTITY):
+        # cfg/tenncor/layer.yml:17-27,64-65,230-251
+        conv = api.identity(api.conv2d(normalized, w, b, zero_padding=((1, 1), (1, 1))))
+        out = api.identity(api.identity(api.relu(conv)))
+        return api.neg(api.reduce_sum(api.mul(outvar, api.log(api.add(out, eps)))))
+
+    error = error_of(weight, bias)
+    updates = approx.adadelta(error, [weight, bias], gold["learning_rate"], gold["l2_decay"])
+    trailed = error_of(updates[0][1], updates[1][1])
+    err = api.identity(trailed, [assign for _, assign in updates])
+    (root,), _ = g.optimize([err])
+    assert _lines(g.to_string(root)) == _expected("cnn_layer.txt")
+    g.evaluate([root])
+    assert abs(root.get()[0] - gold["evdata"]) <= 1e-9 * gold["evdata"]
