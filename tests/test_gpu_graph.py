@@ -51,7 +51,8 @@ def npv(flat, shape):
     return np.asarray(flat).reshape([d for d in reversed(shape)])
 
 
-def test_matmul_chain_golden(g, api):
+@pytest.mark.parametrize("optimized", [False, True], ids=["as_built", "optimized"])
+def test_matmul_chain_golden(g, api, optimized):
     """tenncor/test/test_equation.cpp:26-136, forward and three gradients."""
     for key, mm in (("matmul_complex", api.matmul), ("contract_equivalent", api.contract)):
         fx = EQV[key]
@@ -63,6 +64,8 @@ def test_matmul_chain_golden(g, api):
         f = mm(api.transpose(d), api.transpose(c))
         dest = mm(e, f)
         da, db, dc = g.derive(dest, [a, b, c])
+        if optimized:  # EQUATION.OptimizedMatmulComplex, test_equation.cpp:1146-1154
+            (dest, da, db, dc), _ = g.optimize([dest, da, db, dc])
         g.evaluate([dest, da, db, dc])
         np.testing.assert_allclose(dest.get(), fx["expect_dest"], rtol=1e-13)
         np.testing.assert_allclose(da.get(), fx["expect_ga"], rtol=1e-13)
@@ -88,13 +91,16 @@ def mlp_graph(g, api, fx, np_dtype, slow):
     return err, [w0, b0, w1, b1], x
 
 
+@pytest.mark.parametrize("optimized", [False, True], ids=["as_built", "optimized"])
 @pytest.mark.parametrize("slow", [False, True], ids=["sigmoid_op", "spelled_out"])
-def test_config1_mlp_gradients_golden(g, api, slow):
+def test_config1_mlp_gradients_golden(g, api, slow, optimized):
     """tenncor/test/test_equation.cpp:252-706: exactly the config-1 shapes
     (x{10,3}, W0{9,10}, b0{9}, W1{5,9}, b1{5}) with 17-digit goldens."""
     fx = EQV["sigmoid_mlp_slow" if slow else "sigmoid_mlp_fast"]
     err, params, _ = mlp_graph(g, api, fx, np.float64, slow)
     grads = g.derive(err, params)
+    if optimized:  # EQUATION.OptimizedSlow/FastSigmoidMLP, test_equation.cpp:1157-1176
+        grads, _ = g.optimize(grads)
     g.evaluate(grads)
     for grad, key, shp in zip(grads, ("expect_gw0", "expect_gb0", "expect_gw1", "expect_gb1"),
                               ("weight0_shape", "bias0_shape", "weight1_shape", "bias1_shape")):
@@ -123,7 +129,8 @@ def test_config1_mlp_fp32_and_reassignment(g, api):
         np.testing.assert_array_equal(got, want)
 
 
-def test_tanh_rnn_golden(g, api):
+@pytest.mark.parametrize("optimized", [False, True], ids=["as_built", "optimized"])
+def test_tanh_rnn_golden(g, api, optimized):
     """tenncor/test/test_equation.cpp:709-839: unrolled tanh RNN (SLICE, CONCAT,
     CONTRACT, n-ary CONCAT and their gradients) with golden gradients."""
     fx = EQV["tanh_rnn"]
@@ -139,6 +146,8 @@ def test_tanh_rnn_golden(g, api):
     output = api.concat(states, 1)
     err = api.pow(api.sub(out, output), 2.0)
     dw, db, dstate = g.derive(err, [weight, bias, istate])
+    if optimized:  # EQUATION.OptimizedTanhRNN, test_equation.cpp:1179-1187
+        (dw, db, dstate), _ = g.optimize([dw, db, dstate])
     g.evaluate([dw, db, dstate])
     np.testing.assert_allclose(dw.get(), fx["expect_gw"], rtol=1e-12)
     np.testing.assert_allclose(db.get(), fx["expect_gb"], rtol=1e-12)
