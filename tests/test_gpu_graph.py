@@ -208,21 +208,25 @@ def torch_or_skip():
     return torch
 
 
-@pytest.mark.parametrize("seq,batch,nin,hid", [(6, 5, 7, 8), (64, 256, 256, 512)], ids=["reduced", "full_size"])
-def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid):
+@pytest.mark.parametrize("seq,batch,nin,hid,np_dtype,rtol", [
+    (6, 5, 7, 8, np.float32, 1e-4), (64, 256, 256, 512, np.float32, 1e-4), (8, 256, 256, 512, np.float64, 1e-10)],
+    ids=["reduced", "full_size", "double_on_matrix_cores"])
+def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid, np_dtype, rtol):
     """config 4 at reduced size (seq 6, batch 5, in 7, hidden 8) and at its
     full size: the layer.yml lstm recipe with one fused gate weight {4h, in+h}
     cut by SLICEs, loss = sum(h^2) over the concatenated hidden outputs,
-    against torch autograd in fp64."""
+    against torch autograd in fp64.  The third case is the graph in double at
+    the full widths (its 256x768x2048 products run on the fp64 matrix cores),
+    eight steps long, at 1e-10."""
     torch = torch_or_skip()
     if batch > 16:
         torch.set_num_threads(16)
     rng = np.random.default_rng(4)
-    w_np = rng.normal(0, 0.05, (nin + hid, 4 * hid)).astype(np.float32)   # np[768,2048] in the config
-    x_np = rng.uniform(-1, 1, (batch, seq, nin)).astype(np.float32)       # np[batch,seq,in]
+    w_np = rng.normal(0, 0.05, (nin + hid, 4 * hid)).astype(np_dtype)   # np[768,2048] in the config
+    x_np = rng.uniform(-1, 1, (batch, seq, nin)).astype(np_dtype)       # np[batch,seq,in]
     x = g.variable(x_np, [nin, seq, batch], "x")
     w = g.variable(w_np, [4 * hid, nin + hid], "w")
-    zeros = np.zeros(hid * batch, np.float32)
+    zeros = np.zeros(hid * batch, np_dtype)
     state0 = g.constant(zeros, [hid, 1, batch])
     hidden0 = g.constant(zeros, [hid, 1, batch])
 
@@ -253,9 +257,9 @@ def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid):
     loss_t = (h_all ** 2).sum()
     loss_t.backward()
     assert out.shape[:3] == [hid, seq, batch]
-    close(out.get(), h_all.detach().numpy().reshape(-1), 1e-4)
-    close(loss.get(), [loss_t.item()], 1e-4)
-    close(dw.get(), wt.grad.numpy().reshape(-1), 1e-4)
+    close(out.get(), h_all.detach().numpy().reshape(-1), rtol)
+    close(loss.get(), [loss_t.item()], rtol)
+    close(dw.get(), wt.grad.numpy().reshape(-1), rtol)
 
 
 @pytest.mark.parametrize("batch,hw,c1,c2,ncls", [(3, 12, 4, 6, 5), (16, 20, 8, 32, 10), (128, 28, 32, 64, 10)],
