@@ -262,9 +262,11 @@ def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid, np_dtyp
     close(dw.get(), wt.grad.numpy().reshape(-1), rtol)
 
 
-@pytest.mark.parametrize("batch,hw,c1,c2,ncls", [(3, 12, 4, 6, 5), (16, 20, 8, 32, 10), (128, 28, 32, 64, 10)],
-                         ids=["direct_kernels", "matrix_products", "full_size"])
-def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls):
+@pytest.mark.parametrize("batch,hw,c1,c2,ncls,np_dtype,rtol", [
+    (3, 12, 4, 6, 5, np.float32, 1e-4), (16, 20, 8, 32, 10, np.float32, 1e-4), (128, 28, 32, 64, 10, np.float32, 1e-4),
+    (16, 20, 8, 32, 10, np.float64, 1e-10)],
+    ids=["direct_kernels", "matrix_products", "full_size", "double"])
+def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls, np_dtype, rtol):
     """config 5 at reduced size (5x5 kernels 1->c1->c2, dense c2->ncls): the
     nn.yml conv2d idiom and its gradient idioms (PAD / REVERSE / CONV / PERMUTE
     / SLICE), softmax cross-entropy, against torch.  The first size stays on
@@ -275,14 +277,14 @@ def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls):
         torch.set_num_threads(16)
     F = torch.nn.functional
     rng = np.random.default_rng(5)
-    x_np = rng.uniform(0, 1, (batch, hw, hw, 1)).astype(np.float32)
-    k1_np = rng.normal(0, 0.2, (5, 5, 1, c1)).astype(np.float32)          # np[kh,kw,in,out]
-    k2_np = rng.normal(0, 0.4 / np.sqrt(c1), (5, 5, c1, c2)).astype(np.float32)
+    x_np = rng.uniform(0, 1, (batch, hw, hw, 1)).astype(np_dtype)
+    k1_np = rng.normal(0, 0.2, (5, 5, 1, c1)).astype(np_dtype)          # np[kh,kw,in,out]
+    k2_np = rng.normal(0, 0.4 / np.sqrt(c1), (5, 5, c1, c2)).astype(np_dtype)
     # logits of order one: a saturated softmax makes the comparison with fp64 meaningless
     wd_std = 0.3 if hw <= 12 else 2.0 / ((hw - 8) ** 2 * np.sqrt(c2))
-    wd_np = rng.normal(0, wd_std, (c2, ncls)).astype(np.float32)
+    wd_np = rng.normal(0, wd_std, (c2, ncls)).astype(np_dtype)
     labels = rng.integers(0, ncls, batch)
-    y_np = np.eye(ncls, dtype=np.float32)[labels]
+    y_np = np.eye(ncls, dtype=np_dtype)[labels]
     x = g.variable(x_np, [1, hw, hw, batch], "x")
     k1 = g.variable(k1_np, [c1, 1, 5, 5], "k1")
     k2 = g.variable(k2_np, [c2, c1, 5, 5], "k2")
@@ -307,15 +309,19 @@ def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls):
     a2 = F.relu(F.conv2d(a1, k2t.permute(3, 2, 0, 1)))
     pooled_t = a2.sum(dim=(2, 3))
     logits_t = pooled_t @ wdt
-    ex = torch.exp(logits_t - logits_t.max(dim=1, keepdim=True).values)
+    # the reference's gradient of REDUCE_MAX is EQ(extend(max), arg * extend(gradient))
+    # (tenncor/eteq/backprop.hpp:208-217), which is zero wherever arg * gradient differs
+    # from the maximum, i.e. nothing flows back through the shift of the softmax: detached here.
+    # (With the epsilon in the denominator that path would carry about 1e-8 of the gradient.)
+    ex = torch.exp(logits_t - logits_t.max(dim=1, keepdim=True).values.detach())
     probs_t = ex / (ex.sum(dim=1, keepdim=True) + eps)
     inp = probs_t + eps
     loss_t = -(yt * torch.log(inp) + (1 - yt) * torch.log(1 - inp)).sum()
     loss_t.backward()
-    close(loss.get(), [loss_t.item()], 1e-4)
-    close(grads[2].get(), wdt.grad.numpy().reshape(-1), 1e-4)
-    close(grads[1].get(), k2t.grad.numpy().reshape(-1), 1e-4)
-    close(grads[0].get(), k1t.grad.numpy().reshape(-1), 1e-4)
+    close(loss.get(), [loss_t.item()], rtol)
+    close(grads[2].get(), wdt.grad.numpy().reshape(-1), rtol)
+    close(grads[1].get(), k2t.grad.numpy().reshape(-1), rtol)
+    close(grads[0].get(), k1t.grad.numpy().reshape(-1), rtol)
 
 
 def test_assign_sub_updates_the_leaf_in_place(g, api):
