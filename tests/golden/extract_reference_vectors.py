@@ -7,7 +7,9 @@ It only reads the test sources as text: every ``std::vector<T> name = {...};``
 (or ``name{...}``) inside a given line range becomes ``name -> list``, every
 ``double name = literal;`` becomes ``name -> number``, every printed graph a
 test expects (the adjacent string literals of an ``EXPECT_GRAPHEQ``) becomes
-one string, and the result is committed as data.  Nothing of the reference is executed and no
+one string, and the result is committed as data.  The printed graphs that the
+reference keeps as files of their own (models/test/opt*.txt, cnn_opt.txt:
+expected outputs of its optimisation tests) are copied to optimized/.  Nothing of the reference is executed and no
 source text is kept.
 """
 import ast
@@ -168,6 +170,28 @@ def write_backprop_fixtures():
         json.dump(fixtures, f, indent=0, separators=(",", ":"))
 
 
+# printed graphs the reference's optimisation tests compare against
+# (tenncor/test/test_opt.cpp:211-255,381-386): data files of its test folder
+EXPECTED_GRAPH_FILES = {
+    "models/test/opt0.txt": "rnn_layer_root0.txt",
+    "models/test/opt1.txt": "rnn_layer_root1.txt",
+    "models/test/opt2.txt": "rnn_layer_root2.txt",
+    "models/test/opt3.txt": "rnn_layer_root3.txt",
+    "models/test/cnn_opt.txt": "cnn_layer.txt",
+}
+
+
+def copy_expected_graph_files():
+    outdir = os.path.join(HERE, "optimized")
+    os.makedirs(outdir, exist_ok=True)
+    for src, dst in EXPECTED_GRAPH_FILES.items():
+        with open(os.path.join(REF, src)) as f:
+            text = f.read()
+        with open(os.path.join(outdir, dst), "w") as f:
+            f.write(text)
+        print("%-26s %d lines" % (dst, text.count("\n")))
+
+
 GRAPH_BLOCKS = {
     # optimiser update rules: the graph each builds and the values one step leaves
     "approx_sgd": ("tenncor/test/test_approx.cpp", 21, 45),
@@ -196,6 +220,7 @@ def main():
     write_graph_fixtures()
     write_layer_fixtures()
     write_backprop_fixtures()
+    copy_expected_graph_files()
     fixtures = {}
     for key, (path, first, last) in BLOCKS.items():
         fixtures[key] = read_block(path, first, last)
