@@ -117,6 +117,7 @@ BLOCKS = {
     "tanh_rnn": ("tenncor/test/test_equation.cpp", 709, 839),
     # operator-with-gradient goldens
     "api_matmul": ("tenncor/test/test_api.cpp", 1986, 2085),
+    "api_contract": ("tenncor/test/test_api.cpp", 2089, 2190),
     "api_convolution": ("tenncor/test/test_api.cpp", 2265, 2373),
     "api_group_sum": ("tenncor/test/test_api.cpp", 2376, 2414),
 }

@@ -182,6 +182,28 @@ def test_api_matmul_int32_gradients_golden(g, api):
     np.testing.assert_array_equal(gr.get(), fx["expect_gb"])
 
 
+def test_api_contract_int32_gradients_golden(g, api):
+    """tenncor/test/test_api.cpp:2089-2190: a{3,1,2} and b{4,1,3} contracted
+    over a's dim 0 and b's dim 2 in int32; forward against numpy, both
+    gradients exact, and the gradient of contracting a tensor with itself."""
+    fx = EQV["api_contract"]
+    a = g.constant(np.array(fx["data"], np.int32), fx["alist"])
+    b = g.constant(np.array(fx["data2"], np.int32), fx["blist"])
+    dest = api.contract(a, b, [(0, 2)])
+    assert dest.shape[:4] == [4, 1, 1, 2]
+    (gl,), (gr,) = g.derive(dest, [a]), g.derive(dest, [b])
+    g.evaluate([dest, gl, gr])
+    g.evaluate([dest, gl, gr])  # idempotency check, as the reference does
+    av, bv = npv(fx["data"], fx["alist"]), npv(fx["data2"], fx["blist"])  # np[2,1,3], np[3,1,4]
+    np.testing.assert_array_equal(npv(dest.get(), [4, 1, 1, 2]).reshape(2, 4), av.reshape(2, 3) @ bv.reshape(3, 4))
+    np.testing.assert_array_equal(gl.get(), fx["expect_ga"])
+    np.testing.assert_array_equal(gr.get(), fx["expect_gb"])
+    c = g.constant(np.array(fx["data3"], np.int32), fx["sqrlist"])
+    (gs,) = g.derive(api.contract(c, c, [(0, 0)]), [c])
+    g.evaluate([gs])
+    assert gs.shape[:2] == fx["sqrlist"]
+
+
 def test_group_sum_and_buffers_return_to_the_pool(g, api):
     """tenncor/test/test_api.cpp:2376-2414 (4-argument ADD) and the TTL
     protocol: after an evaluation only leaves and targets hold device memory."""
