@@ -170,3 +170,62 @@ def test_comparisons_in_int32_have_zero_gradients(env, op, shape):
         grad = g.functor("CAST", [g.derive(root, [wrt])[0]], dtype=capi.INT32)
         g.evaluate([grad])
         np.testing.assert_array_equal(grad.get(), np.zeros(n, np.int32))
+
+
+# ---- reductions (test_api.cpp:1540-1873) --------------------------------------
+
+RDATA = np.array([22, 15, 74, 38, 61, 95, 62, 81, 99, 76, 7, 22, 56, 50, 19, 13, 12, 10, 31, 40, 60, 54, 6, 83], np.float64)
+RSHAPE = [2, 3, 4]
+
+
+def np_view(flat, shape):
+    return np.asarray(flat).reshape(shape[::-1])
+
+
+@pytest.mark.parametrize("op,npf", [("REDUCE_SUM", np.sum), ("REDUCE_MIN", np.min), ("REDUCE_MAX", np.max)])
+def test_reductions_and_their_gradients(env, op, npf):
+    from tenncor_amd import capi
+    g, api = env
+    src = g.constant(RDATA, RSHAPE)
+    full = api.reduce(op, src)              # over every dim
+    along = api.reduce(op, src, 1, 1)       # over dim 1
+    g.evaluate([full, along])
+    g.evaluate([full, along])
+    view = np_view(RDATA, RSHAPE)           # np[4,3,2]
+    np.testing.assert_array_equal(full.get(), [npf(RDATA)])
+    assert along.shape[:3] == [2, 1, 4]
+    np.testing.assert_array_equal(np_view(along.get(), [2, 1, 4]), npf(view, axis=1, keepdims=True))
+    gfull = g.functor("CAST", [g.derive(full, [src])[0]], dtype=capi.DOUBLE)
+    galong = g.functor("CAST", [g.derive(along, [src])[0]], dtype=capi.DOUBLE)
+    g.evaluate([gfull, galong])
+    g.evaluate([gfull, galong])
+    if op == "REDUCE_SUM":
+        np.testing.assert_array_equal(gfull.get(), np.ones(24))
+        np.testing.assert_array_equal(galong.get(), np.ones(24))
+    else:
+        # one at the extreme of each reduced group, zero elsewhere
+        np.testing.assert_array_equal(gfull.get(), (RDATA == npf(RDATA)).astype(np.float64))
+        want = (view == npf(view, axis=1, keepdims=True)).astype(np.float64)
+        np.testing.assert_array_equal(np_view(galong.get(), RSHAPE), want)
+
+
+def test_reduce_prod_in_int32_and_its_gradient(env):
+    from tenncor_amd import capi
+    g, api = env
+    data = np.array([2, 1, 7, 3, 6, 9, 6, 8, 9, 7, 7, 2], np.int32)
+    shape = [2, 2, 3]
+    src = g.constant(data, shape)
+    full = api.reduce("REDUCE_PROD", src)
+    along = api.reduce("REDUCE_PROD", src, 1, 1)
+    g.evaluate([full, along])
+    g.evaluate([full, along])
+    assert full.get()[0] == np.prod(data.astype(np.int64))
+    view = np_view(data, shape)
+    np.testing.assert_array_equal(np_view(along.get(), [2, 1, 3]), np.prod(view, axis=1, keepdims=True))
+    gfull = g.functor("CAST", [g.derive(full, [src])[0]], dtype=capi.INT32)
+    galong = g.functor("CAST", [g.derive(along, [src])[0]], dtype=capi.INT32)
+    g.evaluate([gfull, galong])
+    g.evaluate([gfull, galong])
+    np.testing.assert_array_equal(gfull.get(), np.prod(data.astype(np.int64)) // data)
+    # the reference's expected values, test_api.cpp:1693-1700
+    np.testing.assert_array_equal(galong.get(), [7, 3, 2, 1, 6, 8, 6, 9, 7, 2, 9, 7])
