@@ -395,6 +395,12 @@ class Api:
     def assign_sub(self, target, source):
         return self.g.functor("ASSIGN_SUB", [target, source])
 
+    def if_then_else(self, condition, then, otherwise):
+        """core.yml:634-651: choosing between a tensor and itself is that tensor."""
+        if then.id == otherwise.id:
+            return then
+        return self.g.functor("SELECT", [condition, then, otherwise])
+
     def relu(self, x):
         """core.yml:1261-1267: max(arg, 0)."""
         return self.binary("MAX", x, 0.0)

@@ -229,3 +229,96 @@ def test_reduce_prod_in_int32_and_its_gradient(env):
     np.testing.assert_array_equal(gfull.get(), np.prod(data.astype(np.int64)) // data)
     # the reference's expected values, test_api.cpp:1693-1700
     np.testing.assert_array_equal(galong.get(), [7, 3, 2, 1, 6, 8, 6, 9, 7, 2, 9, 7])
+
+
+# ---- data movement and selection (test_api.cpp:1189-1364, 1506-1537, 1876-1983)
+
+def test_slice_and_its_gradient(env):
+    from tenncor_amd import capi
+    g, api = env
+    shape = [3, 2, 4]
+    src = g.constant(BDATA, shape)
+    dest = g.functor("SLICE", [src], dimension_pairs=[0, 3, 1, 1])   # slice(src, {{0,3},{1,1}})
+    g.evaluate([dest])
+    g.evaluate([dest])
+    assert dest.shape[:3] == [3, 1, 4]
+    np.testing.assert_array_equal(dest.get(), np_view(BDATA, shape)[:, 1:2, :].reshape(-1))
+    grad = g.functor("CAST", [g.derive(dest, [src])[0]], dtype=capi.DOUBLE)
+    g.evaluate([grad])
+    g.evaluate([grad])
+    assert grad.shape[:3] == shape
+    np.testing.assert_array_equal(grad.get(), [0, 0, 0, 1, 1, 1] * 4)  # test_api.cpp:1343-1348
+
+
+def test_permute_and_its_gradient(env):
+    from tenncor_amd import capi
+    g, api = env
+    shape, order = [4, 3, 2], [2, 0, 1]
+    data = np.array([70, 36, 93, 50, 59, 98, 39, 5, 54, 84, 100, 94, 75, 64, 30, 17, 90, 79, 21, 54, 6, 7, 69, 53], np.float64)
+    src = g.constant(data, shape)
+    dest = api.permute(src, order)
+    g.evaluate([dest])
+    g.evaluate([dest])
+    oshape = dest.shape[:3]
+    assert oshape == [shape[o] for o in order]
+    got = dest.get()
+    # out coordinate j is in coordinate order[j] (test_api.cpp:1901-1909)
+    for i in range(24):
+        c = [i % 4, (i // 4) % 3, i // 12]
+        oc = [c[order[j]] for j in range(3)]
+        assert got[oc[0] + oshape[0] * (oc[1] + oshape[1] * oc[2])] == data[i]
+    grad = g.functor("CAST", [g.derive(dest, [src])[0]], dtype=capi.DOUBLE)
+    g.evaluate([grad])
+    assert grad.shape[:3] == shape
+    np.testing.assert_array_equal(grad.get(), np.ones(24))
+
+
+def test_extend_and_its_gradient(env):
+    from tenncor_amd import capi
+    g, api = env
+    data = np.array([51, 42, 9, 43, 37, 36, 65, 95, 10, 33], np.float64)
+    src = g.constant(data, [2, 5])
+    dest = api.extend(src, 2, [1, 3])
+    g.evaluate([dest])
+    g.evaluate([dest])
+    assert dest.shape[:4] == [2, 5, 1, 3]
+    np.testing.assert_array_equal(dest.get(), np.tile(data, 3))
+    grad = g.functor("CAST", [g.derive(dest, [src])[0]], dtype=capi.DOUBLE)
+    g.evaluate([grad])
+    assert grad.shape[:2] == [2, 5]
+    np.testing.assert_array_equal(grad.get(), np.full(10, 3.0))
+
+
+@pytest.mark.parametrize("shape", [[3, 2, 4], [3, 2]], ids=["tensor", "matrix"])
+def test_select_and_its_gradients(env, shape):
+    from tenncor_amd import capi
+    g, api = env
+    n = int(np.prod(shape))
+    cond = (np.arange(n) % 3 != 1).astype(np.float64)
+    data, data2 = BDATA[:n], BDATA2[:n]
+    csrc, src, src2 = g.constant(cond, shape), g.constant(data, shape), g.constant(data2, shape)
+    dest = api.if_then_else(csrc, src, src2)
+    g.evaluate([dest])
+    g.evaluate([dest])
+    np.testing.assert_array_equal(dest.get(), np.where(cond != 0, data, data2))
+    # choosing between a tensor and itself is that tensor (test_api.cpp:1253-1254)
+    assert api.if_then_else(csrc, src, src).id == src.id
+    gl = g.functor("CAST", [g.derive(dest, [src])[0]], dtype=capi.DOUBLE)
+    gr = g.functor("CAST", [g.derive(dest, [src2])[0]], dtype=capi.DOUBLE)
+    g.evaluate([gl, gr])
+    g.evaluate([gl, gr])
+    np.testing.assert_array_equal(gl.get(), cond)
+    np.testing.assert_array_equal(gr.get(), (cond == 0).astype(np.float64))
+
+
+def test_argmax_over_everything_and_no_gradient(env):
+    from tenncor_amd import graph
+    g, api = env
+    src = g.constant(RDATA, RSHAPE)
+    dest = g.functor("ARGMAX", [src], rank=8)
+    g.evaluate([dest])
+    g.evaluate([dest])
+    assert dest.shape == [1] * 8
+    assert dest.get()[0] == 8          # the flat index of 99
+    with pytest.raises(graph.GraphError, match="cannot derive ARGMAX"):
+        g.derive(dest, [src])
