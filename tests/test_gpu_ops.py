@@ -236,6 +236,21 @@ def test_select_cast_assign(ctx, ops, oracle):
         np.testing.assert_array_equal(t.get(), ref)
 
 
+def test_assign_and_cast_goldens(ctx, ops):
+    """internal/eigen/test/test_operator.cpp:2647-2879: the reference's vectors
+    for ASSIGN .. ASSIGN_DIV (in place on the target) and CAST."""
+    from tenncor_amd import capi
+    goldens = {"ASSIGN": [1, 0, 3, 9, 10, 11], "ASSIGN_ADD": [3, 8, 7, 14, 16, 18], "ASSIGN_SUB": [1, 8, 1, -4, -4, -4],
+               "ASSIGN_MUL": [2, 0, 12, 45, 60, 77], "ASSIGN_DIV": [2, 4, 4. / 3, 5. / 9, 0.6, 7. / 11]}
+    for op, want in goldens.items():
+        target = ops.from_host(ctx, np.array([2, 8, 4, 5, 6, 7], np.float64), [2, 3])
+        source = ops.from_host(ctx, np.array([1, 2 if op == "ASSIGN_DIV" else 0, 3, 9, 10, 11], np.float64), [2, 3])
+        ops.assign(op, target, source)
+        np.testing.assert_allclose(target.get(), want, rtol=4e-16, err_msg=op)
+    x = ops.from_host(ctx, np.array([2.1, 8.5, 4.3, 5.2, 6.1, 7.2], np.float64), [2, 3])
+    np.testing.assert_array_equal(ops.cast(x, capi.INT32).get(), np.array([2, 8, 4, 5, 6, 7], np.int32))
+
+
 def test_unaligned_operands_take_the_scalar_path(ctx, ops, oracle):
     """Aliased last-dim slices give pointers that are not 16-byte aligned
     (internal/eigen/operator.hpp:231-248)."""

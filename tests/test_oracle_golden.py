@@ -239,6 +239,36 @@ def test_cast_and_assign(oracle):
     np.testing.assert_array_equal(t, np.array([.5, 1.5, -1.], np.float32))
 
 
+# internal/eigen/test/test_operator.cpp:2647-2818 (Assign .. AssignDiv) and
+# :2821-2879 (Cast): the reference's own vectors
+ASSIGN_GOLDENS = {
+    "ASSIGN": [1, 0, 3, 9, 10, 11],
+    "ASSIGN_ADD": [3, 8, 7, 14, 16, 18],
+    "ASSIGN_SUB": [1, 8, 1, -4, -4, -4],
+    "ASSIGN_MUL": [2, 0, 12, 45, 60, 77],
+    "ASSIGN_DIV": [2, 4, 4. / 3, 5. / 9, 0.6, 7. / 11],
+}
+ASSIGN_TARGET = [2, 8, 4, 5, 6, 7]
+ASSIGN_SOURCE = [1, 0, 3, 9, 10, 11]
+ASSIGN_DIV_SOURCE = [1, 2, 3, 9, 10, 11]   # :2789 divides by {1, 2, 3, 9, 10, 11}
+CAST_SOURCE = [2.1, 8.5, 4.3, 5.2, 6.1, 7.2]
+CAST_INT32 = [2, 8, 4, 5, 6, 7]
+
+
+@pytest.mark.parametrize("op", sorted(ASSIGN_GOLDENS))
+def test_assign_goldens(oracle, op):
+    target = np.array(ASSIGN_TARGET, np.float64)
+    source = np.array(ASSIGN_DIV_SOURCE if op == "ASSIGN_DIV" else ASSIGN_SOURCE, np.float64)
+    oracle.assign(op, target, source)
+    np.testing.assert_allclose(target, ASSIGN_GOLDENS[op], rtol=4e-16)
+
+
+def test_cast_golden(oracle):
+    x = np.array(CAST_SOURCE, np.float64)
+    np.testing.assert_array_equal(oracle.cast(x, oracle.DOUBLE), x)
+    np.testing.assert_array_equal(oracle.cast(x, oracle.INT32), np.array(CAST_INT32, np.int32))
+
+
 # ---- the device RAND_UNIF stream -------------------------------------------
 
 # Known-answer vectors of the Random123 distribution (kat_vectors, philox4x32
