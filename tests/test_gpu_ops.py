@@ -825,7 +825,8 @@ def test_full_size_properties_config3(ctx, ops):
     checked without a CPU product: C r against A (B r) in fp64 for a random
     vector r (Freivalds), at the 1e-4 bar relative to the largest entry; the
     int32 product of the same shape exactly (mod 2^32); PERMUTE of the result
-    is an involution and moves rows to columns."""
+    is an involution and moves rows to columns; the 4096^3 product in double
+    by Freivalds at 1e-12."""
     rng = np.random.default_rng(3)
     n = 4096
     a = (rng.standard_normal(n * n) / 64).astype(np.float32)
@@ -849,6 +850,15 @@ def test_full_size_properties_config3(ctx, ops):
     ri = rng.integers(-3, 4, n).astype(np.int64)
     want = ai.reshape(n, n).astype(np.int64) @ (bi.reshape(n, n).astype(np.int64) @ ri)
     np.testing.assert_array_equal((ci.astype(np.int64) @ ri).astype(np.int32), want.astype(np.int32))
+    # the same product in double on the fp64 matrix cores: Freivalds in extended
+    # precision, at 1e-12 relative to the largest entry
+    ad, bd = a.astype(np.float64), b.astype(np.float64)
+    cd = ops.matmul(ops.from_host(ctx, ad, [n, n]), ops.from_host(ctx, bd, [n, n])).get().reshape(n, n)
+    rl = r.astype(np.longdouble)
+    want = ad.reshape(n, n).astype(np.longdouble) @ (bd.reshape(n, n).astype(np.longdouble) @ rl)
+    assert np.abs(cd.astype(np.longdouble) @ rl - want).max() <= 1e-12 * np.abs(want).max()
+    want = (rl @ ad.reshape(n, n).astype(np.longdouble)) @ bd.reshape(n, n).astype(np.longdouble)
+    assert np.abs(rl @ cd.astype(np.longdouble) - want).max() <= 1e-12 * np.abs(want).max()
     # batched: np[64,512,512] x np[64,512,512], every batch by Freivalds
     m, nb = 512, 64
     a3 = (rng.standard_normal(nb * m * m) / 22).astype(np.float32)
