@@ -344,7 +344,12 @@ int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 	const void* a, const void* b, void* out);
 /* Strided row-major GEMM the two above lower to:
  * C[b][m][n] = sum_k A[b][m][k] * B[b][k][n], element strides given;
- * trans_a: A element (m,k) at m*1 + k*lda instead of m*lda + k, same for B */
+ * trans_a: A element (m,k) at m*1 + k*lda instead of m*lda + k, same for B.
+ * float and double products whose operands are 16-byte aligned with even
+ * (double) or fourfold (float) extents along memory run on the matrix cores;
+ * int32, odd shapes and products too small to fill the chip run on a tiled
+ * kernel.  Every route sums k in a fixed order: results do not depend on
+ * scheduling. */
 int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	uint64_t batch, const void* A, uint64_t lda, uint64_t stride_a, int trans_a,
 	const void* B, uint64_t ldb, uint64_t stride_b, int trans_b,
