@@ -82,9 +82,33 @@ def build_libhost(jobs=8, verbose=False):
     return LIBHOST
 
 
+NATIVE_PROGRAMS = {
+    # program -> source (C++ users of the host layer, run by the tests)
+    "mlp_gradients": os.path.join(ROOT, "tests", "cpp", "mlp_gradients.cpp"),
+}
+
+
+def native_program(name):
+    return os.path.join(PKG, "build", name)
+
+
+def build_native_programs(verbose=False):
+    """C++ programs that use the host layer the way a tenncor checkout would."""
+    os.makedirs(os.path.join(PKG, "build"), exist_ok=True)
+    built = []
+    for name, source in NATIVE_PROGRAMS.items():
+        exe = native_program(name)
+        out = _run([CXX, "-std=c++17", "-O1", "-Wall", "-I" + HOST, "-I" + os.path.join(ROOT, "include"), source,
+                    "-o", exe, "-L" + PKG, "-ltenncor_host", "-ltcg", "-Wl,-rpath,$ORIGIN/.."])
+        if verbose and out.strip():
+            print(out)
+        built.append(exe)
+    return built
+
+
 def build_all(verbose=False):
     """Everything native in this package."""
-    return [build_libtcg(verbose=verbose), build_libhost(verbose=verbose)]
+    return [build_libtcg(verbose=verbose), build_libhost(verbose=verbose)] + build_native_programs(verbose=verbose)
 
 
 def main():
