@@ -12,9 +12,14 @@
 #include <vector>
 
 #include "eteq.hpp"
+#include "replay_eval.hpp"
 
-int main (void)
+// mlp_gradients [replay]: with "replay" the process-wide evaluator slot holds
+// the recording evaluator (teq::set_eval) and the targets are evaluated four
+// times with the input re-assigned in between: walk, record, replay, replay
+int main (int argc, char** argv)
 {
+	const bool replay = argc > 1 && std::string(argv[1]) == "replay";
 	std::map<std::string,std::vector<double>> in;
 	std::string name;
 	size_t n;
@@ -52,8 +57,23 @@ int main (void)
 		eigen::Device device;
 		teq::TensSetT targets;
 		for (auto& g : grads) { targets.emplace(g.get()); }
-		teq::Evaluator().evaluate(device, targets);
-		teq::Evaluator().evaluate(device, targets); // nothing to do the second time
+		if (replay)
+		{
+			teq::set_eval(new eigen::ReplayEvaluator());
+			auto input = std::static_pointer_cast<eteq::Variable<double>>(x);
+			for (int pass = 0; pass < 4; ++pass)
+			{
+				input->assign(in.at("in").data(), input->shape()); // a new version: everything recomputes
+				teq::get_eval().evaluate(device, targets, {});
+			}
+			auto stats = static_cast<eigen::ReplayEvaluator&>(teq::get_eval()).stats();
+			std::printf("replayed %zu\n", (size_t) stats.replayed);
+		}
+		else
+		{
+			teq::Evaluator().evaluate(device, targets);
+			teq::Evaluator().evaluate(device, targets); // nothing to do the second time
+		}
 
 		const char* names[] = {"gw0", "gb0", "gw1", "gb1"};
 		for (size_t i = 0; i < grads.size(); ++i)
