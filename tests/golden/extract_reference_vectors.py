@@ -134,6 +134,8 @@ LAYER_BLOCKS = {
     "connect_tanh_rnn_cross_entropy": ("tenncor/test/test_layer.cpp", 816, 1058),
     "connect_tanh_rnn_training": ("tenncor/test/test_layer.cpp", 1061, 1593),
     "bind_softmax": ("tenncor/test/test_layer.cpp", 199, 261),
+    "dense_connection": ("tenncor/test/test_layer.cpp", 36, 96),
+    "conv_connection": ("tenncor/test/test_layer.cpp", 99, 120),
 }
 
 
@@ -141,7 +143,7 @@ def write_layer_fixtures():
     fixtures = {}
     for key, (path, first, last) in LAYER_BLOCKS.items():
         fixtures[key] = read_block(path, first, last)
-        if key == "bind_softmax":
+        if key in ("bind_softmax", "dense_connection", "conv_connection"):
             fixtures[key]["expected_graphs"] = read_expected_graphs(path, first, last)
         names = [k for k in fixtures[key] if not k.startswith("_")]
         print("%-32s %s" % (key, ", ".join(names)))

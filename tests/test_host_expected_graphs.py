@@ -1,4 +1,6 @@
-"""The graphs the optimiser update rules build, line by line against the
+"""Graphs built by the optimiser update rules, by softmax and by the dense and
+convolution layers, line by line against the printed graphs the reference's own
+tests expect.  First the update rules: the graphs they build against the
 printed graphs the reference's own tests expect
 (tenncor/test/test_approx.cpp:21-45 sgd, :48-86 adagrad, :89-193 adadelta,
 :289-327 rms_momentum, :388-478 adam), held in tests/golden/approx_goldens.json.
@@ -104,4 +106,25 @@ def test_softmax_graphs():
     for dim, text in zip((0, 1), expected):
         root = api.identity(api.softmax(x, dim, 1))
         assert lines_of(g.to_string(root)) == lines_of(text % EPS32)
+    g.close()
+
+
+def test_dense_and_convolution_layers_connect_like_the_reference():
+    # DENSE.Connection and CONV.Connection (tenncor/test/test_layer.cpp:36-120):
+    # a dense layer with and without bias, a conv2d layer with a 6x5 kernel
+    from tenncor_amd import graph
+    with open(os.path.join(HERE, "golden", "layer_goldens.json")) as f:
+        gold = json.load(f)
+    g = graph.Graph()
+    api = graph.Api(g)
+    zeros = lambda shape, label: g.variable(np.zeros(int(np.prod(shape)), np.float32), shape, label)
+    biased, plain = gold["dense_connection"]["expected_graphs"]
+    y = api.dense(zeros([6, 2], "x"), zeros([5, 6], "weight"), zeros([5], "bias"))
+    assert lines_of(g.to_string(y)) == lines_of(biased)
+    y = api.dense(zeros([7, 2], "x2"), zeros([6, 7], "weight"))
+    assert lines_of(g.to_string(y)) == lines_of(plain)
+    (conv,) = gold["conv_connection"]["expected_graphs"]
+    # conv2d<float>({6, 5}, 4, 3): kernel {out 3, in 4, width 5, height 6}
+    y = api.identity(api.conv2d(zeros([4, 10, 9, 2], "x"), zeros([3, 4, 5, 6], "weight"), zeros([3], "bias")))
+    assert lines_of(g.to_string(y)) == lines_of(conv)
     g.close()
