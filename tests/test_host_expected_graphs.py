@@ -1,9 +1,8 @@
 """Graphs built by the optimiser update rules, by softmax and by the dense and
 convolution layers, line by line against the printed graphs the reference's own
-tests expect.  First the update rules: the graphs they build against the
-printed graphs the reference's own tests expect
-(tenncor/test/test_approx.cpp:21-45 sgd, :48-86 adagrad, :89-193 adadelta,
-:289-327 rms_momentum, :388-478 adam), held in tests/golden/approx_goldens.json.
+tests expect: tenncor/test/test_approx.cpp:21-45 sgd, :48-86 adagrad, :89-193
+adadelta, :289-327 rms_momentum, :388-478 adam (tests/golden/approx_goldens.json)
+and tenncor/test/test_layer.cpp:36-120, :199-261 (tests/golden/layer_goldens.json).
 The rules are those of cfg/tenncor/approx.yml; the derivative subgraphs inside
 them come from the gradient builder (tenncor/eteq/backprop.hpp).  Lines are
 compared as the reference compares them: leading and trailing '_' and blanks
