@@ -423,6 +423,27 @@ def run_cpu_baseline():
     }
 
 
+def run_matmul_ramp(blocks=12, per_block=10):
+    """4096^3 fp32 products back to back from a cold start, timed in blocks of
+    ten: how long the matrix clock takes to settle (the reason the product
+    metric above is taken after 40 untimed launches)."""
+    from tenncor_amd import capi
+    ctx = capi.Context(0)
+    n = 4096
+    rng = np.random.default_rng(3)
+    a = ctx.upload((rng.standard_normal(n * n) / 64).astype(np.float32))
+    b = ctx.upload((rng.standard_normal(n * n) / 64).astype(np.float32))
+    c = ctx.empty(n * n, np.float32)
+    out = []
+    for _ in range(blocks):
+        ctx.timer_begin()
+        for _ in range(per_block):
+            ctx.matmul(capi.FLOAT, [n, n], [n, n], a.ptr, b.ptr, c.ptr)
+        ms = ctx.timer_end() / per_block
+        out.append(round(2.0 * n ** 3 / (ms * 1e-3) / 1e12, 1))
+    return {"matmul_4096_fp32_TFLOPs_per_block_of_%d" % per_block: out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -436,11 +457,16 @@ def main():
     ap.add_argument("--reps", type=int, default=20, help="timed evaluations with --graph-config 4 or 5")
     ap.add_argument("--optimize", action="store_true",
                     help="with --graph-config: clean the graph up first (duplicates merged, constants folded, conversions)")
+    ap.add_argument("--matmul-ramp", action="store_true",
+                    help="print the 4096^3 product rate of successive blocks of ten launches from a cold start")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs on one GPU; --gpus %d is not supported "
                  "(no collectives or sharding are part of this build)" % args.gpus)
 
+    if args.matmul_ramp:
+        print(json.dumps(run_matmul_ramp()))
+        return
     if args.graph_config is not None:
         print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps, optimize=args.optimize)))
         return
