@@ -8,7 +8,8 @@
 // A[i][k] and B[k][i]; a lane holds C[4 r + lane / 16][lane % 16], r = 0..3).
 // A and B slabs of BK = 8 columns go global -> registers -> LDS (double
 // buffered, one barrier per slab), both kept [k][row] so that the sixteen lanes
-// of a k read sixteen consecutive doubles.  Sums run over k in ascending order.
+// of a k read sixteen consecutive doubles (an operand whose K runs along memory
+// is kept [row][k], see the kernel).  Sums run over k in ascending order.
 // MFMA-bound: 2*M*N*K flops against 78.6 TFLOP/s.
 #include "tcg_internal.hpp"
 
@@ -46,8 +47,14 @@ __global__ __launch_bounds__(256) void dgemm_mfma_k (DGemmArgs g)
 	constexpr int AP = BM + 16, BP = BN + 16;
 	constexpr int A_CHUNKS = BM * DBK / 2, B_CHUNKS = BN * DBK / 2; // double2 per slab
 	constexpr int A_VEC = (A_CHUNKS + 255) / 256, B_VEC = (B_CHUNKS + 255) / 256;
-	__shared__ __attribute__((aligned(16))) double As[2][DBK * AP];
-	__shared__ __attribute__((aligned(16))) double Bs[2][DBK * BP];
+	// an operand whose K runs along memory is kept [row][k] instead, pitch 10:
+	// written with the 128-bit values as they were loaded, and the sixteen rows
+	// times two k of a half-wave read fall on 32 distinct bank pairs
+	constexpr int KP = DBK + 2;
+	constexpr int A_SIZE = TA ? DBK * AP : BM * KP;
+	constexpr int B_SIZE = TB ? BN * KP : DBK * BP;
+	__shared__ __attribute__((aligned(16))) double As[2][A_SIZE];
+	__shared__ __attribute__((aligned(16))) double Bs[2][B_SIZE];
 
 	// workgroups resident on one XCD (ids congruent mod 8) take consecutive
 	// tiles, and consecutive tiles walk down groups of eight tile rows: what an
@@ -143,8 +150,7 @@ __global__ __launch_bounds__(256) void dgemm_mfma_k (DGemmArgs g)
 			if constexpr (!TA)
 			{
 				int mm = idx / (DBK / 2), kq = idx % (DBK / 2);
-				as[(kq * 2) * AP + mm] = ra[v][0];
-				as[(kq * 2 + 1) * AP + mm] = ra[v][1];
+				*reinterpret_cast<f64x2*>(as + mm * KP + kq * 2) = ra[v];
 			}
 			else
 			{
@@ -165,8 +171,7 @@ __global__ __launch_bounds__(256) void dgemm_mfma_k (DGemmArgs g)
 			else
 			{
 				int nn = idx / (DBK / 2), kq = idx % (DBK / 2);
-				bs[(kq * 2) * BP + nn] = rb[v][0];
-				bs[(kq * 2 + 1) * BP + nn] = rb[v][1];
+				*reinterpret_cast<f64x2*>(bs + nn * KP + kq * 2) = rb[v];
 			}
 		}
 	};
@@ -179,16 +184,16 @@ __global__ __launch_bounds__(256) void dgemm_mfma_k (DGemmArgs g)
 	{
 		const int buf = s & 1;
 		if (s + 1 < nslabs) { load_slab((s + 1) * DBK); }
-		const double* as = As[buf] + lk * AP + wm * WM + l16;
-		const double* bs = Bs[buf] + lk * BP + wn * WN + l16;
+		const double* as = TA ? As[buf] + lk * AP + wm * WM + l16 : As[buf] + (wm * WM + l16) * KP + lk;
+		const double* bs = TB ? Bs[buf] + (wn * WN + l16) * KP + lk : Bs[buf] + lk * BP + wn * WN + l16;
 #pragma unroll
 		for (int ks = 0; ks < DBK / 4; ++ks)
 		{
 			double a[TM], b[TN];
 #pragma unroll
-			for (int i = 0; i < TM; ++i) { a[i] = as[ks * 4 * AP + i * 16]; }
+			for (int i = 0; i < TM; ++i) { a[i] = TA ? as[ks * 4 * AP + i * 16] : as[i * 16 * KP + ks * 4]; }
 #pragma unroll
-			for (int j = 0; j < TN; ++j) { b[j] = bs[ks * 4 * BP + j * 16]; }
+			for (int j = 0; j < TN; ++j) { b[j] = TB ? bs[j * 16 * KP + ks * 4] : bs[ks * 4 * BP + j * 16]; }
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 			{
