@@ -113,6 +113,41 @@ __global__ __launch_bounds__(256) void gemm_generic_k (
 	}
 }
 
+// A few thousand results with a long K (a dense head on a batch, its weight
+// gradient): the tiled kernel would run a handful of workgroups through one
+// memory latency per 16 columns of K.  Here every lane owns one result and
+// walks K itself, sixteen pairs of loads in flight; the sum runs in the same order with
+// the same fused multiply-add, so the value equals the tiled kernel's bit for bit.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_small_k (
+	uint32_t M, uint32_t N, uint32_t K, uint32_t batch,
+	const T* __restrict__ A, int64_t sam, int64_t sak, int64_t batch_a,
+	const T* __restrict__ B, int64_t sbk, int64_t sbn, int64_t batch_b,
+	T* __restrict__ C, int64_t ldc, int64_t batch_c)
+{
+	const uint32_t idx = blockIdx.x * 256 + threadIdx.x;
+	if (idx >= M * N * batch) { return; }
+	const uint32_t n = idx % N, m = (idx / N) % M, bz = idx / (N * M);
+	const T* a = A + (int64_t) bz * batch_a + (int64_t) m * sam;
+	const T* b = B + (int64_t) bz * batch_b + (int64_t) n * sbn;
+	T acc = 0;
+	uint32_t k = 0;
+	for (; k + 16 <= K; k += 16)
+	{
+		T av[16], bv[16];
+#pragma unroll
+		for (int e = 0; e < 16; ++e)
+		{
+			av[e] = a[(int64_t) (k + e) * sak];
+			bv[e] = b[(int64_t) (k + e) * sbk];
+		}
+#pragma unroll
+		for (int e = 0; e < 16; ++e) { acc = fma_wrap(av[e], bv[e], acc); }
+	}
+	for (; k < K; ++k) { acc = fma_wrap(a[(int64_t) k * sak], b[(int64_t) k * sbk], acc); }
+	C[(int64_t) bz * batch_c + (int64_t) m * ldc + n] = acc;
+}
+
 template <typename T>
 int gemm_generic (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
 	const T* A, uint64_t lda, uint64_t stride_a, int trans_a,
@@ -126,6 +161,14 @@ int gemm_generic (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_t bat
 		(unsigned long long) M, (unsigned long long) N, (unsigned long long) K, (unsigned long long) batch);
 	int64_t sam = trans_a ? 1 : (int64_t) lda, sak = trans_a ? (int64_t) lda : 1;
 	int64_t sbk = trans_b ? 1 : (int64_t) ldb, sbn = trans_b ? (int64_t) ldb : 1;
+	if (K >= 32 && M * N * batch <= 16384)
+	{
+		const unsigned grid = (unsigned) ((M * N * batch + 255) / 256);
+		gemm_small_k<T><<<grid, 256, 0, ctx->stream>>>((uint32_t) M, (uint32_t) N, (uint32_t) K, (uint32_t) batch,
+			A, sam, sak, (int64_t) stride_a, B, sbk, sbn, (int64_t) stride_b, C, (int64_t) ldc, (int64_t) stride_c);
+		TCG_LAUNCH_CHECK(ctx, "gemm_small");
+		return TCG_OK;
+	}
 	gemm_generic_k<T><<<(unsigned) blocks, 256, 0, ctx->stream>>>((uint32_t) M, (uint32_t) N, (uint32_t) K,
 		A, sam, sak, (int64_t) stride_a, B, sbk, sbn, (int64_t) stride_b, C, (int64_t) ldc, (int64_t) stride_c,
 		(uint32_t) tiles_n, (uint32_t) tiles_m);

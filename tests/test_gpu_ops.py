@@ -493,6 +493,37 @@ def test_gemm_f64_transposed_operands_vs_oracle(ctx, oracle, M, N, K, batch, ta,
     assert_acc_close(dc.get(), ref, rtol=1e-12)
 
 
+SMALL_GEMM_CASES = [(128, 10, 64, 1, 0, 0), (64, 10, 128, 1, 1, 0), (20, 12, 300, 5, 1, 1), (7, 9, 33, 3, 0, 1),
+                    (1, 1, 4000, 1, 0, 0), (128, 128, 32, 1, 0, 0)]
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32])
+@pytest.mark.parametrize("M,N,K,batch,ta,tb", SMALL_GEMM_CASES, ids=[str(c) for c in SMALL_GEMM_CASES])
+def test_small_products_with_a_long_k(ctx, oracle, M, N, K, batch, ta, tb, np_dtype):
+    """Few results, K of 32 or more: every lane owns one result and walks K in
+    ascending order (int32 exact; fp32 against the oracle accumulating in
+    double at 1e-4 of the largest entry, fp64 at 1e-12)."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of(M, N, K, batch, ta, tb, str(np_dtype)))
+    if np_dtype == np.int32:
+        a = rng.integers(-2000, 2000, batch * M * K).astype(np.int32)
+        b = rng.integers(-2000, 2000, batch * K * N).astype(np.int32)
+    else:
+        a = rng.standard_normal(batch * M * K).astype(np_dtype)
+        b = (rng.standard_normal(batch * K * N) / np.sqrt(K)).astype(np_dtype)
+    a_can = a if not ta else oracle.permute(a, [M, K, batch], [1, 0, 2])[0]
+    b_can = b if not tb else oracle.permute(b, [K, N, batch], [1, 0, 2])[0]
+    ref, _ = oracle.matmul(a_can, [K, M, batch], b_can, [N, K, batch], wide_acc=(np_dtype == np.float32))
+    da, db = ctx.upload(a), ctx.upload(b)
+    dc = ctx.empty(batch * M * N, np_dtype)
+    ctx.gemm(capi.dtype_code(np.dtype(np_dtype)), M, N, K, batch, da.ptr, M if ta else K, M * K, ta,
+             db.ptr, K if tb else N, K * N, tb, dc.ptr, N, M * N)
+    if np_dtype == np.int32:
+        np.testing.assert_array_equal(dc.get(), ref)
+    else:
+        assert_acc_close(dc.get(), ref, rtol=ACC_RTOL if np_dtype == np.float32 else 1e-12)
+
+
 CONTRACT_CASES = [
     ([10, 3], [9, 10], [[0, 1]]),                      # dense layer (config 1)
     ([768, 1, 64], [512, 768], [[0, 1]]),              # LSTM gate product (config 4)
