@@ -348,7 +348,8 @@ int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
  * float and double products whose operands are 16-byte aligned with even
  * (double) or fourfold (float) extents along memory run on the matrix cores;
  * int32, odd shapes and products too small to fill the chip run on a tiled
- * kernel.  Every route sums k in a fixed order: results do not depend on
+ * kernel, or with one lane per result when there are few results and K is
+ * long.  Every route sums k in a fixed order: results do not depend on
  * scheduling. */
 int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	uint64_t batch, const void* A, uint64_t lda, uint64_t stride_a, int trans_a,
