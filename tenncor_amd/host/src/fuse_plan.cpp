@@ -70,6 +70,18 @@ bool is_binary (int op)
 	return op >= egen::POW && op <= egen::GT;
 }
 
+bool is_assign (int op)
+{
+	return op >= egen::ASSIGN && op <= egen::ASSIGN_DIV;
+}
+
+/// Nodes whose value is their first operand's buffer (TensRef / UnsafeTensRef):
+/// reading them reads whatever that buffer holds at the time of the read
+bool is_buffer_alias (int op)
+{
+	return op == egen::IDENTITY || op == egen::RESHAPE || op == egen::SLICE;
+}
+
 View dense_view (teq::iTensor* tens, const Shape8& shape)
 {
 	View v;
@@ -129,6 +141,7 @@ struct Planner final
 			}
 			n.kind = classify(n);
 		}
+		find_written();
 		// PERMUTE{1,0} of a matrix-valued CONTRACT nothing else reads: launch the
 		// swapped product instead; the CONTRACT node is looked through like a view
 		for (size_t i = 0; i < nodes_.size(); ++i)
@@ -161,6 +174,8 @@ struct Planner final
 				}
 			}
 			if (free_dims[0] != 1 || free_dims[1] != 1) { continue; }
+			// the product would read its operands where the PERMUTE stands
+			if (written_between(n.args[0], {0, 1}, n.args[0], (int) i)) { continue; }
 			n.kind = OTHER;
 			n.swapped_from = n.args[0];
 			c.kind = VIEW;
@@ -182,11 +197,13 @@ struct Planner final
 			nonzero_box(*n.arg_tens[0], lo, hi);
 			bool plain = hi == inner && std::all_of(lo.begin(), lo.end(), [](uint64_t v) { return v == 0; });
 			if (false == convolved || false == plain) { continue; }
+			if (written_between((int) i, {0}, (int) i, n.consumers.back() + 1)) { continue; }
 			n.absorbed = true;
 			n.through_conv = true;
 			for (int c : n.consumers) { nodes_[c].padded_from = (int) i; }
 		}
 		// a view is folded away when everything that reads it can read through it
+		std::vector<int> last_reader(nodes_.size(), 0); // position of the last launch reading through a folded view
 		for (size_t i = nodes_.size(); i-- > 0;)
 		{
 			Node& n = nodes_[i];
@@ -195,6 +212,19 @@ struct Planner final
 			{
 				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed && false == nodes_[c].through_conv);
 			});
+			if (false == n.absorbed) { continue; }
+			for (int c : n.consumers)
+			{
+				last_reader[i] = std::max(last_reader[i], nodes_[c].kind == EW ? c : last_reader[c]);
+			}
+			// a materialised view holds the operand's value from where it stands
+			// in the pass: it cannot be folded into a launch that runs after an
+			// assignment to that operand (IDENTITY holds nothing: it is the
+			// operand's buffer, whoever reads it)
+			if (n.op != egen::IDENTITY && written_between((int) i, {0}, (int) i, last_reader[i]))
+			{
+				n.absorbed = false;
+			}
 		}
 		for (Node& n : nodes_)
 		{
@@ -223,6 +253,98 @@ struct Planner final
 	{
 		const Node& n = nodes_[i];
 		return n.kind == VIEW && n.absorbed && n.op == egen::IDENTITY;
+	}
+
+	// ---- buffers that ASSIGN* nodes of the pass rewrite ----
+	//
+	// The walk runs node by node, so a node that reads a variable before an
+	// ASSIGN* to it in the walk's order sees the old value and one after it
+	// the new one (internal/eigen/device.hpp:508-544 updates the target's
+	// buffer in place).  Launches are reordered and merged here, so every read
+	// of such a buffer is pinned to its side of every write to it.
+
+	/// The tensor whose buffer an ASSIGN* node (or a chain of aliases) rewrites
+	teq::iTensor* written_base (int i) const
+	{
+		const Node& n = nodes_[i];
+		if (n.args[0] < 0) { return n.arg_tens[0].get(); }
+		const Node& a = nodes_[n.args[0]];
+		if (is_assign(a.op) || is_buffer_alias(a.op)) { return written_base(n.args[0]); }
+		return a.f;
+	}
+
+	void find_written (void)
+	{
+		writes_.assign(nodes_.size(), -1);
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			if (false == is_assign(nodes_[i].op) || nodes_[i].args.empty()) { continue; }
+			teq::iTensor* base = written_base((int) i);
+			auto it = resource_.emplace(base, (int) write_pos_.size()).first;
+			if (it->second == (int) write_pos_.size()) { write_pos_.emplace_back(); }
+			write_pos_[it->second].push_back((int) i);
+			writes_[i] = it->second;
+		}
+	}
+
+	/// Rewritten buffers that are read when operand k of node i is read.
+	/// `folded`: look through every node that can be folded into its reader
+	/// (while that is being decided) instead of those that have been.
+	void touched_by_arg (int i, size_t k, bool folded, std::set<int>& out) const
+	{
+		const Node& n = nodes_[i];
+		int a = n.args[k];
+		auto it = resource_.find(a < 0 ? n.arg_tens[k].get() : (teq::iTensor*) nodes_[a].f);
+		if (it != resource_.end()) { out.insert(it->second); }
+		if (a < 0) { return; }
+		const Node& arg = nodes_[a];
+		if (is_assign(arg.op)) { out.insert(writes_[a]); }
+		else if (is_buffer_alias(arg.op)) { touched_by_arg(a, 0, folded, out); }
+		else if (arg.kind == VIEW && (folded || arg.absorbed))
+		{
+			for (size_t j = 0; j < arg.args.size(); ++j) { touched_by_arg(a, j, folded, out); }
+		}
+	}
+
+	/// Is a buffer that operands `ks` of node i read rewritten after position
+	/// `from` and before position `to`?
+	bool written_between (int i, std::initializer_list<size_t> ks, int from, int to) const
+	{
+		if (resource_.empty()) { return false; }
+		std::set<int> touched;
+		for (size_t k : ks) { touched_by_arg(i, k, true, touched); }
+		for (int r : touched)
+		{
+			for (int w : write_pos_[r])
+			{
+				if (from < w && w < to) { return true; }
+			}
+		}
+		return false;
+	}
+
+	/// Dependence edges that keep launch i on its side of the writes: called
+	/// for every launch in the order of the pass
+	void order_around_writes (int i)
+	{
+		if (resource_.empty()) { return; }
+		const Node& n = nodes_[i];
+		std::set<int> touched;
+		for (size_t k = is_assign(n.op) ? 1 : 0; k < n.args.size(); ++k) { touched_by_arg(i, k, false, touched); }
+		for (int r : touched)
+		{
+			if (last_write_[r] >= 0) { deps_[i].insert(last_write_[r]); }
+			readers_[r].push_back(i);
+		}
+		int w = writes_[i];
+		if (w < 0) { return; }
+		for (int reader : readers_[w])
+		{
+			if (find(reader) != i) { deps_[i].insert(find(reader)); }
+		}
+		if (last_write_[w] >= 0) { deps_[i].insert(last_write_[w]); }
+		readers_[w].clear();
+		last_write_[w] = i;
 	}
 
 	/// Does anything other than the launch described by `inside` read node i?
@@ -425,6 +547,8 @@ struct Planner final
 
 	void group_all (void)
 	{
+		last_write_.assign(write_pos_.size(), -1);
+		readers_.assign(write_pos_.size(), {});
 		for (size_t i = 0; i < nodes_.size(); ++i)
 		{
 			Node& n = nodes_[i];
@@ -433,6 +557,7 @@ struct Planner final
 			std::vector<int> ins;
 			inputs_of((int) i, ins);
 			deps_[i].insert(ins.begin(), ins.end());
+			order_around_writes((int) i);
 			if (n.kind != EW) { continue; }
 			members_[i].push_back((int) i);
 			std::vector<int> cands;
@@ -841,6 +966,12 @@ struct Planner final
 	std::vector<std::set<int>> deps_;
 	std::vector<size_t> stamp_;
 	size_t clock_ = 0;
+	// buffers rewritten by ASSIGN* nodes of the pass
+	std::unordered_map<teq::iTensor*,int> resource_; // tensor owning the buffer -> id
+	std::vector<std::vector<int>> write_pos_;        // id -> positions of the ASSIGN* nodes, ascending
+	std::vector<int> writes_;                        // node -> id it rewrites, -1 for none
+	std::vector<int> last_write_;                    // while grouping: id -> latest ASSIGN* seen
+	std::vector<std::vector<int>> readers_;          // while grouping: id -> launches reading it since
 };
 
 }

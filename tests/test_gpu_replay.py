@@ -411,6 +411,46 @@ def test_fused_views_diamonds_and_wide_groups(np_dtype):
     assert stats["replay_launches"]["replayed"] == 3
 
 
+def test_reads_of_a_variable_stay_on_their_side_of_an_assignment():
+    """ASSIGN* rewrites its target in place: a node that reads the variable before
+    the assignment in the walk's order sees the old value, one after it the new
+    value (internal/eigen/device.hpp:508-544).  The shared launches must keep
+    that, whichever elementwise nodes they merge."""
+    rng = np.random.default_rng(seed=31)
+    feeds = [rng.uniform(-1, 1, 24).astype(np.float32) for _ in range(4)]
+    v0 = rng.uniform(-1, 1, 24).astype(np.float32)
+    w0 = rng.uniform(-1, 1, 6).astype(np.float32)
+
+    def build(g, api):
+        c = g.variable(feeds[0], [6, 4], "c")
+        v = g.variable(v0, [6, 4], "v")
+        w = g.variable(w0, [6], "w")
+        x = api.neg(v)                                      # old v
+        a = api.assign(v, c)
+        y = api.mul(x, v)                                   # new v
+        t = api.add(api.add(x, a), y)
+        wide = api.extend(w, 1, [4])                        # old w, laid out before the update
+        upd = api.assign_add(w, api.reduce_sum(api.mul(api.neg(wide), c), 1, 1))
+        late = api.add(api.extend(upd, 1, [4]), api.mul(wide, c))  # wide: read after the update too
+        mid = api.square(api.identity(a))
+        second = api.assign_sub(v, mid)
+        tail = api.add(api.neg(second), mid)
+        return [t, late, tail], c
+
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+    for kind in ("replay_launches", "replay"):
+        for row, ref in zip(results[kind], results["plain"]):
+            for a, b in zip(row, ref):
+                if kind == "replay":
+                    np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
+                else:
+                    np.testing.assert_array_equal(a, b)
+    # and the walk itself computes what the order of the nodes says
+    c0 = feeds[0].reshape(4, 6)
+    t_first = (-v0.reshape(4, 6)) + c0 + (-v0.reshape(4, 6)) * c0
+    np.testing.assert_allclose(results["plain"][0][0].reshape(4, 6), t_first, rtol=1e-6)
+
+
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
 def test_fused_concat_keeps_every_bit(np_dtype):
     """CONCAT inside a group is an OR of zero-bordered operands: signed zeros,

@@ -369,3 +369,55 @@ def test_launch_plan_reads_the_operand_of_a_pad_that_only_convolutions_read(g, a
     assert g.opcode(padded) == "PAD"
     lines = g.launch_plan([y, padded])
     assert "node PAD" in lines and "node CONV" in lines and not any(l.startswith("padded") for l in lines)
+
+
+def test_launch_plan_keeps_reads_of_a_variable_on_their_side_of_an_assignment(g, api):
+    """ASSIGN* rewrites its target's buffer in place (internal/eigen/device.hpp:508-544).
+    In the walk's children-first order NEG(v) runs before the ASSIGN and MUL(NEG, v)
+    after it, so the two cannot share a launch, although MUL reads NEG and both are
+    elementwise nodes of one shape."""
+    v = var(g, [6, 4], np.float32, "v")
+    c = var(g, [6, 4], np.float32, "c")
+    x = api.neg(v)
+    a = api.assign(v, c)
+    y = api.mul(x, v)
+    t = api.add(api.add(x, a), y)
+    lines = [l for l in g.launch_plan([t]) if not l.startswith("folded")]
+    steps = parse_plan(lines)
+    at = next(i for i, s in enumerate(steps) if s[1] == ["ASSIGN"])
+    before = [op for s in steps[:at] for op in s[1]]
+    after = [op for s in steps[at + 1:] for op in s[1]]
+    assert before == ["NEG"], lines
+    assert sorted(after) == ["ADD", "ADD", "MUL"], lines
+
+    # a view of the variable that is laid out before the assignment and read after it
+    # keeps the old value: it is not folded into the launch that reads it
+    w = var(g, [6], np.float32, "w")
+    d = var(g, [6], np.float32, "d")
+    wide = api.extend(w, 1, [4])
+    upd = api.assign_add(w, api.mul(api.reduce_sum(api.neg(wide), 1, 1), d))
+    late = api.add(api.extend(upd, 1, [4]), api.mul(wide, c))
+    lines = g.launch_plan([late])
+    assert "node EXTEND" in lines, lines
+    steps = parse_plan([l for l in lines if not l.startswith("folded")])
+    assert steps[0][1] == ["EXTEND"], lines
+    names = [s[1] for s in steps]
+    assert names.index(["ASSIGN_ADD"]) < next(i for i, n in enumerate(names) if "MUL" in n and "ADD" in n), lines
+    # when every reader of the view comes before the assignment, it is folded as usual
+    early = api.add(api.mul(api.extend(w, 1, [4]), c), api.extend(api.assign_add(w, d), 1, [4]))
+    lines = g.launch_plan([early])
+    assert "node EXTEND" not in lines and lines.index("node ASSIGN_ADD") == 1, lines
+    # ... and without an assignment in between the same view is folded
+    plain = api.add(api.mul(api.extend(w, 1, [4]), c), c)
+    assert "node EXTEND" not in g.launch_plan([plain])
+
+    # two assignments to one variable keep their order, readers in between stay in between
+    first = api.assign(v, c)
+    mid = api.square(api.identity(first))
+    second = api.assign_sub(v, mid)
+    tail = api.add(api.neg(second), mid)
+    steps = parse_plan([l for l in g.launch_plan([tail]) if not l.startswith("folded")])
+    names = [s[1] for s in steps]
+    i1, i2 = names.index(["ASSIGN"]), names.index(["ASSIGN_SUB"])
+    assert i1 < i2
+    assert any("SQUARE" in n for n in names[i1 + 1:i2]) and any("NEG" in n for n in names[i2 + 1:])
