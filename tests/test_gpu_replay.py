@@ -435,20 +435,25 @@ def test_reads_of_a_variable_stay_on_their_side_of_an_assignment():
         mid = api.square(api.identity(a))
         second = api.assign_sub(v, mid)
         tail = api.add(api.neg(second), mid)
-        return [t, late, tail], c
+        # one target, so that the order of the walk is the order written here
+        # (several targets are walked in the order of an unordered set)
+        return [g.functor("ADD", [t, late, tail])], c
 
     results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
     for kind in ("replay_launches", "replay"):
-        for row, ref in zip(results[kind], results["plain"]):
-            for a, b in zip(row, ref):
-                if kind == "replay":
-                    np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
-                else:
-                    np.testing.assert_array_equal(a, b)
+        for i, (row, ref) in enumerate(zip(results[kind], results["plain"])):
+            if kind == "replay":
+                np.testing.assert_allclose(row[0], ref[0], rtol=1e-5, atol=1e-6, err_msg="%s pass %d" % (kind, i))
+            else:
+                np.testing.assert_array_equal(row[0], ref[0], err_msg="%s pass %d" % (kind, i))
+    assert stats["replay_launches"]["replayed"] == 3
     # and the walk itself computes what the order of the nodes says
-    c0 = feeds[0].reshape(4, 6)
-    t_first = (-v0.reshape(4, 6)) + c0 + (-v0.reshape(4, 6)) * c0
-    np.testing.assert_allclose(results["plain"][0][0].reshape(4, 6), t_first, rtol=1e-6)
+    c0, vold, wold = feeds[0].reshape(4, 6).astype(np.float64), v0.reshape(4, 6).astype(np.float64), w0.astype(np.float64)
+    t = -vold + c0 + (-vold) * c0
+    wnew = wold + (-wold[None, :] * c0).sum(axis=0)
+    late = wnew[None, :] + wold[None, :] * c0
+    tail = -(c0 - c0 * c0) + c0 * c0
+    np.testing.assert_allclose(results["plain"][0][0].reshape(4, 6), t + late + tail, rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
