@@ -290,6 +290,26 @@ int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
 	unsigned rankmask, const void* in, void* out);
 
+/* The same reduction for callers that cannot allocate device memory (code
+ * under HIP graph capture of their own, serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  tcg_reduce takes its
+ * temporaries (partial results of a reduced dim that is split over
+ * workgroups, and what is left of the tensor between the steps of a reduction
+ * over separated dims) from the context's pool, which may call hipMalloc;
+ * this entry point keeps them in a fixed array of device memory that every
+ * GPU the library runs on holds from load to exit, and calls no allocating
+ * routine.  Same kernels, same launch shapes, same results bit for bit.
+ * Limits: the temporaries of one call must fit
+ * TCG_REDUCE_NOALLOC_SCRATCH_BYTES (each piece rounded up to 256 bytes),
+ * otherwise the call fails with TCG_ERR_ARG and nothing is launched for the
+ * step that did not fit; every call on a GPU uses that GPU's one array, so
+ * calls that overlap on one GPU (two contexts, two streams) race -- calls on
+ * one context are ordered on its stream and do not.  Not available inside
+ * tcg_capture_begin_small. */
+#define TCG_REDUCE_NOALLOC_SCRATCH_BYTES ((size_t) 8 << 20)
+int tcg_reduce_noalloc (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
+	unsigned rankmask, const void* in, void* out);
+
 /* ARGMAX (cfg/ops.yml:152-186; internal/eigen/operator.hpp:134-155);
  * return_dim >= 8 gives the flat index of the maximum */
 int tcg_argmax (tcg_ctx* ctx, int dtype, const uint64_t shape[8], int return_dim,

@@ -16,6 +16,8 @@ LIB_PATH = os.path.join(_PKG, "libtcg.so")
 RANK_CAP = 8
 DOUBLE, FLOAT, INT32 = 1, 2, 3
 NP_OF = {DOUBLE: np.float64, FLOAT: np.float32, INT32: np.int32}
+# include/tcg.h: the fixed device memory tcg_reduce_noalloc keeps its temporaries in
+REDUCE_NOALLOC_SCRATCH_BYTES = 8 << 20
 
 OPCODES = [
     "BAD_OP", "IDENTITY", "ABS", "NEG", "SIN", "COS", "TAN", "EXP", "LOG", "SQRT", "ROUND",
@@ -35,7 +37,7 @@ EXPORTS = [
     "tcg_mem_stats", "tcg_h2d", "tcg_d2h", "tcg_d2d", "tcg_fill_zero", "tcg_sync", "tcg_timer_begin",
     "tcg_timer_end", "tcg_event_create", "tcg_event_destroy", "tcg_event_record", "tcg_event_elapsed",
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
-    "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
+    "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
     "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
@@ -109,6 +111,7 @@ def load():
         "tcg_ew_fused": [vp, i32, u64, i32, vpp, i32, ctypes.POINTER(EwInstr), vp],
         "tcg_ew_fusedx": [vp, i32, u64p, i32, ctypes.POINTER(FxLeaf), i32, ctypes.POINTER(FxInstr), i32, vpp],
         "tcg_reduce": [vp, i32, i32, u64p, ctypes.c_uint, vp, vp],
+        "tcg_reduce_noalloc": [vp, i32, i32, u64p, ctypes.c_uint, vp, vp],
         "tcg_argmax": [vp, i32, u64p, i32, vp, vp],
         "tcg_extend": [vp, i32, u64p, u64p, vp, vp],
         "tcg_permute": [vp, i32, u64p, u64p, vp, vp],
@@ -349,6 +352,11 @@ class Context:
     # ---- reductions ----
     def reduce(self, op, dtype, shape, rank_set, src, dst):
         self._check(self.lib.tcg_reduce(self.handle, _opcode(op), dtype, _u64(shape8(shape)), _mask(rank_set), src, dst))
+
+    def reduce_noalloc(self, op, dtype, shape, rank_set, src, dst):
+        """tcg_reduce with its temporaries in the library's fixed device array."""
+        self._check(self.lib.tcg_reduce_noalloc(self.handle, _opcode(op), dtype, _u64(shape8(shape)), _mask(rank_set),
+                                                src, dst))
 
     def argmax(self, dtype, shape, return_dim, src, dst):
         self._check(self.lib.tcg_argmax(self.handle, dtype, _u64(shape8(shape)), int(return_dim), src, dst))

@@ -15,6 +15,16 @@
 
 #include <limits>
 
+// Device memory that exists for as long as the library is loaded, one copy on
+// every GPU: the temporaries of tcg_reduce_noalloc.  Host code never uses the
+// array's name as an address: the address of each GPU's copy is looked up once
+// (tcg_reduce_scratch_init) and kept in g_scratch.
+constexpr size_t NOALLOC_SCRATCH_BYTES = TCG_REDUCE_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+static unsigned char* g_scratch[MAX_DEVICES] = {nullptr};
+
 namespace
 {
 
@@ -306,6 +316,74 @@ __global__ __launch_bounds__(RED_BLOCK) void argmax_k (
 	if (threadIdx.x == 0) { out[blockIdx.x] = (T) sidx[0]; }
 }
 
+// Where the temporaries of a reduction come from: partial results [A, S, B]
+// of a reduced dim split over S workgroups, and what is left of the tensor
+// between two steps of a reduction over separated dims
+struct Scratch
+{
+	virtual ~Scratch (void) = default;
+	virtual int take (tcg_ctx* ctx, size_t bytes, void** out) = 0;
+	virtual void give (tcg_ctx* ctx, void* ptr, size_t bytes) = 0;
+};
+
+/// The context's pool (or the recording, while one is open)
+struct PoolScratch final : public Scratch
+{
+	int take (tcg_ctx* ctx, size_t bytes, void** out) override { return tcg_alloc(ctx, bytes, out); }
+	void give (tcg_ctx* ctx, void* ptr, size_t bytes) override { tcg_free(ctx, ptr, bytes); }
+};
+
+/// Hands out at most four 256-byte aligned pieces of one GPU's scratch array
+/// at a time (a reduction step holds its operand, its result and its partial
+/// results); lowest fitting address first
+struct FixedScratch final : public Scratch
+{
+	FixedScratch (unsigned char* base) : base_(base) {}
+
+	int take (tcg_ctx* ctx, size_t bytes, void** out) override
+	{
+		size_t need = (bytes + 255) & ~(size_t) 255;
+		size_t at = 0;
+		for (bool moved = true; moved;)
+		{
+			moved = false;
+			for (int i = 0; i < 4; ++i)
+			{
+				if (size_[i] > 0 && at < off_[i] + size_[i] && off_[i] < at + need)
+				{
+					at = off_[i] + size_[i];
+					moved = true;
+				}
+			}
+		}
+		int slot = 0;
+		while (slot < 4 && size_[slot] > 0) { ++slot; }
+		if (slot == 4 || at + need > NOALLOC_SCRATCH_BYTES)
+		{
+			return tcg_fail(ctx, TCG_ERR_ARG,
+				"tcg_reduce_noalloc: the temporaries of this reduction (%zu more bytes) do not fit the fixed %zu-byte scratch memory; use tcg_reduce",
+				need, NOALLOC_SCRATCH_BYTES);
+		}
+		off_[slot] = at;
+		size_[slot] = need;
+		*out = base_ + at;
+		return TCG_OK;
+	}
+
+	void give (tcg_ctx*, void* ptr, size_t) override
+	{
+		size_t at = (size_t) ((unsigned char*) ptr - base_);
+		for (int i = 0; i < 4; ++i)
+		{
+			if (size_[i] > 0 && off_[i] == at) { size_[i] = 0; }
+		}
+	}
+
+	unsigned char* base_;
+	size_t off_[4] = {0, 0, 0, 0};
+	size_t size_[4] = {0, 0, 0, 0};
+};
+
 uint32_t ilog2_floor (uint64_t v)
 {
 	uint32_t l = 0;
@@ -340,7 +418,7 @@ int launch_outer (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uin
 
 // [A, R, B] -> [A, B]
 template <typename T, int OP>
-int reduce_step (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint64_t B)
+int reduce_step (tcg_ctx* ctx, Scratch& mem, const T* in, T* out, uint64_t A, uint64_t R, uint64_t B)
 {
 	const uint64_t target_blocks = (uint64_t) ctx->num_cus * TCG_RED_BLOCKS_PER_CU;
 	if (A == 1)
@@ -360,11 +438,11 @@ int reduce_step (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint
 		S = (R + chunk - 1) / chunk;
 		if (S == 1) { return launch_inner<T,OP>(ctx, in, out, R, B, 1, chunk); }
 		void* partial = nullptr;
-		int rc = tcg_alloc(ctx, sizeof(T) * B * S, &partial);
+		int rc = mem.take(ctx, sizeof(T) * B * S, &partial);
 		if (rc != TCG_OK) { return rc; }
 		rc = launch_inner<T,OP>(ctx, in, (T*) partial, R, B, (uint32_t) S, chunk);
 		if (rc == TCG_OK) { rc = launch_inner<T,OP>(ctx, (const T*) partial, out, S, B, 1, S); }
-		tcg_free(ctx, partial, sizeof(T) * B * S);
+		mem.give(ctx, partial, sizeof(T) * B * S);
 		return rc;
 	}
 	bool vec = tcg_aligned16(in) && (A % Vec16<T>::N == 0);
@@ -387,16 +465,16 @@ int reduce_step (tcg_ctx* ctx, const T* in, T* out, uint64_t A, uint64_t R, uint
 	S = (R + chunk - 1) / chunk;
 	if (S == 1) { return launch_outer<T,OP>(ctx, in, out, A, R, B, 1, chunk, txlog2, vec); }
 	void* partial = nullptr;
-	int rc = tcg_alloc(ctx, sizeof(T) * A * S * B, &partial);
+	int rc = mem.take(ctx, sizeof(T) * A * S * B, &partial);
 	if (rc != TCG_OK) { return rc; }
 	rc = launch_outer<T,OP>(ctx, in, (T*) partial, A, R, B, (uint32_t) S, chunk, txlog2, vec);
 	if (rc == TCG_OK) { rc = launch_outer<T,OP>(ctx, (const T*) partial, out, A, S, B, 1, S, txlog2, vec); }
-	tcg_free(ctx, partial, sizeof(T) * A * S * B);
+	mem.give(ctx, partial, sizeof(T) * A * S * B);
 	return rc;
 }
 
 template <typename T, int OP>
-int reduce_impl (tcg_ctx* ctx, const uint64_t shape[8], unsigned mask, const T* in, T* out)
+int reduce_impl (tcg_ctx* ctx, Scratch& mem, const uint64_t shape[8], unsigned mask, const T* in, T* out)
 {
 	// merge neighbouring dims of equal kind, dropping singular dims
 	uint64_t seg[8];
@@ -437,12 +515,12 @@ int reduce_impl (tcg_ctx* ctx, const uint64_t shape[8], unsigned mask, const T* 
 		if (nred > 1)
 		{
 			tmp_bytes = sizeof(T) * A * B;
-			rc = tcg_alloc(ctx, tmp_bytes, &tmp);
+			rc = mem.take(ctx, tmp_bytes, &tmp);
 			if (rc != TCG_OK) { break; }
 			dst = (T*) tmp;
 		}
-		rc = reduce_step<T,OP>(ctx, cur, dst, A, R, B);
-		if (tmp_prev) { tcg_free(ctx, tmp_prev, tmp_prev_bytes); }
+		rc = reduce_step<T,OP>(ctx, mem, cur, dst, A, R, B);
+		if (tmp_prev) { mem.give(ctx, tmp_prev, tmp_prev_bytes); }
 		tmp_prev = tmp;
 		tmp_prev_bytes = tmp_bytes;
 		cur = dst;
@@ -457,11 +535,42 @@ int reduce_impl (tcg_ctx* ctx, const uint64_t shape[8], unsigned mask, const T* 
 			--nseg;
 		}
 	}
-	if (tmp_prev) { tcg_free(ctx, tmp_prev, tmp_prev_bytes); }
+	if (tmp_prev) { mem.give(ctx, tmp_prev, tmp_prev_bytes); }
 	return rc;
 }
 
+int reduce_any (tcg_ctx* ctx, Scratch& mem, int opcode, int dtype, const uint64_t shape[8],
+	unsigned rankmask, const void* in, void* out)
+{
+	TCG_DISPATCH_TYPE(ctx, dtype,
+		switch (opcode)
+		{
+			case TCG_REDUCE_SUM: return reduce_impl<T,TCG_REDUCE_SUM>(ctx, mem, shape, rankmask, (const T*) in, (T*) out);
+			case TCG_REDUCE_PROD: return reduce_impl<T,TCG_REDUCE_PROD>(ctx, mem, shape, rankmask, (const T*) in, (T*) out);
+			case TCG_REDUCE_MIN: return reduce_impl<T,TCG_REDUCE_MIN>(ctx, mem, shape, rankmask, (const T*) in, (T*) out);
+			default: return reduce_impl<T,TCG_REDUCE_MAX>(ctx, mem, shape, rankmask, (const T*) in, (T*) out);
+		});
+	return TCG_OK;
+}
+
 } // namespace
+
+// Called by tcg_ctx_create with the context's device current: looks up where
+// this GPU keeps its copy of the scratch array
+int tcg_reduce_scratch_init (tcg_ctx* ctx)
+{
+	if (ctx->device < 0 || ctx->device >= MAX_DEVICES)
+	{
+		return tcg_fail(ctx, TCG_ERR_ARG, "device %d: at most %d devices", ctx->device, MAX_DEVICES);
+	}
+	if (nullptr == g_scratch[ctx->device])
+	{
+		unsigned char* ptr = nullptr;
+		TCG_HIP(ctx, hipGetSymbolAddress((void**) &ptr, HIP_SYMBOL(scratch)));
+		g_scratch[ctx->device] = ptr;
+	}
+	return TCG_OK;
+}
 
 extern "C" {
 
@@ -474,15 +583,23 @@ int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
 	TCG_REQUIRE(ctx, rankmask < 256, "tcg_reduce: rank set 0x%x names a dim >= 8", rankmask);
 	if (tcg_n_elems(shape) == 0) { return TCG_OK; }
 	if (tcg_small_mode(ctx)) { return tcg_small_reduce(ctx, opcode, dtype, shape, rankmask, in, out); }
-	TCG_DISPATCH_TYPE(ctx, dtype,
-		switch (opcode)
-		{
-			case TCG_REDUCE_SUM: return reduce_impl<T,TCG_REDUCE_SUM>(ctx, shape, rankmask, (const T*) in, (T*) out);
-			case TCG_REDUCE_PROD: return reduce_impl<T,TCG_REDUCE_PROD>(ctx, shape, rankmask, (const T*) in, (T*) out);
-			case TCG_REDUCE_MIN: return reduce_impl<T,TCG_REDUCE_MIN>(ctx, shape, rankmask, (const T*) in, (T*) out);
-			default: return reduce_impl<T,TCG_REDUCE_MAX>(ctx, shape, rankmask, (const T*) in, (T*) out);
-		});
-	return TCG_OK;
+	PoolScratch mem;
+	return reduce_any(ctx, mem, opcode, dtype, shape, rankmask, in, out);
+}
+
+int tcg_reduce_noalloc (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
+	unsigned rankmask, const void* in, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, opcode >= TCG_REDUCE_SUM && opcode <= TCG_REDUCE_MAX, "tcg_reduce_noalloc: opcode %d is not a reduction", opcode);
+	TCG_REQUIRE(ctx, shape && in && out, "tcg_reduce_noalloc: NULL pointer");
+	TCG_REQUIRE(ctx, rankmask < 256, "tcg_reduce_noalloc: rank set 0x%x names a dim >= 8", rankmask);
+	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "tcg_reduce_noalloc"); }
+	unsigned char* base = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch[ctx->device] : nullptr;
+	if (nullptr == base) { return tcg_fail(ctx, TCG_ERR_HIP, "tcg_reduce_noalloc: no scratch memory on device %d", ctx->device); }
+	if (tcg_n_elems(shape) == 0) { return TCG_OK; }
+	FixedScratch mem(base);
+	return reduce_any(ctx, mem, opcode, dtype, shape, rankmask, in, out);
 }
 
 int tcg_argmax (tcg_ctx* ctx, int dtype, const uint64_t shape[8], int return_dim,

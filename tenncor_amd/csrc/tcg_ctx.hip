@@ -79,6 +79,14 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		delete ctx;
 		return rc;
 	}
+	if (tcg_reduce_scratch_init(ctx) != TCG_OK)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: %s", ctx->error.c_str());
+		(void) hipFree(ctx->rng_state);
+		(void) hipHostFree(ctx->staging);
+		delete ctx;
+		return rc;
+	}
 	*out = ctx;
 	return TCG_OK;
 }

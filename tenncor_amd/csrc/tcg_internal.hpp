@@ -161,6 +161,10 @@ int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
 	const float* image, const tcg_conv_operand& op, const float* B, uint64_t ldb,
 	float* C, uint64_t ldc, bool* handled);
 
+// reduce.hip: looks up this GPU's copy of the scratch memory of
+// tcg_reduce_noalloc; called once per context with the device current
+int tcg_reduce_scratch_init (tcg_ctx* ctx);
+
 // Number of workgroups for a streaming kernel: enough to cover `work` items,
 // capped at a multiple of the CU count so that a grid-stride loop takes over
 static inline unsigned tcg_grid (const tcg_ctx* ctx, uint64_t work_items,
