@@ -32,19 +32,53 @@ ROWS, COLS = 4096, 16384
 N = ROWS * COLS
 SHAPE = [COLS, ROWS]  # tenncor order: dim 0 fastest
 
-# HBM bytes per launch from two `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
-# counter reads for the plain NEG copy of known size: FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000.  Per kernel class of the step, bytes per launch.
-MEASURED_TRAFFIC = {
-    "ew_binary_f32": (2 * 262162 + 262144) * 1024,
-    "ew_binary_i32": (2 * 262162 + 262144) * 1024,
-    "ew_unary_f32": (2 * 131096 + 262144) * 1024,
-    "reduce_dim0_f32": (2 * 131089 + 134) * 1024,
-    "reduce_dim0_i32": (2 * 131089 + 134) * 1024,
-    "reduce_dim1_f32": (4 * 65685 + 576) * 1024,   # main launch + second pass
-    "reduce_dim1_i32": (4 * 65685 + 576) * 1024,
+# Which kernels of the profile make up one launch of each kernel class of the step
+CLASS_KERNELS = {
+    "ew_binary_f32": ["ew_binary_vec_k<float, 30>", "ew_binary_vec_k<float, 32>"],
+    "ew_binary_i32": ["ew_binary_vec_k<int, 30>", "ew_binary_vec_k<int, 32>"],
+    "ew_unary_f32": ["ew_unary_vec_k<float, 7>", "ew_unary_vec_k<float, 11>", "ew_unary_vec_k<float, 12>"],
+    "reduce_dim0_f32": ["reduce_inner_k<float, 17, true>", "reduce_inner_k<float, 20, true>"],
+    "reduce_dim0_i32": ["reduce_inner_k<int, 17, true>", "reduce_inner_k<int, 20, true>"],
+    "reduce_dim1_f32": ["reduce_outer_k<float, 17, true>", "reduce_outer_k<float, 20, true>"],
+    "reduce_dim1_i32": ["reduce_outer_k<int, 17, true>", "reduce_outer_k<int, 20, true>"],
 }
+LAUNCHES_PER_STEP = {"ew_binary_f32": 2, "ew_unary_f32": 3, "reduce_dim0_f32": 2, "reduce_dim1_f32": 2,
+                     "ew_binary_i32": 2, "reduce_dim0_i32": 2, "reduce_dim1_i32": 2}
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "config2_hbm_traffic_pmc.txt")
+
+
+def measured_traffic(path=TRAFFIC_SUMMARY):
+    """HBM bytes per launch of every kernel class, from the committed summary of
+    two `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB
+    per dispatch).  The summary states how many passes over the step the
+    profiled command made and the factor each counter is scaled by (what it
+    reads for the plain NEG copy of known size); its table gives the calls and
+    the raw averages per kernel.  A class whose kernels are not all in the
+    table (the kernels changed since the profile was taken) reports None."""
+    try:
+        text = open(path).read().splitlines()
+    except OSError:
+        return {}
+    passes, scale_f, scale_w, rows = None, None, None, {}
+    for line in text:
+        parts = line.split()
+        if line.startswith("passes:"):
+            passes = int(parts[1])
+        elif line.startswith("scale:"):
+            scale_f, scale_w = float(parts[2]), float(parts[4])
+        elif len(parts) >= 4 and parts[-1].replace(".", "").isdigit() and parts[-2].replace(".", "").isdigit() \
+                and parts[-3].isdigit():
+            rows[" ".join(parts[:-3])] = (int(parts[-3]), float(parts[-2]), float(parts[-1]))
+    if not passes or scale_f is None:
+        return {}
+    out = {}
+    for cls, names in CLASS_KERNELS.items():
+        if not all(n in rows for n in names):
+            out[cls] = None
+            continue
+        kib = sum(rows[n][0] * (rows[n][1] * scale_f + rows[n][2] * scale_w) for n in names)
+        out[cls] = int(round(kib * 1024 / (passes * LAUNCHES_PER_STEP[cls])))
+    return out
 
 
 def algorithmic_bytes():
@@ -180,19 +214,8 @@ def run_extras(ctx, capi):
     a = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
     b = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
     c = ctx.empty(M * M, np.float32)
-    # the matrix clock takes some 30 ms of matrix work to settle after the
-    # streaming kernels above: the timed launches start once it has
-    for _ in range(40):
-        ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
-    ctx.timer_begin()
     reps = 20
-    for _ in range(reps):
-        ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
-    ms = ctx.timer_end() / reps
-    tf = 2.0 * M ** 3 / (ms * 1e-3) / 1e12
-    extra["matmul_4096_fp32_TFLOPs"] = round(tf, 2)
-    extra["matmul_4096_fp32_ms"] = round(ms, 4)
-    extra["matmul_4096_frac_of_fp32_mfma_peak"] = round(tf / MFMA_F32_PEAK_TFLOPS, 4)
+    extra.update(time_matmul_4096(ctx, capi, a, b, c, settle=40, reps=reps))
     # the same product in double (v_mfma_f64_16x16x4_f64)
     M2 = 4096
     a64 = ctx.upload(rng.standard_normal(M2 * M2) / 64)
@@ -245,6 +268,46 @@ def run_extras(ctx, capi):
     for buf in (a, b, c, d):
         buf.release()
     return extra
+
+
+def time_matmul_4096(ctx, capi, a, b, c, settle, reps):
+    """`reps` 4096^3 fp32 products timed with HIP events on the launch stream,
+    after `settle` untimed ones: the matrix clock takes some 30 ms of matrix
+    work to settle after streaming kernels."""
+    M = 4096
+    for _ in range(settle):
+        ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
+    ctx.timer_begin()
+    for _ in range(reps):
+        ctx.matmul(capi.FLOAT, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
+    ms = ctx.timer_end() / reps
+    flops = 2 * M ** 3
+    tf = flops / (ms * 1e-3) / 1e12
+    return {
+        "matmul_4096_fp32_TFLOPs": round(tf, 2), "matmul_4096_fp32_ms": round(ms, 4),
+        "matmul_4096_frac_of_fp32_mfma_peak": round(tf / MFMA_F32_PEAK_TFLOPS, 4),
+        "roofline_matmul": {"bound": "mfma", "kernel": "gemm_mfma_k<128, 128, 2, false, false, 0> on 4096^3 fp32",
+                            "flops": flops, "avg_ms": round(ms, 4), "achieved": round(tf, 2),
+                            "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_F32_PEAK_TFLOPS, 4),
+                            "launches": reps, "untimed_launches_before": settle},
+    }
+
+
+def run_matmul_only(settle=100, reps=100):
+    """The product third of the metric alone: nothing but 4096^3 fp32 launches in
+    the process, so that a kernel trace or a counter run of this command holds
+    one kernel at one shape."""
+    from tenncor_amd import capi
+    ctx = capi.Context(0)
+    M = 4096
+    rng = np.random.default_rng(3)
+    a = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
+    b = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
+    c = ctx.empty(M * M, np.float32)
+    out = time_matmul_4096(ctx, capi, a, b, c, settle, reps)
+    out["device"] = ctx.arch
+    ctx.close()
+    return out
 
 
 def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
@@ -454,9 +517,13 @@ def main():
     ap.add_argument("--graph-config", type=int, choices=[1, 4, 5], default=None,
                     help="time only this whole-graph configuration and print its line (for profiling)")
     ap.add_argument("--evaluator", choices=["plain", "replay", "replay_launches", "replay_unfused"], default="replay")
-    ap.add_argument("--reps", type=int, default=20, help="timed evaluations with --graph-config 4 or 5")
+    ap.add_argument("--reps", type=int, default=None,
+                    help="timed evaluations with --graph-config 4 or 5 (default 20), timed launches with --matmul-only (100)")
     ap.add_argument("--optimize", action="store_true",
                     help="with --graph-config: clean the graph up first (duplicates merged, constants folded, conversions)")
+    ap.add_argument("--matmul-only", action="store_true",
+                    help="run only 4096^3 fp32 products (--settle untimed, then --reps timed) and print their line")
+    ap.add_argument("--settle", type=int, default=100, help="untimed launches before the timed ones with --matmul-only")
     ap.add_argument("--matmul-ramp", action="store_true",
                     help="print the 4096^3 product rate of successive blocks of ten launches from a cold start")
     args = ap.parse_args()
@@ -467,13 +534,15 @@ def main():
     if args.matmul_ramp:
         print(json.dumps(run_matmul_ramp()))
         return
+    if args.matmul_only:
+        print(json.dumps(run_matmul_only(settle=args.settle, reps=args.reps or 100)))
+        return
     if args.graph_config is not None:
-        print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps, optimize=args.optimize)))
+        print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps or 20, optimize=args.optimize)))
         return
     wall, per_class, extra, arch = run_gpu(args.steps, args.warmup, graphs=not args.no_graphs)
     abytes = algorithmic_bytes()
-    launches_per_step = {"ew_binary_f32": 2, "ew_unary_f32": 3, "reduce_dim0_f32": 2, "reduce_dim1_f32": 2,
-                         "ew_binary_i32": 2, "reduce_dim0_i32": 2, "reduce_dim1_i32": 2}
+    launches_per_step = LAUNCHES_PER_STEP
     total_bytes = sum(abytes.values())
     ms_per_step = wall * 1e3 / args.steps
     value = total_bytes / (wall / args.steps) / 1e9
@@ -495,7 +564,9 @@ def main():
                                "int32 ADD,MUL + the same reductions)",
                    "algorithmic_bytes_per_step": total_bytes, "device": arch},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": dom["GBps"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": dom["frac"], "traffic": MEASURED_TRAFFIC.get(dominant)},
+                     "unit": "GB/s", "frac": dom["frac"], "traffic": measured_traffic().get(dominant),
+                     "traffic_source": "profiles/config2_hbm_traffic_pmc.txt"},
+        "roofline_matmul": extra.pop("roofline_matmul", None),
         "kernels": kernels,
         "extra": extra,
     }

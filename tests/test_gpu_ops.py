@@ -851,6 +851,79 @@ def test_full_size_properties_config2(ctx, ops):
     np.testing.assert_array_equal(ops.permute(prod, [1, 0]).get().reshape(16384, 4096)[5], p_host[:, 5])
 
 
+def test_full_size_config2_fp32_chain_and_reductions(ctx, ops, oracle):
+    """configs[1] in fp32 at np[4096,16384]: ADD, MUL, EXP, TANH, SIGMOID node by
+    node, every intermediate against the oracle on 256 seeded rows and 256 seeded
+    columns at 1e-5 (the oracle runs on the slices: elementwise results do not
+    depend on their neighbours), then REDUCE_SUM / REDUCE_MAX over each dim
+    against an fp64 sum of the chain result the device itself produced, at 1e-4
+    of max(|ref|, mean|ref|) -- 16384-long fp32 row sums are the case where a
+    sequential fp32 accumulation would fail that bar -- and the same reductions
+    of the oracle's own chain result over the checked rows and columns."""
+    rng = np.random.default_rng(2)
+    shape = [16384, 4096]
+    rows_n, cols_n = 4096, 16384
+    n = rows_n * cols_n
+    a, b, c = (rng.uniform(-1, 1, n).astype(np.float32) for _ in range(3))
+    ta, tb, tc = (ops.from_host(ctx, v, shape) for v in (a, b, c))
+    t1 = ops.binary("ADD", ta, tb)
+    t2 = ops.binary("MUL", t1, tc)
+    t3 = ops.unary("EXP", t2)
+    t4 = ops.unary("TANH", t3)
+    t5 = ops.unary("SIGMOID", t4)
+    rsel = np.sort(rng.choice(rows_n, 256, replace=False))
+    csel = np.sort(rng.choice(cols_n, 256, replace=False))
+
+    def pick(flat):
+        m = flat.reshape(rows_n, cols_n)
+        return np.ascontiguousarray(m[rsel]).reshape(-1), np.ascontiguousarray(m[:, csel]).reshape(-1)
+
+    sa, sb, sc = pick(a), pick(b), pick(c)
+    chain_ref = []
+    for k in range(2):  # rows, then columns
+        r1 = oracle.binary("ADD", sa[k], sb[k])
+        r2 = oracle.binary("MUL", r1, sc[k])
+        r3 = oracle.unary("EXP", r2)
+        r4 = oracle.unary("TANH", r3)
+        r5 = oracle.unary("SIGMOID", r4)
+        chain_ref.append((r1, r2, r3, r4, r5))
+    final = None
+    for idx, t in enumerate((t1, t2, t3, t4, t5)):
+        got = t.get()
+        for k in range(2):
+            ref = chain_ref[k][idx]
+            sel = pick(got)[k]
+            if idx < 2:
+                np.testing.assert_array_equal(sel, ref)  # one rounding each: the same bits
+            else:
+                np.testing.assert_allclose(sel, ref, rtol=EW_RTOL, atol=0)
+        final = got
+    assert np.isfinite(final).all()
+    m64 = final.reshape(rows_n, cols_n).astype(np.float64)
+    for rank_set, axis in (([0], 1), ([1], 0)):
+        got_sum = ops.reduce("REDUCE_SUM", t5, rank_set).get()
+        assert_acc_close(got_sum, m64.sum(axis=axis))
+        got_max = ops.reduce("REDUCE_MAX", t5, rank_set).get()
+        np.testing.assert_array_equal(got_max, final.reshape(rows_n, cols_n).max(axis=axis))
+    # the same against the oracle's chain: row sums of the checked rows, and the
+    # oracle's own reduction (fp64 accumulation) of those rows
+    got_rows = ops.reduce("REDUCE_SUM", t5, [0]).get()[rsel]
+    ref_rows, _ = oracle.reduce("REDUCE_SUM", chain_ref[0][4], [cols_n, 256], [0], wide_acc=True)
+    assert_acc_close(got_rows, ref_rows)
+    got_cols = ops.reduce("REDUCE_SUM", t5, [1]).get()[csel]
+    ref_cols, _ = oracle.reduce("REDUCE_SUM", chain_ref[1][4], [256, rows_n], [1], wide_acc=True)
+    assert_acc_close(got_cols, ref_cols)
+    ref_max, _ = oracle.reduce("REDUCE_MAX", chain_ref[0][4], [cols_n, 256], [0])
+    np.testing.assert_allclose(ops.reduce("REDUCE_MAX", t5, [0]).get()[rsel], ref_max, rtol=EW_RTOL)
+    # inputs whose sums do not hide errors behind a large mean: the signed product t2
+    # (row sums are O(sqrt(n)) around zero), relative to max(|ref|, mean|ref|)
+    p64 = t2.get().reshape(rows_n, cols_n).astype(np.float64)
+    for rank_set, axis in (([0], 1), ([1], 0)):
+        assert_acc_close(ops.reduce("REDUCE_SUM", t2, rank_set).get(), p64.sum(axis=axis))
+        np.testing.assert_array_equal(ops.reduce("REDUCE_MIN", t2, rank_set).get(),
+                                      t2.get().reshape(rows_n, cols_n).min(axis=axis))
+
+
 def test_full_size_properties_config3(ctx, ops):
     """4096^3 fp32 MATMUL and the batched [64,512,512] product at full size,
     checked without a CPU product: C r against A (B r) in fp64 for a random
