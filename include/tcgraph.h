@@ -87,6 +87,10 @@ int tcr_set_evaluator (int kind);
  * served by a recording, out[3] passes with nothing to do, out[4] launches in
  * the latest recording, out[5] device bytes reserved by live recordings */
 int tcr_evaluator_stats (uint64_t out[6]);
+/* How many target sets the replaying evaluator could not record (it walks
+ * them node by node instead) and, in `out`, the message of the failure that
+ * stopped the latest of them ("" when none, or under TCR_EVAL_PLAIN) */
+int tcr_evaluator_record_error (char* out, size_t capacity, uint64_t* failures);
 
 /* Where RAND_UNIF nodes whose operator is built from now on draw their values.
  * TCR_RANDOM_HOST (default): on the host from the seeded std::default_random_engine,

@@ -85,6 +85,7 @@ def build_libhost(jobs=8, verbose=False):
 NATIVE_PROGRAMS = {
     # program -> source (C++ users of the host layer, run by the tests)
     "mlp_gradients": os.path.join(ROOT, "tests", "cpp", "mlp_gradients.cpp"),
+    "runtime_memory": os.path.join(ROOT, "tests", "cpp", "runtime_memory.cpp"),
 }
 
 

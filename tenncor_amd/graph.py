@@ -27,7 +27,7 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_evaluate_ignoring", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
-    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_launch_plan", "tcr_optimize",
+    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_launch_plan", "tcr_optimize",
     "tcr_set_random", "tcr_seed",
 ]
 
@@ -78,6 +78,7 @@ def load():
         "tcr_count_functors": [vp, i32, i32p, i32p],
         "tcr_set_evaluator": [i32],
         "tcr_evaluator_stats": [u64p],
+        "tcr_evaluator_record_error": [ctypes.c_char_p, ctypes.c_size_t, u64p],
         "tcr_launch_plan": [vp, i32, i32p, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
         "tcr_optimize": [vp, i32, i32p, ctypes.c_char_p, i32, i32p, u64p],
         "tcr_set_random": [i32],
@@ -131,7 +132,14 @@ def evaluator_stats():
     if lib.tcr_evaluator_stats(out) != 0:
         raise GraphError(lib.tcr_last_error().decode())
     keys = ("plain", "recorded", "replayed", "skipped", "launches", "reserved_bytes")
-    return dict(zip(keys, [int(v) for v in out]))
+    stats = dict(zip(keys, [int(v) for v in out]))
+    buf = ctypes.create_string_buffer(2048)
+    failures = ctypes.c_uint64()
+    if lib.tcr_evaluator_record_error(buf, len(buf), ctypes.byref(failures)) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+    stats["record_failures"] = int(failures.value)
+    stats["record_error"] = buf.value.decode()
+    return stats
 
 
 def _ints(vals):

@@ -61,8 +61,11 @@ struct RuntimeMemory final : public iRuntimeMemory
 	}
 };
 
-void set_runtime (RTMemptrT mem);
-RTMemptrT get_runtime (void);
+/// The allocator registered in `ctx` under "runtime_memory"
+/// (internal/eigen/memory.hpp:141-143, src/memory.cpp:8-30); defaults to
+/// RuntimeMemory.  A custom allocator must hand out device memory.
+void set_runtime (RTMemptrT mem, global::CfgMapptrT ctx = global::context());
+RTMemptrT get_runtime (const global::CfgMapptrT& ctx = global::context());
 
 /// A borrowed buffer that returns itself after `ttl` consumer reads
 template <typename T>
@@ -445,7 +448,17 @@ struct HipOp final : public iTmpEigen<T>
 		LaunchScope& scope = launch_scope();
 		scope.ttl = ttl;
 		scope.partial = false;
-		op_(hip_context(), this->data_.get(), ptrs);
+		try
+		{
+			op_(hip_context(), this->data_.get(), ptrs);
+		}
+		catch (...)
+		{
+			// nothing was computed: a buffer left in place would read as this
+			// node's value at the next evaluation (its version has moved on)
+			this->data_.expire();
+			throw;
+		}
 		partial_ = scope.partial;
 		// the guards die here: producers whose last reader this was hand their
 		// buffer back to the pool, after this launch in stream order

@@ -401,6 +401,102 @@ struct DerivativeFuncs final : public teq::iDerivativeFuncs
 /// Evaluate `targets` with the registered evaluator on a GPU device
 void run (const teq::TensptrsT& targets, const teq::TensptrsT& ignored = {});
 
+// ---- typed handle (tenncor/eteq/etens.hpp:25-227) -------------------------
+//
+// What user code holds: a tensor plus the context whose evaluator and runtime
+// memory evaluate it.  calc<T>() is the entry of the evaluation path
+// (etens.hpp:152-162).  The reference also files every handle in a registry of
+// tensor identities (for its remote-graph services); that bookkeeping has no
+// part in evaluation and is not kept here.
+struct ETensor
+{
+	ETensor (void) = default;
+
+	ETensor (teq::TensptrT tens, const global::CfgMapptrT& ctx = global::context()) :
+		tens_(nullptr != ctx ? tens : nullptr), ctx_(ctx) {}
+
+	virtual ~ETensor (void) = default;
+
+	friend bool operator == (const ETensor& l, const std::nullptr_t&) { return nullptr == l.get(); }
+	friend bool operator == (const std::nullptr_t&, const ETensor& r) { return nullptr == r.get(); }
+	friend bool operator != (const ETensor& l, const std::nullptr_t&) { return nullptr != l.get(); }
+	friend bool operator != (const std::nullptr_t&, const ETensor& r) { return nullptr != r.get(); }
+
+	operator teq::TensptrT() const { return tens_; }
+
+	teq::iTensor& operator* () const { return *get(); }
+
+	teq::iTensor* operator-> () const { return get(); }
+
+	teq::iTensor* get (void) const { return tens_.get(); }
+
+	/// nullptr once the context is gone: nothing can be evaluated then
+	global::CfgMapptrT get_context (void) const { return ctx_.lock(); }
+
+	/// Host pointer to the value the tensor holds now (nullptr if it holds none)
+	template <typename T>
+	T* data (void)
+	{
+		check_type<T>();
+		return (T*) tens_->device().data();
+	}
+
+	/// The same, with the guard that counts as one read of the value
+	template <typename T>
+	teq::Once<T*> odata (void)
+	{
+		check_type<T>();
+		auto held = tens_->device().odata();
+		return teq::Once<T*>((T*) held.get(), std::move(held));
+	}
+
+	/// Evaluate with the context's evaluator and runtime memory, return the value
+	template <typename T>
+	T* calc (teq::TensSetT ignored = {}, size_t max_version = std::numeric_limits<size_t>::max())
+	{
+		auto ctx = get_context();
+		if (nullptr == ctx || nullptr == tens_) { return nullptr; }
+		eigen::Device device(eigen::get_runtime(ctx), max_version);
+		teq::get_eval(ctx).evaluate(device, {get()}, ignored);
+		return data<T>();
+	}
+
+	/// ... return the value with a guard: the caller's read is its last
+	template <typename T>
+	teq::Once<T*> calc_release (teq::TensSetT ignored = {}, size_t max_version = std::numeric_limits<size_t>::max())
+	{
+		auto ctx = get_context();
+		if (nullptr == ctx || nullptr == tens_) { return teq::Once<T*>(nullptr); }
+		eigen::Device device(eigen::get_runtime(ctx), max_version);
+		teq::get_eval(ctx).evaluate(device, {get()}, ignored);
+		return odata<T>();
+	}
+
+private:
+	template <typename T>
+	void check_type (void) const
+	{
+		if (nullptr == tens_) { global::fatal("cannot read the data of a null ETensor"); }
+		if (tens_->get_meta().type_code() != egen::get_type<T>())
+		{
+			global::fatalf("cannot read %s as %s", tens_->get_meta().type_label().c_str(),
+				egen::name_type(egen::get_type<T>()).c_str());
+		}
+	}
+
+	teq::TensptrT tens_;
+	global::CfgMaprefT ctx_;
+};
+
+using ETensorsT = std::vector<ETensor>;
+
+teq::TensptrsT to_tensors (const ETensorsT& etensors);
+
+/// Evaluate the targets together, in the context of the first
+/// (tenncor/eteq/src/etens.cpp:46-62)
+void run (const ETensorsT& targets, teq::TensSetT ignored = {},
+	size_t max_version = std::numeric_limits<size_t>::max());
+
 }
 
 namespace tcr

@@ -9,9 +9,11 @@
 #include <cstdarg>
 #include <cstdio>
 #include <functional>
+#include <memory>
 #include <random>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 
 namespace global
 {
@@ -50,6 +52,78 @@ inline std::string vformat (const char* fmt, va_list ap)
 	va_end(ap);
 	throw std::runtime_error(msg);
 }
+
+// String-keyed registry of the services an evaluation needs (the evaluator,
+// the runtime memory): what the reference's global::context() returns
+// (internal/global/config.hpp:9-13, src/config.cpp:8-12; its map type is
+// estd::ConfigMap<> of the cppkg library).  An entry is registered with a
+// factory, created the first time it is asked for and deleted, as the type
+// it was registered with, when it is removed or when the map goes away.
+struct ConfigMap final
+{
+	ConfigMap (void) = default;
+	ConfigMap (const ConfigMap&) = delete;
+	ConfigMap& operator = (const ConfigMap&) = delete;
+
+	~ConfigMap (void)
+	{
+		for (auto& kv : entries_) { kv.second.drop(); }
+	}
+
+	template <typename T>
+	void add_entry (const std::string& key, std::function<T*(void)> init)
+	{
+		if (entries_.count(key) > 0) { return; } // the first registration stays
+		Entry entry;
+		entry.init_ = [init]() -> void* { return init(); };
+		entry.del_ = [](void* obj) { delete static_cast<T*>(obj); };
+		entries_.emplace(key, std::move(entry));
+	}
+
+	void rm_entry (const std::string& key)
+	{
+		auto it = entries_.find(key);
+		if (it == entries_.end()) { return; }
+		it->second.drop();
+		entries_.erase(it);
+	}
+
+	bool has_entry (const std::string& key) const { return entries_.count(key) > 0; }
+
+	/// The object behind `key`, created on first use; nullptr for an unknown key
+	void* get_obj (const std::string& key)
+	{
+		auto it = entries_.find(key);
+		if (it == entries_.end()) { return nullptr; }
+		Entry& entry = it->second;
+		if (nullptr == entry.obj_ && entry.init_) { entry.obj_ = entry.init_(); }
+		return entry.obj_;
+	}
+
+private:
+	struct Entry final
+	{
+		void drop (void)
+		{
+			if (nullptr != obj_ && del_) { del_(obj_); }
+			obj_ = nullptr;
+		}
+
+		std::function<void*(void)> init_;
+		std::function<void(void*)> del_;
+		void* obj_ = nullptr;
+	};
+
+	std::unordered_map<std::string,Entry> entries_;
+};
+
+using CfgMapptrT = std::shared_ptr<ConfigMap>;
+
+using CfgMaprefT = std::weak_ptr<ConfigMap>;
+
+/// The process-wide registry; callers that keep their services apart (a test,
+/// a second session) make a map of their own and pass it instead
+CfgMapptrT context (void);
 
 // Diagnostics below `error` are routed to an optional sink (none by default)
 using LogSinkF = std::function<void(const std::string& level, const std::string& msg)>;

@@ -30,8 +30,8 @@ std::string to_string (const PairVecT<T>& pairs)
 	std::string out = "[";
 	for (size_t i = 0; i < pairs.size(); ++i)
 	{
-		out += (i ? "\\" : "") + std::string("[") + std::to_string((int) pairs[i].first) +
-			":" + std::to_string((int) pairs[i].second) + "]";
+		// as integers, first:second
+		out += (i ? "\\" : "") + std::to_string((int) pairs[i].first) + ":" + std::to_string((int) pairs[i].second);
 	}
 	return out + "]";
 }
@@ -47,11 +47,17 @@ std::string range_to_string (IT begin, IT end)
 	return out + "]";
 }
 
+/// A type without an attribute of its own: no key, and packing is an error
 template <typename T>
-struct Packer;
+struct Packer final
+{
+	std::string get_key (void) const { return ""; }
+	void pack (marsh::iAttributed&, T) const { global::fatal("unknown attribute"); }
+	void unpack (T&, const marsh::iAttributed&) const { global::fatal("unknown attribute"); }
+};
 
 template <typename T>
-const marsh::iObject* must_get_attr (const Packer<T>& packer, const marsh::iAttributed& attrib)
+const marsh::iObject* get_attr (const Packer<T>& packer, const marsh::iAttributed& attrib)
 {
 	auto key = packer.get_key();
 	auto attr = attrib.get_attr(key);
@@ -107,7 +113,7 @@ struct Packer<egen::_GENERATED_DTYPE>
 	}
 	void unpack (egen::_GENERATED_DTYPE& out, const marsh::iAttributed& attrib) const
 	{
-		out = egen::get_type(must_get_attr(*this, attrib)->to_string());
+		out = egen::get_type(get_attr(*this, attrib)->to_string());
 	}
 };
 
@@ -121,7 +127,7 @@ struct Packer<PairVecT<teq::DimT>>
 	}
 	void unpack (PairVecT<teq::DimT>& out, const marsh::iAttributed& attrib) const
 	{
-		out = decode_pair<teq::DimT>(int_contents(must_get_attr(*this, attrib)));
+		out = decode_pair<teq::DimT>(int_contents(get_attr(*this, attrib)));
 	}
 };
 
@@ -129,13 +135,20 @@ template <>
 struct Packer<PairVecT<teq::RankT>>
 {
 	std::string get_key (void) const { return "rank_pairs"; }
-	void pack (marsh::iAttributed& attrib, PairVecT<teq::RankT> dims) const
+	void pack (marsh::iAttributed& attrib, PairVecT<teq::RankT> ranks) const
 	{
-		attrib.add_attr(get_key(), std::make_unique<marsh::NumArray<int64_t>>(encode_pair(dims)));
+		for (auto& pr : ranks)
+		{
+			if (pr.first >= teq::rank_cap || pr.second >= teq::rank_cap)
+			{
+				global::fatalf("cannot reference ranks beyond rank_cap %d: %s", (int) teq::rank_cap, to_string(ranks).c_str());
+			}
+		}
+		attrib.add_attr(get_key(), std::make_unique<marsh::NumArray<int64_t>>(encode_pair(ranks)));
 	}
 	void unpack (PairVecT<teq::RankT>& out, const marsh::iAttributed& attrib) const
 	{
-		out = decode_pair<teq::RankT>(int_contents(must_get_attr(*this, attrib)));
+		out = decode_pair<teq::RankT>(int_contents(get_attr(*this, attrib)));
 	}
 };
 
@@ -150,7 +163,7 @@ struct Packer<teq::DimsT>
 	}
 	void unpack (teq::DimsT& out, const marsh::iAttributed& attrib) const
 	{
-		auto& enc = int_contents(must_get_attr(*this, attrib));
+		auto& enc = int_contents(get_attr(*this, attrib));
 		out = teq::DimsT(enc.begin(), enc.end());
 	}
 };
@@ -161,12 +174,20 @@ struct Packer<teq::RanksT>
 	std::string get_key (void) const { return "ranks"; }
 	void pack (marsh::iAttributed& attrib, teq::RanksT ranks) const
 	{
+		for (teq::RankT rank : ranks)
+		{
+			if (rank >= teq::rank_cap)
+			{
+				global::fatalf("cannot reference ranks beyond rank_cap %d: %s", (int) teq::rank_cap,
+					range_to_string(ranks.begin(), ranks.end()).c_str());
+			}
+		}
 		attrib.add_attr(get_key(), std::make_unique<marsh::NumArray<int64_t>>(
 			std::vector<int64_t>(ranks.begin(), ranks.end())));
 	}
 	void unpack (teq::RanksT& out, const marsh::iAttributed& attrib) const
 	{
-		auto& enc = int_contents(must_get_attr(*this, attrib));
+		auto& enc = int_contents(get_attr(*this, attrib));
 		out = teq::RanksT(enc.begin(), enc.end());
 	}
 };
@@ -177,12 +198,22 @@ struct Packer<std::set<teq::RankT>>
 	std::string get_key (void) const { return "rank_set"; }
 	void pack (marsh::iAttributed& attrib, std::set<teq::RankT> ranks) const
 	{
+		if (ranks.size() > teq::rank_cap)
+		{
+			global::fatalf("cannot specify %d ranks when %d (rank_cap) are available", (int) ranks.size(), (int) teq::rank_cap);
+		}
+		// rank_cap itself passes: it stands for "every dim" (internal/eigen/packattr.hpp:262-270)
+		if (false == ranks.empty() && *ranks.rbegin() > teq::rank_cap)
+		{
+			global::fatalf("cannot reference ranks beyond rank_cap %d: %s", (int) teq::rank_cap,
+				range_to_string(ranks.begin(), ranks.end()).c_str());
+		}
 		attrib.add_attr(get_key(), std::make_unique<marsh::NumArray<int64_t>>(
 			std::vector<int64_t>(ranks.begin(), ranks.end())));
 	}
 	void unpack (std::set<teq::RankT>& out, const marsh::iAttributed& attrib) const
 	{
-		auto& enc = int_contents(must_get_attr(*this, attrib));
+		auto& enc = int_contents(get_attr(*this, attrib));
 		out = std::set<teq::RankT>(enc.begin(), enc.end());
 	}
 };
@@ -197,7 +228,7 @@ struct Packer<teq::RankT>
 	}
 	void unpack (teq::RankT& out, const marsh::iAttributed& attrib) const
 	{
-		auto num = dynamic_cast<const marsh::iNumber*>(must_get_attr(*this, attrib));
+		auto num = dynamic_cast<const marsh::iNumber*>(get_attr(*this, attrib));
 		if (nullptr == num) { global::fatal("`rank` attribute is not a number"); }
 		out = (teq::RankT) num->to_int64();
 	}
@@ -214,7 +245,7 @@ struct Packer<teq::Shape>
 	}
 	void unpack (teq::Shape& out, const marsh::iAttributed& attrib) const
 	{
-		auto& enc = int_contents(must_get_attr(*this, attrib));
+		auto& enc = int_contents(get_attr(*this, attrib));
 		out = teq::Shape(teq::DimsT(enc.begin(), enc.end()));
 	}
 };
@@ -229,7 +260,7 @@ struct Packer<teq::TensptrT>
 	}
 	void unpack (teq::TensptrT& out, const marsh::iAttributed& attrib) const
 	{
-		auto obj = dynamic_cast<const teq::TensorObj*>(must_get_attr(*this, attrib));
+		auto obj = dynamic_cast<const teq::TensorObj*>(get_attr(*this, attrib));
 		if (nullptr == obj) { global::fatal("`tensor` attribute does not hold a tensor"); }
 		out = obj->get_tensor();
 	}

@@ -19,6 +19,7 @@
 
 #include <map>
 #include <memory>
+#include <string>
 
 #include "eigen_device.hpp"
 
@@ -35,6 +36,10 @@ struct ReplayEvaluator final : public teq::iEvaluator
 		size_t skipped = 0;   ///< passes with nothing to do
 		size_t launches = 0;  ///< device launches in the most recent recording
 		size_t reserved_bytes = 0; ///< device memory held by live recordings
+		size_t record_failures = 0; ///< target sets whose pass could not be recorded
+		/// why the latest of them could not ("" when none): the message of the
+		/// failure raised while recording; the set is walked node by node instead
+		std::string record_error;
 	};
 
 	/// A set of targets is recorded when it is asked for the

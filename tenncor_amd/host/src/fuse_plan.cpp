@@ -992,8 +992,16 @@ void launch_contract (const SwappedContract& call, const teq::TensSetT& targets,
 	const void* a = eigen_ref(*call.a).device_data();
 	const void* b = eigen_ref(*call.b).device_data();
 	if (nullptr == a || nullptr == b) { global::fatal("operand of a matrix product has no data"); }
-	hip_check(tcg_contract(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
-		(int) (call.pairs.size() / 2), call.pairs.data(), a, b, dst));
+	try
+	{
+		hip_check(tcg_contract(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
+			(int) (call.pairs.size() / 2), call.pairs.data(), a, b, dst));
+	}
+	catch (...)
+	{
+		static_cast<iEigen&>(out->device()).drop(); // an unfilled buffer must not read as a value
+		throw;
+	}
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
@@ -1008,9 +1016,17 @@ void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptr
 	const void* kernel = eigen_ref(*call.kernel).device_data();
 	if (nullptr == image || nullptr == kernel) { global::fatal("operand of a convolution has no data"); }
 	if (call.windowed) { ref.mark_partial(); }
-	hip_check(tcg_conv_dense_box(hip_context(), call.dtype, call.imgshape.data(), call.kshape.data(),
-		(int) call.ranks.size(), call.ranks.data(), call.ilo.data(), call.ihi.data(),
-		call.windowed ? call.olo.data() : nullptr, call.windowed ? call.ohi.data() : nullptr, image, kernel, dst));
+	try
+	{
+		hip_check(tcg_conv_dense_box(hip_context(), call.dtype, call.imgshape.data(), call.kshape.data(),
+			(int) call.ranks.size(), call.ranks.data(), call.ilo.data(), call.ihi.data(),
+			call.windowed ? call.olo.data() : nullptr, call.windowed ? call.ohi.data() : nullptr, image, kernel, dst));
+	}
+	catch (...)
+	{
+		ref.drop();
+		throw;
+	}
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
@@ -1032,8 +1048,16 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 		if (nullptr == view.ptr) { global::fatalf("operand %s has no data", leaf.base->to_string().c_str()); }
 		leaves.push_back(view);
 	}
-	hip_check(tcg_ew_fusedx(hip_context(), group.dtype, group.shape.data(), (int) leaves.size(), leaves.data(),
-		(int) group.program.size(), group.program.data(), (int) outs.size(), outs.data()));
+	try
+	{
+		hip_check(tcg_ew_fusedx(hip_context(), group.dtype, group.shape.data(), (int) leaves.size(), leaves.data(),
+			(int) group.program.size(), group.program.data(), (int) outs.size(), outs.data()));
+	}
+	catch (...)
+	{
+		for (Observable* out : group.outputs) { static_cast<iEigen&>(out->device()).drop(); }
+		throw;
+	}
 	for (teq::iTensor* tens : group.reads) { eigen_ref(*tens).odevice(); }
 }
 

@@ -259,6 +259,27 @@ int tcr_evaluator_stats (uint64_t out[6])
 	});
 }
 
+int tcr_evaluator_record_error (char* out, size_t capacity, uint64_t* failures)
+{
+	return guarded([&]
+	{
+		std::string text;
+		uint64_t count = 0;
+		if (auto replay = dynamic_cast<eigen::ReplayEvaluator*>(&teq::get_eval()))
+		{
+			text = replay->stats().record_error;
+			count = replay->stats().record_failures;
+		}
+		if (failures) { *failures = count; }
+		if (out && capacity)
+		{
+			size_t n = std::min(text.size(), capacity - 1);
+			memcpy(out, text.data(), n);
+			out[n] = '\0';
+		}
+	});
+}
+
 int tcr_shape (tcr_graph* g, int node, uint64_t shape[8])
 {
 	return guarded([&]

@@ -425,7 +425,7 @@ bool foldable (const teq::iFunctor& func)
 /// tenncor/hone/cstrules.hpp:48-65: evaluate, then wrap the values in a constant
 teq::TensptrT evaluated_constant (const teq::TensptrT& root)
 {
-	eteq::run({root});
+	eteq::run(teq::TensptrsT{root});
 	const void* data = static_cast<const teq::iTensor&>(*root).device().data();
 	if (nullptr == data) { global::fatalf("%s holds no value after evaluation", root->to_string().c_str()); }
 	teq::TensptrT out;

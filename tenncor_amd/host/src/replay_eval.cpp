@@ -199,6 +199,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 	}
 	// every value under the targets is recomputed into memory of the recording
 	tcg_ctx* ctx = hip_context();
+	std::string failure;
 	auto attempt = [&](bool as_one_kernel)
 	{
 		for (iEigen* dev : plan->devs) { dev->drop(); }
@@ -227,9 +228,15 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 				}
 			}
 		}
+		catch (const std::exception& err)
+		{
+			// kept: the node-by-node pass that follows may not hit it again
+			failure = err.what();
+			ok = false;
+		}
 		catch (...)
 		{
-			// the node-by-node pass that follows reports whatever went wrong
+			failure = "a failure that is not a std::exception";
 			ok = false;
 		}
 		plan->leaf_fed.assign(plan->leaves.size(), 0);
@@ -251,6 +258,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 				if (teq::IMMUTABLE == leaf->get_usage() || updated.count(leaf) || bytes > 256 || total + bytes > 960) { continue; }
 				const void* host = static_cast<const teq::iTensor*>(leaf)->device().data();
 				ok = TCG_OK == tcg_capture_feed(ctx, plan->leaf_ptrs[i], bytes, host);
+				if (false == ok) { failure = tcg_last_error(ctx); }
 				plan->leaf_fed[i] = bytes;
 				total += (bytes + 15) & ~(size_t) 15;
 			}
@@ -258,6 +266,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		if (ok)
 		{
 			ok = TCG_OK == tcg_capture_end(ctx, &plan->graph);
+			if (false == ok) { failure = tcg_last_error(ctx); }
 		}
 		else
 		{
@@ -274,6 +283,10 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 	if (false == ok)
 	{
 		for (iEigen* dev : plan->devs) { dev->drop(); }
+		++stats_.record_failures;
+		stats_.record_error = failure;
+		global::warnf("pass over %d functors not recorded, walked node by node instead: %s",
+			(int) plan->funcs.size(), failure.c_str());
 		return nullptr;
 	}
 	plan->after.reserve(plan->devs.size());

@@ -32,6 +32,16 @@ bool& process_exiting (void)
 	return exiting;
 }
 
+CfgMapptrT context (void)
+{
+	static CfgMapptrT ctx = std::make_shared<ConfigMap>();
+	// registered after the map exists, so it runs before the map (and the
+	// services it owns) is destroyed
+	static bool registered = (std::atexit([] { process_exiting() = true; }), true);
+	(void) registered;
+	return ctx;
+}
+
 RandEngineT& get_generator (void)
 {
 	static RandEngineT engine;
@@ -66,25 +76,29 @@ TravEvaluator::TravEvaluator (iDevice& device, const TensSetT& targets, const Te
 	}
 }
 
-static std::unique_ptr<iEvaluator>& eval_slot (void)
+// internal/teq/src/evaluator.cpp:9-30
+const std::string eval_key = "evaluater";
+
+void set_eval (iEvaluator* eval, global::CfgMapptrT ctx)
 {
-	static std::unique_ptr<iEvaluator> slot;
-	// registered after the slot exists, so it runs before the slot is destroyed
-	static bool registered = (std::atexit([] { global::process_exiting() = true; }), true);
-	(void) registered;
-	return slot;
+	if (nullptr == ctx) { global::fatal("cannot register an evaluator in a null context"); }
+	ctx->rm_entry(eval_key);
+	if (nullptr != eval)
+	{
+		ctx->add_entry<iEvaluator>(eval_key, [eval] { return eval; });
+	}
 }
 
-void set_eval (iEvaluator* eval)
+iEvaluator& get_eval (const global::CfgMapptrT& ctx)
 {
-	eval_slot().reset(eval);
-}
-
-iEvaluator& get_eval (void)
-{
-	auto& slot = eval_slot();
-	if (nullptr == slot) { slot.reset(new Evaluator()); }
-	return *slot;
+	if (nullptr == ctx) { global::fatal("cannot look an evaluator up in a null context"); }
+	auto eval = static_cast<iEvaluator*>(ctx->get_obj(eval_key));
+	if (nullptr == eval)
+	{
+		eval = new Evaluator();
+		set_eval(eval, ctx);
+	}
+	return *eval;
 }
 
 namespace

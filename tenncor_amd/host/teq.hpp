@@ -345,10 +345,11 @@ struct Evaluator final : public iEvaluator
 	}
 };
 
-/// Process-wide evaluator slot (internal/teq/src/evaluator.cpp:9-30); the
-/// slot owns the pointer.  Defaults to teq::Evaluator.
-void set_eval (iEvaluator* eval);
-iEvaluator& get_eval (void);
+/// The evaluator registered in `ctx` under "evaluater"
+/// (internal/teq/evaluator.hpp:65-67, src/evaluator.cpp:9-30); the context
+/// owns the pointer.  Defaults to teq::Evaluator.
+void set_eval (iEvaluator* eval, global::CfgMapptrT ctx = global::context());
+iEvaluator& get_eval (const global::CfgMapptrT& ctx = global::context());
 
 // ---- derivation (internal/teq/derive.hpp, src/derive.cpp) ------------------
 

@@ -41,3 +41,18 @@ def test_mlp_gradients_through_the_cpp_api(mode):
         assert len(got[parts[0]]) == int(parts[1])
     for name, key in (("gw0", "expect_gw0"), ("gb0", "expect_gb0"), ("gw1", "expect_gw1"), ("gb1", "expect_gb1")):
         np.testing.assert_allclose(got[name], fx[key], rtol=1e-12, err_msg=name)
+
+
+def test_a_callers_runtime_memory_sees_every_buffer_once():
+    """tests/cpp/runtime_memory.cpp: one operator per family run against a recording
+    iRuntimeMemory (exact allocate(bytes) / deallocate(ptr, bytes) pairing, as the
+    reference's operator tests demand of their mock, internal/eigen/test/
+    test_operator.cpp:25-67), aliases that ask for nothing, and a graph evaluated
+    through the allocator registered in a context of its own."""
+    from tenncor_amd import build
+    exe = build.native_program("runtime_memory")
+    if not os.path.exists(exe):
+        build.build_native_programs()
+    ran = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert ran.returncode == 0, ran.stdout[-3000:] + ran.stderr[-2000:]
+    assert "0 failure(s)" in ran.stdout
