@@ -60,6 +60,14 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		delete ctx;
 		return rc;
 	}
+	ctx->pool.raw_alloc = [](size_t bytes, void** out) -> int
+	{
+		hipError_t rc = hipMalloc(out, bytes);
+		if (rc != hipSuccess) { (void) hipGetLastError(); }
+		return rc == hipSuccess ? 0 : 1;
+	};
+	ctx->pool.raw_free = [](void* ptr) { (void) hipFree(ptr); };
+	ctx->pool.drain = [ctx] { (void) hipStreamSynchronize(ctx->stream); };
 	ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	ctx->arch = prop.gcnArchName;
 	size_t colon = ctx->arch.find(':');
@@ -96,7 +104,7 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	if (!ctx) { return TCG_OK; }
 	(void) hipSetDevice(ctx->device);
 	(void) hipStreamSynchronize(ctx->stream);
-	for (auto& kv : ctx->block_size) { (void) hipFree(kv.first); }
+	ctx->pool.release_all();
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
 	if (ctx->rng_state) { (void) hipFree(ctx->rng_state); }
 	(void) hipEventDestroy(ctx->ev_begin);
@@ -116,86 +124,12 @@ const char* tcg_device_arch (const tcg_ctx* ctx)
 	return ctx ? ctx->arch.c_str() : "";
 }
 
-static size_t round_block (size_t bytes)
-{
-	// 256-byte granules up to 1 MiB, then 1/8-octave steps: bounded
-	// fragmentation with few distinct size classes
-	if (bytes == 0) { bytes = 1; }
-	if (bytes <= (1u << 20)) { return (bytes + 255) & ~(size_t) 255; }
-	size_t p = (size_t) 1 << 20;
-	while (p * 2 <= bytes) { p *= 2; }
-	size_t step = p / 8;
-	return (bytes + step - 1) / step * step;
-}
-
-static void graph_adopt_block (tcg_ctx* ctx, tcg_graph* g, void* p, size_t sz)
-{
-	g->blocks[p] = sz;
-	g->held.insert(p);
-	g->bytes += sz;
-	ctx->graph_blocks[p] = g;
-}
-
 int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr)
 {
 	if (!ctx || !devptr) { return TCG_ERR_ARG; }
-	size_t sz = round_block(bytes);
-	tcg_graph* cap = ctx->capturing;
-	if (cap)
-	{
-		// blocks the captured sequence has already given back are reused first:
-		// the recorded launches run in the order they were recorded
-		auto git = cap->free_blocks.find(sz);
-		if (git != cap->free_blocks.end() && !git->second.empty())
-		{
-			*devptr = git->second.back();
-			git->second.pop_back();
-			cap->held.insert(*devptr);
-			return TCG_OK;
-		}
-	}
-	auto it = ctx->free_blocks.find(sz);
-	if (it != ctx->free_blocks.end() && !it->second.empty())
-	{
-		*devptr = it->second.back();
-		it->second.pop_back();
-		ctx->bytes_pooled -= sz;
-		ctx->bytes_in_use += sz;
-		if (cap) { graph_adopt_block(ctx, cap, *devptr, sz); }
-		return TCG_OK;
-	}
-	void* p = nullptr;
-	hipError_t err = hipMalloc(&p, sz);
-	if (err != hipSuccess && cap)
-	{
-		(void) hipGetLastError();
-		return tcg_fail(ctx, TCG_ERR_OOM, "tcg_alloc: %zu bytes while capturing: %s", sz, hipGetErrorString(err));
-	}
-	if (err != hipSuccess)
-	{
-		// give cached blocks back to the driver and retry once
-		(void) hipStreamSynchronize(ctx->stream);
-		for (auto& kv : ctx->free_blocks)
-		{
-			for (void* q : kv.second)
-			{
-				(void) hipFree(q);
-				ctx->block_size.erase(q);
-			}
-			kv.second.clear();
-		}
-		ctx->bytes_pooled = 0;
-		err = hipMalloc(&p, sz);
-		if (err != hipSuccess)
-		{
-			(void) hipGetLastError();
-			return tcg_fail(ctx, TCG_ERR_OOM, "tcg_alloc: %zu bytes: %s", sz, hipGetErrorString(err));
-		}
-	}
-	ctx->block_size[p] = sz;
-	ctx->bytes_in_use += sz;
-	if (cap) { graph_adopt_block(ctx, cap, p, sz); }
-	*devptr = p;
+	std::string why;
+	int rc = ctx->pool.take(bytes, devptr, &why);
+	if (rc != tcg_pool::OK) { return tcg_fail(ctx, TCG_ERR_OOM, "tcg_alloc: %s", why.c_str()); }
 	return TCG_OK;
 }
 
@@ -203,31 +137,17 @@ int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (!devptr) { return TCG_OK; }
-	auto it = ctx->block_size.find(devptr);
-	TCG_REQUIRE(ctx, it != ctx->block_size.end(), "tcg_free: %p was not allocated by this context", devptr);
-	size_t sz = it->second;
-	TCG_REQUIRE(ctx, round_block(bytes) == sz,
-		"tcg_free: %p was allocated with another size (%zu bytes given)", devptr, bytes);
-	auto owner = ctx->graph_blocks.find(devptr);
-	if (owner != ctx->graph_blocks.end())
-	{
-		// stays with its graph; reusable only by the sequence being recorded
-		tcg_graph* g = owner->second;
-		g->held.erase(devptr);
-		if (g == ctx->capturing) { g->free_blocks[sz].push_back(devptr); }
-		return TCG_OK;
-	}
-	ctx->free_blocks[sz].push_back(devptr);
-	ctx->bytes_in_use -= sz;
-	ctx->bytes_pooled += sz;
+	std::string why;
+	int rc = ctx->pool.give(devptr, bytes, &why);
+	if (rc != tcg_pool::OK) { return tcg_fail(ctx, TCG_ERR_ARG, "tcg_free: %p: %s", devptr, why.c_str()); }
 	return TCG_OK;
 }
 
 int tcg_mem_stats (const tcg_ctx* ctx, uint64_t* in_use, uint64_t* pooled)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
-	if (in_use) { *in_use = ctx->bytes_in_use; }
-	if (pooled) { *pooled = ctx->bytes_pooled; }
+	if (in_use) { *in_use = ctx->pool.bytes_in_use; }
+	if (pooled) { *pooled = ctx->pool.bytes_pooled; }
 	return TCG_OK;
 }
 
@@ -373,6 +293,7 @@ int tcg_capture_begin (tcg_ctx* ctx)
 	// relaxed mode: the pool may still call hipMalloc for a size it has not seen
 	TCG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
 	ctx->capturing = new tcg_graph();
+	ctx->pool.recording = ctx->capturing;
 	return TCG_OK;
 }
 
@@ -384,6 +305,7 @@ int tcg_capture_begin_small (tcg_ctx* ctx)
 	// is caught there (and fails tcg_capture_end) instead of running out of turn
 	TCG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
 	ctx->capturing = new tcg_graph();
+	ctx->pool.recording = ctx->capturing;
 	return tcg_small_begin(ctx, ctx->capturing);
 }
 
@@ -401,19 +323,23 @@ int tcg_graph_feed (tcg_ctx* ctx, tcg_graph* graph, const void* devptr, const vo
 	return tcg_small_feed(ctx, graph, devptr, host, bytes);
 }
 
+// The launches of `g` that were enqueued have finished when this returns.
+// Waits on the graph's own event, which is legal while the stream records
+// another sequence (a stream synchronisation would not be).
+static void graph_wait (tcg_graph* g)
+{
+	if (g->launched && g->done) { (void) hipEventSynchronize(g->done); }
+	g->launched = false;
+}
+
 static void graph_release (tcg_ctx* ctx, tcg_graph* g)
 {
+	graph_wait(g);
 	tcg_small_release(g);
 	if (g->exec) { (void) hipGraphExecDestroy(g->exec); }
 	if (g->graph) { (void) hipGraphDestroy(g->graph); }
-	for (auto& kv : g->blocks)
-	{
-		ctx->graph_blocks.erase(kv.first);
-		if (g->held.count(kv.first)) { continue; } // its owner frees it the ordinary way
-		ctx->free_blocks[kv.second].push_back(kv.first);
-		ctx->bytes_in_use -= kv.second;
-		ctx->bytes_pooled += kv.second;
-	}
+	if (g->done) { (void) hipEventDestroy(g->done); }
+	ctx->pool.dissolve(g);
 	delete g;
 }
 
@@ -424,8 +350,9 @@ int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out)
 	TCG_REQUIRE(ctx, ctx->capturing, "tcg_capture_end: no capture in progress");
 	tcg_graph* g = ctx->capturing;
 	ctx->capturing = nullptr;
-	g->free_blocks.clear();
+	ctx->pool.seal(g);
 	hipError_t err = hipStreamEndCapture(ctx->stream, &g->graph);
+	if (err == hipSuccess) { err = hipEventCreateWithFlags(&g->done, hipEventDisableTiming); }
 	size_t nodes = 0;
 	if (err == hipSuccess) { err = hipGraphGetNodes(g->graph, nullptr, &nodes); }
 	if (err == hipSuccess && g->small)
@@ -458,6 +385,7 @@ int tcg_capture_abort (tcg_ctx* ctx)
 	if (!ctx->capturing) { return TCG_OK; }
 	tcg_graph* g = ctx->capturing;
 	ctx->capturing = nullptr;
+	ctx->pool.seal(g);
 	(void) hipStreamEndCapture(ctx->stream, &g->graph);
 	(void) hipGetLastError();
 	graph_release(ctx, g);
@@ -468,16 +396,24 @@ int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph)
 {
 	if (!ctx || !graph) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_graph_launch: cannot launch while capturing");
-	if (graph->small) { return tcg_small_launch(ctx, graph); }
-	TCG_HIP(ctx, hipGraphLaunch(graph->exec, ctx->stream));
-	return TCG_OK;
+	int rc = TCG_OK;
+	if (graph->small) { rc = tcg_small_launch(ctx, graph); }
+	else
+	{
+		hipError_t err = hipGraphLaunch(graph->exec, ctx->stream);
+		if (err != hipSuccess) { rc = tcg_fail(ctx, TCG_ERR_HIP, "hipGraphLaunch failed: %s", hipGetErrorString(err)); }
+	}
+	// even a launch that reported a failure may have enqueued part of the sequence
+	graph->launched = true;
+	hipError_t err = hipEventRecord(graph->done, ctx->stream);
+	if (rc == TCG_OK && err != hipSuccess) { rc = tcg_fail(ctx, TCG_ERR_HIP, "hipEventRecord failed: %s", hipGetErrorString(err)); }
+	return rc;
 }
 
 int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr)
 {
 	if (!ctx || !graph) { return TCG_ERR_ARG; }
-	TCG_REQUIRE(ctx, graph->blocks.count(devptr), "tcg_graph_claim: %p does not belong to this graph", devptr);
-	graph->held.insert(devptr);
+	TCG_REQUIRE(ctx, ctx->pool.claim(graph, devptr), "tcg_graph_claim: %p does not belong to this graph", devptr);
 	return TCG_OK;
 }
 
@@ -494,8 +430,9 @@ int tcg_graph_destroy (tcg_ctx* ctx, tcg_graph* graph)
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (!graph) { return TCG_OK; }
 	TCG_REQUIRE(ctx, graph != ctx->capturing, "tcg_graph_destroy: the graph is still being captured");
-	// a launch of it may still be in flight
-	if (!ctx->capturing) { TCG_HIP(ctx, hipStreamSynchronize(ctx->stream)); }
+	// a launch of it may still be in flight: graph_release waits for the
+	// graph's last launch (also while another sequence is being recorded, when
+	// the stream itself cannot be waited for)
 	graph_release(ctx, graph);
 	return TCG_OK;
 }

@@ -15,25 +15,28 @@
 #include <vector>
 
 #include "tcg.h"
+#include "tcg_pool.hpp"
 
 #define TCG_WAVE 64
 
-// One captured launch sequence and the device memory it owns: every block
-// handed out while it was being captured stays with it (never returns to the
-// context's pool) until the graph is destroyed, because the recorded launches
-// keep addressing it
-struct tcg_graph
+// One captured launch sequence and the device memory it owns (the arena):
+// every block handed out while it was being captured stays with it (never
+// returns to the context's pool) until the graph is destroyed, because the
+// recorded launches keep addressing it
+struct tcg_graph : public tcg_arena
 {
 	hipGraph_t graph = nullptr;
 	hipGraphExec_t exec = nullptr;
-	std::map<void*,size_t> blocks;                      // block -> rounded size
-	std::set<void*> held;                               // blocks a caller currently owns
-	std::map<size_t,std::vector<void*>> free_blocks;    // reuse while capturing
-	uint64_t bytes = 0;
 	uint64_t kernels = 0;
 	// a sequence recorded as the steps of ONE kernel (tcg_capture_begin_small)
 	bool small = false;
 	struct tcg_small_pass* pass = nullptr;
+	// recorded on the context's stream after every launch of the sequence:
+	// destroying the graph waits for it, so that neither the executable graph
+	// (whose kernel arguments live in memory it owns) nor a compiled pass goes
+	// away under a launch that is still running
+	hipEvent_t done = nullptr;
+	bool launched = false;
 };
 
 struct tcg_ctx
@@ -49,10 +52,7 @@ struct tcg_ctx
 	// stream-ordered pool: freed blocks go back to a per-size free list and are
 	// handed out again without a device-wide synchronisation, which is safe
 	// because every launch of the context is ordered on `stream`
-	std::map<size_t,std::vector<void*>> free_blocks;
-	std::map<void*,size_t> block_size; // every block ever hipMalloc'ed
-	uint64_t bytes_in_use = 0;
-	uint64_t bytes_pooled = 0;
+	tcg_pool pool;
 
 	// pinned staging ring for small host->device copies
 	char* staging = nullptr;
@@ -63,10 +63,8 @@ struct tcg_ctx
 	// kernels only so that recorded launches draw fresh values at every replay
 	uint64_t* rng_state = nullptr;
 
-	// launch capture: the graph being recorded and, for every block that
-	// belongs to some graph, its owner
+	// launch capture: the graph being recorded (its arena is pool.recording)
 	tcg_graph* capturing = nullptr;
-	std::map<void*,tcg_graph*> graph_blocks;
 };
 
 int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);

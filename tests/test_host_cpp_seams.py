@@ -29,3 +29,20 @@ def test_node_api_from_cpp(tmp_path):
     ran = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert ran.returncode == 0, ran.stdout[-4000:] + ran.stderr[-2000:]
     assert "0 failure(s)" in ran.stdout
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="no host C++ compiler")
+def test_pool_and_arena_lifetimes_on_the_host(tmp_path):
+    """tests/cpp/pool_lifetimes.cpp: the block pool of a context and the arenas of
+    recorded launch sequences (tenncor_amd/csrc/tcg_pool.hpp, which holds no GPU
+    call) under a model of who holds what: a block of a live sequence is never
+    handed to anybody else, destroying a sequence returns exactly its unheld
+    blocks, nothing is given back twice, the byte counters always add up."""
+    exe = str(tmp_path / "pool_lifetimes")
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(PKG, "csrc"),
+           os.path.join(ROOT, "tests", "cpp", "pool_lifetimes.cpp"), "-o", exe]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr[-4000:]
+    ran = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert ran.returncode == 0, ran.stdout[-4000:] + ran.stderr[-2000:]
+    assert "0 failure(s)" in ran.stdout
