@@ -39,8 +39,8 @@ CLASS_KERNELS = {
     "ew_unary_f32": ["ew_unary_vec_k<float, 7>", "ew_unary_vec_k<float, 11>", "ew_unary_vec_k<float, 12>"],
     "reduce_dim0_f32": ["reduce_inner_k<float, 17, true>", "reduce_inner_k<float, 20, true>"],
     "reduce_dim0_i32": ["reduce_inner_k<int, 17, true>", "reduce_inner_k<int, 20, true>"],
-    "reduce_dim1_f32": ["reduce_outer_k<float, 17, true>", "reduce_outer_k<float, 20, true>"],
-    "reduce_dim1_i32": ["reduce_outer_k<int, 17, true>", "reduce_outer_k<int, 20, true>"],
+    "reduce_dim1_f32": ["reduce_outer_k<float, 17, true, 512, 4>", "reduce_outer_k<float, 20, true, 512, 4>"],
+    "reduce_dim1_i32": ["reduce_outer_k<int, 17, true, 512, 4>", "reduce_outer_k<int, 20, true, 512, 4>"],
 }
 LAUNCHES_PER_STEP = {"ew_binary_f32": 2, "ew_unary_f32": 3, "reduce_dim0_f32": 2, "reduce_dim1_f32": 2,
                      "ew_binary_i32": 2, "reduce_dim0_i32": 2, "reduce_dim1_i32": 2}
@@ -175,19 +175,13 @@ def run_extras(ctx, capi):
     rng = np.random.default_rng(22)
     leaves = [ctx.upload(rng.uniform(-1, 1, N).astype(np.float32)) for _ in range(3)]
     out = ctx.empty(N, np.float32)
-    # the chain as one group launch (the kernel is compiled for the program on
-    # first use) and through the three-register interpreter
+    # the chain as one group launch (the kernel is compiled for the program on first use)
     L, R, NONE = capi.FX_LEAF0, capi.FX_REG0, capi.FX_NONE
     group = [("ADD", L, L + 1, NONE, R), ("MUL", R, L + 2, NONE, R), ("EXP", R, NONE, NONE, R),
              ("TANH", R, NONE, NONE, R), ("SIGMOID", R, NONE, NONE, R), ("STORE", R, NONE, NONE, 0)]
-    O = capi.OPD_LEAF0
-    prog = [("ADD", O, O + 1, capi.OPD_ACC), ("MUL", capi.OPD_ACC, O + 2, capi.OPD_ACC),
-            ("EXP", capi.OPD_ACC, 0, capi.OPD_ACC), ("TANH", capi.OPD_ACC, 0, capi.OPD_ACC),
-            ("SIGMOID", capi.OPD_ACC, 0, capi.OPD_ACC)]
     reps = 10
     runs = {
         "fused_chain": lambda: ctx.ew_fusedx(capi.FLOAT, [COLS, ROWS], [{"ptr": b.ptr} for b in leaves], group, [out.ptr]),
-        "fused_chain_interpreted": lambda: ctx.ew_fused(capi.FLOAT, N, [b.ptr for b in leaves], prog, out.ptr),
     }
     for key, fn in runs.items():
         for _ in range(2):

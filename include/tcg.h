@@ -213,8 +213,10 @@ int tcg_rand_uniform (tcg_ctx* ctx, int dtype, uint64_t n, const void* lo,
 /* A chain of elementwise nodes evaluated in one pass over memory: what a run
  * of consecutive MatOp/TensOp closures (internal/eigen/device.hpp:304-372)
  * computes, without materialising the intermediates.
- * Three registers (ACC, T0, T1); operands name a register, a leaf or the
- * instruction's immediate. */
+ * Three registers (ACC, T0, T1, all zero at the start); operands name a
+ * register, a leaf or the instruction's immediate.  The short form of
+ * tcg_ew_fusedx for dense operands of one length: it runs as such a group
+ * (the kernel is compiled for the program on first use). */
 enum tcg_ew_operand
 {
 	TCG_OPD_NONE = 0, TCG_OPD_ACC = 1, TCG_OPD_T0 = 2, TCG_OPD_T1 = 3,

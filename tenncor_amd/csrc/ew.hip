@@ -224,112 +224,6 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_assign_k (int op, T* target, cons
 	}
 }
 
-// ---- fused chain interpreter ---------------------------------------------
-
-struct FusedProgram
-{
-	int ninstrs;
-	uint8_t opcode[TCG_EW_MAX_INSTRS];
-	uint8_t a[TCG_EW_MAX_INSTRS];
-	uint8_t b[TCG_EW_MAX_INSTRS];
-	uint8_t dst[TCG_EW_MAX_INSTRS];
-	double imm[TCG_EW_MAX_INSTRS];
-};
-
-template <typename T, int NLEAF>
-struct FusedLeaves
-{
-	const T* p[NLEAF];
-};
-
-// Every index below is a compile-time constant or a wave-uniform value taken
-// from kernel arguments, so registers are never indexed dynamically and the
-// dispatch costs scalar branches only.
-template <typename T, int NLEAF, int N>
-__device__ __forceinline__ void fused_eval (const FusedProgram& prog,
-	const T (&leaf)[NLEAF][N], T (&acc)[N])
-{
-	T t0[N], t1[N];
-#pragma unroll
-	for (int e = 0; e < N; ++e) { acc[e] = 0; t0[e] = 0; t1[e] = 0; }
-	for (int pc = 0; pc < prog.ninstrs; ++pc)
-	{
-		const int op = prog.opcode[pc];
-		const int ka = prog.a[pc], kb = prog.b[pc], kd = prog.dst[pc];
-		const T imm = (T) prog.imm[pc];
-		T r[N];
-#pragma unroll
-		for (int e = 0; e < N; ++e)
-		{
-			T va = ka == TCG_OPD_ACC ? acc[e] : ka == TCG_OPD_T0 ? t0[e] : ka == TCG_OPD_T1 ? t1[e] : imm;
-			T vb = kb == TCG_OPD_ACC ? acc[e] : kb == TCG_OPD_T0 ? t0[e] : kb == TCG_OPD_T1 ? t1[e] : imm;
-#pragma unroll
-			for (int k = 0; k < NLEAF; ++k)
-			{
-				if (ka == TCG_OPD_LEAF0 + k) { va = leaf[k][e]; }
-				if (kb == TCG_OPD_LEAF0 + k) { vb = leaf[k][e]; }
-			}
-			r[e] = kb == TCG_OPD_NONE ? apply_unary<T>(op, va) : apply_binary<T>(op, va, vb);
-		}
-#pragma unroll
-		for (int e = 0; e < N; ++e)
-		{
-			if (kd == TCG_OPD_T0) { t0[e] = r[e]; }
-			else if (kd == TCG_OPD_T1) { t1[e] = r[e]; }
-			else { acc[e] = r[e]; }
-		}
-	}
-}
-
-template <typename T, int NLEAF, bool VEC>
-__global__ __launch_bounds__(EW_BLOCK) void ew_fused_k (FusedProgram prog,
-	FusedLeaves<T,NLEAF> leaves, T* __restrict__ out, uint64_t n)
-{
-	constexpr int N = VEC ? Vec16<T>::N : 1;
-	const uint64_t nvec = n / N;
-	uint64_t i = (uint64_t) blockIdx.x * EW_BLOCK + threadIdx.x;
-	const uint64_t step = (uint64_t) gridDim.x * EW_BLOCK;
-	for (; i < nvec; i += step)
-	{
-		T leaf[NLEAF][N];
-		T acc[N];
-#pragma unroll
-		for (int k = 0; k < NLEAF; ++k)
-		{
-			if constexpr (VEC)
-			{
-				VecU<T> x;
-				x.v = ldv(leaves.p[k], i);
-#pragma unroll
-				for (int e = 0; e < N; ++e) { leaf[k][e] = x.e[e]; }
-			}
-			else { leaf[k][0] = leaves.p[k][i]; }
-		}
-		fused_eval<T,NLEAF,N>(prog, leaf, acc);
-		if constexpr (VEC)
-		{
-			VecU<T> y;
-#pragma unroll
-			for (int e = 0; e < N; ++e) { y.e[e] = acc[e]; }
-			stv(out, i, y.v);
-		}
-		else { out[i] = acc[0]; }
-	}
-	if (VEC && blockIdx.x == 0)
-	{
-		uint64_t t = nvec * N + threadIdx.x;
-		if (t < n)
-		{
-			T leaf[NLEAF][1];
-			T acc[1];
-#pragma unroll
-			for (int k = 0; k < NLEAF; ++k) { leaf[k][0] = leaves.p[k][t]; }
-			fused_eval<T,NLEAF,1>(prog, leaf, acc);
-			out[t] = acc[0];
-		}
-	}
-}
-
 // ---- host-side launchers ---------------------------------------------------
 
 template <typename T, int OP>
@@ -436,30 +330,6 @@ int cast_impl (tcg_ctx* ctx, int in_dtype, uint64_t n, const void* in, TO* out)
 		default: return tcg_fail(ctx, TCG_ERR_ARG, "tcg_cast: unknown input dtype %d", in_dtype);
 	}
 	TCG_LAUNCH_CHECK(ctx, "ew_cast");
-	return TCG_OK;
-}
-
-template <typename T, int NLEAF>
-int fused_launch (tcg_ctx* ctx, const FusedProgram& prog, const void* const* leaves, T* out, uint64_t n)
-{
-	FusedLeaves<T,NLEAF> lv;
-	bool vec = tcg_aligned16(out);
-	for (int k = 0; k < NLEAF; ++k)
-	{
-		lv.p[k] = (const T*) leaves[k];
-		vec = vec && tcg_aligned16(leaves[k]);
-	}
-	if (vec)
-	{
-		unsigned grid = tcg_grid(ctx, n / Vec16<T>::N, EW_BLOCK, 32);
-		ew_fused_k<T,NLEAF,true><<<grid, EW_BLOCK, 0, ctx->stream>>>(prog, lv, out, n);
-	}
-	else
-	{
-		unsigned grid = tcg_grid(ctx, n, EW_BLOCK, 32);
-		ew_fused_k<T,NLEAF,false><<<grid, EW_BLOCK, 0, ctx->stream>>>(prog, lv, out, n);
-	}
-	TCG_LAUNCH_CHECK(ctx, "ew_fused");
 	return TCG_OK;
 }
 
@@ -605,14 +475,34 @@ int tcg_ew_fused (tcg_ctx* ctx, int dtype, uint64_t n, int nleaves,
 	TCG_REQUIRE(ctx, nleaves >= 1 && nleaves <= TCG_EW_MAX_LEAVES, "tcg_ew_fused: %d leaves (1..%d allowed)", nleaves, TCG_EW_MAX_LEAVES);
 	TCG_REQUIRE(ctx, ninstrs >= 1 && ninstrs <= TCG_EW_MAX_INSTRS, "tcg_ew_fused: %d instructions (1..%d allowed)", ninstrs, TCG_EW_MAX_INSTRS);
 	TCG_REQUIRE(ctx, leaves && program && out, "tcg_ew_fused: NULL pointer");
-	FusedProgram prog;
-	memset(&prog, 0, sizeof(prog));
-	prog.ninstrs = ninstrs;
 	auto operand_ok = [nleaves](int k, bool allow_none)
 	{
 		if (k == TCG_OPD_NONE) { return allow_none; }
 		if (k >= TCG_OPD_ACC && k <= TCG_OPD_IMM) { return true; }
 		return k >= TCG_OPD_LEAF0 && k < TCG_OPD_LEAF0 + nleaves;
+	};
+	// the chain is a group of tcg_ew_fusedx over dense operands: ACC, T0, T1
+	// become its first three registers, the value of ACC is its one result
+	tcg_fx_instr group[TCG_EW_MAX_INSTRS + 4];
+	memset(group, 0, sizeof(group));
+	int count = 0;
+	bool written[3] = {false, false, false};
+	auto translate = [](int k) -> uint8_t
+	{
+		if (k == TCG_OPD_NONE) { return TCG_FX_NONE; }
+		if (k == TCG_OPD_IMM) { return TCG_FX_IMM; }
+		if (k >= TCG_OPD_LEAF0) { return (uint8_t) (TCG_FX_LEAF0 + (k - TCG_OPD_LEAF0)); }
+		return (uint8_t) (TCG_FX_REG0 + (k - TCG_OPD_ACC));
+	};
+	auto zero = [&](int reg) // registers start at zero
+	{
+		tcg_fx_instr& ins = group[count++];
+		ins.opcode = TCG_IDENTITY;
+		ins.a = TCG_FX_IMM;
+		ins.b = ins.c = TCG_FX_NONE;
+		ins.dst = (uint8_t) (TCG_FX_REG0 + reg);
+		ins.imm = 0;
+		written[reg] = true;
 	};
 	for (int i = 0; i < ninstrs; ++i)
 	{
@@ -622,23 +512,38 @@ int tcg_ew_fused (tcg_ctx* ctx, int dtype, uint64_t n, int nleaves,
 		TCG_REQUIRE(ctx, operand_ok(ins.a, false) && operand_ok(ins.b, unary) && (unary == (ins.b == TCG_OPD_NONE)),
 			"tcg_ew_fused: instruction %d has bad operands (%d, %d)", i, (int) ins.a, (int) ins.b);
 		TCG_REQUIRE(ctx, ins.dst >= TCG_OPD_ACC && ins.dst <= TCG_OPD_T1, "tcg_ew_fused: instruction %d has bad destination %d", i, (int) ins.dst);
-		prog.opcode[i] = ins.opcode;
-		prog.a[i] = ins.a;
-		prog.b[i] = ins.b;
-		prog.dst[i] = ins.dst;
-		prog.imm[i] = ins.imm;
-	}
-	if (n == 0) { return TCG_OK; }
-	for (int k = 0; k < nleaves; ++k) { TCG_REQUIRE(ctx, leaves[k], "tcg_ew_fused: leaf %d is NULL", k); }
-	TCG_DISPATCH_TYPE(ctx, dtype,
-		switch (nleaves)
+		for (int k : {(int) ins.a, (int) ins.b})
 		{
-			case 1: return fused_launch<T,1>(ctx, prog, leaves, (T*) out, n);
-			case 2: return fused_launch<T,2>(ctx, prog, leaves, (T*) out, n);
-			case 3: return fused_launch<T,3>(ctx, prog, leaves, (T*) out, n);
-			default: return fused_launch<T,4>(ctx, prog, leaves, (T*) out, n);
-		});
-	return TCG_OK;
+			if (k >= TCG_OPD_ACC && k <= TCG_OPD_T1 && false == written[k - TCG_OPD_ACC]) { zero(k - TCG_OPD_ACC); }
+		}
+		tcg_fx_instr& to = group[count++];
+		to.opcode = ins.opcode;
+		to.a = translate(ins.a);
+		to.b = translate(ins.b);
+		to.c = TCG_FX_NONE;
+		to.dst = translate(ins.dst);
+		to.imm = ins.imm;
+		written[ins.dst - TCG_OPD_ACC] = true;
+	}
+	if (false == written[0]) { zero(0); }
+	tcg_fx_instr& store = group[count++];
+	store.opcode = TCG_FX_STORE;
+	store.a = TCG_FX_REG0;
+	store.b = store.c = TCG_FX_NONE;
+	store.dst = 0;
+	if (n == 0) { return TCG_OK; }
+	uint64_t shape[8] = {n, 1, 1, 1, 1, 1, 1, 1};
+	tcg_fx_leaf views[TCG_EW_MAX_LEAVES];
+	memset(views, 0, sizeof(views));
+	for (int k = 0; k < nleaves; ++k)
+	{
+		TCG_REQUIRE(ctx, leaves[k], "tcg_ew_fused: leaf %d is NULL", k);
+		views[k].ptr = leaves[k];
+		views[k].stride[0] = 1;
+		for (int d = 0; d < 8; ++d) { views[k].hi[d] = shape[d]; }
+	}
+	void* outs[1] = {out};
+	return tcg_ew_fusedx(ctx, dtype, shape, nleaves, views, count, group, 1, outs);
 }
 
 } // extern "C"

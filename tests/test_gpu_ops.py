@@ -388,6 +388,58 @@ def test_data_movement_bit_exact(ctx, ops, oracle):
             np.testing.assert_array_equal(out.get(), ref, err_msg=name)
 
 
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
+def test_transposing_permutes_with_wide_and_narrow_accesses(ctx, ops, oracle, np_dtype):
+    """PERMUTE that moves the contiguous dim: tiles through LDS with 128-bit
+    accesses when extents, strides and addresses allow it, element by element
+    otherwise (odd extents, an operand at an odd element offset) -- every case
+    bit-exact against the oracle and against numpy's transpose."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of("transpose", np_dtype.__name__))
+    cases = [([64, 64], [1, 0]), ([128, 68], [1, 0]), ([260, 132, 3], [1, 0, 2]), ([512, 512, 5], [1, 0, 2]),
+             ([66, 35], [1, 0]), ([130, 62, 2], [1, 0, 2]), ([64, 6, 128], [2, 1, 0]), ([4, 1028], [1, 0]),
+             ([1028, 4], [1, 0]), ([16, 16, 16, 4], [1, 0, 3, 2])]
+    for shape, order in cases:
+        n = int(np.prod(shape))
+        x = rng.integers(-10 ** 6, 10 ** 6, n).astype(np_dtype)
+        got = ops.permute(ops.from_host(ctx, x, shape), order)
+        ref, oshape = oracle.permute(x, shape, order)
+        assert got.shape == oracle.shape8(oshape)
+        np.testing.assert_array_equal(got.get(), ref, err_msg=str((shape, order)))
+        nd = len(shape)
+        axes = [nd - 1 - order[nd - 1 - k] for k in range(nd)]
+        np.testing.assert_array_equal(ref, x.reshape(shape[::-1]).transpose(axes).reshape(-1))
+    # the same tile shapes from a source and into a destination that are not 16-byte aligned
+    shape, order = [128, 68], [1, 0]
+    n = 128 * 68
+    x = rng.integers(-10 ** 6, 10 ** 6, n + 1).astype(np_dtype)
+    src = ctx.upload(x)
+    dst = ctx.empty(n + 1, np_dtype)
+    item = np.dtype(np_dtype).itemsize
+    ctx.permute(capi.dtype_code(np_dtype), shape, order + list(range(2, 8)), src.ptr + item, dst.ptr + item)
+    np.testing.assert_array_equal(dst.get()[1:], oracle.permute(x[1:], shape, order)[0])
+
+
+def test_column_reductions_with_few_columns_take_one_launch(ctx, ops, oracle):
+    """[A, R] -> [A] with too few columns to fill the chip at full tile width:
+    narrower tiles in one pass (config 2's dim-1 reduction is the case that
+    matters: np[4096,16384] -> [16384]); values against the oracle in all
+    three dtypes, with column counts that leave partial tiles."""
+    rng = np.random.default_rng(seed_of("wide columns"))
+    for np_dtype in (np.float32, np.int32, np.float64):
+        for shape in ([16384, 1030], [4096 + 64, 1500], [20000, 1024], [8192, 2048, 2]):
+            n = int(np.prod(shape))
+            x = rng.integers(-1000, 1001, n).astype(np_dtype) if np_dtype == np.int32 else rng.uniform(-1, 1, n).astype(np_dtype)
+            t = ops.from_host(ctx, x, shape)
+            for op in ("REDUCE_SUM", "REDUCE_MAX", "REDUCE_MIN"):
+                got = ops.reduce(op, t, [1]).get()
+                ref = oracle.reduce(op, x, shape, [1], wide_acc=np_dtype != np.int32)[0]
+                if np_dtype == np.int32 or op != "REDUCE_SUM":
+                    np.testing.assert_array_equal(got, ref, err_msg=str((np_dtype.__name__, shape, op)))
+                else:
+                    assert_acc_close(got, ref)
+
+
 def test_concat_bit_exact(ctx, ops, oracle):
     rng = np.random.default_rng(13)
     sa, sb = [256, 1, 16], [512, 1, 16]
@@ -899,6 +951,22 @@ def test_full_size_config2_fp32_chain_and_reductions(ctx, ops, oracle):
                 np.testing.assert_allclose(sel, ref, rtol=EW_RTOL, atol=0)
         final = got
     assert np.isfinite(final).all()
+    # the chain as one group launch (at this size: non-temporal operand loads, two
+    # indices in flight per lane) gives the bits of the five separate launches
+    from tenncor_amd import capi
+    L, R, NONE = capi.FX_LEAF0, capi.FX_REG0, capi.FX_NONE
+    group = [("ADD", L, L + 1, NONE, R), ("MUL", R, L + 2, NONE, R), ("EXP", R, NONE, NONE, R),
+             ("TANH", R, NONE, NONE, R), ("SIGMOID", R, NONE, NONE, R), ("STORE", R, NONE, NONE, 0)]
+    fused = ctx.empty(n, np.float32)
+    ctx.ew_fusedx(capi.FLOAT, shape, [{"ptr": v.buf.ptr} for v in (ta, tb, tc)], group, [fused.ptr])
+    np.testing.assert_array_equal(fused.get(), final)
+    # ... also when the extent leaves a tail behind the whole tiles
+    odd = [16384, 4095]
+    ctx.fill_zero(fused.ptr, 4 * n)
+    ctx.ew_fusedx(capi.FLOAT, odd, [{"ptr": v.buf.ptr} for v in (ta, tb, tc)], group, [fused.ptr])
+    np.testing.assert_array_equal(fused.get()[:16384 * 4095], final[:16384 * 4095])
+    assert not fused.get()[16384 * 4095:].any()
+    fused.release()
     m64 = final.reshape(rows_n, cols_n).astype(np.float64)
     for rank_set, axis in (([0], 1), ([1], 0)):
         got_sum = ops.reduce("REDUCE_SUM", t5, rank_set).get()
