@@ -364,6 +364,23 @@ int tcg_matmul (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 	const uint64_t bshape[8], int npairs, const uint64_t* pairs,
 	const void* a, const void* b, void* out);
+
+/* out = CONTRACT(a[0], b[0]) + CONTRACT(a[1], b[1]) + ... over `nterms` pairs
+ * of operands of one pair of shapes: what an ADD node over equal CONTRACT
+ * nodes computes.  The gradient builder produces exactly this for a weight
+ * that many nodes read: tenncor/eteq/backprop.hpp:563-567 adds the gradients
+ * that arrive from each reader (internal/teq/src/derive.cpp:62-160), each of
+ * them the CONTRACT of backprop.hpp:269-359 -- sixty-four of them for a
+ * recurrent weight unrolled over sixty-four steps.  In fp32, when every
+ * operand is a matrix in place, the sum runs as ONE matrix-core product over
+ * the concatenated summed index (the operands stay where they are; at most
+ * 128 terms, summed extent a multiple of 16): the order of the fp32 additions
+ * then differs from product-by-product evaluation (same 1e-4 bar as a
+ * contraction).  Otherwise the terms are computed one by one and added in
+ * term order, bit for bit what the separate nodes give. */
+int tcg_contract_sum (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
+	const uint64_t bshape[8], int npairs, const uint64_t* pairs, int nterms,
+	const void* const* a, const void* const* b, void* out);
 /* Strided row-major GEMM the two above lower to:
  * C[b][m][n] = sum_k A[b][m][k] * B[b][k][n], element strides given;
  * trans_a: A element (m,k) at m*1 + k*lda instead of m*lda + k, same for B.

@@ -38,7 +38,7 @@ EXPORTS = [
     "tcg_timer_end", "tcg_event_create", "tcg_event_destroy", "tcg_event_record", "tcg_event_elapsed",
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
-    "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract",
+    "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
     "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
@@ -124,6 +124,7 @@ def load():
         "tcg_concat": [vp, i32, i32, i32, u64p, vpp, vp],
         "tcg_matmul": [vp, i32, u64p, u64p, vp, vp, vp],
         "tcg_contract": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
+        "tcg_contract_sum": [vp, i32, u64p, u64p, i32, u64p, i32, vpp, vpp, vp],
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
@@ -404,6 +405,14 @@ class Context:
         flat = [int(v) for p in pairs for v in p]
         self._check(self.lib.tcg_contract(self.handle, dtype, _u64(shape8(ashape)), _u64(shape8(bshape)),
                                           len(pairs), _u64(flat), a, b, dst))
+
+    def contract_sum(self, dtype, ashape, bshape, pairs, a_list, b_list, dst):
+        """sum_t CONTRACT(a_list[t], b_list[t]) into dst."""
+        flat = [int(v) for p in pairs for v in p]
+        pa = (ctypes.c_void_p * len(a_list))(*a_list)
+        pb = (ctypes.c_void_p * len(b_list))(*b_list)
+        self._check(self.lib.tcg_contract_sum(self.handle, dtype, _u64(shape8(ashape)), _u64(shape8(bshape)),
+                                              len(pairs), _u64(flat), len(a_list), pa, pb, dst))
 
     def gemm(self, dtype, M, N, K, batch, A, lda, stride_a, trans_a, B, ldb, stride_b, trans_b, C, ldc, stride_c):
         self._check(self.lib.tcg_gemm(self.handle, dtype, M, N, K, batch, A, lda, stride_a, int(trans_a),

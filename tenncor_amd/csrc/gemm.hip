@@ -364,4 +364,72 @@ int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 	return rc;
 }
 
+int tcg_contract_sum (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
+	const uint64_t bshape[8], int npairs, const uint64_t* pairs, int nterms,
+	const void* const* a, const void* const* b, void* out)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, ashape && bshape && pairs && a && b && out, "tcg_contract_sum: NULL pointer");
+	TCG_REQUIRE(ctx, nterms >= 1, "tcg_contract_sum: %d terms", nterms);
+	TCG_REQUIRE(ctx, npairs >= 1 && npairs <= 8, "tcg_contract_sum: %d dimension pairs", npairs);
+	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, a[t] && b[t], "tcg_contract_sum: operand of term %d is NULL", t); }
+	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a sum of contractions"); }
+	const size_t esz = tcg_type_size(dtype);
+	TCG_REQUIRE(ctx, esz != 0, "tcg_contract_sum: unknown dtype %d", dtype);
+	// the shape of every term as a matrix product (the rules of tcg_contract)
+	bool acom[8] = {false}, bcom[8] = {false};
+	uint64_t M = 1, N = 1, K = 1, pb_sorted[8], pa_sorted[8];
+	for (int p = 0; p < npairs; ++p)
+	{
+		uint64_t ad = pairs[2 * p], bd = pairs[2 * p + 1];
+		TCG_REQUIRE(ctx, ad < 8 && bd < 8, "tcg_contract_sum: pair %d names a dim >= 8", p);
+		TCG_REQUIRE(ctx, ashape[ad] == bshape[bd], "tcg_contract_sum: invalid shapes do not match common dimensions (pair %d)", p);
+		TCG_REQUIRE(ctx, !acom[ad] && !bcom[bd], "tcg_contract_sum: contraction dimensions must be unique for each side");
+		acom[ad] = bcom[bd] = true;
+		int q = p;
+		while (q > 0 && pa_sorted[q - 1] > ad) { pa_sorted[q] = pa_sorted[q - 1]; pb_sorted[q] = pb_sorted[q - 1]; --q; }
+		pa_sorted[q] = ad;
+		pb_sorted[q] = bd;
+		K *= ashape[ad];
+	}
+	for (int d = 0; d < 8; ++d)
+	{
+		if (!acom[d]) { M *= ashape[d]; }
+		if (!bcom[d]) { N *= bshape[d]; }
+	}
+	if (M == 0 || N == 0) { return TCG_OK; }
+	Operand oa = classify(ashape, acom), ob = classify(bshape, bcom);
+	bool same_order = true, have_last = false;
+	uint64_t last = 0;
+	for (int p = 0; p < npairs; ++p)
+	{
+		if (bshape[pb_sorted[p]] == 1) { continue; }
+		if (have_last && pb_sorted[p] < last) { same_order = false; }
+		last = pb_sorted[p];
+		have_last = true;
+	}
+	if (dtype == TCG_FLOAT && nterms > 1 && oa.direct && ob.direct && same_order)
+	{
+		// every term is a matrix in place: one product over the concatenated summed index
+		int trans_a = oa.contracted_inner ? 0 : 1, trans_b = ob.contracted_inner ? 1 : 0;
+		uint64_t lda = oa.contracted_inner ? K : M, ldb = ob.contracted_inner ? K : N;
+		bool handled = false;
+		int rc = tcg_gemm_f32_mfma_sum(ctx, M, N, K, (uint32_t) nterms, (const float* const*) a, lda, trans_a,
+			(const float* const*) b, ldb, trans_b, (float*) out, N, &handled);
+		if (rc != TCG_OK || handled) { return rc; }
+	}
+	// term by term, added up in term order: what the separate nodes compute
+	int rc = tcg_contract(ctx, dtype, ashape, bshape, npairs, pairs, a[0], b[0], out);
+	if (rc != TCG_OK || nterms == 1) { return rc; }
+	void* term = nullptr;
+	rc = tcg_alloc(ctx, esz * M * N, &term);
+	for (int t = 1; t < nterms && rc == TCG_OK; ++t)
+	{
+		rc = tcg_contract(ctx, dtype, ashape, bshape, npairs, pairs, a[t], b[t], term);
+		if (rc == TCG_OK) { rc = tcg_ew_binary(ctx, TCG_ADD, dtype, M * N, out, term, out); }
+	}
+	if (term) { tcg_free(ctx, term, esz * M * N); }
+	return rc;
+}
+
 } // extern "C"

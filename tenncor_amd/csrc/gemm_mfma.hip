@@ -8,6 +8,8 @@
 // workgroups resident on one XCD (ids congruent mod 8) cover a compact patch of
 // C and share their A/B panels through that XCD's L2.
 // MFMA-bound: 2*M*N*K flops, operands re-read from L2, each C element written once.
+#include <type_traits>
+
 #include "tcg_internal.hpp"
 
 namespace
@@ -39,6 +41,22 @@ struct GemmArgs
 	uint32_t check_ext[4];
 	int ncheck;
 };
+
+// A sum of products C = sum_t A_t B_t of equal shapes is one product over the
+// concatenated summed index: term t supplies the columns [t * k, (t + 1) * k)
+// of A and the rows of B with the same numbers.  The operands stay where they
+// are; the kernel looks the term's pointers up once per slab (k is a multiple
+// of the slab depth, so a slab never straddles two terms).
+constexpr int MAX_TERMS = 128;
+
+struct GemmSegs
+{
+	uint32_t k = 0; // columns of A (rows of B) per term
+	const float* a[MAX_TERMS];
+	const float* b[MAX_TERMS];
+};
+
+struct NoSegs {};
 
 __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_tab& row, const tcg_conv_tab& col)
 {
@@ -73,9 +91,10 @@ __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_t
 // together: one table lookup and one 128-bit load per group.  A lane's row
 // entries stay in registers; the entry of the summed index is fetched one slab
 // ahead of the load that needs it.
-template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL>
-__global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
+template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL, typename SEGS = NoSegs>
+__global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 {
+	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value;
 	constexpr int WGN = 4 / WGM;
 	constexpr int WM = BM / WGM, WN = BN / WGN; // wave tile
 	constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 accumulators per wave
@@ -109,8 +128,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 	const uint32_t tm = first_m + in_group % rows_in_group;
 	const uint32_t tn = in_group / rows_in_group;
 	const uint32_t m0 = tm * BM, n0 = tn * BN;
-	const float* __restrict__ A = g.A + (int64_t) bz * g.batch_a;
-	const float* __restrict__ B = g.B + (int64_t) bz * g.batch_b;
+	const float* __restrict__ Abase = g.A + (int64_t) bz * g.batch_a;
+	const float* __restrict__ Bbase = g.B + (int64_t) bz * g.batch_b;
 	float* __restrict__ C = g.partial ?
 		g.partial + ((int64_t) split * (g.total_tiles / g.tiles_per_batch) + bz) * ((int64_t) g.M * g.N) :
 		g.C + (int64_t) bz * g.batch_c;
@@ -164,6 +183,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 
 	auto load_slab = [&] (uint32_t k0)
 	{
+		// with terms: the operands of the term this slab belongs to, addressed
+		// by the summed index counted from the term's first column
+		const float* __restrict__ A = Abase;
+		const float* __restrict__ B = Bbase;
+		uint32_t kfirst = 0;
+		if constexpr (SEG)
+		{
+			const uint32_t term = k0 / segs.k;
+			A = segs.a[term];
+			B = segs.b[term];
+			kfirst = term * segs.k;
+		}
 #pragma unroll
 		for (int v = 0; v < A_VEC; ++v)
 		{
@@ -190,14 +221,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 				// K contiguous: BK/4 lanes per row
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t m = m0 + mm, k = k0 + kq * 4;
-				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * g.lda + k) : zero4;
+				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * g.lda + (k - kfirst)) : zero4;
 			}
 			else
 			{
 				// M contiguous: BM/4 lanes per k
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
 				uint32_t m = m0 + mq * 4, k = k0 + kk;
-				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) k * g.lda + m) : zero4;
+				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) (k - kfirst) * g.lda + m) : zero4;
 			}
 		}
 #pragma unroll
@@ -210,14 +241,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 				// N contiguous: BN/4 lanes per k
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
 				uint32_t n = n0 + nq * 4, k = k0 + kk;
-				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) k * g.ldb + n) : zero4;
+				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) (k - kfirst) * g.ldb + n) : zero4;
 			}
 			else
 			{
 				// K contiguous: BK/4 lanes per n
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t n = n0 + nn, k = k0 + kq * 4;
-				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * g.ldb + k) : zero4;
+				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * g.ldb + (k - kfirst)) : zero4;
 			}
 		}
 	};
@@ -379,8 +410,9 @@ __global__ __launch_bounds__(256) void gemm_split_sum_vec_k (const f32x4v* __res
 	}
 }
 
-template <int BM, int BN, int WGM, int IMPL>
-int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1)
+template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs>
+int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1,
+	const SEGS& segs = SEGS())
 {
 	GemmArgs g = base;
 	uint64_t tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
@@ -410,12 +442,12 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	}
 	else { splits = 1; }
 	const unsigned grid = g.total_tiles * splits;
-	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL><<<grid, 256, 0, ctx->stream>>>(g); }
+	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	else if constexpr (IMPL == 0)
 	{
-		if (!trans_a) { gemm_mfma_k<BM,BN,WGM,false,true,0><<<grid, 256, 0, ctx->stream>>>(g); }
-		else { gemm_mfma_k<BM,BN,WGM,true,true,0><<<grid, 256, 0, ctx->stream>>>(g); }
+		if (!trans_a) { gemm_mfma_k<BM,BN,WGM,false,true,0,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else { gemm_mfma_k<BM,BN,WGM,true,true,0,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	}
 	else { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
 	if (g.partial)
@@ -493,6 +525,40 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	g.ncheck = 0;
 	*handled = true;
 	return dispatch<0>(ctx, g, batch, trans_a, trans_b);
+}
+
+// C[m][n] = sum_t sum_k A_t[m][k] B_t[k][n]: `terms` products of one shape
+// (K columns each, same layouts and leading dims) as one product of depth
+// terms * K; *handled = false when the shapes do not fit
+int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
+	const float* const* A, uint64_t lda, int trans_a, const float* const* B, uint64_t ldb, int trans_b,
+	float* C, uint64_t ldc, bool* handled)
+{
+	*handled = false;
+	bool ok = terms >= 1 && terms <= (uint32_t) MAX_TERMS && M >= 32 && N >= 32 && K >= BK && K % BK == 0 &&
+		M < (1ull << 31) && N < (1ull << 31) && K * terms < (1ull << 31) &&
+		lda % 4 == 0 && ldb % 4 == 0 && ((trans_a ? M : K) % 4 == 0) && ((trans_b ? K : N) % 4 == 0);
+	for (uint32_t t = 0; t < terms && ok; ++t) { ok = tcg_aligned16(A[t]) && tcg_aligned16(B[t]); }
+	if (!ok) { return TCG_OK; }
+	GemmArgs g;
+	g.A = A[0]; g.B = B[0]; g.C = C;
+	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) (K * terms);
+	g.lda = (int64_t) lda; g.ldb = (int64_t) ldb; g.ldc = (int64_t) ldc;
+	g.batch_a = g.batch_b = g.batch_c = 0;
+	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
+	g.rows = g.sums = nullptr;
+	g.ncheck = 0;
+	GemmSegs segs;
+	segs.k = (uint32_t) K;
+	for (uint32_t t = 0; t < terms; ++t) { segs.a[t] = A[t]; segs.b[t] = B[t]; }
+	*handled = true;
+	// large tiles; ranges of the long summed index spread the tiles over the chip
+	uint64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+	uint64_t splits = (2 * (uint64_t) ctx->num_cus + tiles - 1) / tiles;
+	if (splits > g.K / 256) { splits = g.K / 256; }
+	if (splits > 32) { splits = 32; }
+	if (splits < 2) { splits = 1; }
+	return launch<128,128,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) splits, segs);
 }
 
 int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,

@@ -159,6 +159,12 @@ int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
 	const float* image, const tcg_conv_operand& op, const float* B, uint64_t ldb,
 	float* C, uint64_t ldc, bool* handled);
 
+// C = sum_t A_t B_t over `terms` products of one shape as one matrix-core
+// product over the concatenated summed index (gemm_mfma.hip)
+int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
+	const float* const* A, uint64_t lda, int trans_a, const float* const* B, uint64_t ldb, int trans_b,
+	float* C, uint64_t ldc, bool* handled);
+
 // reduce.hip: looks up this GPU's copy of the scratch memory of
 // tcg_reduce_noalloc; called once per context with the device current
 int tcg_reduce_scratch_init (tcg_ctx* ctx);

@@ -48,6 +48,22 @@ struct SwappedContract final
 	std::vector<teq::iTensor*> reads;
 };
 
+/// ADD over CONTRACT nodes of one pair of shapes (or over their PERMUTE{1,0}
+/// forms, see SwappedContract), each read by the ADD alone: the sum of products
+/// the gradient builder makes for a weight that many nodes read
+/// (tenncor/eteq/backprop.hpp:563-567 over :269-359 -- one term per step of an
+/// unrolled recurrent layer).  Launched as one tcg_contract_sum into the ADD
+/// node's buffer; the terms never hold values of their own.
+struct SummedContracts final
+{
+	Observable* node = nullptr;      ///< the ADD node that receives the result
+	std::vector<teq::iTensor*> a, b; ///< operands of the products as launched, in term order
+	std::array<uint64_t,8> ashape, bshape;
+	std::vector<uint64_t> pairs;     ///< flattened (dim of a, dim of b)
+	int dtype = 0;
+	std::vector<teq::iTensor*> reads;
+};
+
 /// CONV(PAD(x), kernel) where convolutions are all that read the PAD node:
 /// the correlation is computed from x itself, told where it sits inside the
 /// zero border, and the padded image is never laid out (conv2d and its
@@ -74,12 +90,14 @@ struct FusionPlan final
 		Observable* node = nullptr; ///< launched through its own closure, or
 		int group = -1;             ///< index into groups, or
 		int contract = -1;          ///< index into contracts, or
-		int conv = -1;              ///< index into convs
+		int conv = -1;              ///< index into convs, or
+		int sum = -1;               ///< index into sums
 	};
 
 	std::vector<FusedGroup> groups;
 	std::vector<SwappedContract> contracts;
 	std::vector<PaddedConv> convs;
+	std::vector<SummedContracts> sums;
 	std::vector<Step> steps;
 	/// functors that are computed inside a group or folded into operand views
 	/// and therefore never hold a value of their own
@@ -96,6 +114,8 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptrT& memory);
+
+void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 }
 

@@ -49,6 +49,8 @@ struct Node final
 	int swapped_from = -1;      // PERMUTE launched as the swapped product of this CONTRACT node
 	int padded_from = -1;       // CONV reading the operand of this PAD node in place of the padded image
 	bool through_conv = false;  // PAD that only such convolutions read
+	bool summed = false;        // ADD launched as one sum of the products it adds
+	bool summed_term = false;   // CONTRACT / PERMUTE that is a term of such a sum
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
 	teq::TensptrsT arg_tens;
 	std::vector<int> consumers; // functors of this pass reading the node
@@ -202,12 +204,13 @@ struct Planner final
 			n.through_conv = true;
 			for (int c : n.consumers) { nodes_[c].padded_from = (int) i; }
 		}
+		find_summed_products();
 		// a view is folded away when everything that reads it can read through it
 		std::vector<int> last_reader(nodes_.size(), 0); // position of the last launch reading through a folded view
 		for (size_t i = nodes_.size(); i-- > 0;)
 		{
 			Node& n = nodes_[i];
-			if (n.kind != VIEW || n.target || n.consumers.empty() || n.op == egen::CONTRACT || n.through_conv) { continue; }
+			if (n.kind != VIEW || n.target || n.consumers.empty() || n.op == egen::CONTRACT || n.through_conv || n.summed_term) { continue; }
 			n.absorbed = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
 			{
 				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed && false == nodes_[c].through_conv);
@@ -253,6 +256,81 @@ struct Planner final
 	{
 		const Node& n = nodes_[i];
 		return n.kind == VIEW && n.absorbed && n.op == egen::IDENTITY;
+	}
+
+	// ---- sums of products ----
+
+	/// The CONTRACT behind operand `i` of an ADD when it can be a term of a sum
+	/// of products: a CONTRACT node, or the PERMUTE that is launched as a
+	/// swapped product, read by nothing else; -1 otherwise
+	int product_term (int i) const
+	{
+		if (i < 0) { return -1; }
+		const Node& n = nodes_[i];
+		if (n.target || n.consumers.size() != 1) { return -1; }
+		if (n.op == egen::PERMUTE && n.swapped_from >= 0) { return n.swapped_from; }
+		if (n.op == egen::CONTRACT && n.kind == OTHER && n.args.size() == 2) { return i; }
+		return -1;
+	}
+
+	/// fp32 ADD nodes all of whose operands are such products of one pair of
+	/// shapes, pairs and form: one launch over the concatenated summed index
+	void find_summed_products (void)
+	{
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			Node& n = nodes_[i];
+			if (n.op != egen::ADD || n.dtype != egen::FLOAT || n.args.size() < 4 || n.args.size() > 128) { continue; }
+			// results of a few thousand elements gain nothing (and their passes are
+			// recorded as the steps of one kernel, which this launch is not)
+			if (n.f->shape().n_elems() <= 4096) { continue; }
+			std::vector<int> seen(n.args.begin(), n.args.end());
+			std::sort(seen.begin(), seen.end());
+			if (std::adjacent_find(seen.begin(), seen.end()) != seen.end()) { continue; } // x + x: two reads of one node
+			int first = product_term(n.args[0]);
+			if (first < 0) { continue; }
+			const Node& proto = nodes_[first];
+			bool swapped = nodes_[n.args[0]].op == egen::PERMUTE;
+			PairVecT<teq::RankT> dims;
+			Packer<PairVecT<teq::RankT>>().unpack(dims, *proto.f);
+			Shape8 ashape = shape8(proto.arg_tens[0]->shape()), bshape = shape8(proto.arg_tens[1]->shape());
+			bool all = true;
+			int earliest = (int) i;
+			for (int a : n.args)
+			{
+				int c = product_term(a);
+				all = c >= 0 && (nodes_[a].op == egen::PERMUTE) == swapped && nodes_[c].dtype == n.dtype;
+				if (false == all) { break; }
+				const Node& term = nodes_[c];
+				PairVecT<teq::RankT> tdims;
+				Packer<PairVecT<teq::RankT>>().unpack(tdims, *term.f);
+				all = tdims == dims && shape8(term.arg_tens[0]->shape()) == ashape && shape8(term.arg_tens[1]->shape()) == bshape;
+				if (false == all) { break; }
+				earliest = std::min(earliest, c);
+			}
+			if (false == all) { continue; }
+			// the products would read their operands where the ADD stands
+			bool rewritten = false;
+			for (int a : n.args)
+			{
+				int c = product_term(a);
+				rewritten = rewritten || written_between(c, {0, 1}, earliest, (int) i);
+			}
+			if (rewritten) { continue; }
+			n.kind = OTHER;
+			n.summed = true;
+			for (int a : n.args)
+			{
+				int c = product_term(a);
+				for (int t : {a, c})
+				{
+					nodes_[t].kind = VIEW;
+					nodes_[t].absorbed = true;
+					nodes_[t].summed_term = true;
+					nodes_[t].swapped_from = -1;
+				}
+			}
+		}
 	}
 
 	// ---- buffers that ASSIGN* nodes of the pass rewrite ----
@@ -852,6 +930,51 @@ struct Planner final
 				plan.steps.push_back(step);
 				return;
 			}
+			if (nodes_[u].summed)
+			{
+				const Node& n = nodes_[u];
+				SummedContracts call;
+				call.node = n.f;
+				call.dtype = n.dtype;
+				for (size_t k = 0; k < n.args.size(); ++k)
+				{
+					int arg = n.args[k];
+					bool swapped = nodes_[arg].op == egen::PERMUTE;
+					const Node& c = nodes_[swapped ? nodes_[arg].args[0] : arg];
+					// a swapped product is launched with its operands exchanged
+					int ia = swapped ? 1 : 0, ib = swapped ? 0 : 1;
+					call.a.push_back(c.arg_tens[ia].get());
+					call.b.push_back(c.arg_tens[ib].get());
+					if (0 == k)
+					{
+						call.ashape = shape8(c.arg_tens[ia]->shape());
+						call.bshape = shape8(c.arg_tens[ib]->shape());
+						PairVecT<teq::RankT> dims;
+						Packer<PairVecT<teq::RankT>>().unpack(dims, *c.f);
+						for (auto& d : dims)
+						{
+							call.pairs.push_back(swapped ? d.second : d.first);
+							call.pairs.push_back(swapped ? d.first : d.second);
+						}
+					}
+					// the reads the term's nodes would have counted: the product's operands
+					for (size_t j = 0; j < 2; ++j)
+					{
+						int operand = c.args[j];
+						if (operand >= 0 && false == (nodes_[operand].kind == VIEW && nodes_[operand].absorbed))
+						{
+							call.reads.push_back(c.arg_tens[j].get());
+						}
+					}
+					plan.absorbed.push_back(c.f);
+					if (swapped) { plan.absorbed.push_back(nodes_[arg].f); }
+				}
+				FusionPlan::Step step;
+				step.sum = (int) plan.sums.size();
+				plan.sums.push_back(call);
+				plan.steps.push_back(step);
+				return;
+			}
 			if (nodes_[u].kind != EW && nodes_[u].padded_from >= 0)
 			{
 				const Node& n = nodes_[u];
@@ -1000,6 +1123,33 @@ void launch_contract (const SwappedContract& call, const teq::TensSetT& targets,
 	catch (...)
 	{
 		static_cast<iEigen&>(out->device()).drop(); // an unfilled buffer must not read as a value
+		throw;
+	}
+	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
+}
+
+void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMemptrT& memory)
+{
+	Observable* out = call.node;
+	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
+	auto& ref = static_cast<iEigen&>(out->device());
+	void* dst = ref.borrow_output(ttl, memory);
+	if (nullptr == dst) { global::fatalf("%s cannot take a sum of products", out->to_string().c_str()); }
+	std::vector<const void*> a, b;
+	for (size_t t = 0; t < call.a.size(); ++t)
+	{
+		a.push_back(eigen_ref(*call.a[t]).device_data());
+		b.push_back(eigen_ref(*call.b[t]).device_data());
+		if (nullptr == a.back() || nullptr == b.back()) { global::fatal("operand of a matrix product has no data"); }
+	}
+	try
+	{
+		hip_check(tcg_contract_sum(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
+			(int) (call.pairs.size() / 2), call.pairs.data(), (int) a.size(), a.data(), b.data(), dst));
+	}
+	catch (...)
+	{
+		ref.drop();
 		throw;
 	}
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }

@@ -409,6 +409,11 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 				ss << "swapped CONTRACT+PERMUTE\n";
 				continue;
 			}
+			if (step.sum >= 0)
+			{
+				ss << "summed CONTRACT x" << plan.sums[step.sum].a.size() << "\n";
+				continue;
+			}
 			if (step.conv >= 0)
 			{
 				ss << "padded PAD+CONV" << (plan.convs[step.conv].windowed ? "+SLICE" : "") << "\n";

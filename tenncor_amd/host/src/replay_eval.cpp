@@ -222,6 +222,10 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 				{
 					launch_contract(fusion.contracts[step.contract], targets, device.memory());
 				}
+				else if (step.sum >= 0)
+				{
+					launch_sum(fusion.sums[step.sum], targets, device.memory());
+				}
 				else
 				{
 					launch_group(fusion.groups[step.group], targets, device.memory());

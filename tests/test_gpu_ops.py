@@ -440,6 +440,46 @@ def test_column_reductions_with_few_columns_take_one_launch(ctx, ops, oracle):
                     assert_acc_close(got, ref)
 
 
+def test_sum_of_contractions(ctx, ops, oracle):
+    """tcg_contract_sum against the oracle's contractions added up in fp64:
+    the LSTM weight-gradient shape family (operands {F,1,B} x {G,1,B} summed over
+    the batch, one term per time step) on the matrix cores, both operand orders,
+    int32 and odd shapes through the term-by-term route (bit-exact there)."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of("contract_sum"))
+    cases = [
+        (np.float32, [96, 1, 64], [160, 1, 64], [[1, 1], [2, 2]], 9),     # K = 64 per term: one product over 576
+        (np.float32, [64, 48], [64, 80], [[0, 0]], 5),                    # K contiguous in both operands
+        (np.float32, [40, 1, 6], [24, 1, 6], [[1, 1], [2, 2]], 4),        # K = 6: term by term
+        (np.int32, [32, 1, 16], [48, 1, 16], [[1, 1], [2, 2]], 6),
+        (np.float64, [32, 1, 16], [48, 1, 16], [[1, 1], [2, 2]], 3),
+    ]
+    for np_dtype, ashape, bshape, pairs, nterms in cases:
+        na, nb = int(np.prod(ashape)), int(np.prod(bshape))
+        draw = (lambda n: rng.integers(-50, 51, n).astype(np.int32)) if np_dtype == np.int32 else \
+            (lambda n: rng.uniform(-1, 1, n).astype(np_dtype))
+        xs, ys = [draw(na) for _ in range(nterms)], [draw(nb) for _ in range(nterms)]
+        refs = [oracle.contract(x, ashape, y, bshape, pairs, wide_acc=np_dtype != np.int32)[0] for x, y in zip(xs, ys)]
+        da, db = [ctx.upload(x) for x in xs], [ctx.upload(y) for y in ys]
+        out = ctx.empty(refs[0].size, np_dtype)
+        ctx.contract_sum(capi.dtype_code(np_dtype), ashape, bshape, pairs, [d.ptr for d in da], [d.ptr for d in db], out.ptr)
+        got = out.get()[:refs[0].size]
+        if np_dtype == np.int32:
+            total = refs[0].copy()
+            for r in refs[1:]:
+                total = (total.astype(np.int64) + r).astype(np.int32)
+            np.testing.assert_array_equal(got, total)
+        else:
+            assert_acc_close(got, np.sum(np.asarray(refs, dtype=np.float64), axis=0), rtol=ACC_RTOL if np_dtype == np.float32 else 1e-12)
+        # one term is the contraction itself
+        ctx.contract_sum(capi.dtype_code(np_dtype), ashape, bshape, pairs, [da[0].ptr], [db[0].ptr], out.ptr)
+        single = ctx.empty(refs[0].size, np_dtype)
+        ctx.contract(capi.dtype_code(np_dtype), ashape, bshape, pairs, da[0].ptr, db[0].ptr, single.ptr)
+        np.testing.assert_array_equal(out.get(), single.get())
+        for d in da + db + [out, single]:
+            d.release()
+
+
 def test_concat_bit_exact(ctx, ops, oracle):
     rng = np.random.default_rng(13)
     sa, sb = [256, 1, 16], [512, 1, 16]
@@ -1049,7 +1089,8 @@ def test_full_size_properties_config3(ctx, ops):
 def test_full_size_recordings_equal_the_walk(config):
     """configs[3] and configs[4] at their full sizes: the recorded pass (shared
     launches, exchanged products, convolutions reading their operands in
-    place) against the node-by-node walk on the same input, bit for bit."""
+    place) against the node-by-node walk on the same input, bit for bit --
+    except where a sum of products runs as one product."""
     from tenncor_amd import graph, configs
     results = {}
     for kind in ("plain", "replay_launches"):
@@ -1066,8 +1107,15 @@ def test_full_size_recordings_equal_the_walk(config):
         finally:
             g.close()
             graph.set_evaluator("plain")
-    for a, b in zip(results["plain"], results["replay_launches"]):
+    for k, (a, b) in enumerate(zip(results["plain"], results["replay_launches"])):
         assert np.isfinite(a).all()
+        if config == "lstm" and k == 1:
+            # the weight gradient: the walk computes 64 products and adds them up, the
+            # recording runs them as one product over the concatenated summed index
+            # (tcg_contract_sum), so the fp32 additions come in another order --
+            # the bar of a contraction, against the largest entry
+            assert np.abs(a - b).max() <= 1e-5 * np.abs(a).max()
+            continue
         np.testing.assert_array_equal(a, b)
 
 
