@@ -17,7 +17,12 @@
  *     crosses this boundary; tcg_last_error() gives the message
  *   - shapes are uint64_t[8] in tenncor order: dim 0 is the fastest-varying
  *     dim, unused dims are 1 (internal/teq/shape.hpp:56-59)
- *   - dtype codes follow cfg/mintype.yml:4-13: 1 double, 2 float, 3 int32
+ *   - dtype codes: 1 double, 2 float, 3 int32 (the order of cfg/mintype.yml:4-13,
+ *     the default build's types), then the integer widths the full build adds
+ *     (cfg/fulltype.yml:11-34): 4 int8, 5 uint8, 6 int16, 7 uint16, 8 uint32,
+ *     9 int64, 10 uint64.  These codes are this library's and do not move
+ *     with the host layer's build switch (whose own enum follows the yaml it
+ *     is built for).  Integer arithmetic wraps modulo 2^width
  *   - opcodes are the values of egen::_GENERATED_OPCODE, i.e. the key order
  *     of cfg/ops.yml with BAD_OP = 0 (tools/egen/plugins/opcodes.py:16-22)
  *   - data pointers are DEVICE pointers (from tcg_alloc, or any HIP device
@@ -52,7 +57,19 @@ enum tcg_status
 	TCG_ERR_OOM = 4
 };
 
-enum tcg_dtype { TCG_BAD_TYPE = 0, TCG_DOUBLE = 1, TCG_FLOAT = 2, TCG_INT32 = 3 };
+/* Element types.  1..3 are the reference's default configuration in its own
+ * numbering (cfg/mintype.yml:4-13); 4..10 are the integer widths its full
+ * configuration adds (cfg/fulltype.yml:11-34), which the reference numbers in
+ * another order (the enum it generates follows the key order of the file): a
+ * binding built for that configuration maps its codes onto these.  Integer
+ * arithmetic wraps modulo 2^width; integer division by zero, and the lowest
+ * value of a 32- or 64-bit type divided by -1 (both trap on the CPU), give 0. */
+enum tcg_dtype
+{
+	TCG_BAD_TYPE = 0, TCG_DOUBLE = 1, TCG_FLOAT = 2, TCG_INT32 = 3,
+	TCG_INT8 = 4, TCG_UINT8 = 5, TCG_INT16 = 6, TCG_UINT16 = 7, TCG_UINT32 = 8,
+	TCG_INT64 = 9, TCG_UINT64 = 10, TCG_N_DTYPES
+};
 
 enum tcg_opcode
 {

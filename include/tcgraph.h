@@ -31,7 +31,12 @@ int tcr_graph_create (tcr_graph** out);
 int tcr_graph_destroy (tcr_graph* g);
 
 /* eteq::make_variable<T>(data, shape, label) -- tenncor/eteq/make.hpp:50-56.
- * dtype: 1 double, 2 float, 3 int32; shape: 8 dims, dim 0 fastest */
+ * dtype: a code of enum tcg_dtype (include/tcg.h: 1 double, 2 float, 3 int32,
+ * and in the library built for the full type configuration 4 int8 .. 10
+ * uint64), the same numbering in both libraries although the C++ enum
+ * egen::_GENERATED_DTYPE underneath follows the reference's, which differs
+ * between the two configurations; a type the library was not built for is
+ * refused.  shape: 8 dims, dim 0 fastest */
 int tcr_variable (tcr_graph* g, int dtype, const uint64_t shape[8], const void* data,
 	const char* label, int* node);
 /* eteq::make_constant<T>(data, shape) -- tenncor/eteq/make.hpp:108-119 */

@@ -19,7 +19,12 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 RANK_CAP = 8
 DOUBLE, FLOAT, INT32 = 1, 2, 3
-NP_OF = {DOUBLE: np.float64, FLOAT: np.float32, INT32: np.int32}
+# the integer widths the full build adds (cfg/fulltype.yml:11-34)
+INT8, UINT8, INT16, UINT16, UINT32, INT64, UINT64 = 4, 5, 6, 7, 8, 9, 10
+NP_OF = {DOUBLE: np.float64, FLOAT: np.float32, INT32: np.int32,
+         INT8: np.int8, UINT8: np.uint8, INT16: np.int16, UINT16: np.uint16,
+         UINT32: np.uint32, INT64: np.int64, UINT64: np.uint64}
+_CODE_OF = {np.dtype(t): code for code, t in NP_OF.items()}
 
 # cfg/ops.yml key order (tools/egen/plugins/opcodes.py:16-22)
 OPCODES = [
@@ -54,13 +59,9 @@ def lib():
 
 def dtype_code(arr):
     t = np.asarray(arr).dtype
-    if t == np.float64:
-        return DOUBLE
-    if t == np.float32:
-        return FLOAT
-    if t == np.int32:
-        return INT32
-    raise TypeError("unsupported dtype %s" % t)
+    if t not in _CODE_OF:
+        raise TypeError("unsupported dtype %s" % t)
+    return _CODE_OF[t]
 
 
 def shape8(shape, fill=1):

@@ -34,7 +34,13 @@ extern "C" {
 
 #define ORC_RANK_CAP 8
 
-enum orc_dtype { ORC_BAD_TYPE = 0, ORC_DOUBLE = 1, ORC_FLOAT = 2, ORC_INT32 = 3 };
+enum orc_dtype
+{
+	ORC_BAD_TYPE = 0, ORC_DOUBLE = 1, ORC_FLOAT = 2, ORC_INT32 = 3,
+	/* the integer widths the full build adds (cfg/fulltype.yml:11-34) */
+	ORC_INT8 = 4, ORC_UINT8 = 5, ORC_INT16 = 6, ORC_UINT16 = 7, ORC_UINT32 = 8,
+	ORC_INT64 = 9, ORC_UINT64 = 10
+};
 
 /* cfg/ops.yml key order */
 enum orc_opcode {

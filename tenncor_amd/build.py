@@ -59,14 +59,26 @@ LIBHOST = os.path.join(PKG, "libtenncor_host.so")
 CXX = os.environ.get("CXX", "g++")
 
 
-def build_libhost(jobs=8, verbose=False):
-    """Compile the C++ host graph layer (host/src/*.cpp) against libtcg.so."""
+LIBHOST_FULL = os.path.join(PKG, "libtenncor_host_full.so")
+
+
+def build_libhost(jobs=8, verbose=False, full_types=False):
+    """Compile the C++ host graph layer (host/src/*.cpp) against libtcg.so.
+
+    full_types: the type configuration of the reference's cfg/fulltype.yml
+    (INT8 .. UINT64 besides DOUBLE, FLOAT and INT32) instead of cfg/mintype.yml,
+    as libtenncor_host_full.so: the reference picks one of the two when it
+    generates its sources (ETEQ_CFG), this build with -DEGEN_FULLTYPE."""
     from concurrent.futures import ThreadPoolExecutor
     objdir = os.path.join(PKG, "build")
     os.makedirs(objdir, exist_ok=True)
     sources = sorted(glob.glob(os.path.join(HOST, "src", "*.cpp")))
-    objs = [os.path.join(objdir, "host_" + os.path.basename(s)[:-4] + ".o") for s in sources]
+    prefix = "hostfull_" if full_types else "host_"
+    objs = [os.path.join(objdir, prefix + os.path.basename(s)[:-4] + ".o") for s in sources]
     flags = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wextra", "-I" + HOST, "-I" + os.path.join(ROOT, "include")]
+    if full_types:
+        flags.append("-DEGEN_FULLTYPE")
+    target = LIBHOST_FULL if full_types else LIBHOST
 
     def compile_one(pair):
         src, obj = pair
@@ -77,9 +89,9 @@ def build_libhost(jobs=8, verbose=False):
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(compile_one, zip(sources, objs)))
-    _run([CXX, "-shared", "-fPIC", "-o", LIBHOST] + objs +
+    _run([CXX, "-shared", "-fPIC", "-o", target] + objs +
          ["-L" + PKG, "-ltcg", "-Wl,-rpath,$ORIGIN"])
-    return LIBHOST
+    return target
 
 
 NATIVE_PROGRAMS = {
@@ -109,7 +121,8 @@ def build_native_programs(verbose=False):
 
 def build_all(verbose=False):
     """Everything native in this package."""
-    return [build_libtcg(verbose=verbose), build_libhost(verbose=verbose)] + build_native_programs(verbose=verbose)
+    return [build_libtcg(verbose=verbose), build_libhost(verbose=verbose),
+            build_libhost(verbose=verbose, full_types=True)] + build_native_programs(verbose=verbose)
 
 
 def main():

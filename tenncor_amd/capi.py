@@ -14,8 +14,13 @@ _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "libtcg.so")
 
 RANK_CAP = 8
+# enum tcg_dtype (include/tcg.h); the codes after INT32 are the integer widths
+# of the reference's full type configuration (cfg/fulltype.yml:11-34)
 DOUBLE, FLOAT, INT32 = 1, 2, 3
-NP_OF = {DOUBLE: np.float64, FLOAT: np.float32, INT32: np.int32}
+INT8, UINT8, INT16, UINT16, UINT32, INT64, UINT64 = 4, 5, 6, 7, 8, 9, 10
+NP_OF = {DOUBLE: np.float64, FLOAT: np.float32, INT32: np.int32,
+         INT8: np.int8, UINT8: np.uint8, INT16: np.int16, UINT16: np.uint16,
+         UINT32: np.uint32, INT64: np.int64, UINT64: np.uint64}
 # include/tcg.h: the fixed device memory tcg_reduce_noalloc keeps its temporaries in
 REDUCE_NOALLOC_SCRATCH_BYTES = 8 << 20
 

@@ -24,11 +24,21 @@ namespace
 
 template <typename T> struct is_int { static constexpr bool value = false; };
 template <> struct is_int<int32_t> { static constexpr bool value = true; };
+template <> struct is_int<int8_t> { static constexpr bool value = true; };
+template <> struct is_int<uint8_t> { static constexpr bool value = true; };
+template <> struct is_int<int16_t> { static constexpr bool value = true; };
+template <> struct is_int<uint16_t> { static constexpr bool value = true; };
+template <> struct is_int<uint32_t> { static constexpr bool value = true; };
+template <> struct is_int<int64_t> { static constexpr bool value = true; };
+template <> struct is_int<uint64_t> { static constexpr bool value = true; };
+
+// integers wrap modulo 2^width: summed in 32 (64) unsigned bits and truncated
+template <typename T> using Wide = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
 
 template <typename T>
 __device__ __forceinline__ T mac (T acc, T x, T w)
 {
-	if constexpr (is_int<T>::value) { return (T) ((uint32_t) acc + (uint32_t) x * (uint32_t) w); }
+	if constexpr (is_int<T>::value) { return (T) ((Wide<T>) acc + (Wide<T>) x * (Wide<T>) w); }
 	else { return acc + x * w; }
 }
 
@@ -138,7 +148,7 @@ __global__ __launch_bounds__(CV_BLOCK) void conv_boxed_k (ConvPlan p,
 			if ((int) threadIdx.x < s)
 			{
 				T a = smem[threadIdx.x], b = smem[threadIdx.x + s];
-				if constexpr (is_int<T>::value) { smem[threadIdx.x] = (T) ((uint32_t) a + (uint32_t) b); }
+				if constexpr (is_int<T>::value) { smem[threadIdx.x] = (T) ((Wide<T>) a + (Wide<T>) b); }
 				else { smem[threadIdx.x] = a + b; }
 			}
 			__syncthreads();
@@ -689,7 +699,8 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	}
 	ConvGemmPlan gp;
 	const char* gemm_env = getenv("TCG_CONV_GEMM"); // "0": direct kernels only (the parity reference)
-	if (!(gemm_env && gemm_env[0] == '0') && conv_gemm_plan(p, gp))
+	// (the product route exists for the three default types)
+	if (!(gemm_env && gemm_env[0] == '0') && tcg_default_dtype(dtype) && conv_gemm_plan(p, gp))
 	{
 		// An image that is mostly padding (conv2d's image gradient pads the
 		// fastest dim from 1 to 2*C - 1) scatters its non-zero elements over
@@ -754,12 +765,12 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	TCG_REQUIRE(ctx, blocks < (1ull << 31) && p.nwin < (1ull << 32), "tcg_conv: %llu outputs are too many for one launch", (unsigned long long) p.nwin);
 	if (group)
 	{
-		TCG_DISPATCH_TYPE(ctx, dtype, (conv_boxed_k<T,true><<<(unsigned) blocks, CV_BLOCK, 0, ctx->stream>>>(
+		TCG_DISPATCH_ALL(ctx, dtype, (conv_boxed_k<T,true><<<(unsigned) blocks, CV_BLOCK, 0, ctx->stream>>>(
 			p, (const T*) img, (const T*) kernel, (T*) out)));
 	}
 	else
 	{
-		TCG_DISPATCH_TYPE(ctx, dtype, (conv_boxed_k<T,false><<<(unsigned) blocks, CV_BLOCK, 0, ctx->stream>>>(
+		TCG_DISPATCH_ALL(ctx, dtype, (conv_boxed_k<T,false><<<(unsigned) blocks, CV_BLOCK, 0, ctx->stream>>>(
 			p, (const T*) img, (const T*) kernel, (T*) out)));
 	}
 	TCG_LAUNCH_CHECK(ctx, "conv_boxed");

@@ -327,6 +327,13 @@ int cast_impl (tcg_ctx* ctx, int in_dtype, uint64_t n, const void* in, TO* out)
 		case TCG_DOUBLE: ew_cast_k<TO,double><<<grid, EW_BLOCK, 0, ctx->stream>>>((const double*) in, out, n); break;
 		case TCG_FLOAT: ew_cast_k<TO,float><<<grid, EW_BLOCK, 0, ctx->stream>>>((const float*) in, out, n); break;
 		case TCG_INT32: ew_cast_k<TO,int32_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const int32_t*) in, out, n); break;
+		case TCG_INT8: ew_cast_k<TO,int8_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const int8_t*) in, out, n); break;
+		case TCG_UINT8: ew_cast_k<TO,uint8_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const uint8_t*) in, out, n); break;
+		case TCG_INT16: ew_cast_k<TO,int16_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const int16_t*) in, out, n); break;
+		case TCG_UINT16: ew_cast_k<TO,uint16_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const uint16_t*) in, out, n); break;
+		case TCG_UINT32: ew_cast_k<TO,uint32_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const uint32_t*) in, out, n); break;
+		case TCG_INT64: ew_cast_k<TO,int64_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const int64_t*) in, out, n); break;
+		case TCG_UINT64: ew_cast_k<TO,uint64_t><<<grid, EW_BLOCK, 0, ctx->stream>>>((const uint64_t*) in, out, n); break;
 		default: return tcg_fail(ctx, TCG_ERR_ARG, "tcg_cast: unknown input dtype %d", in_dtype);
 	}
 	TCG_LAUNCH_CHECK(ctx, "ew_cast");
@@ -337,10 +344,27 @@ int cast_impl (tcg_ctx* ctx, int in_dtype, uint64_t n, const void* in, TO* out)
 
 extern "C" {
 
-// While a sequence is recorded as one kernel, an elementwise node is a group of one
+// An elementwise node as a group of one (tcg_ew_fusedx): what such a node is
+// while a sequence is recorded as one kernel, and how the integer widths of
+// the full type set run (the streaming kernels of this file are built for
+// double, float and int32; a group is compiled for its dtype at run time)
 static int small_elementwise (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
 	const void* const* ins, void* out)
 {
+	if (nargs > TCG_FX_MAX_LEAVES && false == tcg_small_mode(ctx))
+	{
+		// a long fold: sixteen operands, then the result so far with fifteen more, ...
+		int rc = small_elementwise(ctx, opcode, dtype, n, TCG_FX_MAX_LEAVES, ins, out);
+		for (int done = TCG_FX_MAX_LEAVES; done < nargs && rc == TCG_OK;)
+		{
+			const void* next[TCG_FX_MAX_LEAVES] = {out};
+			int take = nargs - done < TCG_FX_MAX_LEAVES - 1 ? nargs - done : TCG_FX_MAX_LEAVES - 1;
+			for (int k = 0; k < take; ++k) { next[1 + k] = ins[done + k]; }
+			rc = small_elementwise(ctx, opcode, dtype, n, take + 1, next, out);
+			done += take;
+		}
+		return rc;
+	}
 	if (nargs > TCG_FX_MAX_LEAVES) { return tcg_small_unsupported(ctx, "an elementwise node with that many operands"); }
 	uint64_t shape[8] = {n, 1, 1, 1, 1, 1, 1, 1};
 	tcg_fx_leaf leaves[TCG_FX_MAX_LEAVES];
@@ -386,7 +410,7 @@ int tcg_ew_unary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, const void* i
 	TCG_REQUIRE(ctx, is_unary_op(opcode), "tcg_ew_unary: opcode %d is not a unary elementwise op", opcode);
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, in && out, "tcg_ew_unary: NULL pointer");
-	if (tcg_small_mode(ctx)) { return small_elementwise(ctx, opcode, dtype, n, 1, &in, out); }
+	if (tcg_small_mode(ctx) || false == tcg_default_dtype(dtype)) { return small_elementwise(ctx, opcode, dtype, n, 1, &in, out); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return unary_impl<T>(ctx, opcode, n, (const T*) in, (T*) out));
 	return TCG_OK;
 }
@@ -398,7 +422,7 @@ int tcg_ew_binary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n,
 	TCG_REQUIRE(ctx, is_binary_op(opcode), "tcg_ew_binary: opcode %d is not a binary elementwise op", opcode);
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, a && b && out, "tcg_ew_binary: NULL pointer");
-	if (tcg_small_mode(ctx))
+	if (tcg_small_mode(ctx) || false == tcg_default_dtype(dtype))
 	{
 		const void* ins[2] = {a, b};
 		return small_elementwise(ctx, opcode, dtype, n, 2, ins, out);
@@ -416,7 +440,7 @@ int tcg_ew_nary (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
 	if (n == 0) { return TCG_OK; }
 	for (int i = 0; i < nargs; ++i) { TCG_REQUIRE(ctx, ins[i], "tcg_ew_nary: operand %d is NULL", i); }
 	TCG_REQUIRE(ctx, out, "tcg_ew_nary: NULL output");
-	if (tcg_small_mode(ctx)) { return small_elementwise(ctx, opcode, dtype, n, nargs, ins, out); }
+	if (tcg_small_mode(ctx) || false == tcg_default_dtype(dtype)) { return small_elementwise(ctx, opcode, dtype, n, nargs, ins, out); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return nary_impl<T>(ctx, opcode, n, nargs, ins, (T*) out));
 	return TCG_OK;
 }
@@ -427,7 +451,7 @@ int tcg_ew_select (tcg_ctx* ctx, int dtype, uint64_t n, const void* cond,
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, cond && then && otherwise && out, "tcg_ew_select: NULL pointer");
-	if (tcg_small_mode(ctx))
+	if (tcg_small_mode(ctx) || false == tcg_default_dtype(dtype))
 	{
 		const void* ins[3] = {cond, then, otherwise};
 		return small_elementwise(ctx, TCG_SELECT, dtype, n, 3, ins, out);
@@ -444,7 +468,7 @@ int tcg_cast (tcg_ctx* ctx, int out_dtype, int in_dtype, uint64_t n, const void*
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, in && out, "tcg_cast: NULL pointer");
-	TCG_DISPATCH_TYPE(ctx, out_dtype, return cast_impl<T>(ctx, in_dtype, n, in, (T*) out));
+	TCG_DISPATCH_ALL(ctx, out_dtype, return cast_impl<T>(ctx, in_dtype, n, in, (T*) out));
 	return TCG_OK;
 }
 
@@ -454,7 +478,7 @@ int tcg_assign (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, void* target, c
 	TCG_REQUIRE(ctx, opcode >= TCG_ASSIGN && opcode <= TCG_ASSIGN_DIV, "tcg_assign: opcode %d is not an ASSIGN op", opcode);
 	if (n == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, target && source, "tcg_assign: NULL pointer");
-	if (tcg_small_mode(ctx))
+	if (tcg_small_mode(ctx) || false == tcg_default_dtype(dtype))
 	{
 		if (opcode == TCG_ASSIGN) { return small_elementwise(ctx, TCG_ASSIGN, dtype, n, 1, &source, target); }
 		const int fold[] = {TCG_ADD, TCG_SUB, TCG_MUL, TCG_DIV};

@@ -352,7 +352,8 @@ bool fx_jit_enabled (void)
 // typedefs, opcode names, the scalar routines and the argument structs
 void fx_emit_prelude (std::ostringstream& o)
 {
-	o << "typedef signed char int8_t; typedef unsigned char uint8_t; typedef int int32_t;\n"
+	o << "typedef signed char int8_t; typedef unsigned char uint8_t; typedef short int16_t;\n"
+		"typedef unsigned short uint16_t; typedef int int32_t;\n"
 		"typedef unsigned int uint32_t; typedef long int64_t; typedef unsigned long uint64_t;\n"
 		"#ifndef INT32_MIN\n#define INT32_MIN (-2147483647 - 1)\n#endif\n"
 		"#define FX_MAXD " << FX_MAXD << "\n"
@@ -562,7 +563,19 @@ void fx_emit_body (std::ostringstream& o, int N, const FxArgs& p, const bool* de
 
 const char* fx_type_name (int dtype)
 {
-	return dtype == TCG_DOUBLE ? "double" : dtype == TCG_FLOAT ? "float" : "int";
+	switch (dtype)
+	{
+		case TCG_DOUBLE: return "double";
+		case TCG_FLOAT: return "float";
+		case TCG_INT32: return "int32_t";
+		case TCG_INT8: return "int8_t";
+		case TCG_UINT8: return "uint8_t";
+		case TCG_INT16: return "int16_t";
+		case TCG_UINT16: return "uint16_t";
+		case TCG_UINT32: return "uint32_t";
+		case TCG_INT64: return "int64_t";
+		default: return "uint64_t";
+	}
 }
 
 // `unroll` indices per lane and iteration, their loads issued together in
@@ -776,7 +789,7 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 	fx_emit_prelude(o);
 	o << "struct PassPtrs { void* p[" << std::max<size_t>(1, nptrs) << "]; char feed[" << std::max<size_t>(16, feed_bytes) << "]; };\n"
 		"template <typename T> __device__ __forceinline__ T pass_mac (T a, T b, T acc)\n{\n"
-		"if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b + (uint32_t) acc); }\n"
+		"if constexpr (is_int<T>::value) { typedef typename wide_unsigned<T>::type W; return (T) ((W) a * (W) b + (W) acc); }\n"
 		"else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, acc); }\n"
 		"else { return __builtin_fma(a, b, acc); }\n}\n"
 		"extern \"C\" __global__ __launch_bounds__(" << PASS_BLOCK << ") void fx (PassPtrs P)\n{\n";
@@ -1265,7 +1278,7 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		if (L.boxed) { vec = vec && L.lo[0] % N == 0 && L.hi[0] % N == 0; }
 	}
 	if (tcg_small_mode(ctx)) { return small_append_fx(ctx, dtype, p); }
-	if (fx_jit_enabled()) { return fusedx_jit_launch(ctx, dtype, p, vec); }
-	TCG_DISPATCH_TYPE(ctx, dtype, return fusedx_launch<T>(ctx, p, vec));
+	if (fx_jit_enabled() || false == tcg_default_dtype(dtype)) { return fusedx_jit_launch(ctx, dtype, p, vec); }
+	TCG_DISPATCH_TYPE(ctx, dtype, return fusedx_launch<T>(ctx, p, vec)); // the interpreter: double, float, int32
 	return TCG_OK;
 }

@@ -5,6 +5,8 @@
 // 16-byte aligned go to the MFMA kernel (gemm_mfma.hip), such fp64 problems to
 // gemm_mfma_f64.hip; everything else (int32, odd strides, small problems) runs
 // the LDS-tiled kernel below.
+#include <type_traits>
+
 #include "tcg_internal.hpp"
 
 int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_t batch,
@@ -22,11 +24,21 @@ namespace
 
 template <typename T> struct is_int { static constexpr bool value = false; };
 template <> struct is_int<int32_t> { static constexpr bool value = true; };
+template <> struct is_int<int8_t> { static constexpr bool value = true; };
+template <> struct is_int<uint8_t> { static constexpr bool value = true; };
+template <> struct is_int<int16_t> { static constexpr bool value = true; };
+template <> struct is_int<uint16_t> { static constexpr bool value = true; };
+template <> struct is_int<uint32_t> { static constexpr bool value = true; };
+template <> struct is_int<int64_t> { static constexpr bool value = true; };
+template <> struct is_int<uint64_t> { static constexpr bool value = true; };
+
+// integers wrap modulo 2^width: summed in 32 (64) unsigned bits and truncated
+template <typename T> using Wide = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
 
 template <typename T>
 __device__ __forceinline__ T fma_wrap (T a, T b, T c)
 {
-	if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b + (uint32_t) c); }
+	if constexpr (is_int<T>::value) { return (T) ((Wide<T>) a * (Wide<T>) b + (Wide<T>) c); }
 	else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, c); }
 	else { return __builtin_fma(a, b, c); }
 }
@@ -228,7 +240,7 @@ int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 			(const double*) B, ldb, stride_b, trans_b, (double*) C, ldc, stride_c, &handled);
 		if (rc != TCG_OK || handled) { return rc; }
 	}
-	TCG_DISPATCH_TYPE(ctx, dtype, return gemm_generic<T>(ctx, M, N, K, batch,
+	TCG_DISPATCH_ALL(ctx, dtype, return gemm_generic<T>(ctx, M, N, K, batch,
 		(const T*) A, lda, stride_a, trans_a, (const T*) B, ldb, stride_b, trans_b, (T*) C, ldc, stride_c));
 	return TCG_OK;
 }

@@ -321,7 +321,9 @@ int run_plan (tcg_ctx* ctx, CopyPlan& p, const T* src, T* dst, const char* what)
 			hi[d] = p.box ? p.hi[d] : p.size[d];
 		}
 		if (false == dense_dst) { return tcg_small_unsupported(ctx, "a copy into a strided destination"); }
-		int dtype = std::is_same<T,double>::value ? TCG_DOUBLE : std::is_same<T,float>::value ? TCG_FLOAT : TCG_INT32;
+		// a copy: any dtype of this element size will do
+		int dtype = std::is_same<T,double>::value ? TCG_DOUBLE : std::is_same<T,float>::value ? TCG_FLOAT :
+			sizeof(T) == 4 ? TCG_INT32 : sizeof(T) == 2 ? TCG_UINT16 : TCG_UINT8;
 		return tcg_small_copy(ctx, dtype, p.nd, size, p.sstride, p.sbase, lo, hi, src, dst);
 	}
 	constexpr int N = Vec16<T>::N;
@@ -345,6 +347,8 @@ int run_plan (tcg_ctx* ctx, CopyPlan& p, const T* src, T* dst, const char* what)
 				wide = (d == j || p.sstride[d] % N == 0) && (d == 0 || p.dstride[d] % N == 0);
 			}
 			bool launched = false;
+			if constexpr (sizeof(T) >= 4)
+			{
 			if (wide)
 			{
 				// what no cache holds streams through large tiles
@@ -352,6 +356,7 @@ int run_plan (tcg_ctx* ctx, CopyPlan& p, const T* src, T* dst, const char* what)
 				bool large = p.total * sizeof(T) >= ((uint64_t) 128 << 20) && p.size[0] >= BIG && p.size[j] >= BIG;
 				if (large) { launch_transpose_vec<T,BIG,true>(ctx, p, j, batch, src, dst, &launched); }
 				else { launch_transpose_vec<T,32,false>(ctx, p, j, batch, src, dst, &launched); }
+			}
 			}
 			if (false == launched)
 			{
@@ -431,7 +436,7 @@ int tcg_extend (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	contiguous_strides(oshape, os);
 	CopyPlan p;
 	plan_finish(p, oshape, ss, os, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_extend"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_extend"));
 	return TCG_OK;
 }
 
@@ -455,7 +460,7 @@ int tcg_permute (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	contiguous_strides(oshape, os);
 	CopyPlan p;
 	plan_finish(p, oshape, ss, os, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_permute"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_permute"));
 	return TCG_OK;
 }
 
@@ -477,7 +482,7 @@ int tcg_slice (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	}
 	contiguous_strides(extents, os);
 	plan_finish(p, extents, is, os, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_slice"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_slice"));
 	return TCG_OK;
 }
 
@@ -502,7 +507,7 @@ int tcg_pad (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	CHECK_DIMS(ctx, oshape, "tcg_pad");
 	contiguous_strides(oshape, os);
 	plan_finish(p, oshape, is, os, lo, hi);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_pad"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_pad"));
 	return TCG_OK;
 }
 
@@ -521,7 +526,7 @@ int tcg_pad_interior (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	CopyPlan p;
 	for (int d = 0; d < 8; ++d) { p.dbase += (int64_t) before[d] * os[d]; }
 	plan_finish(p, inshape, is, os, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_pad_interior"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_pad_interior"));
 	return TCG_OK;
 }
 
@@ -545,7 +550,7 @@ int tcg_reverse (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		else { ss[d] = is[d]; }
 	}
 	plan_finish(p, shape, ss, is, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_reverse"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_reverse"));
 	return TCG_OK;
 }
 
@@ -568,7 +573,7 @@ int tcg_stride (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	}
 	CopyPlan p;
 	plan_finish(p, outshape, ss, os, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_stride"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_stride"));
 	return TCG_OK;
 }
 
@@ -595,7 +600,7 @@ int tcg_scatter (tcg_ctx* ctx, int dtype, const uint64_t inshape[8],
 	if (rc != TCG_OK) { return rc; }
 	CopyPlan p;
 	plan_finish(p, iter, is, ds, nullptr, nullptr);
-	TCG_DISPATCH_TYPE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_scatter"));
+	TCG_DISPATCH_MOVE(ctx, dtype, return run_plan<T>(ctx, p, (const T*) in, (T*) out, "tcg_scatter"));
 	return TCG_OK;
 }
 
@@ -632,7 +637,7 @@ int tcg_concat (tcg_ctx* ctx, int dtype, int axis, int nargs,
 		CopyPlan p;
 		p.dbase = (int64_t) off * os[axis];
 		plan_finish(p, ishape, is, os, nullptr, nullptr);
-		TCG_DISPATCH_TYPE(ctx, dtype,
+		TCG_DISPATCH_MOVE(ctx, dtype,
 			int rc = run_plan<T>(ctx, p, (const T*) ins[i], (T*) out, "tcg_concat");
 			if (rc != TCG_OK) { return rc; });
 		off += ishape[axis];

@@ -10,6 +10,8 @@
 // real types uniform on [lo, hi), int32 uniform on the inclusive range.
 #include "tcg_internal.hpp"
 
+#include <type_traits>
+
 namespace
 {
 
@@ -39,9 +41,8 @@ __device__ __forceinline__ Philox4 philox4x32_10 (uint64_t counter, uint64_t key
 	return Philox4{{c0, c1, c2, c3}};
 }
 
-// one generator block per 4 elements (float, int32) or 2 elements (double)
-template <typename T> struct PerBlock { static constexpr int N = 4; };
-template <> struct PerBlock<double> { static constexpr int N = 2; };
+// one generator block per 4 elements, or 2 elements of 8 bytes
+template <typename T> struct PerBlock { static constexpr int N = sizeof(T) == 8 ? 2 : 4; };
 
 __device__ __forceinline__ float draw (const Philox4& r, int k, float lo, float hi)
 {
@@ -56,11 +57,25 @@ __device__ __forceinline__ double draw (const Philox4& r, int k, double lo, doub
 	return fma(u, hi - lo, lo);
 }
 
-__device__ __forceinline__ int32_t draw (const Philox4& r, int k, int32_t lo, int32_t hi)
+// integers of at most 32 bits: lo + floor(r * (hi - lo + 1) / 2^32)
+template <typename T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) <= 4, int>::type = 0>
+__device__ __forceinline__ T draw (const Philox4& r, int k, T lo, T hi)
 {
 	if (hi < lo) { return lo; }
 	uint64_t range = (uint64_t) ((int64_t) hi - (int64_t) lo) + 1;
-	return (int32_t) ((int64_t) lo + (int64_t) (((uint64_t) r.v[k] * range) >> 32));
+	return (T) ((int64_t) lo + (int64_t) (((uint64_t) r.v[k] * range) >> 32));
+}
+
+// 64-bit integers: two words per draw, lo + floor(r * (hi - lo + 1) / 2^64);
+// the full range (hi - lo + 1 wraps to 0) takes the 64 bits as they are
+template <typename T, typename std::enable_if<std::is_integral<T>::value && sizeof(T) == 8, int>::type = 0>
+__device__ __forceinline__ T draw (const Philox4& r, int k, T lo, T hi)
+{
+	if (hi < lo) { return lo; }
+	uint64_t bits = ((uint64_t) r.v[2 * k + 1] << 32) | r.v[2 * k];
+	uint64_t range = (uint64_t) hi - (uint64_t) lo + 1;
+	uint64_t off = range == 0 ? bits : __umul64hi(bits, range);
+	return (T) ((uint64_t) lo + off);
 }
 
 template <typename T>
@@ -140,6 +155,13 @@ int tcg_rand_uniform (tcg_ctx* ctx, int dtype, uint64_t n, const void* lo, const
 		case TCG_DOUBLE: return launch<double>(ctx, n, lo, hi, out);
 		case TCG_FLOAT: return launch<float>(ctx, n, lo, hi, out);
 		case TCG_INT32: return launch<int32_t>(ctx, n, lo, hi, out);
+		case TCG_INT8: return launch<int8_t>(ctx, n, lo, hi, out);
+		case TCG_UINT8: return launch<uint8_t>(ctx, n, lo, hi, out);
+		case TCG_INT16: return launch<int16_t>(ctx, n, lo, hi, out);
+		case TCG_UINT16: return launch<uint16_t>(ctx, n, lo, hi, out);
+		case TCG_UINT32: return launch<uint32_t>(ctx, n, lo, hi, out);
+		case TCG_INT64: return launch<int64_t>(ctx, n, lo, hi, out);
+		case TCG_UINT64: return launch<uint64_t>(ctx, n, lo, hi, out);
 		default: return tcg_fail(ctx, TCG_ERR_ARG, "tcg_rand_uniform: unknown dtype %d", dtype);
 	}
 }

@@ -14,6 +14,7 @@
 #include "tcg_internal.hpp"
 
 #include <limits>
+#include <type_traits>
 
 // Device memory that exists for as long as the library is loaded, one copy on
 // every GPU: the temporaries of tcg_reduce_noalloc.  Host code never uses the
@@ -28,8 +29,9 @@ static unsigned char* g_scratch[MAX_DEVICES] = {nullptr};
 namespace
 {
 
-template <typename T> struct is_int { static constexpr bool value = false; };
-template <> struct is_int<int32_t> { static constexpr bool value = true; };
+template <typename T> struct is_int { static constexpr bool value = std::is_integral<T>::value; };
+
+template <typename T> using Wide = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
 
 template <typename T, int OP>
 struct Red
@@ -40,12 +42,12 @@ struct Red
 		else if constexpr (OP == TCG_REDUCE_PROD) { return (T) 1; }
 		else if constexpr (OP == TCG_REDUCE_MIN)
 		{
-			if constexpr (is_int<T>::value) { return INT32_MAX; }
+			if constexpr (is_int<T>::value) { return std::numeric_limits<T>::max(); }
 			else { return (T) INFINITY; }
 		}
 		else
 		{
-			if constexpr (is_int<T>::value) { return INT32_MIN; }
+			if constexpr (is_int<T>::value) { return std::numeric_limits<T>::lowest(); }
 			else { return (T) -INFINITY; }
 		}
 	}
@@ -54,12 +56,13 @@ struct Red
 	{
 		if constexpr (OP == TCG_REDUCE_SUM)
 		{
-			if constexpr (is_int<T>::value) { return (T) ((uint32_t) a + (uint32_t) b); }
+			// integers wrap modulo 2^width
+			if constexpr (is_int<T>::value) { return (T) ((Wide<T>) a + (Wide<T>) b); }
 			else { return a + b; }
 		}
 		else if constexpr (OP == TCG_REDUCE_PROD)
 		{
-			if constexpr (is_int<T>::value) { return (T) ((uint32_t) a * (uint32_t) b); }
+			if constexpr (is_int<T>::value) { return (T) ((Wide<T>) a * (Wide<T>) b); }
 			else { return a * b; }
 		}
 		else if constexpr (OP == TCG_REDUCE_MIN) { return b < a ? b : a; }
@@ -70,7 +73,8 @@ struct Red
 template <typename T>
 __device__ __forceinline__ T shfl_xor_t (T v, int mask)
 {
-	if constexpr (sizeof(T) == 8)
+	if constexpr (sizeof(T) < 4) { return (T) __shfl_xor((int) v, mask, TCG_WAVE); }
+	else if constexpr (sizeof(T) == 8)
 	{
 		union { T t; int i[2]; } u;
 		u.t = v;
@@ -574,7 +578,7 @@ int reduce_impl (tcg_ctx* ctx, Scratch& mem, const uint64_t shape[8], unsigned m
 int reduce_any (tcg_ctx* ctx, Scratch& mem, int opcode, int dtype, const uint64_t shape[8],
 	unsigned rankmask, const void* in, void* out)
 {
-	TCG_DISPATCH_TYPE(ctx, dtype,
+	TCG_DISPATCH_ALL(ctx, dtype,
 		switch (opcode)
 		{
 			case TCG_REDUCE_SUM: return reduce_impl<T,TCG_REDUCE_SUM>(ctx, mem, shape, rankmask, (const T*) in, (T*) out);
@@ -650,7 +654,7 @@ int tcg_argmax (tcg_ctx* ctx, int dtype, const uint64_t shape[8], int return_dim
 		for (int d = return_dim + 1; d < 8; ++d) { B *= shape[d]; }
 	}
 	TCG_REQUIRE(ctx, A * B < (1ull << 31), "tcg_argmax: too many outputs for one launch");
-	TCG_DISPATCH_TYPE(ctx, dtype, (argmax_k<T><<<(unsigned) (A * B), RED_BLOCK, 0, ctx->stream>>>((const T*) in, (T*) out, A, R)));
+	TCG_DISPATCH_ALL(ctx, dtype, (argmax_k<T><<<(unsigned) (A * B), RED_BLOCK, 0, ctx->stream>>>((const T*) in, (T*) out, A, R)));
 	TCG_LAUNCH_CHECK(ctx, "argmax");
 	return TCG_OK;
 }

@@ -90,9 +90,10 @@ static inline size_t tcg_type_size (int dtype)
 {
 	switch (dtype)
 	{
-		case TCG_DOUBLE: return 8;
-		case TCG_FLOAT: return 4;
-		case TCG_INT32: return 4;
+		case TCG_DOUBLE: case TCG_INT64: case TCG_UINT64: return 8;
+		case TCG_FLOAT: case TCG_INT32: case TCG_UINT32: return 4;
+		case TCG_INT16: case TCG_UINT16: return 2;
+		case TCG_INT8: case TCG_UINT8: return 1;
 		default: return 0;
 	}
 }
@@ -189,6 +190,44 @@ static inline unsigned tcg_grid (const tcg_ctx* ctx, uint64_t work_items,
 		default: return tcg_fail(ctx, TCG_ERR_ARG, "unknown dtype %d", (int) (dtype));\
 	} } while (0)
 
+// The same over every dtype, the integer widths of the full type set included
+// (cfg/fulltype.yml:11-34): for the entry points whose kernels exist for all of
+// them (reductions, casts, products, convolutions).  The streaming elementwise
+// kernels are built for the three default types only; the other widths run as
+// groups compiled at run time (tcg_ew_fusedx).
+#define TCG_DISPATCH_ALL(ctx, dtype, ...) do {\
+	switch (dtype) {\
+		case TCG_DOUBLE: { using T = double; __VA_ARGS__; } break;\
+		case TCG_FLOAT: { using T = float; __VA_ARGS__; } break;\
+		case TCG_INT32: { using T = int32_t; __VA_ARGS__; } break;\
+		case TCG_INT8: { using T = int8_t; __VA_ARGS__; } break;\
+		case TCG_UINT8: { using T = uint8_t; __VA_ARGS__; } break;\
+		case TCG_INT16: { using T = int16_t; __VA_ARGS__; } break;\
+		case TCG_UINT16: { using T = uint16_t; __VA_ARGS__; } break;\
+		case TCG_UINT32: { using T = uint32_t; __VA_ARGS__; } break;\
+		case TCG_INT64: { using T = int64_t; __VA_ARGS__; } break;\
+		case TCG_UINT64: { using T = uint64_t; __VA_ARGS__; } break;\
+		default: return tcg_fail(ctx, TCG_ERR_ARG, "unknown dtype %d", (int) (dtype));\
+	} } while (0)
+
+// Data movement only looks at the element size: the integer widths of the
+// full type set share the kernels of a type of their size (bytes are copied,
+// never computed with; zero fill is all-zero bits for every type)
+#define TCG_DISPATCH_MOVE(ctx, dtype, ...) do {\
+	switch (dtype) {\
+		case TCG_DOUBLE: case TCG_INT64: case TCG_UINT64: { using T = double; __VA_ARGS__; } break;\
+		case TCG_FLOAT: { using T = float; __VA_ARGS__; } break;\
+		case TCG_INT32: case TCG_UINT32: { using T = int32_t; __VA_ARGS__; } break;\
+		case TCG_INT16: case TCG_UINT16: { using T = uint16_t; __VA_ARGS__; } break;\
+		case TCG_INT8: case TCG_UINT8: { using T = uint8_t; __VA_ARGS__; } break;\
+		default: return tcg_fail(ctx, TCG_ERR_ARG, "unknown dtype %d", (int) (dtype));\
+	} } while (0)
+
+static inline bool tcg_default_dtype (int dtype)
+{
+	return dtype == TCG_DOUBLE || dtype == TCG_FLOAT || dtype == TCG_INT32;
+}
+
 // 16-byte vector of T (compiler vector types: the non-temporal load/store
 // builtins take these, not the HIP float4 structs)
 typedef float tcg_f32x4 __attribute__((ext_vector_type(4)));
@@ -198,6 +237,20 @@ template <typename T> struct Vec16;
 template <> struct Vec16<float> { using type = tcg_f32x4; static constexpr int N = 4; };
 template <> struct Vec16<int32_t> { using type = tcg_i32x4; static constexpr int N = 4; };
 template <> struct Vec16<double> { using type = tcg_f64x2; static constexpr int N = 2; };
+typedef int8_t tcg_i8x16 __attribute__((ext_vector_type(16)));
+typedef uint8_t tcg_u8x16 __attribute__((ext_vector_type(16)));
+typedef int16_t tcg_i16x8 __attribute__((ext_vector_type(8)));
+typedef uint16_t tcg_u16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t tcg_u32x4 __attribute__((ext_vector_type(4)));
+typedef int64_t tcg_i64x2 __attribute__((ext_vector_type(2)));
+typedef uint64_t tcg_u64x2 __attribute__((ext_vector_type(2)));
+template <> struct Vec16<int8_t> { using type = tcg_i8x16; static constexpr int N = 16; };
+template <> struct Vec16<uint8_t> { using type = tcg_u8x16; static constexpr int N = 16; };
+template <> struct Vec16<int16_t> { using type = tcg_i16x8; static constexpr int N = 8; };
+template <> struct Vec16<uint16_t> { using type = tcg_u16x8; static constexpr int N = 8; };
+template <> struct Vec16<uint32_t> { using type = tcg_u32x4; static constexpr int N = 4; };
+template <> struct Vec16<int64_t> { using type = tcg_i64x2; static constexpr int N = 2; };
+template <> struct Vec16<uint64_t> { using type = tcg_u64x2; static constexpr int N = 2; };
 
 template <typename T>
 union VecU

@@ -16,7 +16,12 @@ import numpy as np
 from . import capi
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "libtenncor_host.so")
+# One type configuration per process, as in the reference (its ETEQ_CFG picks
+# cfg/mintype.yml or cfg/fulltype.yml when the sources are generated): set
+# TENNCOR_AMD_TYPES=full before the first use for the build that also knows
+# INT8, UINT8, INT16, UINT16, UINT32, INT64 and UINT64.
+FULL_TYPES = os.environ.get("TENNCOR_AMD_TYPES", "min") == "full"
+LIB_PATH = os.path.join(_PKG, "libtenncor_host_full.so" if FULL_TYPES else "libtenncor_host.so")
 
 OP = capi.OP
 DOUBLE, FLOAT, INT32 = capi.DOUBLE, capi.FLOAT, capi.INT32

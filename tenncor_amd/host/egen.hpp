@@ -49,8 +49,40 @@ inline bool is_idempotent (_GENERATED_OPCODE code)
 	}
 }
 
+// One X-macro row per element type: ENUM, C type, precision (the rank that
+// type promotion compares), dtype code of the device library (enum tcg_dtype).
+// The codes of the enum follow the key order of the type configuration
+// (tools/egen/plugins/dtypes.py:155-159), so the two configurations number
+// INT32 differently; the device library has one numbering for both.
+#ifdef EGEN_FULLTYPE
+/// cfg/fulltype.yml:1-34 (selected like the reference's ETEQ_CFG: define EGEN_FULLTYPE)
+#define EGEN_DTYPES(ROW)\
+	ROW(DOUBLE, double, 10, 1)\
+	ROW(FLOAT, float, 9, 2)\
+	ROW(INT8, int8_t, 1, 4)\
+	ROW(UINT8, uint8_t, 2, 5)\
+	ROW(INT16, int16_t, 3, 6)\
+	ROW(UINT16, uint16_t, 4, 7)\
+	ROW(INT32, int32_t, 5, 3)\
+	ROW(UINT32, uint32_t, 6, 8)\
+	ROW(INT64, int64_t, 7, 9)\
+	ROW(UINT64, uint64_t, 8, 10)
+#else
 /// cfg/mintype.yml:4-13
-enum _GENERATED_DTYPE { BAD_TYPE = 0, DOUBLE, FLOAT, INT32, _N_GENERATED_DTYPES };
+#define EGEN_DTYPES(ROW)\
+	ROW(DOUBLE, double, 3, 1)\
+	ROW(FLOAT, float, 2, 2)\
+	ROW(INT32, int32_t, 1, 3)
+#endif
+
+enum _GENERATED_DTYPE
+{
+	BAD_TYPE = 0,
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) ENUM,
+	EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
+	_N_GENERATED_DTYPES
+};
 
 const _GENERATED_DTYPE default_dtype = FLOAT;
 
@@ -61,29 +93,43 @@ inline uint8_t type_size (_GENERATED_DTYPE type)
 {
 	switch (type)
 	{
-		case DOUBLE: return 8;
-		case FLOAT: return 4;
-		case INT32: return 4;
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) case ENUM: return sizeof(CTYPE);
+		EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
 		default: global::fatal("cannot get size of bad type");
 	}
 }
 
-/// cfg/mintype.yml: DOUBLE 3, FLOAT 2, INT32 1
+/// The `precision` of the type configuration: the larger wins a promotion
 inline size_t type_precision (_GENERATED_DTYPE type)
 {
 	switch (type)
 	{
-		case DOUBLE: return 3;
-		case FLOAT: return 2;
-		case INT32: return 1;
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) case ENUM: return PRECISION;
+		EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
+		default: return 0;
+	}
+}
+
+/// The code the device library (include/tcg.h, enum tcg_dtype) knows the type by
+inline int device_type (_GENERATED_DTYPE type)
+{
+	switch (type)
+	{
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) case ENUM: return DEVICE;
+		EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
 		default: return 0;
 	}
 }
 
 template <typename T> _GENERATED_DTYPE get_type (void) { return BAD_TYPE; }
-template <> inline _GENERATED_DTYPE get_type<double> (void) { return DOUBLE; }
-template <> inline _GENERATED_DTYPE get_type<float> (void) { return FLOAT; }
-template <> inline _GENERATED_DTYPE get_type<int32_t> (void) { return INT32; }
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) template <> inline _GENERATED_DTYPE get_type<CTYPE> (void) { return ENUM; }
+EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
+
+template <typename T> int device_type (void) { return device_type(get_type<T>()); }
 
 /// static_cast of n elements from `intype` into T
 template <typename T>
@@ -91,9 +137,9 @@ void type_convert (T* out, const void* input, _GENERATED_DTYPE intype, size_t n)
 {
 	switch (intype)
 	{
-		case DOUBLE: for (size_t i = 0; i < n; ++i) { out[i] = (T) ((const double*) input)[i]; } break;
-		case FLOAT: for (size_t i = 0; i < n; ++i) { out[i] = (T) ((const float*) input)[i]; } break;
-		case INT32: for (size_t i = 0; i < n; ++i) { out[i] = (T) ((const int32_t*) input)[i]; } break;
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) case ENUM: for (size_t i = 0; i < n; ++i) { out[i] = (T) ((const CTYPE*) input)[i]; } break;
+		EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
 		default: global::fatalf("invalid input type %s", name_type(intype).c_str());
 	}
 }
@@ -102,10 +148,25 @@ void type_convert (T* out, const void* input, _GENERATED_DTYPE intype, size_t n)
 
 // Runs `MACRO(T)` with the C++ type of a dtype code (TYPE_LOOKUP of the
 // generated dtype.hpp)
+#ifdef EGEN_FULLTYPE
+#define TYPE_LOOKUP(MACRO, DTYPE) switch (DTYPE) {\
+	case egen::DOUBLE: MACRO(double) break;\
+	case egen::FLOAT: MACRO(float) break;\
+	case egen::INT8: MACRO(int8_t) break;\
+	case egen::UINT8: MACRO(uint8_t) break;\
+	case egen::INT16: MACRO(int16_t) break;\
+	case egen::UINT16: MACRO(uint16_t) break;\
+	case egen::INT32: MACRO(int32_t) break;\
+	case egen::UINT32: MACRO(uint32_t) break;\
+	case egen::INT64: MACRO(int64_t) break;\
+	case egen::UINT64: MACRO(uint64_t) break;\
+	default: global::fatal("executing bad type"); }
+#else
 #define TYPE_LOOKUP(MACRO, DTYPE) switch (DTYPE) {\
 	case egen::DOUBLE: MACRO(double) break;\
 	case egen::FLOAT: MACRO(float) break;\
 	case egen::INT32: MACRO(int32_t) break;\
 	default: global::fatal("executing bad type"); }
+#endif
 
 #endif // TCH_EGEN_HPP

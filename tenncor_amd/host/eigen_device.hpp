@@ -637,7 +637,7 @@ struct TensAssign final : public iRefEigen
 		const void* src = eigen_ref(*arg_).device_data();
 		if (nullptr == src) { global::fatalf("operand %s has no data", arg_->to_string().c_str()); }
 		void* dst = static_cast<SrcRef<T>&>(ref_->device()).device_data_mut();
-		hip_check(tcg_assign(hip_context(), opcode_, egen::get_type<T>(), ref_->shape().n_elems(), dst, src));
+		hip_check(tcg_assign(hip_context(), opcode_, egen::device_type<T>(), ref_->shape().n_elems(), dst, src));
 	}
 	void replayed (void) override
 	{

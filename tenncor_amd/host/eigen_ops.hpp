@@ -40,7 +40,7 @@ EigenptrT unary (int opcode, teq::Shape outshape, const teq::iTensor& in)
 	uint64_t n = outshape.n_elems();
 	return make_op<T>(outshape, {&in}, [opcode, n](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_ew_unary(ctx, opcode, egen::get_type<T>(), n, args[0], out));
+		hip_check(tcg_ew_unary(ctx, opcode, egen::device_type<T>(), n, args[0], out));
 	});
 }
 
@@ -50,7 +50,7 @@ EigenptrT binary (int opcode, teq::Shape outshape, const teq::iTensor& a, const 
 	uint64_t n = outshape.n_elems();
 	return make_op<T>(outshape, {&a, &b}, [opcode, n](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_ew_binary(ctx, opcode, egen::get_type<T>(), n, args[0], args[1], out));
+		hip_check(tcg_ew_binary(ctx, opcode, egen::device_type<T>(), n, args[0], args[1], out));
 	});
 }
 
@@ -65,11 +65,11 @@ EigenptrT nnary (int opcode, teq::Shape outshape, const teq::TensptrsT& group)
 	{
 		if (args.size() == 2)
 		{
-			hip_check(tcg_ew_binary(ctx, opcode, egen::get_type<T>(), n, args[0], args[1], out));
+			hip_check(tcg_ew_binary(ctx, opcode, egen::device_type<T>(), n, args[0], args[1], out));
 		}
 		else
 		{
-			hip_check(tcg_ew_nary(ctx, opcode, egen::get_type<T>(), n, (int) args.size(), args.data(), out));
+			hip_check(tcg_ew_nary(ctx, opcode, egen::device_type<T>(), n, (int) args.size(), args.data(), out));
 		}
 	});
 }
@@ -104,7 +104,7 @@ EigenptrT select (teq::Shape outshape, const teq::iTensor& condition,
 	return make_op<T>(outshape, {&condition, &then, &otherwise},
 	[n](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_ew_select(ctx, egen::get_type<T>(), n, args[0], args[1], args[2], out));
+		hip_check(tcg_ew_select(ctx, egen::device_type<T>(), n, args[0], args[1], args[2], out));
 	});
 }
 
@@ -118,7 +118,7 @@ EigenptrT rand_uniform (teq::Shape outshape, const teq::iTensor& a, const teq::i
 		uint64_t n = outshape.n_elems();
 		return make_op<T>(outshape, {&a, &b}, [n](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 		{
-			hip_check(tcg_rand_uniform(ctx, egen::get_type<T>(), n, args[0], args[1], out));
+			hip_check(tcg_rand_uniform(ctx, egen::device_type<T>(), n, args[0], args[1], out));
 		});
 	}
 	return std::make_shared<HostOp<T>>(outshape, teq::CTensT{&a, &b},
@@ -129,13 +129,15 @@ EigenptrT rand_uniform (teq::Shape outshape, const teq::iTensor& a, const teq::i
 		const T* hi = (const T*) args[1];
 		for (size_t i = 0; i < n; ++i)
 		{
+			// drawn as int64_t / double whatever T is and narrowed afterwards
+			// (internal/global/random.hpp:87-98): the same engine gives the same stream
 			if constexpr (std::is_integral<T>::value)
 			{
-				out[i] = std::uniform_int_distribution<T>(lo[i], hi[i])(gen);
+				out[i] = (T) std::uniform_int_distribution<int64_t>((int64_t) lo[i], (int64_t) hi[i])(gen);
 			}
 			else
 			{
-				out[i] = std::uniform_real_distribution<T>(lo[i], hi[i])(gen);
+				out[i] = (T) std::uniform_real_distribution<double>((double) lo[i], (double) hi[i])(gen);
 			}
 		}
 	});
@@ -157,7 +159,7 @@ EigenptrT reduce (int opcode, teq::Shape outshape, const teq::iTensor& in, const
 	Shape8 inshape = shape8(in.shape());
 	return make_op<T>(outshape, {&in}, [opcode, mask, inshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_reduce(ctx, opcode, egen::get_type<T>(), inshape.data(), mask, args[0], out));
+		hip_check(tcg_reduce(ctx, opcode, egen::device_type<T>(), inshape.data(), mask, args[0], out));
 	});
 }
 
@@ -185,7 +187,7 @@ EigenptrT argmax (teq::Shape outshape, const teq::iTensor& in, const marsh::iAtt
 	Shape8 inshape = shape8(in.shape());
 	return make_op<T>(outshape, {&in}, [return_dim, inshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_argmax(ctx, egen::get_type<T>(), inshape.data(), (int) return_dim, args[0], out));
+		hip_check(tcg_argmax(ctx, egen::device_type<T>(), inshape.data(), (int) return_dim, args[0], out));
 	});
 }
 
@@ -203,7 +205,7 @@ EigenptrT extend (teq::Shape outshape, const teq::iTensor& in, const marsh::iAtt
 	Shape8 ishape = shape8(inshape);
 	return make_op<T>(outshape, {&in}, [bcast, ishape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_extend(ctx, egen::get_type<T>(), ishape.data(), bcast.data(), args[0], out));
+		hip_check(tcg_extend(ctx, egen::device_type<T>(), ishape.data(), bcast.data(), args[0], out));
 	});
 }
 
@@ -224,7 +226,7 @@ EigenptrT permute (teq::Shape outshape, const teq::iTensor& in, const marsh::iAt
 	Shape8 ishape = shape8(in.shape());
 	return make_op<T>(outshape, {&in}, [reorder, ishape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_permute(ctx, egen::get_type<T>(), ishape.data(), reorder.data(), args[0], out));
+		hip_check(tcg_permute(ctx, egen::device_type<T>(), ishape.data(), reorder.data(), args[0], out));
 	});
 }
 
@@ -256,7 +258,7 @@ EigenptrT slice (teq::Shape outshape, const teq::TensptrT& in, const marsh::iAtt
 	Shape8 ishape = shape8(shape);
 	return make_op<T>(outshape, {in.get()}, [offsets, extents, ishape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_slice(ctx, egen::get_type<T>(), ishape.data(), offsets.data(), extents.data(), args[0], out));
+		hip_check(tcg_slice(ctx, egen::device_type<T>(), ishape.data(), offsets.data(), extents.data(), args[0], out));
 	});
 }
 
@@ -297,10 +299,10 @@ EigenptrT pad (teq::Shape outshape, const teq::iTensor& in, const marsh::iAttrib
 		if (only_convolved(self))
 		{
 			launch_scope().partial = true;
-			hip_check(tcg_pad_interior(ctx, egen::get_type<T>(), ishape.data(), before.data(), after.data(), args[0], out));
+			hip_check(tcg_pad_interior(ctx, egen::device_type<T>(), ishape.data(), before.data(), after.data(), args[0], out));
 			return;
 		}
-		hip_check(tcg_pad(ctx, egen::get_type<T>(), ishape.data(), before.data(), after.data(), args[0], out));
+		hip_check(tcg_pad(ctx, egen::device_type<T>(), ishape.data(), before.data(), after.data(), args[0], out));
 	});
 }
 
@@ -315,7 +317,7 @@ EigenptrT stride (teq::Shape outshape, const teq::iTensor& in, const marsh::iAtt
 	Shape8 ishape = shape8(in.shape()), oshape = shape8(outshape);
 	return make_op<T>(outshape, {&in}, [incrs, ishape, oshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_stride(ctx, egen::get_type<T>(), ishape.data(), incrs.data(), oshape.data(), args[0], out));
+		hip_check(tcg_stride(ctx, egen::device_type<T>(), ishape.data(), incrs.data(), oshape.data(), args[0], out));
 	});
 }
 
@@ -330,7 +332,7 @@ EigenptrT scatter (teq::Shape outshape, const teq::iTensor& in, const marsh::iAt
 	Shape8 ishape = shape8(in.shape()), oshape = shape8(outshape);
 	return make_op<T>(outshape, {&in}, [incrs, ishape, oshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_scatter(ctx, egen::get_type<T>(), ishape.data(), incrs.data(), oshape.data(), args[0], out));
+		hip_check(tcg_scatter(ctx, egen::device_type<T>(), ishape.data(), incrs.data(), oshape.data(), args[0], out));
 	});
 }
 
@@ -347,7 +349,7 @@ EigenptrT reverse (teq::Shape outshape, const teq::iTensor& in, const marsh::iAt
 	Shape8 shape = shape8(outshape);
 	return make_op<T>(outshape, {&in}, [mask, shape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_reverse(ctx, egen::get_type<T>(), shape.data(), mask, args[0], out));
+		hip_check(tcg_reverse(ctx, egen::device_type<T>(), shape.data(), mask, args[0], out));
 	});
 }
 
@@ -367,7 +369,7 @@ EigenptrT concat (teq::Shape outshape, const teq::TensptrsT& group, const marsh:
 	}
 	return make_op<T>(outshape, args, [axis, shapes](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_concat(ctx, egen::get_type<T>(), (int) axis, (int) args.size(), shapes.data(), args.data(), out));
+		hip_check(tcg_concat(ctx, egen::device_type<T>(), (int) axis, (int) args.size(), shapes.data(), args.data(), out));
 	});
 }
 
@@ -394,7 +396,7 @@ EigenptrT contract (teq::Shape outshape, const teq::iTensor& a, const teq::iTens
 	Shape8 ashape = shape8(a.shape()), bshape = shape8(b.shape());
 	return make_op<T>(outshape, {&a, &b}, [pairs, ashape, bshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_contract(ctx, egen::get_type<T>(), ashape.data(), bshape.data(),
+		hip_check(tcg_contract(ctx, egen::device_type<T>(), ashape.data(), bshape.data(),
 			(int) (pairs.size() / 2), pairs.data(), args[0], args[1], out));
 	});
 }
@@ -405,7 +407,7 @@ EigenptrT matmul (teq::Shape outshape, const teq::iTensor& a, const teq::iTensor
 	Shape8 ashape = shape8(a.shape()), bshape = shape8(b.shape());
 	return make_op<T>(outshape, {&a, &b}, [ashape, bshape](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_matmul(ctx, egen::get_type<T>(), ashape.data(), bshape.data(), args[0], args[1], out));
+		hip_check(tcg_matmul(ctx, egen::device_type<T>(), ashape.data(), bshape.data(), args[0], args[1], out));
 	});
 }
 
@@ -513,7 +515,7 @@ EigenptrT convolution (teq::Shape outshape, const teq::iTensor& input,
 		Shape8 olo, ohi;
 		bool windowed = consumed_window(self, outshape, olo, ohi);
 		launch_scope().partial = windowed;
-		hip_check(tcg_conv_boxed(ctx, egen::get_type<T>(), ishape.data(), ks.data(), (int) ranks.size(),
+		hip_check(tcg_conv_boxed(ctx, egen::device_type<T>(), ishape.data(), ks.data(), (int) ranks.size(),
 			ranks.data(), ilo.data(), ihi.data(), windowed ? olo.data() : nullptr,
 			windowed ? ohi.data() : nullptr, args[0], args[1], out));
 	});
@@ -553,7 +555,7 @@ EigenptrT cast (const teq::TensptrT& input)
 	uint64_t n = input->shape().n_elems();
 	return make_op<T>(input->shape(), {input.get()}, [intype, n](tcg_ctx* ctx, T* out, const std::vector<const void*>& args)
 	{
-		hip_check(tcg_cast(ctx, egen::get_type<T>(), intype, n, args[0], out));
+		hip_check(tcg_cast(ctx, egen::device_type<T>(), egen::device_type(intype), n, args[0], out));
 	});
 }
 

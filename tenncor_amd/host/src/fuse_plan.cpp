@@ -1,6 +1,7 @@
 // Which functors of an evaluation pass share a launch (see fuse_plan.hpp).
 #include "fuse_plan.hpp"
 
+#include <type_traits>
 #include <algorithm>
 #include <functional>
 #include <map>
@@ -109,9 +110,14 @@ bool scalar_constant (const teq::iTensor* tens, double& value)
 	const void* data = leaf->device().data();
 	switch (leaf->get_meta().type_code())
 	{
-		case egen::DOUBLE: value = *(const double*) data; return true;
-		case egen::FLOAT: value = *(const float*) data; return true;
-		case egen::INT32: value = *(const int32_t*) data; return true;
+		// a double carries every value of a type of at most 32 bits; a 64-bit
+		// integer only below 2^53, beyond which the constant stays an operand
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) case egen::ENUM:\
+			value = (double) *(const CTYPE*) data;\
+			return sizeof(CTYPE) < 8 || std::is_floating_point<CTYPE>::value ||\
+				(value > -0x1p53 && value < 0x1p53);
+		EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
 		default: return false;
 	}
 }
@@ -1117,7 +1123,7 @@ void launch_contract (const SwappedContract& call, const teq::TensSetT& targets,
 	if (nullptr == a || nullptr == b) { global::fatal("operand of a matrix product has no data"); }
 	try
 	{
-		hip_check(tcg_contract(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
+		hip_check(tcg_contract(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), call.ashape.data(), call.bshape.data(),
 			(int) (call.pairs.size() / 2), call.pairs.data(), a, b, dst));
 	}
 	catch (...)
@@ -1144,7 +1150,7 @@ void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMe
 	}
 	try
 	{
-		hip_check(tcg_contract_sum(hip_context(), call.dtype, call.ashape.data(), call.bshape.data(),
+		hip_check(tcg_contract_sum(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), call.ashape.data(), call.bshape.data(),
 			(int) (call.pairs.size() / 2), call.pairs.data(), (int) a.size(), a.data(), b.data(), dst));
 	}
 	catch (...)
@@ -1168,7 +1174,7 @@ void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptr
 	if (call.windowed) { ref.mark_partial(); }
 	try
 	{
-		hip_check(tcg_conv_dense_box(hip_context(), call.dtype, call.imgshape.data(), call.kshape.data(),
+		hip_check(tcg_conv_dense_box(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), call.imgshape.data(), call.kshape.data(),
 			(int) call.ranks.size(), call.ranks.data(), call.ilo.data(), call.ihi.data(),
 			call.windowed ? call.olo.data() : nullptr, call.windowed ? call.ohi.data() : nullptr, image, kernel, dst));
 	}
@@ -1200,7 +1206,7 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 	}
 	try
 	{
-		hip_check(tcg_ew_fusedx(hip_context(), group.dtype, group.shape.data(), (int) leaves.size(), leaves.data(),
+		hip_check(tcg_ew_fusedx(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) group.dtype), group.shape.data(), (int) leaves.size(), leaves.data(),
 			(int) group.program.size(), group.program.data(), (int) outs.size(), outs.data()));
 	}
 	catch (...)

@@ -83,6 +83,17 @@ static void print_tree (std::ostringstream& out, const teq::TensptrT& node,
 	}
 }
 
+// The flat API numbers element types like the device library (enum tcg_dtype)
+// in every type configuration; the C++ layer numbers them like the
+// reference's generated enum, which differs between configurations
+static egen::_GENERATED_DTYPE host_dtype (int64_t wire)
+{
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) if (wire == DEVICE) { return egen::ENUM; }
+	EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
+	global::fatalf("element type %d is not part of this build's type configuration", (int) wire);
+}
+
 extern "C" {
 
 const char* tcr_last_error (void) { return g_error.c_str(); }
@@ -105,7 +116,7 @@ int tcr_variable (tcr_graph* g, int dtype, const uint64_t shape[8], const void* 
 		std::string lbl = label ? label : "";
 		teq::TensptrT out;
 #define TCH_VAR(T) out = eteq::make_variable<T>((const T*) data, s, lbl);
-		TYPE_LOOKUP(TCH_VAR, dtype)
+		TYPE_LOOKUP(TCH_VAR, host_dtype(dtype))
 #undef TCH_VAR
 		*node = g->add(out);
 	});
@@ -118,7 +129,7 @@ int tcr_constant (tcr_graph* g, int dtype, const uint64_t shape[8], const void* 
 		teq::Shape s = to_shape(shape);
 		teq::TensptrT out;
 #define TCH_CST(T) out = eteq::make_constant_tensor<T>((const T*) data, s);
-		TYPE_LOOKUP(TCH_CST, dtype)
+		TYPE_LOOKUP(TCH_CST, host_dtype(dtype))
 #undef TCH_CST
 		*node = g->add(out);
 	});
@@ -159,7 +170,7 @@ int tcr_functor (tcr_graph* g, int opcode, int nargs, const int* args, int nattr
 			else if (key == "dtype")
 			{
 				if (v.size() != 1) { global::fatal("`dtype` takes one value"); }
-				attrs.add_attr(key, std::make_unique<marsh::String>(egen::name_type((egen::_GENERATED_DTYPE) v[0])));
+				attrs.add_attr(key, std::make_unique<marsh::String>(egen::name_type(host_dtype(v[0]))));
 			}
 			else if (key == "tensor")
 			{
@@ -291,7 +302,7 @@ int tcr_shape (tcr_graph* g, int node, uint64_t shape[8])
 
 int tcr_dtype (tcr_graph* g, int node, int* dtype)
 {
-	return guarded([&] { *dtype = (int) g->at(node)->get_meta().type_code(); });
+	return guarded([&] { *dtype = egen::device_type((egen::_GENERATED_DTYPE) g->at(node)->get_meta().type_code()); });
 }
 
 int tcr_data (tcr_graph* g, int node, void* out, size_t bytes)

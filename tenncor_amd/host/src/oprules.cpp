@@ -34,18 +34,18 @@ std::string name_type (_GENERATED_DTYPE type)
 {
 	switch (type)
 	{
-		case DOUBLE: return "DOUBLE";
-		case FLOAT: return "FLOAT";
-		case INT32: return "INT32";
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) case ENUM: return #ENUM;
+		EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
 		default: return "BAD_TYPE";
 	}
 }
 
 _GENERATED_DTYPE get_type (const std::string& name)
 {
-	if (name == "DOUBLE") { return DOUBLE; }
-	if (name == "FLOAT") { return FLOAT; }
-	if (name == "INT32") { return INT32; }
+#define EGEN_ROW(ENUM, CTYPE, PRECISION, DEVICE) if (name == #ENUM) { return ENUM; }
+	EGEN_DTYPES(EGEN_ROW)
+#undef EGEN_ROW
 	return BAD_TYPE;
 }
 

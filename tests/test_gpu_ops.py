@@ -900,7 +900,7 @@ def test_errors_are_reported_not_thrown_across_the_abi(ctx, ops):
     with pytest.raises(capi.TcgError):
         ctx.ew_unary("ADD", capi.FLOAT, 12, a.ptr, a.ptr)
     with pytest.raises(capi.TcgError):
-        ctx.ew_unary("EXP", 9, 12, a.ptr, a.ptr)
+        ctx.ew_unary("EXP", 99, 12, a.ptr, a.ptr)  # no such element type
 
 
 def test_pool_recycles_blocks(ctx):
