@@ -438,6 +438,27 @@ int tcg_conv_dense_box (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const uint64_t img_lo[8], const uint64_t img_hi[8],
 	const uint64_t out_lo[8], const uint64_t out_hi[8],
 	const void* box, const void* kernel, void* out);
+/* The same correlation over operands and a result that are laid out in memory
+ * otherwise than densely in dim order: the PERMUTE and REVERSE nodes tenncor
+ * puts round every convolution (cfg/tenncor/nn.yml:88-93 reverses the kernel
+ * and permutes the result; tenncor/eteq/backprop.hpp:372-439 permutes the
+ * upstream gradient in front of the correlation and permutes and reverses the
+ * kernel gradient behind it) become strides instead of passes over memory.
+ * All strides count elements and may be negative (REVERSE):
+ *   image element c, img_lo <= c < img_hi:  box[sum_d (c[d] - img_lo[d]) * box_stride[d]]
+ *   kernel element w:                        kernel[sum_i w[i] * kernel_stride[i]]
+ *   output element c, out_lo <= c < out_hi:  out[sum_d (c[d] - out_lo[d]) * out_stride[d]]
+ * (NULL out_lo / out_hi: every output). Nothing else of `out` is written.
+ * Values are those of tcg_conv_boxed on the materialised operands; where the
+ * result or the kernel already is the row-major matrix of the product that
+ * the correlation is lowered to, the product writes or reads it in place. */
+int tcg_conv_views (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const uint64_t img_lo[8], const uint64_t img_hi[8],
+	const uint64_t out_lo[8], const uint64_t out_hi[8],
+	const void* box, const int64_t box_stride[8],
+	const void* kernel, const int64_t kernel_stride[8],
+	void* out, const int64_t out_stride[8]);
 
 #ifdef __cplusplus
 }

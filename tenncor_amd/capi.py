@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -87,6 +87,7 @@ def load():
     lib = ctypes.CDLL(LIB_PATH)
     vp, u64, i32, sz = ctypes.c_void_p, ctypes.c_uint64, ctypes.c_int, ctypes.c_size_t
     u64p, vpp = ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_void_p)
+    i64p = ctypes.POINTER(ctypes.c_int64)
     sig = {
         "tcg_ctx_create": [i32, ctypes.POINTER(vp)],
         "tcg_ctx_destroy": [vp],
@@ -134,6 +135,7 @@ def load():
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
+        "tcg_conv_views": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, i64p, vp, i64p, vp, i64p],
         "tcg_capture_begin": [vp],
         "tcg_capture_end": [vp, ctypes.POINTER(vp)],
         "tcg_capture_abort": [vp],
@@ -443,6 +445,19 @@ class Context:
         self._check(self.lib.tcg_conv_dense_box(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
                                                 len(r), _u64(r if r else [0]), _u64(img_box[0]), _u64(img_box[1]),
                                                 olo, ohi, box, kernel, dst))
+
+    def conv_views(self, dtype, imgshape, kshape, ranks, img_box, out_box, box, box_stride, kernel, kernel_stride,
+                   dst, out_stride):
+        """conv_dense_box over strided operands and a strided result: `box`,
+        `kernel` and `dst` are the addresses of image element img_box[0], of
+        kernel element 0 and of output element out_box[0]; strides count elements."""
+        r = [int(v) for v in ranks][:RANK_CAP]
+        olo, ohi = (_u64(out_box[0]), _u64(out_box[1])) if out_box else (None, None)
+        i64 = lambda vals: (ctypes.c_int64 * 8)(*[int(v) for v in vals])
+        self._check(self.lib.tcg_conv_views(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
+                                            len(r), _u64(r if r else [0]), _u64(img_box[0]), _u64(img_box[1]),
+                                            olo, ohi, box, i64(box_stride), kernel, i64(kernel_stride),
+                                            dst, i64(out_stride)))
 
     # ---- recorded launch sequences ----
     def capture_begin(self, small=False):

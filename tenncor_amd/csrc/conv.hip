@@ -16,6 +16,8 @@
 // an LDS tree at the end (few outputs, long sums: kernel gradients).
 #include "tcg_internal.hpp"
 
+#include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 #include <type_traits>
 
@@ -56,6 +58,7 @@ struct ConvPlan
 	int32_t ihi[8];
 	uint64_t nwin = 1;   // outputs in the window
 	int64_t ioff0 = 0;   // image offset of coordinate 0 (negative when `img` holds the box only)
+	int64_t ooff0 = 0;   // output offset of coordinate 0 (negative when `out` starts at the window)
 };
 
 constexpr int CV_BLOCK = 256;
@@ -67,7 +70,7 @@ __global__ __launch_bounds__(CV_BLOCK) void conv_boxed_k (ConvPlan p,
 	uint64_t o = GROUP_PER_OUTPUT ? (uint64_t) blockIdx.x : (uint64_t) blockIdx.x * CV_BLOCK + threadIdx.x;
 	if (o >= p.nwin) { return; }
 	// output coordinate, and per image dim the clipped kernel range [k0, k0 + kr)
-	int64_t ibase = p.ioff0, obase = 0, kbase = 0;
+	int64_t ibase = p.ioff0, obase = p.ooff0, kbase = 0;
 	uint32_t kr[8];
 	uint64_t nterms = 1;
 	uint32_t rem = (uint32_t) o; // the host keeps nwin below 2^32
@@ -219,6 +222,14 @@ struct ConvGemmPlan
 	int32_t check_dim[4];
 	uint32_t check_ext[4];
 	int32_t ncheck;     // -1: more than four, the general gather handles them
+	// The order in which the row / summed / column index decomposes into image
+	// dims, fastest first (each lists all eight dims; a dim of extent 1 is a
+	// no-op).  Any order gives the same product as long as A, B and C agree on
+	// it, so each index runs first along the dim that lies closest in memory:
+	// the summed index along the image, rows and columns along the result.
+	// Without tables (ncheck < 0) all three are the identity.
+	uint32_t mord[8], sord[8], nord[8];
+	uint32_t nflip[8];  // column dim counted from its last output coordinate down
 };
 
 // Per row / per summed index: image offset and, for the checked dims, the
@@ -274,18 +285,18 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_tables_k (ConvGemmPlan p, ConvT
 		ConvTabEntry e;
 		e.off = 0;
 		e.c[0] = e.c[1] = e.c[2] = e.c[3] = 0;
-#pragma unroll
-		for (int d = 0; d < 8; ++d)
+		for (int j = 0; j < 8; ++j)
 		{
+			const uint32_t d = p.mord[j];
 			uint32_t qm = conv_div(rm, p.mdiv[d]);
 			int32_t x = (int32_t) (rm - qm * p.msize[d]);
 			rm = qm;
 			int32_t c = p.is_col[d] ? p.ilo[d] : p.xlo[d] + x;
 			e.off += (int64_t) c * p.istr[d];
 #pragma unroll
-			for (int j = 0; j < 4; ++j)
+			for (int k = 0; k < 4; ++k)
 			{
-				if (p.check_dim[j] == d) { e.c[j] = c - p.ilo[d]; }
+				if (p.check_dim[k] == (int32_t) d) { e.c[k] = c - p.ilo[d]; }
 			}
 		}
 		rows[i] = e;
@@ -296,17 +307,17 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_tables_k (ConvGemmPlan p, ConvT
 		ConvTabEntry e;
 		e.off = 0;
 		e.c[0] = e.c[1] = e.c[2] = e.c[3] = 0;
-#pragma unroll
-		for (int d = 0; d < 8; ++d)
+		for (int j = 0; j < 8; ++j)
 		{
+			const uint32_t d = p.sord[j];
 			uint32_t qs = conv_div(rs, p.sdiv[d]);
 			int32_t w = (int32_t) (rs - qs * p.ssize[d]) + p.slo[d];
 			rs = qs;
 			e.off += (int64_t) w * p.istr[d];
 #pragma unroll
-			for (int j = 0; j < 4; ++j)
+			for (int k = 0; k < 4; ++k)
 			{
-				if (p.check_dim[j] == d) { e.c[j] = w; }
+				if (p.check_dim[k] == (int32_t) d) { e.c[k] = w; }
 			}
 		}
 		// padding columns of A: a coordinate no row can complete into the box
@@ -361,16 +372,27 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_k (ConvGemmPlan p
 			uint32_t rs = s, rn = n;
 			int64_t off = 0;
 			bool valid = true;
-#pragma unroll
-			for (int d = 0; d < 8; ++d)
+			// a dim is a column dim (its kernel index follows from the column)
+			// or it is not (its kernel index is the summed one): never both
+			for (int j = 0; j < 8; ++j)
 			{
+				const uint32_t d = p.sord[j];
 				uint32_t qs = conv_div(rs, p.sdiv[d]);
 				int32_t w = (int32_t) (rs - qs * p.ssize[d]) + p.slo[d];
 				rs = qs;
+				if (p.is_col[d]) { continue; }
+				valid = valid && w >= 0 && w < (int32_t) p.ksize[d];
+				off += (int64_t) w * p.kstr[d];
+			}
+			for (int j = 0; j < 8; ++j)
+			{
+				const uint32_t d = p.nord[j];
 				uint32_t qn = conv_div(rn, p.ndiv[d]);
-				int32_t x = (int32_t) (rn - qn * p.nsize[d]) + p.xlo[d];
+				uint32_t xq = rn - qn * p.nsize[d];
 				rn = qn;
-				if (p.is_col[d]) { w = p.ilo[d] - x; }
+				if (0 == p.is_col[d]) { continue; }
+				if (p.nflip[d]) { xq = p.nsize[d] - 1 - xq; }
+				int32_t w = p.ilo[d] - (p.xlo[d] + (int32_t) xq);
 				valid = valid && w >= 0 && w < (int32_t) p.ksize[d];
 				off += (int64_t) w * p.kstr[d];
 			}
@@ -393,16 +415,23 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_scatter_k (ConvGemmPlan p, uint
 		uint32_t n = (uint32_t) (i - (uint64_t) r * p.N);
 		uint32_t rm = m0 + r, rn = n;
 		int64_t off = 0;
-#pragma unroll
-		for (int d = 0; d < 8; ++d)
+		for (int j = 0; j < 8; ++j)
 		{
+			const uint32_t d = p.mord[j];
 			uint32_t qm = conv_div(rm, p.mdiv[d]);
 			int32_t xm = (int32_t) (rm - qm * p.msize[d]);
 			rm = qm;
+			if (0 == p.is_col[d]) { off += (int64_t) (p.oxlo[d] + xm) * p.ostr[d]; }
+		}
+		for (int j = 0; j < 8; ++j)
+		{
+			const uint32_t d = p.nord[j];
 			uint32_t qn = conv_div(rn, p.ndiv[d]);
-			int32_t xn = (int32_t) (rn - qn * p.nsize[d]);
+			uint32_t xq = rn - qn * p.nsize[d];
 			rn = qn;
-			off += (int64_t) (p.oxlo[d] + xm + xn) * p.ostr[d];
+			if (0 == p.is_col[d]) { continue; }
+			if (p.nflip[d]) { xq = p.nsize[d] - 1 - xq; }
+			off += (int64_t) (p.oxlo[d] + (int32_t) xq) * p.ostr[d];
 		}
 		out[off] = C[(uint64_t) r * p.Np + n];
 	}
@@ -447,6 +476,8 @@ bool conv_gemm_plan (const ConvPlan& c, ConvGemmPlan& g)
 		g.mdiv[d] = conv_make_div(g.msize[d]);
 		g.sdiv[d] = conv_make_div(g.ssize[d]);
 		g.ndiv[d] = conv_make_div(g.nsize[d]);
+		g.mord[d] = g.sord[d] = g.nord[d] = (uint32_t) d;
+		g.nflip[d] = 0;
 		M *= g.msize[d];
 		N *= g.nsize[d];
 		S *= g.ssize[d];
@@ -482,6 +513,111 @@ bool conv_gemm_plan (const ConvPlan& c, ConvGemmPlan& g)
 	return true;
 }
 
+// Orders of the three indices once the strides are final (see ConvGemmPlan)
+void conv_choose_orders (ConvGemmPlan& g)
+{
+	if (g.ncheck < 0) { return; } // the general gather decomposes in dim order
+	auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+	auto sorted = [&](uint32_t* ord, const uint32_t* extent, const int64_t* stride)
+	{
+		for (int d = 0; d < 8; ++d) { ord[d] = (uint32_t) d; }
+		std::stable_sort(ord, ord + 8, [&](uint32_t x, uint32_t y)
+		{
+			bool sx = extent[x] == 1, sy = extent[y] == 1;
+			if (sx != sy) { return sy; }
+			return false == sx && mag(stride[x]) < mag(stride[y]);
+		});
+	};
+	sorted(g.sord, g.ssize, g.istr);
+	sorted(g.mord, g.msize, g.ostr);
+	sorted(g.nord, g.nsize, g.ostr);
+	for (int d = 0; d < 8; ++d) { g.nflip[d] = g.is_col[d] && g.nsize[d] > 1 && g.ostr[d] < 0; }
+}
+
+// The product's C is the result itself when the result, restricted to the
+// window, is a row-major [rows][columns] matrix in the chosen orders; *base:
+// offset of C[0][0] from the address of output coordinate 0
+bool conv_result_in_place (const ConvGemmPlan& g, int64_t* base, int64_t* ldc)
+{
+	if (g.ncheck < 0 || g.N % 4 != 0) { return false; }
+	int64_t run = 1;
+	for (int j = 0; j < 8; ++j)
+	{
+		uint32_t d = g.nord[j];
+		if (g.nsize[d] == 1) { continue; }
+		if ((g.nflip[d] ? -g.ostr[d] : g.ostr[d]) != run) { return false; }
+		run *= g.nsize[d];
+	}
+	int64_t ld = 0, expect = 0;
+	for (int j = 0; j < 8; ++j)
+	{
+		uint32_t d = g.mord[j];
+		if (g.msize[d] == 1) { continue; }
+		if (0 == ld)
+		{
+			ld = g.ostr[d];
+			if (ld < (int64_t) g.N) { return false; }
+			expect = ld;
+		}
+		else if (g.ostr[d] != expect) { return false; }
+		expect *= g.msize[d];
+	}
+	if (0 == ld) { return false; }
+	int64_t off = 0;
+	for (int d = 0; d < 8; ++d)
+	{
+		off += (int64_t) (g.oxlo[d] + (g.nflip[d] ? (int32_t) g.nsize[d] - 1 : 0)) * g.ostr[d];
+	}
+	*base = off;
+	*ldc = ld;
+	return true;
+}
+
+// The product's B is the kernel itself when the kernel elements B[s][n] names
+// form a row-major matrix in the chosen orders
+bool conv_kernel_in_place (const ConvGemmPlan& g, int64_t* base, int64_t* ldb)
+{
+	if (g.ncheck < 0 || g.N % 4 != 0 || g.S % 4 != 0) { return false; }
+	int64_t run = 1, off = 0;
+	for (int j = 0; j < 8; ++j)
+	{
+		uint32_t d = g.nord[j];
+		if (0 == g.is_col[d]) { continue; }
+		// the kernel index of column component q is ilo - x(q)
+		int32_t xfirst = g.xlo[d] + (g.nflip[d] ? (int32_t) g.nsize[d] - 1 : 0);
+		int32_t xlast = g.xlo[d] + (g.nflip[d] ? 0 : (int32_t) g.nsize[d] - 1);
+		int32_t wfirst = g.ilo[d] - xfirst, wlast = g.ilo[d] - xlast;
+		if (wfirst < 0 || wlast < 0 || wfirst >= (int32_t) g.ksize[d] || wlast >= (int32_t) g.ksize[d]) { return false; }
+		if (g.nsize[d] > 1)
+		{
+			if ((g.nflip[d] ? g.kstr[d] : -g.kstr[d]) != run) { return false; }
+			run *= g.nsize[d];
+		}
+		off += (int64_t) wfirst * g.kstr[d];
+	}
+	int64_t ld = 0, expect = 0;
+	for (int j = 0; j < 8; ++j)
+	{
+		uint32_t d = g.sord[j];
+		if (g.is_col[d]) { continue; }
+		if (g.slo[d] < 0 || g.slo[d] + (int32_t) g.ssize[d] > (int32_t) g.ksize[d]) { return false; }
+		off += (int64_t) g.slo[d] * g.kstr[d];
+		if (g.ssize[d] == 1) { continue; }
+		if (0 == ld)
+		{
+			ld = g.kstr[d];
+			if (ld < (int64_t) g.N || ld % 4 != 0) { return false; }
+			expect = ld;
+		}
+		else if (g.kstr[d] != expect) { return false; }
+		expect *= g.ssize[d];
+	}
+	if (0 == ld) { return false; }
+	*base = off;
+	*ldb = ld;
+	return true;
+}
+
 // How the matrix-core kernel can read A straight from the image: along which
 // index memory runs, and whether aligned groups of four along it are
 // contiguous, 16-byte aligned and inside or outside the box together
@@ -491,15 +627,25 @@ void conv_operand_mode (const ConvGemmPlan& g, tcg_conv_operand& op)
 	for (int j = 0; j < 4; ++j) { op.check_ext[j] = j < g.ncheck ? g.check_ext[j] : 0; }
 	op.along_m = false;
 	op.vec4 = false;
+	// the dim that lies along memory
 	int f = -1;
 	for (int d = 0; d < 8 && f < 0; ++d)
 	{
-		if (g.msize[d] > 1 || g.ssize[d] > 1) { f = d; }
+		if (0 == g.is_col[d] && (g.msize[d] > 1 || g.ssize[d] > 1) && g.istr[d] == 1) { f = d; }
 	}
-	if (f < 0 || g.istr[f] != 1 || g.is_col[f]) { return; }
+	if (f < 0) { return; }
 	// both indices may step along the contiguous dim (a spatial dim carries an
-	// output coordinate and a kernel coordinate): the longer run wins
+	// output coordinate and a kernel coordinate): the longer run wins, and it
+	// must be the first dim its index steps along
 	op.along_m = g.msize[f] >= g.ssize[f];
+	const uint32_t* ord = op.along_m ? g.mord : g.sord;
+	const uint32_t* extent = op.along_m ? g.msize : g.ssize;
+	for (int j = 0; j < 8; ++j)
+	{
+		if (extent[ord[j]] == 1) { continue; }
+		if ((int) ord[j] != f) { return; }
+		break;
+	}
 	bool checked = false;
 	for (int j = 0; j < g.ncheck; ++j) { checked = checked || g.check_dim[j] == f; }
 	uint32_t run = op.along_m ? g.msize[f] : g.ssize[f], other = op.along_m ? g.ssize[f] : g.msize[f];
@@ -527,23 +673,37 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 	if (max_rows < 64) { max_rows = 64; }
 	max_rows &= ~(uint64_t) 63;
 	uint32_t chunk = (uint32_t) (g.M < max_rows ? g.M : max_rows);
+	const bool tables = g.ncheck >= 0;
+	// operands and results that already are the matrices of the product stay where they are
+	const char* place_env = getenv("TCG_CONV_IN_PLACE"); // "0": always gather B and scatter C (for tests)
+	const bool in_place = !(place_env && place_env[0] == '0');
+	int64_t b_base = 0, b_ld = 0, c_base = 0, c_ld = 0;
+	bool direct_b = in_place && conv_kernel_in_place(g, &b_base, &b_ld) && tcg_aligned16(ker + b_base);
+	bool direct_c = in_place && conv_result_in_place(g, &c_base, &c_ld);
 	size_t a_bytes = sizeof(T) * (size_t) chunk * g.Sp;
 	size_t b_bytes = sizeof(T) * (size_t) g.Sp * g.Np;
 	size_t c_bytes = sizeof(T) * (size_t) chunk * g.Np;
 	size_t rt_bytes = sizeof(ConvTabEntry) * (size_t) g.M, st_bytes = sizeof(ConvTabEntry) * (size_t) g.Sp;
 	void *A = nullptr, *B = nullptr, *C = nullptr, *RT = nullptr, *ST = nullptr;
-	const bool tables = g.ncheck >= 0;
 	// fp32: the product reads A through the tables, nothing is gathered
 	const char* impl_env = getenv("TCG_CONV_IMPLICIT"); // "0": always materialise A (the parity reference)
 	bool implicit = std::is_same<T,float>::value && tables && !(impl_env && impl_env[0] == '0');
-	int rc = tcg_alloc(ctx, b_bytes, &B);
-	if (rc == TCG_OK) { rc = tcg_alloc(ctx, c_bytes, &C); }
+	int rc = TCG_OK;
+	if (false == direct_b) { rc = tcg_alloc(ctx, b_bytes, &B); }
+	if (rc == TCG_OK && false == direct_c) { rc = tcg_alloc(ctx, c_bytes, &C); }
 	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, rt_bytes, &RT); }
 	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, st_bytes, &ST); }
 	if (rc == TCG_OK)
 	{
-		unsigned grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
-		conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
+		unsigned grid = 0;
+		const T* Bmat = direct_b ? ker + b_base : (const T*) B;
+		const uint64_t ldb = direct_b ? (uint64_t) b_ld : g.Np;
+		const uint64_t ldc = direct_c ? (uint64_t) c_ld : g.Np;
+		if (false == direct_b)
+		{
+			grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
+			conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
+		}
 		if (tables)
 		{
 			uint32_t longest = g.M > g.Sp ? g.M : g.Sp;
@@ -564,6 +724,7 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 		for (uint32_t m0 = 0; m0 < g.M && rc == TCG_OK; m0 += chunk)
 		{
 			uint32_t rows = g.M - m0 < chunk ? g.M - m0 : chunk;
+			T* Cmat = direct_c ? out + c_base + (int64_t) m0 * c_ld : (T*) C;
 			if constexpr (std::is_same<T,float>::value)
 			{
 				if (implicit)
@@ -571,13 +732,16 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 					operand.rows = (const ConvTabEntry*) RT + m0;
 					operand.sums = (const ConvTabEntry*) ST;
 					bool handled = false;
-					rc = tcg_gemm_f32_mfma_conv(ctx, rows, g.Np, g.S, img, operand, (const float*) B, g.Np,
-						(float*) C, g.Np, &handled);
+					rc = tcg_gemm_f32_mfma_conv(ctx, rows, g.Np, g.S, img, operand, (const float*) Bmat, ldb,
+						(float*) Cmat, ldc, &handled);
 					if (rc != TCG_OK) { break; }
 					if (handled)
 					{
-						grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
-						conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+						if (false == direct_c)
+						{
+							grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
+							conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+						}
 						continue;
 					}
 					implicit = false; // shapes the matrix-core kernel does not take: gather as below
@@ -607,10 +771,14 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 				grid = tcg_grid(ctx, (uint64_t) rows * g.Sp, CG_BLOCK, 32);
 				conv_gather_image_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, img, (T*) A);
 			}
-			rc = tcg_gemm(ctx, dtype, rows, g.Np, g.Sp, 1, A, g.Sp, 0, 0, B, g.Np, 0, 0, C, g.Np, 0);
+			// (a kernel read in place has S rows: S is then a multiple of four and equals Sp)
+			rc = tcg_gemm(ctx, dtype, rows, g.Np, g.Sp, 1, A, g.Sp, 0, 0, Bmat, ldb, 0, 0, Cmat, ldc, 0);
 			if (rc != TCG_OK) { break; }
-			grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
-			conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+			if (false == direct_c)
+			{
+				grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
+				conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+			}
 		}
 	}
 	if (A) { tcg_free(ctx, A, a_bytes); }
@@ -627,12 +795,17 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 
 extern "C" {
 
-// dense_box: `img` holds only the elements inside [img_lo, img_hi), densely
+// dense_box: `img` holds only the elements inside [img_lo, img_hi), densely,
+// or with the element strides `box_stride` when those are given.
+// kernel_stride (per kernel dim) / out_stride (per output dim; `out` is then
+// the address of the first output of the window): element strides of the
+// kernel and of the result when they are not the dense ones.
 static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
 	const uint64_t img_lo[8], const uint64_t img_hi[8],
 	const uint64_t out_lo[8], const uint64_t out_hi[8],
-	const void* img, const void* kernel, void* out, bool dense_box)
+	const void* img, const void* kernel, void* out, bool dense_box,
+	const int64_t* box_stride = nullptr, const int64_t* kernel_stride = nullptr, const int64_t* out_stride = nullptr)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, imgshape && kshape && img && kernel && out && (ranks || nranks == 0), "tcg_conv: NULL pointer");
@@ -672,7 +845,7 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 		TCG_REQUIRE(ctx, kshape[i] <= oshape[d], "tcg_conv: cannot convolve a kernel against a smaller image (kernel dim %d)", i);
 		oshape[d] -= kshape[i] - 1;
 		p.ksize[d] = (uint32_t) kshape[i];
-		p.kstr[d] = kmem[i];
+		p.kstr[d] = kernel_stride ? kernel_stride[i] : kmem[i];
 	}
 	p.istr[0] = p.ostr[0] = 1;
 	for (int d = 1; d < 8; ++d)
@@ -696,6 +869,14 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 		p.nwin *= p.wsize[d];
 		uint64_t span = ihi - ilo < p.ksize[d] ? ihi - ilo : p.ksize[d];
 		max_terms *= span;
+	}
+	if (out_stride)
+	{
+		for (int d = 0; d < 8; ++d)
+		{
+			p.ostr[d] = out_stride[d];
+			p.ooff0 -= (int64_t) p.wlo[d] * out_stride[d];
+		}
 	}
 	ConvGemmPlan gp;
 	const char* gemm_env = getenv("TCG_CONV_GEMM"); // "0": direct kernels only (the parity reference)
@@ -740,10 +921,16 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 				gp.xlo[d] -= p.ilo[d];
 				gp.ilo[d] = 0;
 				gp.ihi[d] = (int32_t) box[d];
-				gp.istr[d] = run;
+				gp.istr[d] = (dense_box && box_stride) ? box_stride[d] : run;
 				run *= (int64_t) box[d];
 			}
 		}
+		if (out_stride)
+		{
+			// `out` starts at the window
+			for (int d = 0; d < 8; ++d) { gp.oxlo[d] = 0; }
+		}
+		conv_choose_orders(gp);
 		int rc = TCG_OK;
 		TCG_DISPATCH_TYPE(ctx, dtype, rc = conv_gemm_run<T>(ctx, dtype, gp, (const T*) img, (const T*) kernel, (T*) out));
 		if (dense) { tcg_free(ctx, dense, box_elems * esz); }
@@ -754,8 +941,8 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 		int64_t run = 1;
 		for (int d = 0; d < 8; ++d)
 		{
-			p.istr[d] = run;
-			p.ioff0 -= (int64_t) p.ilo[d] * run;
+			p.istr[d] = box_stride ? box_stride[d] : run;
+			p.ioff0 -= (int64_t) p.ilo[d] * p.istr[d];
 			run *= (int64_t) (p.ihi[d] - p.ilo[d]);
 		}
 	}
@@ -797,6 +984,21 @@ int tcg_conv_dense_box (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	TCG_REQUIRE(ctx, img_lo && img_hi, "tcg_conv_dense_box: the box is required");
 	return conv_boxed_impl(ctx, dtype, imgshape, kshape, nranks, ranks, img_lo, img_hi, out_lo, out_hi,
 		box, kernel, out, true);
+}
+
+int tcg_conv_views (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
+	const uint64_t kshape[8], int nranks, const uint64_t* ranks,
+	const uint64_t img_lo[8], const uint64_t img_hi[8],
+	const uint64_t out_lo[8], const uint64_t out_hi[8],
+	const void* box, const int64_t box_stride[8],
+	const void* kernel, const int64_t kernel_stride[8],
+	void* out, const int64_t out_stride[8])
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, img_lo && img_hi && box_stride && kernel_stride && out_stride,
+		"tcg_conv_views: the box and the three stride lists are required");
+	return conv_boxed_impl(ctx, dtype, imgshape, kshape, nranks, ranks, img_lo, img_hi, out_lo, out_hi,
+		box, kernel, out, true, box_stride, kernel_stride, out_stride);
 }
 
 int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],

@@ -1,8 +1,9 @@
 // Grouping of elementwise functors for the replaying evaluator: which nodes
 // of an evaluation pass are computed together in one tcg_ew_fusedx launch,
 // which EXTEND / SLICE / PAD / PERMUTE / IDENTITY nodes are never materialised
-// because elementwise groups read straight through them, and in which order
-// the remaining launches run.  The reference evaluates one node at a time
+// because elementwise groups read straight through them, which PAD / PERMUTE /
+// REVERSE nodes round a convolution become strides of its launch, and in which
+// order the remaining launches run.  The reference evaluates one node at a time
 // (internal/teq/evaluator.hpp:33-45 calling internal/eigen/device.hpp:555-570);
 // Eigen fuses only inside one node's expression.
 #ifndef TCH_FUSE_PLAN_HPP
@@ -64,23 +65,39 @@ struct SummedContracts final
 	std::vector<teq::iTensor*> reads;
 };
 
-/// CONV(PAD(x), kernel) where convolutions are all that read the PAD node:
-/// the correlation is computed from x itself, told where it sits inside the
-/// zero border, and the padded image is never laid out (conv2d and its
-/// gradients pad a singleton axis to 2n-1 before correlating,
-/// cfg/tenncor/nn.yml:88-93, tenncor/eteq/backprop.hpp:372-399)
-struct PaddedConv final
+/// A CONV node computed from the tensors its operands are layouts of, into the
+/// tensor its result is a layout of.  tenncor surrounds every convolution with
+/// nodes that only move data: conv2d reverses the kernel, pads a singleton axis
+/// of the image and permutes the result (cfg/tenncor/nn.yml:88-93); its
+/// gradients permute and pad the upstream gradient in front of the correlation
+/// and permute and reverse what comes out (tenncor/eteq/backprop.hpp:372-439).
+/// Where convolutions are all that read such a PAD / PERMUTE / REVERSE node,
+/// and where one PERMUTE / REVERSE is all that reads the result, none of these
+/// is laid out: the correlation reads and writes through element strides
+/// (tcg_conv_views), and the padded image exists only as the box in which the
+/// operand sits inside the zero border.
+struct ViewedConv final
 {
-	Observable* node = nullptr;      ///< the CONV node
-	teq::iTensor* image = nullptr;   ///< operand of the PAD node
-	teq::iTensor* kernel = nullptr;
-	std::array<uint64_t,8> imgshape, kshape; ///< imgshape: the PAD node's
-	std::array<uint64_t,8> ilo, ihi; ///< where the operand sits in the padded image
+	Observable* node = nullptr;      ///< receives the result: the CONV node, or the last PERMUTE / REVERSE behind it
+	teq::iTensor* image = nullptr;   ///< materialised tensor the image is read from
+	teq::iTensor* kernel = nullptr;  ///< materialised tensor the kernel is read from
+	std::array<uint64_t,8> imgshape, kshape; ///< of the CONV node's operands as it sees them
+	std::array<uint64_t,8> ilo, ihi; ///< where the image is not zero border
+	/// image element c (inside the box) is element image_off + sum c[d] * image_stride[d] of `image`
+	int64_t image_off = 0;
+	std::array<int64_t,8> image_stride;
+	/// kernel element w is element kernel_off + sum w[i] * kernel_stride[i] of `kernel`
+	int64_t kernel_off = 0;
+	std::array<int64_t,8> kernel_stride;
 	bool windowed = false;           ///< only SLICEs read the result:
-	std::array<uint64_t,8> olo, ohi; ///< their bounding box
+	std::array<uint64_t,8> olo, ohi; ///< their bounding box (else the whole result)
+	/// output element c is element out_off + sum c[d] * out_stride[d] of `node`'s buffer
+	int64_t out_off = 0;
+	std::array<int64_t,8> out_stride;
 	std::vector<uint64_t> ranks;
 	int dtype = 0;
 	std::vector<teq::iTensor*> reads;
+	std::string label;               ///< the nodes this launch stands for, for printing
 };
 
 struct FusionPlan final
@@ -96,7 +113,7 @@ struct FusionPlan final
 
 	std::vector<FusedGroup> groups;
 	std::vector<SwappedContract> contracts;
-	std::vector<PaddedConv> convs;
+	std::vector<ViewedConv> convs;
 	std::vector<SummedContracts> sums;
 	std::vector<Step> steps;
 	/// functors that are computed inside a group or folded into operand views
@@ -113,7 +130,7 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
-void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptrT& memory);
+void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMemptrT& memory);
 

@@ -48,8 +48,9 @@ struct Node final
 	bool target = false;
 	bool absorbed = false;      // a VIEW no launch of its own computes
 	int swapped_from = -1;      // PERMUTE launched as the swapped product of this CONTRACT node
-	int padded_from = -1;       // CONV reading the operand of this PAD node in place of the padded image
-	bool through_conv = false;  // PAD that only such convolutions read
+	int conv_from = -1;         // this node receives the result of that CONV node, launched over views (itself, or the end of a chain behind it)
+	bool through_conv = false;  // PAD / PERMUTE / REVERSE that only such convolutions read through, or
+	                            // a node between such a CONV and the node that receives its result
 	bool summed = false;        // ADD launched as one sum of the products it adds
 	bool summed_term = false;   // CONTRACT / PERMUTE that is a term of such a sum
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
@@ -189,27 +190,7 @@ struct Planner final
 			c.kind = VIEW;
 			c.absorbed = true;
 		}
-		// PAD of a plain value read by convolutions only, as their image: they
-		// read the value itself
-		for (size_t i = 0; i < nodes_.size(); ++i)
-		{
-			Node& n = nodes_[i];
-			if (n.op != egen::PAD || n.kind != VIEW || n.target || n.consumers.empty()) { continue; }
-			bool convolved = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
-			{
-				const Node& conv = nodes_[c];
-				return conv.op == egen::CONV && conv.args.size() == 2 && conv.args[0] == (int) i &&
-					conv.args[1] != (int) i && conv.dtype == n.dtype;
-			});
-			Shape8 lo, hi, inner = shape8(n.arg_tens[0]->shape());
-			nonzero_box(*n.arg_tens[0], lo, hi);
-			bool plain = hi == inner && std::all_of(lo.begin(), lo.end(), [](uint64_t v) { return v == 0; });
-			if (false == convolved || false == plain) { continue; }
-			if (written_between((int) i, {0}, (int) i, n.consumers.back() + 1)) { continue; }
-			n.absorbed = true;
-			n.through_conv = true;
-			for (int c : n.consumers) { nodes_[c].padded_from = (int) i; }
-		}
+		find_viewed_convs();
 		find_summed_products();
 		// a view is folded away when everything that reads it can read through it
 		std::vector<int> last_reader(nodes_.size(), 0); // position of the last launch reading through a folded view
@@ -262,6 +243,152 @@ struct Planner final
 	{
 		const Node& n = nodes_[i];
 		return n.kind == VIEW && n.absorbed && n.op == egen::IDENTITY;
+	}
+
+	// ---- convolutions over views ----
+
+	struct ConvFold final
+	{
+		std::vector<int> image, kernel; // folded nodes from the CONV's operand down to (excluding) the tensor that is read
+		std::vector<int> result;        // nodes behind the CONV up to (including) the one that receives the result
+	};
+
+	static bool is_layout (const Node& n)
+	{
+		return (n.op == egen::PERMUTE || n.op == egen::REVERSE) && n.args.size() == 1;
+	}
+
+	bool is_plain_conv (int i) const
+	{
+		const Node& n = nodes_[i];
+		return n.op == egen::CONV && n.kind == OTHER && n.args.size() == 2 &&
+			(int) n.arg_tens[0]->get_meta().type_code() == n.dtype &&
+			(int) n.arg_tens[1]->get_meta().type_code() == n.dtype;
+	}
+
+	/// Position of the last convolution that would read through node v
+	int last_conv_reader (int v) const
+	{
+		int last = -1;
+		for (int c : nodes_[v].consumers)
+		{
+			last = std::max(last, nodes_[c].op == egen::CONV ? c : last_conv_reader(c));
+		}
+		return last;
+	}
+
+	/// PAD node whose only readers are convolutions taking it as their image
+	bool pad_feeds_convs (int v) const
+	{
+		const Node& n = nodes_[v];
+		if (n.op != egen::PAD || n.kind != VIEW || n.target || n.consumers.empty()) { return false; }
+		for (int c : n.consumers)
+		{
+			if (false == is_plain_conv(c) || nodes_[c].args[0] != v || nodes_[c].args[1] == v) { return false; }
+		}
+		// the convolutions read the operand where they stand, not where the PAD does
+		return false == written_between(v, {0}, v, last_conv_reader(v) + 1);
+	}
+
+	/// PERMUTE / REVERSE node that only convolutions read, directly, through
+	/// such a PAD or through further nodes of this kind
+	bool layout_feeds_convs (int v)
+	{
+		auto memo = feeds_convs_.find(v);
+		if (memo != feeds_convs_.end()) { return memo->second; }
+		const Node& n = nodes_[v];
+		bool ok = is_layout(n) && false == n.target && false == n.consumers.empty() &&
+			n.swapped_from < 0 && false == n.summed_term;
+		for (size_t k = 0; k < n.consumers.size() && ok; ++k)
+		{
+			int c = n.consumers[k];
+			if (nodes_[c].op == egen::CONV) { ok = is_plain_conv(c); }
+			else if (nodes_[c].op == egen::PAD) { ok = pad_feeds_convs(c); }
+			else { ok = is_layout(nodes_[c]) && nodes_[c].args[0] == v && layout_feeds_convs(c); }
+		}
+		ok = ok && false == written_between(v, {0}, v, last_conv_reader(v) + 1);
+		feeds_convs_[v] = ok;
+		return ok;
+	}
+
+	void find_viewed_convs (void)
+	{
+		for (size_t i = 0; i < nodes_.size(); ++i)
+		{
+			if (false == is_plain_conv((int) i)) { continue; }
+			ConvFold fold;
+			int cur = nodes_[i].args[0];
+			if (cur >= 0 && cur != nodes_[i].args[1] && pad_feeds_convs(cur))
+			{
+				fold.image.push_back(cur);
+				cur = nodes_[cur].args[0];
+			}
+			while (cur >= 0 && layout_feeds_convs(cur))
+			{
+				fold.image.push_back(cur);
+				cur = nodes_[cur].args[0];
+			}
+			cur = nodes_[i].args[1];
+			while (cur >= 0 && layout_feeds_convs(cur))
+			{
+				fold.kernel.push_back(cur);
+				cur = nodes_[cur].args[0];
+			}
+			// behind the convolution: one reader at a time, each only moving data,
+			// standing where nothing rewrites the operands in between
+			cur = (int) i;
+			while (false == nodes_[cur].target && nodes_[cur].consumers.size() == 1)
+			{
+				int next = nodes_[cur].consumers[0];
+				const Node& m = nodes_[next];
+				if (false == is_layout(m) || m.args[0] != cur || m.swapped_from >= 0 || m.summed_term ||
+					m.dtype != nodes_[i].dtype) { break; }
+				fold.result.push_back(next);
+				cur = next;
+			}
+			if (false == fold.result.empty())
+			{
+				// the launch stands where the last of them does
+				bool rewritten = written_between((int) i, {0, 1}, (int) i, fold.result.back());
+				for (const std::vector<int>* chain : {&fold.image, &fold.kernel})
+				{
+					for (int v : *chain) { rewritten = rewritten || written_between(v, {0}, (int) i, fold.result.back()); }
+				}
+				if (rewritten) { fold.result.clear(); }
+			}
+			if (fold.image.empty() && fold.kernel.empty() && fold.result.empty()) { continue; }
+			folds_.emplace((int) i, fold);
+		}
+		// marks are set once every decision has been taken on the graph as built
+		for (auto& kv : folds_)
+		{
+			const ConvFold& fold = kv.second;
+			for (const std::vector<int>* chain : {&fold.image, &fold.kernel})
+			{
+				for (int v : *chain)
+				{
+					nodes_[v].kind = VIEW;
+					nodes_[v].absorbed = true;
+					nodes_[v].through_conv = true;
+				}
+			}
+			int last = fold.result.empty() ? kv.first : fold.result.back();
+			if (false == fold.result.empty())
+			{
+				nodes_[kv.first].kind = VIEW;
+				nodes_[kv.first].absorbed = true;
+				nodes_[kv.first].through_conv = true;
+				for (int v : fold.result)
+				{
+					if (v == last) { break; }
+					nodes_[v].kind = VIEW;
+					nodes_[v].absorbed = true;
+					nodes_[v].through_conv = true;
+				}
+				nodes_[last].kind = OTHER;
+			}
+			nodes_[last].conv_from = kv.first;
+		}
 	}
 
 	// ---- sums of products ----
@@ -582,9 +709,140 @@ struct Planner final
 				}
 			}
 				break;
+			case egen::REVERSE:
+			{
+				// only for the operands of convolutions: elementwise launches do not walk backwards
+				std::set<teq::RankT> dims;
+				Packer<std::set<teq::RankT>>().unpack(dims, *n.f);
+				for (teq::RankT d : dims)
+				{
+					if (d >= 8) { continue; }
+					out.off += (int64_t) (inshape[d] - 1) * in.stride[d];
+					out.stride[d] = -in.stride[d];
+					out.lo[d] = inshape[d] - in.hi[d];
+					out.hi[d] = inshape[d] - in.lo[d];
+				}
+			}
+				break;
 			default: global::fatal("not a view");
 		}
 		return out;
+	}
+
+	/// The launch of the convolution whose result node u receives
+	ViewedConv viewed_conv (int u, int step, FusionPlan& plan, std::map<int,int>& last_conv)
+	{
+		const int ci = nodes_[u].conv_from;
+		const Node& c = nodes_[ci];
+		const ConvFold& fold = folds_.at(ci);
+		ViewedConv call;
+		call.node = nodes_[u].f;
+		call.dtype = c.dtype;
+		call.imgshape = shape8(c.arg_tens[0]->shape());
+		call.kshape = shape8(c.arg_tens[1]->shape());
+		teq::RanksT order;
+		Packer<teq::RanksT>().unpack(order, *c.f);
+		for (size_t k = 0; k < std::min(order.size(), (size_t) teq::rank_cap); ++k) { call.ranks.push_back(order[k]); }
+		// operands: the views the folded nodes add up to
+		View image = view_of_arg(ci, 0), kernel = view_of_arg(ci, 1);
+		call.image = image.base;
+		call.kernel = kernel.base;
+		call.image_off = image.off;
+		call.kernel_off = kernel.off;
+		for (int d = 0; d < 8; ++d)
+		{
+			call.image_stride[d] = image.stride[d];
+			call.kernel_stride[d] = kernel.stride[d];
+			call.ilo[d] = image.lo[d];
+			call.ihi[d] = image.hi[d];
+			if (kernel.lo[d] != 0 || kernel.hi[d] != call.kshape[d]) { global::fatal("a kernel read through a border"); }
+		}
+		for (const std::vector<int>* chain : {&fold.image, &fold.kernel})
+		{
+			for (int v : *chain) { last_conv[v] = step; }
+		}
+		// the operands the CONV node itself would have counted as read
+		for (size_t k = 0; k < 2; ++k)
+		{
+			int a = c.args[k];
+			if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+			{
+				call.reads.push_back(c.arg_tens[k].get());
+			}
+		}
+		// the result: which output dim each dim of the receiving node is, and in which direction
+		Shape8 oshape = c.shape;
+		call.windowed = fold.result.empty() && false == c.target && slices_window(c.f, c.f->shape(), call.olo, call.ohi);
+		if (false == call.windowed)
+		{
+			for (int d = 0; d < 8; ++d)
+			{
+				call.olo[d] = 0;
+				call.ohi[d] = oshape[d];
+			}
+		}
+		int from[8];          // dim of the receiving node -> output dim of the convolution
+		bool backwards[8];
+		for (int d = 0; d < 8; ++d)
+		{
+			from[d] = d;
+			backwards[d] = false;
+		}
+		for (int v : fold.result)
+		{
+			const Node& m = nodes_[v];
+			if (m.op == egen::PERMUTE)
+			{
+				teq::RanksT perm;
+				Packer<teq::RanksT>().unpack(perm, *m.f);
+				if (perm.size() > 8) { perm.resize(8); }
+				bool visited[8] = {false};
+				for (teq::RankT r : perm) { visited[r] = true; }
+				for (teq::RankT d = 0; d < 8; ++d)
+				{
+					if (false == visited[d]) { perm.push_back(d); }
+				}
+				int was[8];
+				bool wasback[8];
+				std::copy(from, from + 8, was);
+				std::copy(backwards, backwards + 8, wasback);
+				for (int d = 0; d < 8; ++d)
+				{
+					from[d] = was[perm[d]];
+					backwards[d] = wasback[perm[d]];
+				}
+			}
+			else
+			{
+				std::set<teq::RankT> dims;
+				Packer<std::set<teq::RankT>>().unpack(dims, *m.f);
+				for (teq::RankT d : dims)
+				{
+					if (d < 8) { backwards[d] = !backwards[d]; }
+				}
+			}
+			if (v != u) { plan.absorbed.push_back(m.f); }
+		}
+		if (false == fold.result.empty()) { plan.absorbed.push_back(c.f); }
+		Shape8 rshape = nodes_[u].shape;
+		int64_t run = 1;
+		call.out_off = 0;
+		for (int d = 0; d < 8; ++d)
+		{
+			// dim d of the receiving node walks output dim from[d]
+			call.out_stride[from[d]] = backwards[d] ? -run : run;
+			if (backwards[d]) { call.out_off += (int64_t) (rshape[d] - 1) * run; }
+			run *= (int64_t) rshape[d];
+		}
+		// label: image side, kernel side, CONV, result side
+		std::string label;
+		for (auto it = fold.image.rbegin(); it != fold.image.rend(); ++it) { label += nodes_[*it].f->get_opcode().name_ + "+"; }
+		for (auto it = fold.kernel.rbegin(); it != fold.kernel.rend(); ++it) { label += nodes_[*it].f->get_opcode().name_ + "+"; }
+		label += "CONV";
+		for (int v : fold.result) { label += "+" + nodes_[v].f->get_opcode().name_; }
+		if (call.windowed) { label += "+SLICE"; }
+		call.label = label;
+		return call;
 	}
 
 	// ---- units: what is launched as one thing ----
@@ -981,30 +1239,11 @@ struct Planner final
 				plan.steps.push_back(step);
 				return;
 			}
-			if (nodes_[u].kind != EW && nodes_[u].padded_from >= 0)
+			if (nodes_[u].kind != EW && nodes_[u].conv_from >= 0)
 			{
-				const Node& n = nodes_[u];
-				const Node& pad = nodes_[n.padded_from];
-				PaddedConv call;
-				call.node = n.f;
-				call.dtype = n.dtype;
-				call.image = pad.arg_tens[0].get();
-				call.kernel = n.arg_tens[1].get();
-				call.imgshape = pad.shape;
-				call.kshape = shape8(call.kernel->shape());
-				teq::RanksT order;
-				Packer<teq::RanksT>().unpack(order, *n.f);
-				for (size_t k = 0; k < std::min(order.size(), (size_t) teq::rank_cap); ++k) { call.ranks.push_back(order[k]); }
-				nonzero_box(*pad.f, call.ilo, call.ihi);
-				call.windowed = false == n.target && slices_window(n.f, n.f->shape(), call.olo, call.ohi);
-				if (n.args[1] >= 0 && false == (nodes_[n.args[1]].kind == VIEW && nodes_[n.args[1]].absorbed))
-				{
-					call.reads.push_back(call.kernel);
-				}
 				FusionPlan::Step step;
 				step.conv = (int) plan.convs.size();
-				last_conv[n.padded_from] = step.conv;
-				plan.convs.push_back(call);
+				plan.convs.push_back(viewed_conv(u, step.conv, plan, last_conv));
 				plan.steps.push_back(step);
 				return;
 			}
@@ -1061,11 +1300,17 @@ struct Planner final
 		}
 		// a folded view counts one read of its operand, when the last launch
 		// that looks through it has been enqueued
+		// a node folded into convolutions counts one read of its operand, when
+		// the last of them has been enqueued
 		for (auto& kv : last_conv)
 		{
-			const Node& pad = nodes_[kv.first];
-			plan.absorbed.push_back(pad.f);
-			if (pad.args[0] >= 0) { plan.convs[kv.second].reads.push_back(pad.arg_tens[0].get()); }
+			const Node& v = nodes_[kv.first];
+			plan.absorbed.push_back(v.f);
+			int a = v.args[0];
+			if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+			{
+				plan.convs[kv.second].reads.push_back(v.arg_tens[0].get());
+			}
 		}
 		for (auto& kv : last_user)
 		{
@@ -1089,6 +1334,8 @@ struct Planner final
 	}
 
 	std::vector<Node> nodes_;
+	std::map<int,ConvFold> folds_;       // CONV node -> what is folded into its launch
+	std::map<int,bool> feeds_convs_;     // memo of layout_feeds_convs
 	std::unordered_map<teq::iTensor*,int> index_;
 	std::vector<int> uf_, minpos_, maxpos_;
 	std::vector<std::vector<int>> members_;
@@ -1161,7 +1408,7 @@ void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMe
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
-void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptrT& memory)
+void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory)
 {
 	Observable* out = call.node;
 	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
@@ -1172,11 +1419,23 @@ void launch_conv (const PaddedConv& call, const teq::TensSetT& targets, RTMemptr
 	const void* kernel = eigen_ref(*call.kernel).device_data();
 	if (nullptr == image || nullptr == kernel) { global::fatal("operand of a convolution has no data"); }
 	if (call.windowed) { ref.mark_partial(); }
+	// addresses of the first image element inside the box, of kernel element 0
+	// and of the first output of the window
+	const int64_t esz = (int64_t) egen::type_size((egen::_GENERATED_DTYPE) call.dtype);
+	int64_t first_image = call.image_off, first_out = call.out_off;
+	for (int d = 0; d < 8; ++d)
+	{
+		first_image += (int64_t) call.ilo[d] * call.image_stride[d];
+		first_out += (int64_t) call.olo[d] * call.out_stride[d];
+	}
 	try
 	{
-		hip_check(tcg_conv_dense_box(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), call.imgshape.data(), call.kshape.data(),
-			(int) call.ranks.size(), call.ranks.data(), call.ilo.data(), call.ihi.data(),
-			call.windowed ? call.olo.data() : nullptr, call.windowed ? call.ohi.data() : nullptr, image, kernel, dst));
+		hip_check(tcg_conv_views(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype),
+			call.imgshape.data(), call.kshape.data(), (int) call.ranks.size(), call.ranks.data(),
+			call.ilo.data(), call.ihi.data(), call.olo.data(), call.ohi.data(),
+			(const char*) image + esz * first_image, call.image_stride.data(),
+			(const char*) kernel + esz * call.kernel_off, call.kernel_stride.data(),
+			(char*) dst + esz * first_out, call.out_stride.data()));
 	}
 	catch (...)
 	{

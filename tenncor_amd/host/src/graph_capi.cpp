@@ -427,7 +427,7 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 			}
 			if (step.conv >= 0)
 			{
-				ss << "padded PAD+CONV" << (plan.convs[step.conv].windowed ? "+SLICE" : "") << "\n";
+				ss << "viewed " << plan.convs[step.conv].label << "\n";
 				continue;
 			}
 			auto& group = plan.groups[step.group];

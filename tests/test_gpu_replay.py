@@ -368,6 +368,54 @@ def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
     assert stats["replay_launches"]["launches"] < stats["replay_unfused"]["launches"]
 
 
+@pytest.mark.parametrize("np_dtype", [np.int32, np.float32])
+def test_convolutions_over_views_follow_the_walk(np_dtype):
+    """A conv2d layer with its two gradients at a size where the correlations
+    run as matrix products (cfg/tenncor/nn.yml:88-93,
+    tenncor/eteq/backprop.hpp:372-439), followed by an in-place update of the
+    kernel.  The recording reads the operands through the PAD / PERMUTE /
+    REVERSE nodes in front of each CONV and writes where the PERMUTE / REVERSE
+    behind it would: in int32 every result equals the walk's bit for bit
+    (wrapping sums do not depend on their order), in fp32 within 1e-5 of the
+    largest entry; the kernel update must see the gradient of the old kernel."""
+    rng = np.random.default_rng(31)
+    C, W, H, B, O, K = 8, 14, 12, 32, 16, 3
+    if np_dtype == np.int32:
+        feeds = [rng.integers(-9, 10, C * W * H * B).astype(np.int32) for _ in range(4)]
+        k0 = rng.integers(-5, 6, O * C * K * K).astype(np.int32)
+    else:
+        feeds = [rng.uniform(-1, 1, C * W * H * B).astype(np.float32) for _ in range(4)]
+        k0 = rng.uniform(-0.3, 0.3, O * C * K * K).astype(np.float32)
+
+    def build(g, api):
+        x = g.variable(feeds[0], [C, W, H, B], "x")
+        k = g.variable(k0, [O, C, K, K], "k")
+        y = api.conv2d(x, k)
+        loss = api.reduce_sum(api.square(y))
+        dx, dk = g.derive(loss, [x, k])
+        step = api.assign_sub(k, dk)  # the next pass convolves with the updated kernel
+        return [loss, dx, dk, step], x
+
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+    for kind in ("replay_launches", "replay"):
+        assert stats[kind]["recorded"] == 1 and stats[kind]["replayed"] == len(feeds) - 1  # the recording pass launches it too
+        for row, ref in zip(results[kind], results["plain"]):
+            for got, want in zip(row, ref):
+                if np_dtype == np.int32:
+                    np.testing.assert_array_equal(got, want, err_msg=kind)
+                else:
+                    assert np.abs(got.astype(np.float64) - want).max() <= 1e-5 * max(np.abs(want).max(), 1e-30), kind
+    from tenncor_amd import graph
+    g = graph.Graph()
+    try:
+        targets, _ = build(g, graph.Api(g))
+        lines = g.launch_plan(targets)
+        # (a REVERSE of the kernel that a convolution behind the update still reads keeps its own launch)
+        assert sum(1 for l in lines if l.startswith("viewed ")) == 3 and "node CONV" not in lines and "node PAD" not in lines
+    finally:
+        g.close()
+
+
 @pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
 def test_fused_views_diamonds_and_wide_groups(np_dtype):
     """Shapes the grouping has to get right: operands seen through SLICE, PAD,

@@ -271,7 +271,7 @@ def parse_plan(lines):
         elif kind == "group":
             ops, *fields = rest.split(" ")
             steps.append(("group", ops.split("+"), {k: int(v) for k, v in (f.split("=") for f in fields)}))
-        elif kind in ("swapped", "padded"):
+        elif kind in ("swapped", "viewed"):
             steps.append((kind, rest.split("+"), {}))
         else:
             steps.append(("folded", [], {"n": int(rest)}))
@@ -356,19 +356,26 @@ def test_launch_plan_reads_the_operand_of_a_pad_that_only_convolutions_read(g, a
     loss = api.reduce_sum(api.square(y))
     dx, dk = g.derive(loss, [x, k])
     lines = g.launch_plan([loss, dx, dk])
-    # forward, kernel gradient (both read PAD(x)) and image gradient (reads PAD of the
-    # upstream gradient; only one index of its result is sliced back out)
-    assert lines.count("padded PAD+CONV") == 2 and lines.count("padded PAD+CONV+SLICE") == 1
-    assert "node PAD" not in lines and "node CONV" not in lines
+    # forward (reads x where PAD would put it and the kernel through its REVERSE, writes what
+    # PERMUTE would make of the result), kernel gradient (reads PAD(x) too, and the upstream
+    # gradient through its PERMUTE; the PERMUTE and REVERSE behind it are where it writes) and
+    # image gradient (reads the upstream gradient through PERMUTE and PAD, the kernel through
+    # both REVERSEs; only one index of its result is sliced back out)
+    assert lines.count("viewed PAD+REVERSE+CONV+PERMUTE") == 1
+    assert lines.count("viewed PAD+PERMUTE+CONV+PERMUTE+REVERSE") == 1
+    assert lines.count("viewed PERMUTE+PAD+REVERSE+REVERSE+CONV+SLICE") == 1
+    for op in ("PAD", "CONV", "PERMUTE", "REVERSE"):
+        assert "node " + op not in lines
     steps = parse_plan(lines)
-    alone = sum(1 for s in steps if s[0] in ("node", "swapped", "padded"))
+    alone = sum(1 for s in steps if s[0] in ("node", "swapped", "viewed"))
     stores = sum(s[2]["stores"] for s in steps if s[0] == "group")
     assert alone + stores + steps[-1][2]["n"] == g.count_functors([loss, dx, dk])
     # a padded image somebody else reads, or asks for, is laid out as before
     padded = g.args(g.args(y)[0])[0]
     assert g.opcode(padded) == "PAD"
     lines = g.launch_plan([y, padded])
-    assert "node PAD" in lines and "node CONV" in lines and not any(l.startswith("padded") for l in lines)
+    # (the kernel is still read through its REVERSE and the result written as the PERMUTE wants it)
+    assert "node PAD" in lines and "viewed REVERSE+CONV+PERMUTE" in lines and "node CONV" not in lines
 
 
 def test_launch_plan_keeps_reads_of_a_variable_on_their_side_of_an_assignment(g, api):
