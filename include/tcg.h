@@ -275,7 +275,7 @@ enum tcg_fx_operand
 #define TCG_FX_MAX_LEAVES 16
 #define TCG_FX_MAX_REGS 16
 #define TCG_FX_MAX_INSTRS 64
-#define TCG_FX_MAX_OUTS 8
+#define TCG_FX_MAX_OUTS 16
 #define TCG_FX_STORE 255 /* opcode */
 /* opcode: bitwise OR of the two operands' representations. Zero-bordered
  * leaves whose boxes tile the output, OR-ed together, are CONCAT

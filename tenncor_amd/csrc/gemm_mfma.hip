@@ -493,7 +493,12 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 	uint64_t tiles = ((M + 63) / 64) * ((N + 63) / 64) * batch;
 	uint64_t splits = 2 * (uint64_t) ctx->num_cus / tiles;
 	if (splits > K / 64) { splits = K / 64; }
-	if (splits > 32) { splits = 32; }
+	// a sliver of a result under a very long K (the kernel gradient of a
+	// convolution's first layer: 25 x 32 results, K = 73728) may take a
+	// workgroup per CU and more, as long as every range keeps 256 summed indices
+	uint64_t cap = K / 256 > 32 ? K / 256 : 32;
+	if (cap > 256) { cap = 256; }
+	if (splits > cap) { splits = cap; }
 	if (splits < 2 || batch >= (1ull << 16)) { splits = 1; }
 	return launch<64,64,2,IMPL>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
 }

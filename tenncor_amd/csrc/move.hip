@@ -411,6 +411,47 @@ int check_dims (tcg_ctx* ctx, const uint64_t shape[8], const char* what)
 
 #define CHECK_DIMS(ctx, shape, what) do { int rc__ = check_dims(ctx, shape, what); if (rc__ != TCG_OK) { return rc__; } } while (0)
 
+// CONCAT of many operands in one launch: the result seen as
+// [outer][along the axis][inner]; every lane finds the operand its group of V
+// elements comes from in a table of where each operand starts along the axis
+constexpr int CC_MAX = 128;
+
+template <typename T, int V> struct VecOf { typedef T type; };
+template <> struct VecOf<uint32_t,4> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+
+struct ConcatTab
+{
+	const void* src[CC_MAX];
+	uint32_t start[CC_MAX + 1]; // along the axis; start[n] = extent of the result
+	uint32_t n;
+};
+
+template <typename T, int V>
+__global__ __launch_bounds__(MV_BLOCK) void concat_many_k (ConcatTab tab, FastDiv inner_div, FastDiv axis_div,
+	uint32_t inner_vecs, uint32_t nvec, T* __restrict__ dst)
+{
+	typedef typename VecOf<T,V>::type Vec;
+	const uint32_t step = gridDim.x * MV_BLOCK;
+	for (uint32_t idx = blockIdx.x * MV_BLOCK + threadIdx.x; idx < nvec; idx += step)
+	{
+		// idx = (outer * axis_total + along) * inner_vecs + within
+		const uint32_t row = fdiv(idx, inner_div);
+		const uint32_t within = idx - row * inner_vecs;
+		const uint32_t outer = fdiv(row, axis_div);
+		const uint32_t along = row - outer * axis_div.d;
+		// operands are few: halve the table
+		uint32_t lo = 0, hi = tab.n;
+		while (hi - lo > 1)
+		{
+			uint32_t mid = (lo + hi) / 2;
+			if (tab.start[mid] <= along) { lo = mid; } else { hi = mid; }
+		}
+		const uint32_t extent = tab.start[lo + 1] - tab.start[lo];
+		const uint64_t from = ((uint64_t) outer * extent + (along - tab.start[lo])) * inner_vecs + within;
+		reinterpret_cast<Vec*>(dst)[idx] = reinterpret_cast<const Vec*>(tab.src[lo])[from];
+	}
+}
+
 } // namespace
 
 extern "C" {
@@ -625,12 +666,61 @@ int tcg_concat (tcg_ctx* ctx, int dtype, int axis, int nargs,
 		oshape[axis] += shapes[i * 8 + axis];
 	}
 	CHECK_DIMS(ctx, oshape, "tcg_concat");
+	for (int i = 0; i < nargs; ++i) { TCG_REQUIRE(ctx, ins[i], "tcg_concat: operand %d is NULL", i); }
+	// many operands (the outputs of an unrolled recurrent layer, one per step,
+	// cfg/tenncor/layer.yml:297-345, 716-768): one launch instead of one per operand
+	uint64_t inner = 1, outer = 1, total = 1;
+	for (int d = 0; d < 8; ++d)
+	{
+		total *= oshape[d];
+		if (d < axis) { inner *= oshape[d]; }
+		if (d > axis) { outer *= oshape[d]; }
+	}
+	const size_t esz = tcg_type_size(dtype);
+	if (nargs >= 3 && nargs <= CC_MAX && false == tcg_small_mode(ctx) && esz && total > 0 && total < (1ull << 32) &&
+		oshape[axis] < (1ull << 31))
+	{
+		ConcatTab tab;
+		tab.n = (uint32_t) nargs;
+		uint32_t at = 0;
+		// 16 bytes per lane when every row segment on both sides is aligned
+		uint64_t per = 16 / esz;
+		bool wide = inner % per == 0 && tcg_aligned16(out);
+		for (int i = 0; i < nargs; ++i)
+		{
+			tab.src[i] = ins[i];
+			tab.start[i] = at;
+			at += (uint32_t) shapes[i * 8 + axis];
+			wide = wide && tcg_aligned16(ins[i]);
+		}
+		tab.start[nargs] = at;
+		if (false == wide) { per = 1; }
+		const uint32_t inner_vecs = (uint32_t) (inner / per);
+		const uint32_t nvec = (uint32_t) (total / per);
+		const unsigned grid = tcg_grid(ctx, nvec, MV_BLOCK, 32);
+		const FastDiv idiv = make_fastdiv(inner_vecs), adiv = make_fastdiv((uint32_t) oshape[axis]);
+		if (wide)
+		{
+			concat_many_k<uint32_t,4><<<grid, MV_BLOCK, 0, ctx->stream>>>(tab, idiv, adiv, inner_vecs, nvec, (uint32_t*) out);
+		}
+		else
+		{
+			switch (esz)
+			{
+				case 1: concat_many_k<uint8_t,1><<<grid, MV_BLOCK, 0, ctx->stream>>>(tab, idiv, adiv, inner_vecs, nvec, (uint8_t*) out); break;
+				case 2: concat_many_k<uint16_t,1><<<grid, MV_BLOCK, 0, ctx->stream>>>(tab, idiv, adiv, inner_vecs, nvec, (uint16_t*) out); break;
+				case 4: concat_many_k<uint32_t,1><<<grid, MV_BLOCK, 0, ctx->stream>>>(tab, idiv, adiv, inner_vecs, nvec, (uint32_t*) out); break;
+				default: concat_many_k<uint64_t,1><<<grid, MV_BLOCK, 0, ctx->stream>>>(tab, idiv, adiv, inner_vecs, nvec, (uint64_t*) out); break;
+			}
+		}
+		TCG_LAUNCH_CHECK(ctx, "concat_many_k");
+		return TCG_OK;
+	}
 	int64_t os[8];
 	contiguous_strides(oshape, os);
 	uint64_t off = 0;
 	for (int i = 0; i < nargs; ++i)
 	{
-		TCG_REQUIRE(ctx, ins[i], "tcg_concat: operand %d is NULL", i);
 		const uint64_t* ishape = shapes + i * 8;
 		int64_t is[8];
 		contiguous_strides(ishape, is);

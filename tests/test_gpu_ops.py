@@ -498,6 +498,32 @@ def test_concat_bit_exact(ctx, ops, oracle):
     np.testing.assert_array_equal(out.get(), ref)
 
 
+@pytest.mark.parametrize("np_dtype", [np.float32, np.float64, np.int32])
+def test_concat_of_many_operands_is_one_pass(ctx, ops, oracle, np_dtype):
+    """Three operands and more are gathered by one launch through a table of
+    where each starts along the axis: equal and ragged extents, the axis first,
+    in the middle and last, rows that allow 16-byte accesses and rows that do not."""
+    rng = np.random.default_rng(seed_of("concat_many", str(np_dtype)))
+    cases = [
+        (1, [[512, 1, 6]] * 64),                                   # the outputs of 64 steps of a recurrent layer
+        (0, [[3, 5, 2], [1, 5, 2], [7, 5, 2], [4, 5, 2]]),         # ragged along the fastest dim
+        (2, [[6, 5, 1], [6, 5, 4], [6, 5, 2]]),                    # along the slowest dim
+        (1, [[8, 2, 3], [8, 1, 3], [8, 9, 3], [8, 1, 3], [8, 1, 3]]),
+        (1, [[5, k + 1, 3, 2] for k in range(17)]),                # odd rows: element by element
+    ]
+    for axis, shapes in cases:
+        from tenncor_amd import capi
+        xs = [(rng.integers(-1000, 1000, oracle.n_elems(s))).astype(np_dtype) for s in shapes]
+        ref, oshape = oracle.concat(xs, shapes, axis)
+        # (the node API only groups operands of extent 1 along the axis, cfg/ops.yml:613-653; the kernel takes any)
+        bufs = [ctx.upload(x) for x in xs]
+        out = ctx.empty(ref.size, np_dtype)
+        ctx.concat(capi.dtype_code(np_dtype), axis, [oracle.shape8(s) for s in shapes], [b.ptr for b in bufs], out.ptr)
+        np.testing.assert_array_equal(out.get(), ref, err_msg=str((axis, shapes[:2])))
+        for b in bufs + [out]:
+            b.release()
+
+
 MATMUL_CASES = [
     ([10, 3], [9, 10]), ([64, 64], [64, 64]), ([100, 37], [53, 100]), ([256, 128], [192, 256]),
     ([768, 256], [2048, 768]), ([32, 48, 5], [40, 32, 5]), ([128, 128, 3, 2], [128, 128, 3, 2]),
