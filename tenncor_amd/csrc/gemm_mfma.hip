@@ -411,6 +411,26 @@ __global__ __launch_bounds__(256) void gemm_split_sum_vec_k (const f32x4v* __res
 	}
 }
 
+// Many ranges over few results (a sliver of a result under a very long K): a
+// wave per group of four results; lane l adds the ranges l, l + 64, ... in
+// that order, then the 64 lane sums meet in a fixed tree
+__global__ __launch_bounds__(256) void gemm_split_sum_wave_k (const f32x4v* __restrict__ partial,
+	f32x4v* __restrict__ C, uint32_t splits, uint64_t per_split_vec)
+{
+	const uint64_t i = (uint64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+	const uint32_t lane = threadIdx.x & 63;
+	if (i >= per_split_vec) { return; }
+	f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+	for (uint32_t s = lane; s < splits; s += 64) { acc += partial[s * per_split_vec + i]; }
+#pragma unroll
+	for (int w = 32; w >= 1; w >>= 1)
+	{
+#pragma unroll
+		for (int e = 0; e < 4; ++e) { acc[e] += __shfl_xor(acc[e], w, 64); }
+	}
+	if (lane == 0) { C[i] = acc; }
+}
+
 template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs>
 int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1,
 	const SEGS& segs = SEGS())
@@ -455,7 +475,12 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	{
 		uint64_t n = batch * g.M * g.N;
 		bool dense = g.ldc == (int64_t) g.N && (batch == 1 || g.batch_c == (int64_t) g.M * g.N);
-		if (dense && n % 4 == 0 && tcg_aligned16(g.C))
+		if (dense && n % 4 == 0 && tcg_aligned16(g.C) && splits >= 32 && n / 4 <= 16384)
+		{
+			gemm_split_sum_wave_k<<<(unsigned) ((n / 4 + 3) / 4), 256, 0, ctx->stream>>>((const f32x4v*) g.partial,
+				(f32x4v*) g.C, splits, n / 4);
+		}
+		else if (dense && n % 4 == 0 && tcg_aligned16(g.C))
 		{
 			unsigned rgrid = tcg_grid(ctx, n / 4, 256, 8);
 			gemm_split_sum_vec_k<<<rgrid, 256, 0, ctx->stream>>>((const f32x4v*) g.partial, (f32x4v*) g.C, splits, n / 4);
