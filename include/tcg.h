@@ -411,6 +411,22 @@ int tcg_gemm (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	uint64_t batch, const void* A, uint64_t lda, uint64_t stride_a, int trans_a,
 	const void* B, uint64_t ldb, uint64_t stride_b, int trans_b,
 	void* C, uint64_t ldc, uint64_t stride_c);
+/* C = sum_t A_t B_t: `nterms` row-major products of one shape M x N x K with
+ * the flags of tcg_gemm, every term with operand addresses and leading dims of
+ * its own, as ONE product over the concatenated summed index where the
+ * matrix cores take the shape (fp32, 16-byte aligned operands, K a multiple
+ * of 16, at most 128 terms), else term by term in term order.  What
+ * tcg_contract_sum does for whole tensors, for operands that are parts of
+ * tensors: a contraction over a dim along which an operand is a CONCAT of
+ * tensors (cfg/tenncor/layer.yml:716-768 concatenates input and hidden state
+ * in front of the gate product) or an ADD of PADs that tile it (the gradient
+ * of the SLICEs that cut the gates back out, tenncor/eteq/backprop.hpp:402-421)
+ * reads the parts where they are, each with the rows of the other operand it
+ * meets.  C may be a block of a larger matrix (ldc). */
+int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K, int nterms,
+	const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b,
+	void* C, uint64_t ldc);
 /* CONV (cfg/ops.yml:566-607; internal/eigen/operator.hpp:1141-1187):
  * valid cross-correlation, kernel dim i slides along image dim ranks[i] */
 int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],

@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -132,6 +132,7 @@ def load():
         "tcg_contract": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_contract_sum": [vp, i32, u64p, u64p, i32, u64p, i32, vpp, vpp, vp],
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
+        "tcg_gemm_terms": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
@@ -445,6 +446,15 @@ class Context:
         self._check(self.lib.tcg_conv_dense_box(self.handle, dtype, _u64(shape8(imgshape)), _u64(shape8(kshape)),
                                                 len(r), _u64(r if r else [0]), _u64(img_box[0]), _u64(img_box[1]),
                                                 olo, ohi, box, kernel, dst))
+
+    def gemm_terms(self, dtype, M, N, K, a_ptrs, lda, trans_a, b_ptrs, ldb, trans_b, c, ldc):
+        """C = sum_t A_t B_t, every term with its own operand addresses and leading dims."""
+        n = len(a_ptrs)
+        pa = (ctypes.c_void_p * n)(*a_ptrs)
+        pb = (ctypes.c_void_p * n)(*b_ptrs)
+        la = (ctypes.c_uint64 * n)(*[int(v) for v in lda])
+        lb = (ctypes.c_uint64 * n)(*[int(v) for v in ldb])
+        self._check(self.lib.tcg_gemm_terms(self.handle, dtype, M, N, K, n, pa, la, int(trans_a), pb, lb, int(trans_b), c, ldc))
 
     def conv_views(self, dtype, imgshape, kshape, ranks, img_box, out_box, box, box_stride, kernel, kernel_stride,
                    dst, out_stride):

@@ -213,6 +213,21 @@ Operand classify (const uint64_t shape[8], const bool com[8])
 	return o;
 }
 
+// C[m][n] += T[m][n] for a C whose rows are ldc apart (terms of a sum of
+// products added in term order on the routes that compute term by term)
+template <typename T>
+__global__ __launch_bounds__(256) void add_rows_k (uint32_t M, uint32_t N, const T* __restrict__ term, T* __restrict__ C, int64_t ldc)
+{
+	const uint64_t total = (uint64_t) M * N;
+	for (uint64_t i = (uint64_t) blockIdx.x * 256 + threadIdx.x; i < total; i += (uint64_t) gridDim.x * 256)
+	{
+		const uint64_t m = i / N, n = i - m * N;
+		T& c = C[(int64_t) m * ldc + n];
+		if constexpr (is_int<T>::value) { c = (T) ((Wide<T>) c + (Wide<T>) term[i]); }
+		else { c = c + term[i]; }
+	}
+}
+
 } // namespace
 
 extern "C" {
@@ -442,6 +457,47 @@ int tcg_contract_sum (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 	}
 	if (term) { tcg_free(ctx, term, esz * M * N); }
 	return rc;
+}
+
+int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K, int nterms,
+	const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b,
+	void* C, uint64_t ldc)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, A && B && lda && ldb && C, "tcg_gemm_terms: NULL pointer");
+	TCG_REQUIRE(ctx, nterms >= 1, "tcg_gemm_terms: %d terms", nterms);
+	TCG_REQUIRE(ctx, ldc >= N, "tcg_gemm_terms: ldc %llu < N %llu", (unsigned long long) ldc, (unsigned long long) N);
+	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, A[t] && B[t], "tcg_gemm_terms: operand of term %d is NULL", t); }
+	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a sum of matrix products"); }
+	const size_t esz = tcg_type_size(dtype);
+	TCG_REQUIRE(ctx, esz != 0, "tcg_gemm_terms: unknown dtype %d", dtype);
+	if (M == 0 || N == 0) { return TCG_OK; }
+	if (dtype == TCG_FLOAT && nterms > 1)
+	{
+		bool handled = false;
+		int rc = tcg_gemm_f32_mfma_terms(ctx, M, N, K, (uint32_t) nterms, (const float* const*) A, lda, trans_a,
+			(const float* const*) B, ldb, trans_b, (float*) C, ldc, &handled);
+		if (rc != TCG_OK || handled) { return rc; }
+	}
+	// term by term, added up in term order
+	int rc = tcg_gemm(ctx, dtype, M, N, K, 1, A[0], lda[0], 0, trans_a, B[0], ldb[0], 0, trans_b, C, ldc, 0);
+	if (rc != TCG_OK || nterms == 1) { return rc; }
+	TCG_REQUIRE(ctx, M < (1ull << 31) && N < (1ull << 31), "tcg_gemm_terms: too large");
+	void* term = nullptr;
+	rc = tcg_alloc(ctx, esz * M * N, &term);
+	for (int t = 1; t < nterms && rc == TCG_OK; ++t)
+	{
+		rc = tcg_gemm(ctx, dtype, M, N, K, 1, A[t], lda[t], 0, trans_a, B[t], ldb[t], 0, trans_b, term, N, 0);
+		if (rc != TCG_OK) { break; }
+		const unsigned grid = tcg_grid(ctx, M * N, 256, 16);
+		TCG_DISPATCH_ALL(ctx, dtype, (add_rows_k<T><<<grid, 256, 0, ctx->stream>>>((uint32_t) M, (uint32_t) N,
+			(const T*) term, (T*) C, (int64_t) ldc)));
+	}
+	if (term) { tcg_free(ctx, term, esz * M * N); }
+	if (rc != TCG_OK) { return rc; }
+	TCG_LAUNCH_CHECK(ctx, "tcg_gemm_terms");
+	return TCG_OK;
 }
 
 } // extern "C"

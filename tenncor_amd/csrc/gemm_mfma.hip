@@ -55,6 +55,8 @@ struct GemmSegs
 	uint32_t k = 0; // columns of A (rows of B) per term
 	const float* a[MAX_TERMS];
 	const float* b[MAX_TERMS];
+	uint32_t lda[MAX_TERMS]; // the terms may lie in tensors of different row lengths
+	uint32_t ldb[MAX_TERMS];
 };
 
 struct NoSegs {};
@@ -189,11 +191,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 		const float* __restrict__ A = Abase;
 		const float* __restrict__ B = Bbase;
 		uint32_t kfirst = 0;
+		int64_t lda = g.lda, ldb = g.ldb;
 		if constexpr (SEG)
 		{
 			const uint32_t term = k0 / segs.k;
 			A = segs.a[term];
 			B = segs.b[term];
+			lda = segs.lda[term];
+			ldb = segs.ldb[term];
 			kfirst = term * segs.k;
 		}
 #pragma unroll
@@ -222,14 +227,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				// K contiguous: BK/4 lanes per row
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t m = m0 + mm, k = k0 + kq * 4;
-				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * g.lda + (k - kfirst)) : zero4;
+				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * lda + (k - kfirst)) : zero4;
 			}
 			else
 			{
 				// M contiguous: BM/4 lanes per k
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
 				uint32_t m = m0 + mq * 4, k = k0 + kk;
-				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) (k - kfirst) * g.lda + m) : zero4;
+				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) (k - kfirst) * lda + m) : zero4;
 			}
 		}
 #pragma unroll
@@ -242,14 +247,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				// N contiguous: BN/4 lanes per k
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
 				uint32_t n = n0 + nq * 4, k = k0 + kk;
-				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) (k - kfirst) * g.ldb + n) : zero4;
+				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) (k - kfirst) * ldb + n) : zero4;
 			}
 			else
 			{
 				// K contiguous: BK/4 lanes per n
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t n = n0 + nn, k = k0 + kq * 4;
-				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * g.ldb + (k - kfirst)) : zero4;
+				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * ldb + (k - kfirst)) : zero4;
 			}
 		}
 	};
@@ -504,9 +509,10 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 // 16 KW columns of K and wave q multiplies columns [16 q, 16 q + 16) of them.
 // At the end the KW partial blocks meet in LDS and are added in wave order, so
 // the sum does not depend on scheduling and no second kernel is needed.
-template <int TMW, int TNW, int KW, int KPW, bool TA, bool TB>
-__global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g)
+template <int TMW, int TNW, int KW, int KPW, bool TA, bool TB, typename SEGS = NoSegs>
+__global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 {
+	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value;
 	static_assert(TMW * TNW * KW == 4, "four waves");
 	constexpr int BM = 32 * TMW, BN = 32 * TNW, BKW = KPW * KW;
 	constexpr int KP = BKW + 4;
@@ -526,8 +532,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g)
 	const uint32_t t = id - bz * g.tiles_per_batch;
 	const uint32_t tm = t % g.tiles_m, tn = t / g.tiles_m;
 	const uint32_t m0 = tm * BM, n0 = tn * BN;
-	const float* __restrict__ A = g.A + (int64_t) bz * g.batch_a;
-	const float* __restrict__ B = g.B + (int64_t) bz * g.batch_b;
+	const float* __restrict__ Abase = g.A + (int64_t) bz * g.batch_a;
+	const float* __restrict__ Bbase = g.B + (int64_t) bz * g.batch_b;
 	float* __restrict__ C = g.C + (int64_t) bz * g.batch_c;
 
 	const int tid = threadIdx.x;
@@ -544,6 +550,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g)
 
 	auto load_round = [&] (uint32_t k0)
 	{
+		// with terms: a round never straddles two of them (their depth is a multiple of a round's)
+		const float* __restrict__ A = Abase;
+		const float* __restrict__ B = Bbase;
+		uint32_t kfirst = 0;
+		int64_t lda = g.lda, ldb = g.ldb;
+		if constexpr (SEG)
+		{
+			const uint32_t term = k0 / segs.k;
+			A = segs.a[term];
+			B = segs.b[term];
+			lda = segs.lda[term];
+			ldb = segs.ldb[term];
+			kfirst = term * segs.k;
+		}
 #pragma unroll
 		for (int v = 0; v < A_VEC; ++v)
 		{
@@ -553,13 +573,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g)
 			{
 				int mm = idx / (BKW / 4), kq = idx % (BKW / 4);
 				uint32_t m = m0 + mm, k = k0 + kq * 4;
-				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * g.lda + k) : zero4;
+				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * lda + (k - kfirst)) : zero4;
 			}
 			else
 			{
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
 				uint32_t m = m0 + mq * 4, k = k0 + kk;
-				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) k * g.lda + m) : zero4;
+				ra[v] = (m < g.M && k < g.K) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) (k - kfirst) * lda + m) : zero4;
 			}
 		}
 #pragma unroll
@@ -571,13 +591,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g)
 			{
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
 				uint32_t n = n0 + nq * 4, k = k0 + kk;
-				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) k * g.ldb + n) : zero4;
+				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) (k - kfirst) * ldb + n) : zero4;
 			}
 			else
 			{
 				int nn = idx / (BKW / 4), kq = idx % (BKW / 4);
 				uint32_t n = n0 + nn, k = k0 + kq * 4;
-				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * g.ldb + k) : zero4;
+				rb[v] = (n < g.N && k < g.K) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * ldb + (k - kfirst)) : zero4;
 			}
 		}
 	};
@@ -692,8 +712,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g)
 	}
 }
 
-template <int TMW, int TNW, int KW, int KPW>
-int launch_kw (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b)
+template <int TMW, int TNW, int KW, int KPW, typename SEGS = NoSegs>
+int launch_kw (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, const SEGS& segs = SEGS())
 {
 	GemmArgs g = base;
 	constexpr int BM = 32 * TMW, BN = 32 * TNW;
@@ -707,10 +727,10 @@ int launch_kw (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, 
 	g.k_per_split = g.K;
 	g.partial = nullptr;
 	const unsigned grid = g.total_tiles;
-	if (!trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
-	else if (!trans_a) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
-	else { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	if (!trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	else if (trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	else if (!trans_a) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	else { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	TCG_LAUNCH_CHECK(ctx, "gemm_mfma_kw");
 	return TCG_OK;
 }
@@ -789,30 +809,47 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 }
 
 // C[m][n] = sum_t sum_k A_t[m][k] B_t[k][n]: `terms` products of one shape
-// (K columns each, same layouts and leading dims) as one product of depth
-// terms * K; *handled = false when the shapes do not fit
-int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
-	const float* const* A, uint64_t lda, int trans_a, const float* const* B, uint64_t ldb, int trans_b,
+// (K columns each, same layouts; each term with its own leading dims) as one
+// product of depth terms * K; *handled = false when the shapes do not fit
+int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
+	const float* const* A, const uint64_t* lda, int trans_a, const float* const* B, const uint64_t* ldb, int trans_b,
 	float* C, uint64_t ldc, bool* handled)
 {
 	*handled = false;
 	bool ok = terms >= 1 && terms <= (uint32_t) MAX_TERMS && M >= 32 && N >= 32 && K >= BK && K % BK == 0 &&
 		M < (1ull << 31) && N < (1ull << 31) && K * terms < (1ull << 31) &&
-		lda % 4 == 0 && ldb % 4 == 0 && ((trans_a ? M : K) % 4 == 0) && ((trans_b ? K : N) % 4 == 0);
-	for (uint32_t t = 0; t < terms && ok; ++t) { ok = tcg_aligned16(A[t]) && tcg_aligned16(B[t]); }
+		((trans_a ? M : K) % 4 == 0) && ((trans_b ? K : N) % 4 == 0);
+	for (uint32_t t = 0; t < terms && ok; ++t)
+	{
+		ok = tcg_aligned16(A[t]) && tcg_aligned16(B[t]) && lda[t] % 4 == 0 && ldb[t] % 4 == 0 &&
+			lda[t] < (1ull << 32) && ldb[t] < (1ull << 32);
+	}
 	if (!ok) { return TCG_OK; }
 	GemmArgs g;
 	g.A = A[0]; g.B = B[0]; g.C = C;
 	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) (K * terms);
-	g.lda = (int64_t) lda; g.ldb = (int64_t) ldb; g.ldc = (int64_t) ldc;
+	g.lda = (int64_t) lda[0]; g.ldb = (int64_t) ldb[0]; g.ldc = (int64_t) ldc;
 	g.batch_a = g.batch_b = g.batch_c = 0;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	g.rows = g.sums = nullptr;
 	g.ncheck = 0;
 	GemmSegs segs;
 	segs.k = (uint32_t) K;
-	for (uint32_t t = 0; t < terms; ++t) { segs.a[t] = A[t]; segs.b[t] = B[t]; }
+	for (uint32_t t = 0; t < terms; ++t)
+	{
+		segs.a[t] = A[t];
+		segs.b[t] = B[t];
+		segs.lda[t] = (uint32_t) lda[t];
+		segs.ldb[t] = (uint32_t) ldb[t];
+	}
 	*handled = true;
+	// few results (a time step of a recurrent layer): the waves of a workgroup share K
+	const uint64_t cus = (uint64_t) ctx->num_cus;
+	if (!trans_a && !trans_b && K % 128 == 0 && g.K >= 256 && ((M + 31) / 32) * ((N + 31) / 32) >= cus &&
+		((M + 127) / 128) * ((N + 127) / 128) < cus)
+	{
+		return launch_kw<1,1,4,32,GemmSegs>(ctx, g, 1, trans_a, trans_b, segs);
+	}
 	// large tiles; ranges of the long summed index spread the tiles over the chip
 	uint64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
 	uint64_t splits = (2 * (uint64_t) ctx->num_cus + tiles - 1) / tiles;
@@ -820,6 +857,21 @@ int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uin
 	if (splits > 32) { splits = 32; }
 	if (splits < 2) { splits = 1; }
 	return launch<128,128,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) splits, segs);
+}
+
+int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
+	const float* const* A, uint64_t lda, int trans_a, const float* const* B, uint64_t ldb, int trans_b,
+	float* C, uint64_t ldc, bool* handled)
+{
+	*handled = false;
+	if (terms > (uint32_t) MAX_TERMS) { return TCG_OK; }
+	uint64_t ldas[MAX_TERMS], ldbs[MAX_TERMS];
+	for (uint32_t t = 0; t < terms; ++t)
+	{
+		ldas[t] = lda;
+		ldbs[t] = ldb;
+	}
+	return tcg_gemm_f32_mfma_terms(ctx, M, N, K, terms, A, ldas, trans_a, B, ldbs, trans_b, C, ldc, handled);
 }
 
 int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,

@@ -1307,3 +1307,81 @@ def test_device_generator_draws_anew_at_every_launch_of_a_recording(ctx, oracle)
         np.testing.assert_array_equal(out.get(), oracle.rand_uniform(lo, hi, seed, first_block=launch * 250))
     assert ctx.rand_state() == (seed, 1000)
     ctx.graph_destroy(graph)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32, np.float64])
+@pytest.mark.parametrize("case", ["forward", "transposed_weight", "weight_gradient_block", "odd"])
+def test_sum_of_products_over_parts_of_tensors(ctx, oracle, case, np_dtype):
+    """tcg_gemm_terms: a contraction over a dim along which an operand is a
+    concatenation, computed from the parts where they lie -- each term with its
+    own leading dim (a row slice of a [batch, seq, n] input has rows seq * n
+    apart), the other operand's rows taken by pointer offset, the result
+    written into a block of a wider matrix.  Against the product of the
+    materialised concatenation (int32 exactly; fp32 at 1e-4 of the oracle
+    accumulating in double; fp64 at 1e-12)."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of("gemm_terms", case, str(np_dtype)))
+    esz = np.dtype(np_dtype).itemsize
+
+    def draw(n):
+        if np_dtype == np.int32:
+            return rng.integers(-2000, 2000, n).astype(np.int32)
+        return (rng.standard_normal(n) / 8).astype(np_dtype)
+
+    if case == "forward":
+        # [x_t, h] . W with x_t a slice of x[batch][seq][nin]: three terms of K = 128
+        # (enough 32x32 blocks for the kernel whose waves share K)
+        batch, seq, nin, hid, N, t = 256, 5, 128, 256, 2048, 3
+        x, h, w = draw(batch * seq * nin), draw(batch * hid), draw((nin + hid) * N)
+        xt = x.reshape(batch, seq, nin)[:, t, :]
+        ref = np.concatenate([xt, h.reshape(batch, hid)], axis=1).astype(np.float64) @ w.reshape(nin + hid, N).astype(np.float64)
+        dx, dh, dw = ctx.upload(x), ctx.upload(h), ctx.upload(w)
+        K = 128
+        a = [dx.ptr + t * nin * esz, dh.ptr, dh.ptr + K * esz]
+        lda = [seq * nin, hid, hid]
+        b = [dw.ptr, dw.ptr + K * N * esz, dw.ptr + 2 * K * N * esz]
+        M, ldb, ta, tb, ldc, coff, cols = batch, [N] * 3, 0, 0, N, 0, N
+    elif case == "transposed_weight":
+        # sum_g dgate_g . W[:, g-th block]^T, only the columns 64.. of the result, into a wider buffer
+        batch, hid, rows = 64, 128, 192
+        gates = [draw(batch * hid) for _ in range(4)]
+        w = draw(rows * 4 * hid)
+        full = np.concatenate([g.reshape(batch, hid) for g in gates], axis=1).astype(np.float64) @ w.reshape(rows, 4 * hid).astype(np.float64).T
+        n0 = 64
+        ref = full[:, n0:]
+        dg = [ctx.upload(g) for g in gates]
+        dw = ctx.upload(w)
+        K, M, cols = hid, batch, rows - n0
+        a, lda = [d.ptr for d in dg], [hid] * 4
+        b = [dw.ptr + (n0 * 4 * hid + g * hid) * esz for g in range(4)]
+        ldb, ta, tb, ldc, coff = [4 * hid] * 4, 0, 1, rows, n0
+    elif case == "weight_gradient_block":
+        # sum_t h_t^T . dgate_t into the block (rows 32.., columns 128..) of dW
+        steps, batch, hid, gate = 6, 64, 96, 128
+        hs, gs = [draw(batch * hid) for _ in range(steps)], [draw(batch * gate) for _ in range(steps)]
+        ref = sum(h.reshape(batch, hid).astype(np.float64).T @ g.reshape(batch, gate).astype(np.float64) for h, g in zip(hs, gs))
+        dh, dgt = [ctx.upload(h) for h in hs], [ctx.upload(g) for g in gs]
+        K, M, cols = batch, hid, gate
+        a, lda, b, ldb = [d.ptr for d in dh], [hid] * steps, [d.ptr for d in dgt], [gate] * steps
+        ta, tb, ldc, coff = 1, 0, 384, 32 * 384 + 128
+    else:
+        # nothing aligned: term by term on the generic kernels
+        M, cols, K = 7, 9, 5
+        As, Bs = [draw(M * K) for _ in range(3)], [draw(K * cols) for _ in range(3)]
+        ref = sum(x.reshape(M, K).astype(np.float64) @ y.reshape(K, cols).astype(np.float64) for x, y in zip(As, Bs))
+        da, db = [ctx.upload(x) for x in As], [ctx.upload(y) for y in Bs]
+        a, lda, b, ldb, ta, tb, ldc, coff = [d.ptr for d in da], [K] * 3, [d.ptr for d in db], [cols] * 3, 0, 0, cols + 3, 1
+    rows_c = M + (2 if case == "weight_gradient_block" else 0) + 40
+    out = ctx.upload(np.full(rows_c * ldc + 8, 777, dtype=np_dtype))
+    ctx.gemm_terms(capi.dtype_code(np_dtype), M, cols, K, a, lda, ta, b, ldb, tb, out.ptr + coff * esz, ldc)
+    got = out.get()
+    block = np.array([got[coff + m * ldc: coff + m * ldc + cols] for m in range(M)])
+    if np_dtype == np.int32:
+        np.testing.assert_array_equal(block, ref.astype(np.int64).astype(np.int32))
+    else:
+        assert_acc_close(block, ref, ACC_RTOL if np_dtype == np.float32 else 1e-12)
+    # nothing outside the block was written
+    mask = np.ones(got.size, bool)
+    for m in range(M):
+        mask[coff + m * ldc: coff + m * ldc + cols] = False
+    assert (got[mask] == 777).all()
