@@ -510,10 +510,11 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 // At the end the KW partial blocks meet in LDS and are added in wave order, so
 // the sum does not depend on scheduling and no second kernel is needed.
 template <int TMW, int TNW, int KW, int KPW, bool TA, bool TB, typename SEGS = NoSegs>
-__global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
+__global__ __launch_bounds__(64 * TMW * TNW * KW) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 {
 	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value;
-	static_assert(TMW * TNW * KW == 4, "four waves");
+	constexpr int NT = 64 * TMW * TNW * KW; // threads of a workgroup
+	static_assert(NT == 256 || NT == 512, "four or eight waves");
 	constexpr int BM = 32 * TMW, BN = 32 * TNW, BKW = KPW * KW;
 	constexpr int KP = BKW + 4;
 	constexpr int AP = TA ? BM + 4 : KP;
@@ -521,7 +522,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 	constexpr int A_SIZE = TA ? BKW * AP : BM * AP;
 	constexpr int B_SIZE = TB ? BN * BP : BKW * BP;
 	constexpr int A_CHUNKS = BM * BKW / 4, B_CHUNKS = BN * BKW / 4;
-	constexpr int A_VEC = (A_CHUNKS + 255) / 256, B_VEC = (B_CHUNKS + 255) / 256;
+	constexpr int A_VEC = (A_CHUNKS + NT - 1) / NT, B_VEC = (B_CHUNKS + NT - 1) / NT;
 	constexpr int RED = (KW - 1) * TMW * TNW * 1024; // partial blocks parked for the final sum
 	constexpr int STAGE = 2 * (A_SIZE + B_SIZE);
 	__shared__ __attribute__((aligned(16))) float lds[STAGE > RED ? STAGE : RED];
@@ -567,8 +568,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 #pragma unroll
 		for (int v = 0; v < A_VEC; ++v)
 		{
-			int idx = tid + v * 256;
-			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			int idx = tid + v * NT;
+			if (A_CHUNKS % NT != 0 && idx >= A_CHUNKS) { break; }
 			if constexpr (!TA)
 			{
 				int mm = idx / (BKW / 4), kq = idx % (BKW / 4);
@@ -585,8 +586,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 #pragma unroll
 		for (int v = 0; v < B_VEC; ++v)
 		{
-			int idx = tid + v * 256;
-			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			int idx = tid + v * NT;
+			if (B_CHUNKS % NT != 0 && idx >= B_CHUNKS) { break; }
 			if constexpr (!TB)
 			{
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
@@ -609,8 +610,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 #pragma unroll
 		for (int v = 0; v < A_VEC; ++v)
 		{
-			int idx = tid + v * 256;
-			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			int idx = tid + v * NT;
+			if (A_CHUNKS % NT != 0 && idx >= A_CHUNKS) { break; }
 			if constexpr (!TA)
 			{
 				int mm = idx / (BKW / 4), kq = idx % (BKW / 4);
@@ -625,8 +626,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kw_k (GemmArgs g, SEGS segs)
 #pragma unroll
 		for (int v = 0; v < B_VEC; ++v)
 		{
-			int idx = tid + v * 256;
-			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			int idx = tid + v * NT;
+			if (B_CHUNKS % NT != 0 && idx >= B_CHUNKS) { break; }
 			if constexpr (!TB)
 			{
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
@@ -716,7 +717,7 @@ template <int TMW, int TNW, int KW, int KPW, typename SEGS = NoSegs>
 int launch_kw (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, const SEGS& segs = SEGS())
 {
 	GemmArgs g = base;
-	constexpr int BM = 32 * TMW, BN = 32 * TNW;
+	constexpr int BM = 32 * TMW, BN = 32 * TNW, NT = 64 * TMW * TNW * KW;
 	uint64_t tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
 	uint64_t total = tiles_m * tiles_n * batch;
 	TCG_REQUIRE(ctx, total < (1ull << 31), "tcg_gemm: too many tiles for one launch");
@@ -727,10 +728,10 @@ int launch_kw (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, 
 	g.k_per_split = g.K;
 	g.partial = nullptr;
 	const unsigned grid = g.total_tiles;
-	if (!trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-	else if (trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-	else if (!trans_a) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-	else { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	if (!trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,false,SEGS><<<grid, NT, 0, ctx->stream>>>(g, segs); }
+	else if (trans_a && !trans_b) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,false,SEGS><<<grid, NT, 0, ctx->stream>>>(g, segs); }
+	else if (!trans_a) { gemm_mfma_kw_k<TMW,TNW,KW,KPW,false,true,SEGS><<<grid, NT, 0, ctx->stream>>>(g, segs); }
+	else { gemm_mfma_kw_k<TMW,TNW,KW,KPW,true,true,SEGS><<<grid, NT, 0, ctx->stream>>>(g, segs); }
 	TCG_LAUNCH_CHECK(ctx, "gemm_mfma_kw");
 	return TCG_OK;
 }
@@ -852,6 +853,16 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 	}
 	// large tiles; ranges of the long summed index spread the tiles over the chip
 	uint64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+	if (tiles * (g.K / 256 < 32 ? g.K / 256 : 32) < cus)
+	{
+		// not enough of them even so: smaller tiles, ranges as for a plain product of this shape
+		uint64_t small = ((M + 63) / 64) * ((N + 63) / 64);
+		uint64_t ranges = 2 * cus / small;
+		if (ranges > g.K / 64) { ranges = g.K / 64; }
+		if (ranges > 32) { ranges = 32; }
+		if (ranges < 2) { ranges = 1; }
+		return launch<64,64,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) ranges, segs);
+	}
 	uint64_t splits = (2 * (uint64_t) ctx->num_cus + tiles - 1) / tiles;
 	if (splits > g.K / 256) { splits = g.K / 256; }
 	if (splits > 32) { splits = 32; }

@@ -100,6 +100,46 @@ struct ViewedConv final
 	std::string label;               ///< the nodes this launch stands for, for printing
 };
 
+/// Matrix products over operands that are parts of tensors, launched as
+/// tcg_gemm_terms calls into one node's buffer.  A contraction over a dim
+/// along which an operand is a concatenation -- a CONCAT (the input and the
+/// hidden state in front of the gate product of a recurrent cell,
+/// cfg/tenncor/layer.yml:716-768) or an ADD of PADs that tile the dim (the
+/// gradient of the SLICEs that cut the gates back out,
+/// tenncor/eteq/backprop.hpp:402-421) -- is the sum of the products of the
+/// parts with the rows of the other operand they meet; a sum of products
+/// whose operands are concatenations along a dim that survives (the weight
+/// gradient of such a cell) falls into blocks of the result, one sum of
+/// products per pair of parts.  Where products are all that read such a
+/// concatenation it is never laid out.
+struct PartProducts final
+{
+	struct Term final
+	{
+		teq::iTensor* a = nullptr;  ///< materialised tensors the operands are read from,
+		teq::iTensor* b = nullptr;
+		int64_t a_off = 0, b_off = 0; ///< element offsets of A_t(0, 0) and B_t(0, 0) in them
+		uint64_t lda = 0, ldb = 0;
+	};
+
+	/// C[c_off + m * ldc + n] = sum_t sum_k A_t(m, k) B_t(k, n), flags as tcg_gemm
+	struct Product final
+	{
+		uint64_t M = 0, N = 0, K = 0;
+		bool trans_a = false, trans_b = false;
+		std::vector<Term> terms;
+		int64_t c_off = 0;
+		uint64_t ldc = 0;
+	};
+
+	Observable* node = nullptr;      ///< receives the results
+	int dtype = 0;
+	std::vector<Product> products;
+	bool partial = false;            ///< only the window its SLICE readers look at is computed
+	std::vector<teq::iTensor*> reads;
+	std::string label;
+};
+
 struct FusionPlan final
 {
 	struct Step final
@@ -108,13 +148,15 @@ struct FusionPlan final
 		int group = -1;             ///< index into groups, or
 		int contract = -1;          ///< index into contracts, or
 		int conv = -1;              ///< index into convs, or
-		int sum = -1;               ///< index into sums
+		int sum = -1;               ///< index into sums, or
+		int parts = -1;             ///< index into part_products
 	};
 
 	std::vector<FusedGroup> groups;
 	std::vector<SwappedContract> contracts;
 	std::vector<ViewedConv> convs;
 	std::vector<SummedContracts> sums;
+	std::vector<PartProducts> part_products;
 	std::vector<Step> steps;
 	/// functors that are computed inside a group or folded into operand views
 	/// and therefore never hold a value of their own
@@ -133,6 +175,8 @@ void launch_contract (const SwappedContract& call, const teq::TensSetT& targets,
 void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMemptrT& memory);
+
+void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
 }
 

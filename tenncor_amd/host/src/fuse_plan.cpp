@@ -51,6 +51,8 @@ struct Node final
 	int conv_from = -1;         // this node receives the result of that CONV node, launched over views (itself, or the end of a chain behind it)
 	bool through_conv = false;  // PAD / PERMUTE / REVERSE that only such convolutions read through, or
 	                            // a node between such a CONV and the node that receives its result
+	bool parts_folded = false;  // CONCAT / ADD of PADs that only products read, part by part
+	int part_products = -1;     // CONTRACT, or ADD over CONTRACT terms, launched as products over parts (index into part_calls_)
 	bool summed = false;        // ADD launched as one sum of the products it adds
 	bool summed_term = false;   // CONTRACT / PERMUTE that is a term of such a sum
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
@@ -216,6 +218,7 @@ struct Planner final
 				n.absorbed = false;
 			}
 		}
+		find_part_products();
 		for (Node& n : nodes_)
 		{
 			for (int a : n.args)
@@ -388,6 +391,512 @@ struct Planner final
 				nodes_[last].kind = OTHER;
 			}
 			nodes_[last].conv_from = kv.first;
+		}
+	}
+
+	// ---- products over the parts of concatenations ----
+
+	struct Part final
+	{
+		uint64_t start = 0, extent = 0; // along the axis of the concatenation
+		View view;                      // of the part, in its own coordinates
+	};
+
+	struct Parts final
+	{
+		int axis = 0;
+		std::vector<Part> parts;
+	};
+
+	/// A matrix seen in a view: element (f, k) at base[off + f * sf + k * sk]
+	struct Mat final
+	{
+		teq::iTensor* base = nullptr;
+		int64_t off = 0, sf = 0, sk = 0;
+		uint64_t F = 1, K = 1;
+	};
+
+	/// Node z as a concatenation of views along one dim: a CONCAT, or an ADD of
+	/// PADs (each read by the ADD alone) that tile one dim without overlap
+	bool concat_parts (int z, Parts& out)
+	{
+		const Node& n = nodes_[z];
+		if (n.kind != EW || n.target || n.args.size() < 2 || n.consumers.empty()) { return false; }
+		out.parts.clear();
+		if (n.op == egen::CONCAT)
+		{
+			teq::RankT axis = 0;
+			Packer<teq::RankT>().unpack(axis, *n.f);
+			if (axis >= 8) { return false; }
+			out.axis = axis;
+			uint64_t at = 0;
+			for (size_t k = 0; k < n.args.size(); ++k)
+			{
+				Part part;
+				part.start = at;
+				part.extent = shape8(n.arg_tens[k]->shape())[axis];
+				part.view = view_of_arg(z, k);
+				at += part.extent;
+				out.parts.push_back(part);
+			}
+		}
+		else if (n.op == egen::ADD)
+		{
+			int axis = -1;
+			for (size_t k = 0; k < n.args.size(); ++k)
+			{
+				int a = n.args[k];
+				if (a < 0) { return false; }
+				const Node& pad = nodes_[a];
+				if (pad.op != egen::PAD || pad.kind != VIEW || false == pad.absorbed || pad.consumers.size() != 1) { return false; }
+				PairVecT<teq::DimT> encoding;
+				Packer<PairVecT<teq::DimT>>().unpack(encoding, *pad.f);
+				Part part;
+				int padded = -1;
+				for (size_t d = 0, m = std::min(encoding.size(), (size_t) 8); d < m; ++d)
+				{
+					if (encoding[d].first == 0 && encoding[d].second == 0) { continue; }
+					if (padded >= 0) { return false; }
+					padded = (int) d;
+					part.start = encoding[d].first;
+				}
+				if (padded < 0 || (axis >= 0 && padded != axis)) { return false; }
+				axis = padded;
+				part.extent = shape8(pad.arg_tens[0]->shape())[axis];
+				part.view = view_of_arg(a, 0);
+				out.parts.push_back(part);
+			}
+			out.axis = axis;
+			std::sort(out.parts.begin(), out.parts.end(), [](const Part& x, const Part& y) { return x.start < y.start; });
+			uint64_t at = 0;
+			for (const Part& part : out.parts)
+			{
+				if (part.start != at) { return false; }
+				at += part.extent;
+			}
+			if (at != n.shape[axis]) { return false; }
+		}
+		else { return false; }
+		// the views beneath are counted as read with the products: nothing else may read through them
+		for (int a : n.args)
+		{
+			if (a >= 0 && false == sole_chain(a)) { return false; }
+		}
+		// parts that are whole values: no zero border inside them
+		for (const Part& part : out.parts)
+		{
+			Shape8 pshape = n.shape;
+			pshape[out.axis] = part.extent;
+			for (int d = 0; d < 8; ++d)
+			{
+				if (part.view.lo[d] != 0 || part.view.hi[d] != pshape[d]) { return false; }
+			}
+		}
+		return true;
+	}
+
+	/// Folded views from node a down, each with one reader
+	bool sole_chain (int a) const
+	{
+		const Node& n = nodes_[a];
+		if (false == (n.kind == VIEW && n.absorbed)) { return true; }
+		if (n.consumers.size() != 1 || n.target || n.op == egen::REVERSE) { return false; }
+		for (int b : n.args)
+		{
+			if (b >= 0 && false == sole_chain(b)) { return false; }
+		}
+		return true;
+	}
+
+	/// A view of extents `shape` with contracted dim `cdim` as a matrix; false
+	/// when more than one other dim is significant
+	static bool as_matrix (const View& v, const Shape8& shape, int cdim, Mat& out)
+	{
+		out = Mat();
+		out.base = v.base;
+		out.off = v.off;
+		out.K = shape[cdim];
+		out.sk = v.stride[cdim];
+		int fdim = -1;
+		for (int d = 0; d < 8; ++d)
+		{
+			if (d == cdim || shape[d] == 1) { continue; }
+			if (fdim >= 0) { return false; }
+			fdim = d;
+		}
+		if (fdim >= 0)
+		{
+			out.F = shape[fdim];
+			out.sf = v.stride[fdim];
+		}
+		return true;
+	}
+
+	/// One side of a product: the operand as one matrix, or as the matrices of
+	/// its parts when it is a concatenation that is being folded
+	struct Side final
+	{
+		int cdim = 0;
+		int z = -1;              // folded concatenation, -1: a plain operand
+		bool along_k = false;    // the parts split the contracted dim (else the surviving one)
+		std::vector<Mat> mats;   // one per part (one in all for a plain operand)
+		std::vector<uint64_t> starts;
+	};
+
+	bool make_side (int c, size_t k, int cdim, const std::set<int>& folded, Side& out)
+	{
+		const Node& n = nodes_[c];
+		out = Side();
+		out.cdim = cdim;
+		int a = n.args[k];
+		Shape8 shape = shape8(n.arg_tens[k]->shape());
+		if (a >= 0 && folded.count(a))
+		{
+			const Parts& parts = part_lists_.at(a);
+			out.z = a;
+			out.along_k = parts.axis == cdim;
+			for (const Part& part : parts.parts)
+			{
+				Shape8 pshape = shape;
+				pshape[parts.axis] = part.extent;
+				Mat m;
+				if (false == as_matrix(part.view, pshape, cdim, m)) { return false; }
+				// the axis must be the contracted dim or the one that survives
+				if (false == out.along_k && (shape[parts.axis] == 1)) { return false; }
+				out.mats.push_back(m);
+				out.starts.push_back(part.start);
+			}
+			if (false == out.along_k)
+			{
+				// the surviving dim must be the axis
+				int fdim = -1;
+				for (int d = 0; d < 8; ++d)
+				{
+					if (d != cdim && shape[d] > 1) { fdim = d; }
+				}
+				if (fdim != parts.axis) { return false; }
+			}
+			return true;
+		}
+		if (a >= 0 && nodes_[a].kind == VIEW && nodes_[a].absorbed) { return false; }
+		Mat m;
+		if (false == as_matrix(dense_view(n.arg_tens[k].get(), shape), shape, cdim, m)) { return false; }
+		out.mats.push_back(m);
+		out.starts.push_back(0);
+		return true;
+	}
+
+	static uint64_t gcd64 (uint64_t x, uint64_t y)
+	{
+		while (y)
+		{
+			uint64_t r = x % y;
+			x = y;
+			y = r;
+		}
+		return x;
+	}
+
+	/// Layout flags and leading dims of one term; false when the matrices do not
+	/// lie the way the product kernels read them
+	static bool term_layout (const Mat& a, const Mat& b, bool& trans_a, bool& trans_b, PartProducts::Term& term)
+	{
+		term.a = a.base;
+		term.b = b.base;
+		term.a_off = a.off;
+		term.b_off = b.off;
+		// A(m, k) at m * sf + k * sk; B(k, n) at k * sk + n * sf
+		if (a.sk == 1 && (a.F == 1 || a.sf >= (int64_t) a.K)) { trans_a = false; term.lda = a.F == 1 ? a.K : (uint64_t) a.sf; }
+		else if (a.sf == 1 && a.sk >= (int64_t) a.F) { trans_a = true; term.lda = (uint64_t) a.sk; }
+		else { return false; }
+		if (b.sf == 1 && b.sk >= (int64_t) b.F) { trans_b = false; term.ldb = (uint64_t) b.sk; }
+		else if (b.sk == 1 && (b.F == 1 || b.sf >= (int64_t) b.K)) { trans_b = true; term.ldb = b.F == 1 ? b.K : (uint64_t) b.sf; }
+		else { return false; }
+		return true;
+	}
+
+	/// Whether the matrix cores take the product (else the terms would be launched one by one)
+	static bool fast_shape (const PartProducts::Product& p)
+	{
+		bool ok = p.terms.size() >= 1 && p.terms.size() <= 128 && p.M >= 32 && p.N >= 32 && p.K >= 16 && p.K % 16 == 0 &&
+			(p.trans_a ? p.M : p.K) % 4 == 0 && (p.trans_b ? p.K : p.N) % 4 == 0 && p.c_off % 4 == 0 && p.ldc % 4 == 0;
+		for (const PartProducts::Term& t : p.terms)
+		{
+			ok = ok && t.a_off % 4 == 0 && t.b_off % 4 == 0 && t.lda % 4 == 0 && t.ldb % 4 == 0;
+		}
+		return ok;
+	}
+
+	/// The contraction dims of CONTRACT node c when it is a product of two
+	/// matrices over one pair of dims
+	bool single_pair (int c, int& adim, int& bdim) const
+	{
+		const Node& n = nodes_[c];
+		if ((n.op != egen::CONTRACT && n.op != egen::MATMUL) || n.args.size() != 2) { return false; }
+		PairVecT<teq::RankT> dims;
+		if (n.op == egen::MATMUL) { dims.push_back({0, 1}); } // cfg/ops.yml:507-513: dim 0 of a meets dim 1 of b
+		else { Packer<PairVecT<teq::RankT>>().unpack(dims, *n.f); }
+		// pairs of dims of extent 1 change nothing
+		Shape8 ashape = shape8(n.arg_tens[0]->shape()), bshape = shape8(n.arg_tens[1]->shape());
+		int found = 0;
+		for (auto& pr : dims)
+		{
+			if (pr.first >= 8 || pr.second >= 8) { return false; }
+			if (ashape[pr.first] == 1 && bshape[pr.second] == 1) { continue; }
+			adim = pr.first;
+			bdim = pr.second;
+			++found;
+		}
+		return found == 1;
+	}
+
+	/// CONTRACT node c (launched on its own) over the parts of its operands
+	bool terms_of_contract (int c, const std::set<int>& folded, PartProducts& out)
+	{
+		const Node& n = nodes_[c];
+		int adim = 0, bdim = 0;
+		if (n.kind != OTHER || n.dtype != egen::FLOAT || false == single_pair(c, adim, bdim)) { return false; }
+		if (n.f->shape().n_elems() <= 4096) { return false; }
+		Side sa, sb;
+		if (false == make_side(c, 0, adim, folded, sa) || false == make_side(c, 1, bdim, folded, sb)) { return false; }
+		// exactly one side split along the contracted dim, the other one whole
+		const bool a_parts = sa.z >= 0, b_parts = sb.z >= 0;
+		if (a_parts == b_parts) { return false; }
+		const Side& split = a_parts ? sa : sb;
+		const Side& whole = a_parts ? sb : sa;
+		if (false == split.along_k) { return false; }
+		uint64_t chunk = 0;
+		for (const Mat& m : split.mats) { chunk = gcd64(chunk, m.K); }
+		if (chunk == 0) { return false; }
+		PartProducts::Product prod;
+		const Mat& w = whole.mats[0];
+		prod.M = sa.mats[0].F;
+		prod.N = sb.mats[0].F;
+		prod.K = chunk;
+		prod.ldc = prod.N;
+		// the columns (rows) the SLICEs that are all that read the result look at
+		uint64_t m0 = 0, n0 = 0;
+		Shape8 olo, ohi;
+		out.partial = false == n.target && slices_window(n.f, n.f->shape(), olo, ohi);
+		// the result holds b's surviving dim before a's (cfg/ops.yml:547-565)
+		int sig[2] = {-1, -1}, nsig = 0;
+		for (int d = 0; d < 8; ++d)
+		{
+			if (n.shape[d] > 1)
+			{
+				if (nsig < 2) { sig[nsig] = d; }
+				++nsig;
+			}
+		}
+		if (nsig != 2 || n.shape[sig[0]] != prod.N || n.shape[sig[1]] != prod.M) { return false; }
+		if (out.partial)
+		{
+			n0 = olo[sig[0]];
+			m0 = olo[sig[1]];
+			prod.N = ohi[sig[0]] - n0;
+			prod.M = ohi[sig[1]] - m0;
+			out.partial = prod.N < n.shape[sig[0]] || prod.M < n.shape[sig[1]];
+		}
+		prod.c_off = (int64_t) (m0 * prod.ldc + n0);
+		bool first = true;
+		for (size_t p = 0; p < split.mats.size(); ++p)
+		{
+			for (uint64_t k0 = 0; k0 < split.mats[p].K; k0 += chunk)
+			{
+				Mat ma = a_parts ? split.mats[p] : w, mb = a_parts ? w : split.mats[p];
+				Mat& part = a_parts ? ma : mb;
+				Mat& other = a_parts ? mb : ma;
+				part.off += (int64_t) k0 * part.sk;
+				other.off += (int64_t) (split.starts[p] + k0) * other.sk;
+				ma.K = mb.K = chunk;
+				ma.off += (int64_t) m0 * ma.sf;
+				mb.off += (int64_t) n0 * mb.sf;
+				ma.F = prod.M;
+				mb.F = prod.N;
+				PartProducts::Term term;
+				bool ta = false, tb = false;
+				if (false == term_layout(ma, mb, ta, tb, term)) { return false; }
+				if (false == first && (ta != prod.trans_a || tb != prod.trans_b)) { return false; }
+				prod.trans_a = ta;
+				prod.trans_b = tb;
+				first = false;
+				prod.terms.push_back(term);
+			}
+		}
+		if (false == fast_shape(prod)) { return false; }
+		out.node = n.f;
+		out.dtype = n.dtype;
+		out.products = {prod};
+		out.label = "parts " + nodes_[split.z].f->get_opcode().name_ + "+" + n.f->get_opcode().name_ + " x" + std::to_string(prod.terms.size()) +
+			(out.partial ? "+SLICE" : "");
+		return true;
+	}
+
+	/// ADD node s launched as one sum of products (find_summed_products) whose
+	/// terms' operands are concatenations along the dims that survive: one sum
+	/// of products per block of the result
+	bool blocks_of_sum (int s, const std::set<int>& folded, PartProducts& out)
+	{
+		const Node& n = nodes_[s];
+		if (false == n.summed || n.dtype != egen::FLOAT) { return false; }
+		PartProducts::Product proto;
+		std::vector<std::vector<PartProducts::Product>> blocks; // [part of a][part of b]
+		bool any_parts = false;
+		for (size_t t = 0; t < n.args.size(); ++t)
+		{
+			int arg = n.args[t];
+			const bool swapped = nodes_[arg].op == egen::PERMUTE;
+			int c = swapped ? nodes_[arg].args[0] : arg;
+			int adim = 0, bdim = 0;
+			if (false == single_pair(c, adim, bdim)) { return false; }
+			Side s0, s1;
+			if (false == make_side(c, 0, adim, folded, s0) || false == make_side(c, 1, bdim, folded, s1)) { return false; }
+			// the product as launched: operands exchanged under a PERMUTE{1,0}
+			const Side& sa = swapped ? s1 : s0;
+			const Side& sb = swapped ? s0 : s1;
+			if ((sa.z >= 0 && sa.along_k) || (sb.z >= 0 && sb.along_k)) { return false; }
+			any_parts = any_parts || sa.z >= 0 || sb.z >= 0;
+			if (t == 0)
+			{
+				blocks.assign(sa.mats.size(), std::vector<PartProducts::Product>(sb.mats.size()));
+				uint64_t nfull = 0;
+				for (const Mat& m : sb.mats) { nfull += m.F; }
+				for (size_t i = 0; i < sa.mats.size(); ++i)
+				{
+					for (size_t j = 0; j < sb.mats.size(); ++j)
+					{
+						PartProducts::Product& p = blocks[i][j];
+						p.M = sa.mats[i].F;
+						p.N = sb.mats[j].F;
+						p.K = sa.mats[i].K;
+						p.ldc = nfull;
+						p.c_off = (int64_t) (sa.starts[i] * nfull + sb.starts[j]);
+					}
+				}
+			}
+			if (blocks.size() != sa.mats.size() || blocks[0].size() != sb.mats.size()) { return false; }
+			for (size_t i = 0; i < sa.mats.size(); ++i)
+			{
+				for (size_t j = 0; j < sb.mats.size(); ++j)
+				{
+					PartProducts::Product& p = blocks[i][j];
+					if (p.M != sa.mats[i].F || p.N != sb.mats[j].F || p.K != sa.mats[i].K || p.K != sb.mats[j].K) { return false; }
+					PartProducts::Term term;
+					bool ta = false, tb = false;
+					if (false == term_layout(sa.mats[i], sb.mats[j], ta, tb, term)) { return false; }
+					if (t > 0 && (ta != p.trans_a || tb != p.trans_b)) { return false; }
+					p.trans_a = ta;
+					p.trans_b = tb;
+					p.terms.push_back(term);
+				}
+			}
+		}
+		if (false == any_parts) { return false; }
+		out.node = n.f;
+		out.dtype = n.dtype;
+		out.partial = false;
+		out.products.clear();
+		for (auto& row : blocks)
+		{
+			for (auto& p : row)
+			{
+				if (false == fast_shape(p)) { return false; }
+				out.products.push_back(p);
+			}
+		}
+		out.label = "blocks CONTRACT x" + std::to_string(n.args.size()) + " " + std::to_string(blocks.size()) + "x" +
+			std::to_string(blocks[0].size());
+		return true;
+	}
+
+	/// The product that reads concatenation z through consumer c: c itself, or
+	/// the sum c is a term of; -1 when c is neither
+	int product_reading (int c) const
+	{
+		const Node& n = nodes_[c];
+		if (n.op != egen::CONTRACT && n.op != egen::MATMUL) { return -1; }
+		if (false == n.summed_term) { return n.kind == OTHER ? c : -1; }
+		// a term of a sum: the CONTRACT itself or the PERMUTE over it is an operand of the ADD
+		int up = c;
+		for (int hop = 0; hop < 2; ++hop)
+		{
+			if (nodes_[up].consumers.size() != 1) { return -1; }
+			up = nodes_[up].consumers[0];
+			if (nodes_[up].summed) { return up; }
+		}
+		return -1;
+	}
+
+	void find_part_products (void)
+	{
+		std::set<int> folded;
+		for (size_t z = 0; z < nodes_.size(); ++z)
+		{
+			Parts parts;
+			if (concat_parts((int) z, parts))
+			{
+				part_lists_.emplace((int) z, parts);
+				folded.insert((int) z);
+			}
+		}
+		// a concatenation is folded when every reader is a product that takes it
+		// part by part; dropping one may undo products that leaned on it as well
+		std::map<int,PartProducts> calls;
+		for (bool changed = true; changed;)
+		{
+			changed = false;
+			calls.clear();
+			if (folded.empty()) { break; }
+			std::set<int> failed;
+			std::set<int> products;
+			for (int z : folded)
+			{
+				for (int c : nodes_[z].consumers)
+				{
+					int p = product_reading(c);
+					if (p < 0) { failed.insert(z); }
+					else { products.insert(p); }
+				}
+			}
+			for (int p : products)
+			{
+				PartProducts call;
+				bool ok = nodes_[p].summed ? blocks_of_sum(p, folded, call) : terms_of_contract(p, folded, call);
+				// the launch stands where the product does: nothing may rewrite what the parts show in between
+				if (ok) { calls.emplace(p, call); }
+			}
+			for (int z : folded)
+			{
+				for (int c : nodes_[z].consumers)
+				{
+					int p = product_reading(c);
+					if (p < 0 || 0 == calls.count(p)) { failed.insert(z); continue; }
+					std::vector<size_t> all(nodes_[z].args.size());
+					bool rewritten = false;
+					for (size_t k = 0; k < nodes_[z].args.size(); ++k)
+					{
+						rewritten = rewritten || written_between(z, {k}, (int) z, p);
+					}
+					if (rewritten) { failed.insert(z); }
+				}
+			}
+			for (int z : failed)
+			{
+				folded.erase(z);
+				changed = true;
+			}
+		}
+		for (int z : folded)
+		{
+			Node& n = nodes_[z];
+			n.kind = VIEW;
+			n.absorbed = true;
+			n.parts_folded = true;
+		}
+		for (auto& kv : calls)
+		{
+			nodes_[kv.first].part_products = (int) part_calls_.size();
+			part_calls_.push_back(kv.second);
 		}
 	}
 
@@ -1149,6 +1658,7 @@ struct Planner final
 		std::vector<bool> done(nodes_.size(), false);
 		std::map<int,int> last_user; // folded view -> last group reading through it
 		std::map<int,int> last_conv; // PAD read in place -> last convolution of its operand
+		std::map<int,int> last_parts; // folded concatenation, or view beneath it -> last products over its parts
 		std::function<void(int)> visit = [&](int u)
 		{
 			u = find(u);
@@ -1160,6 +1670,43 @@ struct Planner final
 			for (int d : deps)
 			{
 				if (d != u) { visit(d); }
+			}
+			if (nodes_[u].part_products >= 0)
+			{
+				const Node& n = nodes_[u];
+				PartProducts call = part_calls_[n.part_products];
+				FusionPlan::Step step;
+				step.parts = (int) plan.part_products.size();
+				// the products under the node, and their operands: folded
+				// concatenations are counted when the last product through them is out
+				std::vector<int> products;
+				if (n.summed)
+				{
+					for (int arg : n.args)
+					{
+						int c = nodes_[arg].op == egen::PERMUTE ? nodes_[arg].args[0] : arg;
+						plan.absorbed.push_back(nodes_[c].f);
+						if (c != arg) { plan.absorbed.push_back(nodes_[arg].f); }
+						products.push_back(c);
+					}
+				}
+				else { products.push_back(u); }
+				for (int c : products)
+				{
+					for (size_t k = 0; k < 2; ++k)
+					{
+						int a = nodes_[c].args[k];
+						if (a < 0) { continue; }
+						if (nodes_[a].parts_folded) { mark_parts_user(a, step.parts, last_parts); }
+						else if (false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+						{
+							call.reads.push_back(nodes_[c].arg_tens[k].get());
+						}
+					}
+				}
+				plan.part_products.push_back(call);
+				plan.steps.push_back(step);
+				return;
 			}
 			if (nodes_[u].kind != EW && nodes_[u].swapped_from >= 0)
 			{
@@ -1312,6 +1859,19 @@ struct Planner final
 				plan.convs[kv.second].reads.push_back(v.arg_tens[0].get());
 			}
 		}
+		for (auto& kv : last_parts)
+		{
+			const Node& v = nodes_[kv.first];
+			plan.absorbed.push_back(v.f);
+			for (size_t k = 0; k < v.args.size(); ++k)
+			{
+				int a = v.args[k];
+				if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+				{
+					plan.part_products[kv.second].reads.push_back(v.arg_tens[k].get());
+				}
+			}
+		}
 		for (auto& kv : last_user)
 		{
 			const Node& v = nodes_[kv.first];
@@ -1325,6 +1885,16 @@ struct Planner final
 		return plan;
 	}
 
+	/// Folded concatenation z and the views beneath it are read by products `step`
+	void mark_parts_user (int z, int step, std::map<int,int>& last_parts) const
+	{
+		last_parts[z] = step;
+		for (int a : nodes_[z].args)
+		{
+			if (a >= 0 && nodes_[a].kind == VIEW && nodes_[a].absorbed) { mark_parts_user(a, step, last_parts); }
+		}
+	}
+
 	static bool uses_immediate (const FusedGroup& group)
 	{
 		return std::any_of(group.program.begin(), group.program.end(), [](const tcg_fx_instr& ins)
@@ -1334,6 +1904,8 @@ struct Planner final
 	}
 
 	std::vector<Node> nodes_;
+	std::map<int,Parts> part_lists_;     // CONCAT / ADD of PADs -> its parts
+	std::vector<PartProducts> part_calls_;
 	std::map<int,ConvFold> folds_;       // CONV node -> what is folded into its launch
 	std::map<int,bool> feeds_convs_;     // memo of layout_feeds_convs
 	std::unordered_map<teq::iTensor*,int> index_;
@@ -1399,6 +1971,44 @@ void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMe
 	{
 		hip_check(tcg_contract_sum(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), call.ashape.data(), call.bshape.data(),
 			(int) (call.pairs.size() / 2), call.pairs.data(), (int) a.size(), a.data(), b.data(), dst));
+	}
+	catch (...)
+	{
+		ref.drop();
+		throw;
+	}
+	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
+}
+
+void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory)
+{
+	Observable* out = call.node;
+	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
+	auto& ref = static_cast<iEigen&>(out->device());
+	char* dst = (char*) ref.borrow_output(ttl, memory);
+	if (nullptr == dst) { global::fatalf("%s cannot take products over parts", out->to_string().c_str()); }
+	if (call.partial) { ref.mark_partial(); }
+	const int64_t esz = (int64_t) egen::type_size((egen::_GENERATED_DTYPE) call.dtype);
+	try
+	{
+		for (const PartProducts::Product& p : call.products)
+		{
+			std::vector<const void*> a, b;
+			std::vector<uint64_t> lda, ldb;
+			for (const PartProducts::Term& term : p.terms)
+			{
+				const char* pa = (const char*) eigen_ref(*term.a).device_data();
+				const char* pb = (const char*) eigen_ref(*term.b).device_data();
+				if (nullptr == pa || nullptr == pb) { global::fatal("operand of a matrix product has no data"); }
+				a.push_back(pa + esz * term.a_off);
+				b.push_back(pb + esz * term.b_off);
+				lda.push_back(term.lda);
+				ldb.push_back(term.ldb);
+			}
+			hip_check(tcg_gemm_terms(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), p.M, p.N, p.K,
+				(int) p.terms.size(), a.data(), lda.data(), p.trans_a, b.data(), ldb.data(), p.trans_b,
+				dst + esz * p.c_off, p.ldc));
+		}
 	}
 	catch (...)
 	{

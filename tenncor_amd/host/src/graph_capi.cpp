@@ -425,6 +425,11 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 				ss << "summed CONTRACT x" << plan.sums[step.sum].a.size() << "\n";
 				continue;
 			}
+			if (step.parts >= 0)
+			{
+				ss << plan.part_products[step.parts].label << "\n";
+				continue;
+			}
 			if (step.conv >= 0)
 			{
 				ss << "viewed " << plan.convs[step.conv].label << "\n";

@@ -226,6 +226,10 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 				{
 					launch_sum(fusion.sums[step.sum], targets, device.memory());
 				}
+				else if (step.parts >= 0)
+				{
+					launch_parts(fusion.part_products[step.parts], targets, device.memory());
+				}
 				else
 				{
 					launch_group(fusion.groups[step.group], targets, device.memory());

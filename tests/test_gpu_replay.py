@@ -345,6 +345,81 @@ def test_fused_lstm_matches_the_walk_bit_for_bit():
     assert stats["replay_launches"]["launches"] < 0.5 * stats["replay_unfused"]["launches"]
 
 
+def assert_close_to_walk(results, tol=1e-5):
+    base = results["plain"]
+    for kind, rows in results.items():
+        for i, (row, ref) in enumerate(zip(rows, base)):
+            for j, (a, b) in enumerate(zip(row, ref)):
+                assert np.isfinite(b).all()
+                assert np.abs(a - b).max() <= tol * np.abs(b).max(), "%s pass %d target %d" % (kind, i, j)
+
+
+def test_products_over_the_parts_of_concatenations_follow_the_walk():
+    """configs[3] at sizes where the recording never lays out [x_t, h] or the
+    joined gate gradients (cfg/tenncor/layer.yml:716-768,
+    tenncor/eteq/backprop.hpp:269-359): the step's product runs as a sum of
+    products over the parts, the product on the way back over the four gate
+    gradients and only for the columns of h, the weight gradient block by block.
+    The sums over K then come in another order than in the walk: 1e-5 of the
+    largest entry, the bar of a contraction.  The second case has part extents
+    with a small common divisor (12 and 20: chunks of 4), which the matrix
+    cores do not take, so that the concatenations are laid out as before and
+    the results are the walk's bit for bit."""
+    from tenncor_amd import configs, graph
+    rng = np.random.default_rng(41)
+    for (seq, batch, nin, hid), exact in (((6, 64, 32, 64), False), ((5, 48, 12, 20), True)):
+        feeds = [rng.uniform(-1, 1, batch * seq * nin).astype(np.float32) for _ in range(3)]
+
+        def build(g, api):
+            targets, x, w, _ = configs.config4_lstm(g, seq=seq, batch=batch, nin=nin, hid=hid)
+            lines = g.launch_plan(targets)
+            assert any(l.startswith("parts") for l in lines) != exact, lines
+            return targets, x
+
+        results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+        (assert_same_bits if exact else assert_close_to_walk)(results)
+        assert stats["replay"]["replayed"] == 2 and stats["replay"]["record_failures"] == 0
+
+
+def test_products_over_parts_read_each_part_where_the_walk_does():
+    """Two products over one concatenation with an assignment to one of its
+    parts between them in the walk's order: the concatenation holds the part's
+    old value (internal/eigen/device.hpp:508-544 rewrites the variable's
+    buffer only), so it is laid out and both products read that; a second
+    concatenation, built over the assignment, is read part by part and sees the
+    new value.  A concatenation that nothing rewrites is never laid out."""
+    rng = np.random.default_rng(43)
+    xs = [rng.uniform(-1, 1, 32 * 64).astype(np.float32) for _ in range(3)]
+    hv, cv = rng.uniform(-1, 1, 48 * 64).astype(np.float32), rng.uniform(-1, 1, 32 * 64).astype(np.float32)
+    w1v, w2v = (rng.uniform(-1, 1, 96 * 80).astype(np.float32) for _ in range(2))
+
+    def build(g, api):
+        x = g.variable(xs[0], [32, 64], "x")
+        h = g.variable(hv, [48, 64], "h")
+        c = g.variable(cv, [32, 64], "c")
+        w1, w2 = g.variable(w1v, [96, 80], "w1"), g.variable(w2v, [96, 80], "w2")
+        z = api.concat([x, h], 0)
+        clean = api.add(api.matmul(api.concat([h, c], 0), w1), api.matmul(api.concat([h, c], 0), w2))
+        upd = api.assign(x, c)
+        q1, q2 = api.matmul(z, w1), api.matmul(z, w2)
+        late = api.matmul(api.concat([upd, h], 0), w1)
+        targets = [api.add(api.add(q1, late), q2), clean]
+        lines = g.launch_plan(targets)
+        assert sum(l.startswith("parts CONCAT+MATMUL") for l in lines) == 3, lines
+        assert sum(l.startswith(("group CONCAT", "node CONCAT")) for l in lines) == 1, lines
+        return targets, x
+
+    results, stats = run_both(build, xs, kinds=("plain", "replay_launches", "replay"))
+    assert_close_to_walk(results)
+    # the first target depends on x's fed value through the laid-out concatenation only
+    want = np.concatenate([xs[1].reshape(64, 32), hv.reshape(64, 48)], axis=1).astype(np.float64)
+    new = np.concatenate([cv.reshape(64, 32), hv.reshape(64, 48)], axis=1).astype(np.float64)
+    w1m, w2m = w1v.reshape(80, 96).astype(np.float64), w2v.reshape(80, 96).astype(np.float64)
+    ref = want @ w1m + new @ w1m + want @ w2m
+    got = results["replay"][1][0].reshape(64, 96)
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
 def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
     from tenncor_amd import configs
     rng = np.random.default_rng(18)

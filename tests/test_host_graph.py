@@ -271,8 +271,8 @@ def parse_plan(lines):
         elif kind == "group":
             ops, *fields = rest.split(" ")
             steps.append(("group", ops.split("+"), {k: int(v) for k, v in (f.split("=") for f in fields)}))
-        elif kind in ("swapped", "viewed"):
-            steps.append((kind, rest.split("+"), {}))
+        elif kind in ("swapped", "viewed", "summed", "parts", "blocks"):
+            steps.append((kind, rest.split(" ")[0].split("+"), {}))
         else:
             steps.append(("folded", [], {"n": int(rest)}))
     return steps
@@ -428,3 +428,46 @@ def test_launch_plan_keeps_reads_of_a_variable_on_their_side_of_an_assignment(g,
     i1, i2 = names.index(["ASSIGN"]), names.index(["ASSIGN_SUB"])
     assert i1 < i2
     assert any("SQUARE" in n for n in names[i1 + 1:i2]) and any("NEG" in n for n in names[i2 + 1:])
+
+
+def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
+    """The products of an unrolled recurrent layer (cfg/tenncor/layer.yml:716-768 and
+    its gradient, tenncor/eteq/backprop.hpp:269-359) read concatenations: [x_t, h] in
+    the step itself, the ADD of the four PADded gate gradients on the way back, both
+    again in the weight gradient.  A concatenation only products read is never laid
+    out: a product over the joined dim runs as a sum of products over the parts, one
+    over the other dim as a product per block of the result."""
+    from tenncor_amd import configs
+    targets = configs.config4_lstm(g, seq=5, batch=64, nin=32, hid=64)[0]
+    lines = g.launch_plan(targets)
+    assert lines.count("parts CONCAT+CONTRACT x3") == 5, lines   # 32 + 64 joined columns in chunks of 32
+    assert lines.count("parts ADD+CONTRACT x4+SLICE") == 4, lines  # only the columns of h are read back
+    assert lines.count("blocks CONTRACT x5 2x4") == 1, lines
+    assert not any(l.startswith(("summed", "swapped", "node CONTRACT", "node CONCAT", "group CONCAT ")) for l in lines), lines
+    steps = parse_plan(lines)
+    alone = sum(1 for s in steps if s[0] in ("node", "swapped", "viewed", "summed", "parts", "blocks"))
+    stores = sum(s[2]["stores"] for s in steps if s[0] == "group")
+    assert alone + stores + steps[-1][2]["n"] == g.count_functors(targets)
+    # below the sizes the matrix cores take, everything stays as it was
+    small = configs.config4_lstm(g, seq=5, batch=6, nin=8, hid=12)[0]
+    assert not any(l.startswith(("parts", "blocks")) for l in g.launch_plan(small))
+
+    x = var(g, [32, 64], np.float32, "x")
+    h = var(g, [48, 64], np.float32, "h")
+    w1 = var(g, [96, 80], np.float32, "w1")
+    w2 = var(g, [96, 80], np.float32, "w2")
+    c = var(g, [32, 64], np.float32, "c")
+    z = api.concat([x, h], 0)
+    p1, p2 = api.matmul(z, w1), api.matmul(z, w2)
+    lines = g.launch_plan([api.add(p1, p2)])
+    assert lines.count("parts CONCAT+MATMUL x5") == 2 and not any("CONCAT" in l and l.startswith(("group", "node")) for l in lines), lines
+    # a concatenation that an elementwise node reads as well is laid out once, for everybody
+    lines = g.launch_plan([api.add(p1, p2), api.neg(z)])
+    assert not any(l.startswith("parts") for l in lines) and lines.count("node MATMUL") == 2, lines
+    # an assignment to a part between the concatenation and a product that reads it:
+    # the concatenation holds the old value, the part's buffer the new one
+    upd = api.assign(x, c)
+    q1, q2 = api.matmul(z, w1), api.matmul(z, w2)
+    t = api.add(api.add(q1, api.matmul(api.concat([upd, h], 0), w1)), q2)
+    lines = g.launch_plan([t])
+    assert any(l.startswith(("group CONCAT", "node CONCAT")) for l in lines) and lines.count("node MATMUL") >= 2, lines
