@@ -288,6 +288,13 @@ typedef struct tcg_fx_leaf
 	int64_t stride[8];
 	uint64_t lo[8];
 	uint64_t hi[8];
+	/* nsum > 1: the operand's value is the sum, in this order, of the nsum
+	 * elements at distances 0, sum_stride, 2 sum_stride, ... (in elements)
+	 * from where the fields above point: the K ranges a matrix product left
+	 * side by side (tcg_gemm_terms_ranges).  0 and 1 both mean a plain operand. */
+	int64_t sum_stride;
+	uint32_t nsum;
+	uint32_t reserved_;
 } tcg_fx_leaf;
 typedef struct tcg_fx_instr
 {
@@ -427,6 +434,20 @@ int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	const void* const* A, const uint64_t* lda, int trans_a,
 	const void* const* B, const uint64_t* ldb, int trans_b,
 	void* C, uint64_t ldc);
+/* The same sum of products with its summed index cut into `nranges` equal
+ * ranges whose results are left side by side: ranges[r][m][n] (row-major
+ * M x N each) is the sum over range r.  The reader adds them up in range
+ * order -- an elementwise launch that reads a matrix product backwards
+ * through the recurrence of cfg/tenncor/layer.yml:716-768 does so while it
+ * loads its operand (tcg_fx_leaf.nsum), which saves the launch that would add
+ * the ranges of a product with few results under a long K.  Matrix cores only:
+ * fp32, M, N >= 32, K a multiple of 16, nterms * K a multiple of 16 nranges,
+ * 2 <= nranges <= 32, 16-byte aligned operands; anything else fails with
+ * TCG_ERR_UNSUPPORTED (the caller falls back on tcg_gemm_terms). */
+int tcg_gemm_terms_ranges (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K, int nterms,
+	const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b,
+	int nranges, void* ranges);
 /* CONV (cfg/ops.yml:566-607; internal/eigen/operator.hpp:1141-1187):
  * valid cross-correlation, kernel dim i slides along image dim ranks[i] */
 int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],

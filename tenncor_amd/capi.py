@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_gemm_terms", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -63,7 +63,8 @@ class EwInstr(ctypes.Structure):
 
 class FxLeaf(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("offset", ctypes.c_int64), ("stride", ctypes.c_int64 * 8),
-                ("lo", ctypes.c_uint64 * 8), ("hi", ctypes.c_uint64 * 8)]
+                ("lo", ctypes.c_uint64 * 8), ("hi", ctypes.c_uint64 * 8),
+                ("sum_stride", ctypes.c_int64), ("nsum", ctypes.c_uint32), ("reserved_", ctypes.c_uint32)]
 
 
 class FxInstr(ctypes.Structure):
@@ -133,6 +134,7 @@ def load():
         "tcg_contract_sum": [vp, i32, u64p, u64p, i32, u64p, i32, vpp, vpp, vp],
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
         "tcg_gemm_terms": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
+        "tcg_gemm_terms_ranges": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, i32, vp],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
@@ -335,7 +337,8 @@ class Context:
 
     def ew_fusedx(self, dtype, shape, leaves, program, outs):
         """leaves: dicts with ptr, and optionally offset, stride (8 element
-        strides; default: dense over `shape`), lo, hi (default: everything).
+        strides; default: dense over `shape`), lo, hi (default: everything),
+        nsum and sum_stride (the value is the sum of nsum elements that far apart).
         program: tuples (opcode | "STORE", a, b, c, dst[, imm])."""
         shp = shape8(shape)
         dense = [1] * RANK_CAP
@@ -349,6 +352,8 @@ class Context:
                 lv[k].stride[d] = int(leaf.get("stride", dense)[d])
                 lv[k].lo[d] = int(leaf.get("lo", [0] * RANK_CAP)[d])
                 lv[k].hi[d] = int(leaf.get("hi", shp)[d])
+            lv[k].nsum = int(leaf.get("nsum", 0))
+            lv[k].sum_stride = int(leaf.get("sum_stride", 0))
         instrs = (FxInstr * len(program))()
         for i, ins in enumerate(program):
             instrs[i].opcode = {"STORE": FX_STORE, "BITOR": FX_BITOR}.get(ins[0]) or _opcode(ins[0])
@@ -455,6 +460,16 @@ class Context:
         la = (ctypes.c_uint64 * n)(*[int(v) for v in lda])
         lb = (ctypes.c_uint64 * n)(*[int(v) for v in ldb])
         self._check(self.lib.tcg_gemm_terms(self.handle, dtype, M, N, K, n, pa, la, int(trans_a), pb, lb, int(trans_b), c, ldc))
+
+    def gemm_terms_ranges(self, dtype, M, N, K, a_ptrs, lda, trans_a, b_ptrs, ldb, trans_b, nranges, ranges):
+        """The same sum with its summed index cut into nranges ranges left side by side."""
+        n = len(a_ptrs)
+        pa = (ctypes.c_void_p * n)(*a_ptrs)
+        pb = (ctypes.c_void_p * n)(*b_ptrs)
+        la = (ctypes.c_uint64 * n)(*[int(v) for v in lda])
+        lb = (ctypes.c_uint64 * n)(*[int(v) for v in ldb])
+        self._check(self.lib.tcg_gemm_terms_ranges(self.handle, dtype, M, N, K, n, pa, la, int(trans_a), pb, lb,
+                                                   int(trans_b), int(nranges), ranges))
 
     def conv_views(self, dtype, imgshape, kshape, ranks, img_box, out_box, box, box_stride, kernel, kernel_stride,
                    dst, out_stride):

@@ -211,10 +211,16 @@ __global__ __launch_bounds__(FX_BLOCK) void ew_fusedx_k (FxArgs p)
 					VecU<T> v;
 					v.v = *reinterpret_cast<const typename Vec16<T>::type*>(src);
 					FX_EACH(file[k][e_] = v.e[e_])
+					for (uint32_t r = 1; r < p.leaf[k].nsum; ++r)
+					{
+						v.v = *reinterpret_cast<const typename Vec16<T>::type*>(src + (int64_t) r * p.leaf[k].sum_stride);
+						FX_EACH(file[k][e_] += v.e[e_])
+					}
 				}
 				else
 				{
 					T s = *src;
+					for (uint32_t r = 1; r < p.leaf[k].nsum; ++r) { s += src[(int64_t) r * p.leaf[k].sum_stride]; }
 					FX_EACH(file[k][e_] = s)
 				}
 			}
@@ -417,6 +423,7 @@ void fx_emit_parts (FxParts& parts, int N, const FxArgs& p, const bool* dense, c
 	{
 		return bake ? std::to_string(p.leaf[k].hi[d]) + "u" : "p.leaf[" + std::to_string(k) + "].hi[" + std::to_string(d) + "]";
 	};
+	auto r_sum_stride = [&](uint32_t k) { return bake ? num(p.leaf[k].sum_stride) : "p.leaf[" + std::to_string(k) + "].sum_stride"; };
 	auto r_leaf = [&](uint32_t k) { return bake ? bake->leaf_ptr[k] : "p.leaf[" + std::to_string(k) + "].ptr"; };
 	auto r_out = [&](uint32_t k) { return bake ? bake->out_ptr[k] : "p.out[" + std::to_string(k) + "]"; };
 	auto r_imm = [&](uint32_t i) -> std::string
@@ -482,11 +489,23 @@ void fx_emit_parts (FxParts& parts, int N, const FxArgs& p, const bool* dense, c
 		if (N > 1 && !L.bcast0)
 		{
 			o << "VU v; v.v = " << (once ? "__builtin_nontemporal_load((const VT*) src)" : "*(const VT*) src") << ";\n";
+			if (L.nsum > 1)
+			{
+				// the ranges are added in their order; the loads of several are in flight together
+				o << "_Pragma(\"unroll 8\")\nfor (uint32_t r = 1; r < " << L.nsum << "u; ++r)\n{\n"
+					"VU w; w.v = *(const VT*) (src + (int64_t) r * " << r_sum_stride(k) << ");\n";
+				for (int e = 0; e < N; ++e) { o << "v.e[" << e << "] += w.e[" << e << "];\n"; }
+				o << "}\n";
+			}
 			for (int e = 0; e < N; ++e) { o << "l" << k << sfx << "[" << e << "] = v.e[" << e << "];\n"; }
 		}
 		else
 		{
-			o << "const T s = *src;\n";
+			o << "T s = *src;\n";
+			if (L.nsum > 1)
+			{
+				o << "_Pragma(\"unroll 8\")\nfor (uint32_t r = 1; r < " << L.nsum << "u; ++r) { s += src[(int64_t) r * " << r_sum_stride(k) << "]; }\n";
+			}
 			for (int e = 0; e < N; ++e) { o << "l" << k << sfx << "[" << e << "] = s;\n"; }
 		}
 		o << "}\n";
@@ -1267,6 +1286,9 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		FxLeaf& L = p.leaf[k];
 		L.ptr = leaves[k].ptr;
 		L.off = leaves[k].offset;
+		L.nsum = leaves[k].nsum > 1 ? leaves[k].nsum : 1;
+		L.sum_stride = L.nsum > 1 ? leaves[k].sum_stride : 0;
+		if (L.nsum > 1) { vec = vec && L.sum_stride % N == 0; }
 		L.boxed = 0;
 		for (uint32_t d = 0; d < nd; ++d) { L.boxed |= !(L.lo[d] == 0 && L.hi[d] >= p.size[d]); }
 		L.bcast0 = L.stride[0] == 0;

@@ -500,4 +500,29 @@ int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	return TCG_OK;
 }
 
+int tcg_gemm_terms_ranges (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K, int nterms,
+	const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b,
+	int nranges, void* ranges)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, A && B && lda && ldb && ranges, "tcg_gemm_terms_ranges: NULL pointer");
+	TCG_REQUIRE(ctx, nterms >= 1, "tcg_gemm_terms_ranges: %d terms", nterms);
+	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, A[t] && B[t], "tcg_gemm_terms_ranges: operand of term %d is NULL", t); }
+	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "the K ranges of a matrix product"); }
+	bool handled = false;
+	if (dtype == TCG_FLOAT && nranges >= 2)
+	{
+		int rc = tcg_gemm_f32_mfma_ranges(ctx, M, N, K, (uint32_t) nterms, (const float* const*) A, lda, trans_a,
+			(const float* const*) B, ldb, trans_b, (uint32_t) nranges, (float*) ranges, &handled);
+		if (rc != TCG_OK) { return rc; }
+	}
+	if (!handled)
+	{
+		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED,
+			"tcg_gemm_terms_ranges: fp32 only, M, N >= 32, K a multiple of 16, 2..32 ranges of whole 16-column slabs, 16-byte aligned operands");
+	}
+	return TCG_OK;
+}
+
 } // extern "C"

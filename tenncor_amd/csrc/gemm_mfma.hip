@@ -436,9 +436,10 @@ __global__ __launch_bounds__(256) void gemm_split_sum_wave_k (const f32x4v* __re
 	if (lane == 0) { C[i] = acc; }
 }
 
+// `ranges_out`: the K ranges stay side by side there ([range][batch][M][N]) and nothing adds them up
 template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs>
 int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1,
-	const SEGS& segs = SEGS())
+	const SEGS& segs = SEGS(), float* ranges_out = nullptr)
 {
 	GemmArgs g = base;
 	uint64_t tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
@@ -457,7 +458,12 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 		g.k_per_split = ((g.K + splits - 1) / splits + BK - 1) / BK * BK;
 		splits = (g.K + g.k_per_split - 1) / g.k_per_split;
 	}
-	if (splits > 1)
+	if (ranges_out)
+	{
+		TCG_REQUIRE(ctx, splits > 1 && total * splits < (1ull << 31), "tcg_gemm: %u ranges of K", splits);
+		g.partial = ranges_out;
+	}
+	else if (splits > 1)
 	{
 		TCG_REQUIRE(ctx, total * splits < (1ull << 31), "tcg_gemm: too many tiles for one launch");
 		partial_bytes = sizeof(float) * splits * batch * g.M * g.N;
@@ -476,7 +482,7 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 		else { gemm_mfma_k<BM,BN,WGM,true,true,0,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	}
 	else { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
-	if (g.partial)
+	if (g.partial && !ranges_out)
 	{
 		uint64_t n = batch * g.M * g.N;
 		bool dense = g.ldc == (int64_t) g.N && (batch == 1 || g.batch_c == (int64_t) g.M * g.N);
@@ -868,6 +874,45 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 	if (splits > 32) { splits = 32; }
 	if (splits < 2) { splits = 1; }
 	return launch<128,128,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) splits, segs);
+}
+
+// The same sum of products with its K ranges left side by side:
+// ranges[r][m][n] = sum over the r-th of `nranges` equal parts of the
+// concatenated summed index; whoever reads them adds them up in range order
+int tcg_gemm_f32_mfma_ranges (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
+	const float* const* A, const uint64_t* lda, int trans_a, const float* const* B, const uint64_t* ldb, int trans_b,
+	uint32_t nranges, float* ranges, bool* handled)
+{
+	*handled = false;
+	bool ok = terms >= 1 && terms <= (uint32_t) MAX_TERMS && M >= 32 && N >= 32 && K >= BK && K % BK == 0 &&
+		M < (1ull << 31) && N < (1ull << 31) && K * terms < (1ull << 31) &&
+		((trans_a ? M : K) % 4 == 0) && ((trans_b ? K : N) % 4 == 0) &&
+		nranges >= 2 && nranges <= 32 && (K * terms) % ((uint64_t) nranges * BK) == 0 && tcg_aligned16(ranges);
+	for (uint32_t t = 0; t < terms && ok; ++t)
+	{
+		ok = tcg_aligned16(A[t]) && tcg_aligned16(B[t]) && lda[t] % 4 == 0 && ldb[t] % 4 == 0 &&
+			lda[t] < (1ull << 32) && ldb[t] < (1ull << 32);
+	}
+	if (!ok) { return TCG_OK; }
+	GemmArgs g;
+	g.A = A[0]; g.B = B[0]; g.C = ranges;
+	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) (K * terms);
+	g.lda = (int64_t) lda[0]; g.ldb = (int64_t) ldb[0]; g.ldc = (int64_t) N;
+	g.batch_a = g.batch_b = g.batch_c = 0;
+	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
+	g.rows = g.sums = nullptr;
+	g.ncheck = 0;
+	GemmSegs segs;
+	segs.k = (uint32_t) K;
+	for (uint32_t t = 0; t < terms; ++t)
+	{
+		segs.a[t] = A[t];
+		segs.b[t] = B[t];
+		segs.lda[t] = (uint32_t) lda[t];
+		segs.ldb[t] = (uint32_t) ldb[t];
+	}
+	*handled = true;
+	return launch<64,64,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, nranges, segs, ranges);
 }
 
 int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,

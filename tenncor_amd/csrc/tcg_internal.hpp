@@ -171,6 +171,11 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 	const float* const* A, const uint64_t* lda, int trans_a, const float* const* B, const uint64_t* ldb, int trans_b,
 	float* C, uint64_t ldc, bool* handled);
 
+// the same with the K ranges left side by side for the reader to add up
+int tcg_gemm_f32_mfma_ranges (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
+	const float* const* A, const uint64_t* lda, int trans_a, const float* const* B, const uint64_t* ldb, int trans_b,
+	uint32_t nranges, float* ranges, bool* handled);
+
 // reduce.hip: looks up this GPU's copy of the scratch memory of
 // tcg_reduce_noalloc; called once per context with the device current
 int tcg_reduce_scratch_init (tcg_ctx* ctx);

@@ -20,7 +20,10 @@ struct FusedGroup final
 	struct Leaf final
 	{
 		teq::iTensor* base = nullptr; ///< materialised tensor the view starts from
-		tcg_fx_leaf view;             ///< ptr is filled in at launch
+		tcg_fx_leaf view = {};        ///< ptr is filled in at launch
+		/// >= 0: the operand is the sum of the K ranges that product
+		/// (FusionPlan::part_products) left side by side instead of a tensor's value
+		int ranges_of = -1;
 	};
 
 	int dtype = 0;
@@ -32,6 +35,8 @@ struct FusedGroup final
 	/// materialised tensors that count one read when this group has launched:
 	/// what the members and the views folded into them would have read
 	std::vector<teq::iTensor*> reads;
+	/// products (FusionPlan::part_products) whose K ranges nothing reads after this group
+	std::vector<int> frees;
 };
 
 /// PERMUTE{1,0}(CONTRACT(a, b)) with a matrix result is CONTRACT(b, a) with
@@ -136,6 +141,10 @@ struct PartProducts final
 	int dtype = 0;
 	std::vector<Product> products;
 	bool partial = false;            ///< only the window its SLICE readers look at is computed
+	/// > 0: the node is never laid out; the product leaves that many K ranges of
+	/// its window side by side in temporary memory ([range][M][N]) and the
+	/// elementwise groups that read the node add them up while they load
+	uint32_t ranges = 0;
 	std::vector<teq::iTensor*> reads;
 	std::string label;
 };
@@ -168,7 +177,12 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 
 /// Enqueue one group: borrows the outputs' buffers (lifetimes as
 /// eigen::Device::calc gives them), launches, counts the reads
-void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory);
+/// Temporary memory of the products that leave K ranges, by index into
+/// FusionPlan::part_products: {address, bytes}, held from the product's
+/// launch to the last group that reads it
+using RangeTempsT = std::vector<std::pair<void*,size_t>>;
+
+void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps);
 
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
@@ -176,7 +190,7 @@ void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptr
 
 void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
-void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory);
+void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory, std::pair<void*,size_t>& temp);
 
 }
 

@@ -53,6 +53,7 @@ struct Node final
 	                            // a node between such a CONV and the node that receives its result
 	bool parts_folded = false;  // CONCAT / ADD of PADs that only products read, part by part
 	int part_products = -1;     // CONTRACT, or ADD over CONTRACT terms, launched as products over parts (index into part_calls_)
+	bool ranged = false;        // such a product that leaves its K ranges for the groups that read it: never laid out
 	bool summed = false;        // ADD launched as one sum of the products it adds
 	bool summed_term = false;   // CONTRACT / PERMUTE that is a term of such a sum
 	std::vector<int> args;      // index of the functor operand, -1 for a leaf
@@ -240,6 +241,13 @@ struct Planner final
 		members_.resize(nodes_.size());
 		deps_.resize(nodes_.size());
 		stamp_.assign(nodes_.size(), 0);
+	}
+
+	/// Node a has a buffer of its own when its launch has run (whose reads are counted)
+	bool holds_value (int a) const
+	{
+		const Node& n = nodes_[a];
+		return false == (n.kind == VIEW && n.absorbed) && false == n.ranged;
 	}
 
 	bool is_alias (int i) const
@@ -896,8 +904,58 @@ struct Planner final
 		for (auto& kv : calls)
 		{
 			nodes_[kv.first].part_products = (int) part_calls_.size();
+			choose_ranges(kv.first, kv.second);
 			part_calls_.push_back(kv.second);
 		}
+	}
+
+	/// Do only elementwise groups read node v, and only through SLICE / PAD /
+	/// IDENTITY nodes folded into them (views that still walk the result row by row)?
+	bool only_groups_read_through (int v, bool top = true) const
+	{
+		const Node& n = nodes_[v];
+		if (n.target || n.consumers.empty()) { return false; }
+		for (int c : n.consumers)
+		{
+			const Node& m = nodes_[c];
+			if (m.kind == EW && false == top) { continue; }
+			bool folded_view = m.kind == VIEW && m.absorbed && false == m.through_conv && false == m.parts_folded &&
+				false == m.summed_term && (m.op == egen::SLICE || m.op == egen::PAD || m.op == egen::IDENTITY);
+			if (false == folded_view || false == only_groups_read_through(c, false)) { return false; }
+		}
+		return true;
+	}
+
+	/// A product with few results under a long K runs as K ranges on separate
+	/// workgroups, and a launch of its own would add them up.  When elementwise
+	/// groups reading through SLICEs are all that reads the node, the ranges
+	/// stay side by side and those groups add them while they load.
+	void choose_ranges (int c, PartProducts& call)
+	{
+		const Node& n = nodes_[c];
+		if (n.summed || call.products.size() != 1 || n.dtype != egen::FLOAT) { return; }
+		const PartProducts::Product& p = call.products[0];
+		// the shapes the product kernels split: a transposed operand (row-major
+		// operands with enough 32 x 32 blocks share K between the waves of a workgroup)
+		if (false == (p.trans_a || p.trans_b)) { return; }
+		const uint64_t depth = p.K * p.terms.size();
+		const uint64_t cus = 256;
+		uint64_t tiles128 = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+		if (tiles128 * std::min<uint64_t>(32, depth / 256) >= cus) { return; }
+		uint64_t tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
+		uint64_t want = std::min<uint64_t>({32, 2 * cus / tiles, depth / 128});
+		uint32_t ranges = 1;
+		while (2 * ranges <= want && depth % (2 * ranges * 16) == 0) { ranges *= 2; }
+		if (ranges < 2) { return; }
+		// every reader adds the ranges up again: worth it for one or two
+		if (false == only_groups_read_through(c)) { return; }
+		size_t readers = 0;
+		for (int v : n.consumers) { readers += nodes_[v].consumers.size(); }
+		if (readers > 2) { return; }
+		// ... and the groups must see the product's dtype (a view changes none)
+		call.ranges = ranges;
+		call.label += " ranges=" + std::to_string(ranges);
+		nodes_[c].ranged = true;
 	}
 
 	// ---- sums of products ----
@@ -1274,7 +1332,7 @@ struct Planner final
 		for (size_t k = 0; k < 2; ++k)
 		{
 			int a = c.args[k];
-			if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+			if (a >= 0 && holds_value(a))
 			{
 				call.reads.push_back(c.arg_tens[k].get());
 			}
@@ -1558,12 +1616,42 @@ struct Planner final
 						continue;
 					}
 				}
+				// an operand whose launch left K ranges: the window lies there as a dense matrix
+				int ranges_of = -1;
+				uint32_t nsum = 0;
+				int64_t sum_stride = 0;
+				auto producer = index_.find(v.base);
+				if (producer != index_.end() && nodes_[producer->second].ranged)
+				{
+					ranges_of = nodes_[producer->second].part_products;
+					const PartProducts& call = part_calls_[ranges_of];
+					const PartProducts::Product& prod = call.products[0];
+					// from the first element the view reads: steps along a row stay steps
+					// of one, steps from row to row become steps of the window's width
+					const int64_t ld = (int64_t) prod.ldc, m0 = prod.c_off / ld, n0 = prod.c_off % ld;
+					int64_t first = v.off;
+					for (int d = 0; d < 8; ++d) { first += (int64_t) v.lo[d] * v.stride[d]; }
+					if (first < 0 || first / ld < m0 || first % ld < n0) { return false; }
+					int64_t at = (first / ld - m0) * (int64_t) prod.N + (first % ld - n0);
+					for (int d = 0; d < 8; ++d)
+					{
+						if (v.stride[d] < 0 || (v.stride[d] >= ld && v.stride[d] % ld != 0)) { return false; }
+						v.stride[d] = (v.stride[d] / ld) * (int64_t) prod.N + v.stride[d] % ld;
+						at -= (int64_t) v.lo[d] * v.stride[d];
+					}
+					v.off = at;
+					nsum = call.ranges;
+					sum_stride = (int64_t) (prod.M * prod.N);
+				}
 				auto it = leaf_of.find(v);
 				if (it == leaf_of.end())
 				{
 					if (out.leaves.size() >= TCG_FX_MAX_LEAVES) { return false; }
 					FusedGroup::Leaf leaf;
 					leaf.base = v.base;
+					leaf.ranges_of = ranges_of;
+					leaf.view.nsum = nsum;
+					leaf.view.sum_stride = sum_stride;
 					leaf.view.ptr = nullptr;
 					leaf.view.offset = v.off;
 					std::copy(v.stride, v.stride + 8, leaf.view.stride);
@@ -1645,7 +1733,7 @@ struct Planner final
 			{
 				int a = n.args[k];
 				if (a < 0) { continue; }
-				bool materialised = inside(a) ? stored[pos[a]] : false == (nodes_[a].kind == VIEW && nodes_[a].absorbed);
+				bool materialised = inside(a) ? stored[pos[a]] : holds_value(a);
 				if (materialised) { out.reads.push_back(n.arg_tens[k].get()); }
 			}
 		}
@@ -1659,6 +1747,7 @@ struct Planner final
 		std::map<int,int> last_user; // folded view -> last group reading through it
 		std::map<int,int> last_conv; // PAD read in place -> last convolution of its operand
 		std::map<int,int> last_parts; // folded concatenation, or view beneath it -> last products over its parts
+		std::map<int,int> last_ranges; // product that leaves K ranges (index into plan.part_products) -> last group adding them up
 		std::function<void(int)> visit = [&](int u)
 		{
 			u = find(u);
@@ -1698,12 +1787,14 @@ struct Planner final
 						int a = nodes_[c].args[k];
 						if (a < 0) { continue; }
 						if (nodes_[a].parts_folded) { mark_parts_user(a, step.parts, last_parts); }
-						else if (false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+						else if (holds_value(a))
 						{
 							call.reads.push_back(nodes_[c].arg_tens[k].get());
 						}
 					}
 				}
+				if (call.ranges > 0) { plan.absorbed.push_back(n.f); }
+				emitted_parts_[n.part_products] = step.parts;
 				plan.part_products.push_back(call);
 				plan.steps.push_back(step);
 				return;
@@ -1729,7 +1820,7 @@ struct Planner final
 				for (size_t k = 0; k < 2; ++k)
 				{
 					int a = c.args[k];
-					if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+					if (a >= 0 && holds_value(a))
 					{
 						call.reads.push_back(c.arg_tens[k].get());
 					}
@@ -1772,7 +1863,7 @@ struct Planner final
 					for (size_t j = 0; j < 2; ++j)
 					{
 						int operand = c.args[j];
-						if (operand >= 0 && false == (nodes_[operand].kind == VIEW && nodes_[operand].absorbed))
+						if (operand >= 0 && holds_value(operand))
 						{
 							call.reads.push_back(c.arg_tens[j].get());
 						}
@@ -1827,6 +1918,12 @@ struct Planner final
 				{
 					step.group = (int) plan.groups.size();
 					for (int v : views) { last_user[v] = step.group; }
+					for (FusedGroup::Leaf& leaf : group.leaves)
+					{
+						if (leaf.ranges_of < 0) { continue; }
+						leaf.ranges_of = emitted_parts_.at(leaf.ranges_of);
+						last_ranges[leaf.ranges_of] = step.group;
+					}
 					for (size_t p = lo; p < hi; ++p)
 					{
 						const Node& n = nodes_[members[p]];
@@ -1854,11 +1951,12 @@ struct Planner final
 			const Node& v = nodes_[kv.first];
 			plan.absorbed.push_back(v.f);
 			int a = v.args[0];
-			if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+			if (a >= 0 && holds_value(a))
 			{
 				plan.convs[kv.second].reads.push_back(v.arg_tens[0].get());
 			}
 		}
+		for (auto& kv : last_ranges) { plan.groups[kv.second].frees.push_back(kv.first); }
 		for (auto& kv : last_parts)
 		{
 			const Node& v = nodes_[kv.first];
@@ -1866,7 +1964,7 @@ struct Planner final
 			for (size_t k = 0; k < v.args.size(); ++k)
 			{
 				int a = v.args[k];
-				if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+				if (a >= 0 && holds_value(a))
 				{
 					plan.part_products[kv.second].reads.push_back(v.arg_tens[k].get());
 				}
@@ -1877,7 +1975,7 @@ struct Planner final
 			const Node& v = nodes_[kv.first];
 			plan.absorbed.push_back(v.f);
 			int a = v.args[0];
-			if (a >= 0 && false == (nodes_[a].kind == VIEW && nodes_[a].absorbed))
+			if (a >= 0 && holds_value(a))
 			{
 				plan.groups[kv.second].reads.push_back(v.arg_tens[0].get());
 			}
@@ -1906,6 +2004,7 @@ struct Planner final
 	std::vector<Node> nodes_;
 	std::map<int,Parts> part_lists_;     // CONCAT / ADD of PADs -> its parts
 	std::vector<PartProducts> part_calls_;
+	std::map<int,int> emitted_parts_;    // index into part_calls_ -> index into the plan's part_products
 	std::map<int,ConvFold> folds_;       // CONV node -> what is folded into its launch
 	std::map<int,bool> feeds_convs_;     // memo of layout_feeds_convs
 	std::unordered_map<teq::iTensor*,int> index_;
@@ -1980,15 +2079,40 @@ void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMe
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
-void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory)
+void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory, std::pair<void*,size_t>& temp)
 {
 	Observable* out = call.node;
+	const int64_t esz = (int64_t) egen::type_size((egen::_GENERATED_DTYPE) call.dtype);
+	if (call.ranges > 0)
+	{
+		// the node gets no buffer: its K ranges wait in `temp` for the groups that add them up
+		const PartProducts::Product& p = call.products.at(0);
+		std::vector<const void*> a, b;
+		std::vector<uint64_t> lda, ldb;
+		for (const PartProducts::Term& term : p.terms)
+		{
+			const char* pa = (const char*) eigen_ref(*term.a).device_data();
+			const char* pb = (const char*) eigen_ref(*term.b).device_data();
+			if (nullptr == pa || nullptr == pb) { global::fatal("operand of a matrix product has no data"); }
+			a.push_back(pa + esz * term.a_off);
+			b.push_back(pb + esz * term.b_off);
+			lda.push_back(term.lda);
+			ldb.push_back(term.ldb);
+		}
+		if (nullptr == memory) { global::fatal("cannot borrow from null memory"); }
+		temp.second = (size_t) esz * call.ranges * p.M * p.N;
+		temp.first = memory->allocate(temp.second);
+		hip_check(tcg_gemm_terms_ranges(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), p.M, p.N, p.K,
+			(int) p.terms.size(), a.data(), lda.data(), p.trans_a, b.data(), ldb.data(), p.trans_b,
+			(int) call.ranges, temp.first));
+		for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
+		return;
+	}
 	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
 	auto& ref = static_cast<iEigen&>(out->device());
 	char* dst = (char*) ref.borrow_output(ttl, memory);
 	if (nullptr == dst) { global::fatalf("%s cannot take products over parts", out->to_string().c_str()); }
 	if (call.partial) { ref.mark_partial(); }
-	const int64_t esz = (int64_t) egen::type_size((egen::_GENERATED_DTYPE) call.dtype);
 	try
 	{
 		for (const PartProducts::Product& p : call.products)
@@ -2055,7 +2179,7 @@ void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptr
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
-void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory)
+void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps)
 {
 	std::vector<void*> outs;
 	for (Observable* out : group.outputs)
@@ -2069,7 +2193,7 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 	for (auto& leaf : group.leaves)
 	{
 		tcg_fx_leaf view = leaf.view;
-		view.ptr = eigen_ref(*leaf.base).device_data();
+		view.ptr = leaf.ranges_of >= 0 ? temps.at(leaf.ranges_of).first : eigen_ref(*leaf.base).device_data();
 		if (nullptr == view.ptr) { global::fatalf("operand %s has no data", leaf.base->to_string().c_str()); }
 		leaves.push_back(view);
 	}
@@ -2084,6 +2208,13 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 		throw;
 	}
 	for (teq::iTensor* tens : group.reads) { eigen_ref(*tens).odevice(); }
+	for (int done : group.frees)
+	{
+		// after this launch in stream order
+		std::pair<void*,size_t>& temp = temps.at(done);
+		if (nullptr != temp.first) { memory->deallocate(temp.first, temp.second); }
+		temp = {nullptr, 0};
+	}
 }
 
 }

@@ -206,6 +206,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		for (Observable* f : plan->funcs) { f->prop_version(device.max_version_); }
 		hip_check(as_one_kernel ? tcg_capture_begin_small(ctx) : tcg_capture_begin(ctx));
 		bool ok = true;
+		RangeTempsT temps(fusion.part_products.size(), {nullptr, 0});
 		try
 		{
 			for (auto& step : fusion.steps)
@@ -228,11 +229,11 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 				}
 				else if (step.parts >= 0)
 				{
-					launch_parts(fusion.part_products[step.parts], targets, device.memory());
+					launch_parts(fusion.part_products[step.parts], targets, device.memory(), temps[step.parts]);
 				}
 				else
 				{
-					launch_group(fusion.groups[step.group], targets, device.memory());
+					launch_group(fusion.groups[step.group], targets, device.memory(), temps);
 				}
 			}
 		}
@@ -246,6 +247,11 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		{
 			failure = "a failure that is not a std::exception";
 			ok = false;
+		}
+		for (auto& temp : temps)
+		{
+			// a pass that failed half way: what its products borrowed goes back
+			if (nullptr != temp.first) { device.memory()->deallocate(temp.first, temp.second); }
 		}
 		plan->leaf_fed.assign(plan->leaves.size(), 0);
 		if (ok && as_one_kernel)

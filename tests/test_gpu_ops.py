@@ -1387,3 +1387,83 @@ def test_sum_of_products_over_parts_of_tensors(ctx, oracle, case, np_dtype):
     for m in range(M):
         mask[coff + m * ldc: coff + m * ldc + cols] = False
     assert (got[mask] == 777).all()
+
+
+@pytest.mark.parametrize("jit", ["1", "0"])
+def test_product_ranges_are_added_by_the_launch_that_reads_them(ctx, jit):
+    """tcg_gemm_terms_ranges leaves the K ranges of a sum of products side by
+    side and a tcg_ew_fusedx operand with nsum > 1 adds them in range order
+    while it loads: the product backwards through a recurrent step
+    (cfg/tenncor/layer.yml:716-768, tenncor/eteq/backprop.hpp:269-359: the four
+    gate gradients times the transposed weight, few results under a long K) then
+    needs no launch of its own for the sum.  The ranges added on the host in
+    fp32, in order, fix every bit of what the reading launch must see; their sum
+    is held against the product in double at 1e-4.  The run-time compiled kernel
+    (both lane widths, a boxed operand) and the interpreter are covered; the
+    interpreter runs in a process of its own, the switch being read once."""
+    import subprocess
+    import sys
+    if jit == "0":
+        if os.environ.get("TCG_FX_JIT") != "0":
+            env = dict(os.environ, TCG_FX_JIT="0")
+            here = os.path.abspath(__file__)
+            res = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", here + "::" +
+                                  "test_product_ranges_are_added_by_the_launch_that_reads_them"],
+                                 env=env, capture_output=True, text=True, timeout=600)
+            assert res.returncode == 0, res.stdout[-3000:] + res.stderr[-2000:]
+            return
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of("ranges", jit))
+    batch, hid, rows, n0, R = 64, 128, 192, 64, 8
+    gates = [(rng.standard_normal(batch * hid) / 8).astype(np.float32) for _ in range(4)]
+    w = (rng.standard_normal(rows * 4 * hid) / 8).astype(np.float32)
+    full = np.concatenate([g.reshape(batch, hid) for g in gates], axis=1).astype(np.float64) @ w.reshape(rows, 4 * hid).astype(np.float64).T
+    ref = full[:, n0:]
+    M, N, K = batch, rows - n0, hid
+    dg = [ctx.upload(g) for g in gates]
+    dw = ctx.upload(w)
+    a, lda = [d.ptr for d in dg], [hid] * 4
+    b, ldb = [dw.ptr + (n0 * 4 * hid + g * hid) * 4 for g in range(4)], [4 * hid] * 4
+    guard = 64
+    parts = ctx.upload(np.full(R * M * N + 2 * guard, 777, np.float32))
+    ctx.gemm_terms_ranges(capi.FLOAT, M, N, K, a, lda, 0, b, ldb, 1, R, parts.ptr + guard * 4)
+    got = parts.get()
+    assert (got[:guard] == 777).all() and (got[-guard:] == 777).all()
+    ranges = got[guard:-guard].reshape(R, M, N)
+    want = ranges[0].copy()
+    for r in range(1, R):
+        want = want + ranges[r]  # fp32, in range order
+    assert_acc_close(want, ref, ACC_RTOL)
+    # every range is the product over its part of K
+    for r in (0, R - 1):
+        k0, k1 = r * 4 * K // R, (r + 1) * 4 * K // R
+        cat = np.concatenate([g.reshape(batch, hid) for g in gates], axis=1).astype(np.float64)
+        piece = cat[:, k0:k1] @ w.reshape(rows, 4 * hid).astype(np.float64).T[k0:k1, n0:]
+        assert_acc_close(ranges[r], piece, ACC_RTOL)
+    other = (rng.standard_normal(M * N) / 8).astype(np.float32)
+    dother = ctx.upload(other)
+    # out0 = sum of the ranges * other; out1 = sum of the ranges (128-bit lanes)
+    out0, out1 = ctx.empty(M * N, np.float32), ctx.empty(M * N, np.float32)
+    leaf = {"ptr": parts.ptr, "offset": guard, "nsum": R, "sum_stride": M * N}
+    prog = [("MUL", capi.FX_LEAF0, capi.FX_LEAF0 + 1, capi.FX_NONE, capi.FX_REG0), ("STORE", capi.FX_REG0, capi.FX_NONE, capi.FX_NONE, 0),
+            ("STORE", capi.FX_LEAF0, capi.FX_NONE, capi.FX_NONE, 1)]
+    ctx.ew_fusedx(capi.FLOAT, [N, M], [leaf, {"ptr": dother.ptr}], prog, [out0.ptr, out1.ptr])
+    np.testing.assert_array_equal(out1.get().reshape(M, N), want)
+    np.testing.assert_array_equal(out0.get().reshape(M, N), want * other.reshape(M, N))
+    # a window of the sums read through a border of zeros, one element per lane:
+    # rows 3.. and columns 5.. of the result, shifted by (2, 1) into a [N - 4, M - 2] box
+    shape = [N - 4, M - 2]
+    view = {"ptr": parts.ptr, "offset": guard + 3 * N + 5 - (2 * N + 1), "stride": [1, N] + [0] * 6,
+            "lo": [1, 2] + [0] * 6, "hi": [N - 5 + 1, M - 3 + 2] + [1] * 6, "nsum": R, "sum_stride": M * N}
+    out2 = ctx.empty(shape[0] * shape[1], np.float32)
+    ctx.ew_fusedx(capi.FLOAT, shape, [view], [("NEG", capi.FX_LEAF0, capi.FX_NONE, capi.FX_NONE, capi.FX_REG0),
+                                              ("STORE", capi.FX_REG0, capi.FX_NONE, capi.FX_NONE, 0)], [out2.ptr])
+    expect = np.zeros((shape[1], shape[0]), np.float32)
+    hi_m, hi_n = min(shape[1], M - 3 + 2), min(shape[0], N - 5 + 1)
+    expect[2:hi_m, 1:hi_n] = want[3:3 + hi_m - 2, 5:5 + hi_n - 1]
+    np.testing.assert_array_equal(out2.get().reshape(shape[1], shape[0]), -expect)
+    # shapes the matrix cores do not take are refused, not approximated
+    with pytest.raises(RuntimeError, match="tcg_gemm_terms_ranges"):
+        ctx.gemm_terms_ranges(capi.FLOAT, M, N, K, a, lda, 0, b, ldb, 1, 3, parts.ptr + guard * 4)
+    with pytest.raises(RuntimeError, match="tcg_gemm_terms_ranges"):
+        ctx.gemm_terms_ranges(capi.INT32, M, N, K, a, lda, 0, b, ldb, 1, R, parts.ptr + guard * 4)

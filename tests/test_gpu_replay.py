@@ -420,6 +420,44 @@ def test_products_over_parts_read_each_part_where_the_walk_does():
     assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
 
 
+def test_groups_add_the_k_ranges_of_a_product_they_read():
+    """A product with a transposed operand, few results and a long K runs as K
+    ranges on separate workgroups.  Where elementwise groups reading through
+    SLICEs are all that reads it, the recording never lays the result out: the
+    ranges stay side by side (tcg_gemm_terms_ranges) and the groups add them up
+    in range order while they load.  Against the walk (1e-5 of the largest
+    entry) and against numpy in double (1e-4); the second reader goes through a
+    PAD of a narrower SLICE, so its leaf starts off the window's first row."""
+    rng = np.random.default_rng(47)
+    g0s = [rng.uniform(-1, 1, 128 * 64).astype(np.float32) for _ in range(3)]
+    g1v, sv = rng.uniform(-1, 1, 128 * 64).astype(np.float32), rng.uniform(-1, 1, 128 * 64).astype(np.float32)
+    wv = rng.uniform(-1, 1, 256 * 192).astype(np.float32)
+
+    def build(g, api):
+        g0, g1 = g.variable(g0s[0], [128, 64], "g0"), g.variable(g1v, [128, 64], "g1")
+        wt = g.variable(wv, [256, 192], "wt")
+        scale = g.variable(sv, [128, 64], "scale")
+        back = api.contract(api.concat([g0, g1], 0), wt, ((0, 0),))
+        first = api.mul(api.slice(back, 64, 128, 0), scale)
+        second = api.add(api.pad(api.slice(api.slice(back, 96, 64, 0), 8, 40, 1), [[32, 32], [8, 16]]), scale)
+        lines = g.launch_plan([first, second])
+        assert lines[0].startswith("parts CONCAT+CONTRACT x2+SLICE ranges="), lines
+        return [first, second], g0
+
+    results, stats = run_both(build, g0s, kinds=("plain", "replay_launches", "replay"))
+    assert_close_to_walk(results)
+    cat = np.concatenate([g0s[2].reshape(64, 128), g1v.reshape(64, 128)], axis=1).astype(np.float64)
+    full = cat @ wv.reshape(192, 256).astype(np.float64).T        # [64, 192]
+    want = full[:, 64:192] * sv.reshape(64, 128)
+    got = results["replay"][2][0].reshape(64, 128)
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    padded = np.zeros((64, 128))
+    padded[8:48, 32:96] = full[8:48, 96:160]
+    want2 = padded + sv.reshape(64, 128)
+    got2 = results["replay"][2][1].reshape(64, 128)
+    assert np.abs(got2 - want2).max() <= 1e-4 * np.abs(want2).max()
+
+
 def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
     from tenncor_amd import configs
     rng = np.random.default_rng(18)

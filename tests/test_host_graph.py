@@ -441,13 +441,16 @@ def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
     targets = configs.config4_lstm(g, seq=5, batch=64, nin=32, hid=64)[0]
     lines = g.launch_plan(targets)
     assert lines.count("parts CONCAT+CONTRACT x3") == 5, lines   # 32 + 64 joined columns in chunks of 32
-    assert lines.count("parts ADD+CONTRACT x4+SLICE") == 4, lines  # only the columns of h are read back
+    # only the columns of h are read back, and the groups that read them add the product's two K ranges up
+    assert lines.count("parts ADD+CONTRACT x4+SLICE ranges=2") == 4, lines
     assert lines.count("blocks CONTRACT x5 2x4") == 1, lines
     assert not any(l.startswith(("summed", "swapped", "node CONTRACT", "node CONCAT", "group CONCAT ")) for l in lines), lines
     steps = parse_plan(lines)
     alone = sum(1 for s in steps if s[0] in ("node", "swapped", "viewed", "summed", "parts", "blocks"))
     stores = sum(s[2]["stores"] for s in steps if s[0] == "group")
-    assert alone + stores + steps[-1][2]["n"] == g.count_functors(targets)
+    # (a product that leaves its K ranges to its readers is a launch and never holds a value: counted twice)
+    ranged = sum(" ranges=" in l for l in lines)
+    assert alone + stores + steps[-1][2]["n"] - ranged == g.count_functors(targets)
     # below the sizes the matrix cores take, everything stays as it was
     small = configs.config4_lstm(g, seq=5, batch=6, nin=8, hid=12)[0]
     assert not any(l.startswith(("parts", "blocks")) for l in g.launch_plan(small))
@@ -464,6 +467,18 @@ def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
     # a concatenation that an elementwise node reads as well is laid out once, for everybody
     lines = g.launch_plan([api.add(p1, p2), api.neg(z)])
     assert not any(l.startswith("parts") for l in lines) and lines.count("node MATMUL") == 2, lines
+    # K ranges are left to the readers only where elementwise groups reading through SLICEs are all there is:
+    # a transposed operand, few results, a long K
+    g0, g1 = var(g, [128, 64], np.float32, "g0"), var(g, [128, 64], np.float32, "g1")
+    wt = var(g, [256, 192], np.float32, "wt")
+    scale = var(g, [128, 64], np.float32, "scale")
+    back = api.contract(api.concat([g0, g1], 0), wt, ((0, 0),))      # [192, 64], K = 256 along the memory of both
+    lines = g.launch_plan([api.mul(api.slice(back, 64, 128, 0), scale)])
+    assert lines[0] == "parts CONCAT+CONTRACT x2+SLICE ranges=2" and lines[1].startswith("group MUL leaves=2"), lines
+    # ... a reduction reads the slice as a tensor: the product adds its ranges up itself, into the window
+    back2 = api.contract(api.concat([g0, g1], 0), wt, ((0, 0),))
+    lines = g.launch_plan([api.reduce_sum(api.slice(back2, 64, 128, 0), 0, 1)])
+    assert lines[0] == "parts CONCAT+CONTRACT x2+SLICE", lines
     # an assignment to a part between the concatenation and a product that reads it:
     # the concatenation holds the old value, the part's buffer the new one
     upd = api.assign(x, c)
