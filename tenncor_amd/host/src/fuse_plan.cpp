@@ -240,6 +240,7 @@ struct Planner final
 		maxpos_.resize(nodes_.size());
 		members_.resize(nodes_.size());
 		deps_.resize(nodes_.size());
+		vdeps_.resize(nodes_.size());
 		stamp_.assign(nodes_.size(), 0);
 	}
 
@@ -1466,6 +1467,18 @@ struct Planner final
 			std::vector<int> ins;
 			inputs_of((int) i, ins);
 			deps_[i].insert(ins.begin(), ins.end());
+			// what the node reads through a folded view it reads from memory, at other
+			// coordinates than its own: that value must come from an earlier launch
+			for (int a : n.args)
+			{
+				while (a >= 0 && is_alias(a)) { a = nodes_[a].args[0]; }
+				if (a >= 0 && nodes_[a].kind == VIEW && nodes_[a].absorbed)
+				{
+					std::vector<int> through;
+					inputs_of(a, through);
+					vdeps_[i].insert(through.begin(), through.end());
+				}
+			}
 			order_around_writes((int) i);
 			if (n.kind != EW) { continue; }
 			members_[i].push_back((int) i);
@@ -1493,6 +1506,8 @@ struct Planner final
 	/// No launch outside the two units may sit between them
 	bool mergeable (int g, int cand)
 	{
+		for (int d : vdeps_[g]) { if (find(d) == cand) { return false; } }
+		for (int d : vdeps_[cand]) { if (find(d) == g) { return false; } }
 		for (int d : deps_[g])
 		{
 			d = find(d);
@@ -1521,6 +1536,8 @@ struct Planner final
 		for (int d : deps_[other]) { if (find(d) != root) { deps.insert(find(d)); } }
 		deps_[root] = deps;
 		deps_[other].clear();
+		vdeps_[root].insert(vdeps_[other].begin(), vdeps_[other].end());
+		vdeps_[other].clear();
 		minpos_[root] = std::min(minpos_[root], minpos_[other]);
 		maxpos_[root] = std::max(maxpos_[root], maxpos_[other]);
 		return root;
@@ -2011,6 +2028,7 @@ struct Planner final
 	std::vector<int> uf_, minpos_, maxpos_;
 	std::vector<std::vector<int>> members_;
 	std::vector<std::set<int>> deps_;
+	std::vector<std::set<int>> vdeps_;   // unit -> units whose results it reads through folded views
 	std::vector<size_t> stamp_;
 	size_t clock_ = 0;
 	// buffers rewritten by ASSIGN* nodes of the pass

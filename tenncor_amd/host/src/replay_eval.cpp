@@ -172,7 +172,12 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		auto dev = &static_cast<iEigen&>(f->device());
 		if (false == dev->replayable()) { return nullptr; }
 		plan->devs.push_back(dev);
-		if (false == egen::is_idempotent((egen::_GENERATED_OPCODE) f->get_opcode().code_))
+		// nodes that run at every pass of the walk: the non-idempotent ones, and
+		// plain ASSIGN too, which leaves its target newer than itself
+		// (tenncor/eteq/functor.hpp:246-268 compares the operands' versions with
+		// the node's; internal/eigen/device.hpp:508-544 bumps the target's)
+		auto op = (egen::_GENERATED_OPCODE) f->get_opcode().code_;
+		if (false == egen::is_idempotent(op) || op == egen::ASSIGN)
 		{
 			plan->effects.push_back(dev);
 		}

@@ -458,6 +458,186 @@ def test_groups_add_the_k_ranges_of_a_product_they_read():
     assert np.abs(got2 - want2).max() <= 1e-4 * np.abs(want2).max()
 
 
+def random_products_graph(g, api, seed, x0, with_updates=False):
+    """Matrix products over concatenations, gate-like SLICEs of their results
+    and gradients of it all, at sizes where the planner rewrites what it can
+    (products over parts, windows, K ranges left to the groups, sums of
+    products): returns (targets, fed variable, plan lines).  `with_updates`
+    adds assignments to operands in between; everything then hangs under ONE
+    root, a sum whose terms come in a seeded order, because the order in which
+    an evaluator visits several targets is its own business
+    (internal/teq/evaluator.hpp:33-45 walks a set) and with it which side of an
+    assignment a read in another target falls on."""
+    rng = np.random.default_rng(seed)
+    batch = 64
+    widths = [32, 48, 64, 96, 128]
+
+    def variable(width, name, scale=1.0, rows=batch):
+        data = rng.uniform(-scale, scale, width * rows).astype(np.float32)
+        return g.variable(data, [width, rows], name)
+
+    x = g.variable(x0, [64, batch], "x")
+    pool = [x] + [variable(int(rng.choice(widths)), "v%d" % k) for k in range(3)]
+    variables = list(pool)
+    weights = []
+    results = []
+    updates = []
+    for step in range(int(rng.integers(3, 6))):
+        a, b = (pool[int(i)] for i in rng.choice(len(pool), 2, replace=False))
+        z = api.concat([a, b], 0)
+        k = z.shape[0]
+        n = int(rng.choice([64, 128, 192, 256]))
+        kind = int(rng.integers(0, 3))
+        if kind == 0:
+            w = variable(n, "w%d" % step, 0.2, rows=k)           # [n, k]
+            p = api.matmul(z, w)
+        elif kind == 1:
+            w = variable(k, "w%d" % step, 0.2, rows=n)           # [k, n]: K along the memory of both
+            p = api.contract(z, w, ((0, 0),))
+        else:
+            w = variable(n, "w%d" % step, 0.2, rows=k)
+            p = api.contract(z, w, ((0, 1),))
+        weights.append(w)
+        # gates: halves of the result through SLICEs, recombined elementwise
+        half = n // 2
+        lo, hi = api.slice(p, 0, half, 0), api.slice(p, half, half, 0)
+        h = api.mul(api.sigmoid(lo), api.tanh(hi))                # [half, batch]
+        if rng.uniform() < 0.4:
+            h = api.add(h, api.pad(api.slice(hi, 8, half - 24, 0), [[8, 16]]))
+        results.append(h)
+        pool.append(h)
+        if with_updates and rng.uniform() < 0.5:
+            target = variables[int(rng.integers(0, len(variables)))]
+            source = next((t for t in reversed(pool) if t.shape == target.shape and t is not target), None)
+            if source is not None:
+                updates.append(api.reduce_sum(api.assign(target, api.tanh(source))))
+    loss = api.reduce_sum(api.square(results[0]))
+    for r in results[1:]:
+        loss = api.add(loss, api.reduce_sum(api.square(r)))
+    grads = g.derive(loss, weights[:2] + [x])
+    targets = [loss] + grads
+    if with_updates:
+        # (ASSIGN has no derivative: the updates stand beside the loss)
+        terms = [loss] + [api.reduce_sum(api.square(gr)) for gr in grads] + updates
+        order = rng.permutation(len(terms))
+        root = terms[int(order[0])]
+        for i in order[1:]:
+            root = api.add(root, terms[int(i)])
+        targets = [root]
+    return targets, x, g.launch_plan(targets)
+
+
+@pytest.mark.parametrize("with_updates", [False, True], ids=["pure", "updates"])
+@pytest.mark.parametrize("seed", range(10))
+def test_random_graphs_of_products_over_parts_follow_the_walk(seed, with_updates):
+    """Seeded random graphs of the shapes the planner rewrites (products over
+    CONCATs, SLICEd gates, their gradients: ADDs of PADs, sums of products,
+    transposed weights; with assignments to operands in between in the second
+    variant), three passes with new inputs each: the recording and its replays
+    against the node-by-node walk at 1e-4 of each target's largest entry (sums
+    over K come in another order where a rewrite applies; a read on the wrong
+    side of an update, or of a value its own launch is still to write, is an
+    error of order one)."""
+    rng = np.random.default_rng(1000 + seed)
+    feeds = [rng.uniform(-1, 1, 64 * 64).astype(np.float32) for _ in range(3)]
+    seen = {}
+
+    def build(g, api):
+        targets, x, lines = random_products_graph(g, api, seed, feeds[0], with_updates)
+        seen["lines"] = lines
+        return targets, x
+
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+    assert stats["replay"]["record_failures"] == 0 and stats["replay"]["replayed"] >= 1, stats
+    assert_close_to_walk(results, tol=1e-4)
+
+
+def test_random_graphs_exercise_the_rewrites():
+    """The generator above reaches every rewrite at least once over its seeds
+    (host logic only: the plans)."""
+    from tenncor_amd import graph
+    kinds = set()
+    for seed in range(10):
+        g = graph.Graph()
+        try:
+            _, _, lines = random_products_graph(g, graph.Api(g), seed, np.zeros(64 * 64, np.float32))
+        finally:
+            g.close()
+        for line in lines:
+            kinds.add(line.split(" ")[0])
+            if " ranges=" in line:
+                kinds.add("ranges")
+            if line.startswith("parts") and "+SLICE" in line:
+                kinds.add("window")
+    assert {"parts", "ranges", "window", "group"} <= kinds, kinds
+
+
+def test_a_view_of_a_group_result_is_read_after_the_group_has_stored_it():
+    """h is computed by an elementwise group; y adds h and PAD(SLICE(h)) -- the
+    shape the gradient of a SLICE added back onto its operand takes.  The view
+    is read from memory, so y's launch must come after the one that stores h;
+    in one launch it would read what the buffer held before."""
+    rng = np.random.default_rng(53)
+    feeds = [rng.uniform(-1, 1, 64 * 16).astype(np.float32) for _ in range(3)]
+    bv = rng.uniform(-1, 1, 64 * 16).astype(np.float32)
+
+    def build(g, api):
+        a, b = g.variable(feeds[0], [64, 16], "a"), g.variable(bv, [64, 16], "b")
+        h = api.mul(api.sigmoid(a), api.tanh(b))
+        y = api.add(h, api.pad(api.slice(h, 8, 40, 0), [[8, 16]]))
+        return [api.square(y), api.neg(h)], a
+
+    results, _ = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+    assert_same_bits(results)
+    h = (1 / (1 + np.exp(-feeds[2].astype(np.float64)))) * np.tanh(bv.astype(np.float64))
+    h = h.reshape(16, 64)
+    y = h.copy()
+    y[:, 8:48] += h[:, 8:48]
+    assert np.abs(results["replay"][2][0].reshape(16, 64) - y * y).max() <= 1e-5
+
+
+def test_a_recording_with_a_plain_assign_runs_at_every_pass():
+    """ASSIGN leaves its target newer than itself (internal/eigen/device.hpp:508-544
+    bumps the target's version; tenncor/eteq/functor.hpp:246-268 compares the
+    operands' versions with the node's), so the walk runs it, and everything
+    that reads the target, at every pass -- also when no input was fed in
+    between.  A state that feeds back on itself then moves with every
+    evaluation; the recording must do the same and not take the pass for
+    unchanged."""
+    from tenncor_amd import graph
+    rng = np.random.default_rng(59)
+    s0 = rng.uniform(-1, 1, 32 * 8).astype(np.float32)
+    wv = rng.uniform(-0.5, 0.5, 32 * 32).astype(np.float32)
+    seen = {}
+    for kind in ("plain", "replay_launches", "replay"):
+        graph.set_evaluator(kind)
+        g = graph.Graph()
+        try:
+            api = graph.Api(g)
+            state = g.variable(s0, [32, 8], "state")
+            w = g.variable(wv, [32, 32], "w")
+            nxt = api.tanh(api.matmul(state, w))
+            root = api.reduce_sum(api.square(api.assign(state, nxt)))
+            rows = []
+            for _ in range(5):
+                g.evaluate([root])
+                rows.append(float(root.get()[0]))
+            seen[kind] = rows
+            if kind != "plain":
+                st = graph.evaluator_stats()
+                assert st["replayed"] >= 3 and st["skipped"] == 0, st
+        finally:
+            g.close()
+            graph.set_evaluator("plain")
+    assert len(set(seen["plain"])) == 5          # the state moves
+    x = s0.reshape(8, 32).astype(np.float64)
+    for k in range(5):
+        x = np.tanh(x @ wv.reshape(32, 32).astype(np.float64))
+        assert abs(seen["plain"][k] - (x * x).sum()) <= 1e-4 * (x * x).sum()
+    for kind in ("replay_launches", "replay"):
+        assert np.allclose(seen[kind], seen["plain"], rtol=1e-5, atol=0), (kind, seen)
+
+
 def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
     from tenncor_amd import configs
     rng = np.random.default_rng(18)

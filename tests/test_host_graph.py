@@ -486,3 +486,22 @@ def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
     t = api.add(api.add(q1, api.matmul(api.concat([upd, h], 0), w1)), q2)
     lines = g.launch_plan([t])
     assert any(l.startswith(("group CONCAT", "node CONCAT")) for l in lines) and lines.count("node MATMUL") >= 2, lines
+
+
+def test_launch_plan_reads_a_view_of_a_group_result_in_a_later_launch(g, api):
+    """A node that reads another elementwise node through a folded view reads it
+    from memory, at other coordinates than its own: the two cannot share a
+    launch (whose loads all come before its stores), even when the reader also
+    reads the same node directly.  The gradient of a SLICE that was added back
+    onto its own operand has this shape."""
+    a = var(g, [64, 16], np.float32, "a")
+    b = var(g, [64, 16], np.float32, "b")
+    h = api.mul(api.sigmoid(a), api.tanh(b))
+    y = api.add(h, api.pad(api.slice(h, 8, 40, 0), [[8, 16]]))
+    lines = g.launch_plan([api.square(y)])
+    steps = [s for s in parse_plan(lines) if s[0] == "group"]
+    assert len(steps) == 2 and "MUL" in steps[0][1] and steps[0][2]["stores"] == 1, lines
+    assert steps[1][1] == ["ADD", "SQUARE"] and steps[1][2]["leaves"] == 2, lines
+    # through an IDENTITY (the same coordinates) the value stays in a register
+    lines = g.launch_plan([api.add(h, api.identity(h))])
+    assert len([l for l in lines if l.startswith("group")]) == 1, lines
