@@ -435,12 +435,21 @@ struct HipOp final : public iTmpEigen<T>
 		std::vector<teq::Once<const void*>> onces;
 		ptrs.reserve(args_.size());
 		onces.reserve(args_.size());
-		for (auto& arg : args_)
+		for (size_t k = 0, n = args_.size(); k < n; ++k)
 		{
-			teq::Once<const void*> argdata = eigen_ref(*arg).odevice();
+			// an operand that appears twice (MUL(x, x)) is one consumer of x, as the
+			// producer counts them (a set of observers): one read, one pointer
+			size_t same = 0;
+			while (same < k && args_[same] != args_[k]) { ++same; }
+			if (same < k)
+			{
+				ptrs.push_back(ptrs[same]);
+				continue;
+			}
+			teq::Once<const void*> argdata = eigen_ref(*args_[k]).odevice();
 			if (nullptr == argdata.get())
 			{
-				global::fatalf("operand %s has no data", arg->to_string().c_str());
+				global::fatalf("operand %s has no data", args_[k]->to_string().c_str());
 			}
 			ptrs.push_back(argdata.get());
 			onces.push_back(std::move(argdata));
@@ -499,9 +508,16 @@ struct HostOp final : public iTmpEigen<T>
 		else { this->data_.extend_life(ttl); }
 		std::vector<const void*> ptrs;
 		std::vector<teq::Once<const void*>> onces;
-		for (auto& arg : args_)
+		for (size_t k = 0, n = args_.size(); k < n; ++k)
 		{
-			teq::Once<const void*> argdata = arg->device().odata();
+			size_t same = 0;
+			while (same < k && args_[same] != args_[k]) { ++same; }
+			if (same < k)
+			{
+				ptrs.push_back(ptrs[same]);
+				continue;
+			}
+			teq::Once<const void*> argdata = args_[k]->device().odata();
 			ptrs.push_back(argdata.get());
 			onces.push_back(std::move(argdata));
 		}

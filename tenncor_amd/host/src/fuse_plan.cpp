@@ -251,6 +251,17 @@ struct Planner final
 		return false == (n.kind == VIEW && n.absorbed) && false == n.ranged;
 	}
 
+	/// Operand k of a node is the first occurrence of that tensor among its operands:
+	/// a node is one consumer of a tensor however often it names it (MUL(x, x))
+	static bool first_occurrence (const Node& n, size_t k)
+	{
+		for (size_t j = 0; j < k; ++j)
+		{
+			if (n.arg_tens[j] == n.arg_tens[k]) { return false; }
+		}
+		return true;
+	}
+
 	bool is_alias (int i) const
 	{
 		const Node& n = nodes_[i];
@@ -1333,7 +1344,7 @@ struct Planner final
 		for (size_t k = 0; k < 2; ++k)
 		{
 			int a = c.args[k];
-			if (a >= 0 && holds_value(a))
+			if (a >= 0 && holds_value(a) && first_occurrence(c, k))
 			{
 				call.reads.push_back(c.arg_tens[k].get());
 			}
@@ -1751,7 +1762,7 @@ struct Planner final
 				int a = n.args[k];
 				if (a < 0) { continue; }
 				bool materialised = inside(a) ? stored[pos[a]] : holds_value(a);
-				if (materialised) { out.reads.push_back(n.arg_tens[k].get()); }
+				if (materialised && first_occurrence(n, k)) { out.reads.push_back(n.arg_tens[k].get()); }
 			}
 		}
 		return true;
@@ -1804,7 +1815,7 @@ struct Planner final
 						int a = nodes_[c].args[k];
 						if (a < 0) { continue; }
 						if (nodes_[a].parts_folded) { mark_parts_user(a, step.parts, last_parts); }
-						else if (holds_value(a))
+						else if (holds_value(a) && first_occurrence(nodes_[c], k))
 						{
 							call.reads.push_back(nodes_[c].arg_tens[k].get());
 						}
@@ -1837,7 +1848,7 @@ struct Planner final
 				for (size_t k = 0; k < 2; ++k)
 				{
 					int a = c.args[k];
-					if (a >= 0 && holds_value(a))
+					if (a >= 0 && holds_value(a) && first_occurrence(c, k))
 					{
 						call.reads.push_back(c.arg_tens[k].get());
 					}
@@ -1880,7 +1891,7 @@ struct Planner final
 					for (size_t j = 0; j < 2; ++j)
 					{
 						int operand = c.args[j];
-						if (operand >= 0 && holds_value(operand))
+						if (operand >= 0 && holds_value(operand) && first_occurrence(c, j))
 						{
 							call.reads.push_back(c.arg_tens[j].get());
 						}

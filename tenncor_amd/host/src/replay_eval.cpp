@@ -1,5 +1,7 @@
 // Recording and replaying whole evaluation passes (see replay_eval.hpp).
 #include "replay_eval.hpp"
+
+#include <unordered_map>
 #include "fuse_plan.hpp"
 
 #include <algorithm>
@@ -37,6 +39,7 @@ struct ReplayEvaluator::Plan final
 	std::vector<iEigen*> devs;
 	std::vector<iEigen::LifeState> after;
 	std::vector<iEigen*> effects; // launches with host-side effects (ASSIGN*)
+	bool plain_assigns = false;   // the pass holds a plain ASSIGN, which the walk may skip
 	std::vector<iEigen*> targets;
 	std::vector<teq::iLeaf*> leaves;
 	std::vector<const void*> leaf_ptrs;
@@ -103,6 +106,54 @@ void ReplayEvaluator::evict (void)
 	}
 }
 
+/// Would the walk skip a plain ASSIGN among `funcs` (children first) at this
+/// pass?  It runs a node whose operands are newer than the node
+/// (tenncor/eteq/functor.hpp:246-268); an ASSIGN leaves its target at least one
+/// version past its source (eteq/variable.hpp:129-132), so with two writers of
+/// one variable, or a target that was fed after the source last moved, an
+/// ASSIGN can find nothing newer than itself and keep out of a pass in which
+/// another writer of its target runs.  A recording runs every node, so such a
+/// pass must be walked.  Versions are carried forward as the walk would.
+static bool walk_skips_an_assign (const std::vector<Observable*>& funcs, size_t max_version)
+{
+	std::unordered_map<const teq::iTensor*,size_t> moved;
+	auto version_of = [&](const teq::iTensor* tens)
+	{
+		auto it = moved.find(tens);
+		return it == moved.end() ? tens->get_meta().state_version() : it->second;
+	};
+	for (Observable* f : funcs)
+	{
+		auto op = (egen::_GENERATED_OPCODE) f->get_opcode().code_;
+		auto args = f->get_args();
+		size_t wanted = 0;
+		for (auto& arg : args) { wanted = std::max(wanted, version_of(arg.get())); }
+		const size_t held = f->get_meta().state_version();
+		if (wanted <= held && false == egen::is_idempotent(op)) { wanted = held + 1; }
+		wanted = std::min(wanted, max_version);
+		const bool runs = held < wanted;
+		if (runs) { moved[f] = wanted; }
+		if (op < egen::ASSIGN || op > egen::ASSIGN_DIV) { continue; }
+		if (false == runs)
+		{
+			if (op == egen::ASSIGN) { return true; }
+			continue;
+		}
+		// the target: through the nodes that stand for their operand's buffer
+		const teq::iTensor* target = args.front().get();
+		while (auto inner = dynamic_cast<const teq::iFunctor*>(target))
+		{
+			auto code = (egen::_GENERATED_OPCODE) inner->get_opcode().code_;
+			bool alias = (code >= egen::ASSIGN && code <= egen::ASSIGN_DIV) || code == egen::IDENTITY ||
+				code == egen::RESHAPE || code == egen::SLICE;
+			if (false == alias) { break; }
+			target = inner->get_args().front().get();
+		}
+		moved[target] = std::max(version_of(target), version_of(args.back().get()) + 1);
+	}
+	return false;
+}
+
 void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targets, const teq::TensSetT& ignored)
 {
 	auto gpu = dynamic_cast<Device*>(&device);
@@ -131,6 +182,7 @@ void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 		plain(device, targets, ignored);
 		return;
 	}
+	bool checked = false;
 	if (nullptr == slot.plan)
 	{
 		if (slot.seen++ < warm_passes_)
@@ -139,6 +191,7 @@ void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 			return;
 		}
 		slot.plan = record(*gpu, key, targets);
+		checked = true; // record() looks before it moves any version
 		if (nullptr == slot.plan)
 		{
 			slot.unplannable = true;
@@ -148,7 +201,8 @@ void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 		stats_.reserved_bytes += slot.plan->bytes;
 		evict();
 	}
-	if (false == replay(*gpu, *slot.plan))
+	bool walk = false == checked && slot.plan->plain_assigns && walk_skips_an_assign(slot.plan->funcs, gpu->max_version_);
+	if (walk || false == replay(*gpu, *slot.plan))
 	{
 		stats_.reserved_bytes -= slot.plan->bytes;
 		release(*slot.plan);
@@ -166,6 +220,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 	auto plan = std::make_unique<Plan>();
 	plan->funcs = collector.funcs_;
 	plan->leaves = collector.leaves_;
+	if (walk_skips_an_assign(plan->funcs, device.max_version_)) { return nullptr; }
 	for (Observable* f : plan->funcs)
 	{
 		// device() builds the launch closure of a functor that has none yet
@@ -181,6 +236,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		{
 			plan->effects.push_back(dev);
 		}
+		plan->plain_assigns = plan->plain_assigns || op == egen::ASSIGN;
 		if (targets.count(f)) { plan->targets.push_back(dev); }
 	}
 	// leaves reach the device before recording starts: uploads are not recorded

@@ -506,8 +506,9 @@ def random_products_graph(g, api, seed, x0, with_updates=False):
             h = api.add(h, api.pad(api.slice(hi, 8, half - 24, 0), [[8, 16]]))
         results.append(h)
         pool.append(h)
-        if with_updates and rng.uniform() < 0.5:
-            target = variables[int(rng.integers(0, len(variables)))]
+        if with_updates and rng.uniform() < 0.5 and variables:
+            # (each variable at most once: two assignments to one variable keep a pass on the walk)
+            target = variables.pop(int(rng.integers(0, len(variables))))
             source = next((t for t in reversed(pool) if t.shape == target.shape and t is not target), None)
             if source is not None:
                 updates.append(api.reduce_sum(api.assign(target, api.tanh(source))))
@@ -636,6 +637,138 @@ def test_a_recording_with_a_plain_assign_runs_at_every_pass():
         assert abs(seen["plain"][k] - (x * x).sum()) <= 1e-4 * (x * x).sum()
     for kind in ("replay_launches", "replay"):
         assert np.allclose(seen[kind], seen["plain"], rtol=1e-5, atol=0), (kind, seen)
+
+
+def random_elementwise_graph(g, api, seed, x0, shape, np_dtype, with_updates):
+    """Elementwise nodes over views of each other (EXTEND of reduced rows,
+    SLICE + PAD back to shape, transposes, CONCATs of halves, SELECT, IDENTITY)
+    and, with `with_updates`, assignments to the variables in between, all
+    under one root."""
+    rng = np.random.default_rng(seed)
+    a, b = shape
+    integer = np.issubdtype(np_dtype, np.integer)
+
+    def draw(n):
+        if integer:
+            return rng.integers(-9, 10, n).astype(np_dtype)
+        return rng.uniform(-1, 1, n).astype(np_dtype)
+
+    x = g.variable(x0, [a, b], "x")
+    variables = [x] + [g.variable(draw(a * b), [a, b], "v%d" % k) for k in range(2)]
+    row = g.variable(draw(a), [a], "row")
+    pool = list(variables)
+    unassigned = list(variables)
+    unary = ["NEG", "SQUARE", "ABS"] + ([] if integer else ["TANH", "SIGMOID"])
+    binary = ["ADD", "SUB", "MUL", "MIN", "MAX"]
+    updates = []
+    for step in range(int(rng.integers(8, 16))):
+        kind = int(rng.integers(0, 9))
+        p = pool[int(rng.integers(0, len(pool)))]
+        q = pool[int(rng.integers(0, len(pool)))]
+        if kind == 0:
+            node = api.unary(str(rng.choice(unary)), p)
+        elif kind == 1:
+            node = api.binary(str(rng.choice(binary)), p, q)
+        elif kind == 2:
+            node = api.binary(str(rng.choice(binary)), p, api.extend(row, 1, [b]))
+        elif kind == 3:
+            lo = int(rng.integers(0, a // 2))
+            ext = int(rng.integers(1, a - lo))
+            node = api.add(q, api.pad(api.slice(p, lo, ext, 0), [[lo, a - lo - ext]]))
+        elif kind == 4:
+            node = api.sub(api.permute(api.mul(api.permute(p, [1, 0]), api.permute(q, [1, 0])), [1, 0]), p)
+        elif kind == 5:
+            summed = api.reduce_sum(p, 1, 1) if integer else api.tanh(api.reduce_sum(p, 1, 1))
+            node = api.binary("ADD" if integer else "MUL", q, api.extend(summed, 1, [b]))
+        elif kind == 6:
+            half = a // 2
+            node = api.concat([api.slice(p, half, a - half, 0), api.slice(q, 0, half, 0)], 0)
+        elif kind == 7:
+            node = api.if_then_else(api.binary("LT", p, q), api.identity(p), api.neg(q))
+        else:
+            node = api.binary("MAX", api.reverse(p, [0]), q)
+        if not integer:
+            node = api.tanh(node)    # keeps every value in (-1, 1)
+        pool.append(node)
+        if with_updates and rng.uniform() < 0.3 and unassigned:
+            # (each variable at most once: two assignments to one variable keep a pass on the walk)
+            target = unassigned.pop(int(rng.integers(0, len(unassigned))))
+            updates.append(api.reduce_sum(api.assign(target, node)))
+    terms = [api.reduce_sum(api.square(t)) for t in pool[len(variables):]] + updates
+    order = rng.permutation(len(terms))
+    root = terms[int(order[0])]
+    for i in order[1:]:
+        root = api.add(root, terms[int(i)])
+    targets = [root] if with_updates else [root, pool[-1], pool[len(pool) // 2]]
+    return targets, x
+
+
+@pytest.mark.parametrize("with_updates", [False, True], ids=["pure", "updates"])
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32], ids=["f32", "i32"])
+@pytest.mark.parametrize("shape", [(12, 10), (96, 80)], ids=["one_kernel", "launches"])
+@pytest.mark.parametrize("seed", range(6))
+def test_random_elementwise_graphs_follow_the_walk(seed, shape, np_dtype, with_updates):
+    """Seeded random graphs of elementwise nodes reading each other through
+    views, at a size whose pass is recorded as the steps of one kernel and at
+    one recorded launch by launch: int32 must equal the walk bit for bit
+    (wrapping arithmetic does not depend on the order of a sum), fp32 launch by
+    launch too (same scalar routines, same order), fp32 as one kernel within
+    1e-5 of the largest entry (its reductions run in index order)."""
+    rng = np.random.default_rng(2000 + seed)
+    n = shape[0] * shape[1]
+    if np_dtype == np.int32:
+        feeds = [rng.integers(-9, 10, n).astype(np.int32) for _ in range(3)]
+    else:
+        feeds = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(3)]
+
+    def build(g, api):
+        return random_elementwise_graph(g, api, seed, feeds[0], shape, np_dtype, with_updates)
+
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+    assert stats["replay"]["record_failures"] == 0 and stats["replay"]["replayed"] >= 1, stats
+    if np_dtype == np.int32:
+        assert_same_bits(results)
+    else:
+        assert_same_bits({k: v for k, v in results.items() if k != "replay"})
+        assert_close_to_walk(results, tol=1e-5)
+
+
+def test_two_assignments_to_one_variable_stay_with_the_walk():
+    """Which of two ASSIGNs to one variable the walk runs at a later pass
+    depends on the versions they left behind (tenncor/eteq/functor.hpp:246-268,
+    eteq/variable.hpp:129-132): with nothing fed, the first runs again and the
+    second, no older than the variable, does not, so the variable ends the
+    pass with the first one's value.  A recording would run both; such passes
+    are never recorded, and every evaluator gives what the walk gives."""
+    from tenncor_amd import graph
+    rng = np.random.default_rng(61)
+    v0, cv, dv = (rng.uniform(-1, 1, 24).astype(np.float32) for _ in range(3))
+    seen = {}
+    for kind in ("plain", "replay_launches", "replay"):
+        graph.set_evaluator(kind)
+        g = graph.Graph()
+        try:
+            api = graph.Api(g)
+            v = g.variable(v0, [6, 4], "v")
+            c, d = g.variable(cv, [6, 4], "c"), g.variable(dv, [6, 4], "d")
+            first = api.reduce_sum(api.assign(v, api.tanh(c)))
+            second = api.reduce_sum(api.assign(v, api.neg(d)))
+            root = api.add(api.add(first, second), api.reduce_sum(api.abs(v)) if hasattr(api, "abs") else api.reduce_sum(api.unary("ABS", v)))
+            rows = []
+            for _ in range(4):
+                g.evaluate([root])
+                rows.append((float(root.get()[0]), v.get().copy()))
+            seen[kind] = rows
+            if kind != "plain":
+                st = graph.evaluator_stats()
+                assert st["recorded"] == 0 and st["plain"] == 4, st
+        finally:
+            g.close()
+            graph.set_evaluator("plain")
+    for kind in ("replay_launches", "replay"):
+        for (a, va), (b, vb) in zip(seen[kind], seen["plain"]):
+            assert a == b
+            np.testing.assert_array_equal(va, vb)
 
 
 def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
