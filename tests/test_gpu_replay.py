@@ -771,6 +771,75 @@ def test_two_assignments_to_one_variable_stay_with_the_walk():
             np.testing.assert_array_equal(va, vb)
 
 
+def random_conv_graph(g, api, seed, x0, dims, np_dtype):
+    """One or two conv2d layers (cfg/tenncor/nn.yml:48-98) with seeded channel
+    counts, kernel extents and zero padding, a nonlinearity between them, the
+    gradients with respect to image and kernels
+    (tenncor/eteq/backprop.hpp:372-439), and an elementwise reader of the first
+    layer's output beside the second layer: the PAD / PERMUTE / REVERSE nodes
+    round every CONV are folded into its launch where convolutions are all
+    that reads them and laid out where something else does."""
+    rng = np.random.default_rng(seed)
+    c, w, h, b = dims
+    integer = np.issubdtype(np_dtype, np.integer)
+
+    def draw(n, scale):
+        if integer:
+            return rng.integers(-3, 4, n).astype(np_dtype)
+        return rng.uniform(-scale, scale, n).astype(np_dtype)
+
+    x = g.variable(x0, [c, w, h, b], "x")
+    o1 = int(rng.choice([4, 8, 12, 16]))
+    k1w, k1h = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    k1 = g.variable(draw(o1 * c * k1w * k1h, 0.3), [o1, c, k1w, k1h], "k1")
+    pad = ((int(rng.integers(0, 2)), int(rng.integers(0, 2))), (int(rng.integers(0, 2)), int(rng.integers(0, 2))))
+    y1 = api.conv2d(x, k1, zero_padding=pad)
+    act = api.relu(y1) if integer or rng.uniform() < 0.5 else api.tanh(y1)
+    kernels = [k1]
+    terms = [api.reduce_sum(api.square(act))]
+    if rng.uniform() < 0.7:
+        o2 = int(rng.choice([4, 8, 16]))
+        k2w = int(rng.integers(1, min(3, act.shape[1]) + 1))
+        k2h = int(rng.integers(1, min(3, act.shape[2]) + 1))
+        k2 = g.variable(draw(o2 * o1 * k2w * k2h, 0.3), [o2, o1, k2w, k2h], "k2")
+        y2 = api.conv2d(act, k2)
+        kernels.append(k2)
+        terms.append(api.reduce_sum(api.square(y2)))
+    loss = terms[0]
+    for t in terms[1:]:
+        loss = api.add(loss, t)
+    grads = g.derive(loss, [x] + kernels)
+    return [loss] + grads, x
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32], ids=["f32", "i32"])
+@pytest.mark.parametrize("dims", [(4, 9, 8, 6), (8, 14, 12, 32)], ids=["direct", "products"])
+@pytest.mark.parametrize("seed", range(6))
+def test_random_conv_graphs_follow_the_walk(seed, dims, np_dtype):
+    """Seeded convolution layers with their gradients, at a size the direct
+    kernels take and at one where the correlations run as matrix products:
+    int32 equals the walk bit for bit by every route (wrapping sums do not
+    depend on their order), fp32 within 1e-5 of each target's largest entry
+    (a convolution that reads an operand through a PERMUTE sums along the
+    operand's memory: another order of the same additions)."""
+    rng = np.random.default_rng(3000 + seed)
+    n = dims[0] * dims[1] * dims[2] * dims[3]
+    if np_dtype == np.int32:
+        feeds = [rng.integers(-4, 5, n).astype(np.int32) for _ in range(3)]
+    else:
+        feeds = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(3)]
+
+    def build(g, api):
+        return random_conv_graph(g, api, seed, feeds[0], dims, np_dtype)
+
+    results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+    assert stats["replay"]["record_failures"] == 0 and stats["replay"]["replayed"] >= 1, stats
+    if np_dtype == np.int32:
+        assert_same_bits(results)
+    else:
+        assert_close_to_walk(results, tol=1e-5)
+
+
 def test_fused_cnn_and_mlp_match_the_walk_bit_for_bit():
     from tenncor_amd import configs
     rng = np.random.default_rng(18)
