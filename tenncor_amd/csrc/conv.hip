@@ -691,8 +691,39 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 	int rc = TCG_OK;
 	if (false == direct_b) { rc = tcg_alloc(ctx, b_bytes, &B); }
 	if (rc == TCG_OK && false == direct_c) { rc = tcg_alloc(ctx, c_bytes, &C); }
-	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, rt_bytes, &RT); }
-	if (rc == TCG_OK && tables) { rc = tcg_alloc(ctx, st_bytes, &ST); }
+	// the tables depend on the plan alone: kept with the context, filled once
+	bool kept_tables = false, fill_tables = tables;
+	if (rc == TCG_OK && tables)
+	{
+		std::string key((const char*) &g, sizeof(g));
+		auto it = ctx->conv_tables.find(key);
+		if (it != ctx->conv_tables.end())
+		{
+			RT = it->second.rows;
+			ST = it->second.sums;
+			kept_tables = true;
+			fill_tables = false;
+		}
+		else if (ctx->conv_table_bytes + rt_bytes + st_bytes <= tcg_ctx::conv_table_limit)
+		{
+			tcg_ctx::ConvTables kept;
+			if (hipMalloc(&kept.rows, rt_bytes) == hipSuccess && hipMalloc(&kept.sums, st_bytes) == hipSuccess)
+			{
+				RT = kept.rows;
+				ST = kept.sums;
+				kept_tables = true;
+				ctx->conv_tables.emplace(key, kept);
+				ctx->conv_table_bytes += rt_bytes + st_bytes;
+			}
+			else
+			{
+				(void) hipGetLastError();
+				if (kept.rows) { (void) hipFree(kept.rows); }
+			}
+		}
+	}
+	if (rc == TCG_OK && tables && false == kept_tables) { rc = tcg_alloc(ctx, rt_bytes, &RT); }
+	if (rc == TCG_OK && tables && false == kept_tables) { rc = tcg_alloc(ctx, st_bytes, &ST); }
 	if (rc == TCG_OK)
 	{
 		unsigned grid = 0;
@@ -704,11 +735,23 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
 			conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
 		}
-		if (tables)
+		if (fill_tables)
 		{
 			uint32_t longest = g.M > g.Sp ? g.M : g.Sp;
-			conv_tables_k<<<(longest + CG_BLOCK - 1) / CG_BLOCK, CG_BLOCK, 0, ctx->stream>>>(g,
+			hipStream_t where = ctx->stream;
+			if (kept_tables && ctx->capturing)
+			{
+				// kept tables are filled once, now, not by the recording at every replay
+				if (nullptr == ctx->side_stream && hipStreamCreate(&ctx->side_stream) != hipSuccess)
+				{
+					(void) hipGetLastError();
+					ctx->side_stream = nullptr;
+				}
+				if (ctx->side_stream) { where = ctx->side_stream; }
+			}
+			conv_tables_k<<<(longest + CG_BLOCK - 1) / CG_BLOCK, CG_BLOCK, 0, where>>>(g,
 				(ConvTabEntry*) RT, (ConvTabEntry*) ST);
+			if (where != ctx->stream) { rc = hipStreamSynchronize(where) == hipSuccess ? TCG_OK : tcg_fail(ctx, TCG_ERR_HIP, "conv tables: %s", hipGetErrorString(hipGetLastError())); }
 		}
 		tcg_conv_operand operand;
 		if (implicit)
@@ -784,8 +827,8 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 	if (A) { tcg_free(ctx, A, a_bytes); }
 	if (B) { tcg_free(ctx, B, b_bytes); }
 	if (C) { tcg_free(ctx, C, c_bytes); }
-	if (RT) { tcg_free(ctx, RT, rt_bytes); }
-	if (ST) { tcg_free(ctx, ST, st_bytes); }
+	if (RT && false == kept_tables) { tcg_free(ctx, RT, rt_bytes); }
+	if (ST && false == kept_tables) { tcg_free(ctx, ST, st_bytes); }
 	if (rc != TCG_OK) { return rc; }
 	TCG_LAUNCH_CHECK(ctx, "conv_gemm");
 	return TCG_OK;
@@ -879,6 +922,7 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 		}
 	}
 	ConvGemmPlan gp;
+	memset((void*) &gp, 0, sizeof(gp)); // its bytes name the tables computed from it
 	const char* gemm_env = getenv("TCG_CONV_GEMM"); // "0": direct kernels only (the parity reference)
 	// (the product route exists for the three default types)
 	if (!(gemm_env && gemm_env[0] == '0') && tcg_default_dtype(dtype) && conv_gemm_plan(p, gp))

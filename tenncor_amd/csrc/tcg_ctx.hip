@@ -107,6 +107,16 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	ctx->pool.release_all();
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
 	if (ctx->rng_state) { (void) hipFree(ctx->rng_state); }
+	if (ctx->side_stream)
+	{
+		(void) hipStreamSynchronize(ctx->side_stream);
+		(void) hipStreamDestroy(ctx->side_stream);
+	}
+	for (auto& kv : ctx->conv_tables)
+	{
+		(void) hipFree(kv.second.rows);
+		(void) hipFree(kv.second.sums);
+	}
 	(void) hipEventDestroy(ctx->ev_begin);
 	(void) hipEventDestroy(ctx->ev_end);
 	(void) hipStreamDestroy(ctx->stream);

@@ -63,6 +63,19 @@ struct tcg_ctx
 	// kernels only so that recorded launches draw fresh values at every replay
 	uint64_t* rng_state = nullptr;
 
+	// row / summed-index tables of convolutions lowered to products, by the bytes
+	// of the plan they were computed from: a pass over the same layers finds them
+	// again instead of launching the kernel that fills them.  Never evicted
+	// (recorded launches keep their addresses); new plans stop being kept at
+	// conv_table_limit bytes.
+	struct ConvTables { void* rows = nullptr; void* sums = nullptr; };
+	std::map<std::string,ConvTables> conv_tables;
+	size_t conv_table_bytes = 0;
+	// tables first met while launches are being recorded are filled at once on
+	// this stream, so that the recording does not fill them again at every replay
+	hipStream_t side_stream = nullptr;
+	static constexpr size_t conv_table_limit = (size_t) 256 << 20;
+
 	// launch capture: the graph being recorded (its arena is pool.recording)
 	tcg_graph* capturing = nullptr;
 };
