@@ -122,8 +122,35 @@ def evaluate_on_gpu():
     graph.set_evaluator("plain")
 
 
+def random_graphs_on_gpu():
+    """The seeded elementwise / view graphs of tests/test_gpu_replay.py in the
+    seven integer types beyond INT32: the recordings (launch by launch, and as
+    one kernel at the small size) against the walk, bit for bit."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("replay_cases", os.path.join(ROOT, "tests", "test_gpu_replay.py"))
+    cases = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(cases)
+    for t in INTS:
+        if t == np.int32:
+            continue
+        for shape in ((12, 10), (96, 80)):
+            for seed in range(3):
+                for with_updates in (False, True):
+                    rng = np.random.default_rng(4000 + seed)
+                    feeds = [rng.integers(-9, 10, shape[0] * shape[1]).astype(t) for _ in range(3)]
+
+                    def build(g, api):
+                        return cases.random_elementwise_graph(g, api, seed, feeds[0], shape, t, with_updates)
+
+                    results, stats = cases.run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
+                    assert stats["replay"]["record_failures"] == 0 and stats["replay"]["replayed"] >= 1, stats
+                    cases.assert_same_bits(results)
+        print("random %s ok" % np.dtype(t).name, flush=True)
+
+
 if __name__ == "__main__":
     build_only()
     if sys.argv[1:] != ["build"]:
         evaluate_on_gpu()
+        random_graphs_on_gpu()
     print("done")

@@ -62,3 +62,5 @@ def test_graphs_of_every_type_evaluate_bit_exact_on_the_gpu():
             for n in (1221, 36900):
                 assert "%s %s %d ok" % (evaluator, name, n) in out
         assert "%s mixed ok" % evaluator in out
+    for name in ("int8", "uint8", "int16", "uint16", "uint32", "int64", "uint64"):
+        assert "random %s ok" % name in out
