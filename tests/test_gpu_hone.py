@@ -233,3 +233,75 @@ def test_optimised_cnn_training_step_equals_the_reference_graph(g):
     assert _lines(g.to_string(root)) == _expected("cnn_layer.txt")
     g.evaluate([root])
     assert abs(root.get()[0] - gold["evdata"]) <= 1e-9 * gold["evdata"]
+
+
+@pytest.mark.parametrize("np_dtype", [np.float64, np.int32], ids=["f64", "i32"])
+def test_random_expressions_keep_their_values_through_the_clean_up(np_dtype):
+    """Seeded expression trees over variables and the constants the conversions
+    look for (0, 1, -1, 2, 3; operands in either order, NEG / ABS / SQUARE
+    stacked on each other, shared subtrees): the cleaned-up graph must compute
+    what the graph computed before -- in double within 1e-12 of the largest
+    entry (a conversion such as x * (1 / y) -> x / y rounds differently), in
+    int32 bit for bit (no conversion rounds there; DIV and POW stay out, they
+    have no exact integer counterpart for these patterns)."""
+    from tenncor_amd import graph
+    integer = np_dtype == np.int32
+    converted = 0
+    for seed in range(24):
+        rng = np.random.default_rng(5000 + seed)
+        g = graph.Graph()
+        try:
+            api = graph.Api(g)
+            shape = [4, 3]
+            if integer:
+                leaves = [g.variable(rng.integers(1, 6, 12).astype(np.int32), shape, "v%d" % k) for k in range(3)]
+            else:
+                leaves = [g.variable(rng.uniform(1, 2, 12), shape, "v%d" % k) for k in range(3)]
+            constants = [g.scalar(np_dtype(c), np_dtype, shape) for c in (0, 1, -1, 2, 3)]
+            pool = list(leaves)
+
+            def pick(allow_constant=True):
+                if allow_constant and rng.uniform() < 0.35:
+                    return constants[int(rng.integers(0, len(constants)))]
+                return pool[int(rng.integers(0, len(pool)))]
+
+            for step in range(int(rng.integers(6, 14))):
+                kind = int(rng.integers(0, 8))
+                if kind == 0:
+                    node = api.unary(str(rng.choice(["NEG", "ABS", "SQUARE"])), pick(False))
+                elif kind == 1:
+                    node = api.unary("NEG", api.unary(str(rng.choice(["NEG", "ABS"])), pick(False)))
+                elif kind == 2 and not integer:
+                    node = g.functor("POW", [pick(False), constants[int(rng.integers(0, 5))]])
+                elif kind == 3 and not integer:
+                    # denominators stay away from zero: variables only
+                    node = g.functor("DIV", [pick(), pool[int(rng.integers(0, 3))]])
+                elif kind == 4 and not integer:
+                    one_over = g.functor("DIV", [constants[1], pool[int(rng.integers(0, 3))]])
+                    node = g.functor("MUL", [pick(False), one_over])
+                else:
+                    op = str(rng.choice(["ADD", "SUB", "MUL"]))
+                    a, b = pick(), pick()
+                    if rng.uniform() < 0.3:
+                        b = api.unary("NEG", pick(False))
+                    node = g.functor(op, [a, b])
+                if not integer:
+                    node = api.unary("TANH", node) if rng.uniform() < 0.3 else node
+                pool.append(node)
+            root = pool[-1]
+            for extra in pool[-4:-1]:
+                root = g.functor("ADD", [root, extra])
+            g.evaluate([root])
+            before = root.get().copy()
+            (out,), stats = g.optimize([root])
+            converted += stats["converted"]
+            g.evaluate([out])
+            after = out.get()
+            assert np.isfinite(before).all(), seed
+            if integer:
+                np.testing.assert_array_equal(after, before, err_msg="seed %d" % seed)
+            else:
+                assert np.abs(after - before).max() <= 1e-12 * max(1.0, np.abs(before).max()), seed
+        finally:
+            g.close()
+    assert converted >= 24    # the generator does reach the conversions
