@@ -229,3 +229,62 @@ def test_elementwise_at_random_lengths_and_alignments(ctx, oracle, np_dtype):
             np.testing.assert_allclose(res, ref, rtol=2e-6 if np_dtype == np.float32 else 1e-14, atol=1e-30)
         for buf in (da, db, out):
             buf.release()
+
+
+@pytest.mark.parametrize("np_dtype", DTYPES, ids=lambda t: np.dtype(t).name)
+def test_medium_sizes_reach_the_tiled_kernels(ctx, oracle, np_dtype):
+    """The same sweeps at a few hundred thousand to a few million elements, where
+    transposes go through LDS tiles, reductions split a dim over workgroups and
+    products run on the matrix cores with edge tiles, K ranges or waves that
+    share K: extents that are multiples of the tile sizes, one off either way,
+    and odd."""
+    from tenncor_amd import ops
+    rng = np.random.default_rng(seed_of("medium", np.dtype(np_dtype).name))
+    edge = [31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 250, 256, 257, 500, 512, 513]
+    # PERMUTE: two or three significant dims, every order
+    for case in range(18):
+        rank = int(rng.choice([2, 3]))
+        shape = [int(rng.choice(edge)) for _ in range(rank)]
+        if rank == 3:
+            shape[int(rng.integers(0, 3))] = int(rng.choice([2, 3, 5, 8]))
+        order = [int(v) for v in rng.permutation(rank)]
+        x = draw(rng, int(np.prod(shape)), np_dtype)
+        t = ops.from_host(ctx, x, shape)
+        np.testing.assert_array_equal(ops.permute(t, order).get(), oracle.permute(x, shape, order)[0],
+                                      err_msg="permute %s %s" % (shape, order))
+        t.release()
+    # reductions of each dim and of pairs of dims
+    for case in range(18):
+        shape = [int(rng.choice(edge)), int(rng.choice(edge)), int(rng.choice([1, 2, 3, 7]))]
+        ranks = [[0], [1], [2], [0, 1], [1, 2], [0, 2], [0, 1, 2]][case % 7]
+        op = str(rng.choice(["REDUCE_SUM", "REDUCE_MAX", "REDUCE_MIN"]))
+        x = draw(rng, int(np.prod(shape)), np_dtype)
+        t = ops.from_host(ctx, x, shape)
+        got = ops.reduce(op, t, ranks).get()
+        ref, _ = oracle.reduce(op, x, shape, ranks, wide_acc=np_dtype == np.float32)
+        close(got, ref, np_dtype, exact=op != "REDUCE_SUM")
+        t.release()
+    # products: [k, m] x [n, k], sometimes batched; long K over few results among them
+    for case in range(18):
+        m, n = int(rng.choice(edge)), int(rng.choice(edge))
+        k = int(rng.choice([16, 64, 100, 256, 1000, 2048, 4100])) if case % 3 else int(rng.choice(edge))
+        if m * n * k > 60_000_000:
+            k = max(16, 60_000_000 // (m * n))
+        batch = [int(rng.choice([2, 3]))] if case % 5 == 0 else []
+        ashape, bshape = [k, m] + batch, [n, k] + batch
+        a, b = draw(rng, int(np.prod(ashape)), np_dtype, -2, 2), draw(rng, int(np.prod(bshape)), np_dtype, -2, 2)
+        ta, tb = ops.from_host(ctx, a, ashape), ops.from_host(ctx, b, bshape)
+        got = ops.matmul(ta, tb).get()
+        ref, _ = oracle.matmul(a, ashape, b, bshape, wide_acc=np_dtype == np.float32)
+        close(got, ref, np_dtype)
+        # the four operand layouts of a contraction over one pair
+        if case % 2 == 0 and not batch:
+            for pairs, sa, sb in ((((0, 0),), [k, m], [k, n]), (((1, 0),), [m, k], [k, n]), (((1, 1),), [m, k], [n, k])):
+                ta2, tb2 = ops.from_host(ctx, a, sa), ops.from_host(ctx, b, sb)
+                got = ops.contract(ta2, tb2, pairs).get()
+                ref, _ = oracle.contract(a, sa, b, sb, pairs, wide_acc=np_dtype == np.float32)
+                close(got, ref, np_dtype)
+                ta2.release()
+                tb2.release()
+        ta.release()
+        tb.release()

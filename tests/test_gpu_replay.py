@@ -662,7 +662,7 @@ def random_elementwise_graph(g, api, seed, x0, shape, np_dtype, with_updates):
     binary = ["ADD", "SUB", "MUL", "MIN", "MAX"]
     updates = []
     for step in range(int(rng.integers(8, 16))):
-        kind = int(rng.integers(0, 9))
+        kind = int(rng.integers(0, 11))
         p = pool[int(rng.integers(0, len(pool)))]
         q = pool[int(rng.integers(0, len(pool)))]
         if kind == 0:
@@ -685,8 +685,16 @@ def random_elementwise_graph(g, api, seed, x0, shape, np_dtype, with_updates):
             node = api.concat([api.slice(p, half, a - half, 0), api.slice(q, 0, half, 0)], 0)
         elif kind == 7:
             node = api.if_then_else(api.binary("LT", p, q), api.identity(p), api.neg(q))
-        else:
+        elif kind == 8:
             node = api.binary("MAX", api.reverse(p, [0]), q)
+        elif kind == 9:
+            # a product of two nodes, its rows summed and spread back over the shape
+            prod = api.matmul(p, api.permute(q, [1, 0]))                       # [b, b]
+            if not integer:
+                prod = api.tanh(prod)
+            node = api.binary("ADD", p, api.extend(api.reduce_sum(prod, 0, 1), 0, [a]))
+        else:
+            node = api.binary("SUB", q, api.extend(api.reduce("REDUCE_MAX", api.contract(p, q, ((1, 1),)), 1, 1), 1, [b]))
         if not integer:
             node = api.tanh(node)    # keeps every value in (-1, 1)
         pool.append(node)
