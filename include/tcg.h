@@ -434,6 +434,20 @@ int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	const void* const* A, const uint64_t* lda, int trans_a,
 	const void* const* B, const uint64_t* ldb, int trans_b,
 	void* C, uint64_t ldc);
+/* Sums of products whose operands are concatenations along the dims that
+ * survive (the weight gradient of the recurrent cell above: [x_t, h] against
+ * the four gate gradients, one term per time step): the result falls into
+ * mparts x nparts blocks, block (i, j) = sum_t A[i * nterms + t] B[j * nterms + t]
+ * with Mp[i] rows and Np[j] columns, at rows sum(Mp[..i]) and columns
+ * sum(Np[..j]) of C.  lda / ldb: one leading dim per part.  Where every part
+ * is a multiple of 128 rows / columns (fp32, 16-byte aligned, at most 4 x 8
+ * parts and 384 operand addresses) the blocks run as ONE matrix-core product
+ * over the whole result, whose tiles look their parts up; otherwise block by
+ * block through tcg_gemm_terms.  Same sums per element either way up to the
+ * order in which K ranges are added. */
+int tcg_gemm_terms_grid (tcg_ctx* ctx, int dtype, int mparts, const uint64_t* Mp, int nparts, const uint64_t* Np,
+	uint64_t K, int nterms, const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b, void* C, uint64_t ldc);
 /* The same sum of products with its summed index cut into `nranges` equal
  * ranges whose results are left side by side: ranges[r][m][n] (row-major
  * M x N each) is the sum over range r.  The reader adds them up in range

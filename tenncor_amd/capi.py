@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -135,6 +135,7 @@ def load():
         "tcg_gemm": [vp, i32, u64, u64, u64, u64, vp, u64, u64, i32, vp, u64, u64, i32, vp, u64, u64],
         "tcg_gemm_terms": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
         "tcg_gemm_terms_ranges": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, i32, vp],
+        "tcg_gemm_terms_grid": [vp, i32, i32, u64p, i32, u64p, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
@@ -460,6 +461,16 @@ class Context:
         la = (ctypes.c_uint64 * n)(*[int(v) for v in lda])
         lb = (ctypes.c_uint64 * n)(*[int(v) for v in ldb])
         self._check(self.lib.tcg_gemm_terms(self.handle, dtype, M, N, K, n, pa, la, int(trans_a), pb, lb, int(trans_b), c, ldc))
+
+    def gemm_terms_grid(self, dtype, Mp, Np, K, a_ptrs, lda, trans_a, b_ptrs, ldb, trans_b, c, ldc):
+        """a_ptrs[i][t], b_ptrs[j][t]: block (i, j) of C = sum_t A[i][t] B[j][t]; lda / ldb per part."""
+        nterms = len(a_ptrs[0])
+        flat_a = [p for row in a_ptrs for p in row]
+        flat_b = [p for row in b_ptrs for p in row]
+        pa = (ctypes.c_void_p * len(flat_a))(*flat_a)
+        pb = (ctypes.c_void_p * len(flat_b))(*flat_b)
+        self._check(self.lib.tcg_gemm_terms_grid(self.handle, dtype, len(Mp), _u64(Mp), len(Np), _u64(Np), K, nterms,
+                                                 pa, _u64(lda), int(trans_a), pb, _u64(ldb), int(trans_b), c, ldc))
 
     def gemm_terms_ranges(self, dtype, M, N, K, a_ptrs, lda, trans_a, b_ptrs, ldb, trans_b, nranges, ranges):
         """The same sum with its summed index cut into nranges ranges left side by side."""

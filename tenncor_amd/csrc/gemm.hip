@@ -6,6 +6,7 @@
 // gemm_mfma_f64.hip; everything else (int32, odd strides, small problems) runs
 // the LDS-tiled kernel below.
 #include <type_traits>
+#include <vector>
 
 #include "tcg_internal.hpp"
 
@@ -497,6 +498,51 @@ int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	if (term) { tcg_free(ctx, term, esz * M * N); }
 	if (rc != TCG_OK) { return rc; }
 	TCG_LAUNCH_CHECK(ctx, "tcg_gemm_terms");
+	return TCG_OK;
+}
+
+int tcg_gemm_terms_grid (tcg_ctx* ctx, int dtype, int mparts, const uint64_t* Mp, int nparts, const uint64_t* Np,
+	uint64_t K, int nterms, const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b, void* C, uint64_t ldc)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, Mp && Np && A && B && lda && ldb && C, "tcg_gemm_terms_grid: NULL pointer");
+	TCG_REQUIRE(ctx, mparts >= 1 && nparts >= 1 && nterms >= 1, "tcg_gemm_terms_grid: %d x %d parts, %d terms", mparts, nparts, nterms);
+	uint64_t N = 0;
+	for (int j = 0; j < nparts; ++j) { N += Np[j]; }
+	TCG_REQUIRE(ctx, ldc >= N, "tcg_gemm_terms_grid: ldc %llu < N %llu", (unsigned long long) ldc, (unsigned long long) N);
+	for (int i = 0; i < mparts * nterms; ++i) { TCG_REQUIRE(ctx, A[i], "tcg_gemm_terms_grid: operand A[%d] is NULL", i); }
+	for (int j = 0; j < nparts * nterms; ++j) { TCG_REQUIRE(ctx, B[j], "tcg_gemm_terms_grid: operand B[%d] is NULL", j); }
+	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a sum of matrix products"); }
+	TCG_REQUIRE(ctx, tcg_type_size(dtype) != 0, "tcg_gemm_terms_grid: unknown dtype %d", dtype);
+	if (dtype == TCG_FLOAT)
+	{
+		bool handled = false;
+		int rc = tcg_gemm_f32_mfma_grid(ctx, (uint32_t) mparts, Mp, (uint32_t) nparts, Np, K, (uint32_t) nterms,
+			(const float* const*) A, lda, trans_a, (const float* const*) B, ldb, trans_b, (float*) C, ldc, &handled);
+		if (rc != TCG_OK || handled) { return rc; }
+	}
+	// block by block
+	const size_t esz = tcg_type_size(dtype);
+	std::vector<uint64_t> la((size_t) nterms), lb((size_t) nterms);
+	uint64_t m0 = 0;
+	for (int i = 0; i < mparts; ++i)
+	{
+		uint64_t n0 = 0;
+		for (int j = 0; j < nparts; ++j)
+		{
+			for (int t = 0; t < nterms; ++t)
+			{
+				la[t] = lda[i];
+				lb[t] = ldb[j];
+			}
+			int rc = tcg_gemm_terms(ctx, dtype, Mp[i], Np[j], K, nterms, A + (size_t) i * nterms, la.data(), trans_a,
+				B + (size_t) j * nterms, lb.data(), trans_b, (char*) C + esz * (m0 * ldc + n0), ldc);
+			if (rc != TCG_OK) { return rc; }
+			n0 += Np[j];
+		}
+		m0 += Mp[i];
+	}
 	return TCG_OK;
 }
 

@@ -61,6 +61,25 @@ struct GemmSegs
 
 struct NoSegs {};
 
+// The same for operands that are concatenations along the dims that survive:
+// the result falls into mparts x nparts blocks, block (i, j) being the sum
+// over the terms of A[i][t] B[j][t].  Every part is a whole number of tiles,
+// so a tile looks its part up once; the operands stay where they are.
+constexpr int MAX_GRID_PTRS = 384;
+constexpr int MAX_GRID_MPARTS = 4, MAX_GRID_NPARTS = 8;
+
+struct GemmGrid
+{
+	uint32_t k = 0;      // columns of A (rows of B) per term
+	uint32_t terms = 0;
+	uint32_t mparts = 0, nparts = 0;
+	uint32_t mstart[MAX_GRID_MPARTS + 1]; // first row of each part of A, then M
+	uint32_t nstart[MAX_GRID_NPARTS + 1]; // first column of each part of B, then N
+	uint32_t lda[MAX_GRID_MPARTS];
+	uint32_t ldb[MAX_GRID_NPARTS];
+	const float* ptr[MAX_GRID_PTRS];      // a[part][term], then b[part][term]
+};
+
 __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_tab& row, const tcg_conv_tab& col)
 {
 	bool inside = true;
@@ -97,7 +116,8 @@ __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_t
 template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL, typename SEGS = NoSegs>
 __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 {
-	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value;
+	constexpr bool GRID = std::is_same<SEGS,GemmGrid>::value;
+	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value && !GRID;
 	constexpr int WGN = 4 / WGM;
 	constexpr int WM = BM / WGM, WN = BN / WGN; // wave tile
 	constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 accumulators per wave
@@ -158,6 +178,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 	f32x4v ra[A_VEC], rb[B_VEC];
 	const f32x4v zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
+	// a grid of blocks: the parts this tile lies in, and what takes a row / column
+	// of the whole result to a row / column of the part
+	uint32_t part_a = 0, part_b = 0;
+	int64_t shift_a = 0, shift_b = 0;
+	if constexpr (GRID)
+	{
+		while (part_a + 1 < segs.mparts && m0 >= segs.mstart[part_a + 1]) { ++part_a; }
+		while (part_b + 1 < segs.nparts && n0 >= segs.nstart[part_b + 1]) { ++part_b; }
+		shift_a = (int64_t) segs.mstart[part_a] * (TA ? 1 : (int64_t) segs.lda[part_a]);
+		shift_b = (int64_t) segs.nstart[part_b] * (TB ? (int64_t) segs.ldb[part_b] : 1);
+	}
+
 	// the table rows a lane gathers from stay the same for every slab
 	constexpr int ROW_ENTS = IMPL == 0 ? 1 : (!TA ? A_VEC : 1);
 	tcg_conv_tab rowent[ROW_ENTS], colent[A_VEC];
@@ -199,6 +231,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 			B = segs.b[term];
 			lda = segs.lda[term];
 			ldb = segs.ldb[term];
+			kfirst = term * segs.k;
+		}
+		if constexpr (GRID)
+		{
+			const uint32_t term = k0 / segs.k;
+			A = segs.ptr[part_a * segs.terms + term] - shift_a;
+			B = segs.ptr[(segs.mparts + part_b) * segs.terms + term] - shift_b;
+			lda = segs.lda[part_a];
+			ldb = segs.ldb[part_b];
 			kfirst = term * segs.k;
 		}
 #pragma unroll
@@ -742,6 +783,33 @@ int launch_kw (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, 
 	return TCG_OK;
 }
 
+// How many ranges of K for `tiles` large tiles: the fewest that put at least
+// two workgroups on every CU and leave the last round of workgroups at least
+// nine tenths full (96 tiles on 256 CUs: 6 ranges make 2.25 rounds, of which
+// the last quarter runs alone; 8 make three full ones), every range keeping
+// 256 summed indices
+uint32_t ranges_for_tiles (uint64_t tiles, uint64_t cus, uint64_t depth)
+{
+	uint64_t most = depth / 256 < 32 ? depth / 256 : 32;
+	if (most < 2 || tiles >= 2 * cus) { return 1; }
+	uint64_t best = 1;
+	double best_fill = 0.0;
+	for (uint64_t r = 2; r <= most; ++r)
+	{
+		uint64_t groups = tiles * r;
+		if (groups < 2 * cus && r < most) { continue; }
+		uint64_t rounds = (groups + cus - 1) / cus;
+		double fill = (double) groups / (double) (rounds * cus);
+		if (fill >= 0.9) { return (uint32_t) r; }
+		if (fill > best_fill)
+		{
+			best_fill = fill;
+			best = r;
+		}
+	}
+	return (uint32_t) best;
+}
+
 // Tile shapes by problem shape
 template <int IMPL>
 int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int trans_b)
@@ -764,6 +832,14 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
 	// small problems: smaller tiles so that the grid still covers the chip
 	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
+	if (big_tiles >= 2 * cus) { return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
+	// fewer large tiles than two per CU under a long K: ranges of K chosen so that the
+	// workgroups come in full rounds (768 x 2048 x 16384: 72 -> 110 TFLOP/s, 1024 x 1024 x 4096:
+	// 63 -> 85, 512 x 512 x 8192: 57 -> 76; with K = 1024 the small tiles below stay ahead)
+	if (big_tiles >= 16 && K >= 1536 && batch < (1ull << 16))
+	{
+		return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b, ranges_for_tiles(big_tiles, cus, K));
+	}
 	if (big_tiles >= cus) { return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
 	// still too few tiles for the chip and a long K: several workgroups share a
 	// tile, each summing a range of K, and a second kernel adds the ranges up
@@ -875,11 +951,64 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 		if (ranges < 2) { ranges = 1; }
 		return launch<64,64,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) ranges, segs);
 	}
-	uint64_t splits = (2 * (uint64_t) ctx->num_cus + tiles - 1) / tiles;
-	if (splits > g.K / 256) { splits = g.K / 256; }
-	if (splits > 32) { splits = 32; }
-	if (splits < 2) { splits = 1; }
-	return launch<128,128,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) splits, segs);
+	return launch<128,128,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, ranges_for_tiles(tiles, cus, g.K), segs);
+}
+
+// C = the mparts x nparts blocks sum_t A[i][t] B[j][t] as one product of
+// (sum of the parts' rows) x (sum of the parts' columns) x (terms * K)
+int tcg_gemm_f32_mfma_grid (tcg_ctx* ctx, uint32_t mparts, const uint64_t* Mp, uint32_t nparts, const uint64_t* Np,
+	uint64_t K, uint32_t terms, const float* const* A, const uint64_t* lda, int trans_a,
+	const float* const* B, const uint64_t* ldb, int trans_b, float* C, uint64_t ldc, bool* handled)
+{
+	*handled = false;
+	bool ok = mparts >= 1 && mparts <= (uint32_t) MAX_GRID_MPARTS && nparts >= 1 && nparts <= (uint32_t) MAX_GRID_NPARTS &&
+		terms >= 1 && (uint64_t) (mparts + nparts) * terms <= (uint64_t) MAX_GRID_PTRS &&
+		K >= BK && K % BK == 0 && K * terms < (1ull << 31) && ldc % 4 == 0 && tcg_aligned16(C);
+	uint64_t M = 0, N = 0;
+	GemmGrid grid;
+	for (uint32_t i = 0; i < mparts && ok; ++i)
+	{
+		ok = Mp[i] >= 128 && Mp[i] % 128 == 0 && lda[i] % 4 == 0 && lda[i] < (1ull << 32);
+		grid.mstart[i] = (uint32_t) M;
+		grid.lda[i] = (uint32_t) lda[i];
+		M += Mp[i];
+		for (uint32_t t = 0; t < terms && ok; ++t)
+		{
+			ok = tcg_aligned16(A[i * terms + t]);
+			grid.ptr[i * terms + t] = A[i * terms + t];
+		}
+	}
+	for (uint32_t j = 0; j < nparts && ok; ++j)
+	{
+		ok = Np[j] >= 128 && Np[j] % 128 == 0 && ldb[j] % 4 == 0 && ldb[j] < (1ull << 32);
+		grid.nstart[j] = (uint32_t) N;
+		grid.ldb[j] = (uint32_t) ldb[j];
+		N += Np[j];
+		for (uint32_t t = 0; t < terms && ok; ++t)
+		{
+			ok = tcg_aligned16(B[j * terms + t]);
+			grid.ptr[(mparts + j) * terms + t] = B[j * terms + t];
+		}
+	}
+	ok = ok && M < (1ull << 31) && N < (1ull << 31) && ldc >= N;
+	if (!ok) { return TCG_OK; }
+	grid.mstart[mparts] = (uint32_t) M;
+	grid.nstart[nparts] = (uint32_t) N;
+	grid.k = (uint32_t) K;
+	grid.terms = terms;
+	grid.mparts = mparts;
+	grid.nparts = nparts;
+	GemmArgs g;
+	g.A = A[0]; g.B = B[0]; g.C = C;
+	g.M = (uint32_t) M; g.N = (uint32_t) N; g.K = (uint32_t) (K * terms);
+	g.lda = (int64_t) lda[0]; g.ldb = (int64_t) ldb[0]; g.ldc = (int64_t) ldc;
+	g.batch_a = g.batch_b = g.batch_c = 0;
+	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
+	g.rows = g.sums = nullptr;
+	g.ncheck = 0;
+	*handled = true;
+	const uint32_t splits = ranges_for_tiles((M / 128) * (N / 128), (uint64_t) ctx->num_cus, g.K);
+	return launch<128,128,2,0,GemmGrid>(ctx, g, 1, trans_a, trans_b, splits, grid);
 }
 
 // The same sum of products with its K ranges left side by side:

@@ -184,6 +184,11 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 	const float* const* A, const uint64_t* lda, int trans_a, const float* const* B, const uint64_t* ldb, int trans_b,
 	float* C, uint64_t ldc, bool* handled);
 
+// blocks of a result whose operands are concatenations along the dims that survive, as one product
+int tcg_gemm_f32_mfma_grid (tcg_ctx* ctx, uint32_t mparts, const uint64_t* Mp, uint32_t nparts, const uint64_t* Np,
+	uint64_t K, uint32_t terms, const float* const* A, const uint64_t* lda, int trans_a,
+	const float* const* B, const uint64_t* ldb, int trans_b, float* C, uint64_t ldc, bool* handled);
+
 // the same with the K ranges left side by side for the reader to add up
 int tcg_gemm_f32_mfma_ranges (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
 	const float* const* A, const uint64_t* lda, int trans_a, const float* const* B, const uint64_t* ldb, int trans_b,

@@ -145,6 +145,11 @@ struct PartProducts final
 	/// its window side by side in temporary memory ([range][M][N]) and the
 	/// elementwise groups that read the node add them up while they load
 	uint32_t ranges = 0;
+	/// > 0: `products` are the grid_m x grid_n blocks (row by row) of one result
+	/// whose operands are concatenated along the dims that survive, every block
+	/// (i, j) with the A operands of row i and the B operands of column j and
+	/// one leading dim per part: launched as one tcg_gemm_terms_grid
+	uint32_t grid_m = 0, grid_n = 0;
 	std::vector<teq::iTensor*> reads;
 	std::string label;
 };

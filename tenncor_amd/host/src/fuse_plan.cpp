@@ -826,6 +826,25 @@ struct Planner final
 		}
 		out.label = "blocks CONTRACT x" + std::to_string(n.args.size()) + " " + std::to_string(blocks.size()) + "x" +
 			std::to_string(blocks[0].size());
+		// one launch for all of them when every part keeps one leading dim over the terms
+		bool uniform = true;
+		for (auto& row : blocks)
+		{
+			for (auto& p : row)
+			{
+				for (const PartProducts::Term& t : p.terms)
+				{
+					uniform = uniform && t.lda == p.terms[0].lda && t.ldb == p.terms[0].ldb;
+				}
+				uniform = uniform && p.trans_a == blocks[0][0].trans_a && p.trans_b == blocks[0][0].trans_b &&
+					p.K == blocks[0][0].K && p.terms.size() == blocks[0][0].terms.size();
+			}
+		}
+		if (uniform)
+		{
+			out.grid_m = (uint32_t) blocks.size();
+			out.grid_n = (uint32_t) blocks[0].size();
+		}
 		return true;
 	}
 
@@ -2142,6 +2161,48 @@ void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMem
 	char* dst = (char*) ref.borrow_output(ttl, memory);
 	if (nullptr == dst) { global::fatalf("%s cannot take products over parts", out->to_string().c_str()); }
 	if (call.partial) { ref.mark_partial(); }
+	if (call.grid_m > 0)
+	{
+		// the blocks of one result: row i brings the A operands, column j the B operands
+		const size_t nterms = call.products.at(0).terms.size();
+		std::vector<uint64_t> mp, np, lda, ldb;
+		std::vector<const void*> a, b;
+		auto address = [&](teq::iTensor* tens, int64_t off)
+		{
+			const char* base = (const char*) eigen_ref(*tens).device_data();
+			if (nullptr == base) { global::fatal("operand of a matrix product has no data"); }
+			return (const void*) (base + esz * off);
+		};
+		for (uint32_t i = 0; i < call.grid_m; ++i)
+		{
+			const PartProducts::Product& p = call.products.at((size_t) i * call.grid_n);
+			mp.push_back(p.M);
+			lda.push_back(p.terms[0].lda);
+			for (const PartProducts::Term& term : p.terms) { a.push_back(address(term.a, term.a_off)); }
+		}
+		for (uint32_t j = 0; j < call.grid_n; ++j)
+		{
+			const PartProducts::Product& p = call.products.at(j);
+			np.push_back(p.N);
+			ldb.push_back(p.terms[0].ldb);
+			for (const PartProducts::Term& term : p.terms) { b.push_back(address(term.b, term.b_off)); }
+		}
+		const PartProducts::Product& first = call.products[0];
+		try
+		{
+			hip_check(tcg_gemm_terms_grid(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype),
+				(int) call.grid_m, mp.data(), (int) call.grid_n, np.data(), first.K, (int) nterms,
+				a.data(), lda.data(), first.trans_a, b.data(), ldb.data(), first.trans_b,
+				dst + esz * first.c_off, first.ldc));
+		}
+		catch (...)
+		{
+			ref.drop();
+			throw;
+		}
+		for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
+		return;
+	}
 	try
 	{
 		for (const PartProducts::Product& p : call.products)

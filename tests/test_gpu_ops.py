@@ -1467,3 +1467,59 @@ def test_product_ranges_are_added_by_the_launch_that_reads_them(ctx, jit):
         ctx.gemm_terms_ranges(capi.FLOAT, M, N, K, a, lda, 0, b, ldb, 1, 3, parts.ptr + guard * 4)
     with pytest.raises(RuntimeError, match="tcg_gemm_terms_ranges"):
         ctx.gemm_terms_ranges(capi.INT32, M, N, K, a, lda, 0, b, ldb, 1, R, parts.ptr + guard * 4)
+
+
+@pytest.mark.parametrize("np_dtype", [np.float32, np.int32])
+@pytest.mark.parametrize("case", ["one_product", "block_by_block"])
+def test_blocks_of_a_sum_of_products_over_concatenated_operands(ctx, oracle, case, np_dtype):
+    """tcg_gemm_terms_grid: dW = sum_t [x_t, h_t]^T [g0_t .. g3_t], the weight
+    gradient of a recurrent cell (tenncor/eteq/backprop.hpp:269-359 over the
+    CONCAT and the ADD of PADs of cfg/tenncor/layer.yml:716-768), from the
+    parts where they lie.  With parts of whole 128-row / column tiles the fp32
+    blocks run as one matrix-core product; other extents and int32 go block by
+    block.  Against the sum of products of the laid-out concatenations (fp32
+    at 1e-4 of a double accumulation, int32 exactly), with a guard band round
+    the result in a wider matrix."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed_of("grid", case, str(np_dtype)))
+    esz = 4
+    steps, batch = 5, 64
+    if case == "one_product":
+        Mp, Np = [128, 256], [128, 128, 256]
+    else:
+        Mp, Np = [96, 40], [128, 72]
+
+    def draw(n):
+        if np_dtype == np.int32:
+            return rng.integers(-50, 51, n).astype(np.int32)
+        return (rng.standard_normal(n) / 4).astype(np.float32)
+
+    # x parts live in one [batch][steps][Mp0] tensor (rows steps * Mp0 apart), h parts are tensors of their own
+    x = draw(batch * steps * Mp[0])
+    hs = [draw(batch * Mp[1]) for _ in range(steps)]
+    gs = [[draw(batch * n) for _ in range(steps)] for n in Np]
+    dx, dh = ctx.upload(x), [ctx.upload(h) for h in hs]
+    dg = [[ctx.upload(v) for v in part] for part in gs]
+    a_ptrs = [[dx.ptr + t * Mp[0] * esz for t in range(steps)], [d.ptr for d in dh]]
+    lda = [steps * Mp[0], Mp[1]]
+    b_ptrs = [[d.ptr for d in part] for part in dg]
+    ldb = list(Np)
+    M, N = sum(Mp), sum(Np)
+    ldc, guard = N + 12, 64
+    out = ctx.upload(np.full(guard + M * ldc + guard, 777, np_dtype))
+    ctx.gemm_terms_grid(capi.dtype_code(np_dtype), Mp, Np, batch, a_ptrs, lda, 1, b_ptrs, ldb, 0,
+                        out.ptr + guard * esz, ldc)
+    got = out.get()
+    assert (got[:guard] == 777).all() and (got[-guard:] == 777).all()
+    C = got[guard:-guard].reshape(M, ldc)
+    assert (C[:, N:] == 777).all()
+    want = np.zeros((M, N), np.float64)
+    x3 = x.reshape(batch, steps, Mp[0])
+    for t in range(steps):
+        left = np.concatenate([x3[:, t, :], hs[t].reshape(batch, Mp[1])], axis=1).astype(np.float64)
+        right = np.concatenate([gs[j][t].reshape(batch, Np[j]) for j in range(len(Np))], axis=1).astype(np.float64)
+        want += left.T @ right
+    if np_dtype == np.int32:
+        np.testing.assert_array_equal(C[:, :N], want.astype(np.int64).astype(np.int32))
+    else:
+        assert_acc_close(C[:, :N], want, ACC_RTOL)
