@@ -113,9 +113,13 @@ __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_t
 // together: one table lookup and one 128-bit load per group.  A lane's row
 // entries stay in registers; the entry of the summed index is fetched one slab
 // ahead of the load that needs it.
-template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL, typename SEGS = NoSegs>
+//
+// AHEAD: slabs on their way from memory into registers while one is multiplied.
+template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL, typename SEGS = NoSegs, int AHEAD = 1>
 __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 {
+	static_assert(AHEAD == 1 || AHEAD == 2, "slabs on their way from memory while one is multiplied");
+	static_assert(IMPL == 0 || AHEAD == 2, "a convolution's operand is read two slabs ahead");
 	constexpr bool GRID = std::is_same<SEGS,GemmGrid>::value;
 	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value && !GRID;
 	constexpr int WGN = 4 / WGM;
@@ -175,7 +179,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 		}
 	}
 
-	f32x4v ra[A_VEC], rb[B_VEC];
+	f32x4v ra[AHEAD][A_VEC], rb[AHEAD][B_VEC];
 	const f32x4v zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
 	// a grid of blocks: the parts this tile lies in, and what takes a row / column
@@ -192,7 +196,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 
 	// the table rows a lane gathers from stay the same for every slab
 	constexpr int ROW_ENTS = IMPL == 0 ? 1 : (!TA ? A_VEC : 1);
-	tcg_conv_tab rowent[ROW_ENTS], colent[A_VEC];
+	// ... and with K along memory every chunk of a lane has the same summed indices
+	constexpr int COL_ENTS = !TA ? 1 : A_VEC;
+	tcg_conv_tab rowent[ROW_ENTS], colent[AHEAD][COL_ENTS];
 	// summed index of chunk v in the slab that starts at k0
 	auto chunk_k = [&] (uint32_t k0, int v) -> uint32_t
 	{
@@ -209,15 +215,42 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 			rowent[e] = g.rows[m < g.M ? m : g.M - 1];
 		}
 #pragma unroll
-		for (int v = 0; v < A_VEC; ++v)
+		for (int v = 0; v < COL_ENTS; ++v)
 		{
 			uint32_t k = chunk_k(k_begin, v);
-			colent[v] = g.sums[k < g.K ? k : g.K - 1];
+			colent[0][v] = g.sums[k < g.K ? k : g.K - 1];
 		}
 	}
 
-	auto load_slab = [&] (uint32_t k0)
+	// AHEAD == 2: two slabs are on their way from memory while one is multiplied.
+	// The hardware counts loads that are still out, and they come back in the order
+	// they were issued; "slab s + 1 has arrived" can only be waited for as "at most
+	// the loads of slab s + 2 are out" when that number is known, so no load sits
+	// under a predicate: an element that does not exist is read from the start of
+	// the operand instead and replaced by zero (`okm`) on its way into LDS.
+	constexpr bool EAGER = AHEAD == 2;
+	uint32_t okm[AHEAD];
+	auto fetch = [&] (const float* p, bool ok, const float* safe) -> f32x4v
 	{
+		if constexpr (EAGER) { return *reinterpret_cast<const f32x4v*>(ok ? p : safe); }
+		else { return ok ? *reinterpret_cast<const f32x4v*>(p) : zero4; }
+	};
+
+	// `set`: the registers the slab waits in (slab x in set x % AHEAD)
+	auto load_slab = [&] (uint32_t k0, auto set_c)
+	{
+		constexpr int set = decltype(set_c)::value;
+		if constexpr (IMPL != 0)
+		{
+			// the table entries of the slab after this one go first: waiting for
+			// them later then waits for nothing of this slab
+#pragma unroll
+			for (int v = 0; v < COL_ENTS; ++v)
+			{
+				uint32_t kn = chunk_k(k0, v) + BK;
+				colent[set ^ 1][v] = g.sums[kn < g.K ? kn : g.K - 1];
+			}
+		}
 		// with terms: the operands of the term this slab belongs to, addressed
 		// by the summed index counted from the term's first column
 		const float* __restrict__ A = Abase;
@@ -242,66 +275,77 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 			ldb = segs.ldb[part_b];
 			kfirst = term * segs.k;
 		}
+		uint32_t oks = 0;
 #pragma unroll
 		for (int v = 0; v < A_VEC; ++v)
 		{
 			int idx = tid + v * 256;
-			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			if constexpr (!EAGER)
+			{
+				if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			}
+			bool ok = A_CHUNKS % 256 == 0 || idx < A_CHUNKS;
 			if constexpr (IMPL != 0)
 			{
 				// four consecutive k of one row, or four consecutive rows at one k
 				uint32_t m = !TA ? m0 + idx / (BK / 4) : m0 + (idx % (BM / 4)) * 4;
 				uint32_t k = chunk_k(k0, v);
 				const tcg_conv_tab& row = rowent[!TA ? v : 0];
-				f32x4v val = zero4;
-				if (m < g.M && k < k_end && conv_inside(g, row, colent[v]))
-				{
-					val = *reinterpret_cast<const f32x4v*>(A + row.off + colent[v].off);
-				}
-				ra[v] = val;
-				// the entry the next slab needs is on its way while this one is multiplied
-				uint32_t kn = k + BK;
-				colent[v] = g.sums[kn < g.K ? kn : g.K - 1];
+				const tcg_conv_tab& col = colent[set][!TA ? 0 : v];
+				ok = ok && m < g.M && k < k_end && conv_inside(g, row, col);
+				ra[set][v] = fetch(A + row.off + col.off, ok, g.A);
 			}
 			else if constexpr (!TA)
 			{
 				// K contiguous: BK/4 lanes per row
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t m = m0 + mm, k = k0 + kq * 4;
-				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) m * lda + (k - kfirst)) : zero4;
+				ok = ok && m < g.M && k < k_end;
+				ra[set][v] = fetch(A + (int64_t) m * lda + (k - kfirst), ok, g.A);
 			}
 			else
 			{
 				// M contiguous: BM/4 lanes per k
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
 				uint32_t m = m0 + mq * 4, k = k0 + kk;
-				ra[v] = (m < g.M && k < k_end) ? *reinterpret_cast<const f32x4v*>(A + (int64_t) (k - kfirst) * lda + m) : zero4;
+				ok = ok && m < g.M && k < k_end;
+				ra[set][v] = fetch(A + (int64_t) (k - kfirst) * lda + m, ok, g.A);
 			}
+			oks |= (uint32_t) ok << v;
 		}
 #pragma unroll
 		for (int v = 0; v < B_VEC; ++v)
 		{
 			int idx = tid + v * 256;
-			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			if constexpr (!EAGER)
+			{
+				if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			}
+			bool ok = B_CHUNKS % 256 == 0 || idx < B_CHUNKS;
 			if constexpr (!TB)
 			{
 				// N contiguous: BN/4 lanes per k
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
 				uint32_t n = n0 + nq * 4, k = k0 + kk;
-				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) (k - kfirst) * ldb + n) : zero4;
+				ok = ok && n < g.N && k < k_end;
+				rb[set][v] = fetch(B + (int64_t) (k - kfirst) * ldb + n, ok, g.B);
 			}
 			else
 			{
 				// K contiguous: BK/4 lanes per n
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t n = n0 + nn, k = k0 + kq * 4;
-				rb[v] = (n < g.N && k < k_end) ? *reinterpret_cast<const f32x4v*>(B + (int64_t) n * ldb + (k - kfirst)) : zero4;
+				ok = ok && n < g.N && k < k_end;
+				rb[set][v] = fetch(B + (int64_t) n * ldb + (k - kfirst), ok, g.B);
 			}
+			oks |= (uint32_t) ok << (16 + v);
 		}
+		okm[set] = oks;
 	};
 
-	auto store_slab = [&] (int buf)
+	auto store_slab = [&] (int buf, auto set_c)
 	{
+		constexpr int set = decltype(set_c)::value;
 		float* as = As[buf];
 		float* bs = Bs[buf];
 #pragma unroll
@@ -309,15 +353,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 		{
 			int idx = tid + v * 256;
 			if (A_CHUNKS % 256 != 0 && idx >= A_CHUNKS) { break; }
+			f32x4v val = ra[set][v];
+			if constexpr (EAGER) { val = (okm[set] >> v & 1u) ? val : zero4; }
 			if constexpr (!TA)
 			{
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
-				*reinterpret_cast<f32x4v*>(as + mm * AP + kq * 4) = ra[v];
+				*reinterpret_cast<f32x4v*>(as + mm * AP + kq * 4) = val;
 			}
 			else
 			{
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
-				*reinterpret_cast<f32x4v*>(as + kk * AP + mq * 4) = ra[v];
+				*reinterpret_cast<f32x4v*>(as + kk * AP + mq * 4) = val;
 			}
 		}
 #pragma unroll
@@ -325,27 +371,24 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 		{
 			int idx = tid + v * 256;
 			if (B_CHUNKS % 256 != 0 && idx >= B_CHUNKS) { break; }
+			f32x4v val = rb[set][v];
+			if constexpr (EAGER) { val = (okm[set] >> (16 + v) & 1u) ? val : zero4; }
 			if constexpr (!TB)
 			{
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
-				*reinterpret_cast<f32x4v*>(bs + kk * BP + nq * 4) = rb[v];
+				*reinterpret_cast<f32x4v*>(bs + kk * BP + nq * 4) = val;
 			}
 			else
 			{
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
-				*reinterpret_cast<f32x4v*>(bs + nn * BP + kq * 4) = rb[v];
+				*reinterpret_cast<f32x4v*>(bs + nn * BP + kq * 4) = val;
 			}
 		}
 	};
 
-	const uint32_t nslabs = (k_end - k_begin + BK - 1) / BK;
-	load_slab(k_begin);
-	store_slab(0);
-	__syncthreads();
-	for (uint32_t s = 0; s < nslabs; ++s)
+	// slab `buf` of LDS times itself into the accumulators
+	auto multiply = [&] (int buf)
 	{
-		const int buf = s & 1;
-		if (s + 1 < nslabs) { load_slab(k_begin + (s + 1) * BK); }
 		const float* as = As[buf];
 		const float* bs = Bs[buf];
 #pragma unroll
@@ -389,8 +432,50 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				}
 			}
 		}
-		if (s + 1 < nslabs) { store_slab(buf ^ 1); }
+	};
+
+	const uint32_t nslabs = (k_end - k_begin + BK - 1) / BK;
+	using I0 = std::integral_constant<int,0>;
+	using I1 = std::integral_constant<int,1>;
+	load_slab(k_begin, I0());
+	store_slab(0, I0());
+	if constexpr (AHEAD == 1)
+	{
 		__syncthreads();
+		for (uint32_t s = 0; s < nslabs; ++s)
+		{
+			const int buf = s & 1;
+			if (s + 1 < nslabs) { load_slab(k_begin + (s + 1) * BK, I0()); }
+			multiply(buf);
+			if (s + 1 < nslabs) { store_slab(buf ^ 1, I0()); }
+			__syncthreads();
+		}
+	}
+	else
+	{
+		// slab s (s % 2 == par) is multiplied out of LDS while slab s + 2 sets out for the
+		// registers slab s came through and slab s + 1 is still on its way; slab s + 1
+		// goes into the other half of LDS afterwards.  Past the end the last slab is
+		// fetched again and never used, so that every step issues the same loads.
+		const uint32_t last = k_begin + (nslabs - 1) * BK;
+		auto slab_at = [&] (uint32_t s) -> uint32_t { return s < nslabs ? k_begin + s * BK : last; };
+		load_slab(slab_at(1), I1());
+		__syncthreads();
+		auto step = [&] (uint32_t s, auto par_c)
+		{
+			constexpr int par = decltype(par_c)::value;
+			load_slab(slab_at(s + 2), std::integral_constant<int,par>());
+			multiply(par);
+			if (s + 1 < nslabs) { store_slab(par ^ 1, std::integral_constant<int,par ^ 1>()); }
+			__syncthreads();
+		};
+		uint32_t s = 0;
+		for (; s + 1 < nslabs; s += 2)
+		{
+			step(s, I0());
+			step(s + 1, I1());
+		}
+		if (s < nslabs) { step(s, I0()); }
 	}
 
 	// lane holds column l32; register r is row 8*(r/4) + 4*lh + r%4 of the 32x32 block
@@ -478,7 +563,7 @@ __global__ __launch_bounds__(256) void gemm_split_sum_wave_k (const f32x4v* __re
 }
 
 // `ranges_out`: the K ranges stay side by side there ([range][batch][M][N]) and nothing adds them up
-template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs>
+template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs, int AHEAD = 1>
 int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1,
 	const SEGS& segs = SEGS(), float* ranges_out = nullptr)
 {
@@ -515,8 +600,8 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	}
 	else { splits = 1; }
 	const unsigned grid = g.total_tiles * splits;
-	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	else if constexpr (IMPL == 0)
 	{
 		if (!trans_a) { gemm_mfma_k<BM,BN,WGM,false,true,0,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
@@ -818,29 +903,33 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 	// narrow results (the column count of a convolution lowered to a product is
 	// its channel count): tiles as wide as N, so that no lane multiplies padding
 	const uint64_t cus = (uint64_t) ctx->num_cus;
+	// a convolution's operand read through its tables: two slabs on their way (64-column
+	// products 91 -> 84 us, 32-column 111 -> 106, kernel gradient 96 -> 76); plain operands
+	// gain nothing from it (4096^3, and the products of a recurrent layer's steps)
+	constexpr int AHEAD = IMPL == 1 ? 2 : 1;
 	if (N <= 32 && (M + 127) / 128 * batch >= cus)
 	{
-		if ((M + 255) / 256 * batch >= 2 * cus) { return launch<256,32,4,IMPL>(ctx, g, batch, trans_a, trans_b); }
+		if ((M + 255) / 256 * batch >= 2 * cus) { return launch<256,32,4,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
 		// two workgroups per CU hide little of a slab's load latency behind its eight
 		// matrix instructions per wave: up to four ranges of a long K fill the CUs
 		// (the image gradient of a convolution, 73728 x 32 x 1600: 156 -> 111 + 10 us)
 		uint64_t ranges = (M + 127) / 128 * batch < 4 * cus ? 4 : 1;
 		if (ranges > K / 256) { ranges = K / 256; }
 		if (ranges < 2 || batch != 1) { ranges = 1; }
-		return launch<128,32,4,IMPL>(ctx, g, batch, trans_a, trans_b, (uint32_t) ranges);
+		return launch<128,32,4,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, (uint32_t) ranges);
 	}
-	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
+	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
 	// small problems: smaller tiles so that the grid still covers the chip
 	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
-	if (big_tiles >= 2 * cus) { return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
+	if (big_tiles >= 2 * cus) { return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
 	// fewer large tiles than two per CU under a long K: ranges of K chosen so that the
 	// workgroups come in full rounds (768 x 2048 x 16384: 72 -> 110 TFLOP/s, 1024 x 1024 x 4096:
 	// 63 -> 85, 512 x 512 x 8192: 57 -> 76; with K = 1024 the small tiles below stay ahead)
 	if (big_tiles >= 16 && K >= 1536 && batch < (1ull << 16))
 	{
-		return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b, ranges_for_tiles(big_tiles, cus, K));
+		return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, ranges_for_tiles(big_tiles, cus, K));
 	}
-	if (big_tiles >= cus) { return launch<128,128,2,IMPL>(ctx, g, batch, trans_a, trans_b); }
+	if (big_tiles >= cus) { return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
 	// still too few tiles for the chip and a long K: several workgroups share a
 	// tile, each summing a range of K, and a second kernel adds the ranges up
 	// in a fixed order (so that results do not depend on scheduling)
@@ -865,7 +954,7 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 			return launch_kw<1,1,4,32>(ctx, g, batch, trans_a, trans_b);
 		}
 	}
-	return launch<64,64,2,IMPL>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
+	return launch<64,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
 }
 
 } // namespace
