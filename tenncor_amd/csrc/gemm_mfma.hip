@@ -2,9 +2,12 @@
 //
 // One workgroup of 256 lanes (4 waves, 2x2) owns a BM x BN tile of C; each wave
 // owns a (BM/2) x (BN/2) sub-tile built from 32x32 accumulators fed by
-// v_mfma_f32_32x32x2_f32.  A and B slabs of BK columns go global -> registers
-// -> LDS (double buffered, one barrier per slab) so that the loads of slab i+1
-// fly while slab i is multiplied.  Workgroup ids are remapped so that the
+// v_mfma_f32_32x32x2_f32.  A and B slabs of BK columns go global -> LDS
+// directly where the operands are plain matrices and K is a whole number of
+// slabs (gemm_mfma_direct_k: three slabs in LDS, two on their way), and global
+// -> registers -> LDS (double buffered, one barrier per slab) everywhere else
+// (gemm_mfma_k: sums of products over terms, operands gathered from a
+// convolution's image, ragged K).  Workgroup ids are remapped so that the
 // workgroups resident on one XCD (ids congruent mod 8) cover a compact patch of
 // C and share their A/B panels through that XCD's L2.
 // MFMA-bound: 2*M*N*K flops, operands re-read from L2, each C element written once.
@@ -497,6 +500,212 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 	}
 }
 
+// K a multiple of the slab depth: the slabs go from memory straight into LDS
+// (global_load_lds_dwordx4: lane l of a wave's load leaves its 16 bytes at the
+// wave's LDS base + 16 l), no registers and no LDS stores in between, three
+// slabs in LDS: one being multiplied, two on their way.  A wave's load fills
+// 1 KiB of LDS in lane order, so conflict-free reads come from which chunk a
+// lane fetches, not from padding.  An operand whose K runs along memory is kept
+// [row][16 k], 16 rows x 4 chunks per load, the chunk in slot q of row r being
+// q ^ ((r >> 1) & 3); an operand whose rows run along memory is kept
+// [k][rows], the rows of k-rows 4..7 and 12..15 exchanged in halves of 32 (the
+// two lane halves of a matrix instruction read k and k + 4).  Rows and columns
+// past the edge are fetched from the last ones inside and never stored.
+template <int ROWS, bool KALONG>
+__device__ __forceinline__ void direct_issue (const float* __restrict__ P, int64_t ld, uint32_t first, uint32_t extent,
+	uint32_t k0, float* lds, int wave, int lane)
+{
+	constexpr int LOADS = ROWS / 64; // per wave and slab
+#pragma unroll
+	for (int j = 0; j < LOADS; ++j)
+	{
+		const int load = wave * LOADS + j;
+		const float* src;
+		if constexpr (KALONG)
+		{
+			const int rows = load * 16;
+			const int r = rows + lane / 4, q = lane % 4;
+			const int chunk = q ^ ((r >> 1) & 3);
+			uint32_t row = first + r;
+			row = row < extent ? row : extent - 1;
+			src = P + (int64_t) row * ld + k0 + chunk * 4;
+		}
+		else
+		{
+			// 256 floats of the [k][rows] slab: 256 / ROWS k-rows
+			const int at = load * 256 + lane * 4;
+			const int k = at / ROWS, q = (at % ROWS) / 4;
+			const int chunk = q ^ (8 * ((k >> 2) & 1));
+			uint32_t row = first + chunk * 4;
+			row = row + 4 <= extent ? row : extent - 4;
+			src = P + (int64_t) (k0 + k) * ld + row;
+		}
+		const uint32_t base = __builtin_amdgcn_readfirstlane(
+			(uint32_t) (uintptr_t) (const __attribute__((address_space(3))) float*) (lds + load * 256));
+		// written as the instruction itself: the compiler keeps one score for every
+		// such load it knows of and waits for all of them before any later LDS read,
+		// which would leave nothing on its way while a slab is multiplied
+		asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+	}
+}
+
+template <int BM, int BN, bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g)
+{
+	constexpr int TM = BM / 64, TN = BN / 64; // waves 2 x 2, 32 x 32 accumulators per wave
+	constexpr int A_SIZE = BM * BK, B_SIZE = BN * BK;
+	__shared__ __attribute__((aligned(1024))) float As0[A_SIZE];
+	__shared__ __attribute__((aligned(1024))) float As1[A_SIZE];
+	__shared__ __attribute__((aligned(1024))) float As2[A_SIZE];
+	__shared__ __attribute__((aligned(1024))) float Bs0[B_SIZE];
+	__shared__ __attribute__((aligned(1024))) float Bs1[B_SIZE];
+	__shared__ __attribute__((aligned(1024))) float Bs2[B_SIZE];
+
+	// block id / total_tiles picks a K range (whole slabs), as in gemm_mfma_k
+	const uint32_t split = blockIdx.x / g.total_tiles;
+	uint32_t id = blockIdx.x - split * g.total_tiles;
+	const uint32_t k_begin = split * g.k_per_split;
+	const uint32_t k_end = g.K - k_begin < g.k_per_split ? g.K : k_begin + g.k_per_split;
+	if (g.total_tiles % NXCD == 0) { id = (id % NXCD) * (g.total_tiles / NXCD) + id / NXCD; }
+	const uint32_t bz = id / g.tiles_per_batch;
+	const uint32_t t = id - bz * g.tiles_per_batch;
+	const uint32_t group_size = GROUP_M * g.tiles_n;
+	const uint32_t group = t / group_size;
+	const uint32_t first_m = group * GROUP_M;
+	const uint32_t rows_in_group = g.tiles_m - first_m < (uint32_t) GROUP_M ? g.tiles_m - first_m : GROUP_M;
+	const uint32_t in_group = t - group * group_size;
+	const uint32_t m0 = (first_m + in_group % rows_in_group) * BM, n0 = (in_group / rows_in_group) * BN;
+	const float* __restrict__ A = g.A + (int64_t) bz * g.batch_a;
+	const float* __restrict__ B = g.B + (int64_t) bz * g.batch_b;
+	float* __restrict__ C = g.partial ?
+		g.partial + ((int64_t) split * (g.total_tiles / g.tiles_per_batch) + bz) * ((int64_t) g.M * g.N) :
+		g.C + (int64_t) bz * g.batch_c;
+	const int64_t ldc = g.partial ? (int64_t) g.N : g.ldc;
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63, wave = tid >> 6;
+	const int wm = wave / 2, wn = wave % 2;
+	const int l32 = lane & 31, lh = lane >> 5;
+
+	f32x16 acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+	{
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+		{
+#pragma unroll
+			for (int r = 0; r < 16; ++r) { acc[i][j][r] = 0.0f; }
+		}
+	}
+
+	auto issue = [&] (uint32_t k0, float* as, float* bs)
+	{
+		direct_issue<BM,!TA>(A, g.lda, m0, g.M, k0, as, wave, lane);
+		direct_issue<BN,TB>(B, g.ldb, n0, g.N, k0, bs, wave, lane);
+	};
+	auto multiply = [&] (const float* as, const float* bs)
+	{
+#pragma unroll
+		for (int half = 0; half < BK / 8; ++half)
+		{
+			const int kb = half * 8 + lh * 4; // this lane's four k of the half slab
+			f32x4v a[TM], b[TN];
+#pragma unroll
+			for (int i = 0; i < TM; ++i)
+			{
+				const int row = wm * (BM / 2) + i * 32 + l32;
+				if constexpr (!TA) { a[i] = *reinterpret_cast<const f32x4v*>(as + row * BK + ((half * 2 + lh) ^ ((row >> 1) & 3)) * 4); }
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; ++e) { a[i][e] = as[(kb + e) * BM + (row ^ (32 * lh))]; }
+				}
+			}
+#pragma unroll
+			for (int j = 0; j < TN; ++j)
+			{
+				const int col = wn * (BN / 2) + j * 32 + l32;
+				if constexpr (TB) { b[j] = *reinterpret_cast<const f32x4v*>(bs + col * BK + ((half * 2 + lh) ^ ((col >> 1) & 3)) * 4); }
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; ++e) { b[j][e] = bs[(kb + e) * BN + (col ^ (32 * lh))]; }
+				}
+			}
+#pragma unroll
+			for (int e = 0; e < 4; ++e)
+			{
+#pragma unroll
+				for (int i = 0; i < TM; ++i)
+				{
+#pragma unroll
+					for (int j = 0; j < TN; ++j)
+					{
+						acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
+					}
+				}
+			}
+		}
+	};
+	// Every step issues the loads of one slab, so "at most that many loads out"
+	// means that everything but the newest slab has landed (loads complete in
+	// order); the LDS reads of the step are done as well before the barrier, since
+	// the next step's loads overwrite the slab the step before this one read.
+	auto landed = [&] ()
+	{
+		constexpr int PER_SLAB = (BM + BN) / 64;
+		static_assert(PER_SLAB < 16, "the count is written into four bits");
+		__builtin_amdgcn_s_waitcnt(0x0070 | PER_SLAB); // vmcnt(PER_SLAB) lgkmcnt(0)
+		__syncthreads();
+	};
+	const uint32_t nslabs = (k_end - k_begin) / BK;
+	// past the end the last slab is fetched again and never used
+	auto slab_at = [&] (uint32_t s) -> uint32_t { return k_begin + (s < nslabs ? s : nslabs - 1) * BK; };
+	issue(slab_at(0), As0, Bs0);
+	issue(slab_at(1), As1, Bs1);
+	landed();
+	uint32_t s = 0;
+	for (; s + 3 <= nslabs; s += 3)
+	{
+		issue(slab_at(s + 2), As2, Bs2);
+		multiply(As0, Bs0);
+		landed();
+		issue(slab_at(s + 3), As0, Bs0);
+		multiply(As1, Bs1);
+		landed();
+		issue(slab_at(s + 4), As1, Bs1);
+		multiply(As2, Bs2);
+		landed();
+	}
+	if (s < nslabs)
+	{
+		issue(slab_at(s + 2), As2, Bs2);
+		multiply(As0, Bs0);
+		landed();
+		if (s + 1 < nslabs) { multiply(As1, Bs1); }
+	}
+	// nothing of this workgroup's is on its way into LDS when it ends
+	__builtin_amdgcn_s_waitcnt(0);
+
+#pragma unroll
+	for (int i = 0; i < TM; ++i)
+	{
+#pragma unroll
+		for (int j = 0; j < TN; ++j)
+		{
+			const uint32_t n = n0 + wn * (BN / 2) + j * 32 + l32;
+			if (n >= g.N) { continue; }
+#pragma unroll
+			for (int r = 0; r < 16; ++r)
+			{
+				const uint32_t m = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+				if (m < g.M) { C[(int64_t) m * ldc + n] = acc[i][j][r]; }
+			}
+		}
+	}
+}
+
 // C[b][m][n] = partial[0][b][m][n] + partial[1][b][m][n] + ... in that order
 __global__ __launch_bounds__(256) void gemm_split_sum_k (const float* __restrict__ partial, float* __restrict__ C,
 	uint32_t splits, uint32_t M, uint32_t N, uint32_t batch, int64_t ldc, int64_t batch_c)
@@ -563,7 +772,8 @@ __global__ __launch_bounds__(256) void gemm_split_sum_wave_k (const f32x4v* __re
 }
 
 // `ranges_out`: the K ranges stay side by side there ([range][batch][M][N]) and nothing adds them up
-template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs, int AHEAD = 1>
+// DIRECT: gemm_mfma_direct_k (plain operands, K a whole number of slabs)
+template <int BM, int BN, int WGM, int IMPL, typename SEGS = NoSegs, int AHEAD = 1, bool DIRECT = false>
 int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int trans_b, uint32_t splits = 1,
 	const SEGS& segs = SEGS(), float* ranges_out = nullptr)
 {
@@ -600,7 +810,15 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	}
 	else { splits = 1; }
 	const unsigned grid = g.total_tiles * splits;
-	if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+	if constexpr (DIRECT)
+	{
+		static_assert(IMPL == 0 && std::is_same<SEGS,NoSegs>::value, "plain operands");
+		if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
+		else if (trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
+		else if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
+		else { gemm_mfma_direct_k<BM,BN,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+	}
+	else if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	else if constexpr (IMPL == 0)
 	{
@@ -918,18 +1136,39 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 		if (ranges < 2 || batch != 1) { ranges = 1; }
 		return launch<128,32,4,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, (uint32_t) ranges);
 	}
-	if (N <= 64 && (M + 127) / 128 * batch >= cus) { return launch<128,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
+	// plain operands under a K of whole slabs go from memory straight into LDS (4096^3:
+	// 129 -> 136 TFLOP/s, 51200 x 64 x 800: 72 -> 65 us, 512 x 4096 x 1024: 53 -> 45 us);
+	// rows and columns past the edge are read from the last four inside
+	const bool direct = IMPL == 0 && K % BK == 0 && M >= 4 && N >= 4;
+	if (N <= 64 && (M + 127) / 128 * batch >= cus)
+	{
+		if constexpr (IMPL == 0)
+		{
+			if (direct) { return launch<128,64,2,0,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b); }
+		}
+		return launch<128,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b);
+	}
 	// small problems: smaller tiles so that the grid still covers the chip
 	uint64_t big_tiles = ((M + 127) / 128) * ((N + 127) / 128) * batch;
-	if (big_tiles >= 2 * cus) { return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
+	auto large = [&] (uint32_t ranges)
+	{
+		if constexpr (IMPL == 0)
+		{
+			if (direct) { return launch<128,128,2,0,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b, ranges); }
+		}
+		return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, ranges);
+	};
+	if (big_tiles >= 2 * cus) { return large(1); }
 	// fewer large tiles than two per CU under a long K: ranges of K chosen so that the
 	// workgroups come in full rounds (768 x 2048 x 16384: 72 -> 110 TFLOP/s, 1024 x 1024 x 4096:
 	// 63 -> 85, 512 x 512 x 8192: 57 -> 76; with K = 1024 the small tiles below stay ahead)
 	if (big_tiles >= 16 && K >= 1536 && batch < (1ull << 16))
 	{
-		return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, ranges_for_tiles(big_tiles, cus, K));
+		// (a single full round of tiles that go straight into LDS needs no ranges)
+		if (direct && big_tiles == cus) { return large(1); }
+		return large(ranges_for_tiles(big_tiles, cus, K));
 	}
-	if (big_tiles >= cus) { return launch<128,128,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b); }
+	if (big_tiles >= cus) { return large(1); }
 	// still too few tiles for the chip and a long K: several workgroups share a
 	// tile, each summing a range of K, and a second kernel adds the ranges up
 	// in a fixed order (so that results do not depend on scheduling)
@@ -953,6 +1192,10 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 		{
 			return launch_kw<1,1,4,32>(ctx, g, batch, trans_a, trans_b);
 		}
+	}
+	if constexpr (IMPL == 0)
+	{
+		if (direct) { return launch<64,64,2,0,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits); }
 	}
 	return launch<64,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
 }
