@@ -118,13 +118,11 @@ __device__ __forceinline__ bool conv_inside (const GemmArgs& g, const tcg_conv_t
 // ahead of the load that needs it.
 //
 // AHEAD: slabs on their way from memory into registers while one is multiplied.
-template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL, typename SEGS = NoSegs, int AHEAD = 1>
-__global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
+template <int BM, int BN, int WGM, bool TA, bool TB, int IMPL, int AHEAD = 1>
+__global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 {
 	static_assert(AHEAD == 1 || AHEAD == 2, "slabs on their way from memory while one is multiplied");
 	static_assert(IMPL == 0 || AHEAD == 2, "a convolution's operand is read two slabs ahead");
-	constexpr bool GRID = std::is_same<SEGS,GemmGrid>::value;
-	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value && !GRID;
 	constexpr int WGN = 4 / WGM;
 	constexpr int WM = BM / WGM, WN = BN / WGN; // wave tile
 	constexpr int TM = WM / 32, TN = WN / 32;   // 32x32 accumulators per wave
@@ -185,18 +183,6 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 	f32x4v ra[AHEAD][A_VEC], rb[AHEAD][B_VEC];
 	const f32x4v zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
-	// a grid of blocks: the parts this tile lies in, and what takes a row / column
-	// of the whole result to a row / column of the part
-	uint32_t part_a = 0, part_b = 0;
-	int64_t shift_a = 0, shift_b = 0;
-	if constexpr (GRID)
-	{
-		while (part_a + 1 < segs.mparts && m0 >= segs.mstart[part_a + 1]) { ++part_a; }
-		while (part_b + 1 < segs.nparts && n0 >= segs.nstart[part_b + 1]) { ++part_b; }
-		shift_a = (int64_t) segs.mstart[part_a] * (TA ? 1 : (int64_t) segs.lda[part_a]);
-		shift_b = (int64_t) segs.nstart[part_b] * (TB ? (int64_t) segs.ldb[part_b] : 1);
-	}
-
 	// the table rows a lane gathers from stay the same for every slab
 	constexpr int ROW_ENTS = IMPL == 0 ? 1 : (!TA ? A_VEC : 1);
 	// ... and with K along memory every chunk of a lane has the same summed indices
@@ -254,30 +240,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				colent[set ^ 1][v] = g.sums[kn < g.K ? kn : g.K - 1];
 			}
 		}
-		// with terms: the operands of the term this slab belongs to, addressed
-		// by the summed index counted from the term's first column
 		const float* __restrict__ A = Abase;
 		const float* __restrict__ B = Bbase;
-		uint32_t kfirst = 0;
-		int64_t lda = g.lda, ldb = g.ldb;
-		if constexpr (SEG)
-		{
-			const uint32_t term = k0 / segs.k;
-			A = segs.a[term];
-			B = segs.b[term];
-			lda = segs.lda[term];
-			ldb = segs.ldb[term];
-			kfirst = term * segs.k;
-		}
-		if constexpr (GRID)
-		{
-			const uint32_t term = k0 / segs.k;
-			A = segs.ptr[part_a * segs.terms + term] - shift_a;
-			B = segs.ptr[(segs.mparts + part_b) * segs.terms + term] - shift_b;
-			lda = segs.lda[part_a];
-			ldb = segs.ldb[part_b];
-			kfirst = term * segs.k;
-		}
+		const int64_t lda = g.lda, ldb = g.ldb;
 		uint32_t oks = 0;
 #pragma unroll
 		for (int v = 0; v < A_VEC; ++v)
@@ -304,7 +269,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				int mm = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t m = m0 + mm, k = k0 + kq * 4;
 				ok = ok && m < g.M && k < k_end;
-				ra[set][v] = fetch(A + (int64_t) m * lda + (k - kfirst), ok, g.A);
+				ra[set][v] = fetch(A + (int64_t) m * lda + k, ok, g.A);
 			}
 			else
 			{
@@ -312,7 +277,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				int kk = idx / (BM / 4), mq = idx % (BM / 4);
 				uint32_t m = m0 + mq * 4, k = k0 + kk;
 				ok = ok && m < g.M && k < k_end;
-				ra[set][v] = fetch(A + (int64_t) (k - kfirst) * lda + m, ok, g.A);
+				ra[set][v] = fetch(A + (int64_t) k * lda + m, ok, g.A);
 			}
 			oks |= (uint32_t) ok << v;
 		}
@@ -331,7 +296,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				int kk = idx / (BN / 4), nq = idx % (BN / 4);
 				uint32_t n = n0 + nq * 4, k = k0 + kk;
 				ok = ok && n < g.N && k < k_end;
-				rb[set][v] = fetch(B + (int64_t) (k - kfirst) * ldb + n, ok, g.B);
+				rb[set][v] = fetch(B + (int64_t) k * ldb + n, ok, g.B);
 			}
 			else
 			{
@@ -339,7 +304,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g, SEGS segs)
 				int nn = idx / (BK / 4), kq = idx % (BK / 4);
 				uint32_t n = n0 + nn, k = k0 + kq * 4;
 				ok = ok && n < g.N && k < k_end;
-				rb[set][v] = fetch(B + (int64_t) n * ldb + (k - kfirst), ok, g.B);
+				rb[set][v] = fetch(B + (int64_t) n * ldb + k, ok, g.B);
 			}
 			oks |= (uint32_t) ok << (16 + v);
 		}
@@ -549,9 +514,11 @@ __device__ __forceinline__ void direct_issue (const float* __restrict__ P, int64
 	}
 }
 
-template <int BM, int BN, bool TA, bool TB>
-__global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g)
+template <int BM, int BN, bool TA, bool TB, typename SEGS = NoSegs>
+__global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs)
 {
+	constexpr bool GRID = std::is_same<SEGS,GemmGrid>::value;
+	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value && !GRID;
 	constexpr int TM = BM / 64, TN = BN / 64; // waves 2 x 2, 32 x 32 accumulators per wave
 	constexpr int A_SIZE = BM * BK, B_SIZE = BN * BK;
 	__shared__ __attribute__((aligned(1024))) float As0[A_SIZE];
@@ -599,10 +566,44 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g)
 		}
 	}
 
+	// a grid of blocks: the parts this tile lies in, and what takes a row / column
+	// of the whole result to a row / column of the part (see gemm_mfma_k)
+	uint32_t part_a = 0, part_b = 0;
+	int64_t shift_a = 0, shift_b = 0;
+	if constexpr (GRID)
+	{
+		while (part_a + 1 < segs.mparts && m0 >= segs.mstart[part_a + 1]) { ++part_a; }
+		while (part_b + 1 < segs.nparts && n0 >= segs.nstart[part_b + 1]) { ++part_b; }
+		shift_a = (int64_t) segs.mstart[part_a] * (TA ? 1 : (int64_t) segs.lda[part_a]);
+		shift_b = (int64_t) segs.nstart[part_b] * (TB ? (int64_t) segs.ldb[part_b] : 1);
+	}
 	auto issue = [&] (uint32_t k0, float* as, float* bs)
 	{
-		direct_issue<BM,!TA>(A, g.lda, m0, g.M, k0, as, wave, lane);
-		direct_issue<BN,TB>(B, g.ldb, n0, g.N, k0, bs, wave, lane);
+		// with terms: the operands of the term this slab belongs to, addressed by
+		// the summed index counted from the term's first column
+		const float* __restrict__ At = A;
+		const float* __restrict__ Bt = B;
+		int64_t lda = g.lda, ldb = g.ldb;
+		if constexpr (SEG)
+		{
+			const uint32_t term = k0 / segs.k;
+			At = segs.a[term];
+			Bt = segs.b[term];
+			lda = segs.lda[term];
+			ldb = segs.ldb[term];
+			k0 -= term * segs.k;
+		}
+		if constexpr (GRID)
+		{
+			const uint32_t term = k0 / segs.k;
+			At = segs.ptr[part_a * segs.terms + term] - shift_a;
+			Bt = segs.ptr[(segs.mparts + part_b) * segs.terms + term] - shift_b;
+			lda = segs.lda[part_a];
+			ldb = segs.ldb[part_b];
+			k0 -= term * segs.k;
+		}
+		direct_issue<BM,!TA>(At, lda, m0, g.M, k0, as, wave, lane);
+		direct_issue<BN,TB>(Bt, ldb, n0, g.N, k0, bs, wave, lane);
 	};
 	auto multiply = [&] (const float* as, const float* bs)
 	{
@@ -812,20 +813,24 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	const unsigned grid = g.total_tiles * splits;
 	if constexpr (DIRECT)
 	{
-		static_assert(IMPL == 0 && std::is_same<SEGS,NoSegs>::value, "plain operands");
-		if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false><<<grid, 256, 0, ctx->stream>>>(g); }
-		else if (trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,true,false><<<grid, 256, 0, ctx->stream>>>(g); }
-		else if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,true><<<grid, 256, 0, ctx->stream>>>(g); }
-		else { gemm_mfma_direct_k<BM,BN,true,true><<<grid, 256, 0, ctx->stream>>>(g); }
+		static_assert(IMPL == 0, "operands that are matrices in memory");
+		if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else if (trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,true,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else { gemm_mfma_direct_k<BM,BN,true,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	}
-	else if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-	else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL,SEGS,AHEAD><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-	else if constexpr (IMPL == 0)
+	else
 	{
-		if (!trans_a) { gemm_mfma_k<BM,BN,WGM,false,true,0,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-		else { gemm_mfma_k<BM,BN,WGM,true,true,0,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		static_assert(DIRECT || std::is_same<SEGS,NoSegs>::value, "sums over terms take the direct kernel");
+		if (!trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,false,false,IMPL,AHEAD><<<grid, 256, 0, ctx->stream>>>(g); }
+		else if (trans_a && !trans_b) { gemm_mfma_k<BM,BN,WGM,true,false,IMPL,AHEAD><<<grid, 256, 0, ctx->stream>>>(g); }
+		else if constexpr (IMPL == 0)
+		{
+			if (!trans_a) { gemm_mfma_k<BM,BN,WGM,false,true,0><<<grid, 256, 0, ctx->stream>>>(g); }
+			else { gemm_mfma_k<BM,BN,WGM,true,true,0><<<grid, 256, 0, ctx->stream>>>(g); }
+		}
+		else { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
 	}
-	else { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
 	if (g.partial && !ranges_out)
 	{
 		uint64_t n = batch * g.M * g.N;
@@ -1281,9 +1286,9 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 		if (ranges > g.K / 64) { ranges = g.K / 64; }
 		if (ranges > 32) { ranges = 32; }
 		if (ranges < 2) { ranges = 1; }
-		return launch<64,64,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, (uint32_t) ranges, segs);
+		return launch<64,64,2,0,GemmSegs,1,true>(ctx, g, 1, trans_a, trans_b, (uint32_t) ranges, segs);
 	}
-	return launch<128,128,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, ranges_for_tiles(tiles, cus, g.K), segs);
+	return launch<128,128,2,0,GemmSegs,1,true>(ctx, g, 1, trans_a, trans_b, ranges_for_tiles(tiles, cus, g.K), segs);
 }
 
 // C = the mparts x nparts blocks sum_t A[i][t] B[j][t] as one product of
@@ -1340,7 +1345,7 @@ int tcg_gemm_f32_mfma_grid (tcg_ctx* ctx, uint32_t mparts, const uint64_t* Mp, u
 	g.ncheck = 0;
 	*handled = true;
 	const uint32_t splits = ranges_for_tiles((M / 128) * (N / 128), (uint64_t) ctx->num_cus, g.K);
-	return launch<128,128,2,0,GemmGrid>(ctx, g, 1, trans_a, trans_b, splits, grid);
+	return launch<128,128,2,0,GemmGrid,1,true>(ctx, g, 1, trans_a, trans_b, splits, grid);
 }
 
 // The same sum of products with its K ranges left side by side:
@@ -1379,7 +1384,7 @@ int tcg_gemm_f32_mfma_ranges (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, 
 		segs.ldb[t] = (uint32_t) ldb[t];
 	}
 	*handled = true;
-	return launch<64,64,2,0,GemmSegs>(ctx, g, 1, trans_a, trans_b, nranges, segs, ranges);
+	return launch<64,64,2,0,GemmSegs,1,true>(ctx, g, 1, trans_a, trans_b, nranges, segs, ranges);
 }
 
 int tcg_gemm_f32_mfma_sum (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint32_t terms,
