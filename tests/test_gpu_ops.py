@@ -561,6 +561,12 @@ GEMM_CASES = [
     # tall with few columns (a convolution lowered to a product): tiles 32 or 64 columns wide
     (33000, 32, 40, 1, 0, 0), (33000, 24, 40, 1, 1, 0), (131300, 32, 24, 1, 0, 1), (2100, 28, 52, 16, 1, 1),
     (33000, 64, 40, 1, 0, 0), (33000, 40, 36, 1, 1, 1), (4200, 64, 72, 8, 0, 1),
+    # K a whole number of 16-slabs: operands go from memory straight into LDS; ragged M and N in every
+    # layout, for the 128 x 128 tiles (one round, and K ranges), the 128 x 64 ones and the 64 x 64 ones
+    (2052, 2052, 32, 1, 0, 0), (2052, 2052, 32, 1, 1, 0), (2052, 2052, 32, 1, 0, 1), (2052, 2052, 32, 1, 1, 1),
+    (516, 644, 1600, 1, 0, 0), (516, 644, 1600, 1, 1, 1), (644, 516, 1616, 1, 1, 0), (644, 516, 1616, 1, 0, 1),
+    (33000, 60, 48, 1, 0, 0), (33000, 60, 48, 1, 1, 0), (4200, 64, 80, 8, 0, 1), (4200, 44, 80, 8, 1, 1),
+    (100, 36, 48, 3, 1, 1), (260, 132, 80, 2, 0, 1), (260, 132, 80, 2, 1, 0), (68, 68, 16, 5, 0, 0),
     # off the matrix-core path: odd extents
     (33, 35, 17, 2, 0, 0), (33, 35, 17, 2, 1, 1),
 ]
