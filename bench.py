@@ -287,14 +287,31 @@ def time_matmul_4096(ctx, capi, a, b, c, settle, reps):
     }
 
 
-def run_matmul_only(settle=100, reps=100):
+def run_matmul_only(settle=100, reps=100, f64=False):
     """The product third of the metric alone: nothing but 4096^3 fp32 launches in
     the process, so that a kernel trace or a counter run of this command holds
-    one kernel at one shape."""
+    one kernel at one shape.  f64: the same product in double (not part of the
+    metric; its line has no roofline_matmul object)."""
     from tenncor_amd import capi
     ctx = capi.Context(0)
     M = 4096
     rng = np.random.default_rng(3)
+    if f64:
+        a = ctx.upload(rng.standard_normal(M * M) / 64)
+        b = ctx.upload(rng.standard_normal(M * M) / 64)
+        c = ctx.empty(M * M, np.float64)
+        for _ in range(settle):
+            ctx.matmul(capi.DOUBLE, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
+        ctx.timer_begin()
+        for _ in range(reps):
+            ctx.matmul(capi.DOUBLE, [M, M], [M, M], a.ptr, b.ptr, c.ptr)
+        ms = ctx.timer_end() / reps
+        tf = 2 * M ** 3 / (ms * 1e-3) / 1e12
+        out = {"matmul_4096_fp64_TFLOPs": round(tf, 2), "matmul_4096_fp64_ms": round(ms, 4),
+               "matmul_4096_frac_of_fp64_mfma_peak": round(tf / MFMA_F64_PEAK_TFLOPS, 4),
+               "launches": reps, "untimed_launches_before": settle, "device": ctx.arch}
+        ctx.close()
+        return out
     a = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
     b = ctx.upload((rng.standard_normal(M * M) / 64).astype(np.float32))
     c = ctx.empty(M * M, np.float32)
@@ -512,6 +529,7 @@ def main():
     ap.add_argument("--graph-config", type=int, choices=[1, 4, 5], default=None,
                     help="time only this whole-graph configuration and print its line (for profiling)")
     ap.add_argument("--evaluator", choices=["plain", "replay", "replay_launches", "replay_unfused"], default="replay")
+    ap.add_argument("--f64", action="store_true", help="with --matmul-only: the 4096^3 product in double")
     ap.add_argument("--reps", type=int, default=None,
                     help="timed evaluations with --graph-config 4 or 5 (default 20), timed launches with --matmul-only (100)")
     ap.add_argument("--optimize", action="store_true",
@@ -530,7 +548,7 @@ def main():
         print(json.dumps(run_matmul_ramp()))
         return
     if args.matmul_only:
-        print(json.dumps(run_matmul_only(settle=args.settle, reps=args.reps or 100)))
+        print(json.dumps(run_matmul_only(settle=args.settle, reps=args.reps or 100, f64=args.f64)))
         return
     if args.graph_config is not None:
         print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps or 20, optimize=args.optimize)))
