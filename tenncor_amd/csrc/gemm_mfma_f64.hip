@@ -338,7 +338,7 @@ __global__ __launch_bounds__(256) void dgemm_mfma_direct_k (DGemmArgs g)
 		for (int j = 0; j < TN; ++j) { boff[j][ks] = at(TB, BN, wn * WN + j * 16 + l16, ks * 4 + lk); }
 	}
 	// live: false for the steps past the last slab (the loop runs in threes), whose
-	// operands count as zero
+	// operands count as zero on both sides (what is in LDS then may hold infinities)
 	auto multiply = [&] (auto buf_c, bool live)
 	{
 		constexpr int buf = decltype(buf_c)::value;
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256) void dgemm_mfma_direct_k (DGemmArgs g)
 #pragma unroll
 			for (int i = 0; i < TM; ++i) { a[i] = live ? As[buf][aoff[i][ks]] : 0.0; }
 #pragma unroll
-			for (int j = 0; j < TN; ++j) { b[j] = Bs[buf][boff[j][ks]]; }
+			for (int j = 0; j < TN; ++j) { b[j] = live ? Bs[buf][boff[j][ks]] : 0.0; }
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 			{

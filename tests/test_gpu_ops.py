@@ -590,6 +590,22 @@ def test_gemm_transposed_operands_vs_oracle(ctx, oracle, M, N, K, batch, ta, tb)
     assert_acc_close(dc.get(), ref)
 
 
+@pytest.mark.parametrize("np_dtype,K", [(np.float64, 32), (np.float64, 8), (np.float32, 64), (np.float32, 16)])
+def test_gemm_infinity_in_the_last_slab_stays_an_infinity(ctx, np_dtype, K):
+    """The matrix-core kernels fetch slabs past the end of K again to keep their
+    loads countable; what those steps multiply must not reach the result (an
+    infinity times a zero would be a NaN)."""
+    from tenncor_amd import capi
+    M = N = 256
+    A, B = np.ones((M, K), np_dtype), np.ones((K, N), np_dtype)
+    B[K - 1, 5] = np.inf
+    a, b, c = ctx.upload(A.ravel()), ctx.upload(B.ravel()), ctx.empty(M * N, np_dtype)
+    ctx.gemm(capi.dtype_code(np_dtype), M, N, K, 1, a.ptr, K, 0, 0, b.ptr, N, 0, 0, c.ptr, N, 0)
+    out = c.get().reshape(M, N)
+    assert np.isposinf(out[:, 5]).all() and not np.isnan(out).any()
+    assert (np.delete(out, 5, axis=1) == K).all()
+
+
 GEMM_F64_CASES = [
     # on the fp64 matrix-core path: even extents, enough tiles to fill the chip
     (1024, 1024, 64, 1, 0, 0), (1024, 1024, 64, 1, 1, 0), (1024, 1024, 64, 1, 0, 1), (1024, 1024, 64, 1, 1, 1),
