@@ -44,6 +44,7 @@ struct GemmArgs
 	const tcg_conv_tab* sums;
 	uint32_t check_ext[4];
 	int ncheck;
+	const float* zeros; // 16 zero bytes and more in device memory
 };
 
 // A sum of products C = sum_t A_t B_t of equal shapes is one product over the
@@ -514,9 +515,23 @@ __device__ __forceinline__ void direct_issue (const float* __restrict__ P, int64
 	}
 }
 
-template <int BM, int BN, bool TA, bool TB, typename SEGS = NoSegs>
+// IMPL 1: A[m][k] = image[rows[m].off + sums[k].off] or zero, as in gemm_mfma_k.
+// The entries of the summed indices of the workgroup's K range wait in LDS
+// (direct_tab() of them at most), so that the loop holds no load but the ones that
+// go into LDS and the kernel's own count of those stays exact; a lane's row
+// entries stay in registers; an element of the zero border is fetched from a
+// buffer of zeros.
+constexpr int direct_tab (int BM, int BN)
+{
+	// what the 64 KiB of a workgroup's static LDS leave beside the three slabs, in whole slabs
+	int room = (65536 - 3 * (BM + BN) * BK * 4) / (int) sizeof(tcg_conv_tab) / BK * BK;
+	return room < 1408 ? room : 1408;
+}
+
+template <int BM, int BN, bool TA, bool TB, typename SEGS = NoSegs, int IMPL = 0>
 __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs)
 {
+	static_assert(IMPL == 0 || (std::is_same<SEGS,NoSegs>::value && !TB), "a convolution's operand against a row-major matrix");
 	constexpr bool GRID = std::is_same<SEGS,GemmGrid>::value;
 	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value && !GRID;
 	constexpr int TM = BM / 64, TN = BN / 64; // waves 2 x 2, 32 x 32 accumulators per wave
@@ -577,6 +592,51 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 		shift_a = (int64_t) segs.mstart[part_a] * (TA ? 1 : (int64_t) segs.lda[part_a]);
 		shift_b = (int64_t) segs.nstart[part_b] * (TB ? (int64_t) segs.ldb[part_b] : 1);
 	}
+	// a convolution's operand: the entries of this workgroup's summed indices, and the
+	// row entries of the chunks this lane fetches (the same for every slab)
+	constexpr int A_LOADS = BM / 64;
+	__shared__ tcg_conv_tab tab[IMPL != 0 ? direct_tab(BM, BN) : 1];
+	tcg_conv_tab rowent[IMPL != 0 ? A_LOADS : 1];
+	if constexpr (IMPL != 0)
+	{
+		for (uint32_t e = tid; e < k_end - k_begin; e += 256) { tab[e] = g.sums[k_begin + e]; }
+#pragma unroll
+		for (int j = 0; j < A_LOADS; ++j)
+		{
+			const int load = wave * A_LOADS + j;
+			uint32_t m;
+			if constexpr (!TA) { m = m0 + load * 16 + lane / 4; }
+			else
+			{
+				const int at = load * 256 + lane * 4;
+				const int k = at / BM, q = (at % BM) / 4;
+				m = m0 + (q ^ (8 * ((k >> 2) & 1))) * 4;
+				m = m + 4 <= g.M ? m : g.M - 4;
+			}
+			rowent[j] = g.rows[m < g.M ? m : g.M - 1];
+		}
+		__syncthreads();
+	}
+	auto issue_gathered = [&] (uint32_t k0, float* as)
+	{
+#pragma unroll
+		for (int j = 0; j < A_LOADS; ++j)
+		{
+			const int load = wave * A_LOADS + j;
+			int k; // the summed index of this lane's chunk, counted from the slab's first
+			if constexpr (!TA)
+			{
+				const int r = load * 16 + lane / 4, q = lane % 4;
+				k = (q ^ ((r >> 1) & 3)) * 4;
+			}
+			else { k = (load * 256 + lane * 4) / BM; }
+			const tcg_conv_tab col = tab[k0 - k_begin + k];
+			const float* src = conv_inside(g, rowent[j], col) ? g.A + rowent[j].off + col.off : g.zeros;
+			const uint32_t base = __builtin_amdgcn_readfirstlane(
+				(uint32_t) (uintptr_t) (const __attribute__((address_space(3))) float*) (as + load * 256));
+			asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+		}
+	};
 	auto issue = [&] (uint32_t k0, float* as, float* bs)
 	{
 		// with terms: the operands of the term this slab belongs to, addressed by
@@ -602,7 +662,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 			ldb = segs.ldb[part_b];
 			k0 -= term * segs.k;
 		}
-		direct_issue<BM,!TA>(At, lda, m0, g.M, k0, as, wave, lane);
+		if constexpr (IMPL != 0) { issue_gathered(k0, as); }
+		else { direct_issue<BM,!TA>(At, lda, m0, g.M, k0, as, wave, lane); }
 		direct_issue<BN,TB>(Bt, ldb, n0, g.N, k0, bs, wave, lane);
 	};
 	auto multiply = [&] (const float* as, const float* bs)
@@ -813,8 +874,14 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 	const unsigned grid = g.total_tiles * splits;
 	if constexpr (DIRECT)
 	{
-		static_assert(IMPL == 0, "operands that are matrices in memory");
-		if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		if constexpr (IMPL != 0)
+		{
+			// (the caller has seen to it that a K range fits the table in LDS)
+			if (trans_b) { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
+			if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,false,SEGS,IMPL><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+			else { gemm_mfma_direct_k<BM,BN,true,false,SEGS,IMPL><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		}
+		else if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 		else if (trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,true,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 		else if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 		else { gemm_mfma_direct_k<BM,BN,true,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
@@ -1151,6 +1218,15 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 		{
 			if (direct) { return launch<128,64,2,0,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b); }
 		}
+		else
+		{
+			// the gathered operand goes straight into LDS as well when the table entries of K
+			// fit beside the slabs (a 5 x 5 x 32 convolution forwards: 84 -> 71 us)
+			if (K % BK == 0 && K <= (uint64_t) direct_tab(128, 64) && M >= 4 && N >= 4 && batch == 1)
+			{
+				return launch<128,64,2,1,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b);
+			}
+		}
 		return launch<128,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b);
 	}
 	// small problems: smaller tiles so that the grid still covers the chip
@@ -1202,6 +1278,16 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 	{
 		if (direct) { return launch<64,64,2,0,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits); }
 	}
+	else
+	{
+		// a K range is K / splits rounded up to whole slabs (the kernel gradient of that
+		// convolution, 800 x 64 x 51200 in 39 ranges: 76 -> 65 us)
+		uint64_t range = ((K + splits - 1) / splits + BK - 1) / BK * BK;
+		if (K % BK == 0 && range <= (uint64_t) direct_tab(64, 64) && M >= 4 && N >= 4 && batch == 1)
+		{
+			return launch<64,64,2,1,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
+		}
+	}
 	return launch<64,64,2,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, (uint32_t) splits);
 }
 
@@ -1229,6 +1315,7 @@ int tcg_gemm_f32_mfma (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, uint64_
 	g.batch_a = (int64_t) stride_a; g.batch_b = (int64_t) stride_b; g.batch_c = (int64_t) stride_c;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	g.rows = g.sums = nullptr;
+	g.zeros = nullptr;
 	g.ncheck = 0;
 	*handled = true;
 	return dispatch<0>(ctx, g, batch, trans_a, trans_b);
@@ -1258,6 +1345,7 @@ int tcg_gemm_f32_mfma_terms (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, u
 	g.batch_a = g.batch_b = g.batch_c = 0;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	g.rows = g.sums = nullptr;
+	g.zeros = nullptr;
 	g.ncheck = 0;
 	GemmSegs segs;
 	segs.k = (uint32_t) K;
@@ -1342,6 +1430,7 @@ int tcg_gemm_f32_mfma_grid (tcg_ctx* ctx, uint32_t mparts, const uint64_t* Mp, u
 	g.batch_a = g.batch_b = g.batch_c = 0;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	g.rows = g.sums = nullptr;
+	g.zeros = nullptr;
 	g.ncheck = 0;
 	*handled = true;
 	const uint32_t splits = ranges_for_tiles((M / 128) * (N / 128), (uint64_t) ctx->num_cus, g.K);
@@ -1373,6 +1462,7 @@ int tcg_gemm_f32_mfma_ranges (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, 
 	g.batch_a = g.batch_b = g.batch_c = 0;
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	g.rows = g.sums = nullptr;
+	g.zeros = nullptr;
 	g.ncheck = 0;
 	GemmSegs segs;
 	segs.k = (uint32_t) K;
@@ -1420,6 +1510,7 @@ int tcg_gemm_f32_mfma_conv (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S,
 	g.tiles_m = g.tiles_n = g.tiles_per_batch = g.total_tiles = 0;
 	g.rows = op.rows;
 	g.sums = op.sums;
+	g.zeros = ctx->zeros;
 	g.ncheck = op.ncheck;
 	for (int j = 0; j < 4; ++j) { g.check_ext[j] = op.check_ext[j]; }
 	*handled = true;

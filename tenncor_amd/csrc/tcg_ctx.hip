@@ -87,9 +87,19 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		delete ctx;
 		return rc;
 	}
+	if ((err = hipMalloc((void**) &ctx->zeros, 256)) != hipSuccess ||
+		(err = hipMemset(ctx->zeros, 0, 256)) != hipSuccess)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: zero buffer: %s", hipGetErrorString(err));
+		(void) hipFree(ctx->rng_state);
+		(void) hipHostFree(ctx->staging);
+		delete ctx;
+		return rc;
+	}
 	if (tcg_reduce_scratch_init(ctx) != TCG_OK)
 	{
 		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: %s", ctx->error.c_str());
+		(void) hipFree(ctx->zeros);
 		(void) hipFree(ctx->rng_state);
 		(void) hipHostFree(ctx->staging);
 		delete ctx;
@@ -107,6 +117,7 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	ctx->pool.release_all();
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
 	if (ctx->rng_state) { (void) hipFree(ctx->rng_state); }
+	if (ctx->zeros) { (void) hipFree(ctx->zeros); }
 	if (ctx->side_stream)
 	{
 		(void) hipStreamSynchronize(ctx->side_stream);

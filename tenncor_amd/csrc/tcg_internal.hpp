@@ -74,6 +74,9 @@ struct tcg_ctx
 	// tables first met while launches are being recorded are filled at once on
 	// this stream, so that the recording does not fill them again at every replay
 	hipStream_t side_stream = nullptr;
+	// 256 bytes of zeros in device memory: what a load that goes from memory straight
+	// into LDS fetches for an element of a convolution's zero border
+	float* zeros = nullptr;
 	static constexpr size_t conv_table_limit = (size_t) 256 << 20;
 
 	// launch capture: the graph being recorded (its arena is pool.recording)
