@@ -477,15 +477,21 @@ __global__ __launch_bounds__(256) void gemm_mfma_k (GemmArgs g)
 // [k][rows], the rows of k-rows 4..7 and 12..15 exchanged in halves of 32 (the
 // two lane halves of a matrix instruction read k and k + 4).  Rows and columns
 // past the edge are fetched from the last ones inside and never stored.
+// rows exchanged in the k-rows the upper lane half reads: halves of 32, of 16 in a slab of 32 rows
+constexpr int direct_swap (int rows) { return rows >= 64 ? 32 : 16; }
+
 template <int ROWS, bool KALONG>
 __device__ __forceinline__ void direct_issue (const float* __restrict__ P, int64_t ld, uint32_t first, uint32_t extent,
 	uint32_t k0, float* lds, int wave, int lane)
 {
-	constexpr int LOADS = ROWS / 64; // per wave and slab
+	// a slab of 32 rows is two loads: the waves of the second pair repeat them, so
+	// that every wave has the same number of loads out
+	constexpr int TOTAL = ROWS * BK / 256;          // loads per slab
+	constexpr int LOADS = TOTAL >= 4 ? TOTAL / 4 : 1; // per wave
 #pragma unroll
 	for (int j = 0; j < LOADS; ++j)
 	{
-		const int load = wave * LOADS + j;
+		const int load = (wave * LOADS + j) % TOTAL;
 		const float* src;
 		if constexpr (KALONG)
 		{
@@ -501,7 +507,7 @@ __device__ __forceinline__ void direct_issue (const float* __restrict__ P, int64
 			// 256 floats of the [k][rows] slab: 256 / ROWS k-rows
 			const int at = load * 256 + lane * 4;
 			const int k = at / ROWS, q = (at % ROWS) / 4;
-			const int chunk = q ^ (8 * ((k >> 2) & 1));
+			const int chunk = q ^ (direct_swap(ROWS) / 4 * ((k >> 2) & 1));
 			uint32_t row = first + chunk * 4;
 			row = row + 4 <= extent ? row : extent - 4;
 			src = P + (int64_t) (k0 + k) * ld + row;
@@ -528,13 +534,16 @@ constexpr int direct_tab (int BM, int BN)
 	return room < 1408 ? room : 1408;
 }
 
-template <int BM, int BN, bool TA, bool TB, typename SEGS = NoSegs, int IMPL = 0>
+template <int BM, int BN, bool TA, bool TB, typename SEGS = NoSegs, int IMPL = 0, int WGM = 2>
 __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs)
 {
+	// WGM: waves along M (2: waves 2 x 2; 4: waves 4 x 1 for a result of 32 columns)
+	constexpr int WGN = 4 / WGM, WM = BM / WGM, WN = BN / WGN;
+	static_assert(WM % 32 == 0 && WN % 32 == 0 && WM >= 32 && WN >= 32, "wave tiles are made of 32 x 32 blocks");
 	static_assert(IMPL == 0 || (std::is_same<SEGS,NoSegs>::value && !TB), "a convolution's operand against a row-major matrix");
 	constexpr bool GRID = std::is_same<SEGS,GemmGrid>::value;
 	constexpr bool SEG = !std::is_same<SEGS,NoSegs>::value && !GRID;
-	constexpr int TM = BM / 64, TN = BN / 64; // waves 2 x 2, 32 x 32 accumulators per wave
+	constexpr int TM = WM / 32, TN = WN / 32; // 32 x 32 accumulators per wave
 	constexpr int A_SIZE = BM * BK, B_SIZE = BN * BK;
 	__shared__ __attribute__((aligned(1024))) float As0[A_SIZE];
 	__shared__ __attribute__((aligned(1024))) float As1[A_SIZE];
@@ -566,7 +575,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63, wave = tid >> 6;
-	const int wm = wave / 2, wn = wave % 2;
+	const int wm = wave / WGN, wn = wave % WGN;
 	const int l32 = lane & 31, lh = lane >> 5;
 
 	f32x16 acc[TM][TN];
@@ -610,7 +619,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 			{
 				const int at = load * 256 + lane * 4;
 				const int k = at / BM, q = (at % BM) / 4;
-				m = m0 + (q ^ (8 * ((k >> 2) & 1))) * 4;
+				m = m0 + (q ^ (direct_swap(BM) / 4 * ((k >> 2) & 1))) * 4;
 				m = m + 4 <= g.M ? m : g.M - 4;
 			}
 			rowent[j] = g.rows[m < g.M ? m : g.M - 1];
@@ -676,23 +685,23 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 #pragma unroll
 			for (int i = 0; i < TM; ++i)
 			{
-				const int row = wm * (BM / 2) + i * 32 + l32;
+				const int row = wm * WM + i * 32 + l32;
 				if constexpr (!TA) { a[i] = *reinterpret_cast<const f32x4v*>(as + row * BK + ((half * 2 + lh) ^ ((row >> 1) & 3)) * 4); }
 				else
 				{
 #pragma unroll
-					for (int e = 0; e < 4; ++e) { a[i][e] = as[(kb + e) * BM + (row ^ (32 * lh))]; }
+					for (int e = 0; e < 4; ++e) { a[i][e] = as[(kb + e) * BM + (row ^ (direct_swap(BM) * lh))]; }
 				}
 			}
 #pragma unroll
 			for (int j = 0; j < TN; ++j)
 			{
-				const int col = wn * (BN / 2) + j * 32 + l32;
+				const int col = wn * WN + j * 32 + l32;
 				if constexpr (TB) { b[j] = *reinterpret_cast<const f32x4v*>(bs + col * BK + ((half * 2 + lh) ^ ((col >> 1) & 3)) * 4); }
 				else
 				{
 #pragma unroll
-					for (int e = 0; e < 4; ++e) { b[j][e] = bs[(kb + e) * BN + (col ^ (32 * lh))]; }
+					for (int e = 0; e < 4; ++e) { b[j][e] = bs[(kb + e) * BN + (col ^ (direct_swap(BN) * lh))]; }
 				}
 			}
 #pragma unroll
@@ -716,7 +725,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 	// the next step's loads overwrite the slab the step before this one read.
 	auto landed = [&] ()
 	{
-		constexpr int PER_SLAB = (BM + BN) / 64;
+		constexpr int PER_SLAB = (BM >= 64 ? BM / 64 : 1) + (BN >= 64 ? BN / 64 : 1);
 		static_assert(PER_SLAB < 16, "the count is written into four bits");
 		__builtin_amdgcn_s_waitcnt(0x0070 | PER_SLAB); // vmcnt(PER_SLAB) lgkmcnt(0)
 		__syncthreads();
@@ -756,12 +765,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 #pragma unroll
 		for (int j = 0; j < TN; ++j)
 		{
-			const uint32_t n = n0 + wn * (BN / 2) + j * 32 + l32;
+			const uint32_t n = n0 + wn * WN + j * 32 + l32;
 			if (n >= g.N) { continue; }
 #pragma unroll
 			for (int r = 0; r < 16; ++r)
 			{
-				const uint32_t m = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+				const uint32_t m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
 				if (m < g.M) { C[(int64_t) m * ldc + n] = acc[i][j][r]; }
 			}
 		}
@@ -878,13 +887,13 @@ int launch (tcg_ctx* ctx, const GemmArgs& base, uint64_t batch, int trans_a, int
 		{
 			// (the caller has seen to it that a K range fits the table in LDS)
 			if (trans_b) { return tcg_fail(ctx, TCG_ERR_ARG, "gemm_mfma: a convolution's B operand is row-major"); }
-			if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,false,SEGS,IMPL><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-			else { gemm_mfma_direct_k<BM,BN,true,false,SEGS,IMPL><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+			if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,false,SEGS,IMPL,WGM><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+			else { gemm_mfma_direct_k<BM,BN,true,false,SEGS,IMPL,WGM><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 		}
-		else if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-		else if (trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,true,false,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-		else if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
-		else { gemm_mfma_direct_k<BM,BN,true,true,SEGS><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else if (!trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,false,false,SEGS,0,WGM><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else if (trans_a && !trans_b) { gemm_mfma_direct_k<BM,BN,true,false,SEGS,0,WGM><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else if (!trans_a) { gemm_mfma_direct_k<BM,BN,false,true,SEGS,0,WGM><<<grid, 256, 0, ctx->stream>>>(g, segs); }
+		else { gemm_mfma_direct_k<BM,BN,true,true,SEGS,0,WGM><<<grid, 256, 0, ctx->stream>>>(g, segs); }
 	}
 	else
 	{
@@ -1206,6 +1215,12 @@ int dispatch (tcg_ctx* ctx, const GemmArgs& g, uint64_t batch, int trans_a, int 
 		uint64_t ranges = (M + 127) / 128 * batch < 4 * cus ? 4 : 1;
 		if (ranges > K / 256) { ranges = K / 256; }
 		if (ranges < 2 || batch != 1) { ranges = 1; }
+		// plain operands under a K of whole slabs go straight into LDS here too (73728 x 32 x 1600:
+		// 147 -> 139 us); the gathering form of this tile gains nothing from it and stays as it is
+		if constexpr (IMPL == 0)
+		{
+			if (K % BK == 0 && M >= 4 && N >= 4) { return launch<128,32,4,0,NoSegs,1,true>(ctx, g, batch, trans_a, trans_b, (uint32_t) ranges); }
+		}
 		return launch<128,32,4,IMPL,NoSegs,AHEAD>(ctx, g, batch, trans_a, trans_b, (uint32_t) ranges);
 	}
 	// plain operands under a K of whole slabs go from memory straight into LDS (4096^3:

@@ -567,6 +567,9 @@ GEMM_CASES = [
     (516, 644, 1600, 1, 0, 0), (516, 644, 1600, 1, 1, 1), (644, 516, 1616, 1, 1, 0), (644, 516, 1616, 1, 0, 1),
     (33000, 60, 48, 1, 0, 0), (33000, 60, 48, 1, 1, 0), (4200, 64, 80, 8, 0, 1), (4200, 44, 80, 8, 1, 1),
     (100, 36, 48, 3, 1, 1), (260, 132, 80, 2, 0, 1), (260, 132, 80, 2, 1, 0), (68, 68, 16, 5, 0, 0),
+    # ... and the 128 x 32 tiles of a tall result with few columns (waves 4 x 1)
+    (33000, 32, 48, 1, 0, 0), (33000, 24, 48, 1, 1, 0), (131300, 32, 32, 1, 0, 1), (2100, 28, 64, 16, 1, 1),
+    (33000, 32, 1024, 1, 0, 0),
     # off the matrix-core path: odd extents
     (33, 35, 17, 2, 0, 0), (33, 35, 17, 2, 1, 1),
 ]
