@@ -516,8 +516,10 @@ __device__ __forceinline__ void direct_issue (const float* __restrict__ P, int64
 			(uint32_t) (uintptr_t) (const __attribute__((address_space(3))) float*) (lds + load * 256));
 		// written as the instruction itself: the compiler keeps one score for every
 		// such load it knows of and waits for all of them before any later LDS read,
-		// which would leave nothing on its way while a slab is multiplied
-		asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+		// which would leave nothing on its way while a slab is multiplied.  The s_nop is
+		// the wait state the hardware wants between a scalar write of M0 and a load into
+		// LDS that reads it (the compiler adds it for its builtin, not inside this text)
+		asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
 	}
 }
 
@@ -643,7 +645,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_direct_k (GemmArgs g, SEGS segs
 			const float* src = conv_inside(g, rowent[j], col) ? g.A + rowent[j].off + col.off : g.zeros;
 			const uint32_t base = __builtin_amdgcn_readfirstlane(
 				(uint32_t) (uintptr_t) (const __attribute__((address_space(3))) float*) (as + load * 256));
-			asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+			asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
 		}
 	};
 	auto issue = [&] (uint32_t k0, float* as, float* bs)

@@ -273,7 +273,7 @@ __device__ __forceinline__ void ddirect_issue (const double* __restrict__ P, int
 			(uint32_t) (uintptr_t) (const __attribute__((address_space(3))) double*) (lds + load * 128));
 		// written as the instruction itself, and counted by the kernel: through the
 		// builtin the compiler waits for every such load before any later LDS read
-		asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
+		asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(base) : "memory", "m0");
 	}
 }
 

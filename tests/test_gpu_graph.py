@@ -22,6 +22,15 @@ with open(os.path.join(GOLDEN, "equation_vectors.json")) as f:
     EQV = json.load(f)
 
 
+@pytest.fixture(autouse=True)
+def plain_evaluator_afterwards():
+    """Set up before the graph of a test, so that it runs after the graph is
+    closed: a test that installs another evaluator leaves the default behind."""
+    yield
+    from tenncor_amd import graph
+    graph.set_evaluator("plain")
+
+
 @pytest.fixture()
 def g():
     from tenncor_amd import graph
@@ -235,16 +244,37 @@ def torch_reference():
     return torch
 
 
+def evaluate_under(g, evaluator, targets, fed, fed_value):
+    """One evaluation under the walk, or three under the replaying evaluator
+    with the input assigned anew before each (walked, recorded, replayed):
+    the values the targets hold afterwards come from the recording."""
+    from tenncor_amd import graph
+    if evaluator == "plain":
+        g.evaluate(targets)
+        return
+    graph.set_evaluator(evaluator)  # until the end of the test (plain_evaluator_afterwards)
+    for _ in range(3):
+        g.assign(fed, fed_value)
+        g.evaluate(targets)
+    stats = graph.evaluator_stats()
+    assert stats["recorded"] == 1 and stats["replayed"] >= 1, stats
+
+
+@pytest.mark.parametrize("evaluator", ["plain", "replay"])
 @pytest.mark.parametrize("seq,batch,nin,hid,np_dtype,rtol", [
     (6, 5, 7, 8, np.float32, 1e-4), (64, 256, 256, 512, np.float32, 1e-4), (8, 256, 256, 512, np.float64, 1e-10)],
     ids=["reduced", "full_size", "double_on_matrix_cores"])
-def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid, np_dtype, rtol):
+def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid, np_dtype, rtol, evaluator):
     """config 4 at reduced size (seq 6, batch 5, in 7, hidden 8) and at its
     full size: the layer.yml lstm recipe with one fused gate weight {4h, in+h}
     cut by SLICEs, loss = sum(h^2) over the concatenated hidden outputs,
     against torch autograd in fp64.  The third case is the graph in double at
     the full widths (its 256x768x2048 products run on the fp64 matrix cores),
-    eight steps long, at 1e-10."""
+    eight steps long, at 1e-10.  Under "replay" the values compared are those
+    of the third evaluation, which a recording serves: the launches the
+    benchmark times (shared launches, products over parts of concatenations,
+    products with their reading group as epilogue) are held to torch
+    directly, at the same bar."""
     torch = torch_reference()
     if batch > 16:
         torch.set_num_threads(16)
@@ -266,7 +296,7 @@ def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid, np_dtyp
     out = api.lstm(x, state0, hidden0, {"g": gate(0), "i": gate(1), "f": gate(2), "o": gate(3)}, seq_dim=1)
     loss = api.reduce_sum(api.square(out))
     (dw,) = g.derive(loss, [w])
-    g.evaluate([out, loss, dw])
+    evaluate_under(g, evaluator, [out, loss, dw], x, x_np)
 
     xt = torch.tensor(x_np, dtype=torch.float64)
     wt = torch.tensor(w_np, dtype=torch.float64, requires_grad=True)
@@ -293,12 +323,15 @@ def test_config4_lstm_forward_and_gradient(g, api, seq, batch, nin, hid, np_dtyp
     (3, 12, 4, 6, 5, np.float32, 1e-4), (16, 20, 8, 32, 10, np.float32, 1e-4), (128, 28, 32, 64, 10, np.float32, 1e-4),
     (16, 20, 8, 32, 10, np.float64, 1e-10)],
     ids=["direct_kernels", "matrix_products", "full_size", "double"])
-def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls, np_dtype, rtol):
+@pytest.mark.parametrize("evaluator", ["plain", "replay"])
+def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls, np_dtype, rtol, evaluator):
     """config 5 at reduced size (5x5 kernels 1->c1->c2, dense c2->ncls): the
     nn.yml conv2d idiom and its gradient idioms (PAD / REVERSE / CONV / PERMUTE
     / SLICE), softmax cross-entropy, against torch.  The first size stays on
     the direct convolution kernels; at the second the second layer's forward,
-    image-gradient and kernel-gradient convolutions run as matrix products."""
+    image-gradient and kernel-gradient convolutions run as matrix products.
+    Under "replay" the values compared are those of the third evaluation,
+    served by a recording (convolutions over views, shared launches)."""
     torch = torch_reference()
     if batch > 16:
         torch.set_num_threads(16)
@@ -324,7 +357,7 @@ def test_config5_cnn_forward_and_gradient(g, api, batch, hw, c1, c2, ncls, np_dt
     probs = api.softmax(logits, 0, 1)
     loss = api.reduce_sum(api.cross_entropy(y, probs))
     grads = g.derive(loss, [k1, k2, wd])
-    g.evaluate([loss] + grads)
+    evaluate_under(g, evaluator, [loss] + grads, x, x_np)
 
     xt = torch.tensor(x_np, dtype=torch.float64).permute(0, 3, 1, 2)
     k1t = torch.tensor(k1_np, dtype=torch.float64, requires_grad=True)
