@@ -294,7 +294,11 @@ typedef struct tcg_fx_leaf
 	 * side by side (tcg_gemm_terms_ranges).  0 and 1 both mean a plain operand. */
 	int64_t sum_stride;
 	uint32_t nsum;
-	uint32_t reserved_;
+	/* 1: the operand is (a part of) the result of the matrix product that
+	 * tcg_gemm_terms_fx computes in the same launch, never laid out in memory:
+	 * ptr is ignored, offset / stride address the M x N result as a row-major
+	 * matrix of row length N.  0 everywhere else. */
+	uint32_t from_product;
 } tcg_fx_leaf;
 typedef struct tcg_fx_instr
 {
@@ -464,6 +468,36 @@ int tcg_gemm_terms_ranges (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint
 	const void* const* A, const uint64_t* lda, int trans_a,
 	const void* const* B, const uint64_t* ldb, int trans_b,
 	int nranges, void* ranges);
+/* tcg_gemm_terms whose result is read by one group of elementwise nodes and by
+ * nothing else, product and group as ONE launch: the product's values go from
+ * the matrix cores to the group's arithmetic in registers and are never laid
+ * out.  A time step of a recurrent cell is such a pair -- the gate product
+ * over [x_t, h] followed by the gate activations and the state update
+ * (cfg/tenncor/layer.yml:297-345, 716-768), and backwards the product of the
+ * gate gradients with the transposed weight followed by the derivative
+ * factors of the step before (tenncor/eteq/backprop.hpp:269-359) -- and as two
+ * launches it is bound by being launched, not by arithmetic.
+ * The group is given as to tcg_ew_fusedx; the leaves that read the product
+ * set from_product and address its M x N result as a row-major matrix with
+ * row length N.  Every such leaf must walk the result row by row the way the
+ * group walks its own elements: with J = shape[0] and rows = shape[1] * ... *
+ * shape[7] = M, group element (j, row) reads result element (row, offset + j),
+ * 0 <= offset, offset + J <= N (the SLICEs that cut the gates out of one
+ * product are four such leaves with offsets 0, J, 2J, 3J).  Results equal
+ * tcg_gemm_terms followed by tcg_ew_fusedx up to the order of the additions
+ * over K (each element is summed in a fixed order, in K ranges that are added
+ * in range order: results do not depend on scheduling); the group's own
+ * arithmetic is the same scalar code in the same order.
+ * fp32 only, trans_a = 0, K a multiple of 16, 16-byte aligned operands with
+ * leading dims that are multiples of four, at most 8 terms; anything else fails
+ * with TCG_ERR_UNSUPPORTED and launches nothing (the caller then runs the two
+ * launches).  The kernel is compiled at run time for the shape of the product
+ * and the program of the group and kept for the life of the process. */
+int tcg_gemm_terms_fx (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K, int nterms,
+	const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b,
+	const uint64_t shape[8], int nleaves, const tcg_fx_leaf* leaves,
+	int ninstrs, const tcg_fx_instr* program, int nouts, void* const* outs);
 /* CONV (cfg/ops.yml:566-607; internal/eigen/operator.hpp:1141-1187):
  * valid cross-correlation, kernel dim i slides along image dim ranks[i] */
 int tcg_conv (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],

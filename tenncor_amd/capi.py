@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -64,7 +64,7 @@ class EwInstr(ctypes.Structure):
 class FxLeaf(ctypes.Structure):
     _fields_ = [("ptr", ctypes.c_void_p), ("offset", ctypes.c_int64), ("stride", ctypes.c_int64 * 8),
                 ("lo", ctypes.c_uint64 * 8), ("hi", ctypes.c_uint64 * 8),
-                ("sum_stride", ctypes.c_int64), ("nsum", ctypes.c_uint32), ("reserved_", ctypes.c_uint32)]
+                ("sum_stride", ctypes.c_int64), ("nsum", ctypes.c_uint32), ("from_product", ctypes.c_uint32)]
 
 
 class FxInstr(ctypes.Structure):
@@ -136,6 +136,8 @@ def load():
         "tcg_gemm_terms": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
         "tcg_gemm_terms_ranges": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32, i32, vp],
         "tcg_gemm_terms_grid": [vp, i32, i32, u64p, i32, u64p, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
+        "tcg_gemm_terms_fx": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32,
+                              u64p, i32, ctypes.POINTER(FxLeaf), i32, ctypes.POINTER(FxInstr), i32, vpp],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
@@ -336,18 +338,15 @@ class Context:
         ptrs = (ctypes.c_void_p * len(leaves))(*leaves)
         self._check(self.lib.tcg_ew_fused(self.handle, dtype, n, len(leaves), ptrs, len(program), instrs, dst))
 
-    def ew_fusedx(self, dtype, shape, leaves, program, outs):
-        """leaves: dicts with ptr, and optionally offset, stride (8 element
-        strides; default: dense over `shape`), lo, hi (default: everything),
-        nsum and sum_stride (the value is the sum of nsum elements that far apart).
-        program: tuples (opcode | "STORE", a, b, c, dst[, imm])."""
+    @staticmethod
+    def _fx_group(shape, leaves, program, outs):
         shp = shape8(shape)
         dense = [1] * RANK_CAP
         for d in range(1, RANK_CAP):
             dense[d] = dense[d - 1] * shp[d - 1]
         lv = (FxLeaf * len(leaves))()
         for k, leaf in enumerate(leaves):
-            lv[k].ptr = leaf["ptr"]
+            lv[k].ptr = leaf.get("ptr")
             lv[k].offset = int(leaf.get("offset", 0))
             for d in range(RANK_CAP):
                 lv[k].stride[d] = int(leaf.get("stride", dense)[d])
@@ -355,14 +354,36 @@ class Context:
                 lv[k].hi[d] = int(leaf.get("hi", shp)[d])
             lv[k].nsum = int(leaf.get("nsum", 0))
             lv[k].sum_stride = int(leaf.get("sum_stride", 0))
+            lv[k].from_product = int(leaf.get("from_product", 0))
         instrs = (FxInstr * len(program))()
         for i, ins in enumerate(program):
             instrs[i].opcode = {"STORE": FX_STORE, "BITOR": FX_BITOR}.get(ins[0]) or _opcode(ins[0])
             instrs[i].a, instrs[i].b, instrs[i].c, instrs[i].dst = ins[1], ins[2], ins[3], ins[4]
             instrs[i].imm = float(ins[5]) if len(ins) > 5 else 0.0
         ptrs = (ctypes.c_void_p * len(outs))(*outs)
+        return shp, lv, instrs, ptrs
+
+    def ew_fusedx(self, dtype, shape, leaves, program, outs):
+        """leaves: dicts with ptr, and optionally offset, stride (8 element
+        strides; default: dense over `shape`), lo, hi (default: everything),
+        nsum and sum_stride (the value is the sum of nsum elements that far apart).
+        program: tuples (opcode | "STORE", a, b, c, dst[, imm])."""
+        shp, lv, instrs, ptrs = self._fx_group(shape, leaves, program, outs)
         self._check(self.lib.tcg_ew_fusedx(self.handle, dtype, _u64(shp), len(leaves), lv, len(program), instrs,
                                            len(outs), ptrs))
+
+    def gemm_terms_fx(self, dtype, M, N, K, a_ptrs, lda, trans_a, b_ptrs, ldb, trans_b, shape, leaves, program, outs):
+        """gemm_terms with the group that reads its result as the epilogue of
+        the same launch.  Leaves with from_product=1 address the M x N result
+        (row length N): offset = first column, stride as over a [N, M] tensor."""
+        n = len(a_ptrs)
+        pa = (ctypes.c_void_p * n)(*a_ptrs)
+        pb = (ctypes.c_void_p * n)(*b_ptrs)
+        la = (ctypes.c_uint64 * n)(*[int(v) for v in lda])
+        lb = (ctypes.c_uint64 * n)(*[int(v) for v in ldb])
+        shp, lv, instrs, ptrs = self._fx_group(shape, leaves, program, outs)
+        self._check(self.lib.tcg_gemm_terms_fx(self.handle, dtype, M, N, K, n, pa, la, int(trans_a), pb, lb, int(trans_b),
+                                               _u64(shp), len(leaves), lv, len(program), instrs, len(outs), ptrs))
 
     # ---- reductions ----
     def reduce(self, op, dtype, shape, rank_set, src, dst):

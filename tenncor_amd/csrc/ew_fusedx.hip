@@ -402,9 +402,11 @@ struct FxParts
 
 /// `sfx` is appended to every local name (several indices in one scope);
 /// `idx` names the index variable; `stream`: leaves whose every element is
-/// read exactly once are loaded with the non-temporal hint
+/// read exactly once are loaded with the non-temporal hint; `supplied[k]`:
+/// leaf k is not loaded -- the caller declares `T l<k><sfx>[N]` itself, between
+/// the loads and the arithmetic
 void fx_emit_parts (FxParts& parts, int N, const FxArgs& p, const bool* dense, const FxBake* bake,
-	const std::string& sfx, const std::string& idx, bool stream)
+	const std::string& sfx, const std::string& idx, bool stream, const bool* supplied = nullptr)
 {
 	std::ostringstream& o = parts.load;
 	// how the generated code names a launch argument: a field of `p`, or (baked)
@@ -437,7 +439,7 @@ void fx_emit_parts (FxParts& parts, int N, const FxArgs& p, const bool* dense, c
 		return std::string("(") + text + ")";
 	};
 	bool need_coords = false;
-	for (uint32_t k = 0; k < p.nleaf; ++k) { need_coords = need_coords || !dense[k]; }
+	for (uint32_t k = 0; k < p.nleaf; ++k) { need_coords = need_coords || (!dense[k] && !(supplied && supplied[k])); }
 	if (need_coords)
 	{
 		o << "uint32_t rem" << sfx << " = " << idx << ";\n";
@@ -458,6 +460,7 @@ void fx_emit_parts (FxParts& parts, int N, const FxArgs& p, const bool* dense, c
 	for (uint32_t k = 0; k < p.nleaf; ++k)
 	{
 		const FxLeaf& L = p.leaf[k];
+		if (supplied && supplied[k]) { continue; }
 		// every element read once: no zero stride over an extent above one
 		bool once = stream && !L.bcast0 && !L.boxed;
 		for (uint32_t d = 0; d < p.nd && once; ++d) { once = dense[k] || p.size[d] == 1 || L.stride[d] != 0; }
@@ -1154,11 +1157,19 @@ namespace
 {
 } // namespace
 
-extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
-	int nleaves, const tcg_fx_leaf* leaves, int ninstrs, const tcg_fx_instr* program,
-	int nouts, void* const* outs)
+namespace
 {
-	if (!ctx) { return TCG_ERR_ARG; }
+
+// Checks a group as tcg_ew_fusedx receives it and turns it into the launch
+// arguments of its kernels: iteration dims merged, views per dim, the program.
+// `vec`: every operand and result can be moved 16 bytes at a time.
+// A leaf whose `from_product` is set has no memory of its own (its values are
+// handed to the group by the matrix product the group is the epilogue of):
+// its pointer may be NULL and says nothing about alignment.
+int fx_prepare (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
+	int nleaves, const tcg_fx_leaf* leaves, int ninstrs, const tcg_fx_instr* program,
+	int nouts, void* const* outs, FxArgs& p, bool& vec)
+{
 	TCG_REQUIRE(ctx, shape && leaves && program && outs, "tcg_ew_fusedx: NULL pointer");
 	TCG_REQUIRE(ctx, nleaves >= 1 && nleaves <= TCG_FX_MAX_LEAVES, "tcg_ew_fusedx: %d leaves (1..%d allowed)", nleaves, TCG_FX_MAX_LEAVES);
 	TCG_REQUIRE(ctx, ninstrs >= 1 && ninstrs <= TCG_FX_MAX_INSTRS, "tcg_ew_fusedx: %d instructions (1..%d allowed)", ninstrs, TCG_FX_MAX_INSTRS);
@@ -1175,12 +1186,11 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 	{
 		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_ew_fusedx: %llu elements exceed the 2^32 limit of one launch", (unsigned long long) total);
 	}
-	for (int k = 0; k < nleaves; ++k) { TCG_REQUIRE(ctx, leaves[k].ptr, "tcg_ew_fusedx: leaf %d is NULL", k); }
+	for (int k = 0; k < nleaves; ++k) { TCG_REQUIRE(ctx, leaves[k].ptr || leaves[k].from_product, "tcg_ew_fusedx: leaf %d is NULL", k); }
 	for (int k = 0; k < nouts; ++k) { TCG_REQUIRE(ctx, outs[k], "tcg_ew_fusedx: output %d is NULL", k); }
 
 	// the program: every operand names a leaf, a register written earlier or
 	// the immediate; every output is stored
-	FxArgs p;
 	memset(&p, 0, sizeof(p));
 	bool written[TCG_FX_MAX_REGS] = {false};
 	bool stored[TCG_FX_MAX_OUTS] = {false};
@@ -1275,7 +1285,7 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 	p.total = total;
 	for (uint32_t d = 0; d < nd; ++d) { p.div[d] = fx_make_div(p.size[d]); }
 	const int N = (int) (16 / esz);
-	bool vec = p.size[0] % N == 0;
+	vec = p.size[0] % N == 0;
 	for (int k = 0; k < nouts; ++k)
 	{
 		p.out[k] = outs[k];
@@ -1294,13 +1304,430 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 		L.bcast0 = L.stride[0] == 0;
 		if (!L.bcast0)
 		{
-			vec = vec && L.stride[0] == 1 && L.off % N == 0 && tcg_aligned16(L.ptr);
+			vec = vec && L.stride[0] == 1 && L.off % N == 0 && (leaves[k].from_product || tcg_aligned16(L.ptr));
 			for (uint32_t d = 1; d < nd; ++d) { vec = vec && L.stride[d] % N == 0; }
 		}
 		if (L.boxed) { vec = vec && L.lo[0] % N == 0 && L.hi[0] % N == 0; }
 	}
+	return TCG_OK;
+}
+
+} // namespace
+
+extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
+	int nleaves, const tcg_fx_leaf* leaves, int ninstrs, const tcg_fx_instr* program,
+	int nouts, void* const* outs)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	FxArgs p;
+	bool vec = false;
+	int rc = fx_prepare(ctx, dtype, shape, nleaves, leaves, ninstrs, program, nouts, outs, p, vec);
+	if (rc != TCG_OK) { return rc; }
+	for (int k = 0; k < nleaves; ++k)
+	{
+		TCG_REQUIRE(ctx, 0 == leaves[k].from_product, "tcg_ew_fusedx: leaf %d names a matrix product (tcg_gemm_terms_fx takes such groups)", k);
+	}
 	if (tcg_small_mode(ctx)) { return small_append_fx(ctx, dtype, p); }
 	if (fx_jit_enabled() || false == tcg_default_dtype(dtype)) { return fusedx_jit_launch(ctx, dtype, p, vec); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return fusedx_launch<T>(ctx, p, vec)); // the interpreter: double, float, int32
+	return TCG_OK;
+}
+
+// ---- a matrix product with the group that reads it as its epilogue -----------
+//
+// C = sum_t A_t B_t (M x N, fp32) is read by one elementwise group and by
+// nothing else; the group's shape is [J, rows = M] and its product leaves read
+// C(row, off_g + j).  One workgroup owns TM rows x TJ group columns, that is the
+// TM x (G TJ) results the G product leaves need there, and its NW waves split
+// the summed index between them: a wave multiplies its range of K for the whole
+// tile with v_mfma_f32_16x16x4_f32, operands going from memory to registers in
+// the layout the instruction takes (lane l holds row / column l % 16 and the
+// four summed indices 4 (l / 16) .. + 3 of a step of 16, one 128-bit load), a
+// few steps ahead of the arithmetic: no LDS, no barrier inside the loop.  The
+// NW partial tiles meet in LDS and are added in wave order by the lane that
+// then runs the group's program on that element, with the other operands of
+// the group loaded before the product started.
+// The source is generated for the shape (tile, leading dims, terms, layouts) and
+// the program; pointers are the only launch arguments.
+
+namespace
+{
+
+struct GfxTile
+{
+	int NW = 0, TM = 0, TJ = 0, N = 1; // waves, rows, group columns per workgroup; elements per lane in the epilogue
+};
+
+// the tile with the least operand traffic among those that put a workgroup on every CU
+bool gfx_choose_tile (const tcg_ctx* ctx, uint64_t M, uint64_t J, int G, uint64_t ktot, bool trans_b, bool vec, GfxTile& out)
+{
+	int nw = 0;
+	for (int w : {8, 4, 2, 1})
+	{
+		if (ktot % (16 * (uint64_t) w) == 0) { nw = w; break; }
+	}
+	if (nw == 0) { return false; }
+	double best = 0.0;
+	bool found = false;
+	for (int tm : {16, 32, 64})
+	{
+		for (int tj : {4, 8, 16, 32, 64, 128})
+		{
+			const int nc = G * tj;
+			if (J % (uint64_t) tj != 0) { continue; }
+			if (trans_b ? nc % 16 != 0 : nc % 64 != 0) { continue; }
+			const int accs = (tm / 16) * (nc / 16) * 4; // accumulator registers per lane
+			if (accs > 128) { continue; }
+			if ((size_t) nw * tm * nc * sizeof(float) > 65536) { continue; }
+			// one element (or one 16-byte vector of elements) of the group per lane
+			int n = 1;
+			if (tm * tj > 64 * nw)
+			{
+				if (!vec || tj % 4 != 0 || tm * tj / 4 > 64 * nw) { continue; }
+				n = 4;
+			}
+			const uint64_t groups = ((M + tm - 1) / tm) * (J / tj);
+			const double fill = groups >= (uint64_t) ctx->num_cus ? 1.0 : (double) groups / ctx->num_cus;
+			// operand elements fetched per result: 1 / rows + 1 / columns of the tile
+			const double score = fill * fill / (1.0 / tm + 1.0 / nc);
+			if (!found || score > best)
+			{
+				best = score;
+				found = true;
+				out.NW = nw;
+				out.TM = tm;
+				out.TJ = tj;
+				out.N = n;
+			}
+		}
+	}
+	return found;
+}
+
+struct GfxShape
+{
+	uint32_t M = 0, J = 0, KT = 0, nterms = 0;
+	bool trans_b = false;
+	uint32_t lda[8], ldb[8];
+	int G = 0;
+	uint32_t noff[TCG_FX_MAX_LEAVES]; // first column of product leaf g
+	int leaf_of[TCG_FX_MAX_LEAVES];   // product leaf g -> leaf of the group
+};
+
+std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, const bool* dense, const bool* supplied)
+{
+	const int NT = 64 * t.NW, RB = t.TM / 16, NC = sh.G * t.TJ, CB = NC / 16, CG = NC / 64;
+	const uint32_t ktot = sh.KT * sh.nterms, KW = ktot / t.NW, NSTEPS = KW / 16;
+	const int BL = sh.trans_b ? CB : 4 * CG; // 128-bit loads of B per step and lane
+	// steps on their way while one is multiplied: about sixteen loads per wave
+	int depth = 16 / (RB + BL) + 1;
+	if (depth < 2) { depth = 2; }
+	if (depth > 6) { depth = 6; }
+	if ((uint32_t) depth > NSTEPS) { depth = (int) NSTEPS; }
+	const uint32_t tiles_m = (sh.M + t.TM - 1) / t.TM, tiles_j = sh.J / t.TJ;
+	const int items = t.TM * t.TJ / t.N;
+	std::ostringstream o;
+	fx_emit_prelude(o);
+	o << "typedef float T;\ntypedef float f4 __attribute__((ext_vector_type(4)));\n";
+	if (t.N > 1) { o << "typedef T VT __attribute__((ext_vector_type(" << t.N << ")));\nunion VU { VT v; T e[" << t.N << "]; };\n"; }
+	o << "struct GfxArgs { const float* A[" << sh.nterms << "]; const float* B[" << sh.nterms << "]; const void* leaf["
+		<< TCG_FX_MAX_LEAVES << "]; void* out[" << TCG_FX_MAX_OUTS << "]; };\n";
+	auto pick = [&](const char* name, const uint32_t* vals)
+	{
+		// leading dim of the term a step belongs to (wave-uniform)
+		o << "__device__ __forceinline__ uint32_t " << name << " (uint32_t term) { return ";
+		for (uint32_t k = 0; k + 1 < sh.nterms; ++k) { o << "term == " << k << "u ? " << vals[k] << "u : "; }
+		o << vals[sh.nterms - 1] << "u; }\n";
+	};
+	pick("lda_of", sh.lda);
+	pick("ldb_of", sh.ldb);
+	o << "__device__ __forceinline__ uint32_t col_of (uint32_t c, uint32_t j0) { const uint32_t g = c / " << t.TJ << "u; return j0 + (c - g * "
+		<< t.TJ << "u) + (";
+	for (int g = 0; g + 1 < sh.G; ++g) { o << "g == " << g << "u ? " << sh.noff[g] << "u : "; }
+	o << sh.noff[sh.G - 1] << "u); }\n";
+	o << "extern \"C\" __global__ __launch_bounds__(" << NT << ") void fx (GfxArgs a)\n{\n"
+		"__shared__ __attribute__((aligned(16))) float red[" << t.NW * t.TM * NC << "];\n"
+		"const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);\n"
+		"const uint32_t r16 = lane & 15u, q = lane >> 4;\n";
+	// workgroups are dealt to the eight XCDs in turn: each XCD keeps a band of
+	// columns, whose part of B then stays in that XCD's L2 from launch to launch
+	if (tiles_j % 8 == 0)
+	{
+		o << "const uint32_t local = blockIdx.x >> 3;\n"
+			"const uint32_t tj = (blockIdx.x & 7u) * " << tiles_j / 8 << "u + local % " << tiles_j / 8 << "u, tm = local / " << tiles_j / 8 << "u;\n";
+	}
+	else { o << "const uint32_t tm = blockIdx.x % " << tiles_m << "u, tj = blockIdx.x / " << tiles_m << "u;\n"; }
+	o << "const uint32_t m0 = tm * " << t.TM << "u, j0 = tj * " << t.TJ << "u;\n";
+	// the element of the group this lane computes at the end, and its other operands
+	o << "const uint32_t er = tid / " << t.TJ / t.N << "u, ej = (tid % " << t.TJ / t.N << "u) * " << t.N << "u;\n"
+		"const bool item = tid < " << items << "u && m0 + er < " << sh.M << "u;\n"
+		"const uint32_t idx = item ? ((m0 + er) * " << sh.J << "u + j0 + ej) / " << t.N << "u : 0u;\n";
+	FxBake bake;
+	for (uint32_t k = 0; k < p.nleaf; ++k) { bake.leaf_ptr[k] = "a.leaf[" + std::to_string(k) + "]"; }
+	for (uint32_t k = 0; k < p.nout; ++k) { bake.out_ptr[k] = "a.out[" + std::to_string(k) + "]"; }
+	FxParts parts;
+	fx_emit_parts(parts, t.N, p, dense, &bake, "", "idx", false, supplied);
+	o << parts.load.str();
+	// ---- the product ----
+	o << "uint32_t arow[" << RB << "];\n";
+	for (int rb = 0; rb < RB; ++rb)
+	{
+		o << "arow[" << rb << "] = m0 + " << rb * 16 << "u + r16 < " << sh.M << "u ? m0 + " << rb * 16 << "u + r16 : " << sh.M - 1 << "u;\n";
+	}
+	if (sh.trans_b)
+	{
+		o << "uint32_t bcol[" << CB << "];\n";
+		for (int cb = 0; cb < CB; ++cb) { o << "bcol[" << cb << "] = col_of(" << cb * 16 << "u + r16, j0);\n"; }
+	}
+	else
+	{
+		o << "uint32_t bcol[" << CG << "];\n";
+		for (int cg = 0; cg < CG; ++cg) { o << "bcol[" << cg << "] = col_of(" << cg * 64 << "u + 4u * r16, j0);\n"; }
+	}
+	o << "f4 acc[" << RB << "][" << CB << "];\n"
+		"_Pragma(\"unroll\") for (int i = 0; i < " << RB << "; ++i) { _Pragma(\"unroll\") for (int j = 0; j < " << CB << "; ++j) { acc[i][j] = (f4) (0.0f); } }\n"
+		"f4 ra[" << depth << "][" << RB << "], rb[" << depth << "][" << BL << "];\n"
+		"const uint32_t kbase = wave * " << KW << "u;\n";
+	auto issue = [&](uint32_t s, int slot)
+	{
+		o << "{\nconst uint32_t k = kbase + " << s * 16 << "u;\n";
+		if (sh.nterms > 1) { o << "const uint32_t term = k / " << sh.KT << "u, kk = k - term * " << sh.KT << "u + 4u * q;\n"; }
+		else { o << "const uint32_t term = 0u, kk = k + 4u * q;\n"; }
+		o << "const float* __restrict__ A = a.A[term];\nconst float* __restrict__ B = a.B[term];\n"
+			"const uint32_t lda = lda_of(term), ldb = ldb_of(term);\n";
+		for (int rb = 0; rb < RB; ++rb)
+		{
+			o << "ra[" << slot << "][" << rb << "] = *(const f4*) (A + (uint64_t) arow[" << rb << "] * lda + kk);\n";
+		}
+		if (sh.trans_b)
+		{
+			for (int cb = 0; cb < CB; ++cb)
+			{
+				o << "rb[" << slot << "][" << cb << "] = *(const f4*) (B + (uint64_t) bcol[" << cb << "] * ldb + kk);\n";
+			}
+		}
+		else
+		{
+			for (int s4 = 0; s4 < 4; ++s4)
+			{
+				for (int cg = 0; cg < CG; ++cg)
+				{
+					o << "rb[" << slot << "][" << s4 * CG + cg << "] = *(const f4*) (B + (uint64_t) (kk + " << s4 << "u) * ldb + bcol[" << cg << "]);\n";
+				}
+			}
+		}
+		o << "}\n";
+	};
+	auto multiply = [&](int slot)
+	{
+		for (int s4 = 0; s4 < 4; ++s4)
+		{
+			for (int rb = 0; rb < RB; ++rb)
+			{
+				for (int cb = 0; cb < CB; ++cb)
+				{
+					o << "acc[" << rb << "][" << cb << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[" << slot << "][" << rb << "][" << s4 << "], ";
+					if (sh.trans_b) { o << "rb[" << slot << "][" << cb << "][" << s4 << "]"; }
+					else { o << "rb[" << slot << "][" << s4 * CG + cb / 4 << "][" << cb % 4 << "]"; }
+					o << ", acc[" << rb << "][" << cb << "], 0, 0, 0);\n";
+				}
+			}
+		}
+	};
+	if (NSTEPS <= 32)
+	{
+		for (uint32_t s = 0; s + 1 < (uint32_t) depth; ++s) { issue(s, (int) s); }
+		for (uint32_t s = 0; s < NSTEPS; ++s)
+		{
+			if (s + depth - 1 < NSTEPS) { issue(s + depth - 1, (int) ((s + depth - 1) % depth)); }
+			multiply((int) (s % depth));
+		}
+	}
+	else
+	{
+		// a long K: the steps in a loop, one at a time on its way
+		o << "for (uint32_t s = 0; s < " << NSTEPS << "u; ++s)\n{\n"
+			"const uint32_t k = kbase + s * 16u;\n";
+		if (sh.nterms > 1) { o << "const uint32_t term = k / " << sh.KT << "u, kk = k - term * " << sh.KT << "u + 4u * q;\n"; }
+		else { o << "const uint32_t term = 0u, kk = k + 4u * q;\n"; }
+		o << "const float* __restrict__ A = a.A[term];\nconst float* __restrict__ B = a.B[term];\n"
+			"const uint32_t lda = lda_of(term), ldb = ldb_of(term);\n";
+		for (int rb = 0; rb < RB; ++rb) { o << "ra[0][" << rb << "] = *(const f4*) (A + (uint64_t) arow[" << rb << "] * lda + kk);\n"; }
+		if (sh.trans_b)
+		{
+			for (int cb = 0; cb < CB; ++cb) { o << "rb[0][" << cb << "] = *(const f4*) (B + (uint64_t) bcol[" << cb << "] * ldb + kk);\n"; }
+		}
+		else
+		{
+			for (int s4 = 0; s4 < 4; ++s4)
+			{
+				for (int cg = 0; cg < CG; ++cg)
+				{
+					o << "rb[0][" << s4 * CG + cg << "] = *(const f4*) (B + (uint64_t) (kk + " << s4 << "u) * ldb + bcol[" << cg << "]);\n";
+				}
+			}
+		}
+		multiply(0);
+		o << "}\n";
+	}
+	// ---- the partial tiles meet in LDS: red[wave][row][column of the tile] ----
+	o << "{\nfloat* mine = red + wave * " << t.TM * NC << "u;\n";
+	for (int rb = 0; rb < RB; ++rb)
+	{
+		for (int i = 0; i < 4; ++i)
+		{
+			if (sh.trans_b)
+			{
+				for (int cb = 0; cb < CB; ++cb)
+				{
+					o << "mine[(" << rb * 16 + i << "u + 4u * q) * " << NC << "u + " << cb * 16 << "u + r16] = acc[" << rb << "][" << cb << "][" << i << "];\n";
+				}
+			}
+			else
+			{
+				for (int cg = 0; cg < CG; ++cg)
+				{
+					o << "{ f4 v; ";
+					for (int e = 0; e < 4; ++e) { o << "v[" << e << "] = acc[" << rb << "][" << cg * 4 + e << "][" << i << "]; "; }
+					o << "*(f4*) (mine + (" << rb * 16 + i << "u + 4u * q) * " << NC << "u + " << cg * 64 << "u + 4u * r16) = v; }\n";
+				}
+			}
+		}
+	}
+	o << "}\n__syncthreads();\nif (!item) { return; }\n";
+	for (int g = 0; g < sh.G; ++g)
+	{
+		const int k = sh.leaf_of[g];
+		o << "T l" << k << "[" << t.N << "];\n{\nconst float* at = red + er * " << NC << "u + " << g * t.TJ << "u + ej;\n";
+		for (int e = 0; e < t.N; ++e)
+		{
+			o << "{ float s = at[" << e << "];";
+			for (int w = 1; w < t.NW; ++w) { o << " s += at[" << w * t.TM * NC + e << "];"; }
+			o << " l" << k << "[" << e << "] = s; }\n";
+		}
+		o << "}\n";
+	}
+	o << parts.compute.str() << parts.store.str() << "}\n";
+	return o.str();
+}
+
+} // namespace
+
+extern "C" int tcg_gemm_terms_fx (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K, int nterms,
+	const void* const* A, const uint64_t* lda, int trans_a,
+	const void* const* B, const uint64_t* ldb, int trans_b,
+	const uint64_t shape[8], int nleaves, const tcg_fx_leaf* leaves,
+	int ninstrs, const tcg_fx_instr* program, int nouts, void* const* outs)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, A && B && lda && ldb, "tcg_gemm_terms_fx: NULL pointer");
+	TCG_REQUIRE(ctx, nterms >= 1, "tcg_gemm_terms_fx: %d terms", nterms);
+	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, A[t] && B[t], "tcg_gemm_terms_fx: operand of term %d is NULL", t); }
+	FxArgs p;
+	bool vec = false;
+	int rc = fx_prepare(ctx, dtype, shape, nleaves, leaves, ninstrs, program, nouts, outs, p, vec);
+	if (rc != TCG_OK) { return rc; }
+	auto unsupported = [&](const char* why)
+	{
+		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_gemm_terms_fx: %s", why);
+	};
+	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a matrix product with an epilogue"); }
+	if (dtype != TCG_FLOAT || trans_a) { return unsupported("fp32 products with a row-major first operand only"); }
+	if (nterms > 8 || K < 16 || K % 16 != 0 || M < 1 || N < 4 || M >= (1ull << 31) || N >= (1ull << 31) || K * (uint64_t) nterms >= (1ull << 31))
+	{
+		return unsupported("at most 8 terms, K a multiple of 16");
+	}
+	GfxShape sh;
+	sh.M = (uint32_t) M;
+	sh.J = (uint32_t) shape[0];
+	sh.KT = (uint32_t) K;
+	sh.nterms = (uint32_t) nterms;
+	sh.trans_b = trans_b != 0;
+	for (int t = 0; t < nterms; ++t)
+	{
+		bool ok = tcg_aligned16(A[t]) && tcg_aligned16(B[t]) && lda[t] % 4 == 0 && ldb[t] % 4 == 0 &&
+			lda[t] < (1ull << 31) && ldb[t] < (1ull << 31) && lda[t] >= K && ldb[t] >= (trans_b ? K : N);
+		if (!ok) { return unsupported("operands must be 16-byte aligned with leading dims that are multiples of four"); }
+		sh.lda[t] = (uint32_t) lda[t];
+		sh.ldb[t] = (uint32_t) ldb[t];
+	}
+	// the group walks [J, rows]; a product leaf reads result element (row, offset + j)
+	uint64_t rows = 1;
+	for (int d = 1; d < 8; ++d) { rows *= shape[d]; }
+	if (rows != M || shape[0] > N) { return unsupported("the group must have one row per row of the product"); }
+	bool supplied[TCG_FX_MAX_LEAVES] = {false};
+	for (int k = 0; k < nleaves; ++k)
+	{
+		const tcg_fx_leaf& L = leaves[k];
+		if (!L.from_product) { continue; }
+		bool ok = L.nsum <= 1 && L.offset >= 0 && (uint64_t) L.offset + shape[0] <= N && L.offset % 4 == 0;
+		int64_t run = (int64_t) N;
+		for (int d = 0; d < 8 && ok; ++d)
+		{
+			ok = L.lo[d] == 0 && L.hi[d] >= shape[d];
+			if (shape[d] == 1) { continue; }
+			ok = ok && L.stride[d] == (d == 0 ? 1 : run);
+			if (d > 0) { run *= (int64_t) shape[d]; }
+		}
+		if (!ok) { return unsupported("a leaf does not walk the product row by row"); }
+		supplied[k] = true;
+		sh.leaf_of[sh.G] = k;
+		sh.noff[sh.G] = (uint32_t) L.offset;
+		++sh.G;
+	}
+	if (sh.G == 0) { return unsupported("no leaf reads the product"); }
+	if (M * shape[0] >= (1ull << 31)) { return unsupported("too many elements"); }
+	GfxTile tile;
+	if (!gfx_choose_tile(ctx, M, shape[0], sh.G, K * (uint64_t) nterms, sh.trans_b, vec, tile))
+	{
+		return unsupported("no tile fits the shape");
+	}
+	// offsets go into the pointers, so that launches that differ in them share a kernel
+	struct { const float* A[8]; const float* B[8]; const void* leaf[TCG_FX_MAX_LEAVES]; void* out[TCG_FX_MAX_OUTS]; } args;
+	static_assert(sizeof(args) <= 4096, "launch arguments must fit the kernel argument segment");
+	memset(&args, 0, sizeof(args));
+	const size_t esz = tcg_type_size(dtype);
+	for (uint32_t k = 0; k < p.nleaf; ++k)
+	{
+		if (supplied[k]) { continue; }
+		args.leaf[k] = (const char*) p.leaf[k].ptr + (int64_t) esz * p.leaf[k].off;
+		p.leaf[k].off = 0;
+		p.leaf[k].ptr = nullptr;
+	}
+	for (uint32_t k = 0; k < p.nout; ++k)
+	{
+		args.out[k] = p.out[k];
+		p.out[k] = nullptr;
+	}
+	if (tile.N > 1) { p.div[0] = fx_make_div(p.size[0] / tile.N); }
+	bool dense[TCG_FX_MAX_LEAVES];
+	fx_dense_leaves(p, dense);
+	std::string source = gfx_source(sh, tile, p, dense, supplied);
+	// the kernel's arguments: the term pointers, then the group's
+	std::vector<char> packed(sizeof(void*) * (2 * (size_t) nterms + TCG_FX_MAX_LEAVES + TCG_FX_MAX_OUTS));
+	{
+		char* at = packed.data();
+		for (int t = 0; t < nterms; ++t) { memcpy(at, &A[t], sizeof(void*)); at += sizeof(void*); }
+		for (int t = 0; t < nterms; ++t) { memcpy(at, &B[t], sizeof(void*)); at += sizeof(void*); }
+		memcpy(at, args.leaf, sizeof(args.leaf)); at += sizeof(args.leaf);
+		memcpy(at, args.out, sizeof(args.out));
+	}
+	FxJit& jit = fx_jit();
+	hipFunction_t fn = nullptr;
+	{
+		std::lock_guard<std::mutex> lock(jit.mu);
+		auto it = jit.kernels.find(source);
+		if (it == jit.kernels.end())
+		{
+			rc = fx_compile(ctx, source, &fn);
+			if (rc != TCG_OK) { return rc; }
+			jit.kernels.emplace(source, fn);
+		}
+		else { fn = it->second; }
+	}
+	const unsigned grid = (unsigned) (((M + tile.TM - 1) / tile.TM) * (shape[0] / tile.TJ));
+	size_t size = packed.size();
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, packed.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+	TCG_HIP(ctx, hipModuleLaunchKernel(fn, grid, 1, 1, 64 * tile.NW, 1, 1, 0, ctx->stream, nullptr, config));
 	return TCG_OK;
 }

@@ -145,6 +145,10 @@ struct PartProducts final
 	/// its window side by side in temporary memory ([range][M][N]) and the
 	/// elementwise groups that read the node add them up while they load
 	uint32_t ranges = 0;
+	/// With `ranges` > 0: when one launch of elementwise nodes is all that reads
+	/// the node, the product may run as one launch with that group as its
+	/// epilogue (tcg_gemm_terms_fx) instead of leaving anything in memory
+	bool epilogue = false;
 	/// > 0: `products` are the grid_m x grid_n blocks (row by row) of one result
 	/// whose operands are concatenated along the dims that survive, every block
 	/// (i, j) with the A operands of row i and the B operands of column j and
@@ -164,6 +168,8 @@ struct FusionPlan final
 		int conv = -1;              ///< index into convs, or
 		int sum = -1;               ///< index into sums, or
 		int parts = -1;             ///< index into part_products
+		/// parts and group both >= 0: the product with the group that reads it as
+		/// its epilogue, one launch where the kernel takes the shapes, else the two
 	};
 
 	std::vector<FusedGroup> groups;
@@ -187,7 +193,10 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 /// launch to the last group that reads it
 using RangeTempsT = std::vector<std::pair<void*,size_t>>;
 
-void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps);
+/// `producer` (with its index into the plan's part_products): the product whose
+/// result only this group reads, launched with it (see FusionPlan::Step)
+void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps,
+	const PartProducts* producer = nullptr, int producer_index = -1);
 
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 

@@ -203,7 +203,11 @@ struct Planner final
 			if (n.kind != VIEW || n.target || n.consumers.empty() || n.op == egen::CONTRACT || n.through_conv || n.summed_term) { continue; }
 			n.absorbed = std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
 			{
-				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed && false == nodes_[c].through_conv);
+				// (a CONTRACT that is launched as the swapped product of the PERMUTE behind it, or
+				// as a term of a sum of products, is marked like a view but reads its operands
+				// from memory)
+				return nodes_[c].kind == EW || (nodes_[c].kind == VIEW && nodes_[c].absorbed && false == nodes_[c].through_conv &&
+					nodes_[c].op != egen::CONTRACT && false == nodes_[c].summed_term);
 			});
 			if (false == n.absorbed) { continue; }
 			for (int c : n.consumers)
@@ -966,27 +970,56 @@ struct Planner final
 		const Node& n = nodes_[c];
 		if (n.summed || call.products.size() != 1 || n.dtype != egen::FLOAT) { return; }
 		const PartProducts::Product& p = call.products[0];
-		// the shapes the product kernels split: a transposed operand (row-major
-		// operands with enough 32 x 32 blocks share K between the waves of a workgroup)
-		if (false == (p.trans_a || p.trans_b)) { return; }
 		const uint64_t depth = p.K * p.terms.size();
 		const uint64_t cus = 256;
-		uint64_t tiles128 = ((p.M + 127) / 128) * ((p.N + 127) / 128);
-		if (tiles128 * std::min<uint64_t>(32, depth / 256) >= cus) { return; }
-		uint64_t tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
-		uint64_t want = std::min<uint64_t>({32, 2 * cus / tiles, depth / 128});
-		uint32_t ranges = 1;
-		while (2 * ranges <= want && depth % (2 * ranges * 16) == 0) { ranges *= 2; }
-		if (ranges < 2) { return; }
-		// every reader adds the ranges up again: worth it for one or two
 		if (false == only_groups_read_through(c)) { return; }
-		size_t readers = 0;
-		for (int v : n.consumers) { readers += nodes_[v].consumers.size(); }
-		if (readers > 2) { return; }
+		// few results that elementwise nodes are all that reads (a time step of a recurrent
+		// cell): the product may take the launch of those nodes as its epilogue, which
+		// finish() decides when it knows the launches.  Until then, and when it decides
+		// otherwise, the result waits for them in temporary memory like K ranges do
+		const uint64_t tiles128 = ((p.M + 127) / 128) * ((p.N + 127) / 128);
+		const bool few = tiles128 < 2 * cus;
+		call.epilogue = few && false == p.trans_a && p.terms.size() <= 8 && epilogues_enabled();
+		// the shapes the product kernels split: a transposed operand (row-major
+		// operands with enough 32 x 32 blocks share K between the waves of a workgroup)
+		uint32_t ranges = 1;
+		if ((p.trans_a || p.trans_b) && tiles128 * std::min<uint64_t>(32, depth / 256) < cus)
+		{
+			uint64_t tiles = ((p.M + 63) / 64) * ((p.N + 63) / 64);
+			uint64_t want = std::min<uint64_t>({32, 2 * cus / tiles, depth / 128});
+			while (2 * ranges <= want && depth % (2 * ranges * 16) == 0) { ranges *= 2; }
+			// every reader adds the ranges up again: worth it for one or two
+			size_t readers = 0;
+			for (int v : n.consumers) { readers += nodes_[v].consumers.size(); }
+			if (readers > 2) { ranges = 1; }
+		}
+		if (ranges < 2 && false == call.epilogue) { return; }
 		// ... and the groups must see the product's dtype (a view changes none)
 		call.ranges = ranges;
 		call.label += " ranges=" + std::to_string(ranges);
 		nodes_[c].ranged = true;
+	}
+
+	/// TCR_EPILOGUES=0 keeps every product and the group that reads it apart (two
+	/// launches, as the check of the single one)
+	static bool epilogues_enabled (void)
+	{
+		static const bool on = []
+		{
+			const char* env = getenv("TCR_EPILOGUES");
+			return !(env && env[0] == '0');
+		}();
+		return on;
+	}
+
+	/// The elementwise nodes that read node v through folded views
+	void readers_through (int v, std::vector<int>& out) const
+	{
+		for (int c : nodes_[v].consumers)
+		{
+			if (nodes_[c].kind == EW) { out.push_back(c); }
+			else { readers_through(c, out); }
+		}
 	}
 
 	// ---- sums of products ----
@@ -1965,11 +1998,26 @@ struct Planner final
 				{
 					step.group = (int) plan.groups.size();
 					for (int v : views) { last_user[v] = step.group; }
+					const int producer = epilogue_producer(members, lo, hi, group);
 					for (FusedGroup::Leaf& leaf : group.leaves)
 					{
 						if (leaf.ranges_of < 0) { continue; }
 						leaf.ranges_of = emitted_parts_.at(leaf.ranges_of);
 						last_ranges[leaf.ranges_of] = step.group;
+					}
+					if (producer >= 0)
+					{
+						// the product moves from where it stood to this launch
+						const int at = emitted_parts_.at(producer);
+						auto old = std::find_if(plan.steps.begin(), plan.steps.end(), [&](const FusionPlan::Step& st)
+						{
+							return st.parts == at && st.group < 0;
+						});
+						if (old != plan.steps.end())
+						{
+							plan.steps.erase(old);
+							step.parts = at;
+						}
 					}
 					for (size_t p = lo; p < hi; ++p)
 					{
@@ -2030,6 +2078,50 @@ struct Planner final
 		return plan;
 	}
 
+	/// The product (index into part_calls_) that can take the launch of members
+	/// [lo, hi) as its epilogue: the only product whose result the launch reads in
+	/// place of a tensor, read by nothing outside the launch, with nothing
+	/// rewriting its operands between where it stands and where the launch does;
+	/// -1 when there is none
+	int epilogue_producer (const std::vector<int>& members, size_t lo, size_t hi, const FusedGroup& group) const
+	{
+		int producer = -1;
+		for (const FusedGroup::Leaf& leaf : group.leaves)
+		{
+			if (leaf.ranges_of < 0) { continue; }
+			if (producer >= 0 && producer != leaf.ranges_of) { return -1; }
+			producer = leaf.ranges_of;
+		}
+		if (producer < 0 || false == part_calls_[producer].epilogue) { return -1; }
+		int c = -1;
+		for (size_t i = 0; i < nodes_.size() && c < 0; ++i)
+		{
+			if (nodes_[i].part_products == producer) { c = (int) i; }
+		}
+		if (c < 0) { return -1; }
+		std::vector<int> readers;
+		readers_through(c, readers);
+		for (int r : readers)
+		{
+			if (std::find(members.begin() + lo, members.begin() + hi, r) == members.begin() + hi) { return -1; }
+		}
+		// the product would read its operands where the launch stands
+		const int last = members[hi - 1];
+		for (size_t k = 0; k < nodes_[c].args.size(); ++k)
+		{
+			int a = nodes_[c].args[k];
+			if (written_between(c, {k}, c, last)) { return -1; }
+			if (a >= 0 && nodes_[a].parts_folded)
+			{
+				for (size_t j = 0; j < nodes_[a].args.size(); ++j)
+				{
+					if (written_between(a, {j}, a, last)) { return -1; }
+				}
+			}
+		}
+		return producer;
+	}
+
 	/// Folded concatenation z and the views beneath it are read by products `step`
 	void mark_parts_user (int z, int step, std::map<int,int>& last_parts) const
 	{
@@ -2086,7 +2178,11 @@ void launch_contract (const SwappedContract& call, const teq::TensSetT& targets,
 	if (nullptr == dst) { global::fatalf("%s cannot take a product", out->to_string().c_str()); }
 	const void* a = eigen_ref(*call.a).device_data();
 	const void* b = eigen_ref(*call.b).device_data();
-	if (nullptr == a || nullptr == b) { global::fatal("operand of a matrix product has no data"); }
+	if (nullptr == a || nullptr == b)
+	{
+		global::fatalf("operand %s of the matrix product behind %s has no data",
+			(nullptr == a ? call.a : call.b)->to_string().c_str(), out->to_string().c_str());
+	}
 	try
 	{
 		hip_check(tcg_contract(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), call.ashape.data(), call.bshape.data(),
@@ -2112,7 +2208,11 @@ void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMe
 	{
 		a.push_back(eigen_ref(*call.a[t]).device_data());
 		b.push_back(eigen_ref(*call.b[t]).device_data());
-		if (nullptr == a.back() || nullptr == b.back()) { global::fatal("operand of a matrix product has no data"); }
+		if (nullptr == a.back() || nullptr == b.back())
+		{
+			global::fatalf("operand %s of term %d of the sum of products %s has no data",
+				(nullptr == a.back() ? call.a[t] : call.b[t])->to_string().c_str(), (int) t, out->to_string().c_str());
+		}
 	}
 	try
 	{
@@ -2141,7 +2241,11 @@ void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMem
 		{
 			const char* pa = (const char*) eigen_ref(*term.a).device_data();
 			const char* pb = (const char*) eigen_ref(*term.b).device_data();
-			if (nullptr == pa || nullptr == pb) { global::fatal("operand of a matrix product has no data"); }
+			if (nullptr == pa || nullptr == pb)
+			{
+				global::fatalf("operand %s of the products over parts %s has no data",
+					(nullptr == pa ? term.a : term.b)->to_string().c_str(), call.label.c_str());
+			}
 			a.push_back(pa + esz * term.a_off);
 			b.push_back(pb + esz * term.b_off);
 			lda.push_back(term.lda);
@@ -2150,9 +2254,18 @@ void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMem
 		if (nullptr == memory) { global::fatal("cannot borrow from null memory"); }
 		temp.second = (size_t) esz * call.ranges * p.M * p.N;
 		temp.first = memory->allocate(temp.second);
-		hip_check(tcg_gemm_terms_ranges(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), p.M, p.N, p.K,
-			(int) p.terms.size(), a.data(), lda.data(), p.trans_a, b.data(), ldb.data(), p.trans_b,
-			(int) call.ranges, temp.first));
+		if (call.ranges == 1)
+		{
+			// (a product that waited for a launch it could have been the epilogue of)
+			hip_check(tcg_gemm_terms(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), p.M, p.N, p.K,
+				(int) p.terms.size(), a.data(), lda.data(), p.trans_a, b.data(), ldb.data(), p.trans_b, temp.first, p.N));
+		}
+		else
+		{
+			hip_check(tcg_gemm_terms_ranges(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), p.M, p.N, p.K,
+				(int) p.terms.size(), a.data(), lda.data(), p.trans_a, b.data(), ldb.data(), p.trans_b,
+				(int) call.ranges, temp.first));
+		}
 		for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 		return;
 	}
@@ -2170,7 +2283,7 @@ void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMem
 		auto address = [&](teq::iTensor* tens, int64_t off)
 		{
 			const char* base = (const char*) eigen_ref(*tens).device_data();
-			if (nullptr == base) { global::fatal("operand of a matrix product has no data"); }
+			if (nullptr == base) { global::fatalf("operand %s of the blocks %s has no data", tens->to_string().c_str(), call.label.c_str()); }
 			return (const void*) (base + esz * off);
 		};
 		for (uint32_t i = 0; i < call.grid_m; ++i)
@@ -2213,7 +2326,11 @@ void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMem
 			{
 				const char* pa = (const char*) eigen_ref(*term.a).device_data();
 				const char* pb = (const char*) eigen_ref(*term.b).device_data();
-				if (nullptr == pa || nullptr == pb) { global::fatal("operand of a matrix product has no data"); }
+				if (nullptr == pa || nullptr == pb)
+			{
+				global::fatalf("operand %s of the products over parts %s has no data",
+					(nullptr == pa ? term.a : term.b)->to_string().c_str(), call.label.c_str());
+			}
 				a.push_back(pa + esz * term.a_off);
 				b.push_back(pb + esz * term.b_off);
 				lda.push_back(term.lda);
@@ -2269,7 +2386,59 @@ void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptr
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
-void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps)
+/// The product of `call` with `group` as its epilogue, one launch; false when
+/// the kernel does not take the shapes (nothing has been launched then)
+static bool launch_with_epilogue (const PartProducts& call, const FusedGroup& group, int producer_index,
+	const std::vector<void*>& outs)
+{
+	const PartProducts::Product& p = call.products.at(0);
+	const int64_t esz = (int64_t) egen::type_size((egen::_GENERATED_DTYPE) call.dtype);
+	std::vector<const void*> a, b;
+	std::vector<uint64_t> lda, ldb;
+	for (const PartProducts::Term& term : p.terms)
+	{
+		const char* pa = (const char*) eigen_ref(*term.a).device_data();
+		const char* pb = (const char*) eigen_ref(*term.b).device_data();
+		if (nullptr == pa || nullptr == pb)
+		{
+			global::fatalf("operand %s of the products over parts %s has no data",
+				(nullptr == pa ? term.a : term.b)->to_string().c_str(), call.label.c_str());
+		}
+		a.push_back(pa + esz * term.a_off);
+		b.push_back(pb + esz * term.b_off);
+		lda.push_back(term.lda);
+		ldb.push_back(term.ldb);
+	}
+	std::vector<tcg_fx_leaf> leaves;
+	for (auto& leaf : group.leaves)
+	{
+		tcg_fx_leaf view = leaf.view;
+		if (leaf.ranges_of == producer_index)
+		{
+			// the view over the dense window, as the kernel's own result
+			view.ptr = nullptr;
+			view.from_product = 1;
+			view.nsum = 0;
+			view.sum_stride = 0;
+		}
+		else
+		{
+			view.ptr = eigen_ref(*leaf.base).device_data();
+			if (nullptr == view.ptr) { global::fatalf("operand %s has no data", leaf.base->to_string().c_str()); }
+		}
+		leaves.push_back(view);
+	}
+	int rc = tcg_gemm_terms_fx(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) call.dtype), p.M, p.N, p.K,
+		(int) p.terms.size(), a.data(), lda.data(), p.trans_a, b.data(), ldb.data(), p.trans_b,
+		group.shape.data(), (int) leaves.size(), leaves.data(), (int) group.program.size(), group.program.data(),
+		(int) outs.size(), outs.data());
+	if (TCG_ERR_UNSUPPORTED == rc) { return false; }
+	hip_check(rc);
+	return true;
+}
+
+void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps,
+	const PartProducts* producer, int producer_index)
 {
 	std::vector<void*> outs;
 	for (Observable* out : group.outputs)
@@ -2279,18 +2448,35 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 		if (nullptr == ptr) { global::fatalf("%s cannot take a fused result", out->to_string().c_str()); }
 		outs.push_back(ptr);
 	}
-	std::vector<tcg_fx_leaf> leaves;
-	for (auto& leaf : group.leaves)
-	{
-		tcg_fx_leaf view = leaf.view;
-		view.ptr = leaf.ranges_of >= 0 ? temps.at(leaf.ranges_of).first : eigen_ref(*leaf.base).device_data();
-		if (nullptr == view.ptr) { global::fatalf("operand %s has no data", leaf.base->to_string().c_str()); }
-		leaves.push_back(view);
-	}
 	try
 	{
-		hip_check(tcg_ew_fusedx(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) group.dtype), group.shape.data(), (int) leaves.size(), leaves.data(),
-			(int) group.program.size(), group.program.data(), (int) outs.size(), outs.data()));
+		bool done = false;
+		if (nullptr != producer)
+		{
+			done = launch_with_epilogue(*producer, group, producer_index, outs);
+			if (false == done)
+			{
+				// two launches after all: the product into temporary memory first
+				launch_parts(*producer, targets, memory, temps.at(producer_index));
+			}
+			else
+			{
+				for (teq::iTensor* tens : producer->reads) { eigen_ref(*tens).odevice(); }
+			}
+		}
+		if (false == done)
+		{
+			std::vector<tcg_fx_leaf> leaves;
+			for (auto& leaf : group.leaves)
+			{
+				tcg_fx_leaf view = leaf.view;
+				view.ptr = leaf.ranges_of >= 0 ? temps.at(leaf.ranges_of).first : eigen_ref(*leaf.base).device_data();
+				if (nullptr == view.ptr) { global::fatalf("operand %s has no data", leaf.base->to_string().c_str()); }
+				leaves.push_back(view);
+			}
+			hip_check(tcg_ew_fusedx(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) group.dtype), group.shape.data(), (int) leaves.size(), leaves.data(),
+				(int) group.program.size(), group.program.data(), (int) outs.size(), outs.data()));
+		}
 	}
 	catch (...)
 	{

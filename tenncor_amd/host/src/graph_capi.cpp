@@ -425,7 +425,7 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 				ss << "summed CONTRACT x" << plan.sums[step.sum].a.size() << "\n";
 				continue;
 			}
-			if (step.parts >= 0)
+			if (step.parts >= 0 && step.group < 0)
 			{
 				ss << plan.part_products[step.parts].label << "\n";
 				continue;
@@ -436,6 +436,7 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 				continue;
 			}
 			auto& group = plan.groups[step.group];
+			if (step.parts >= 0) { ss << plan.part_products[step.parts].label << " with epilogue "; }
 			ss << "group ";
 			for (size_t i = 0; i < group.members.size(); ++i)
 			{

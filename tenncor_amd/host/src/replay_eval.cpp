@@ -288,6 +288,11 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 				{
 					launch_sum(fusion.sums[step.sum], targets, device.memory());
 				}
+				else if (step.parts >= 0 && step.group >= 0)
+				{
+					launch_group(fusion.groups[step.group], targets, device.memory(), temps,
+						&fusion.part_products[step.parts], step.parts);
+				}
 				else if (step.parts >= 0)
 				{
 					launch_parts(fusion.part_products[step.parts], targets, device.memory(), temps[step.parts]);

@@ -265,6 +265,12 @@ def test_mlp_gradient_graph_only_uses_table_opcodes(g, api):
 def parse_plan(lines):
     steps = []
     for line in lines:
+        product, marker, epilogue = line.partition(" with epilogue ")
+        if marker:
+            # a product and the group that reads it as one launch: both steps, the first one flagged
+            kind, _, rest = product.partition(" ")
+            steps.append((kind, rest.split(" ")[0].split("+"), {"epilogue": 1}))
+            line = epilogue
         kind, _, rest = line.partition(" ")
         if kind == "node":
             steps.append(("node", [rest], {}))
@@ -440,10 +446,14 @@ def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
     from tenncor_amd import configs
     targets = configs.config4_lstm(g, seq=5, batch=64, nin=32, hid=64)[0]
     lines = g.launch_plan(targets)
-    assert lines.count("parts CONCAT+CONTRACT x3") == 5, lines   # 32 + 64 joined columns in chunks of 32
-    # only the columns of h are read back, and the groups that read them add the product's two K ranges up
-    assert lines.count("parts ADD+CONTRACT x4+SLICE ranges=2") == 4, lines
+    # 32 + 64 joined columns in chunks of 32; the gate group of a step is all that reads the product,
+    # so the two are one launch and the product's result is never laid out
+    assert sum(l.startswith("parts CONCAT+CONTRACT x3 ranges=1 with epilogue group ") and "TANH" in l for l in lines) == 5, lines
+    # only the columns of h are read back; the group that reads them is the product's epilogue (on its own
+    # it would add the product's two K ranges up)
+    assert sum(l.startswith("parts ADD+CONTRACT x4+SLICE ranges=2 with epilogue group ") for l in lines) == 4, lines
     assert lines.count("blocks CONTRACT x5 2x4") == 1, lines
+    # TCR_EPILOGUES=0 (read once per process) keeps the two launches apart: not exercised here
     assert not any(l.startswith(("summed", "swapped", "node CONTRACT", "node CONCAT", "group CONCAT ")) for l in lines), lines
     steps = parse_plan(lines)
     alone = sum(1 for s in steps if s[0] in ("node", "swapped", "viewed", "summed", "parts", "blocks"))
@@ -474,7 +484,13 @@ def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
     scale = var(g, [128, 64], np.float32, "scale")
     back = api.contract(api.concat([g0, g1], 0), wt, ((0, 0),))      # [192, 64], K = 256 along the memory of both
     lines = g.launch_plan([api.mul(api.slice(back, 64, 128, 0), scale)])
-    assert lines[0] == "parts CONCAT+CONTRACT x2+SLICE ranges=2" and lines[1].startswith("group MUL leaves=2"), lines
+    # ... one launch reads them: it becomes the product's epilogue
+    assert lines[0] == "parts CONCAT+CONTRACT x2+SLICE ranges=2 with epilogue group MUL leaves=2 stores=1 instrs=2", lines
+    # ... two launches of different shapes read them: the ranges wait in memory for both
+    back3 = api.contract(api.concat([g0, g1], 0), wt, ((0, 0),))
+    half = var(g, [64, 64], np.float32, "half")
+    lines = g.launch_plan([api.mul(api.slice(back3, 64, 128, 0), scale), api.mul(api.slice(back3, 0, 64, 0), half)])
+    assert lines[0] == "parts CONCAT+CONTRACT x2 ranges=2" and sum(l.startswith("group MUL leaves=2") for l in lines) == 2, lines
     # ... a reduction reads the slice as a tensor: the product adds its ranges up itself, into the window
     back2 = api.contract(api.concat([g0, g1], 0), wt, ((0, 0),))
     lines = g.launch_plan([api.reduce_sum(api.slice(back2, 64, 128, 0), 0, 1)])
@@ -486,6 +502,24 @@ def test_launch_plan_multiplies_the_parts_of_concatenations(g, api):
     t = api.add(api.add(q1, api.matmul(api.concat([upd, h], 0), w1)), q2)
     lines = g.launch_plan([t])
     assert any(l.startswith(("group CONCAT", "node CONCAT")) for l in lines) and lines.count("node MATMUL") >= 2, lines
+
+
+def test_launch_plan_lays_out_a_view_that_only_a_swapped_product_reads(g, api):
+    """The gradient of a weight behind a SLICE of its product is
+    PERMUTE{1,0}(CONTRACT(PAD(gradient), x)) (tenncor/eteq/backprop.hpp:269-359,
+    402-421).  The PERMUTE is launched as the product with its operands
+    exchanged, the CONTRACT beneath it is looked through -- but that product
+    reads its operands from memory, so a PAD that nothing else reads is still
+    laid out in front of it (it used to be folded away like a view under an
+    elementwise node, and the recording failed for want of its data)."""
+    x = var(g, [15, 1, 5], np.float32, "x")
+    w = var(g, [32, 15], np.float32, "w")
+    gate = api.slice(api.contract(x, w), 8, 8, 0)
+    loss = api.reduce_sum(api.square(api.tanh(gate)))
+    (dw,) = g.derive(loss, [w])
+    lines = g.launch_plan([loss, dw])
+    assert "node PAD" in lines and "swapped CONTRACT+PERMUTE" in lines, lines
+    assert lines.index("node PAD") < lines.index("swapped CONTRACT+PERMUTE"), lines
 
 
 def test_launch_plan_reads_a_view_of_a_group_result_in_a_later_launch(g, api):
