@@ -647,8 +647,19 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense, int
 	return o.str();
 }
 
-int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out)
+int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out, const char* name = "fx")
 {
+	if (const char* dir = getenv("TCG_FX_DUMP"))
+	{
+		// the generated sources, for reading: <dir>/<kernel>_<hash of the text>.hip
+		char path[512];
+		snprintf(path, sizeof(path), "%s/%s_%016zx.hip", dir, name, std::hash<std::string>()(source));
+		if (FILE* f = fopen(path, "w"))
+		{
+			fwrite(source.data(), 1, source.size(), f);
+			fclose(f);
+		}
+	}
 	hiprtcProgram prog;
 	hiprtcResult rc = hiprtcCreateProgram(&prog, source.c_str(), "fused_group.hip", 0, nullptr, nullptr);
 	if (rc != HIPRTC_SUCCESS)
@@ -679,7 +690,7 @@ int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out)
 	hiprtcDestroyProgram(&prog);
 	hipModule_t module;
 	TCG_HIP(ctx, hipModuleLoadData(&module, code.data()));
-	TCG_HIP(ctx, hipModuleGetFunction(out, module, "fx"));
+	TCG_HIP(ctx, hipModuleGetFunction(out, module, name));
 	return TCG_OK;
 }
 
@@ -1379,13 +1390,11 @@ bool gfx_choose_tile (const tcg_ctx* ctx, uint64_t M, uint64_t J, int G, uint64_
 			const int accs = (tm / 16) * (nc / 16) * 4; // accumulator registers per lane
 			if (accs > 128) { continue; }
 			if ((size_t) nw * tm * nc * sizeof(float) > 65536) { continue; }
-			// one element (or one 16-byte vector of elements) of the group per lane
+			// a lane computes one element of the group, or 16-byte vectors of them when
+			// the tile holds more elements than the workgroup lanes; at most 8 per lane
 			int n = 1;
-			if (tm * tj > 64 * nw)
-			{
-				if (!vec || tj % 4 != 0 || tm * tj / 4 > 64 * nw) { continue; }
-				n = 4;
-			}
+			if (tm * tj > 64 * nw && vec && tj % 4 == 0) { n = 4; }
+			if (tm * tj / n > 8 * 64 * nw) { continue; }
 			const uint64_t groups = ((M + tm - 1) / tm) * (J / tj);
 			const double fill = groups >= (uint64_t) ctx->num_cus ? 1.0 : (double) groups / ctx->num_cus;
 			// operand elements fetched per result: 1 / rows + 1 / columns of the tile
@@ -1414,15 +1423,26 @@ struct GfxShape
 	int leaf_of[TCG_FX_MAX_LEAVES];   // product leaf g -> leaf of the group
 };
 
+// what a profile shows: the layout of B and the number of blocks of the result the group reads
+std::string gfx_name (const GfxShape& sh)
+{
+	return std::string("gemm_fx_") + (sh.trans_b ? "nt" : "nn") + "_" + std::to_string(sh.G);
+}
+
 std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, const bool* dense, const bool* supplied)
 {
 	const int NT = 64 * t.NW, RB = t.TM / 16, NC = sh.G * t.TJ, CB = NC / 16, CG = NC / 64;
 	const uint32_t ktot = sh.KT * sh.nterms, KW = ktot / t.NW, NSTEPS = KW / 16;
 	const int BL = sh.trans_b ? CB : 4 * CG; // 128-bit loads of B per step and lane
-	// steps on their way while one is multiplied: about sixteen loads per wave
-	int depth = 16 / (RB + BL) + 1;
-	if (depth < 2) { depth = 2; }
-	if (depth > 6) { depth = 6; }
+	// The source names the loads of a step one step ahead of its arithmetic and leaves
+	// the order to the compiler, which sinks each load to just before its first use;
+	// with two waves on a SIMD that is the fastest form measured for the steps of a
+	// recurrent cell.  Holding the loads two to five steps ahead with scheduling
+	// barriers made the 256 x 2048 x 768 step slower (10.4 -> 13.0 .. 16.0 us) and left
+	// the 256 x 512 x 2048 one where it was (12.2 us): with the arithmetic taken out the
+	// loads alone take 8.0 and 12.1 us, so what bounds these tiles is how fast the
+	// operands come out of L2, not how long a single load takes.
+	int depth = 2;
 	if ((uint32_t) depth > NSTEPS) { depth = (int) NSTEPS; }
 	const uint32_t tiles_m = (sh.M + t.TM - 1) / t.TM, tiles_j = sh.J / t.TJ;
 	const int items = t.TM * t.TJ / t.N;
@@ -1445,7 +1465,11 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 		<< t.TJ << "u) + (";
 	for (int g = 0; g + 1 < sh.G; ++g) { o << "g == " << g << "u ? " << sh.noff[g] << "u : "; }
 	o << sh.noff[sh.G - 1] << "u); }\n";
-	o << "extern \"C\" __global__ __launch_bounds__(" << NT << ") void fx (GfxArgs a)\n{\n"
+	// the steps on their way from memory wait in registers: the compiler may use the
+	// registers of a CU that holds at most two such workgroups, instead of keeping to
+	// the few that the largest number of resident waves would leave each of them
+	o << "extern \"C\" __global__ __launch_bounds__(" << NT << ") __attribute__((amdgpu_waves_per_eu(1, " << std::max(2, NT / 128)
+		<< "))) void " << gfx_name(sh) << " (GfxArgs a)\n{\n"
 		"__shared__ __attribute__((aligned(16))) float red[" << t.NW * t.TM * NC << "];\n"
 		"const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);\n"
 		"const uint32_t r16 = lane & 15u, q = lane >> 4;\n";
@@ -1458,16 +1482,23 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 	}
 	else { o << "const uint32_t tm = blockIdx.x % " << tiles_m << "u, tj = blockIdx.x / " << tiles_m << "u;\n"; }
 	o << "const uint32_t m0 = tm * " << t.TM << "u, j0 = tj * " << t.TJ << "u;\n";
-	// the element of the group this lane computes at the end, and its other operands
-	o << "const uint32_t er = tid / " << t.TJ / t.N << "u, ej = (tid % " << t.TJ / t.N << "u) * " << t.N << "u;\n"
-		"const bool item = tid < " << items << "u && m0 + er < " << sh.M << "u;\n"
-		"const uint32_t idx = item ? ((m0 + er) * " << sh.J << "u + j0 + ej) / " << t.N << "u : 0u;\n";
+	// the elements of the group this lane computes at the end (lane, lane + NT, ...),
+	// and their other operands, loaded before the product starts
+	const int per_lane = (items + NT - 1) / NT;
 	FxBake bake;
 	for (uint32_t k = 0; k < p.nleaf; ++k) { bake.leaf_ptr[k] = "a.leaf[" + std::to_string(k) + "]"; }
 	for (uint32_t k = 0; k < p.nout; ++k) { bake.out_ptr[k] = "a.out[" + std::to_string(k) + "]"; }
-	FxParts parts;
-	fx_emit_parts(parts, t.N, p, dense, &bake, "", "idx", false, supplied);
-	o << parts.load.str();
+	std::vector<FxParts> parts((size_t) per_lane);
+	for (int it = 0; it < per_lane; ++it)
+	{
+		const std::string x = "_" + std::to_string(it);
+		o << "const uint32_t et" << x << " = tid + " << it * NT << "u;\n"
+			"const uint32_t er" << x << " = et" << x << " / " << t.TJ / t.N << "u, ej" << x << " = (et" << x << " % " << t.TJ / t.N << "u) * " << t.N << "u;\n"
+			"const bool item" << x << " = et" << x << " < " << items << "u && m0 + er" << x << " < " << sh.M << "u;\n"
+			"const uint32_t idx" << x << " = item" << x << " ? ((m0 + er" << x << ") * " << sh.J << "u + j0 + ej" << x << ") / " << t.N << "u : 0u;\n";
+		fx_emit_parts(parts[(size_t) it], t.N, p, dense, &bake, x, "idx" + x, false, supplied);
+		o << parts[(size_t) it].load.str();
+	}
 	// ---- the product ----
 	o << "uint32_t arow[" << RB << "];\n";
 	for (int rb = 0; rb < RB; ++rb)
@@ -1594,20 +1625,26 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 			}
 		}
 	}
-	o << "}\n__syncthreads();\nif (!item) { return; }\n";
-	for (int g = 0; g < sh.G; ++g)
+	o << "}\n__syncthreads();\n";
+	for (int it = 0; it < per_lane; ++it)
 	{
-		const int k = sh.leaf_of[g];
-		o << "T l" << k << "[" << t.N << "];\n{\nconst float* at = red + er * " << NC << "u + " << g * t.TJ << "u + ej;\n";
-		for (int e = 0; e < t.N; ++e)
+		const std::string x = "_" + std::to_string(it);
+		o << "if (item" << x << ")\n{\n";
+		for (int g = 0; g < sh.G; ++g)
 		{
-			o << "{ float s = at[" << e << "];";
-			for (int w = 1; w < t.NW; ++w) { o << " s += at[" << w * t.TM * NC + e << "];"; }
-			o << " l" << k << "[" << e << "] = s; }\n";
+			const int k = sh.leaf_of[g];
+			o << "T l" << k << x << "[" << t.N << "];\n{\nconst float* at = red + er" << x << " * " << NC << "u + " << g * t.TJ << "u + ej" << x << ";\n";
+			for (int e = 0; e < t.N; ++e)
+			{
+				o << "{ float s = at[" << e << "];";
+				for (int w = 1; w < t.NW; ++w) { o << " s += at[" << w * t.TM * NC + e << "];"; }
+				o << " l" << k << x << "[" << e << "] = s; }\n";
+			}
+			o << "}\n";
 		}
-		o << "}\n";
+		o << parts[(size_t) it].compute.str() << parts[(size_t) it].store.str() << "}\n";
 	}
-	o << parts.compute.str() << parts.store.str() << "}\n";
+	o << "}\n";
 	return o.str();
 }
 
@@ -1719,7 +1756,7 @@ extern "C" int tcg_gemm_terms_fx (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t 
 		auto it = jit.kernels.find(source);
 		if (it == jit.kernels.end())
 		{
-			rc = fx_compile(ctx, source, &fn);
+			rc = fx_compile(ctx, source, &fn, gfx_name(sh).c_str());
 			if (rc != TCG_OK) { return rc; }
 			jit.kernels.emplace(source, fn);
 		}
