@@ -344,11 +344,13 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
             ts.append(time.perf_counter() - t0)
         return float(np.median(ts))
 
-    kinds = (("plain", ""), ("replay", "_replay")) if evaluator is None else ((evaluator, ""),)
+    # no suffix: the evaluator a context gets when nothing was registered (teq::get_eval's
+    # default: the one that records a target set's launches on its second pass and enqueues
+    # the recording afterwards); "_walk": teq::Evaluator, the node-by-node walk
+    kinds = (("default", ""), ("plain", "_walk")) if evaluator is None else ((evaluator, ""),)
     for kind, tag in kinds:
-        # "replay": the evaluator that records a target set's launches on its
-        # second pass and enqueues the recording afterwards
         tg.set_evaluator(kind)
+        replays = kind != "plain"
         if only is not None:
             # one configuration under one evaluator (the form profiles are taken in)
             g = tg.Graph()
@@ -374,7 +376,7 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
                    "functors": g.count_functors(targets), "evaluator_stats": tg.evaluator_stats()}
             if cleanup is not None:
                 out["optimize"] = cleanup
-            tg.set_evaluator("plain")
+            tg.set_evaluator("default")
             return out
         g = tg.Graph()
         targets, x, _ = configs.config1_mlp(g)
@@ -382,16 +384,16 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
         out["config1_mlp%s_evals_per_sec" % tag] = round(1.0 / t, 1)
         out["config1_mlp%s_us_per_eval" % tag] = round(t * 1e6, 1)
         out["config1_mlp_functors"] = g.count_functors(targets)
-        if kind == "replay":
-            out["config1_mlp_replay_launches_per_eval"] = tg.evaluator_stats()["launches"]
+        if replays:
+            out["config1_mlp_launches_per_eval"] = tg.evaluator_stats()["launches"]
         g.close()
-        if kind == "replay":
+        if replays:
             # the same recording kept launch by launch (bit-identical to the walk)
             tg.set_evaluator("replay_launches")
             g = tg.Graph()
             targets, x, _ = configs.config1_mlp(g)
             t = timed(g, targets, x, lambda: rng.uniform(-1, 1, 30).astype(np.float32), 300)
-            out["config1_mlp_replay_launch_by_launch_us_per_eval"] = round(t * 1e6, 1)
+            out["config1_mlp_launch_by_launch_us_per_eval"] = round(t * 1e6, 1)
             g.close()
             tg.set_evaluator(kind)
 
@@ -399,23 +401,26 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
         targets, x, _, flops = configs.config4_lstm(g)
         xs = rng.uniform(-1, 1, 256 * 64 * 256).astype(np.float32)
         # medians over enough passes for the clocks to settle (a recorded pass takes 4 ms, a walked one 14)
-        t = timed(g, targets, x, lambda: xs, 40 if kind == "replay" else 10)
+        t = timed(g, targets, x, lambda: xs, 40 if replays else 10)
         out["config4_lstm%s_ms_per_step" % tag] = round(t * 1e3, 3)
         out["config4_lstm%s_gemm_TFLOPs" % tag] = round(flops / t / 1e12, 2)
         out["config4_lstm_functors"] = g.count_functors(targets)
+        if replays:
+            out["config4_lstm_launches"] = tg.evaluator_stats()["launches"]
         g.close()
 
         g = tg.Graph()
         targets, x, _, flops = configs.config5_cnn(g)
         xs = rng.uniform(0, 1, 128 * 28 * 28).astype(np.float32)
-        t = timed(g, targets, x, lambda: xs, 60 if kind == "replay" else 20)
+        t = timed(g, targets, x, lambda: xs, 60 if replays else 20)
         out["config5_cnn%s_ms_per_step" % tag] = round(t * 1e3, 3)
         out["config5_cnn%s_useful_TFLOPs" % tag] = round(flops / t / 1e12, 3)
         out["config5_cnn_functors"] = g.count_functors(targets)
-        if kind == "replay":
-            out["config5_cnn_replay_launches"] = tg.evaluator_stats()["launches"]
+        if replays:
+            out["config5_cnn_launches"] = tg.evaluator_stats()["launches"]
         g.close()
-    tg.set_evaluator("plain")
+    tg.set_evaluator("default")
+    out["default_evaluator"] = "replay (teq::get_eval registers eigen::ReplayEvaluator; TCR_EVAL_PLAIN=1 keeps the walk)"
     return out
 
 
@@ -536,7 +541,7 @@ def main():
     ap.add_argument("--no-graphs", action="store_true", help="skip the whole-graph side metrics (configs 1, 4, 5)")
     ap.add_argument("--graph-config", type=int, choices=[1, 4, 5], default=None,
                     help="time only this whole-graph configuration and print its line (for profiling)")
-    ap.add_argument("--evaluator", choices=["plain", "replay", "replay_launches", "replay_unfused"], default="replay")
+    ap.add_argument("--evaluator", choices=["default", "plain", "replay", "replay_launches", "replay_unfused"], default="replay")
     ap.add_argument("--f64", action="store_true", help="with --matmul-only: the 4096^3 product in double")
     ap.add_argument("--reps", type=int, default=None,
                     help="timed evaluations with --graph-config 4 or 5 (default 20), timed launches with --matmul-only (100)")

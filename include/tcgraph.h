@@ -71,7 +71,14 @@ int tcr_evaluate_ignoring (tcr_graph* g, int ntargets, const int* targets, int n
 int tcr_sync (tcr_graph* g);
 
 /* teq::set_eval (internal/teq/src/evaluator.cpp:9-20): which evaluator the
- * process uses from now on. TCR_EVAL_PLAIN is teq::Evaluator, the node-by-node
+ * process uses from now on. TCR_EVAL_DEFAULT removes the registered one, so
+ * that teq::get_eval makes its default again: TCR_EVAL_REPLAY, or
+ * TCR_EVAL_PLAIN when the environment holds TCR_EVAL_PLAIN=1 (the reference's
+ * default is the plain walk; a backend that is dropped in without a call to
+ * teq::set_eval should not be the slow one for graphs evaluated again and
+ * again, and the replaying evaluator walks a set of targets it sees for the
+ * first time exactly like the plain one).
+ * TCR_EVAL_PLAIN is teq::Evaluator, the node-by-node
  * walk; TCR_EVAL_REPLAY records the launches of a set of targets the second
  * time it is evaluated and enqueues the recording as a whole afterwards, with
  * elementwise functors that feed one another computed in shared launches, and
@@ -86,6 +93,7 @@ int tcr_sync (tcr_graph* g);
 #define TCR_EVAL_REPLAY 1
 #define TCR_EVAL_REPLAY_UNFUSED 2
 #define TCR_EVAL_REPLAY_LAUNCHES 3
+#define TCR_EVAL_DEFAULT 4
 int tcr_set_evaluator (int kind);
 /* Counters of the replaying evaluator (zeros under TCR_EVAL_PLAIN):
  * out[0] passes walked node by node, out[1] recordings made, out[2] passes

@@ -36,7 +36,7 @@ EXPORTS = [
     "tcr_set_random", "tcr_seed",
 ]
 
-EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED, EVAL_REPLAY_LAUNCHES = 0, 1, 2, 3
+EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED, EVAL_REPLAY_LAUNCHES, EVAL_DEFAULT = 0, 1, 2, 3, 4
 
 # conversions shipped with the package (the reference's cfg/optimizations.json
 # is a git-lfs pointer without content)
@@ -100,7 +100,8 @@ def load():
 
 
 def set_evaluator(kind):
-    """teq::set_eval: "plain" (node-by-node walk, the default), "replay"
+    """teq::set_eval: "default" (no evaluator registered: teq::get_eval then
+    makes "replay", or "plain" under TCR_EVAL_PLAIN=1), "plain" (node-by-node walk), "replay"
     (record a target set's launches on its second evaluation, with elementwise
     functors sharing launches and the pass of a graph of small tensors as one
     kernel, and enqueue the recording afterwards), "replay_launches" (the same
@@ -109,7 +110,7 @@ def set_evaluator(kind):
     reference's evaluator slot."""
     lib = load()
     code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY, "replay_unfused": EVAL_REPLAY_UNFUSED,
-            "replay_launches": EVAL_REPLAY_LAUNCHES}[kind]
+            "replay_launches": EVAL_REPLAY_LAUNCHES, "default": EVAL_DEFAULT}[kind]
     if lib.tcr_set_evaluator(code) != 0:
         raise GraphError(lib.tcr_last_error().decode())
 

@@ -247,6 +247,7 @@ int tcr_set_evaluator (int kind)
 			case TCR_EVAL_REPLAY: teq::set_eval(new eigen::ReplayEvaluator()); break;
 			case TCR_EVAL_REPLAY_UNFUSED: teq::set_eval(new eigen::ReplayEvaluator(1, 16, false)); break;
 			case TCR_EVAL_REPLAY_LAUNCHES: teq::set_eval(new eigen::ReplayEvaluator(1, 16, true, false)); break;
+			case TCR_EVAL_DEFAULT: teq::set_eval(nullptr); break;
 			default: global::fatalf("unknown evaluator kind %d", kind);
 		}
 	});

@@ -33,6 +33,18 @@ private:
 
 }
 
+namespace
+{
+
+// a context without an evaluator of its own gets this one (teq::get_eval)
+[[maybe_unused]] const bool default_registered = []
+{
+	teq::set_default_eval_factory([]() -> teq::iEvaluator* { return new ReplayEvaluator(); });
+	return true;
+}();
+
+}
+
 struct ReplayEvaluator::Plan final
 {
 	std::vector<Observable*> funcs;
@@ -157,7 +169,11 @@ static bool walk_skips_an_assign (const std::vector<Observable*>& funcs, size_t 
 void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targets, const teq::TensSetT& ignored)
 {
 	auto gpu = dynamic_cast<Device*>(&device);
-	if (nullptr == gpu || false == ignored.empty() || targets.empty())
+	// a caller's own runtime memory is asked for every buffer of every pass
+	// (internal/eigen/memory.hpp:14-22); the buffers of a recording stay with the
+	// recording, so such a device is walked
+	if (nullptr == gpu || false == ignored.empty() || targets.empty() ||
+		nullptr == std::dynamic_pointer_cast<RuntimeMemory>(gpu->memory()))
 	{
 		plain(device, targets, ignored);
 		return;

@@ -89,13 +89,26 @@ void set_eval (iEvaluator* eval, global::CfgMapptrT ctx)
 	}
 }
 
+static EvalFactoryT& default_eval_factory (void)
+{
+	static EvalFactoryT factory = nullptr;
+	return factory;
+}
+
+void set_default_eval_factory (EvalFactoryT factory)
+{
+	default_eval_factory() = factory;
+}
+
 iEvaluator& get_eval (const global::CfgMapptrT& ctx)
 {
 	if (nullptr == ctx) { global::fatal("cannot look an evaluator up in a null context"); }
 	auto eval = static_cast<iEvaluator*>(ctx->get_obj(eval_key));
 	if (nullptr == eval)
 	{
-		eval = new Evaluator();
+		const char* plain = getenv("TCR_EVAL_PLAIN");
+		EvalFactoryT factory = default_eval_factory();
+		eval = (nullptr != factory && false == (plain && plain[0] == '1')) ? factory() : new Evaluator();
 		set_eval(eval, ctx);
 	}
 	return *eval;

@@ -347,9 +347,16 @@ struct Evaluator final : public iEvaluator
 
 /// The evaluator registered in `ctx` under "evaluater"
 /// (internal/teq/evaluator.hpp:65-67, src/evaluator.cpp:9-30); the context
-/// owns the pointer.  Defaults to teq::Evaluator.
+/// owns the pointer.  A context without one gets what the default factory
+/// makes: teq::Evaluator in the reference, and here too until a layer above
+/// names another (the GPU layer names its replaying evaluator, which walks a
+/// set of targets like teq::Evaluator the first time it sees it and records
+/// its launches the second time; TCR_EVAL_PLAIN=1 in the environment keeps
+/// the plain walk).
 void set_eval (iEvaluator* eval, global::CfgMapptrT ctx = global::context());
 iEvaluator& get_eval (const global::CfgMapptrT& ctx = global::context());
+using EvalFactoryT = iEvaluator* (*) (void);
+void set_default_eval_factory (EvalFactoryT factory);
 
 // ---- derivation (internal/teq/derive.hpp, src/derive.cpp) ------------------
 

@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "eteq.hpp"
+#include "replay_eval.hpp"
 
 static int failures = 0;
 
@@ -261,8 +262,10 @@ static void context_registries (void)
 
 	// replacing and removing: the default comes back (src/evaluator.cpp:21-30,
 	// src/memory.cpp:19-28)
+	// (the default evaluator is the replaying one, which walks like teq::Evaluator
+	// whatever it sees for the first time)
 	teq::set_eval(nullptr, ctx);
-	EXPECT(nullptr != dynamic_cast<teq::Evaluator*>(&teq::get_eval(ctx)));
+	EXPECT(nullptr != dynamic_cast<eigen::ReplayEvaluator*>(&teq::get_eval(ctx)));
 	eigen::set_runtime(nullptr, ctx);
 	EXPECT(nullptr != std::dynamic_pointer_cast<eigen::RuntimeMemory>(eigen::get_runtime(ctx)));
 	EXPECT(memory != eigen::get_runtime(ctx));

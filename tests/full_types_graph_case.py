@@ -119,7 +119,7 @@ def evaluate_on_gpu():
         assert got.dtype == np.int16 and got.min() >= -7 and got.max() <= 9 and len(np.unique(got)) == 17
         g.close()
         print("%s mixed ok" % evaluator, flush=True)
-    graph.set_evaluator("plain")
+    graph.set_evaluator("default")
 
 
 def random_graphs_on_gpu():

@@ -27,7 +27,7 @@ def env(request):
         yield g, graph.Api(g), graph
     finally:
         g.close()
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 def lines_of(text, shapes=True):

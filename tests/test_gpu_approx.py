@@ -38,7 +38,7 @@ def env(request):
         yield g, api, graph.Approx(api)
     finally:
         g.close()
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 def assert_rel(got, expected, rtol):

@@ -28,7 +28,7 @@ def plain_evaluator_afterwards():
     closed: a test that installs another evaluator leaves the default behind."""
     yield
     from tenncor_amd import graph
-    graph.set_evaluator("plain")
+    graph.set_evaluator("default")
 
 
 @pytest.fixture()
@@ -540,4 +540,4 @@ def test_optimiser_steps_stay_on_the_device(rule, kw, evaluator):
             assert graph.evaluator_stats()["replayed"] >= 3
     finally:
         g.close()
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")

@@ -150,7 +150,7 @@ def test_configuration_graphs_keep_their_values(config, evaluator):
             scale = np.abs(raw).max() + 1e-30
             assert np.abs(raw - cleaned).max() <= 1e-5 * scale
     finally:
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 # ---- the reference's expected optimised graphs --------------------------------

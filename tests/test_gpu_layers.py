@@ -37,7 +37,7 @@ def env(request):
         yield g, graph.Api(g)
     finally:
         g.close()
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 def close_to(got, expected, what):

@@ -1161,7 +1161,7 @@ def test_full_size_recordings_equal_the_walk(config):
                 assert st["recorded"] == 1 and st["launches"] < 0.4 * g.count_functors(targets) + 40
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     for k, (a, b) in enumerate(zip(results["plain"], results["replay_launches"])):
         assert np.isfinite(a).all()
         if config == "lstm":

@@ -122,7 +122,7 @@ def replay_graph():
         yield g, graph.Api(g), graph
     finally:
         g.close()
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 def mlp(g, api, fx, np_dtype):
@@ -202,7 +202,7 @@ def test_replayed_training_loop_updates_leaves_in_place(replay_graph):
         seen.append(w.get().copy())
     st = graph.evaluator_stats()
     assert st["replayed"] >= 4
-    graph.set_evaluator("plain")
+    graph.set_evaluator("default")
     g2 = graph.Graph()
     w2, x2, loss2, step2 = build(g2, graph.Api(g2))
     for i, xv in enumerate(xs):
@@ -243,7 +243,7 @@ def test_replay_mixes_with_other_target_sets_and_aliases(replay_graph):
             g.evaluate([conv])
             mid = conv.get().copy()
     assert graph.evaluator_stats()["replayed"] >= 3
-    graph.set_evaluator("plain")
+    graph.set_evaluator("default")
     g2 = graph.Graph()
     api2 = graph.Api(g2)
     x2 = g2.variable(xv, [C, W, H, B], "x")
@@ -287,7 +287,7 @@ def test_recordings_are_dropped_when_nodes_go_away():
             np.testing.assert_array_equal(y.get(), (np.arange(6, dtype=np.float32) + i) ** 2)
         g.close()
     finally:
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 # ---- shared launches ---------------------------------------------------------
@@ -311,7 +311,7 @@ def run_both(build, feeds, kinds=("plain", "replay_launches", "replay_unfused"))
             stats[kind] = graph.evaluator_stats()
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     return results, stats
 
 
@@ -629,7 +629,7 @@ def test_a_recording_with_a_plain_assign_runs_at_every_pass():
                 assert st["replayed"] >= 3 and st["skipped"] == 0, st
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     assert len(set(seen["plain"])) == 5          # the state moves
     x = s0.reshape(8, 32).astype(np.float64)
     for k in range(5):
@@ -772,7 +772,7 @@ def test_two_assignments_to_one_variable_stay_with_the_walk():
                 assert st["recorded"] == 0 and st["plain"] == 4, st
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     for kind in ("replay_launches", "replay"):
         for (a, va), (b, vb) in zip(seen[kind], seen["plain"]):
             assert a == b
@@ -1075,7 +1075,7 @@ def test_rand_unif_on_the_device_under_both_evaluators(evaluator):
         g.close()
     finally:
         graph.set_random("host")
-        graph.set_evaluator("plain")
+        graph.set_evaluator("default")
 
 
 # ---- a whole pass recorded as one kernel ---------------------------------------
@@ -1198,7 +1198,7 @@ def test_small_graph_pass_is_one_launch_and_matches_golden_and_walk():
                 assert st["plain"] == 1 and st["recorded"] == 1 and st["replayed"] == 3 and st["launches"] == 1
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     for key, val in zip(("expect_gw0", "expect_gb0", "expect_gw1", "expect_gb1"), rows["replay"][3][1:]):
         np.testing.assert_allclose(val, np.array(fx[key]), rtol=1e-12)
     for got, ref in zip(rows["replay"], rows["plain"]):
@@ -1242,7 +1242,7 @@ def test_small_graph_passes_follow_the_walk(config):
                 assert st["recorded"] == 1 and st["replayed"] == len(feeds) - 1 and st["launches"] == 1
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     for got, ref in zip(rows["replay"], rows["plain"]):
         for a, b in zip(got, ref):
             close_to(a, b, 1e-5)
@@ -1274,7 +1274,7 @@ def test_graphs_with_steps_one_kernel_cannot_take_are_recorded_launch_by_launch(
                 assert st["recorded"] == 1 and st["replayed"] == 3 and st["launches"] > 1
         finally:
             g.close()
-            graph.set_evaluator("plain")
+            graph.set_evaluator("default")
     for a, b in zip(rows["replay"], rows["plain"]):
         np.testing.assert_array_equal(a, b)
 
