@@ -384,7 +384,15 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
         out["config1_mlp%s_evals_per_sec" % tag] = round(1.0 / t, 1)
         out["config1_mlp%s_us_per_eval" % tag] = round(t * 1e6, 1)
         out["config1_mlp_functors"] = g.count_functors(targets)
+        def recording_cost(name):
+            # what the first passes cost and no timed pass shows: planning, kernels compiled
+            # at run time (or loaded from the files an earlier process left), the capture
+            st = tg.evaluator_stats()
+            out[name + "_record_ms"] = st["record_ms"]
+            out[name + "_record_jit"] = {"ms": st["jit_ms"], "compiled": st["jit_compiled"], "from_disk": st["jit_from_disk"]}
+
         if replays:
+            recording_cost("config1_mlp")
             out["config1_mlp_launches_per_eval"] = tg.evaluator_stats()["launches"]
         g.close()
         if replays:
@@ -406,6 +414,7 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
         out["config4_lstm%s_gemm_TFLOPs" % tag] = round(flops / t / 1e12, 2)
         out["config4_lstm_functors"] = g.count_functors(targets)
         if replays:
+            recording_cost("config4_lstm")
             out["config4_lstm_launches"] = tg.evaluator_stats()["launches"]
         g.close()
 
@@ -417,6 +426,7 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
         out["config5_cnn%s_useful_TFLOPs" % tag] = round(flops / t / 1e12, 3)
         out["config5_cnn_functors"] = g.count_functors(targets)
         if replays:
+            recording_cost("config5_cnn")
             out["config5_cnn_launches"] = tg.evaluator_stats()["launches"]
         g.close()
     tg.set_evaluator("default")

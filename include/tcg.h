@@ -312,6 +312,16 @@ int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 	int nleaves, const tcg_fx_leaf* leaves, int ninstrs, const tcg_fx_instr* program,
 	int nouts, void* const* outs);
 
+/* What the kernels compiled at run time have cost this process so far (groups
+ * of elementwise nodes, whole passes of small graphs, products with an
+ * epilogue; no counterpart in the reference, whose expressions are compiled
+ * with it): kernels compiled here, kernels loaded from the files an earlier
+ * process left, and the milliseconds spent on both.  Compiled code is kept
+ * under $TCG_FX_CACHE (default ~/.cache/tenncor_amd/fx; TCG_FX_CACHE=0: nowhere),
+ * one file per kernel holding the text it was compiled from in front of the
+ * code, and is only used for exactly that text, those flags and that compiler. */
+int tcg_jit_stats (const tcg_ctx* ctx, uint64_t* compiled, uint64_t* from_disk, double* ms);
+
 /* ---- reductions ------------------------------------------------------- */
 
 /* REDUCE_SUM / REDUCE_PROD / REDUCE_MIN / REDUCE_MAX

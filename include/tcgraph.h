@@ -100,6 +100,11 @@ int tcr_set_evaluator (int kind);
  * served by a recording, out[3] passes with nothing to do, out[4] launches in
  * the latest recording, out[5] device bytes reserved by live recordings */
 int tcr_evaluator_stats (uint64_t out[6]);
+/* What the most recent recording cost on the host: milliseconds from planning
+ * to the finished launch sequence, the part of them spent on kernels compiled
+ * at run time, how many of those were compiled and how many came from the
+ * files an earlier process left (tcg_jit_stats).  Zeros without a recording. */
+int tcr_evaluator_record_cost (double* record_ms, double* jit_ms, uint64_t* jit_compiled, uint64_t* jit_from_disk);
 /* How many target sets the replaying evaluator could not record (it walks
  * them node by node instead) and, in `out`, the message of the failure that
  * stopped the latest of them ("" when none, or under TCR_EVAL_PLAIN) */

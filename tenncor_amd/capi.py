@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_jit_stats", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -138,6 +138,7 @@ def load():
         "tcg_gemm_terms_grid": [vp, i32, i32, u64p, i32, u64p, u64, i32, vpp, u64p, i32, vpp, u64p, i32, vp, u64],
         "tcg_gemm_terms_fx": [vp, i32, u64, u64, u64, i32, vpp, u64p, i32, vpp, u64p, i32,
                               u64p, i32, ctypes.POINTER(FxLeaf), i32, ctypes.POINTER(FxInstr), i32, vpp],
+        "tcg_jit_stats": [vp, u64p, u64p, ctypes.POINTER(ctypes.c_double)],
         "tcg_conv": [vp, i32, u64p, u64p, i32, u64p, vp, vp, vp],
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
@@ -515,6 +516,13 @@ class Context:
                                             len(r), _u64(r if r else [0]), _u64(img_box[0]), _u64(img_box[1]),
                                             olo, ohi, box, i64(box_stride), kernel, i64(kernel_stride),
                                             dst, i64(out_stride)))
+
+    def jit_stats(self):
+        """Kernels compiled at run time by this process, kernels loaded from the
+        disk cache instead, and the milliseconds both took."""
+        compiled, from_disk, ms = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_double()
+        self._check(self.lib.tcg_jit_stats(self.handle, ctypes.byref(compiled), ctypes.byref(from_disk), ctypes.byref(ms)))
+        return {"compiled": compiled.value, "from_disk": from_disk.value, "ms": ms.value}
 
     # ---- recorded launch sequences ----
     def capture_begin(self, small=False):

@@ -14,6 +14,10 @@
 
 #include <hip/hiprtc.h>
 
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <chrono>
 #include <cstdlib>
 #include <map>
 #include <mutex>
@@ -336,6 +340,10 @@ struct FxJit
 {
 	std::mutex mu;
 	std::unordered_map<std::string,hipFunction_t> kernels;
+	// what the kernels of this process cost (under `mu`): compiled here, loaded
+	// from the files an earlier process left, milliseconds spent on either
+	uint64_t compiled = 0, from_disk = 0;
+	double ms = 0.0;
 };
 
 FxJit& fx_jit (void)
@@ -647,6 +655,78 @@ std::string fx_source (int dtype, int N, const FxArgs& p, const bool* dense, int
 	return o.str();
 }
 
+// Compiled kernels are kept on disk between processes: a graph of a few thousand
+// nodes needs a handful of kernels of 0.1-0.5 s each, which its first recording
+// would otherwise pay again in every process.  One file per kernel under
+// $TCG_FX_CACHE, else $XDG_CACHE_HOME/tenncor_amd/fx, else ~/.cache/tenncor_amd/fx
+// (TCG_FX_CACHE=0: none), named by a hash of what identifies the code -- compiler
+// version, kernel name, flags, source text -- and holding that text in full in
+// front of the code object, so that a file is only ever used for the text it
+// was compiled from.  Written under another name and moved into place.
+std::string fx_cache_dir (void)
+{
+	const char* env = getenv("TCG_FX_CACHE");
+	if (env && env[0] == '0' && env[1] == '\0') { return ""; }
+	std::string dir;
+	if (env && env[0]) { dir = env; }
+	else if (const char* xdg = getenv("XDG_CACHE_HOME")) { dir = std::string(xdg) + "/tenncor_amd/fx"; }
+	else if (const char* home = getenv("HOME")) { dir = std::string(home) + "/.cache/tenncor_amd/fx"; }
+	else { return ""; }
+	// every level, ignoring the ones that exist; a directory that cannot be made
+	// shows when the file cannot be written, and nothing is cached then
+	for (size_t at = 1; at <= dir.size(); ++at)
+	{
+		if (at == dir.size() || dir[at] == '/') { mkdir(dir.substr(0, at).c_str(), 0700); }
+	}
+	return dir;
+}
+
+std::string fx_cache_path (const std::string& identity)
+{
+	static const std::string dir = fx_cache_dir();
+	if (dir.empty()) { return ""; }
+	uint64_t h1 = 1469598103934665603ull, h2 = 0x9e3779b97f4a7c15ull; // two 64-bit hashes of the text
+	for (unsigned char c : identity)
+	{
+		h1 = (h1 ^ c) * 1099511628211ull;
+		h2 = (h2 + c) * 0xff51afd7ed558ccdull;
+		h2 ^= h2 >> 29;
+	}
+	char name[64];
+	snprintf(name, sizeof(name), "/%016llx%016llx.co", (unsigned long long) h1, (unsigned long long) h2);
+	return dir + name;
+}
+
+bool fx_cache_read (const std::string& path, const std::string& identity, std::vector<char>& code)
+{
+	if (path.empty()) { return false; }
+	FILE* f = fopen(path.c_str(), "rb");
+	if (nullptr == f) { return false; }
+	bool ok = false;
+	uint64_t lens[2] = {0, 0};
+	if (1 == fread(lens, sizeof(lens), 1, f) && lens[0] == identity.size() && lens[1] > 0 && lens[1] < (1ull << 30))
+	{
+		std::string text(lens[0], '\0');
+		code.assign(lens[1], '\0');
+		ok = (lens[0] == 0 || 1 == fread(&text[0], lens[0], 1, f)) && text == identity && 1 == fread(code.data(), lens[1], 1, f);
+	}
+	fclose(f);
+	return ok;
+}
+
+void fx_cache_write (const std::string& path, const std::string& identity, const std::vector<char>& code)
+{
+	if (path.empty() || code.empty()) { return; }
+	const std::string tmp = path + "." + std::to_string((long) getpid()) + ".tmp";
+	FILE* f = fopen(tmp.c_str(), "wb");
+	if (nullptr == f) { return; }
+	uint64_t lens[2] = {identity.size(), code.size()};
+	bool ok = 1 == fwrite(lens, sizeof(lens), 1, f) && 1 == fwrite(identity.data(), identity.size(), 1, f) &&
+		1 == fwrite(code.data(), code.size(), 1, f);
+	ok = 0 == fclose(f) && ok;
+	if (false == ok || 0 != rename(tmp.c_str(), path.c_str())) { remove(tmp.c_str()); }
+}
+
 int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out, const char* name = "fx")
 {
 	if (const char* dir = getenv("TCG_FX_DUMP"))
@@ -660,18 +740,46 @@ int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out, con
 			fclose(f);
 		}
 	}
-	hiprtcProgram prog;
-	hiprtcResult rc = hiprtcCreateProgram(&prog, source.c_str(), "fused_group.hip", 0, nullptr, nullptr);
-	if (rc != HIPRTC_SUCCESS)
-	{
-		return tcg_fail(ctx, TCG_ERR_HIP, "tcg_ew_fusedx: hiprtcCreateProgram: %s", hiprtcGetErrorString(rc));
-	}
 	std::string arch = "--offload-arch=" + ctx->arch;
 	// the flags libtcg itself is built with (packed fp32 forms stay off), and
 	// no contraction: a multiply node feeding an add node must round twice, as
 	// it does when the two nodes run as separate kernels
 	const char* opts[] = {arch.c_str(), "-O3", "-std=c++17", "-ffp-contract=off",
 		"-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+	const auto begun = std::chrono::steady_clock::now();
+	FxJit& jit = fx_jit();
+	auto spent = [&]
+	{
+		jit.ms += std::chrono::duration<double,std::milli>(std::chrono::steady_clock::now() - begun).count();
+	};
+	// code compiled by an earlier process for this text, these flags and this compiler
+	std::string identity = "tcg-fx-1\n";
+	{
+		int major = 0, minor = 0;
+		hiprtcVersion(&major, &minor);
+		identity += std::to_string(major) + "." + std::to_string(minor) + "\n" + name + "\n";
+		for (const char* opt : opts) { identity += std::string(opt) + " "; }
+		identity += "\n" + source;
+	}
+	const std::string cached = fx_cache_path(identity);
+	std::vector<char> code;
+	if (fx_cache_read(cached, identity, code))
+	{
+		hipModule_t module;
+		if (hipSuccess == hipModuleLoadData(&module, code.data()) && hipSuccess == hipModuleGetFunction(out, module, name))
+		{
+			++jit.from_disk;
+			spent();
+			return TCG_OK;
+		}
+		(void) hipGetLastError(); // a file that does not load is compiled over
+	}
+	hiprtcProgram prog;
+	hiprtcResult rc = hiprtcCreateProgram(&prog, source.c_str(), "fused_group.hip", 0, nullptr, nullptr);
+	if (rc != HIPRTC_SUCCESS)
+	{
+		return tcg_fail(ctx, TCG_ERR_HIP, "tcg_ew_fusedx: hiprtcCreateProgram: %s", hiprtcGetErrorString(rc));
+	}
 	rc = hiprtcCompileProgram(prog, (int) (sizeof(opts) / sizeof(opts[0])), opts);
 	if (rc != HIPRTC_SUCCESS)
 	{
@@ -685,12 +793,15 @@ int fx_compile (tcg_ctx* ctx, const std::string& source, hipFunction_t* out, con
 	}
 	size_t size = 0;
 	hiprtcGetCodeSize(prog, &size);
-	std::vector<char> code(size);
+	code.assign(size, '\0');
 	hiprtcGetCode(prog, code.data());
 	hiprtcDestroyProgram(&prog);
 	hipModule_t module;
 	TCG_HIP(ctx, hipModuleLoadData(&module, code.data()));
 	TCG_HIP(ctx, hipModuleGetFunction(out, module, name));
+	fx_cache_write(cached, identity, code);
+	++jit.compiled;
+	spent();
 	return TCG_OK;
 }
 
@@ -1766,5 +1877,16 @@ extern "C" int tcg_gemm_terms_fx (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t 
 	size_t size = packed.size();
 	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, packed.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
 	TCG_HIP(ctx, hipModuleLaunchKernel(fn, grid, 1, 1, 64 * tile.NW, 1, 1, 0, ctx->stream, nullptr, config));
+	return TCG_OK;
+}
+
+extern "C" int tcg_jit_stats (const tcg_ctx* ctx, uint64_t* compiled, uint64_t* from_disk, double* ms)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	FxJit& jit = fx_jit();
+	std::lock_guard<std::mutex> lock(jit.mu);
+	if (compiled) { *compiled = jit.compiled; }
+	if (from_disk) { *from_disk = jit.from_disk; }
+	if (ms) { *ms = jit.ms; }
 	return TCG_OK;
 }

@@ -32,7 +32,7 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_evaluate_ignoring", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
-    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_launch_plan", "tcr_optimize",
+    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_evaluator_record_cost", "tcr_launch_plan", "tcr_optimize",
     "tcr_set_random", "tcr_seed",
 ]
 
@@ -84,6 +84,7 @@ def load():
         "tcr_set_evaluator": [i32],
         "tcr_evaluator_stats": [u64p],
         "tcr_evaluator_record_error": [ctypes.c_char_p, ctypes.c_size_t, u64p],
+        "tcr_evaluator_record_cost": [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), u64p, u64p],
         "tcr_launch_plan": [vp, i32, i32p, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
         "tcr_optimize": [vp, i32, i32p, ctypes.c_char_p, i32, i32p, u64p],
         "tcr_set_random": [i32],
@@ -143,6 +144,12 @@ def evaluator_stats():
     failures = ctypes.c_uint64()
     if lib.tcr_evaluator_record_error(buf, len(buf), ctypes.byref(failures)) != 0:
         raise GraphError(lib.tcr_last_error().decode())
+    record_ms, jit_ms = ctypes.c_double(), ctypes.c_double()
+    compiled, from_disk = ctypes.c_uint64(), ctypes.c_uint64()
+    if lib.tcr_evaluator_record_cost(ctypes.byref(record_ms), ctypes.byref(jit_ms), ctypes.byref(compiled), ctypes.byref(from_disk)) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+    stats.update(record_ms=round(record_ms.value, 3), jit_ms=round(jit_ms.value, 3), jit_compiled=int(compiled.value),
+                 jit_from_disk=int(from_disk.value))
     stats["record_failures"] = int(failures.value)
     stats["record_error"] = buf.value.decode()
     return stats

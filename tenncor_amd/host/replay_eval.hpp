@@ -37,6 +37,12 @@ struct ReplayEvaluator final : public teq::iEvaluator
 		size_t launches = 0;  ///< device launches in the most recent recording
 		size_t reserved_bytes = 0; ///< device memory held by live recordings
 		size_t record_failures = 0; ///< target sets whose pass could not be recorded
+		/// What the most recent recording cost on the host: milliseconds from
+		/// planning to the finished launch sequence, of which `jit_ms` went into
+		/// `jit_compiled` kernels compiled at run time and `jit_from_disk`
+		/// kernels an earlier process had left on disk
+		double record_ms = 0.0, jit_ms = 0.0;
+		size_t jit_compiled = 0, jit_from_disk = 0;
 		/// why the latest of them could not ("" when none): the message of the
 		/// failure raised while recording; the set is walked node by node instead
 		std::string record_error;

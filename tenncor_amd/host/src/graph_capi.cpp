@@ -271,6 +271,19 @@ int tcr_evaluator_stats (uint64_t out[6])
 	});
 }
 
+int tcr_evaluator_record_cost (double* record_ms, double* jit_ms, uint64_t* jit_compiled, uint64_t* jit_from_disk)
+{
+	return guarded([&]
+	{
+		eigen::ReplayEvaluator::Stats st;
+		if (auto replay = dynamic_cast<eigen::ReplayEvaluator*>(&teq::get_eval())) { st = replay->stats(); }
+		if (record_ms) { *record_ms = st.record_ms; }
+		if (jit_ms) { *jit_ms = st.jit_ms; }
+		if (jit_compiled) { *jit_compiled = st.jit_compiled; }
+		if (jit_from_disk) { *jit_from_disk = st.jit_from_disk; }
+	});
+}
+
 int tcr_evaluator_record_error (char* out, size_t capacity, uint64_t* failures)
 {
 	return guarded([&]

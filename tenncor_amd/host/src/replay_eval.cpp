@@ -5,6 +5,7 @@
 #include "fuse_plan.hpp"
 
 #include <algorithm>
+#include <chrono>
 #include <cstdlib>
 
 namespace eigen
@@ -230,6 +231,10 @@ void ReplayEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 
 std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, const KeyT& key, const teq::TensSetT& targets)
 {
+	const auto begun = std::chrono::steady_clock::now();
+	uint64_t compiled0 = 0, disk0 = 0;
+	double jit0 = 0.0;
+	tcg_jit_stats(hip_context(), &compiled0, &disk0, &jit0);
 	Collector collector;
 	teq::multi_visit(collector, key);
 	if (collector.funcs_.empty()) { return nullptr; }
@@ -391,6 +396,13 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 	tcg_graph_stats(plan->graph, &launches, &plan->bytes);
 	++stats_.recorded;
 	stats_.launches = launches;
+	uint64_t compiled1 = 0, disk1 = 0;
+	double jit1 = 0.0;
+	tcg_jit_stats(ctx, &compiled1, &disk1, &jit1);
+	stats_.record_ms = std::chrono::duration<double,std::milli>(std::chrono::steady_clock::now() - begun).count();
+	stats_.jit_ms = jit1 - jit0;
+	stats_.jit_compiled = (size_t) (compiled1 - compiled0);
+	stats_.jit_from_disk = (size_t) (disk1 - disk0);
 	return plan;
 }
 
