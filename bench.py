@@ -513,12 +513,91 @@ def run_cpu_baseline():
                                   "through Eigen's blocked kernel)" % (mb, blas_reps)}
     return {
         "matmul": matmul,
+        "graphs": run_cpu_graph_baseline(matmul["port_GFLOPs"], cores),
         "value": round(passes * nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
         "sample": "the same graph on np[%d,%d] (the whole workload), %d passes, %.1f s single-thread"
                   % (rows, COLS, passes, dt),
         "all_cores": {"value": round(mpasses * nbytes / mdt / 1e9, 3), "unit": "GB/s", "cores": cores,
                       "sample": "row slabs of the same workload on %d threads, %d passes, %.1f s" % (cores, mpasses, mdt)},
     }
+
+
+def run_cpu_graph_baseline(port_gflops, cores):
+    """The graph third of the metric on the host (tenncor/bm/benchmark.cpp:334-393:
+    re-assign the input, time evaluate).  configs[0]: the whole graph, node by
+    node in the evaluator's order, every node by the oracle's scalar routine,
+    inside one C call (oracle/graph_tape.c), one core -- the reference's
+    evaluator is single-threaded too.  configs[3] and [4]: their matrix
+    products at full size through the host's BLAS (what an optimised CPU
+    library reaches; the reference multiplies through Eigen's blocked kernel
+    on one core), the port's triple loop extrapolated from its measured rate,
+    and the whole graph on the port at reduced size."""
+    from tenncor_amd import graph as tg, configs
+    from oracle import graph_tape
+    out = {}
+    rng = np.random.default_rng(0)
+    g = tg.Graph()
+    targets, x, _ = configs.config1_mlp(g)
+    tape = graph_tape.Tape(g, targets)
+    tape.run(200)
+    secs = []
+    for _ in range(10):
+        tape.set(x, rng.uniform(-1, 1, 30).astype(np.float32))
+        secs += tape.run(200)
+    us = float(np.median(secs)) * 1e6
+    out["config1_mlp"] = {"us_per_eval": round(us, 2), "evals_per_sec": round(1e6 / us, 1), "cores": 1, "kind": "port",
+                          "sample": "the whole graph (%d functors), 2000 evaluations, median" % tape.nops}
+    g.close()
+
+    def blas_ms(shapes, reps=2):
+        mats = [(rng.standard_normal((m, k)).astype(np.float32), rng.standard_normal((k, n)).astype(np.float32)) for m, k, n, _ in shapes]
+        for a, b in mats:
+            a @ b
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            for (a, b), (_, _, _, count) in zip(mats, shapes):
+                for _ in range(count):
+                    a @ b
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    # configs[3]: per time step the gate product [x_t, h] W, its transpose-weight product
+    # backwards and its weight-gradient term, 64 steps (the walk multiplies all 768 columns back)
+    shapes4 = [(256, 768, 2048, 64), (256, 2048, 768, 64), (768, 256, 2048, 64)]
+    flops4 = sum(2.0 * m * k * n * c for m, k, n, c in shapes4)
+    ms4 = blas_ms(shapes4, reps=1)
+    g = tg.Graph()
+    small = dict(seq=8, batch=32, nin=32, hid=64)
+    targets, x, _, small_flops = configs.config4_lstm(g, **small)
+    tape = graph_tape.Tape(g, targets)
+    small_ms = float(np.median(tape.run(5))) * 1e3
+    out["config4_lstm"] = {
+        "products_host_blas_ms": round(ms4, 1), "products_host_blas_GFLOPs": round(flops4 / ms4 / 1e6, 1), "host_blas_cores": cores,
+        "products_port_extrapolated_s": round(flops4 / (port_gflops * 1e9), 1), "port_cores": 1,
+        "sample": "the 192 products of the configuration at full size (%.1f GFLOP) through numpy's BLAS; the port's time is "
+                  "that work at the rate of its 1024^3 product" % (flops4 / 1e9),
+        "reduced_graph_on_port": {"ms_per_eval": round(small_ms, 2), "functors": tape.nops, "size": small,
+                                  "product_GFLOP": round(small_flops / 1e9, 4)}}
+    g.close()
+    # configs[4]: the convolutions of both layers as the products they lower to (forward, image
+    # gradient of the second layer as executed, both kernel gradients)
+    shapes5 = [(73728, 25, 32, 1), (51200, 800, 64, 1), (73728, 1600, 32, 1), (800, 51200, 64, 1), (25, 73728, 32, 1)]
+    flops5 = sum(2.0 * m * k * n * c for m, k, n, c in shapes5)
+    ms5 = blas_ms(shapes5, reps=2)
+    g = tg.Graph()
+    small = dict(batch=4, hw=16, c1=8, c2=8, ncls=10)
+    targets, x, _, small_flops = configs.config5_cnn(g, **small)
+    tape = graph_tape.Tape(g, targets)
+    small_ms = float(np.median(tape.run(3))) * 1e3
+    out["config5_cnn"] = {
+        "products_host_blas_ms": round(ms5, 2), "products_host_blas_GFLOPs": round(flops5 / ms5 / 1e6, 1), "host_blas_cores": cores,
+        "products_port_extrapolated_s": round(flops5 / (port_gflops * 1e9), 1), "port_cores": 1,
+        "sample": "the five products the convolutions lower to at batch 128 (%.1f GFLOP, operands already gathered) through "
+                  "numpy's BLAS" % (flops5 / 1e9),
+        "reduced_graph_on_port": {"ms_per_eval": round(small_ms, 2), "functors": tape.nops, "size": small,
+                                  "useful_GFLOP": round(small_flops / 1e9, 4),
+                                  "note": "the port evaluates the padded convolutions of the conv2d idiom literally"}}
+    g.close()
+    return out
 
 
 def run_matmul_ramp(blocks=12, per_block=10):

@@ -132,6 +132,11 @@ int tcr_dtype (tcr_graph* g, int node, int* dtype);
 int tcr_data (tcr_graph* g, int node, void* out, size_t bytes);
 int tcr_version (tcr_graph* g, int node, uint64_t* version);
 
+/* An attribute of a functor as tcr_functor takes them (marsh::iAttributed::
+ * get_attr, internal/marsh/attrs.hpp): the integer list under `key`; for
+ * "tensor" the node id, for "dtype" the type code.  *len = -1 when the node
+ * has no such attribute (or is a leaf); vals may be NULL to ask for the length. */
+int tcr_attr (tcr_graph* g, int node, const char* key, int64_t* vals, int capacity, int* len);
 /* Structure: opcode (0 for leaves), operands, and the indented dump used by
  * the reference's graph-equality tests (testutil/tutil.hpp) */
 int tcr_opcode (tcr_graph* g, int node, int* opcode);

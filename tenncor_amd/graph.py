@@ -32,7 +32,7 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_evaluate_ignoring", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
-    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_evaluator_record_cost", "tcr_launch_plan", "tcr_optimize",
+    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_evaluator_record_cost", "tcr_attr", "tcr_launch_plan", "tcr_optimize",
     "tcr_set_random", "tcr_seed",
 ]
 
@@ -80,6 +80,7 @@ def load():
         "tcr_nargs": [vp, i32, i32p],
         "tcr_args": [vp, i32, i32p, i32],
         "tcr_to_string": [vp, i32, ctypes.c_char_p, ctypes.c_size_t],
+        "tcr_attr": [vp, i32, ctypes.c_char_p, ctypes.POINTER(ctypes.c_int64), i32, i32p],
         "tcr_count_functors": [vp, i32, i32p, i32p],
         "tcr_set_evaluator": [i32],
         "tcr_evaluator_stats": [u64p],
@@ -298,6 +299,19 @@ class Graph:
         buf = (ctypes.c_int * max(n.value, 1))()
         self._check(self.lib.tcr_args(self.h, node.id, buf, n.value))
         return [Node(self, buf[i]) for i in range(n.value)]
+
+    def attr(self, node, key):
+        """The integer list a functor holds under an attribute key (None when
+        it has none): "tensor" gives the node, "dtype" the type code."""
+        n = ctypes.c_int()
+        self._check(self.lib.tcr_attr(self.h, node.id, key.encode(), None, 0, ctypes.byref(n)))
+        if n.value < 0:
+            return None
+        buf = (ctypes.c_int64 * max(n.value, 1))()
+        self._check(self.lib.tcr_attr(self.h, node.id, key.encode(), buf, n.value, ctypes.byref(n)))
+        if key == "tensor":
+            return Node(self, int(buf[0]))
+        return [int(buf[i]) for i in range(n.value)]
 
     def to_string(self, node):
         buf = ctypes.create_string_buffer(1 << 20)

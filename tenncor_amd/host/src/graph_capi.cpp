@@ -367,6 +367,34 @@ int tcr_args (tcr_graph* g, int node, int* args, int capacity)
 	});
 }
 
+int tcr_attr (tcr_graph* g, int node, const char* key, int64_t* vals, int capacity, int* len)
+{
+	return guarded([&]
+	{
+		*len = -1;
+		auto f = dynamic_cast<teq::iFunctor*>(g->at(node).get());
+		if (nullptr == f) { return; }
+		const marsh::iObject* obj = f->get_attr(key);
+		if (nullptr == obj) { return; }
+		std::vector<int64_t> out;
+		if (auto arr = dynamic_cast<const marsh::NumArray<int64_t>*>(obj)) { out = arr->contents_; }
+		else if (auto num = dynamic_cast<const marsh::iNumber*>(obj)) { out.push_back(num->to_int64()); }
+		else if (auto tens = dynamic_cast<const teq::TensorObj*>(obj)) { out.push_back(g->add(tens->get_tensor())); }
+		else if (auto text = dynamic_cast<const marsh::String*>(obj))
+		{
+			// a type name: its code in the numbering of tcr_variable
+			out.push_back((int64_t) egen::device_type(egen::get_type(text->to_string())));
+		}
+		else { global::fatalf("attribute `%s` holds neither numbers nor a tensor", key); }
+		*len = (int) out.size();
+		if (nullptr != vals)
+		{
+			if ((int) out.size() > capacity) { global::fatal("attribute buffer is too small"); }
+			std::copy(out.begin(), out.end(), vals);
+		}
+	});
+}
+
 int tcr_to_string (tcr_graph* g, int node, char* out, size_t capacity)
 {
 	return guarded([&]
