@@ -63,7 +63,16 @@ enum tcg_status
  * another order (the enum it generates follows the key order of the file): a
  * binding built for that configuration maps its codes onto these.  Integer
  * arithmetic wraps modulo 2^width; integer division by zero, and the lowest
- * value of a 32- or 64-bit type divided by -1 (both trap on the CPU), give 0. */
+ * value of a 32- or 64-bit type divided by -1 (both trap on the CPU), give 0.
+ * The transcendental operators of an integer type (SIN .. SIGMOID, TANH, and
+ * POW through its repeated multiplication) go through double and convert back
+ * the way the reference's `(T) std::exp(x)` does: the double becomes an integer
+ * of 32 bits (64 for the 64-bit types) of the type's signedness, which is then
+ * narrowed.  Where the double does not fit that integer -- EXP of more than 21
+ * (signed) or 22 (unsigned), 43 / 44 for the 64-bit types, and SIGMOID of less
+ * than minus those -- C++ leaves the conversion undefined and the results are
+ * unspecified here too (the device saturates where x86 gives its indefinite
+ * value); inside those bounds device and CPU agree. */
 enum tcg_dtype
 {
 	TCG_BAD_TYPE = 0, TCG_DOUBLE = 1, TCG_FLOAT = 2, TCG_INT32 = 3,
@@ -104,6 +113,12 @@ int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr);
 int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes);
 /* Bytes currently handed out / held by the pool (for leak checks in tests) */
 int tcg_mem_stats (const tcg_ctx* ctx, uint64_t* in_use, uint64_t* pooled);
+/* Device memory the context holds outside the pool until it is destroyed: the
+ * row / summed-index tables of convolutions lowered to matrix products, kept
+ * by the plan they were computed from so that a pass over the same layers
+ * finds them again (at most 256 MiB; recorded launches keep their addresses,
+ * so they are never given back earlier). */
+int tcg_mem_stats_kept (const tcg_ctx* ctx, uint64_t* conv_tables);
 
 /* Replaces: the memcpy in eigen::SrcRef<T>::assign (internal/eigen/device.hpp:
  * 200-247) and host reads through iDeviceRef::data()
@@ -343,9 +358,15 @@ int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
  * TCG_REDUCE_NOALLOC_SCRATCH_BYTES (each piece rounded up to 256 bytes),
  * otherwise the call fails with TCG_ERR_ARG and nothing is launched for the
  * step that did not fit; every call on a GPU uses that GPU's one array, so
- * calls that overlap on one GPU (two contexts, two streams) race -- calls on
- * one context are ordered on its stream and do not.  Not available inside
- * tcg_capture_begin_small. */
+ * calls that overlap on one GPU (two contexts, two streams) would race --
+ * calls on one context are ordered on its stream and do not.  A call from
+ * another context while the launches of the context that used the array last
+ * are still running is refused with TCG_ERR_ARG (nothing is launched; try
+ * again once that context has been synchronised).  Launches that are being
+ * recorded -- by tcg_capture_begin or by the caller's own capture of the
+ * stream -- run when the recording is launched, which the library cannot
+ * order against other users of the array: keeping them apart is then up to
+ * the caller.  Not available inside tcg_capture_begin_small. */
 #define TCG_REDUCE_NOALLOC_SCRATCH_BYTES ((size_t) 8 << 20)
 int tcg_reduce_noalloc (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
 	unsigned rankmask, const void* in, void* out);

@@ -204,6 +204,10 @@ __device__ __forceinline__ uint32_t conv_div (uint32_t n, const ConvDiv& f)
 
 struct ConvGemmPlan
 {
+	// The bytes of a plan are the key under which its tables are kept
+	// (tcg_ctx::conv_tables): every byte, padding included, starts at zero.
+	ConvGemmPlan (void) { memset((void*) this, 0, sizeof(*this)); }
+
 	// per image dim: extents of its row, summed and column component (1 = none)
 	uint32_t msize[8], ssize[8], nsize[8];
 	ConvDiv mdiv[8], sdiv[8], ndiv[8];
@@ -742,12 +746,7 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			if (kept_tables && ctx->capturing)
 			{
 				// kept tables are filled once, now, not by the recording at every replay
-				if (nullptr == ctx->side_stream && hipStreamCreate(&ctx->side_stream) != hipSuccess)
-				{
-					(void) hipGetLastError();
-					ctx->side_stream = nullptr;
-				}
-				if (ctx->side_stream) { where = ctx->side_stream; }
+				where = ctx->side_stream;
 			}
 			conv_tables_k<<<(longest + CG_BLOCK - 1) / CG_BLOCK, CG_BLOCK, 0, where>>>(g,
 				(ConvTabEntry*) RT, (ConvTabEntry*) ST);
@@ -921,8 +920,7 @@ static int conv_boxed_impl (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 			p.ooff0 -= (int64_t) p.wlo[d] * out_stride[d];
 		}
 	}
-	ConvGemmPlan gp;
-	memset((void*) &gp, 0, sizeof(gp)); // its bytes name the tables computed from it
+	ConvGemmPlan gp; // (zeroed by its constructor: its bytes name the tables computed from it)
 	const char* gemm_env = getenv("TCG_CONV_GEMM"); // "0": direct kernels only (the parity reference)
 	// (the product route exists for the three default types)
 	if (!(gemm_env && gemm_env[0] == '0') && tcg_default_dtype(dtype) && conv_gemm_plan(p, gp))

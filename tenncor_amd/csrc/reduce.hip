@@ -14,6 +14,7 @@
 #include "tcg_internal.hpp"
 
 #include <limits>
+#include <mutex>
 #include <type_traits>
 
 // Device memory that exists for as long as the library is loaded, one copy on
@@ -25,6 +26,16 @@ static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 
 constexpr int MAX_DEVICES = 64;
 static unsigned char* g_scratch[MAX_DEVICES] = {nullptr};
+// Every context on a GPU shares that GPU's array, and every call starts at its
+// first byte: the context that used it last, with the event recorded behind its
+// launches.  Another context is let in once that event has passed.
+struct ScratchOwner
+{
+	tcg_ctx* ctx = nullptr;
+	hipEvent_t done = nullptr;
+};
+static ScratchOwner g_owner[MAX_DEVICES];
+static std::mutex g_scratch_mu; // g_scratch and g_owner
 
 namespace
 {
@@ -599,13 +610,27 @@ int tcg_reduce_scratch_init (tcg_ctx* ctx)
 	{
 		return tcg_fail(ctx, TCG_ERR_ARG, "device %d: at most %d devices", ctx->device, MAX_DEVICES);
 	}
+	std::lock_guard<std::mutex> lock(g_scratch_mu);
 	if (nullptr == g_scratch[ctx->device])
 	{
 		unsigned char* ptr = nullptr;
 		TCG_HIP(ctx, hipGetSymbolAddress((void**) &ptr, HIP_SYMBOL(scratch)));
 		g_scratch[ctx->device] = ptr;
 	}
+	if (nullptr == ctx->scratch_done) { TCG_HIP(ctx, hipEventCreateWithFlags(&ctx->scratch_done, hipEventDisableTiming)); }
 	return TCG_OK;
+}
+
+// Called by tcg_ctx_destroy once the context's stream has drained
+void tcg_reduce_scratch_release (tcg_ctx* ctx)
+{
+	std::lock_guard<std::mutex> lock(g_scratch_mu);
+	if (ctx->device >= 0 && ctx->device < MAX_DEVICES && g_owner[ctx->device].ctx == ctx) { g_owner[ctx->device] = ScratchOwner(); }
+	if (nullptr != ctx->scratch_done)
+	{
+		(void) hipEventDestroy(ctx->scratch_done);
+		ctx->scratch_done = nullptr;
+	}
 }
 
 extern "C" {
@@ -634,8 +659,28 @@ int tcg_reduce_noalloc (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shap
 	unsigned char* base = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch[ctx->device] : nullptr;
 	if (nullptr == base) { return tcg_fail(ctx, TCG_ERR_HIP, "tcg_reduce_noalloc: no scratch memory on device %d", ctx->device); }
 	if (tcg_n_elems(shape) == 0) { return TCG_OK; }
+	// Launches that are being recorded (by tcg_capture_begin or by the caller's own
+	// capture of this stream) run when their recording is launched, which nothing
+	// here can order against other users of the array: no check, and no event.
+	hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+	(void) hipStreamIsCapturing(ctx->stream, &capture);
+	const bool recorded = nullptr != ctx->capturing || capture != hipStreamCaptureStatusNone;
+	if (false == recorded)
+	{
+		std::lock_guard<std::mutex> lock(g_scratch_mu);
+		ScratchOwner& owner = g_owner[ctx->device];
+		if (nullptr != owner.ctx && owner.ctx != ctx && hipErrorNotReady == hipEventQuery(owner.done))
+		{
+			return tcg_fail(ctx, TCG_ERR_ARG, "tcg_reduce_noalloc: another context's reduction is still using "
+				"the scratch array of device %d (calls that overlap on one GPU would race)", ctx->device);
+		}
+		owner.ctx = ctx;
+		owner.done = ctx->scratch_done;
+	}
 	FixedScratch mem(base);
-	return reduce_any(ctx, mem, opcode, dtype, shape, rankmask, in, out);
+	int rc = reduce_any(ctx, mem, opcode, dtype, shape, rankmask, in, out);
+	if (false == recorded) { (void) hipEventRecord(ctx->scratch_done, ctx->stream); }
+	return rc;
 }
 
 int tcg_argmax (tcg_ctx* ctx, int dtype, const uint64_t shape[8], int return_dim,

@@ -96,9 +96,21 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		delete ctx;
 		return rc;
 	}
+	// the stream on which convolution tables first met during a recording are filled
+	// (made here so that it cannot fail in the middle of a recording)
+	if ((err = hipStreamCreate(&ctx->side_stream)) != hipSuccess)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: second stream: %s", hipGetErrorString(err));
+		(void) hipFree(ctx->zeros);
+		(void) hipFree(ctx->rng_state);
+		(void) hipHostFree(ctx->staging);
+		delete ctx;
+		return rc;
+	}
 	if (tcg_reduce_scratch_init(ctx) != TCG_OK)
 	{
 		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: %s", ctx->error.c_str());
+		(void) hipStreamDestroy(ctx->side_stream);
 		(void) hipFree(ctx->zeros);
 		(void) hipFree(ctx->rng_state);
 		(void) hipHostFree(ctx->staging);
@@ -114,6 +126,7 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	if (!ctx) { return TCG_OK; }
 	(void) hipSetDevice(ctx->device);
 	(void) hipStreamSynchronize(ctx->stream);
+	tcg_reduce_scratch_release(ctx);
 	ctx->pool.release_all();
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
 	if (ctx->rng_state) { (void) hipFree(ctx->rng_state); }
@@ -169,6 +182,13 @@ int tcg_mem_stats (const tcg_ctx* ctx, uint64_t* in_use, uint64_t* pooled)
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (in_use) { *in_use = ctx->pool.bytes_in_use; }
 	if (pooled) { *pooled = ctx->pool.bytes_pooled; }
+	return TCG_OK;
+}
+
+int tcg_mem_stats_kept (const tcg_ctx* ctx, uint64_t* conv_tables)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (conv_tables) { *conv_tables = ctx->conv_table_bytes; }
 	return TCG_OK;
 }
 

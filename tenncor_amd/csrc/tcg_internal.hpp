@@ -81,6 +81,9 @@ struct tcg_ctx
 
 	// launch capture: the graph being recorded (its arena is pool.recording)
 	tcg_graph* capturing = nullptr;
+
+	// recorded behind the launches of this context's latest tcg_reduce_noalloc
+	hipEvent_t scratch_done = nullptr;
 };
 
 int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);
@@ -200,6 +203,7 @@ int tcg_gemm_f32_mfma_ranges (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t K, 
 // reduce.hip: looks up this GPU's copy of the scratch memory of
 // tcg_reduce_noalloc; called once per context with the device current
 int tcg_reduce_scratch_init (tcg_ctx* ctx);
+void tcg_reduce_scratch_release (tcg_ctx* ctx);
 
 // Number of workgroups for a streaming kernel: enough to cover `work` items,
 // capped at a multiple of the CU count so that a grid-stride loop takes over

@@ -849,6 +849,35 @@ def test_conv_as_matrix_product_equals_direct_kernels(ctx, oracle, which):
                     os.environ.pop(key, None)
 
 
+def test_kept_convolution_tables_are_counted_and_found_again():
+    """The row / summed-index tables of a convolution lowered to a product stay
+    with the context (outside its pool): tcg_mem_stats_kept counts them, a second
+    correlation of the same plan finds them again instead of adding to them,
+    and neither call leaves anything handed out."""
+    from tenncor_amd import capi
+    from oracle import oracle as orc
+    own = capi.Context(0)
+    try:
+        ishape, kshape, ranks, ibox, obox = conv2d_idiom_cases(C=12, W=15, H=13, B=12, O=24, KW=3, KH=4)["forward"]
+        rng = np.random.default_rng(seed_of("kept tables"))
+        img = rng.uniform(-1, 1, orc.n_elems(ishape)).astype(np.float32)
+        ker = rng.uniform(-1, 1, orc.n_elems(kshape)).astype(np.float32)
+        n_out = orc.n_elems(orc.conv_shape(ishape, kshape, ranks))
+        dimg, dker, out = own.upload(img), own.upload(ker), own.empty(n_out, np.float32)
+        assert own.mem_stats_kept() == 0
+        in_use = own.mem_stats()[0]
+        own.conv_boxed(capi.FLOAT, ishape, kshape, ranks, ibox, obox, dimg.ptr, dker.ptr, out.ptr)
+        first = out.get().copy()
+        kept = own.mem_stats_kept()
+        assert 0 < kept <= 256 << 20
+        own.conv_boxed(capi.FLOAT, ishape, kshape, ranks, ibox, obox, dimg.ptr, dker.ptr, out.ptr)
+        np.testing.assert_array_equal(out.get(), first)
+        assert own.mem_stats_kept() == kept
+        assert own.mem_stats()[0] == in_use
+    finally:
+        own.close()
+
+
 @pytest.mark.parametrize("which", ["forward", "image_gradient", "kernel_gradient"])
 @pytest.mark.parametrize("channels", [(8, 32), (6, 36)], ids=["groups_of_four", "element_by_element"])
 def test_conv_product_reading_the_image_in_place(ctx, oracle, which, channels):

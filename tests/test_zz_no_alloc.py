@@ -125,3 +125,91 @@ def test_sizes_beyond_the_fixed_memory_are_refused(ctx):
     np.testing.assert_array_equal(got, small.reshape(2, 3, 4).sum(axis=(0, 2)))
     src.release()
     dst.release()
+
+
+@pytest.mark.parametrize("np_dtype", [np.int8, np.int64])
+def test_the_narrowest_and_the_widest_integers(ctx, np_dtype):
+    """The integer widths of the full type configuration share the kernels:
+    two calls in a row, the second smaller, bit for bit with tcg_reduce."""
+    rng = np.random.default_rng(seed=31 + np.dtype(np_dtype).itemsize)
+    info = np.iinfo(np_dtype)
+    for shape, rank_set in (([4096, 2048], [1]), ([1024, 512], [1]), ([64, 512, 48, 8], [1, 3]), ([129, 65, 3], [0, 2])):
+        n = int(np.prod(shape))
+        data = rng.integers(max(info.min, -1000), min(info.max, 1000) + 1, n).astype(np_dtype)
+        for op in ("REDUCE_SUM", "REDUCE_MAX"):
+            print("case", np_dtype.__name__, op, shape, rank_set, flush=True)
+            want, got, before, after = both(ctx, op, np_dtype, shape, rank_set, data)
+            np.testing.assert_array_equal(got, want)
+            assert before == after
+
+
+def test_a_recorded_reduction_replayed_after_the_array_was_used_again(ctx):
+    """The use the entry point names first: under tcg_capture_begin the launches
+    of tcg_reduce_noalloc are recorded with the array's address in them.  An
+    eager reduction in between leaves its own partial results there; the
+    replay, over new input, must still equal tcg_reduce bit for bit (every
+    replay writes its partial results before it reads them)."""
+    from tenncor_amd import capi
+    rng = np.random.default_rng(seed=91)
+    shape, rank_set = [4096, 2048], [1]
+    n = 4096 * 2048
+    src = ctx.upload(rng.uniform(-1, 1, n).astype(np.float32))
+    got = ctx.empty(4096, np.float32)
+    want = ctx.empty(4096, np.float32)
+    ctx.capture_begin()
+    ctx.reduce_noalloc("REDUCE_SUM", capi.FLOAT, shape, rank_set, src.ptr, got.ptr)
+    graph = ctx.capture_end()
+    try:
+        for round_ in range(3):
+            fresh = rng.uniform(-1, 1, n).astype(np.float32)
+            ctx.h2d(src.ptr, fresh)
+            # another reduction through the same array, of another shape, eagerly
+            other = ctx.upload(rng.integers(-1000, 1001, 1 << 20).astype(np.int32))
+            other_out = ctx.empty(1, np.int32)
+            ctx.reduce_noalloc("REDUCE_SUM", capi.INT32, [1 << 20], [0], other.ptr, other_out.ptr)
+            ctx.graph_launch(graph)
+            ctx.reduce("REDUCE_SUM", capi.FLOAT, shape, rank_set, src.ptr, want.ptr)
+            ctx.sync()
+            print("replay", round_, flush=True)
+            np.testing.assert_array_equal(got.get(), want.get())
+            other.release()
+            other_out.release()
+    finally:
+        ctx.graph_destroy(graph)
+
+
+def test_another_context_waits_for_the_owner_of_the_array(ctx):
+    """Two contexts on one GPU share the array.  While the launches of the one
+    that used it last may still be running, the other is refused (TCG_ERR_ARG,
+    nothing launched); once the first has been synchronised it is let in, and
+    both compute what tcg_reduce computes."""
+    from tenncor_amd import capi
+    other = capi.Context(0)
+    try:
+        rng = np.random.default_rng(seed=17)
+        shape, rank_set = [4096, 8192], [1]
+        data = rng.integers(-1000, 1001, 4096 * 8192).astype(np.int32)
+        src, out = ctx.upload(data), ctx.empty(4096, np.int32)
+        src2, out2 = other.upload(data[:1 << 20]), other.empty(1, np.int32)
+        ctx.sync()
+        other.sync()
+        for _ in range(8):
+            ctx.reduce_noalloc("REDUCE_SUM", capi.INT32, shape, rank_set, src.ptr, out.ptr)
+        refused = False
+        try:
+            other.reduce_noalloc("REDUCE_SUM", capi.INT32, [1 << 20], [0], src2.ptr, out2.ptr)
+        except capi.TcgError as err:
+            refused = True
+            assert err.status == 1 and "another context" in str(err)
+        print("refused while the owner was busy:", refused, flush=True)
+        ctx.sync()
+        other.reduce_noalloc("REDUCE_SUM", capi.INT32, [1 << 20], [0], src2.ptr, out2.ptr)
+        other.sync()
+        np.testing.assert_array_equal(out2.get(), data[:1 << 20].sum(dtype=np.int64).astype(np.int32))
+        np.testing.assert_array_equal(out.get(), data.reshape(8192, 4096).sum(axis=0, dtype=np.int64).astype(np.int32))
+        # and back: the first context after the second has finished
+        ctx.reduce_noalloc("REDUCE_MAX", capi.INT32, shape, rank_set, src.ptr, out.ptr)
+        ctx.sync()
+        np.testing.assert_array_equal(out.get(), data.reshape(8192, 4096).max(axis=0))
+    finally:
+        other.close()
