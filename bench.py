@@ -376,6 +376,8 @@ def run_graph_configs(only=None, evaluator=None, reps=20, optimize=False):
                    "functors": g.count_functors(targets), "evaluator_stats": tg.evaluator_stats()}
             if cleanup is not None:
                 out["optimize"] = cleanup
+            if kind == "timing":
+                out["timing_report"] = tg.evaluator_timing().splitlines()
             tg.set_evaluator("default")
             return out
         g = tg.Graph()
@@ -630,7 +632,9 @@ def main():
     ap.add_argument("--no-graphs", action="store_true", help="skip the whole-graph side metrics (configs 1, 4, 5)")
     ap.add_argument("--graph-config", type=int, choices=[1, 4, 5], default=None,
                     help="time only this whole-graph configuration and print its line (for profiling)")
-    ap.add_argument("--evaluator", choices=["default", "plain", "replay", "replay_launches", "replay_unfused"], default="replay")
+    ap.add_argument("--evaluator", choices=["default", "plain", "replay", "replay_launches", "replay_unfused", "timing"], default="replay",
+                    help="with --graph-config; timing: the recording's launches run one by one between HIP events, "
+                         "device microseconds per kind of launch in the line's timing_report")
     ap.add_argument("--f64", action="store_true", help="with --matmul-only: the 4096^3 product in double")
     ap.add_argument("--reps", type=int, default=None,
                     help="timed evaluations with --graph-config 4 or 5 (default 20), timed launches with --matmul-only (100)")

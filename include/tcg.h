@@ -142,6 +142,16 @@ int tcg_event_destroy (tcg_ctx* ctx, void* event);
 int tcg_event_record (tcg_ctx* ctx, void* event);
 int tcg_event_elapsed (tcg_ctx* ctx, void* start, void* stop, float* ms);
 
+/* For measurements: everything enqueued on the context's stream after tcg_hold
+ * waits until tcg_release, and then runs back to back, so that events recorded
+ * in between (tcg_event_record) measure the device and not the pace at which
+ * the host enqueues.  tcg_release returns when the held work has run.  Calls
+ * that wait for the stream themselves (tcg_sync, tcg_d2h, tcg_timer_end,
+ * tcg_event_elapsed) must not be made while it is held: they would wait for
+ * the release.  No counterpart in the reference. */
+int tcg_hold (tcg_ctx* ctx);
+int tcg_release (tcg_ctx* ctx);
+
 /* ---- recorded launch sequences ---------------------------------------- */
 
 /* What one pass of teq::Evaluator::evaluate enqueues (internal/teq/

@@ -94,7 +94,13 @@ int tcr_sync (tcr_graph* g);
 #define TCR_EVAL_REPLAY_UNFUSED 2
 #define TCR_EVAL_REPLAY_LAUNCHES 3
 #define TCR_EVAL_DEFAULT 4
+/* the launches TCR_EVAL_REPLAY would record, run one after the other with a
+ * HIP event in front of and behind each (the slot the reference's debugging
+ * evaluator takes, dbg/peval/plugin_eval.hpp:21-42): tcr_evaluator_timing
+ * returns the device microseconds per kind of launch as text */
+#define TCR_EVAL_TIMING 5
 int tcr_set_evaluator (int kind);
+int tcr_evaluator_timing (char* out, size_t capacity, size_t* needed);
 /* Counters of the replaying evaluator (zeros under TCR_EVAL_PLAIN):
  * out[0] passes walked node by node, out[1] recordings made, out[2] passes
  * served by a recording, out[3] passes with nothing to do, out[4] launches in

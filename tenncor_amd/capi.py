@@ -39,7 +39,7 @@ OPD_NONE, OPD_ACC, OPD_T0, OPD_T1, OPD_IMM, OPD_LEAF0 = 0, 1, 2, 3, 4, 8
 # every symbol include/tcg.h declares
 EXPORTS = [
     "tcg_ctx_create", "tcg_ctx_destroy", "tcg_last_error", "tcg_device_arch", "tcg_alloc", "tcg_free",
-    "tcg_mem_stats", "tcg_mem_stats_kept", "tcg_h2d", "tcg_d2h", "tcg_d2d", "tcg_fill_zero", "tcg_sync", "tcg_timer_begin",
+    "tcg_mem_stats", "tcg_mem_stats_kept", "tcg_hold", "tcg_release", "tcg_h2d", "tcg_d2h", "tcg_d2d", "tcg_fill_zero", "tcg_sync", "tcg_timer_begin",
     "tcg_timer_end", "tcg_event_create", "tcg_event_destroy", "tcg_event_record", "tcg_event_elapsed",
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
@@ -96,6 +96,8 @@ def load():
         "tcg_free": [vp, vp, sz],
         "tcg_mem_stats": [vp, u64p, u64p],
         "tcg_mem_stats_kept": [vp, u64p],
+        "tcg_hold": [vp],
+        "tcg_release": [vp],
         "tcg_h2d": [vp, vp, vp, sz],
         "tcg_d2h": [vp, vp, vp, sz],
         "tcg_d2d": [vp, vp, vp, sz],

@@ -67,7 +67,8 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		return rc == hipSuccess ? 0 : 1;
 	};
 	ctx->pool.raw_free = [](void* ptr) { (void) hipFree(ptr); };
-	ctx->pool.drain = [ctx] { (void) hipStreamSynchronize(ctx->stream); };
+	// (a held stream cannot be waited for: see tcg_hold)
+	ctx->pool.drain = [ctx] { if (nullptr == ctx->hold) { (void) hipStreamSynchronize(ctx->stream); } };
 	ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	ctx->arch = prop.gcnArchName;
 	size_t colon = ctx->arch.find(':');
@@ -125,6 +126,7 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_OK; }
 	(void) hipSetDevice(ctx->device);
+	(void) tcg_release(ctx);
 	(void) hipStreamSynchronize(ctx->stream);
 	tcg_reduce_scratch_release(ctx);
 	ctx->pool.release_all();
@@ -182,6 +184,47 @@ int tcg_mem_stats (const tcg_ctx* ctx, uint64_t* in_use, uint64_t* pooled)
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (in_use) { *in_use = ctx->pool.bytes_in_use; }
 	if (pooled) { *pooled = ctx->pool.bytes_pooled; }
+	return TCG_OK;
+}
+
+// Launches enqueued between tcg_hold and tcg_release start only at the release,
+// back to back: events recorded between them then measure the device, not how
+// fast the host enqueues
+int tcg_hold (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, nullptr == ctx->capturing, "tcg_hold: not while launches are being recorded");
+	TCG_REQUIRE(ctx, nullptr == ctx->hold, "tcg_hold: the stream is held already");
+	ctx->hold = new tcg_ctx::Hold();
+	hipError_t err = hipLaunchHostFunc(ctx->stream, [](void* arg)
+	{
+		auto hold = static_cast<tcg_ctx::Hold*>(arg);
+		std::unique_lock<std::mutex> lock(hold->mu);
+		hold->cv.wait(lock, [hold] { return hold->open; });
+	}, ctx->hold);
+	if (err != hipSuccess)
+	{
+		delete ctx->hold;
+		ctx->hold = nullptr;
+		return tcg_fail(ctx, TCG_ERR_HIP, "tcg_hold: %s", hipGetErrorString(err));
+	}
+	return TCG_OK;
+}
+
+int tcg_release (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (nullptr == ctx->hold) { return TCG_OK; }
+	{
+		std::lock_guard<std::mutex> lock(ctx->hold->mu);
+		ctx->hold->open = true;
+	}
+	ctx->hold->cv.notify_all();
+	// the host function still holds the pointer until it has run
+	hipError_t err = hipStreamSynchronize(ctx->stream);
+	delete ctx->hold;
+	ctx->hold = nullptr;
+	if (err != hipSuccess) { return tcg_fail(ctx, TCG_ERR_HIP, "tcg_release: %s", hipGetErrorString(err)); }
 	return TCG_OK;
 }
 

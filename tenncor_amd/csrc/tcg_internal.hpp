@@ -8,8 +8,10 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <condition_variable>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <set>
 #include <string>
 #include <vector>
@@ -84,6 +86,15 @@ struct tcg_ctx
 
 	// recorded behind the launches of this context's latest tcg_reduce_noalloc
 	hipEvent_t scratch_done = nullptr;
+
+	// tcg_hold: the stream waits in a host function until tcg_release opens this
+	struct Hold
+	{
+		std::mutex mu;
+		std::condition_variable cv;
+		bool open = false;
+	};
+	Hold* hold = nullptr;
 };
 
 int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);

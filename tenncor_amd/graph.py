@@ -32,11 +32,11 @@ EXPORTS = [
     "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
     "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_evaluate_ignoring", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
-    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_evaluator_record_cost", "tcr_attr", "tcr_launch_plan", "tcr_optimize",
+    "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_evaluator_record_cost", "tcr_evaluator_timing", "tcr_attr", "tcr_launch_plan", "tcr_optimize",
     "tcr_set_random", "tcr_seed",
 ]
 
-EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED, EVAL_REPLAY_LAUNCHES, EVAL_DEFAULT = 0, 1, 2, 3, 4
+EVAL_PLAIN, EVAL_REPLAY, EVAL_REPLAY_UNFUSED, EVAL_REPLAY_LAUNCHES, EVAL_DEFAULT, EVAL_TIMING = 0, 1, 2, 3, 4, 5
 
 # conversions shipped with the package (the reference's cfg/optimizations.json
 # is a git-lfs pointer without content)
@@ -85,6 +85,7 @@ def load():
         "tcr_set_evaluator": [i32],
         "tcr_evaluator_stats": [u64p],
         "tcr_evaluator_record_error": [ctypes.c_char_p, ctypes.c_size_t, u64p],
+        "tcr_evaluator_timing": [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
         "tcr_evaluator_record_cost": [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double), u64p, u64p],
         "tcr_launch_plan": [vp, i32, i32p, ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)],
         "tcr_optimize": [vp, i32, i32p, ctypes.c_char_p, i32, i32p, u64p],
@@ -112,7 +113,7 @@ def set_evaluator(kind):
     reference's evaluator slot."""
     lib = load()
     code = {"plain": EVAL_PLAIN, "replay": EVAL_REPLAY, "replay_unfused": EVAL_REPLAY_UNFUSED,
-            "replay_launches": EVAL_REPLAY_LAUNCHES, "default": EVAL_DEFAULT}[kind]
+            "replay_launches": EVAL_REPLAY_LAUNCHES, "default": EVAL_DEFAULT, "timing": EVAL_TIMING}[kind]
     if lib.tcr_set_evaluator(code) != 0:
         raise GraphError(lib.tcr_last_error().decode())
 
@@ -131,6 +132,19 @@ def seed(value):
     lib = load()
     if lib.tcr_seed(int(value)) != 0:
         raise GraphError(lib.tcr_last_error().decode())
+
+
+def evaluator_timing():
+    """Under set_evaluator("timing"): device microseconds per kind of launch, as text
+    (the launches the replaying evaluator would record, run and timed one by one)."""
+    lib = load()
+    need = ctypes.c_size_t()
+    if lib.tcr_evaluator_timing(None, 0, ctypes.byref(need)) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+    buf = ctypes.create_string_buffer(need.value + 1)
+    if lib.tcr_evaluator_timing(buf, len(buf), None) != 0:
+        raise GraphError(lib.tcr_last_error().decode())
+    return buf.value.decode()
 
 
 def evaluator_stats():

@@ -206,6 +206,13 @@ void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMe
 
 void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMemptrT& memory, std::pair<void*,size_t>& temp);
 
+/// One line for a step: what is launched (tcr_launch_plan prints these)
+std::string describe_step (const FusionPlan& plan, const FusionPlan::Step& step);
+
+/// Enqueues the launches of one step, whatever its kind
+void launch_step (const FusionPlan& plan, const FusionPlan::Step& step, Device& device, const teq::TensSetT& targets,
+	RangeTempsT& temps);
+
 }
 
 #endif // TCH_FUSE_PLAN_HPP

@@ -2170,6 +2170,37 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 	return planner.finish();
 }
 
+std::string describe_step (const FusionPlan& plan, const FusionPlan::Step& step)
+{
+	if (nullptr != step.node) { return "node " + step.node->get_opcode().name_; }
+	if (step.contract >= 0) { return "swapped CONTRACT+PERMUTE"; }
+	if (step.sum >= 0) { return "summed CONTRACT x" + std::to_string(plan.sums[step.sum].a.size()); }
+	if (step.parts >= 0 && step.group < 0) { return plan.part_products[step.parts].label; }
+	if (step.conv >= 0) { return "viewed " + plan.convs[step.conv].label; }
+	const FusedGroup& group = plan.groups[step.group];
+	std::string out;
+	if (step.parts >= 0) { out = plan.part_products[step.parts].label + " with epilogue "; }
+	out += "group ";
+	for (size_t i = 0; i < group.members.size(); ++i) { out += (i ? "+" : "") + group.members[i]->get_opcode().name_; }
+	return out + " leaves=" + std::to_string(group.leaves.size()) + " stores=" + std::to_string(group.outputs.size()) +
+		" instrs=" + std::to_string(group.program.size());
+}
+
+void launch_step (const FusionPlan& plan, const FusionPlan::Step& step, Device& device, const teq::TensSetT& targets,
+	RangeTempsT& temps)
+{
+	if (nullptr != step.node) { device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0)); }
+	else if (step.conv >= 0) { launch_conv(plan.convs[step.conv], targets, device.memory()); }
+	else if (step.contract >= 0) { launch_contract(plan.contracts[step.contract], targets, device.memory()); }
+	else if (step.sum >= 0) { launch_sum(plan.sums[step.sum], targets, device.memory()); }
+	else if (step.parts >= 0 && step.group >= 0)
+	{
+		launch_group(plan.groups[step.group], targets, device.memory(), temps, &plan.part_products[step.parts], step.parts);
+	}
+	else if (step.parts >= 0) { launch_parts(plan.part_products[step.parts], targets, device.memory(), temps[step.parts]); }
+	else { launch_group(plan.groups[step.group], targets, device.memory(), temps); }
+}
+
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory)
 {
 	Observable* out = call.node;

@@ -7,6 +7,7 @@
 
 #include "eteq.hpp"
 #include "replay_eval.hpp"
+#include "timing_eval.hpp"
 #include "fuse_plan.hpp"
 #include "hone.hpp"
 
@@ -248,6 +249,7 @@ int tcr_set_evaluator (int kind)
 			case TCR_EVAL_REPLAY_UNFUSED: teq::set_eval(new eigen::ReplayEvaluator(1, 16, false)); break;
 			case TCR_EVAL_REPLAY_LAUNCHES: teq::set_eval(new eigen::ReplayEvaluator(1, 16, true, false)); break;
 			case TCR_EVAL_DEFAULT: teq::set_eval(nullptr); break;
+			case TCR_EVAL_TIMING: teq::set_eval(new eigen::TimingEvaluator()); break;
 			default: global::fatalf("unknown evaluator kind %d", kind);
 		}
 	});
@@ -267,6 +269,22 @@ int tcr_evaluator_stats (uint64_t out[6])
 			out[3] = st.skipped;
 			out[4] = st.launches;
 			out[5] = st.reserved_bytes;
+		}
+	});
+}
+
+int tcr_evaluator_timing (char* out, size_t capacity, size_t* needed)
+{
+	return guarded([&]
+	{
+		std::string text;
+		if (auto timing = dynamic_cast<eigen::TimingEvaluator*>(&teq::get_eval())) { text = timing->report(); }
+		if (needed) { *needed = text.size(); }
+		if (out && capacity)
+		{
+			size_t n = std::min(text.size(), capacity - 1);
+			memcpy(out, text.data(), n);
+			out[n] = '\0';
 		}
 	});
 }
@@ -450,43 +468,7 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 		teq::multi_visit(collector, key);
 		eigen::FusionPlan plan = eigen::plan_fusion(collector.funcs, tset);
 		std::stringstream ss;
-		for (auto& step : plan.steps)
-		{
-			if (nullptr != step.node)
-			{
-				ss << "node " << step.node->get_opcode().name_ << "\n";
-				continue;
-			}
-			if (step.contract >= 0)
-			{
-				ss << "swapped CONTRACT+PERMUTE\n";
-				continue;
-			}
-			if (step.sum >= 0)
-			{
-				ss << "summed CONTRACT x" << plan.sums[step.sum].a.size() << "\n";
-				continue;
-			}
-			if (step.parts >= 0 && step.group < 0)
-			{
-				ss << plan.part_products[step.parts].label << "\n";
-				continue;
-			}
-			if (step.conv >= 0)
-			{
-				ss << "viewed " << plan.convs[step.conv].label << "\n";
-				continue;
-			}
-			auto& group = plan.groups[step.group];
-			if (step.parts >= 0) { ss << plan.part_products[step.parts].label << " with epilogue "; }
-			ss << "group ";
-			for (size_t i = 0; i < group.members.size(); ++i)
-			{
-				ss << (i ? "+" : "") << group.members[i]->get_opcode().name_;
-			}
-			ss << " leaves=" << group.leaves.size() << " stores=" << group.outputs.size()
-				<< " instrs=" << group.program.size() << "\n";
-		}
+		for (auto& step : plan.steps) { ss << eigen::describe_step(plan, step) << "\n"; }
 		ss << "folded " << plan.absorbed.size() << "\n";
 		std::string text = ss.str();
 		if (needed) { *needed = text.size(); }

@@ -291,38 +291,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		RangeTempsT temps(fusion.part_products.size(), {nullptr, 0});
 		try
 		{
-			for (auto& step : fusion.steps)
-			{
-				if (nullptr != step.node)
-				{
-					device.calc_forced(*step.node, (size_t) (targets.count(step.node) > 0));
-				}
-				else if (step.conv >= 0)
-				{
-					launch_conv(fusion.convs[step.conv], targets, device.memory());
-				}
-				else if (step.contract >= 0)
-				{
-					launch_contract(fusion.contracts[step.contract], targets, device.memory());
-				}
-				else if (step.sum >= 0)
-				{
-					launch_sum(fusion.sums[step.sum], targets, device.memory());
-				}
-				else if (step.parts >= 0 && step.group >= 0)
-				{
-					launch_group(fusion.groups[step.group], targets, device.memory(), temps,
-						&fusion.part_products[step.parts], step.parts);
-				}
-				else if (step.parts >= 0)
-				{
-					launch_parts(fusion.part_products[step.parts], targets, device.memory(), temps[step.parts]);
-				}
-				else
-				{
-					launch_group(fusion.groups[step.group], targets, device.memory(), temps);
-				}
-			}
+			for (auto& step : fusion.steps) { launch_step(fusion, step, device, targets, temps); }
 		}
 		catch (const std::exception& err)
 		{

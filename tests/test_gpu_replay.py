@@ -1309,3 +1309,43 @@ def test_inputs_that_travel_with_the_launch(ctx):
     ctx.capture_feed(x.ptr, xs[0])
     with pytest.raises(capi.TcgError, match="written by a step"):
         ctx.capture_end()
+
+
+def test_timing_evaluator_runs_the_planned_launches_between_events():
+    """eigen::TimingEvaluator in the evaluator slot (the place of the reference's
+    dbg::PlugableEvaluator, dbg/peval/plugin_eval.hpp:21-42): the launches a
+    recording would hold, run one by one with an event on either side.  The
+    values are those of the recording's launches (held to the walk like them);
+    the report names every kind of launch with its count and device time."""
+    from tenncor_amd import graph, configs
+    results = {}
+    try:
+        for kind in ("plain", "timing"):
+            graph.set_evaluator(kind)
+            g = graph.Graph()
+            try:
+                targets, x, _, _ = configs.config4_lstm(g, seq=5, batch=64, nin=32, hid=64)
+                for _ in range(3):
+                    g.assign(x, g.data(x))
+                    g.evaluate(targets)
+                results[kind] = [t.get().copy() for t in targets]
+                if kind == "timing":
+                    report = graph.evaluator_timing()
+                    planned = [l for l in g.launch_plan(targets) if not l.startswith("folded")]
+            finally:
+                g.close()
+    finally:
+        graph.set_evaluator("default")
+    for a, b in zip(results["plain"], results["timing"]):
+        assert np.abs(a - b).max() <= 1e-5 * np.abs(a).max()
+    lines = report.splitlines()
+    assert lines[0].startswith("3 passes timed launch by launch (%d launches in the latest), 0 walked" % len(planned)), lines[0]
+    rows = {}
+    for line in lines[1:]:
+        head, _, what = line.partition(" us  ")
+        count, _, rest = head.strip().partition(" x ")
+        rows[what] = (int(count), float(rest.split("=")[1]))
+    # every planned launch is in the table, three times (one per pass), with a positive time
+    for what in set(planned):
+        assert rows[what][0] == 3 * planned.count(what) and rows[what][1] > 0, (what, rows.get(what))
+    assert any(" with epilogue group " in what for what in rows)
