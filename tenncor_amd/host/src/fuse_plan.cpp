@@ -18,6 +18,7 @@ namespace
 enum Kind { OTHER = 0, EW, VIEW };
 
 constexpr size_t max_members = 48;
+constexpr int far_behind = 32;  // positions in the pass between a launch and a node that could still join it
 
 struct View final
 {
@@ -1555,6 +1556,21 @@ struct Planner final
 			}
 			std::sort(cands.begin(), cands.end(), [&](int x, int y) { return maxpos_[x] > maxpos_[y]; });
 			cands.erase(std::unique(cands.begin(), cands.end()), cands.end());
+			// A node that stands far behind the launch its operands come from, and that only
+			// elementwise nodes of its shape read, waits for those readers instead: the factors
+			// the gradient builder derives from a forward value (1 - s, s (1 - s) of a gate,
+			// tenncor/eteq/backprop.hpp:58-560) stand with the backward pass.  Computed in the
+			// forward launch each is one more tensor stored there and loaded again much later;
+			// computed where it is read it costs an instruction and the forward value is
+			// stored once for all of them.
+			if (n.consumers.size() > 0 && std::all_of(n.consumers.begin(), n.consumers.end(), [&](int c)
+				{ return nodes_[c].kind == EW && nodes_[c].shape == n.shape && nodes_[c].op != egen::CONCAT; }))
+			{
+				cands.erase(std::remove_if(cands.begin(), cands.end(), [&](int cand)
+				{
+					return (int) i - maxpos_[find(cand)] > far_behind;
+				}), cands.end());
+			}
 			int self = (int) i;
 			for (int cand : cands)
 			{
