@@ -1483,12 +1483,20 @@ struct GfxTile
 // the tile with the least operand traffic among those that put a workgroup on every CU
 bool gfx_choose_tile (const tcg_ctx* ctx, uint64_t M, uint64_t J, int G, uint64_t ktot, bool trans_b, bool vec, GfxTile& out)
 {
+	// Eight waves, two on a SIMD.  Sixteen (TCG_GFX_WAVES=16: four on a SIMD, the upper
+	// eight handing their partial tiles to the lower eight first) were measured on the
+	// steps of a recurrent cell and are slower -- 256 x 2048 x 768: 10.4 -> 11.8 us,
+	// 256 x 512 x 2048: 12.2 -> 12.7 us: more loads in flight do not help, as with the
+	// loads held further ahead (see gfx_source)
 	int nw = 0;
-	for (int w : {8, 4, 2, 1})
+	static const int most = [] { const char* e = getenv("TCG_GFX_WAVES"); return e ? atoi(e) : 8; }();
+	for (int w : {16, 8, 4, 2, 1})
 	{
+		if (w > most || (w == 16 && ktot < 512)) { continue; }
 		if (ktot % (16 * (uint64_t) w) == 0) { nw = w; break; }
 	}
 	if (nw == 0) { return false; }
+	const int slots = nw < 8 ? nw : 8; // partial tiles that meet in LDS
 	double best = 0.0;
 	bool found = false;
 	for (int tm : {16, 32, 64})
@@ -1500,7 +1508,7 @@ bool gfx_choose_tile (const tcg_ctx* ctx, uint64_t M, uint64_t J, int G, uint64_
 			if (trans_b ? nc % 16 != 0 : nc % 64 != 0) { continue; }
 			const int accs = (tm / 16) * (nc / 16) * 4; // accumulator registers per lane
 			if (accs > 128) { continue; }
-			if ((size_t) nw * tm * nc * sizeof(float) > 65536) { continue; }
+			if ((size_t) slots * tm * nc * sizeof(float) > 65536) { continue; }
 			// a lane computes one element of the group, or 16-byte vectors of them when
 			// the tile holds more elements than the workgroup lanes; at most 8 per lane
 			int n = 1;
@@ -1545,6 +1553,7 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 	const int NT = 64 * t.NW, RB = t.TM / 16, NC = sh.G * t.TJ, CB = NC / 16, CG = NC / 64;
 	const uint32_t ktot = sh.KT * sh.nterms, KW = ktot / t.NW, NSTEPS = KW / 16;
 	const int BL = sh.trans_b ? CB : 4 * CG; // 128-bit loads of B per step and lane
+	const int SLOTS = t.NW < 8 ? t.NW : 8;   // partial tiles in LDS: waves 8.. hand theirs to waves 0..7 first
 	// The source names the loads of a step one step ahead of its arithmetic and leaves
 	// the order to the compiler, which sinks each load to just before its first use;
 	// with two waves on a SIMD that is the fastest form measured for the steps of a
@@ -1579,9 +1588,9 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 	// the steps on their way from memory wait in registers: the compiler may use the
 	// registers of a CU that holds at most two such workgroups, instead of keeping to
 	// the few that the largest number of resident waves would leave each of them
-	o << "extern \"C\" __global__ __launch_bounds__(" << NT << ") __attribute__((amdgpu_waves_per_eu(1, " << std::max(2, NT / 128)
+	o << "extern \"C\" __global__ __launch_bounds__(" << NT << ") __attribute__((amdgpu_waves_per_eu(1, " << std::min(4, std::max(2, NT / 128))
 		<< "))) void " << gfx_name(sh) << " (GfxArgs a)\n{\n"
-		"__shared__ __attribute__((aligned(16))) float red[" << t.NW * t.TM * NC << "];\n"
+		"__shared__ __attribute__((aligned(16))) float red[" << SLOTS * t.TM * NC << "];\n"
 		"const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);\n"
 		"const uint32_t r16 = lane & 15u, q = lane >> 4;\n";
 	// workgroups are dealt to the eight XCDs in turn: each XCD keeps a band of
@@ -1713,30 +1722,57 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 		o << "}\n";
 	}
 	// ---- the partial tiles meet in LDS: red[wave][row][column of the tile] ----
-	o << "{\nfloat* mine = red + wave * " << t.TM * NC << "u;\n";
-	for (int rb = 0; rb < RB; ++rb)
+	// park: a wave's partial tile goes to its slot; take: the tile in the slot is
+	// added to the wave's own (lane for lane what the other wave's lane left there)
+	auto exchange = [&](bool take)
 	{
-		for (int i = 0; i < 4; ++i)
+		o << "{\nfloat* mine = red + (wave & 7u) * " << t.TM * NC << "u;\n";
+		for (int rb = 0; rb < RB; ++rb)
 		{
-			if (sh.trans_b)
+			for (int i = 0; i < 4; ++i)
 			{
-				for (int cb = 0; cb < CB; ++cb)
+				if (sh.trans_b)
 				{
-					o << "mine[(" << rb * 16 + i << "u + 4u * q) * " << NC << "u + " << cb * 16 << "u + r16] = acc[" << rb << "][" << cb << "][" << i << "];\n";
+					for (int cb = 0; cb < CB; ++cb)
+					{
+						const std::string at = "mine[(" + std::to_string(rb * 16 + i) + "u + 4u * q) * " + std::to_string(NC) + "u + " +
+							std::to_string(cb * 16) + "u + r16]";
+						const std::string reg = "acc[" + std::to_string(rb) + "][" + std::to_string(cb) + "][" + std::to_string(i) + "]";
+						o << (take ? reg + " += " + at : at + " = " + reg) << ";\n";
+					}
 				}
-			}
-			else
-			{
-				for (int cg = 0; cg < CG; ++cg)
+				else
 				{
-					o << "{ f4 v; ";
-					for (int e = 0; e < 4; ++e) { o << "v[" << e << "] = acc[" << rb << "][" << cg * 4 + e << "][" << i << "]; "; }
-					o << "*(f4*) (mine + (" << rb * 16 + i << "u + 4u * q) * " << NC << "u + " << cg * 64 << "u + 4u * r16) = v; }\n";
+					for (int cg = 0; cg < CG; ++cg)
+					{
+						const std::string at = "*(f4*) (mine + (" + std::to_string(rb * 16 + i) + "u + 4u * q) * " + std::to_string(NC) + "u + " +
+							std::to_string(cg * 64) + "u + 4u * r16)";
+						o << "{ f4 v; ";
+						if (take) { o << "v = " << at << "; "; }
+						for (int e = 0; e < 4; ++e)
+						{
+							const std::string reg = "acc[" + std::to_string(rb) + "][" + std::to_string(cg * 4 + e) + "][" + std::to_string(i) + "]";
+							o << (take ? reg + " += v[" + std::to_string(e) + "]; " : "v[" + std::to_string(e) + "] = " + reg + "; ");
+						}
+						if (!take) { o << at << " = v; "; }
+						o << "}\n";
+					}
 				}
 			}
 		}
+		o << "}\n";
+	};
+	if (t.NW > 8)
+	{
+		o << "if (wave >= 8u)\n";
+		exchange(false);
+		o << "__syncthreads();\nif (wave < 8u)\n";
+		exchange(true);
+		o << "__syncthreads();\nif (wave < 8u)\n";
+		exchange(false);
 	}
-	o << "}\n__syncthreads();\n";
+	else { exchange(false); }
+	o << "__syncthreads();\n";
 	for (int it = 0; it < per_lane; ++it)
 	{
 		const std::string x = "_" + std::to_string(it);
@@ -1748,7 +1784,7 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 			for (int e = 0; e < t.N; ++e)
 			{
 				o << "{ float s = at[" << e << "];";
-				for (int w = 1; w < t.NW; ++w) { o << " s += at[" << w * t.TM * NC + e << "];"; }
+				for (int w = 1; w < SLOTS; ++w) { o << " s += at[" << w * t.TM * NC + e << "];"; }
 				o << " l" << k << x << "[" << e << "] = s; }\n";
 			}
 			o << "}\n";
