@@ -1561,7 +1561,11 @@ std::string gfx_source (const GfxShape& sh, const GfxTile& t, const FxArgs& p, c
 	// barriers made the 256 x 2048 x 768 step slower (10.4 -> 13.0 .. 16.0 us) and left
 	// the 256 x 512 x 2048 one where it was (12.2 us): with the arithmetic taken out the
 	// loads alone take 8.0 and 12.1 us, so what bounds these tiles is how fast the
-	// operands come out of L2, not how long a single load takes.
+	// operands come out of L2, not how long a single load takes.  Steps of 32 summed
+	// indices, in which a lane reads whole 128-byte lines of a K-contiguous operand,
+	// changed neither (10.1 and 12.3 us); leading dimensions padded by 32 floats, which
+	// spread the rows of such an operand over the channels, took the second to 9.0 us,
+	// but the operands of a step are the caller's buffers and keep their layout.
 	int depth = 2;
 	if ((uint32_t) depth > NSTEPS) { depth = (int) NSTEPS; }
 	const uint32_t tiles_m = (sh.M + t.TM - 1) / t.TM, tiles_j = sh.J / t.TJ;
