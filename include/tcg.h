@@ -198,6 +198,28 @@ int tcg_capture_begin_small (tcg_ctx* ctx);
 int tcg_capture_feed (tcg_ctx* ctx, const void* devptr, size_t bytes, const void* host);
 int tcg_graph_feed (tcg_ctx* ctx, tcg_graph* graph, const void* devptr, const void* host, size_t bytes);
 int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph);
+/* The small launches of a LONGER sequence, a few at a time (the dense layer and
+ * the softmax behind a convolutional network: a dozen launches over a few
+ * thousand elements each).  After tcg_batch_begin the entry points named for
+ * tcg_capture_begin_small hold their work back as a step when one workgroup
+ * does it in a few hundred iterations; tcg_batch_end sends the steps held so
+ * far out as ONE kernel on the context's stream (a recording of the stream
+ * holds it as one node) and ends the batch.  A call of one of those entry
+ * points that cannot be a step sends the held steps out first, ends the batch
+ * and runs as itself, so the order of the work is kept; a batch that grows past
+ * what one workgroup does in microseconds goes out and a new one starts.  Any
+ * OTHER entry point must not be called between begin and end (its launch would
+ * overtake the steps held back); tcg_sync, tcg_d2h, tcg_capture_end and
+ * tcg_graph_launch end an open batch first.  The buffers the steps name must
+ * stay allocated until the batch is sent.  Steps compute what they compute in
+ * a single-launch recording (see there for the summation orders), except that
+ * a reduction with fewer outputs than lanes folds each output as 2..64
+ * interleaved ascending folds combined by halves.  Both calls
+ * may be repeated: begin inside a batch and end outside one do nothing.  No
+ * counterpart in the reference: its evaluator calls one Eigen expression per
+ * node (internal/teq/evaluator.hpp:35-62) and has no launches to save. */
+int tcg_batch_begin (tcg_ctx* ctx);
+int tcg_batch_end (tcg_ctx* ctx);
 int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr);
 int tcg_graph_stats (const tcg_graph* graph, uint64_t* nodes, uint64_t* arena_bytes);
 int tcg_graph_destroy (tcg_ctx* ctx, tcg_graph* graph);

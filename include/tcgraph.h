@@ -83,10 +83,13 @@ int tcr_sync (tcr_graph* g);
  * time it is evaluated and enqueues the recording as a whole afterwards, with
  * elementwise functors that feed one another computed in shared launches, and
  * the whole pass of a graph of small tensors (4096 elements at most each) as
- * the steps of one kernel (tcg_capture_begin_small: sums then run in index
+ * the steps of one kernel (tcg_capture_begin_small: sums then run in another
  * order, equal to the walk's within the tolerance of reductions and
- * contractions rather than bit for bit);
- * TCR_EVAL_REPLAY_LAUNCHES is the same without such single-kernel passes:
+ * contractions rather than bit for bit); in a larger graph, runs of launches
+ * over at most 16384 elements each (the dense layer and the loss behind a
+ * convolutional network) go out as one kernel per run in the same way
+ * (tcg_batch_begin; TCR_BATCHES=0 in the environment keeps them apart);
+ * TCR_EVAL_REPLAY_LAUNCHES is the same without such single-kernel passes and runs:
  * every value equals the walk's bit for bit;
  * TCR_EVAL_REPLAY_UNFUSED records one launch per functor, as the walk issues. */
 #define TCR_EVAL_PLAIN 0
@@ -158,8 +161,10 @@ int tcr_count_functors (tcr_graph* g, int nnodes, const int* nodes, int* count);
  * a launch, or "swapped CONTRACT+PERMUTE" for a transposed matrix product
  * launched as the product with its operands exchanged, or "padded PAD+CONV"
  * ("padded PAD+CONV+SLICE" when only slices read the result) for a convolution
- * computed from the operand of its PAD node; a last line "folded N" counts the functors that never hold a value
- * of their own. Returns the length the text needs (it is cut to `capacity`). */
+ * computed from the operand of its PAD node; a line "batch N" says that the N
+ * lines behind it are steps over a few thousand elements each that go out as
+ * ONE launch (tcg_batch_begin); a last line "folded N" counts the functors that
+ * never hold a value of their own. Returns the length the text needs (it is cut to `capacity`). */
 int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, size_t capacity, size_t* needed);
 
 /* ---- graph clean-up (tenncor/hone/optimize.hpp:19-38: `hone::optimize(roots, rulestream)`) ----

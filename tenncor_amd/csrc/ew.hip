@@ -351,7 +351,11 @@ extern "C" {
 static int small_elementwise (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, int nargs,
 	const void* const* ins, void* out)
 {
-	if (nargs > TCG_FX_MAX_LEAVES && false == tcg_small_mode(ctx))
+	if (nargs > TCG_FX_MAX_LEAVES && tcg_small_mode(ctx))
+	{
+		TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "an elementwise node with that many operands"));
+	}
+	if (nargs > TCG_FX_MAX_LEAVES)
 	{
 		// a long fold: sixteen operands, then the result so far with fifteen more, ...
 		int rc = small_elementwise(ctx, opcode, dtype, n, TCG_FX_MAX_LEAVES, ins, out);
@@ -365,7 +369,6 @@ static int small_elementwise (tcg_ctx* ctx, int opcode, int dtype, uint64_t n, i
 		}
 		return rc;
 	}
-	if (nargs > TCG_FX_MAX_LEAVES) { return tcg_small_unsupported(ctx, "an elementwise node with that many operands"); }
 	uint64_t shape[8] = {n, 1, 1, 1, 1, 1, 1, 1};
 	tcg_fx_leaf leaves[TCG_FX_MAX_LEAVES];
 	memset(leaves, 0, sizeof(leaves));

@@ -866,7 +866,8 @@ int fusedx_jit_launch (tcg_ctx* ctx, int dtype, FxArgs& p, bool vec)
 // that one workgroup finishes in microseconds; anything else refuses the
 // recording and the caller records the sequence launch by launch.
 
-constexpr int PASS_BLOCK = 256;
+constexpr int PASS_BLOCK = 256;    // lanes of a whole pass
+constexpr int BATCH_BLOCK = 1024;  // lanes of a batch: its steps are a few thousand elements each
 constexpr uint64_t PASS_MAX_WORK = 4096;  // iterations of the busiest lane, all steps together
 constexpr size_t PASS_MAX_STEPS = 256;
 
@@ -887,6 +888,14 @@ struct tcg_small_pass
 {
 	std::vector<PassStep> steps;
 	uint64_t work = 0;
+	size_t ptr_bound = 0;  // pointers the steps name, counted with repeats
+	// batches: blocks handed out since the batch began (or was last sent): the
+	// bytes asked for, whether a caller still owns them, and whether the block
+	// had an owner before (it was given back inside the batch by somebody who took
+	// it earlier: steps held back may still read what that owner left in memory)
+	struct Born { size_t bytes = 0; bool live = false; bool used_before = false; };
+	std::map<const void*,Born> born;
+	std::set<const void*> given_back; // blocks not born here that were given back here
 	hipFunction_t fn = nullptr;
 	// the kernel's argument block: pointers, then the bytes of the buffers whose
 	// content the caller supplies with every launch
@@ -899,21 +908,55 @@ struct tcg_small_pass
 namespace
 {
 
-int small_charge (tcg_ctx* ctx, uint64_t items, uint64_t per_item)
+// lanes of a wave that fold one output of a reduction between them: few outputs,
+// each over many elements
+uint32_t reduce_share (uint64_t nout, uint64_t R, uint64_t block)
 {
-	tcg_small_pass* pass = ctx->capturing->pass;
-	uint64_t cost = (items + PASS_BLOCK - 1) / PASS_BLOCK * (per_item ? per_item : 1);
-	if (pass->steps.size() >= PASS_MAX_STEPS || pass->work + cost > PASS_MAX_WORK)
+	uint32_t share = 1;
+	while (share < 64 && share * 2 <= R && nout * share * 2 <= block) { share *= 2; }
+	return share;
+}
+
+// the steps being collected: those of a batch, or of the single-launch recording
+tcg_small_pass* small_current (tcg_ctx* ctx)
+{
+	return ctx->batch ? ctx->batch : ctx->capturing->pass;
+}
+
+// a step of a batch stays below what a launch of its own would cost; a batch that
+// is full goes out and the next one starts
+constexpr uint64_t BATCH_MAX_STEP_WORK = 512;
+constexpr size_t BATCH_MAX_PTRS = 384;
+
+int small_charge (tcg_ctx* ctx, uint64_t items, uint64_t per_item, size_t nptrs)
+{
+	tcg_small_pass* pass = small_current(ctx);
+	const uint64_t lanes = ctx->batch ? BATCH_BLOCK : PASS_BLOCK;
+	uint64_t cost = (items + lanes - 1) / lanes * (per_item ? per_item : 1);
+	if (ctx->batch)
+	{
+		if (cost > BATCH_MAX_STEP_WORK)
+		{
+			return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "too much work for a step of a batch");
+		}
+		if (pass->steps.size() >= PASS_MAX_STEPS || pass->work + cost > PASS_MAX_WORK || pass->ptr_bound + nptrs > BATCH_MAX_PTRS)
+		{
+			int rc = tcg_batch_send(ctx);
+			if (rc != TCG_OK) { return rc; }
+		}
+	}
+	else if (pass->steps.size() >= PASS_MAX_STEPS || pass->work + cost > PASS_MAX_WORK)
 	{
 		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "the sequence is too long for a single-launch pass");
 	}
 	pass->work += cost;
+	pass->ptr_bound += nptrs;
 	return TCG_OK;
 }
 
 int small_append_fx (tcg_ctx* ctx, int dtype, const FxArgs& p)
 {
-	int rc = small_charge(ctx, p.total, p.ninstr);
+	int rc = small_charge(ctx, p.total, p.ninstr, p.nleaf + p.nout);
 	if (rc != TCG_OK) { return rc; }
 	PassStep step;
 	memset(&step, 0, sizeof(step));
@@ -921,13 +964,14 @@ int small_append_fx (tcg_ctx* ctx, int dtype, const FxArgs& p)
 	step.dtype = dtype;
 	step.fx = p;
 	fx_dense_leaves(p, step.dense);
-	ctx->capturing->pass->steps.push_back(step);
+	small_current(ctx)->steps.push_back(step);
 	return TCG_OK;
 }
 
 // resolve: the expression the kernel uses for a device pointer of the recording
 template <typename Resolve>
-std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_t feed_bytes, size_t lds_bytes, Resolve resolve)
+std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_t feed_bytes, size_t lds_bytes, Resolve resolve,
+	const int block = PASS_BLOCK)
 {
 	std::ostringstream o;
 	fx_emit_prelude(o);
@@ -936,7 +980,13 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 		"if constexpr (is_int<T>::value) { typedef typename wide_unsigned<T>::type W; return (T) ((W) a * (W) b + (W) acc); }\n"
 		"else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, acc); }\n"
 		"else { return __builtin_fma(a, b, acc); }\n}\n"
-		"extern \"C\" __global__ __launch_bounds__(" << PASS_BLOCK << ") void fx (PassPtrs P)\n{\n";
+		// the value of lane (lane ^ m) of the wave
+		"template <typename T> __device__ __forceinline__ T pass_xor (T v, int m)\n{\n"
+		"const int from = (int) (((threadIdx.x & 63u) ^ (uint32_t) m) << 2);\n"
+		"if constexpr (sizeof(T) == 8) { union { T t; int w[2]; } u; u.t = v; u.w[0] = __builtin_amdgcn_ds_bpermute(from, u.w[0]); "
+		"u.w[1] = __builtin_amdgcn_ds_bpermute(from, u.w[1]); return u.t; }\n"
+		"else { union { T t; int w; } u; u.w = 0; u.t = v; u.w = __builtin_amdgcn_ds_bpermute(from, u.w); return u.t; }\n}\n"
+		"extern \"C\" __global__ __launch_bounds__(" << block << ") void fx (PassPtrs P)\n{\n";
 	if (lds_bytes) { o << "__shared__ __attribute__((aligned(256))) char lds[" << lds_bytes << "];\n"; }
 	// fed buffers are read where the launch put them: in the argument block
 	o << "const char* feed = (const char*) __builtin_amdgcn_kernarg_segment_ptr() + " << std::max<size_t>(1, nptrs) * sizeof(void*) << ";\n";
@@ -963,7 +1013,7 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 			FxBake bake;
 			for (uint32_t k = 0; k < s.fx.nleaf; ++k) { bake.leaf_ptr[k] = resolve(s.fx.leaf[k].ptr); }
 			for (uint32_t k = 0; k < s.fx.nout; ++k) { bake.out_ptr[k] = resolve(s.fx.out[k]); }
-			o << "for (uint32_t idx = threadIdx.x; idx < " << s.fx.total << "u; idx += " << PASS_BLOCK << ")\n{\n";
+			o << "for (uint32_t idx = threadIdx.x; idx < " << s.fx.total << "u; idx += " << block << ")\n{\n";
 			fx_emit_body(o, 1, s.fx, s.dense, &bake);
 			o << "}\n";
 		}
@@ -972,10 +1022,13 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 			const PassContract& c = s.ct;
 			o << "const T* a = (const T*) " << resolve(c.a) << "; const T* b = (const T*) " << resolve(c.b)
 				<< "; T* out = (T*) " << resolve(c.out) << ";\n"
-				"for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << PASS_BLOCK << ")\n{\n"
+				"for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << block << ")\n{\n"
 				"uint32_t rem = o; int64_t ao = 0, bo = 0;\n";
 			decompose("rem", c.nod, c.osize, {{"ao", c.oastr}, {"bo", c.obstr}});
+			// unrolled so that the loads of several terms are in flight together; the
+			// sum itself stays one chain in ascending order
 			o << "T acc = (T) 0;\n"
+				"#pragma unroll 16\n"
 				"for (uint32_t k = 0; k < " << c.K << "u; ++k)\n{\n"
 				"uint32_t r = k; int64_t ak = ao, bk = bo;\n";
 			decompose("r", c.nkd, c.ksize, {{"ak", c.kastr}, {"bk", c.kbstr}});
@@ -985,16 +1038,42 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 		else
 		{
 			const PassReduce& c = s.rd;
-			o << "const T* in = (const T*) " << resolve(c.in) << "; T* out = (T*) " << resolve(c.out) << ";\n"
-				"for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << PASS_BLOCK << ")\n{\n"
-				"uint32_t rem = o; int64_t base = 0;\n";
-			decompose("rem", c.nod, c.osize, {{"base", c.oistr}});
-			o << "T acc = in[base];\n"
-				"for (uint32_t k = 1; k < " << c.R << "u; ++k)\n{\n"
-				"uint32_t r = k; int64_t off = base;\n";
-			decompose("r", c.nrd, c.rsize, {{"off", c.ristr}});
-			o << "acc = apply_binary<T>(" << s.opcode << ", acc, in[off]);\n}\n"
-				"out[o] = acc;\n}\n";
+			o << "const T* in = (const T*) " << resolve(c.in) << "; T* out = (T*) " << resolve(c.out) << ";\n";
+			// few outputs, each over many elements: `share` lanes of a wave fold one output
+			// between them (each every share-th element, ascending) and combine by halves
+			// (batches only: a whole pass folds in ascending order, like the kernels its
+			// results are compared with bit for bit at these sizes)
+			const uint32_t share = block == BATCH_BLOCK ? reduce_share(c.nout, c.R, (uint64_t) block) : 1;
+			if (share > 1)
+			{
+				o << "const uint32_t sub = threadIdx.x % " << share << "u, grp = threadIdx.x / " << share << "u;\n"
+					"for (uint32_t o0 = 0; o0 < " << c.nout << "u; o0 += " << block / share << "u)\n{\n"
+					"const uint32_t o = o0 + grp; const bool live = o < " << c.nout << "u;\n"
+					"T acc = (T) 0;\n"
+					"if (live)\n{\n"
+					"uint32_t rem = o; int64_t base = 0;\n";
+				decompose("rem", c.nod, c.osize, {{"base", c.oistr}});
+				o << "#pragma unroll 4\n"
+					"for (uint32_t k = sub; k < " << c.R << "u; k += " << share << "u)\n{\n"
+					"uint32_t r = k; int64_t off = base;\n";
+				decompose("r", c.nrd, c.rsize, {{"off", c.ristr}});
+				o << "acc = k == sub ? in[off] : apply_binary<T>(" << s.opcode << ", acc, in[off]);\n}\n}\n"
+					"for (int m = " << share / 2 << "; m >= 1; m >>= 1) { acc = apply_binary<T>(" << s.opcode << ", acc, pass_xor<T>(acc, m)); }\n"
+					"if (live && sub == 0) { out[o] = acc; }\n}\n";
+			}
+			else
+			{
+				o << "for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << block << ")\n{\n"
+					"uint32_t rem = o; int64_t base = 0;\n";
+				decompose("rem", c.nod, c.osize, {{"base", c.oistr}});
+				o << "T acc = in[base];\n"
+					"#pragma unroll 8\n"
+					"for (uint32_t k = 1; k < " << c.R << "u; ++k)\n{\n"
+					"uint32_t r = k; int64_t off = base;\n";
+				decompose("r", c.nrd, c.rsize, {{"off", c.ristr}});
+				o << "acc = apply_binary<T>(" << s.opcode << ", acc, in[off]);\n}\n"
+					"out[o] = acc;\n}\n";
+			}
 		}
 		o << "}\n";
 	}
@@ -1108,6 +1187,123 @@ int tcg_small_finish (tcg_ctx* ctx, tcg_graph* g)
 	return TCG_OK;
 }
 
+// ---- batches: the small launches of a longer sequence, a few at a time ----------
+//
+// The same steps, collected between tcg_batch_begin and tcg_batch_end wherever
+// the caller allows it.  All their buffers are reached through pointers (the
+// buffers outlive the batch); the kernel is launched on the context's stream
+// like any other, so a recording of the stream holds it as one node.
+
+int tcg_batch_send (tcg_ctx* ctx)
+{
+	tcg_small_pass* pass = ctx->batch;
+	if (nullptr == pass || pass->steps.empty()) { return TCG_OK; }
+	// A block that was handed out and taken back since the batch began is read and
+	// written by these steps alone: it lives in LDS.  Everything else is reached
+	// through a pointer argument.
+	constexpr size_t lds_cap = 48u << 10;
+	std::map<const void*,size_t> lds_offset;
+	size_t lds_bytes = 0;
+	std::map<const void*,size_t> slot;
+	auto resolve = [&](const void* ptr) -> std::string
+	{
+		auto it = pass->born.upper_bound(ptr);
+		if (it != pass->born.begin())
+		{
+			--it;
+			const char* begin = (const char*) it->first;
+			if ((const char*) ptr < begin + it->second.bytes && false == it->second.live && false == it->second.used_before)
+			{
+				auto at = lds_offset.find(it->first);
+				size_t bytes = (it->second.bytes + 255) & ~(size_t) 255;
+				if (at == lds_offset.end() && lds_bytes + bytes <= lds_cap)
+				{
+					at = lds_offset.emplace(it->first, lds_bytes).first;
+					lds_bytes += bytes;
+				}
+				if (at != lds_offset.end())
+				{
+					return "((void*) (lds + " + std::to_string(at->second + (size_t) ((const char*) ptr - begin)) + "))";
+				}
+			}
+		}
+		auto at = slot.find(ptr);
+		if (at == slot.end()) { at = slot.emplace(ptr, slot.size()).first; }
+		return "P.p[" + std::to_string(at->second) + "]";
+	};
+	// two passes: the first finds out how much LDS and how many pointers there are
+	(void) pass_source(pass->steps, 1, 0, 0, resolve, BATCH_BLOCK);
+	std::string source = pass_source(pass->steps, slot.size(), 0, lds_bytes, resolve, BATCH_BLOCK);
+	hipFunction_t fn = nullptr;
+	FxJit& jit = fx_jit();
+	{
+		std::lock_guard<std::mutex> lock(jit.mu);
+		auto it = jit.kernels.find(source);
+		if (it == jit.kernels.end())
+		{
+			int rc = fx_compile(ctx, source, &fn);
+			if (rc != TCG_OK) { return rc; }
+			jit.kernels.emplace(source, fn);
+		}
+		else { fn = it->second; }
+	}
+	// the argument block: the pointers, then the (unused) 16 bytes of fed values
+	std::vector<void*> args(std::max<size_t>(1, slot.size()) + 2, nullptr);
+	for (auto& kv : slot) { args[kv.second] = const_cast<void*>(kv.first); }
+	size_t size = args.size() * sizeof(void*);
+	void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+	pass->steps.clear();
+	pass->work = 0;
+	pass->ptr_bound = 0;
+	pass->born.clear(); // what lives on from here holds its values in memory
+	pass->given_back.clear();
+	TCG_HIP(ctx, hipModuleLaunchKernel(fn, 1, 1, 1, BATCH_BLOCK, 1, 1, 0, ctx->stream, nullptr, config));
+	return TCG_OK;
+}
+
+int tcg_batch_decline (tcg_ctx* ctx)
+{
+	int rc = tcg_batch_send(ctx);
+	delete ctx->batch;
+	ctx->batch = nullptr;
+	return rc;
+}
+
+void tcg_batch_note_alloc (tcg_ctx* ctx, const void* ptr, size_t bytes)
+{
+	auto& entry = ctx->batch->born[ptr];
+	entry.bytes = std::max(entry.bytes, bytes);
+	entry.live = true;
+	entry.used_before = entry.used_before || ctx->batch->given_back.count(ptr) > 0;
+}
+
+void tcg_batch_note_free (tcg_ctx* ctx, const void* ptr)
+{
+	auto it = ctx->batch->born.find(ptr);
+	if (it != ctx->batch->born.end()) { it->second.live = false; }
+	else { ctx->batch->given_back.insert(ptr); }
+}
+
+void tcg_batch_discard (tcg_ctx* ctx)
+{
+	delete ctx->batch;
+	ctx->batch = nullptr;
+}
+
+extern "C" int tcg_batch_begin (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	// a single-launch recording already takes every call as a step
+	if (nullptr == ctx->batch && false == (ctx->capturing && ctx->capturing->small)) { ctx->batch = new tcg_small_pass(); }
+	return TCG_OK;
+}
+
+extern "C" int tcg_batch_end (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	return ctx->batch ? tcg_batch_decline(ctx) : TCG_OK;
+}
+
 int tcg_small_launch (tcg_ctx* ctx, tcg_graph* g)
 {
 	tcg_small_pass* pass = g->pass;
@@ -1196,12 +1392,12 @@ int tcg_small_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8], const
 			nout *= shape[d];
 		}
 	}
-	TCG_REQUIRE(ctx, nout < (1ull << 31) && K < (1ull << 31), "tcg_contract: too large");
+	if (nout >= (1ull << 31) || K >= (1ull << 31)) { return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_contract: too large for a step"); }
 	c.nout = (uint32_t) nout;
 	c.K = (uint32_t) K;
-	int rc = small_charge(ctx, nout, K);
+	int rc = small_charge(ctx, nout, K, 3);
 	if (rc != TCG_OK) { return rc; }
-	ctx->capturing->pass->steps.push_back(step);
+	small_current(ctx)->steps.push_back(step);
 	return TCG_OK;
 }
 
@@ -1242,12 +1438,13 @@ int tcg_small_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[
 		}
 		stride *= (int64_t) shape[d];
 	}
-	TCG_REQUIRE(ctx, nout < (1ull << 31) && R < (1ull << 31), "tcg_reduce: too large");
+	if (nout >= (1ull << 31) || R >= (1ull << 31)) { return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_reduce: too large for a step"); }
 	c.nout = (uint32_t) nout;
 	c.R = (uint32_t) R;
-	int rc = small_charge(ctx, nout, R);
+	const uint32_t share = ctx->batch ? reduce_share(nout, R, BATCH_BLOCK) : 1;
+	int rc = small_charge(ctx, nout * share, (R + share - 1) / share + (share > 1 ? 8 : 0), 2);
 	if (rc != TCG_OK) { return rc; }
-	ctx->capturing->pass->steps.push_back(step);
+	small_current(ctx)->steps.push_back(step);
 	return TCG_OK;
 }
 
@@ -1449,7 +1646,7 @@ extern "C" int tcg_ew_fusedx (tcg_ctx* ctx, int dtype, const uint64_t shape[8],
 	{
 		TCG_REQUIRE(ctx, 0 == leaves[k].from_product, "tcg_ew_fusedx: leaf %d names a matrix product (tcg_gemm_terms_fx takes such groups)", k);
 	}
-	if (tcg_small_mode(ctx)) { return small_append_fx(ctx, dtype, p); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, small_append_fx(ctx, dtype, p)); }
 	if (fx_jit_enabled() || false == tcg_default_dtype(dtype)) { return fusedx_jit_launch(ctx, dtype, p, vec); }
 	TCG_DISPATCH_TYPE(ctx, dtype, return fusedx_launch<T>(ctx, p, vec)); // the interpreter: double, float, int32
 	return TCG_OK;
@@ -1819,7 +2016,7 @@ extern "C" int tcg_gemm_terms_fx (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t 
 	{
 		return tcg_fail(ctx, TCG_ERR_UNSUPPORTED, "tcg_gemm_terms_fx: %s", why);
 	};
-	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a matrix product with an epilogue"); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "a matrix product with an epilogue")); }
 	if (dtype != TCG_FLOAT || trans_a) { return unsupported("fp32 products with a row-major first operand only"); }
 	if (nterms > 8 || K < 16 || K % 16 != 0 || M < 1 || N < 4 || M >= (1ull << 31) || N >= (1ull << 31) || K * (uint64_t) nterms >= (1ull << 31))
 	{

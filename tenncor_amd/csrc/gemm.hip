@@ -276,9 +276,9 @@ int tcg_matmul (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 	}
 	if (tcg_small_mode(ctx))
 	{
-		if (batch != 1) { return tcg_small_unsupported(ctx, "a batched matrix product"); }
 		const uint64_t pair[2] = {0, 1};
-		return tcg_small_contract(ctx, dtype, ashape, bshape, 1, pair, a, b, out);
+		TCG_SMALL_RETURN(ctx, batch != 1 ? tcg_small_unsupported(ctx, "a batched matrix product") :
+			tcg_small_contract(ctx, dtype, ashape, bshape, 1, pair, a, b, out));
 	}
 	return tcg_gemm(ctx, dtype, M, N, K, batch, a, K, M * K, 0, b, N, K * N, 0, out, N, M * N);
 }
@@ -315,7 +315,7 @@ int tcg_contract (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 			sorted[2 * p] = pa[p];
 			sorted[2 * p + 1] = pb[p];
 		}
-		return tcg_small_contract(ctx, dtype, ashape, bshape, npairs, sorted, a, b, out);
+		TCG_SMALL_RETURN(ctx, tcg_small_contract(ctx, dtype, ashape, bshape, npairs, sorted, a, b, out));
 	}
 	for (int d = 0; d < 8; ++d)
 	{
@@ -401,7 +401,7 @@ int tcg_contract_sum (tcg_ctx* ctx, int dtype, const uint64_t ashape[8],
 	TCG_REQUIRE(ctx, nterms >= 1, "tcg_contract_sum: %d terms", nterms);
 	TCG_REQUIRE(ctx, npairs >= 1 && npairs <= 8, "tcg_contract_sum: %d dimension pairs", npairs);
 	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, a[t] && b[t], "tcg_contract_sum: operand of term %d is NULL", t); }
-	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a sum of contractions"); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "a sum of contractions")); }
 	const size_t esz = tcg_type_size(dtype);
 	TCG_REQUIRE(ctx, esz != 0, "tcg_contract_sum: unknown dtype %d", dtype);
 	// the shape of every term as a matrix product (the rules of tcg_contract)
@@ -470,7 +470,7 @@ int tcg_gemm_terms (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint64_t K,
 	TCG_REQUIRE(ctx, nterms >= 1, "tcg_gemm_terms: %d terms", nterms);
 	TCG_REQUIRE(ctx, ldc >= N, "tcg_gemm_terms: ldc %llu < N %llu", (unsigned long long) ldc, (unsigned long long) N);
 	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, A[t] && B[t], "tcg_gemm_terms: operand of term %d is NULL", t); }
-	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a sum of matrix products"); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "a sum of matrix products")); }
 	const size_t esz = tcg_type_size(dtype);
 	TCG_REQUIRE(ctx, esz != 0, "tcg_gemm_terms: unknown dtype %d", dtype);
 	if (M == 0 || N == 0) { return TCG_OK; }
@@ -513,7 +513,7 @@ int tcg_gemm_terms_grid (tcg_ctx* ctx, int dtype, int mparts, const uint64_t* Mp
 	TCG_REQUIRE(ctx, ldc >= N, "tcg_gemm_terms_grid: ldc %llu < N %llu", (unsigned long long) ldc, (unsigned long long) N);
 	for (int i = 0; i < mparts * nterms; ++i) { TCG_REQUIRE(ctx, A[i], "tcg_gemm_terms_grid: operand A[%d] is NULL", i); }
 	for (int j = 0; j < nparts * nterms; ++j) { TCG_REQUIRE(ctx, B[j], "tcg_gemm_terms_grid: operand B[%d] is NULL", j); }
-	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "a sum of matrix products"); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "a sum of matrix products")); }
 	TCG_REQUIRE(ctx, tcg_type_size(dtype) != 0, "tcg_gemm_terms_grid: unknown dtype %d", dtype);
 	if (dtype == TCG_FLOAT)
 	{
@@ -555,7 +555,7 @@ int tcg_gemm_terms_ranges (tcg_ctx* ctx, int dtype, uint64_t M, uint64_t N, uint
 	TCG_REQUIRE(ctx, A && B && lda && ldb && ranges, "tcg_gemm_terms_ranges: NULL pointer");
 	TCG_REQUIRE(ctx, nterms >= 1, "tcg_gemm_terms_ranges: %d terms", nterms);
 	for (int t = 0; t < nterms; ++t) { TCG_REQUIRE(ctx, A[t] && B[t], "tcg_gemm_terms_ranges: operand of term %d is NULL", t); }
-	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "the K ranges of a matrix product"); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "the K ranges of a matrix product")); }
 	bool handled = false;
 	if (dtype == TCG_FLOAT && nranges >= 2)
 	{

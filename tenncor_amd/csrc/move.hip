@@ -328,11 +328,11 @@ int run_plan (tcg_ctx* ctx, CopyPlan& p, const T* src, T* dst, const char* what)
 			lo[d] = p.box ? p.lo[d] : 0;
 			hi[d] = p.box ? p.hi[d] : p.size[d];
 		}
-		if (false == dense_dst) { return tcg_small_unsupported(ctx, "a copy into a strided destination"); }
 		// a copy: any dtype of this element size will do
 		int dtype = std::is_same<T,double>::value ? TCG_DOUBLE : std::is_same<T,float>::value ? TCG_FLOAT :
 			sizeof(T) == 4 ? TCG_INT32 : sizeof(T) == 2 ? TCG_UINT16 : TCG_UINT8;
-		return tcg_small_copy(ctx, dtype, p.nd, size, p.sstride, p.sbase, lo, hi, src, dst);
+		TCG_SMALL_RETURN(ctx, false == dense_dst ? tcg_small_unsupported(ctx, "a copy into a strided destination") :
+			tcg_small_copy(ctx, dtype, p.nd, size, p.sstride, p.sbase, lo, hi, src, dst));
 	}
 	constexpr int N = Vec16<T>::N;
 	// transpose path: destination contiguous along dim 0, source along dim j

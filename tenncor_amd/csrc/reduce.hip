@@ -643,7 +643,7 @@ int tcg_reduce (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shape[8],
 	TCG_REQUIRE(ctx, shape && in && out, "tcg_reduce: NULL pointer");
 	TCG_REQUIRE(ctx, rankmask < 256, "tcg_reduce: rank set 0x%x names a dim >= 8", rankmask);
 	if (tcg_n_elems(shape) == 0) { return TCG_OK; }
-	if (tcg_small_mode(ctx)) { return tcg_small_reduce(ctx, opcode, dtype, shape, rankmask, in, out); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_reduce(ctx, opcode, dtype, shape, rankmask, in, out)); }
 	PoolScratch mem;
 	return reduce_any(ctx, mem, opcode, dtype, shape, rankmask, in, out);
 }
@@ -655,7 +655,7 @@ int tcg_reduce_noalloc (tcg_ctx* ctx, int opcode, int dtype, const uint64_t shap
 	TCG_REQUIRE(ctx, opcode >= TCG_REDUCE_SUM && opcode <= TCG_REDUCE_MAX, "tcg_reduce_noalloc: opcode %d is not a reduction", opcode);
 	TCG_REQUIRE(ctx, shape && in && out, "tcg_reduce_noalloc: NULL pointer");
 	TCG_REQUIRE(ctx, rankmask < 256, "tcg_reduce_noalloc: rank set 0x%x names a dim >= 8", rankmask);
-	if (tcg_small_mode(ctx)) { return tcg_small_unsupported(ctx, "tcg_reduce_noalloc"); }
+	if (tcg_small_mode(ctx)) { TCG_SMALL_RETURN(ctx, tcg_small_unsupported(ctx, "tcg_reduce_noalloc")); }
 	unsigned char* base = ctx->device >= 0 && ctx->device < MAX_DEVICES ? g_scratch[ctx->device] : nullptr;
 	if (nullptr == base) { return tcg_fail(ctx, TCG_ERR_HIP, "tcg_reduce_noalloc: no scratch memory on device %d", ctx->device); }
 	if (tcg_n_elems(shape) == 0) { return TCG_OK; }

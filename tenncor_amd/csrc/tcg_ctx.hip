@@ -126,6 +126,7 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_OK; }
 	(void) hipSetDevice(ctx->device);
+	tcg_batch_discard(ctx);
 	(void) tcg_release(ctx);
 	(void) hipStreamSynchronize(ctx->stream);
 	tcg_reduce_scratch_release(ctx);
@@ -166,6 +167,7 @@ int tcg_alloc (tcg_ctx* ctx, size_t bytes, void** devptr)
 	std::string why;
 	int rc = ctx->pool.take(bytes, devptr, &why);
 	if (rc != tcg_pool::OK) { return tcg_fail(ctx, TCG_ERR_OOM, "tcg_alloc: %s", why.c_str()); }
+	if (ctx->batch) { tcg_batch_note_alloc(ctx, *devptr, bytes); }
 	return TCG_OK;
 }
 
@@ -176,6 +178,7 @@ int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes)
 	std::string why;
 	int rc = ctx->pool.give(devptr, bytes, &why);
 	if (rc != tcg_pool::OK) { return tcg_fail(ctx, TCG_ERR_ARG, "tcg_free: %p: %s", devptr, why.c_str()); }
+	if (ctx->batch) { tcg_batch_note_free(ctx, devptr); }
 	return TCG_OK;
 }
 
@@ -267,6 +270,7 @@ int tcg_d2h (tcg_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes)
 	if (bytes == 0) { return TCG_OK; }
 	TCG_REQUIRE(ctx, dst_host && src_dev, "tcg_d2h: NULL pointer");
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_d2h: host transfers cannot be part of a captured sequence");
+	if (ctx->batch) { int rc = tcg_batch_end(ctx); if (rc != TCG_OK) { return rc; } }
 	TCG_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
 	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
 	return TCG_OK;
@@ -314,6 +318,7 @@ int tcg_sync (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_sync: cannot wait while a sequence is being captured");
+	if (ctx->batch) { int rc = tcg_batch_end(ctx); if (rc != TCG_OK) { return rc; } }
 	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
 	return TCG_OK;
 }
@@ -432,6 +437,13 @@ int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out)
 	if (!ctx || !out) { return TCG_ERR_ARG; }
 	*out = nullptr;
 	TCG_REQUIRE(ctx, ctx->capturing, "tcg_capture_end: no capture in progress");
+	// steps still held back belong to the sequence
+	int sent = ctx->batch ? tcg_batch_end(ctx) : TCG_OK;
+	if (sent != TCG_OK)
+	{
+		(void) tcg_capture_abort(ctx);
+		return sent;
+	}
 	tcg_graph* g = ctx->capturing;
 	ctx->capturing = nullptr;
 	ctx->pool.seal(g);
@@ -466,6 +478,7 @@ int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out)
 int tcg_capture_abort (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
+	tcg_batch_discard(ctx);
 	if (!ctx->capturing) { return TCG_OK; }
 	tcg_graph* g = ctx->capturing;
 	ctx->capturing = nullptr;
@@ -480,6 +493,7 @@ int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph)
 {
 	if (!ctx || !graph) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_graph_launch: cannot launch while capturing");
+	if (ctx->batch) { int sent = tcg_batch_end(ctx); if (sent != TCG_OK) { return sent; } }
 	int rc = TCG_OK;
 	if (graph->small) { rc = tcg_small_launch(ctx, graph); }
 	else

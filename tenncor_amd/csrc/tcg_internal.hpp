@@ -41,6 +41,7 @@ struct tcg_graph : public tcg_arena
 	bool launched = false;
 };
 
+struct tcg_small_pass;
 struct tcg_ctx
 {
 	int device = 0;
@@ -95,6 +96,9 @@ struct tcg_ctx
 		bool open = false;
 	};
 	Hold* hold = nullptr;
+
+	// tcg_batch_begin: steps of small work held back, to go out as one launch
+	tcg_small_pass* batch = nullptr;
 };
 
 int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);
@@ -145,8 +149,21 @@ static inline bool tcg_aligned16 (const void* p)
 // instead of launching; anything that cannot be a step fails the recording.
 static inline bool tcg_small_mode (const tcg_ctx* ctx)
 {
-	return ctx->capturing && ctx->capturing->small;
+	return (ctx->capturing && ctx->capturing->small) || nullptr != ctx->batch;
 }
+// Between tcg_batch_begin and tcg_batch_end the same entry points hand their
+// work over when it is small and hold it back; a call that cannot be a step
+// sends out the steps held so far, ends the batch and runs as itself.
+int tcg_batch_send (tcg_ctx* ctx);     // the steps held so far as one launch; the batch stays open
+int tcg_batch_decline (tcg_ctx* ctx);  // tcg_batch_send, and the batch is over
+void tcg_batch_discard (tcg_ctx* ctx);  // the batch is over and its steps are dropped
+void tcg_batch_note_alloc (tcg_ctx* ctx, const void* ptr, size_t bytes); // tcg_alloc / tcg_free inside a batch
+void tcg_batch_note_free (tcg_ctx* ctx, const void* ptr);
+#define TCG_SMALL_RETURN(ctx, expr) do {\
+	int rc__ = (expr);\
+	if (rc__ != TCG_ERR_UNSUPPORTED || nullptr == (ctx)->batch) { return rc__; }\
+	rc__ = tcg_batch_decline(ctx);\
+	if (rc__ != TCG_OK) { return rc__; } } while (0)
 int tcg_small_begin (tcg_ctx* ctx, tcg_graph* g);
 int tcg_small_finish (tcg_ctx* ctx, tcg_graph* g);   // compiles; the recording is closed
 int tcg_small_launch (tcg_ctx* ctx, tcg_graph* g);

@@ -213,6 +213,19 @@ std::string describe_step (const FusionPlan& plan, const FusionPlan::Step& step)
 void launch_step (const FusionPlan& plan, const FusionPlan::Step& step, Device& device, const teq::TensSetT& targets,
 	RangeTempsT& temps);
 
+/// What goes out together: one step, or a run [first, second) of steps over a
+/// few thousand elements each (elementwise groups, reductions, contractions),
+/// which are handed over between tcg_batch_begin and tcg_batch_end and run as
+/// the steps of one kernel.  TCR_BATCHES=0 makes every step a unit of its own.
+using LaunchUnit = std::pair<size_t,size_t>;
+
+std::vector<LaunchUnit> launch_units (const FusionPlan& plan, bool batches = true);
+
+std::string describe_unit (const FusionPlan& plan, const LaunchUnit& unit);
+
+void launch_unit (const FusionPlan& plan, const LaunchUnit& unit, Device& device, const teq::TensSetT& targets,
+	RangeTempsT& temps);
+
 }
 
 #endif // TCH_FUSE_PLAN_HPP

@@ -2202,6 +2202,105 @@ std::string describe_step (const FusionPlan& plan, const FusionPlan::Step& step)
 		" instrs=" + std::to_string(group.program.size());
 }
 
+bool step_batchable (const FusionPlan& plan, const FusionPlan::Step& step)
+{
+	// a few iterations per lane of one workgroup: more is declined by the launch anyway
+	constexpr size_t most = (size_t) 1 << 14;
+	if (nullptr != step.node)
+	{
+		int op = (int) step.node->get_opcode().code_;
+		bool known = is_unary(op) || is_binary(op) || op == egen::CONTRACT || op == egen::MATMUL ||
+			op == egen::REDUCE_SUM || op == egen::REDUCE_PROD || op == egen::REDUCE_MIN || op == egen::REDUCE_MAX;
+		if (false == known || step.node->shape().n_elems() > most) { return false; }
+		for (auto& arg : step.node->get_args())
+		{
+			if (arg->shape().n_elems() > most) { return false; }
+		}
+		return true;
+	}
+	if (step.group >= 0 && step.parts < 0)
+	{
+		size_t n = 1;
+		for (uint64_t extent : plan.groups[step.group].shape) { n *= (size_t) extent; }
+		return n <= most;
+	}
+	return false;
+}
+
+static bool batches_enabled (void)
+{
+	static const bool on = []
+	{
+		const char* env = getenv("TCR_BATCHES");
+		return !(env && env[0] == '0');
+	}();
+	return on;
+}
+
+std::vector<LaunchUnit> launch_units (const FusionPlan& plan, bool batches)
+{
+	std::vector<LaunchUnit> units;
+	batches = batches && batches_enabled();
+	for (size_t i = 0, n = plan.steps.size(); i < n;)
+	{
+		size_t end = i + 1;
+		if (batches && step_batchable(plan, plan.steps[i]))
+		{
+			while (end < n && step_batchable(plan, plan.steps[end])) { ++end; }
+		}
+		units.push_back({i, end});
+		i = end;
+	}
+	return units;
+}
+
+std::string describe_unit (const FusionPlan& plan, const LaunchUnit& unit)
+{
+	if (unit.second - unit.first < 2) { return describe_step(plan, plan.steps[unit.first]); }
+	std::string out = "batch of " + std::to_string(unit.second - unit.first) + ":";
+	for (size_t i = unit.first; i < unit.second; ++i)
+	{
+		const FusionPlan::Step& step = plan.steps[i];
+		out += " ";
+		if (nullptr != step.node) { out += step.node->get_opcode().name_; }
+		else
+		{
+			auto& members = plan.groups[step.group].members;
+			out += "(";
+			for (size_t k = 0; k < members.size(); ++k) { out += (k ? "+" : "") + members[k]->get_opcode().name_; }
+			out += ")";
+		}
+	}
+	return out;
+}
+
+void launch_unit (const FusionPlan& plan, const LaunchUnit& unit, Device& device, const teq::TensSetT& targets,
+	RangeTempsT& temps)
+{
+	if (unit.second - unit.first < 2)
+	{
+		launch_step(plan, plan.steps[unit.first], device, targets, temps);
+		return;
+	}
+	// small steps in a row: held back and sent out as one launch where the launch
+	// takes them (a step it does not take goes out by itself, in its place)
+	tcg_ctx* ctx = hip_context();
+	try
+	{
+		for (size_t i = unit.first; i < unit.second; ++i)
+		{
+			hip_check(tcg_batch_begin(ctx));
+			launch_step(plan, plan.steps[i], device, targets, temps);
+		}
+	}
+	catch (...)
+	{
+		(void) tcg_batch_end(ctx);
+		throw;
+	}
+	hip_check(tcg_batch_end(ctx));
+}
+
 void launch_step (const FusionPlan& plan, const FusionPlan::Step& step, Device& device, const teq::TensSetT& targets,
 	RangeTempsT& temps)
 {

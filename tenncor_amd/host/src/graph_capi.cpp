@@ -468,7 +468,12 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 		teq::multi_visit(collector, key);
 		eigen::FusionPlan plan = eigen::plan_fusion(collector.funcs, tset);
 		std::stringstream ss;
-		for (auto& step : plan.steps) { ss << eigen::describe_step(plan, step) << "\n"; }
+		// "batch N": the N steps that follow are small and go out as one launch
+		for (auto& unit : eigen::launch_units(plan))
+		{
+			if (unit.second - unit.first > 1) { ss << "batch " << unit.second - unit.first << "\n"; }
+			for (size_t i = unit.first; i < unit.second; ++i) { ss << eigen::describe_step(plan, plan.steps[i]) << "\n"; }
+		}
 		ss << "folded " << plan.absorbed.size() << "\n";
 		std::string text = ss.str();
 		if (needed) { *needed = text.size(); }

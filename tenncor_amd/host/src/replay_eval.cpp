@@ -291,7 +291,14 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		RangeTempsT temps(fusion.part_products.size(), {nullptr, 0});
 		try
 		{
-			for (auto& step : fusion.steps) { launch_step(fusion, step, device, targets, temps); }
+			if (as_one_kernel)
+			{
+				for (auto& step : fusion.steps) { launch_step(fusion, step, device, targets, temps); }
+			}
+			else
+			{
+				for (auto& unit : launch_units(fusion, small_passes_)) { launch_unit(fusion, unit, device, targets, temps); }
+			}
 		}
 		catch (const std::exception& err)
 		{

@@ -73,7 +73,8 @@ void TimingEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 		f->prop_version(gpu->max_version_);
 	}
 	tcg_ctx* ctx = hip_context();
-	std::vector<void*> events(plan.steps.size() + 1, nullptr);
+	std::vector<LaunchUnit> units = launch_units(plan);
+	std::vector<void*> events(units.size() + 1, nullptr);
 	for (void*& ev : events) { hip_check(tcg_event_create(ctx, &ev)); }
 	RangeTempsT temps(plan.part_products.size(), {nullptr, 0});
 	auto give_back = [&]
@@ -93,9 +94,9 @@ void TimingEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 		try
 		{
 			hip_check(tcg_event_record(ctx, events[0]));
-			for (size_t i = 0; i < plan.steps.size(); ++i)
+			for (size_t i = 0; i < units.size(); ++i)
 			{
-				launch_step(plan, plan.steps[i], *gpu, targets, temps);
+				launch_unit(plan, units[i], *gpu, targets, temps);
 				hip_check(tcg_event_record(ctx, events[i + 1]));
 			}
 		}
@@ -105,11 +106,11 @@ void TimingEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 			throw;
 		}
 		hip_check(tcg_release(ctx));
-		for (size_t i = 0; i < plan.steps.size(); ++i)
+		for (size_t i = 0; i < units.size(); ++i)
 		{
 			float ms = 0.0f;
 			hip_check(tcg_event_elapsed(ctx, events[i], events[i + 1], &ms));
-			Row& row = table_[describe_step(plan, plan.steps[i])];
+			Row& row = table_[describe_unit(plan, units[i])];
 			++row.launches;
 			row.us += 1e3 * (double) ms;
 		}
@@ -121,7 +122,7 @@ void TimingEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 	}
 	give_back();
 	++passes_;
-	launches_ = plan.steps.size();
+	launches_ = units.size();
 }
 
 std::vector<TimingEvaluator::Row> TimingEvaluator::rows (void) const

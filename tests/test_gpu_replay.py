@@ -364,7 +364,8 @@ def test_products_over_the_parts_of_concatenations_follow_the_walk():
     largest entry, the bar of a contraction.  The second case has part extents
     with a small common divisor (12 and 20: chunks of 4), which the matrix
     cores do not take, so that the concatenations are laid out as before and
-    the results are the walk's bit for bit."""
+    the results of the recording without single-kernel runs are the walk's bit
+    for bit (with them, the small steps of such a graph sum in another order)."""
     from tenncor_amd import configs, graph
     rng = np.random.default_rng(41)
     for (seq, batch, nin, hid), exact in (((6, 64, 32, 64), False), ((5, 48, 12, 20), True)):
@@ -377,7 +378,9 @@ def test_products_over_the_parts_of_concatenations_follow_the_walk():
             return targets, x
 
         results, stats = run_both(build, feeds, kinds=("plain", "replay_launches", "replay"))
-        (assert_same_bits if exact else assert_close_to_walk)(results)
+        assert_close_to_walk(results)
+        if exact:
+            assert_same_bits({kind: results[kind] for kind in ("plain", "replay_launches")})
         assert stats["replay"]["replayed"] == 2 and stats["replay"]["record_failures"] == 0
 
 
@@ -1331,7 +1334,18 @@ def test_timing_evaluator_runs_the_planned_launches_between_events():
                 results[kind] = [t.get().copy() for t in targets]
                 if kind == "timing":
                     report = graph.evaluator_timing()
-                    planned = [l for l in g.launch_plan(targets) if not l.startswith("folded")]
+                    # "batch N": the N steps behind that line go out as one launch
+                    planned, skip = [], 0
+                    for l in g.launch_plan(targets):
+                        if l.startswith("folded"):
+                            continue
+                        if skip:
+                            skip -= 1
+                        elif l.startswith("batch "):
+                            skip = int(l.split(" ")[1])
+                            planned.append("batch of %d:" % skip)
+                        else:
+                            planned.append(l)
             finally:
                 g.close()
     finally:
@@ -1347,5 +1361,9 @@ def test_timing_evaluator_runs_the_planned_launches_between_events():
         rows[what] = (int(count), float(rest.split("=")[1]))
     # every planned launch is in the table, three times (one per pass), with a positive time
     for what in set(planned):
-        assert rows[what][0] == 3 * planned.count(what) and rows[what][1] > 0, (what, rows.get(what))
+        if what.startswith("batch of "):
+            found = [v for k, v in rows.items() if k.startswith(what)]
+            assert sum(v[0] for v in found) == 3 * planned.count(what) and all(v[1] > 0 for v in found), (what, found)
+        else:
+            assert rows[what][0] == 3 * planned.count(what) and rows[what][1] > 0, (what, rows.get(what))
     assert any(" with epilogue group " in what for what in rows)

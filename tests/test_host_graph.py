@@ -262,9 +262,15 @@ def test_mlp_gradient_graph_only_uses_table_opcodes(g, api):
 
 # ---- launch planning of the replaying evaluator (host logic only) -------------
 
-def parse_plan(lines):
+def parse_plan(lines, batches=None):
+    """batches: a list that receives (index of the first step, number of steps) for every run
+    of small steps that goes out as one launch"""
     steps = []
     for line in lines:
+        if line.startswith("batch "):
+            if batches is not None:
+                batches.append((len(steps), int(line.split(" ")[1])))
+            continue
         product, marker, epilogue = line.partition(" with epilogue ")
         if marker:
             # a product and the group that reads it as one launch: both steps, the first one flagged
