@@ -220,6 +220,26 @@ int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph);
  * node (internal/teq/evaluator.hpp:35-62) and has no launches to save. */
 int tcg_batch_begin (tcg_ctx* ctx);
 int tcg_batch_end (tcg_ctx* ctx);
+/* Work that nothing waits for yet, beside the work that follows it (the two
+ * gradients of a convolution, neither of which reads the other: each leaves
+ * part of the chip idle at the end of its grid).  tcg_fork: the launches of
+ * the calls that follow go to a second stream of the context, which starts
+ * when everything enqueued so far has run.  tcg_fork_end: the calls that follow
+ * go to the context's own stream again and run BESIDE what was forked.
+ * tcg_join: the context's stream waits for the forked launches; memory given
+ * back (tcg_free) between tcg_fork and tcg_fork_end returns to the pool only
+ * now, because the forked launches use it.  The caller keeps what the forked
+ * launches read and write untouched by the calls between tcg_fork_end and
+ * tcg_join (no writes to their inputs, no reads of their results, inputs not
+ * given back).  One fork at a time.  Inside a recording the second stream is
+ * part of the recording (a branch of the graph); tcg_sync, tcg_d2h,
+ * tcg_capture_begin/end and tcg_graph_launch join first.  In a single-launch
+ * recording (tcg_capture_begin_small) the three calls do nothing.  No
+ * counterpart in the reference, whose device runs one expression at a time
+ * (internal/eigen/device.hpp:555-570). */
+int tcg_fork (tcg_ctx* ctx);
+int tcg_fork_end (tcg_ctx* ctx);
+int tcg_join (tcg_ctx* ctx);
 int tcg_graph_claim (tcg_ctx* ctx, tcg_graph* graph, void* devptr);
 int tcg_graph_stats (const tcg_graph* graph, uint64_t* nodes, uint64_t* arena_bytes);
 int tcg_graph_destroy (tcg_ctx* ctx, tcg_graph* graph);

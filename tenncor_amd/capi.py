@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_jit_stats", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort", "tcg_batch_begin", "tcg_batch_end",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_jit_stats", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort", "tcg_batch_begin", "tcg_batch_end", "tcg_fork", "tcg_fork_end", "tcg_join",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -98,6 +98,9 @@ def load():
         "tcg_mem_stats_kept": [vp, u64p],
         "tcg_hold": [vp],
         "tcg_batch_begin": [vp],
+        "tcg_fork": [vp],
+        "tcg_fork_end": [vp],
+        "tcg_join": [vp],
         "tcg_batch_end": [vp],
         "tcg_release": [vp],
         "tcg_h2d": [vp, vp, vp, sz],
@@ -542,6 +545,16 @@ class Context:
 
     def batch_end(self):
         self._check(self.lib.tcg_batch_end(self.handle))
+
+    def fork(self):
+        """Calls from here to fork_end() run on a second stream, beside what follows fork_end()."""
+        self._check(self.lib.tcg_fork(self.handle))
+
+    def fork_end(self):
+        self._check(self.lib.tcg_fork_end(self.handle))
+
+    def join(self):
+        self._check(self.lib.tcg_join(self.handle))
 
     def capture_begin(self, small=False):
         """small: record the sequence as the steps of one kernel."""

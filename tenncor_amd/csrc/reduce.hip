@@ -501,7 +501,10 @@ int reduce_step (tcg_ctx* ctx, Scratch& mem, const T* in, T* out, uint64_t A, ui
 			}
 		}
 	}
-	if (base_blocks < target_blocks && R >= (uint64_t) TY * 16)
+	// (not below 256 KiB per workgroup: the launch that adds the partial rows up
+	// then costs more than the split saves -- [64, 400, 128] -> [64, 128] takes
+	// 4.5 + 4.8 us in three ranges)
+	if (base_blocks < target_blocks && R >= (uint64_t) TY * 16 && A * R * sizeof(T) >= ((uint64_t) 256 << 10))
 	{
 		S = (target_blocks + base_blocks - 1) / base_blocks;
 		uint64_t maxs = R / ((uint64_t) TY * 8);

@@ -68,7 +68,12 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 	};
 	ctx->pool.raw_free = [](void* ptr) { (void) hipFree(ptr); };
 	// (a held stream cannot be waited for: see tcg_hold)
-	ctx->pool.drain = [ctx] { if (nullptr == ctx->hold) { (void) hipStreamSynchronize(ctx->stream); } };
+	ctx->pool.drain = [ctx]
+	{
+		if (nullptr != ctx->hold) { return; }
+		(void) hipStreamSynchronize(ctx->stream);
+		if (ctx->fork_state) { (void) hipStreamSynchronize(ctx->fork_state == 1 ? ctx->main_stream : ctx->fork_stream); }
+	};
 	ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
 	ctx->arch = prop.gcnArchName;
 	size_t colon = ctx->arch.find(':');
@@ -108,9 +113,27 @@ int tcg_ctx_create (int device, tcg_ctx** out)
 		delete ctx;
 		return rc;
 	}
+	// the stream and the events of tcg_fork / tcg_join (default priority, like the others)
+	if ((err = hipStreamCreate(&ctx->fork_stream)) != hipSuccess ||
+		(err = hipEventCreateWithFlags(&ctx->ev_fork, hipEventDisableTiming)) != hipSuccess ||
+		(err = hipEventCreateWithFlags(&ctx->ev_join, hipEventDisableTiming)) != hipSuccess)
+	{
+		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: third stream: %s", hipGetErrorString(err));
+		if (ctx->ev_fork) { (void) hipEventDestroy(ctx->ev_fork); }
+		if (ctx->fork_stream) { (void) hipStreamDestroy(ctx->fork_stream); }
+		(void) hipStreamDestroy(ctx->side_stream);
+		(void) hipFree(ctx->zeros);
+		(void) hipFree(ctx->rng_state);
+		(void) hipHostFree(ctx->staging);
+		delete ctx;
+		return rc;
+	}
 	if (tcg_reduce_scratch_init(ctx) != TCG_OK)
 	{
 		int rc = tcg_fail(nullptr, TCG_ERR_HIP, "tcg_ctx_create: %s", ctx->error.c_str());
+		(void) hipEventDestroy(ctx->ev_join);
+		(void) hipEventDestroy(ctx->ev_fork);
+		(void) hipStreamDestroy(ctx->fork_stream);
 		(void) hipStreamDestroy(ctx->side_stream);
 		(void) hipFree(ctx->zeros);
 		(void) hipFree(ctx->rng_state);
@@ -128,12 +151,20 @@ int tcg_ctx_destroy (tcg_ctx* ctx)
 	(void) hipSetDevice(ctx->device);
 	tcg_batch_discard(ctx);
 	(void) tcg_release(ctx);
+	(void) tcg_join(ctx);
 	(void) hipStreamSynchronize(ctx->stream);
 	tcg_reduce_scratch_release(ctx);
 	ctx->pool.release_all();
 	if (ctx->staging) { (void) hipHostFree(ctx->staging); }
 	if (ctx->rng_state) { (void) hipFree(ctx->rng_state); }
 	if (ctx->zeros) { (void) hipFree(ctx->zeros); }
+	if (ctx->fork_stream)
+	{
+		(void) hipStreamSynchronize(ctx->fork_stream);
+		(void) hipStreamDestroy(ctx->fork_stream);
+		(void) hipEventDestroy(ctx->ev_fork);
+		(void) hipEventDestroy(ctx->ev_join);
+	}
 	if (ctx->side_stream)
 	{
 		(void) hipStreamSynchronize(ctx->side_stream);
@@ -175,6 +206,13 @@ int tcg_free (tcg_ctx* ctx, void* devptr, size_t bytes)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	if (!devptr) { return TCG_OK; }
+	if (ctx->fork_state == 1)
+	{
+		// used by launches of the second stream: back to the pool when the context's
+		// own stream has waited for them
+		ctx->fork_frees.emplace_back(devptr, bytes);
+		return TCG_OK;
+	}
 	std::string why;
 	int rc = ctx->pool.give(devptr, bytes, &why);
 	if (rc != tcg_pool::OK) { return tcg_fail(ctx, TCG_ERR_ARG, "tcg_free: %p: %s", devptr, why.c_str()); }
@@ -231,6 +269,50 @@ int tcg_release (tcg_ctx* ctx)
 	return TCG_OK;
 }
 
+// ---- a second stream for work nothing waits for yet -------------------------------
+int tcg_fork (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	TCG_REQUIRE(ctx, 0 == ctx->fork_state, "tcg_fork: the launches of an earlier tcg_fork have not been joined");
+	// a single-launch recording has no streams to spread its steps over
+	if (tcg_small_mode(ctx)) { return TCG_OK; }
+	TCG_HIP(ctx, hipEventRecord(ctx->ev_fork, ctx->stream));
+	TCG_HIP(ctx, hipStreamWaitEvent(ctx->fork_stream, ctx->ev_fork, 0));
+	ctx->main_stream = ctx->stream;
+	ctx->stream = ctx->fork_stream;
+	ctx->fork_state = 1;
+	return TCG_OK;
+}
+
+int tcg_fork_end (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (ctx->fork_state != 1) { return TCG_OK; }
+	hipError_t err = hipEventRecord(ctx->ev_join, ctx->fork_stream);
+	ctx->stream = ctx->main_stream;
+	ctx->fork_state = 2;
+	if (err != hipSuccess) { return tcg_fail(ctx, TCG_ERR_HIP, "tcg_fork_end: %s", hipGetErrorString(err)); }
+	return TCG_OK;
+}
+
+int tcg_join (tcg_ctx* ctx)
+{
+	if (!ctx) { return TCG_ERR_ARG; }
+	if (0 == ctx->fork_state) { return TCG_OK; }
+	int rc = tcg_fork_end(ctx);
+	hipError_t err = hipStreamWaitEvent(ctx->stream, ctx->ev_join, 0);
+	ctx->fork_state = 0;
+	std::vector<std::pair<void*,size_t>> frees;
+	frees.swap(ctx->fork_frees);
+	for (auto& f : frees)
+	{
+		int freed = tcg_free(ctx, f.first, f.second);
+		if (rc == TCG_OK) { rc = freed; }
+	}
+	if (rc == TCG_OK && err != hipSuccess) { rc = tcg_fail(ctx, TCG_ERR_HIP, "tcg_join: %s", hipGetErrorString(err)); }
+	return rc;
+}
+
 int tcg_mem_stats_kept (const tcg_ctx* ctx, uint64_t* conv_tables)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
@@ -271,6 +353,7 @@ int tcg_d2h (tcg_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes)
 	TCG_REQUIRE(ctx, dst_host && src_dev, "tcg_d2h: NULL pointer");
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_d2h: host transfers cannot be part of a captured sequence");
 	if (ctx->batch) { int rc = tcg_batch_end(ctx); if (rc != TCG_OK) { return rc; } }
+	if (ctx->fork_state) { int rc = tcg_join(ctx); if (rc != TCG_OK) { return rc; } }
 	TCG_HIP(ctx, hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
 	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
 	return TCG_OK;
@@ -319,6 +402,7 @@ int tcg_sync (tcg_ctx* ctx)
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_sync: cannot wait while a sequence is being captured");
 	if (ctx->batch) { int rc = tcg_batch_end(ctx); if (rc != TCG_OK) { return rc; } }
+	if (ctx->fork_state) { int rc = tcg_join(ctx); if (rc != TCG_OK) { return rc; } }
 	TCG_HIP(ctx, hipStreamSynchronize(ctx->stream));
 	return TCG_OK;
 }
@@ -379,6 +463,7 @@ int tcg_capture_begin (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_capture_begin: a capture is already in progress");
+	if (ctx->fork_state) { int rc = tcg_join(ctx); if (rc != TCG_OK) { return rc; } }
 	// relaxed mode: the pool may still call hipMalloc for a size it has not seen
 	TCG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
 	ctx->capturing = new tcg_graph();
@@ -390,6 +475,7 @@ int tcg_capture_begin_small (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_capture_begin_small: a capture is already in progress");
+	if (ctx->fork_state) { int rc = tcg_join(ctx); if (rc != TCG_OK) { return rc; } }
 	// the stream captures as well: a launch that is not handed over as a step
 	// is caught there (and fails tcg_capture_end) instead of running out of turn
 	TCG_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
@@ -439,6 +525,8 @@ int tcg_capture_end (tcg_ctx* ctx, tcg_graph** out)
 	TCG_REQUIRE(ctx, ctx->capturing, "tcg_capture_end: no capture in progress");
 	// steps still held back belong to the sequence
 	int sent = ctx->batch ? tcg_batch_end(ctx) : TCG_OK;
+	// the second stream is part of the recording until it has been waited for
+	if (sent == TCG_OK && ctx->fork_state) { sent = tcg_join(ctx); }
 	if (sent != TCG_OK)
 	{
 		(void) tcg_capture_abort(ctx);
@@ -479,6 +567,7 @@ int tcg_capture_abort (tcg_ctx* ctx)
 {
 	if (!ctx) { return TCG_ERR_ARG; }
 	tcg_batch_discard(ctx);
+	(void) tcg_join(ctx);
 	if (!ctx->capturing) { return TCG_OK; }
 	tcg_graph* g = ctx->capturing;
 	ctx->capturing = nullptr;
@@ -494,6 +583,7 @@ int tcg_graph_launch (tcg_ctx* ctx, tcg_graph* graph)
 	if (!ctx || !graph) { return TCG_ERR_ARG; }
 	TCG_REQUIRE(ctx, !ctx->capturing, "tcg_graph_launch: cannot launch while capturing");
 	if (ctx->batch) { int sent = tcg_batch_end(ctx); if (sent != TCG_OK) { return sent; } }
+	if (ctx->fork_state) { int joined = tcg_join(ctx); if (joined != TCG_OK) { return joined; } }
 	int rc = TCG_OK;
 	if (graph->small) { rc = tcg_small_launch(ctx, graph); }
 	else

@@ -99,6 +99,14 @@ struct tcg_ctx
 
 	// tcg_batch_begin: steps of small work held back, to go out as one launch
 	tcg_small_pass* batch = nullptr;
+
+	// tcg_fork: 1 while launches go to fork_stream (`stream` IS fork_stream then and
+	// main_stream holds the context's own), 2 while what was enqueued there may
+	// still run; memory given back in state 1 is kept until tcg_join
+	int fork_state = 0;
+	hipStream_t fork_stream = nullptr, main_stream = nullptr;
+	hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+	std::vector<std::pair<void*,size_t>> fork_frees;
 };
 
 int tcg_fail (tcg_ctx* ctx, int status, const char* fmt, ...);

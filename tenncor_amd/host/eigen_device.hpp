@@ -10,6 +10,7 @@
 #ifndef TCH_EIGEN_DEVICE_HPP
 #define TCH_EIGEN_DEVICE_HPP
 
+#include <atomic>
 #include <limits>
 
 #include "tcg.h"
@@ -685,6 +686,11 @@ struct Observable : public teq::iFunctor
 
 	virtual ~Observable (void) = default;
 
+	/// Position in the order in which the functors of this process were made: a
+	/// way to enumerate a set of them that does not depend on where they lie in
+	/// memory (launch plans then come out the same from run to run)
+	uint64_t born (void) const { return born_; }
+
 	void subscribe (Observable* sub) { subs_.emplace(sub); }
 	void unsubscribe (Observable* sub) { subs_.erase(sub); }
 	std::unordered_set<Observable*> get_observables (void) const { return subs_; }
@@ -712,7 +718,14 @@ protected:
 	std::unordered_set<Observable*> subs_;
 
 private:
+	static uint64_t next_born (void)
+	{
+		static std::atomic<uint64_t> count{0};
+		return count.fetch_add(1);
+	}
+
 	marsh::Maps attrs_;
+	const uint64_t born_ = next_born();
 };
 
 // ---- the device (internal/eigen/device.hpp:546-576) ------------------------

@@ -183,6 +183,12 @@ struct FusionPlan final
 	std::vector<Observable*> absorbed;
 };
 
+/// The tensors in the order their functors were made (leaves last): the targets
+/// of a pass come as an unordered set, and which launches share a kernel depends
+/// on the order in which the functors under them are met, so they are walked in
+/// this order rather than in the order of their addresses
+std::vector<teq::iTensor*> birth_order (std::vector<teq::iTensor*> tensors);
+
 /// `funcs`: every functor under the targets, children first
 FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSetT& targets);
 
@@ -200,7 +206,11 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
-void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory);
+/// later_reads: the operands are not counted as read now but appended there, for
+/// a launch that runs beside the launches that follow it (the caller counts them
+/// when it has waited for the launch)
+void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory,
+	std::vector<teq::iTensor*>* later_reads = nullptr);
 
 void launch_sum (const SummedContracts& call, const teq::TensSetT& targets, RTMemptrT& memory);
 
@@ -225,6 +235,15 @@ std::string describe_unit (const FusionPlan& plan, const LaunchUnit& unit);
 
 void launch_unit (const FusionPlan& plan, const LaunchUnit& unit, Device& device, const teq::TensSetT& targets,
 	RangeTempsT& temps);
+
+/// The whole pass, unit by unit.  forks: a convolution whose result nothing
+/// reads before another convolution or product has been launched goes to the
+/// context's second stream (tcg_fork) and runs beside what follows, up to the
+/// first launch that reads it, rewrites a leaf, or the end of the pass; its
+/// operands stay allocated until then.  Only with TCR_FORKS=1 in the environment
+/// (measured without gain on the gradients of a convolutional layer).
+void launch_pass (const FusionPlan& plan, Device& device, const teq::TensSetT& targets, RangeTempsT& temps,
+	bool batches, bool forks);
 
 }
 

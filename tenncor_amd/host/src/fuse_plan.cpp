@@ -1,6 +1,7 @@
 // Which functors of an evaluation pass share a launch (see fuse_plan.hpp).
 #include "fuse_plan.hpp"
 
+#include <limits>
 #include <type_traits>
 #include <algorithm>
 #include <functional>
@@ -2179,6 +2180,20 @@ struct Planner final
 
 }
 
+/// The tensors in the order their functors were made (leaves last): the targets
+/// of a pass come as an unordered set, and which launches share a kernel depends
+/// on the order in which the functors under them are met
+std::vector<teq::iTensor*> birth_order (std::vector<teq::iTensor*> tensors)
+{
+	auto born = [](teq::iTensor* t)
+	{
+		auto f = dynamic_cast<Observable*>(t);
+		return nullptr == f ? std::numeric_limits<uint64_t>::max() : f->born();
+	};
+	std::stable_sort(tensors.begin(), tensors.end(), [&](teq::iTensor* a, teq::iTensor* b) { return born(a) < born(b); });
+	return tensors;
+}
+
 FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSetT& targets)
 {
 	Planner planner(funcs, targets);
@@ -2224,6 +2239,11 @@ bool step_batchable (const FusionPlan& plan, const FusionPlan::Step& step)
 		for (uint64_t extent : plan.groups[step.group].shape) { n *= (size_t) extent; }
 		return n <= most;
 	}
+	if (step.contract >= 0)
+	{
+		const SwappedContract& c = plan.contracts[step.contract];
+		return c.node->shape().n_elems() <= most && c.a->shape().n_elems() <= most && c.b->shape().n_elems() <= most;
+	}
 	return false;
 }
 
@@ -2263,6 +2283,7 @@ std::string describe_unit (const FusionPlan& plan, const LaunchUnit& unit)
 		const FusionPlan::Step& step = plan.steps[i];
 		out += " ";
 		if (nullptr != step.node) { out += step.node->get_opcode().name_; }
+		else if (step.contract >= 0) { out += "CONTRACT+PERMUTE"; }
 		else
 		{
 			auto& members = plan.groups[step.group].members;
@@ -2299,6 +2320,146 @@ void launch_unit (const FusionPlan& plan, const LaunchUnit& unit, Device& device
 		throw;
 	}
 	hip_check(tcg_batch_end(ctx));
+}
+
+/// Off unless TCR_FORKS=1: on the two gradients of a 5x5 convolution over
+/// 128 x 20 x 20 x 64 outputs the launches did overlap, and each ran as much
+/// slower as the other took (0.413 ms per pass with the second stream, 0.401
+/// without): neither leaves the compute units idle for the other to use
+static bool forks_enabled (void)
+{
+	static const bool on = []
+	{
+		const char* env = getenv("TCR_FORKS");
+		return env && env[0] == '1';
+	}();
+	return on;
+}
+
+/// Whether `tens` is `node` or shares its buffer (IDENTITY / RESHAPE / SLICE of it)
+static bool same_buffer (const teq::iTensor* tens, const teq::iTensor* node)
+{
+	while (nullptr != tens)
+	{
+		if (tens == node) { return true; }
+		auto f = dynamic_cast<const teq::iFunctor*>(tens);
+		if (nullptr == f || false == is_buffer_alias((int) f->get_opcode().code_)) { return false; }
+		tens = f->get_args().front().get();
+	}
+	return false;
+}
+
+/// Whether the step reads (or may write over) the value of `node`
+static bool step_touches (const FusionPlan& plan, const FusionPlan::Step& step, const teq::iTensor* node)
+{
+	auto any = [node](const std::vector<teq::iTensor*>& reads)
+	{
+		return std::any_of(reads.begin(), reads.end(), [node](const teq::iTensor* t) { return same_buffer(t, node); });
+	};
+	if (nullptr != step.node)
+	{
+		if (is_assign((int) step.node->get_opcode().code_)) { return true; } // may rewrite a leaf the node's launch reads
+		for (auto& arg : step.node->get_args())
+		{
+			if (same_buffer(arg.get(), node)) { return true; }
+		}
+		return false;
+	}
+	bool hit = false;
+	if (step.conv >= 0)
+	{
+		const ViewedConv& c = plan.convs[step.conv];
+		hit = any(c.reads) || same_buffer(c.image, node) || same_buffer(c.kernel, node);
+	}
+	if (step.contract >= 0)
+	{
+		const SwappedContract& c = plan.contracts[step.contract];
+		hit = hit || any(c.reads) || same_buffer(c.a, node) || same_buffer(c.b, node);
+	}
+	if (step.sum >= 0) { hit = hit || any(plan.sums[step.sum].reads) || any(plan.sums[step.sum].a) || any(plan.sums[step.sum].b); }
+	if (step.parts >= 0)
+	{
+		const PartProducts& p = plan.part_products[step.parts];
+		hit = hit || any(p.reads);
+		for (auto& product : p.products)
+		{
+			for (auto& term : product.terms) { hit = hit || same_buffer(term.a, node) || same_buffer(term.b, node); }
+		}
+	}
+	if (step.group >= 0)
+	{
+		const FusedGroup& g = plan.groups[step.group];
+		hit = hit || any(g.reads);
+		for (auto& leaf : g.leaves) { hit = hit || (nullptr != leaf.base && same_buffer(leaf.base, node)); }
+	}
+	return hit;
+}
+
+static bool heavy_step (const FusionPlan::Step& step)
+{
+	if (nullptr != step.node)
+	{
+		int op = (int) step.node->get_opcode().code_;
+		return op == egen::CONV || op == egen::CONTRACT || op == egen::MATMUL;
+	}
+	return step.conv >= 0 || step.contract >= 0 || step.sum >= 0 || step.parts >= 0;
+}
+
+void launch_pass (const FusionPlan& plan, Device& device, const teq::TensSetT& targets, RangeTempsT& temps,
+	bool batches, bool forks)
+{
+	forks = forks && forks_enabled();
+	tcg_ctx* ctx = hip_context();
+	const std::vector<LaunchUnit> units = launch_units(plan, batches);
+	const teq::iTensor* forked = nullptr;     // the node whose launch runs on the second stream
+	std::vector<teq::iTensor*> forked_reads;  // what it reads: counted as read when it has been waited for
+	auto join = [&]
+	{
+		hip_check(tcg_join(ctx));
+		for (teq::iTensor* tens : forked_reads) { eigen_ref(*tens).odevice(); }
+		forked_reads.clear();
+		forked = nullptr;
+	};
+	try
+	{
+		for (size_t u = 0; u < units.size(); ++u)
+		{
+			const LaunchUnit& unit = units[u];
+			if (nullptr != forked)
+			{
+				bool touches = false;
+				for (size_t i = unit.first; i < unit.second && false == touches; ++i) { touches = step_touches(plan, plan.steps[i], forked); }
+				if (touches) { join(); }
+			}
+			const FusionPlan::Step& step = plan.steps[unit.first];
+			if (forks && nullptr == forked && unit.second - unit.first == 1 && step.conv >= 0)
+			{
+				// a convolution whose result nothing reads before another product has been
+				// launched: the two run side by side
+				const teq::iTensor* node = plan.convs[step.conv].node;
+				bool beside = false;
+				for (size_t i = unit.second; i < plan.steps.size() && false == step_touches(plan, plan.steps[i], node); ++i)
+				{
+					beside = beside || heavy_step(plan.steps[i]);
+				}
+				if (beside)
+				{
+					hip_check(tcg_fork(ctx));
+					forked = node;
+					launch_conv(plan.convs[step.conv], targets, device.memory(), &forked_reads);
+					hip_check(tcg_fork_end(ctx));
+					continue;
+				}
+			}
+			launch_unit(plan, unit, device, targets, temps);
+		}
+		if (nullptr != forked) { join(); }
+	}
+	catch (...)
+	{
+		(void) tcg_join(ctx);
+		throw;
+	}
 }
 
 void launch_step (const FusionPlan& plan, const FusionPlan::Step& step, Device& device, const teq::TensSetT& targets,
@@ -2495,7 +2656,8 @@ void launch_parts (const PartProducts& call, const teq::TensSetT& targets, RTMem
 	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
 }
 
-void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory)
+void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptrT& memory,
+	std::vector<teq::iTensor*>* later_reads)
 {
 	Observable* out = call.node;
 	size_t ttl = std::max<size_t>(1, out->nsubs() + (size_t) (targets.count(out) > 0));
@@ -2529,7 +2691,8 @@ void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptr
 		ref.drop();
 		throw;
 	}
-	for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); }
+	if (nullptr != later_reads) { later_reads->insert(later_reads->end(), call.reads.begin(), call.reads.end()); }
+	else { for (teq::iTensor* tens : call.reads) { eigen_ref(*tens).odevice(); } }
 }
 
 /// The product of `call` with `group` as its epilogue, one launch; false when

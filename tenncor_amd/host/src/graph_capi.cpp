@@ -465,7 +465,7 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 		for (int i = 0; i < ntargets; ++i) { key.push_back(g->at(targets[i]).get()); }
 		tset.insert(key.begin(), key.end());
 		std::sort(key.begin(), key.end());
-		teq::multi_visit(collector, key);
+		teq::multi_visit(collector, eigen::birth_order(key));
 		eigen::FusionPlan plan = eigen::plan_fusion(collector.funcs, tset);
 		std::stringstream ss;
 		// "batch N": the N steps that follow are small and go out as one launch

@@ -1,6 +1,7 @@
 // Recording and replaying whole evaluation passes (see replay_eval.hpp).
 #include "replay_eval.hpp"
 
+#include <limits>
 #include <unordered_map>
 #include "fuse_plan.hpp"
 
@@ -236,7 +237,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 	double jit0 = 0.0;
 	tcg_jit_stats(hip_context(), &compiled0, &disk0, &jit0);
 	Collector collector;
-	teq::multi_visit(collector, key);
+	teq::multi_visit(collector, birth_order(key));
 	if (collector.funcs_.empty()) { return nullptr; }
 	auto plan = std::make_unique<Plan>();
 	plan->funcs = collector.funcs_;
@@ -297,7 +298,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 			}
 			else
 			{
-				for (auto& unit : launch_units(fusion, small_passes_)) { launch_unit(fusion, unit, device, targets, temps); }
+				launch_pass(fusion, device, targets, temps, small_passes_, small_passes_);
 			}
 		}
 		catch (const std::exception& err)

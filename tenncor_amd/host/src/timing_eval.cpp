@@ -42,7 +42,7 @@ void TimingEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 	key.erase(std::remove(key.begin(), key.end(), nullptr), key.end());
 	std::sort(key.begin(), key.end());
 	Collector collector;
-	teq::multi_visit(collector, key);
+	teq::multi_visit(collector, birth_order(key));
 	bool launchable = false == collector.funcs_.empty();
 	for (Observable* f : collector.funcs_)
 	{
