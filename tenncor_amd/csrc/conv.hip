@@ -519,7 +519,14 @@ bool conv_gemm_plan (const ConvPlan& c, ConvGemmPlan& g)
 	return true;
 }
 
-// Orders of the three indices once the strides are final (see ConvGemmPlan)
+// Orders of the three indices once the strides are final (see ConvGemmPlan).
+// (Rows enumerated batch first, so that the rows of a tile of the product sit at
+// one position of the padded dims and the tile can leave out the slabs of the
+// summed index that meet nothing but zero border -- 31% of them for the image
+// gradient of a 5x5 convolution over 20x20 outputs -- were measured slower than
+// multiplying the zeros: 111.4 against 104.7 us.  The rows of such a tile lie a
+// whole image apart, and nothing a slab loads is found in L1 again by the next
+// kernel position, as it is when neighbouring rows are neighbouring pixels.)
 void conv_choose_orders (ConvGemmPlan& g)
 {
 	if (g.ncheck < 0) { return; } // the general gather decomposes in dim order
