@@ -280,7 +280,7 @@ def time_matmul_4096(ctx, capi, a, b, c, settle, reps):
     return {
         "matmul_4096_fp32_TFLOPs": round(tf, 2), "matmul_4096_fp32_ms": round(ms, 4),
         "matmul_4096_frac_of_fp32_mfma_peak": round(tf / MFMA_F32_PEAK_TFLOPS, 4),
-        "roofline_matmul": {"bound": "mfma", "kernel": "gemm_mfma_direct_k<128, 128, false, false> on 4096^3 fp32",
+        "roofline_matmul": {"bound": "mfma", "kernel": "gemm_mfma_direct_k (128 x 128 tiles, slabs from memory straight into LDS) on 4096^3 fp32",
                             "flops": flops, "avg_ms": round(ms, 4), "achieved": round(tf, 2),
                             "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_F32_PEAK_TFLOPS, 4),
                             "launches": reps, "untimed_launches_before": settle},

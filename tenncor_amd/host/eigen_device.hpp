@@ -68,50 +68,46 @@ struct RuntimeMemory final : public iRuntimeMemory
 void set_runtime (RTMemptrT mem, global::CfgMapptrT ctx = global::context());
 RTMemptrT get_runtime (const global::CfgMapptrT& ctx = global::context());
 
-/// A borrowed buffer that returns itself after `ttl` consumer reads
+/// The buffer a functor's value lives in, on loan from the runtime memory for a
+/// number of reads (internal/eigen/memory.hpp:60-115): every consumer that has
+/// read the value ticks once, and the tick that uses up the last read hands the
+/// buffer back.  Names and error texts are the reference's (its tests name them).
 template <typename T>
 struct Expirable final
 {
-	void expire (void)
-	{
-		if (ptr_ != nullptr)
-		{
-			allocator_->deallocate(ptr_, size_);
-			ptr_ = nullptr;
-			size_ = 0;
-			allocator_ = nullptr;
-		}
-		ttl_ = 0;
-	}
+	T* get (void) { return loan_.ptr; }
 
-	void tick (void)
-	{
-		if (ttl_ > 0 && 0 == (--ttl_)) { expire(); }
-	}
+	size_t get_ttl (void) const { return reads_left_; }
 
-	bool is_expired (void) const { return 0 == ttl_; }
-
-	size_t get_ttl (void) const { return ttl_; }
-
-	T* get (void) { return ptr_; }
+	bool is_expired (void) const { return 0 == reads_left_; }
 
 	void borrow (RTMemptrT& memory, size_t nelems, size_t ttl)
 	{
 		if (nullptr == memory) { global::fatal("cannot borrow from null memory"); }
-		if (false == is_expired())
-		{
-			global::throw_err("cannot borrow memory when Expirable is not expired");
-		}
-		size_ = sizeof(T) * nelems;
-		ptr_ = (T*) memory->allocate(size_);
-		allocator_ = memory;
+		if (reads_left_ > 0) { global::throw_err("cannot borrow memory when Expirable is not expired"); }
+		const size_t bytes = nelems * sizeof(T);
+		loan_ = Loan{static_cast<T*>(memory->allocate(bytes)), bytes, memory};
 		extend_life(ttl);
 	}
 
+	/// The count only ever grows here: a second reader asking for fewer reads
+	/// than are already promised changes nothing
 	void extend_life (size_t ttl)
 	{
-		if (nullptr == ptr_) { global::fatal("cannot extend ttl of expired Expirable"); }
-		if (ttl_ < ttl) { ttl_ = ttl; }
+		if (nullptr == loan_.ptr) { global::fatal("cannot extend ttl of expired Expirable"); }
+		reads_left_ = std::max(reads_left_, ttl);
+	}
+
+	void tick (void)
+	{
+		if (0 == reads_left_) { return; }
+		if (0 == --reads_left_) { give_back(); }
+	}
+
+	void expire (void)
+	{
+		give_back();
+		reads_left_ = 0;
 	}
 
 	/// Become the owner of `ptr` (a buffer a replayed launch sequence has just
@@ -123,21 +119,30 @@ struct Expirable final
 			expire();
 			return;
 		}
-		if (ptr_ != ptr)
+		if (loan_.ptr != ptr)
 		{
-			expire();
-			ptr_ = ptr;
-			size_ = sizeof(T) * nelems;
-			allocator_ = memory;
+			give_back();
+			loan_ = Loan{ptr, nelems * sizeof(T), memory};
 		}
-		ttl_ = ttl;
+		reads_left_ = ttl;
 	}
 
 private:
-	size_t ttl_ = 0;
-	T* ptr_ = nullptr;
-	size_t size_ = 0;
-	RTMemptrT allocator_ = nullptr;
+	struct Loan final
+	{
+		T* ptr = nullptr;
+		size_t bytes = 0;
+		RTMemptrT owner = nullptr;
+	};
+
+	void give_back (void)
+	{
+		if (nullptr != loan_.ptr) { loan_.owner->deallocate(loan_.ptr, loan_.bytes); }
+		loan_ = Loan();
+	}
+
+	Loan loan_;
+	size_t reads_left_ = 0;
 };
 
 // ---- metadata (internal/eigen/emeta.hpp) -----------------------------------
