@@ -244,13 +244,16 @@ def run_extras(ctx, capi):
     b = ctx.upload((rng.standard_normal(nb * m * m) / np.sqrt(m)).astype(np.float32))
     c = ctx.empty(nb * m * m, np.float32)
     d = ctx.empty(nb * m * m, np.float32)
-    for _ in range(40):
+    # (300 untimed launches: the same 40 ms of matrix work that settle the clock before
+    # the 4096^3 product is timed; 40 launches, 6 ms, read 107-110 TFLOP/s on the way up)
+    for _ in range(300):
         ctx.matmul(capi.FLOAT, [m, m, nb], [m, m, nb], a.ptr, b.ptr, c.ptr)
     ctx.timer_begin()
     for _ in range(reps):
         ctx.matmul(capi.FLOAT, [m, m, nb], [m, m, nb], a.ptr, b.ptr, c.ptr)
     ms = ctx.timer_end() / reps
     extra["matmul_64x512_fp32_TFLOPs"] = round(nb * 2.0 * m ** 3 / (ms * 1e-3) / 1e12, 2)
+    extra["matmul_64x512_untimed_launches_before"] = 300
     order = [1, 0, 2, 3, 4, 5, 6, 7]
     for _ in range(2):
         ctx.permute(capi.FLOAT, [m, m, nb], order, c.ptr, d.ptr)
@@ -287,15 +290,35 @@ def time_matmul_4096(ctx, capi, a, b, c, settle, reps):
     }
 
 
-def run_matmul_only(settle=100, reps=100, f64=False):
+def run_matmul_only(settle=100, reps=100, f64=False, batched=None):
     """The product third of the metric alone: nothing but 4096^3 fp32 launches in
     the process, so that a kernel trace or a counter run of this command holds
     one kernel at one shape.  f64: the same product in double (not part of the
-    metric; its line has no roofline_matmul object)."""
+    metric; its line has no roofline_matmul object).  batched = (count, size):
+    the batched CONTRACT of configs[2] alone (the untimed launches settle the
+    matrix clock: 300 of 64 x 512^3 are 45 ms of matrix work)."""
     from tenncor_amd import capi
     ctx = capi.Context(0)
     M = 4096
     rng = np.random.default_rng(3)
+    if batched:
+        nb, m = batched
+        a = ctx.upload((rng.standard_normal(nb * m * m) / np.sqrt(m)).astype(np.float32))
+        b = ctx.upload((rng.standard_normal(nb * m * m) / np.sqrt(m)).astype(np.float32))
+        c = ctx.empty(nb * m * m, np.float32)
+        shape = [m, m, nb]
+        for _ in range(settle):
+            ctx.matmul(capi.FLOAT, shape, shape, a.ptr, b.ptr, c.ptr)
+        ctx.timer_begin()
+        for _ in range(reps):
+            ctx.matmul(capi.FLOAT, shape, shape, a.ptr, b.ptr, c.ptr)
+        ms = ctx.timer_end() / reps
+        tf = nb * 2.0 * m ** 3 / (ms * 1e-3) / 1e12
+        out = {"matmul_batched": "%d x %d^3 fp32" % (nb, m), "TFLOPs": round(tf, 2), "ms": round(ms, 4),
+               "frac_of_fp32_mfma_peak": round(tf / MFMA_F32_PEAK_TFLOPS, 4), "launches": reps,
+               "untimed_launches_before": settle, "device": ctx.arch}
+        ctx.close()
+        return out
     if f64:
         a = ctx.upload(rng.standard_normal(M * M) / 64)
         b = ctx.upload(rng.standard_normal(M * M) / 64)
@@ -636,6 +659,8 @@ def main():
                     help="with --graph-config; timing: the recording's launches run one by one between HIP events, "
                          "device microseconds per kind of launch in the line's timing_report")
     ap.add_argument("--f64", action="store_true", help="with --matmul-only: the 4096^3 product in double")
+    ap.add_argument("--batched", default=None, metavar="COUNTxSIZE",
+                    help="with --matmul-only: COUNT products of SIZE^3 in one launch (64x512 is the batched CONTRACT of configs[2])")
     ap.add_argument("--reps", type=int, default=None,
                     help="timed evaluations with --graph-config 4 or 5 (default 20), timed launches with --matmul-only (100)")
     ap.add_argument("--optimize", action="store_true",
@@ -654,7 +679,8 @@ def main():
         print(json.dumps(run_matmul_ramp()))
         return
     if args.matmul_only:
-        print(json.dumps(run_matmul_only(settle=args.settle, reps=args.reps or 100, f64=args.f64)))
+        batched = tuple(int(v) for v in args.batched.lower().split("x")) if args.batched else None
+        print(json.dumps(run_matmul_only(settle=args.settle, reps=args.reps or 100, f64=args.f64, batched=batched)))
         return
     if args.graph_config is not None:
         print(json.dumps(run_graph_configs(only=args.graph_config, evaluator=args.evaluator, reps=args.reps or 20, optimize=args.optimize)))
