@@ -43,6 +43,12 @@ int tcr_variable (tcr_graph* g, int dtype, const uint64_t shape[8], const void* 
 int tcr_constant (tcr_graph* g, int dtype, const uint64_t shape[8], const void* data, int* node);
 /* Variable<T>::assign(data) -- tenncor/eteq/variable.hpp:72-90 */
 int tcr_assign (tcr_graph* g, int variable, const void* data);
+/* Brings the device copy of a leaf up to date now (one host-to-device copy when
+ * the host copy is newer, nothing otherwise) instead of at the next evaluation
+ * that reads it: a caller that assigns the next batch while the device still
+ * runs the last one keeps the copy out of the evaluation's time.  What the
+ * reference has no need for: its leaves are read where they lie. */
+int tcr_prefetch (tcr_graph* g, int leaf);
 
 /* eteq::make_funcattr(opcode, children, attrs) -- tenncor/eteq/src/make.cpp:14-29.
  * Attribute i has key keys[i] and the integer list vals[i][0..lens[i]);

@@ -29,7 +29,7 @@ RANK_CAP = 8
 DIM_MAX = 65535  # std::numeric_limits<teq::DimT>::max()
 
 EXPORTS = [
-    "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign",
+    "tcr_last_error", "tcr_graph_create", "tcr_graph_destroy", "tcr_variable", "tcr_constant", "tcr_assign", "tcr_prefetch",
     "tcr_functor", "tcr_derive", "tcr_local_derivative", "tcr_evaluate", "tcr_evaluate_ignoring", "tcr_sync", "tcr_shape", "tcr_dtype", "tcr_data",
     "tcr_version", "tcr_opcode", "tcr_nargs", "tcr_args", "tcr_to_string", "tcr_count_functors",
     "tcr_set_evaluator", "tcr_evaluator_stats", "tcr_evaluator_record_error", "tcr_evaluator_record_cost", "tcr_evaluator_timing", "tcr_attr", "tcr_launch_plan", "tcr_optimize",
@@ -65,6 +65,7 @@ def load():
         "tcr_variable": [vp, i32, u64p, vp, ctypes.c_char_p, i32p],
         "tcr_constant": [vp, i32, u64p, vp, i32p],
         "tcr_assign": [vp, i32, vp],
+        "tcr_prefetch": [vp, i32],
         "tcr_functor": [vp, i32, i32, i32p, i32, ctypes.POINTER(ctypes.c_char_p),
                         ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)), i32p, i32p],
         "tcr_derive": [vp, i32, i32, i32p, i32p],
@@ -235,6 +236,10 @@ class Graph:
         data = np.ascontiguousarray(data, dtype=capi.NP_OF[var.dtype]).reshape(-1)
         assert data.size == capi.n_elems(var.shape)
         self._check(self.lib.tcr_assign(self.h, var.id, data.ctypes.data))
+
+    def prefetch(self, leaf):
+        """Copy the leaf's value to the device now rather than inside the next evaluation."""
+        self._check(self.lib.tcr_prefetch(self.h, leaf.id))
 
     # ---- functors ----
     def functor(self, op, args, **attrs):

@@ -151,6 +151,16 @@ int tcr_assign (tcr_graph* g, int variable, const void* data)
 	});
 }
 
+int tcr_prefetch (tcr_graph* g, int leaf)
+{
+	return guarded([&]
+	{
+		teq::TensptrT tens = g->at(leaf);
+		if (nullptr == dynamic_cast<teq::iLeaf*>(tens.get())) { global::fatalf("node %d is not a leaf", leaf); }
+		(void) eigen::eigen_ref(*tens).device_data();
+	});
+}
+
 int tcr_functor (tcr_graph* g, int opcode, int nargs, const int* args, int nattrs,
 	const char* const* keys, const int64_t* const* vals, const int* lens, int* node)
 {
