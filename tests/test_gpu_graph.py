@@ -541,3 +541,21 @@ def test_optimiser_steps_stay_on_the_device(rule, kw, evaluator):
     finally:
         g.close()
         graph.set_evaluator("default")
+
+
+def test_prefetch_uploads_a_leaf_ahead_of_the_evaluation(g, api):
+    """tcr_prefetch: the device copy of a re-assigned leaf is brought up to date at the call;
+    the evaluation that follows computes from the new value either way, and a functor is refused."""
+    from tenncor_amd import graph
+    x = g.variable(np.arange(12, dtype=np.float32), [4, 3], "x")
+    y = api.square(x)
+    for i in range(4):
+        v = np.arange(12, dtype=np.float32) + i
+        g.assign(x, v)
+        if i % 2:
+            g.prefetch(x)
+            g.prefetch(x)  # nothing left to copy
+        g.evaluate([y])
+        np.testing.assert_array_equal(y.get(), v * v)
+    with pytest.raises(graph.GraphError):
+        g.prefetch(y)
