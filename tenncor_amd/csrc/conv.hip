@@ -330,43 +330,13 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_tables_k (ConvGemmPlan p, ConvT
 	}
 }
 
-constexpr int CG_ROWS = 16;
-
-// A[m - m0][s] from the two tables: one summed index per lane, CG_ROWS rows per workgroup
-template <typename T, int NCHECK>
-__global__ __launch_bounds__(CG_BLOCK) void conv_gather_tab_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
-	const ConvTabEntry* __restrict__ rowtab, const ConvTabEntry* __restrict__ sumtab,
-	const T* __restrict__ img, T* __restrict__ A)
-{
-	const uint32_t s = blockIdx.x * CG_BLOCK + threadIdx.x;
-	if (s >= p.Sp) { return; }
-	const ConvTabEntry col = sumtab[s];
-	const bool pad_col = s >= p.S;
-	const uint32_t r0 = blockIdx.y * CG_ROWS;
-#pragma unroll 4
-	for (uint32_t r = r0; r < r0 + CG_ROWS && r < rows; ++r)
-	{
-		const ConvTabEntry row = rowtab[m0 + r];
-		bool inside = !pad_col;
-#pragma unroll
-		for (int j = 0; j < NCHECK; ++j)
-		{
-			inside = inside && (uint32_t) (row.c[j] + col.c[j]) < p.check_ext[j];
-		}
-		T v = 0;
-		if (inside) { v = img[row.off + col.off]; }
-		A[(uint64_t) r * p.Sp + s] = v;
-	}
-}
-
-// B[s][n]
+// B[s][n], elements first, first + step, ...
 template <typename T>
-__global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_k (ConvGemmPlan p,
-	const T* __restrict__ ker, T* __restrict__ B)
+__device__ __forceinline__ void conv_gather_kernel_part (const ConvGemmPlan& p, const T* __restrict__ ker, T* __restrict__ B,
+	uint64_t first, uint64_t step)
 {
 	const uint64_t total = (uint64_t) p.Sp * p.Np;
-	const uint64_t step = (uint64_t) gridDim.x * CG_BLOCK;
-	for (uint64_t i = (uint64_t) blockIdx.x * CG_BLOCK + threadIdx.x; i < total; i += step)
+	for (uint64_t i = first; i < total; i += step)
 	{
 		uint32_t s = (uint32_t) (i / p.Np);
 		uint32_t n = (uint32_t) (i - (uint64_t) s * p.Np);
@@ -403,6 +373,80 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_k (ConvGemmPlan p
 			if (valid) { v = ker[off]; }
 		}
 		B[i] = v;
+	}
+}
+
+template <typename T>
+__global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_k (ConvGemmPlan p,
+	const T* __restrict__ ker, T* __restrict__ B)
+{
+	conv_gather_kernel_part<T>(p, ker, B, (uint64_t) blockIdx.x * CG_BLOCK + threadIdx.x, (uint64_t) gridDim.x * CG_BLOCK);
+}
+
+constexpr int CG_ROWS = 16;
+constexpr int CG_NARROW_ROWS = 128; // rows per workgroup when the summed index is at most CG_BLOCK / 2 long
+
+// A[m - m0][s] from the two tables: one summed index per lane, CG_ROWS rows per workgroup.
+// With `B`: the workgroups behind those of the rows (blockIdx.y >= row_blocks, blockIdx.x == 0)
+// gather the kernel as well, which saves its launch where both operands are laid out
+template <typename T, int NCHECK>
+__global__ __launch_bounds__(CG_BLOCK) void conv_gather_tab_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
+	const ConvTabEntry* __restrict__ rowtab, const ConvTabEntry* __restrict__ sumtab,
+	const T* __restrict__ img, T* __restrict__ A, uint32_t row_blocks, const T* __restrict__ ker, T* __restrict__ B)
+{
+	if (blockIdx.y >= row_blocks)
+	{
+		if (blockIdx.x == 0)
+		{
+			conv_gather_kernel_part<T>(p, ker, B, (uint64_t) (blockIdx.y - row_blocks) * CG_BLOCK + threadIdx.x,
+				(uint64_t) (gridDim.y - row_blocks) * CG_BLOCK);
+		}
+		return;
+	}
+	if (p.Sp <= CG_BLOCK / 2)
+	{
+		// a short summed index (a 5x5 window over one channel: 28 columns) would leave
+		// most lanes of a workgroup without a column: the lanes walk the CG_ROWS x Sp
+		// elements of the workgroup's rows in memory order instead
+		// (CG_NARROW_ROWS rows per workgroup: every lane has several independent elements in flight)
+		const uint32_t r0 = blockIdx.y * CG_NARROW_ROWS;
+		const uint32_t count = (rows - r0 < (uint32_t) CG_NARROW_ROWS ? rows - r0 : (uint32_t) CG_NARROW_ROWS) * p.Sp;
+#pragma unroll 4
+		for (uint32_t i = threadIdx.x; i < count; i += CG_BLOCK)
+		{
+			const uint32_t r = i / p.Sp, s = i - r * p.Sp;
+			const ConvTabEntry row = rowtab[m0 + r0 + r];
+			const ConvTabEntry col = sumtab[s];
+			bool inside = s < p.S;
+#pragma unroll
+			for (int j = 0; j < NCHECK; ++j)
+			{
+				inside = inside && (uint32_t) (row.c[j] + col.c[j]) < p.check_ext[j];
+			}
+			T v = 0;
+			if (inside) { v = img[row.off + col.off]; }
+			A[(uint64_t) (r0 + r) * p.Sp + s] = v;
+		}
+		return;
+	}
+	const uint32_t s = blockIdx.x * CG_BLOCK + threadIdx.x;
+	if (s >= p.Sp) { return; }
+	const ConvTabEntry col = sumtab[s];
+	const bool pad_col = s >= p.S;
+	const uint32_t r0 = blockIdx.y * CG_ROWS;
+#pragma unroll 4
+	for (uint32_t r = r0; r < r0 + CG_ROWS && r < rows; ++r)
+	{
+		const ConvTabEntry row = rowtab[m0 + r];
+		bool inside = !pad_col;
+#pragma unroll
+		for (int j = 0; j < NCHECK; ++j)
+		{
+			inside = inside && (uint32_t) (row.c[j] + col.c[j]) < p.check_ext[j];
+		}
+		T v = 0;
+		if (inside) { v = img[row.off + col.off]; }
+		A[(uint64_t) r * p.Sp + s] = v;
 	}
 }
 
@@ -743,11 +787,6 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 		const T* Bmat = direct_b ? ker + b_base : (const T*) B;
 		const uint64_t ldb = direct_b ? (uint64_t) b_ld : g.Np;
 		const uint64_t ldc = direct_c ? (uint64_t) c_ld : g.Np;
-		if (false == direct_b)
-		{
-			grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
-			conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
-		}
 		if (fill_tables)
 		{
 			uint32_t longest = g.M > g.Sp ? g.M : g.Sp;
@@ -771,6 +810,15 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			// 285 vs 300 us for both steps, but 214-253 vs 76 us on a kernel gradient
 			// with 25 rows, whichever index ran along the lanes)
 			implicit = operand.vec4;
+		}
+		// the kernel laid out as B: by a launch of its own, or by the workgroups that the
+		// launch which lays out the first rows of A has left over
+		bool gather_b = false == direct_b;
+		if (gather_b && (implicit || false == tables))
+		{
+			grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
+			conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
+			gather_b = false;
 		}
 		for (uint32_t m0 = 0; m0 < g.M && rc == TCG_OK; m0 += chunk)
 		{
@@ -805,17 +853,27 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			}
 			if (tables)
 			{
-				dim3 tgrid((g.Sp + CG_BLOCK - 1) / CG_BLOCK, (rows + CG_ROWS - 1) / CG_ROWS);
+				const uint32_t per_block = g.Sp <= CG_BLOCK / 2 ? CG_NARROW_ROWS : CG_ROWS;
+				const uint32_t row_blocks = (rows + per_block - 1) / per_block;
+				uint32_t kernel_blocks = 0;
+				if (gather_b)
+				{
+					kernel_blocks = (uint32_t) (((uint64_t) g.Sp * g.Np + CG_BLOCK - 1) / CG_BLOCK);
+					if (kernel_blocks > 1024) { kernel_blocks = 1024; }
+				}
+				dim3 tgrid((g.Sp + CG_BLOCK - 1) / CG_BLOCK, row_blocks + kernel_blocks);
 				const ConvTabEntry* rt = (const ConvTabEntry*) RT;
 				const ConvTabEntry* st = (const ConvTabEntry*) ST;
+				const T* kb = gather_b ? ker : nullptr;
 				switch (g.ncheck)
 				{
-					case 0: conv_gather_tab_k<T,0><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
-					case 1: conv_gather_tab_k<T,1><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
-					case 2: conv_gather_tab_k<T,2><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
-					case 3: conv_gather_tab_k<T,3><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
-					default: conv_gather_tab_k<T,4><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A); break;
+					case 0: conv_gather_tab_k<T,0><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A, row_blocks, kb, (T*) B); break;
+					case 1: conv_gather_tab_k<T,1><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A, row_blocks, kb, (T*) B); break;
+					case 2: conv_gather_tab_k<T,2><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A, row_blocks, kb, (T*) B); break;
+					case 3: conv_gather_tab_k<T,3><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A, row_blocks, kb, (T*) B); break;
+					default: conv_gather_tab_k<T,4><<<tgrid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, (T*) A, row_blocks, kb, (T*) B); break;
 				}
+				gather_b = false;
 			}
 			else
 			{

@@ -970,12 +970,16 @@ int small_append_fx (tcg_ctx* ctx, int dtype, const FxArgs& p)
 
 // resolve: the expression the kernel uses for a device pointer of the recording
 template <typename Resolve>
+// stage_cap (batches): bytes of LDS into which a contraction's operands are copied
+// first when they lie in memory and fit -- one coalesced pass of all lanes instead
+// of a round trip to memory per term of every sum
 std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_t feed_bytes, size_t lds_bytes, Resolve resolve,
-	const int block = PASS_BLOCK)
+	const int block = PASS_BLOCK, const size_t stage_cap = 0)
 {
-	std::ostringstream o;
-	fx_emit_prelude(o);
-	o << "struct PassPtrs { void* p[" << std::max<size_t>(1, nptrs) << "]; char feed[" << std::max<size_t>(16, feed_bytes) << "]; };\n"
+	std::ostringstream head, o;
+	size_t stage_need = 0;
+	fx_emit_prelude(head);
+	head << "struct PassPtrs { void* p[" << std::max<size_t>(1, nptrs) << "]; char feed[" << std::max<size_t>(16, feed_bytes) << "]; };\n"
 		"template <typename T> __device__ __forceinline__ T pass_mac (T a, T b, T acc)\n{\n"
 		"if constexpr (is_int<T>::value) { typedef typename wide_unsigned<T>::type W; return (T) ((W) a * (W) b + (W) acc); }\n"
 		"else if constexpr (sizeof(T) == 4) { return __builtin_fmaf(a, b, acc); }\n"
@@ -987,9 +991,9 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 		"u.w[1] = __builtin_amdgcn_ds_bpermute(from, u.w[1]); return u.t; }\n"
 		"else { union { T t; int w; } u; u.w = 0; u.t = v; u.w = __builtin_amdgcn_ds_bpermute(from, u.w); return u.t; }\n}\n"
 		"extern \"C\" __global__ __launch_bounds__(" << block << ") void fx (PassPtrs P)\n{\n";
-	if (lds_bytes) { o << "__shared__ __attribute__((aligned(256))) char lds[" << lds_bytes << "];\n"; }
+	if (lds_bytes) { head << "__shared__ __attribute__((aligned(256))) char lds[" << lds_bytes << "];\n"; }
 	// fed buffers are read where the launch put them: in the argument block
-	o << "const char* feed = (const char*) __builtin_amdgcn_kernarg_segment_ptr() + " << std::max<size_t>(1, nptrs) * sizeof(void*) << ";\n";
+	head << "const char* feed = (const char*) __builtin_amdgcn_kernarg_segment_ptr() + " << std::max<size_t>(1, nptrs) * sizeof(void*) << ";\n";
 	auto lit = [](int64_t v) { return "((int64_t) " + std::to_string(v) + "ll)"; };
 	// index -> coordinates over `n` dims with literal extents, accumulating offsets
 	auto decompose = [&](const char* index, uint32_t n, const uint32_t* size,
@@ -1020,7 +1024,38 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 		else if (s.kind == 1)
 		{
 			const PassContract& c = s.ct;
-			o << "const T* a = (const T*) " << resolve(c.a) << "; const T* b = (const T*) " << resolve(c.b)
+			// elements an operand spans (0: some stride runs backwards, leave it where it is)
+			auto span = [&](const int64_t* ostr, const int64_t* kstr) -> uint64_t
+			{
+				int64_t last = 0;
+				for (uint32_t d = 0; d < c.nod; ++d)
+				{
+					if (ostr[d] < 0) { return 0; }
+					last += (int64_t) (c.osize[d] - 1) * ostr[d];
+				}
+				for (uint32_t d = 0; d < c.nkd; ++d)
+				{
+					if (kstr[d] < 0) { return 0; }
+					last += (int64_t) (c.ksize[d] - 1) * kstr[d];
+				}
+				return (uint64_t) last + 1;
+			};
+			size_t staged = 0;
+			auto in_lds = [&](const void* ptr, uint64_t elems) -> std::string
+			{
+				std::string where = resolve(ptr);
+				size_t bytes = (elems * tcg_type_size(s.dtype) + 15) & ~(size_t) 15;
+				if (0 == elems || where.compare(0, 4, "P.p[") != 0 || staged + bytes > stage_cap) { return where; }
+				o << "for (uint32_t i = threadIdx.x; i < " << elems << "u; i += " << block << ") { ((T*) (stage + " << staged
+					<< "))[i] = ((const T*) " << where << ")[i]; }\n";
+				where = "((void*) (stage + " + std::to_string(staged) + "))";
+				staged += bytes;
+				return where;
+			};
+			const std::string pa = in_lds(c.a, span(c.oastr, c.kastr)), pb = in_lds(c.b, span(c.obstr, c.kbstr));
+			if (staged > 0) { o << "__syncthreads();\n"; }
+			stage_need = std::max(stage_need, staged);
+			o << "const T* a = (const T*) " << pa << "; const T* b = (const T*) " << pb
 				<< "; T* out = (T*) " << resolve(c.out) << ";\n"
 				"for (uint32_t o = threadIdx.x; o < " << c.nout << "u; o += " << block << ")\n{\n"
 				"uint32_t rem = o; int64_t ao = 0, bo = 0;\n";
@@ -1078,7 +1113,8 @@ std::string pass_source (const std::vector<PassStep>& steps, size_t nptrs, size_
 		o << "}\n";
 	}
 	o << "}\n";
-	return o.str();
+	if (stage_need > 0) { head << "__shared__ __attribute__((aligned(256))) char stage[" << stage_need << "];\n"; }
+	return head.str() + o.str();
 }
 
 } // namespace
@@ -1233,7 +1269,9 @@ int tcg_batch_send (tcg_ctx* ctx)
 	};
 	// two passes: the first finds out how much LDS and how many pointers there are
 	(void) pass_source(pass->steps, 1, 0, 0, resolve, BATCH_BLOCK);
-	std::string source = pass_source(pass->steps, slot.size(), 0, lds_bytes, resolve, BATCH_BLOCK);
+	// what the temporaries leave of the 64 KiB a workgroup may declare stages operands of contractions
+	const size_t stage_cap = ((size_t) 64 << 10) - ((lds_bytes + 255) & ~(size_t) 255) - 256;
+	std::string source = pass_source(pass->steps, slot.size(), 0, lds_bytes, resolve, BATCH_BLOCK, stage_cap);
 	hipFunction_t fn = nullptr;
 	FxJit& jit = fx_jit();
 	{
