@@ -125,6 +125,9 @@ struct PartProducts final
 		teq::iTensor* b = nullptr;
 		int64_t a_off = 0, b_off = 0; ///< element offsets of A_t(0, 0) and B_t(0, 0) in them
 		uint64_t lda = 0, ldb = 0;
+		/// >= 0: B_t is read from that copy of `b` with a longer leading dim
+		/// (FusionPlan::padded) by the launch that has the epilogue
+		int b_padded = -1;
 	};
 
 	/// C[c_off + m * ldc + n] = sum_t sum_k A_t(m, k) B_t(k, n), flags as tcg_gemm
@@ -177,6 +180,23 @@ struct FusionPlan final
 	std::vector<ViewedConv> convs;
 	std::vector<SummedContracts> sums;
 	std::vector<PartProducts> part_products;
+	/// A leaf that many products with an epilogue read as their K-contiguous B
+	/// operand under a leading dim that is a multiple of 32 elements (the
+	/// transposed weight of every backward step of an unrolled recurrent layer):
+	/// such a product loads its operands straight into registers in the layout
+	/// of the matrix instruction, sixteen rows a power of two apart per load, and
+	/// runs a quarter faster when the rows are `pad` elements further apart
+	/// (measured: 12.3 -> 9.2 us per step with 16).  The pass makes one copy with
+	/// the longer leading dim in front of the first product that reads it
+	/// (`rows` x `ld` elements, one tcg_pad) and gives it back at its end; it lives
+	/// in the pass's temporaries behind those of part_products.
+	struct PaddedOperand final
+	{
+		teq::iTensor* tensor = nullptr;
+		uint64_t rows = 0, ld = 0, pad = 0;
+		int dtype = 0;
+	};
+	std::vector<PaddedOperand> padded;
 	std::vector<Step> steps;
 	/// functors that are computed inside a group or folded into operand views
 	/// and therefore never hold a value of their own
@@ -199,10 +219,18 @@ FusionPlan plan_fusion (const std::vector<Observable*>& funcs, const teq::TensSe
 /// launch to the last group that reads it
 using RangeTempsT = std::vector<std::pair<void*,size_t>>;
 
+/// An empty set of temporaries for one pass over `plan`: one slot per product
+/// that may leave K ranges, then one per padded operand
+inline RangeTempsT pass_temps (const FusionPlan& plan)
+{
+	return RangeTempsT(plan.part_products.size() + plan.padded.size(), {nullptr, 0});
+}
+
 /// `producer` (with its index into the plan's part_products): the product whose
 /// result only this group reads, launched with it (see FusionPlan::Step)
+/// `plan`: where the padded operands of the producer's terms are described
 void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps,
-	const PartProducts* producer = nullptr, int producer_index = -1);
+	const PartProducts* producer = nullptr, int producer_index = -1, const FusionPlan* plan = nullptr);
 
 void launch_contract (const SwappedContract& call, const teq::TensSetT& targets, RTMemptrT& memory);
 

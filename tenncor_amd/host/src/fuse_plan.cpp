@@ -2092,7 +2092,75 @@ struct Planner final
 				plan.groups[kv.second].reads.push_back(v.arg_tens[0].get());
 			}
 		}
+		pad_shared_operands(plan);
 		return plan;
+	}
+
+	/// TCR_PADDED_OPERANDS=0 leaves every operand where it lies
+	static bool padding_enabled (void)
+	{
+		static const bool on = []
+		{
+			const char* env = getenv("TCR_PADDED_OPERANDS");
+			return !(env && env[0] == '0');
+		}();
+		return on;
+	}
+
+	/// See FusionPlan::PaddedOperand: leaves that eight and more products with an
+	/// epilogue read as a K-contiguous B operand whose rows are a multiple of 32
+	/// elements long, and that nothing in the pass assigns to
+	void pad_shared_operands (FusionPlan& plan) const
+	{
+		if (false == padding_enabled()) { return; }
+		std::set<const teq::iTensor*> assigned;
+		for (const Node& n : nodes_)
+		{
+			if (nullptr != n.f && is_assign((int) n.f->get_opcode().code_)) { assigned.insert(n.f->get_args().front().get()); }
+		}
+		std::map<teq::iTensor*,size_t> uses;
+		auto candidate = [&](const FusionPlan::Step& step, const PartProducts::Term& term) -> bool
+		{
+			if (step.parts < 0 || step.group < 0) { return false; }
+			const PartProducts& call = plan.part_products[step.parts];
+			const PartProducts::Product& p = call.products.at(0);
+			if (false == p.trans_b || call.dtype != (int) egen::FLOAT || nullptr == dynamic_cast<teq::iLeaf*>(term.b)) { return false; }
+			teq::Shape shape = term.b->shape();
+			return term.ldb == shape.at(0) && term.ldb % 32 == 0 && term.ldb >= 256 && shape.n_elems() % term.ldb == 0 &&
+				0 == assigned.count(term.b);
+		};
+		for (const FusionPlan::Step& step : plan.steps)
+		{
+			if (step.parts < 0 || step.group < 0) { continue; }
+			std::set<teq::iTensor*> seen;
+			for (const PartProducts::Term& term : plan.part_products[step.parts].products.at(0).terms)
+			{
+				if (candidate(step, term) && seen.insert(term.b).second) { ++uses[term.b]; }
+			}
+		}
+		std::map<teq::iTensor*,int> index;
+		for (const FusionPlan::Step& step : plan.steps)
+		{
+			if (step.parts < 0 || step.group < 0) { continue; }
+			PartProducts& call = plan.part_products[step.parts];
+			for (PartProducts::Term& term : call.products.at(0).terms)
+			{
+				if (false == candidate(step, term) || uses[term.b] < 8) { continue; }
+				auto it = index.find(term.b);
+				if (it == index.end())
+				{
+					FusionPlan::PaddedOperand op;
+					op.tensor = term.b;
+					op.ld = term.ldb;
+					op.rows = term.b->shape().n_elems() / term.ldb;
+					op.pad = 16;
+					op.dtype = call.dtype;
+					it = index.emplace(term.b, (int) plan.padded.size()).first;
+					plan.padded.push_back(op);
+				}
+				term.b_padded = it->second;
+			}
+		}
 	}
 
 	/// The product (index into part_calls_) that can take the launch of members
@@ -2471,7 +2539,7 @@ void launch_step (const FusionPlan& plan, const FusionPlan::Step& step, Device& 
 	else if (step.sum >= 0) { launch_sum(plan.sums[step.sum], targets, device.memory()); }
 	else if (step.parts >= 0 && step.group >= 0)
 	{
-		launch_group(plan.groups[step.group], targets, device.memory(), temps, &plan.part_products[step.parts], step.parts);
+		launch_group(plan.groups[step.group], targets, device.memory(), temps, &plan.part_products[step.parts], step.parts, &plan);
 	}
 	else if (step.parts >= 0) { launch_parts(plan.part_products[step.parts], targets, device.memory(), temps[step.parts]); }
 	else { launch_group(plan.groups[step.group], targets, device.memory(), temps); }
@@ -2697,8 +2765,30 @@ void launch_conv (const ViewedConv& call, const teq::TensSetT& targets, RTMemptr
 
 /// The product of `call` with `group` as its epilogue, one launch; false when
 /// the kernel does not take the shapes (nothing has been launched then)
+/// The copy of a padded operand (FusionPlan::padded) for this pass: made by the
+/// first launch that asks for it, given back with the pass's temporaries
+static const char* padded_copy (const FusionPlan& plan, int index, RTMemptrT& memory, RangeTempsT& temps)
+{
+	const FusionPlan::PaddedOperand& op = plan.padded.at(index);
+	std::pair<void*,size_t>& slot = temps.at(plan.part_products.size() + (size_t) index);
+	if (nullptr == slot.first)
+	{
+		const void* src = eigen_ref(*op.tensor).device_data();
+		if (nullptr == src) { global::fatalf("operand %s has no data", op.tensor->to_string().c_str()); }
+		size_t bytes = (size_t) (op.rows * (op.ld + op.pad)) * egen::type_size((egen::_GENERATED_DTYPE) op.dtype);
+		void* dst = memory->allocate(bytes);
+		if (nullptr == dst) { global::fatal("no memory for the copy of an operand"); }
+		slot = {dst, bytes};
+		const uint64_t shape[8] = {op.ld, op.rows, 1, 1, 1, 1, 1, 1};
+		const uint64_t before[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+		const uint64_t after[8] = {op.pad, 0, 0, 0, 0, 0, 0, 0};
+		hip_check(tcg_pad(hip_context(), egen::device_type((egen::_GENERATED_DTYPE) op.dtype), shape, before, after, src, dst));
+	}
+	return (const char*) slot.first;
+}
+
 static bool launch_with_epilogue (const PartProducts& call, const FusedGroup& group, int producer_index,
-	const std::vector<void*>& outs)
+	const std::vector<void*>& outs, const FusionPlan* plan, RTMemptrT& memory, RangeTempsT& temps)
 {
 	const PartProducts::Product& p = call.products.at(0);
 	const int64_t esz = (int64_t) egen::type_size((egen::_GENERATED_DTYPE) call.dtype);
@@ -2714,9 +2804,20 @@ static bool launch_with_epilogue (const PartProducts& call, const FusedGroup& gr
 				(nullptr == pa ? term.a : term.b)->to_string().c_str(), call.label.c_str());
 		}
 		a.push_back(pa + esz * term.a_off);
-		b.push_back(pb + esz * term.b_off);
 		lda.push_back(term.lda);
-		ldb.push_back(term.ldb);
+		if (term.b_padded >= 0 && nullptr != plan)
+		{
+			// the same element of the copy: rows are `pad` elements further apart there
+			const FusionPlan::PaddedOperand& op = plan->padded.at(term.b_padded);
+			const int64_t row = term.b_off / (int64_t) op.ld, col = term.b_off % (int64_t) op.ld;
+			b.push_back(padded_copy(*plan, term.b_padded, memory, temps) + esz * (row * (int64_t) (op.ld + op.pad) + col));
+			ldb.push_back(op.ld + op.pad);
+		}
+		else
+		{
+			b.push_back(pb + esz * term.b_off);
+			ldb.push_back(term.ldb);
+		}
 	}
 	std::vector<tcg_fx_leaf> leaves;
 	for (auto& leaf : group.leaves)
@@ -2747,7 +2848,7 @@ static bool launch_with_epilogue (const PartProducts& call, const FusedGroup& gr
 }
 
 void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemptrT& memory, RangeTempsT& temps,
-	const PartProducts* producer, int producer_index)
+	const PartProducts* producer, int producer_index, const FusionPlan* plan)
 {
 	std::vector<void*> outs;
 	for (Observable* out : group.outputs)
@@ -2762,7 +2863,7 @@ void launch_group (const FusedGroup& group, const teq::TensSetT& targets, RTMemp
 		bool done = false;
 		if (nullptr != producer)
 		{
-			done = launch_with_epilogue(*producer, group, producer_index, outs);
+			done = launch_with_epilogue(*producer, group, producer_index, outs, plan, memory, temps);
 			if (false == done)
 			{
 				// two launches after all: the product into temporary memory first

@@ -484,6 +484,9 @@ int tcr_launch_plan (tcr_graph* g, int ntargets, const int* targets, char* out, 
 			if (unit.second - unit.first > 1) { ss << "batch " << unit.second - unit.first << "\n"; }
 			for (size_t i = unit.first; i < unit.second; ++i) { ss << eigen::describe_step(plan, plan.steps[i]) << "\n"; }
 		}
+		// "padded N": leaves that the pass copies once with a longer leading dim for the
+		// products that read them (FusionPlan::padded); only printed when there are any
+		if (false == plan.padded.empty()) { ss << "padded " << plan.padded.size() << "\n"; }
 		ss << "folded " << plan.absorbed.size() << "\n";
 		std::string text = ss.str();
 		if (needed) { *needed = text.size(); }

@@ -289,7 +289,7 @@ std::unique_ptr<ReplayEvaluator::Plan> ReplayEvaluator::record (Device& device, 
 		for (Observable* f : plan->funcs) { f->prop_version(device.max_version_); }
 		hip_check(as_one_kernel ? tcg_capture_begin_small(ctx) : tcg_capture_begin(ctx));
 		bool ok = true;
-		RangeTempsT temps(fusion.part_products.size(), {nullptr, 0});
+		RangeTempsT temps = pass_temps(fusion);
 		try
 		{
 			if (as_one_kernel)

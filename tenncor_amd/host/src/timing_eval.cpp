@@ -76,7 +76,7 @@ void TimingEvaluator::evaluate (teq::iDevice& device, const teq::TensSetT& targe
 	std::vector<LaunchUnit> units = launch_units(plan);
 	std::vector<void*> events(units.size() + 1, nullptr);
 	for (void*& ev : events) { hip_check(tcg_event_create(ctx, &ev)); }
-	RangeTempsT temps(plan.part_products.size(), {nullptr, 0});
+	RangeTempsT temps = pass_temps(plan);
 	auto give_back = [&]
 	{
 		for (auto& temp : temps)

@@ -271,6 +271,8 @@ def parse_plan(lines, batches=None):
             if batches is not None:
                 batches.append((len(steps), int(line.split(" ")[1])))
             continue
+        if line.startswith("padded "):
+            continue
         product, marker, epilogue = line.partition(" with epilogue ")
         if marker:
             # a product and the group that reads it as one launch: both steps, the first one flagged
@@ -545,3 +547,25 @@ def test_launch_plan_reads_a_view_of_a_group_result_in_a_later_launch(g, api):
     # through an IDENTITY (the same coordinates) the value stays in a register
     lines = g.launch_plan([api.add(h, api.identity(h))])
     assert len([l for l in lines if l.startswith("group")]) == 1, lines
+
+
+def test_launch_plan_pads_a_weight_that_many_backward_steps_read():
+    """The transposed weight of the backward steps of an unrolled LSTM (cfg/tenncor/layer.yml:716-768
+    through tenncor/eteq/backprop.hpp:269-359) is read by every step's product as a K-contiguous
+    operand with rows of 4 * hid elements: with nine and more steps and rows of 256 and more the
+    plan lists it as copied once per pass with a longer leading dim; a short sequence, or a leaf the
+    pass assigns to, is left where it lies."""
+    from tenncor_amd import graph, configs
+    for seq, want in ((12, 1), (4, 0)):
+        g = graph.Graph()
+        try:
+            targets, x, w, _ = configs.config4_lstm(g, seq=seq, batch=64, nin=32, hid=64)
+            lines = g.launch_plan(targets)
+            assert sum(int(l.split(" ")[1]) for l in lines if l.startswith("padded ")) == want, lines
+            if want:
+                # a training step in the same pass rewrites the weight: no copy may stand in for it
+                loss, dw = targets
+                lines = g.launch_plan([loss, graph.Api(g).assign_sub(w, dw)])
+                assert not any(l.startswith("padded ") for l in lines), lines
+        finally:
+            g.close()
