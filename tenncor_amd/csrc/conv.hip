@@ -19,7 +19,9 @@
 #include <algorithm>
 #include <cstdint>
 #include <cstdlib>
+#include <string>
 #include <type_traits>
+#include <vector>
 
 namespace
 {
@@ -717,6 +719,119 @@ void conv_operand_mode (const ConvGemmPlan& g, tcg_conv_operand& op)
 	op.vec4 = vec;
 }
 
+// Whether the product can read its A operand out of a patch of the image in LDS
+// (conv_patch.hip), and with which of that kernel's tiles: worked out on the host
+// from the same formulas as the tables.  It pays when the rows of a tile meet
+// the same image elements many times over and the tiles fill the chip evenly.
+tcg_conv_patch conv_patch_prepare (const tcg_ctx* ctx, const ConvGemmPlan& g, const tcg_conv_operand& op)
+{
+	tcg_conv_patch none, pp;
+	if (op.along_m || false == op.vec4 || g.ncheck < 0 || g.ncheck > 2 || g.S != g.Sp || g.S % 32 != 0 || g.S < 128 || g.S > 8192 ||
+		g.N % 32 != 0 || g.N != g.Np || (uint64_t) g.M * g.N * g.S < (1ull << 28))
+	{
+		return none;
+	}
+	const int64_t limit = (int64_t) 1 << 30;
+	// image elements that exist
+	int64_t vlo = 0, vhi = 1;
+	for (int d = 0; d < 8; ++d)
+	{
+		const int64_t first = g.ilo[d], last = g.is_col[d] ? g.ilo[d] : g.ihi[d] - 1;
+		if (g.istr[d] < 0) { return none; }
+		vlo += first * g.istr[d];
+		vhi += last * g.istr[d];
+	}
+	if (vlo % 4 != 0 || vhi % 4 != 0 || vlo < -limit || vhi > limit) { return none; }
+	// offsets of the summed index at the multiples of four
+	int64_t smin = INT64_MAX, smax = INT64_MIN;
+	for (uint32_t s = 0; s < g.S; s += 4)
+	{
+		uint32_t rs = s;
+		int64_t off = 0;
+		for (int j = 0; j < 8; ++j)
+		{
+			const uint32_t d = g.sord[j];
+			const int64_t w = (int64_t) (rs % g.ssize[d]) + g.slo[d];
+			rs /= g.ssize[d];
+			off += w * g.istr[d];
+		}
+		smin = std::min(smin, off);
+		smax = std::max(smax, off);
+	}
+	// offsets of the rows
+	std::vector<int64_t> rowoff(g.M);
+	for (uint32_t m = 0; m < g.M; ++m)
+	{
+		uint32_t rm = m;
+		int64_t off = 0;
+		for (int j = 0; j < 8; ++j)
+		{
+			const uint32_t d = g.mord[j];
+			const int64_t x = rm % g.msize[d];
+			rm /= g.msize[d];
+			off += (g.is_col[d] ? (int64_t) g.ilo[d] : (int64_t) g.xlo[d] + x) * g.istr[d];
+		}
+		if (off < -limit || off > limit || (off + smin) % 4 != 0) { return none; }
+		rowoff[m] = off;
+	}
+	if (smin < -limit || smax > limit) { return none; }
+	// neighbouring rows a power of two apart: padding behind every such stretch keeps
+	// the sixteen rows of a matrix instruction in different banks
+	uint32_t pad_shift = 31;
+	if (g.M > 1)
+	{
+		const int64_t step = rowoff[1] > rowoff[0] ? rowoff[1] - rowoff[0] : rowoff[0] - rowoff[1];
+		if (step >= 16 && step <= 4096 && (step & (step - 1)) == 0)
+		{
+			pad_shift = 0;
+			while (((int64_t) 1 << pad_shift) < step) { ++pad_shift; }
+		}
+	}
+	double best = 0;
+	for (int which = 0; which < tcg_conv_patch_shapes(); ++which)
+	{
+		uint32_t tm = 0, tn = 0, threads = 0;
+		tcg_conv_patch_shape(which, &tm, &tn, &threads);
+		if (g.N % tn != 0) { continue; }
+		int64_t span = 0;
+		for (uint32_t m0 = 0; m0 < g.M; m0 += tm)
+		{
+			const uint32_t m1 = std::min(g.M, m0 + tm);
+			const auto mm = std::minmax_element(rowoff.begin() + m0, rowoff.begin() + m1);
+			span = std::max(span, *mm.second - *mm.first);
+		}
+		const int64_t stretch = span + (smax - smin) + 4;
+		if (stretch > (int64_t) (TCG_CONV_PATCH_LDS / sizeof(float))) { continue; }
+		const uint32_t floats = (uint32_t) (stretch + ((stretch >> pad_shift) << 2) + 4);
+		const size_t lds = tcg_conv_patch_lds(which, floats, g.S, g.ncheck);
+		if (lds > TCG_CONV_PATCH_LDS) { continue; }
+		// elements of A a tile reads per element it copies
+		if ((double) tm * g.S < 4.0 * (double) stretch) { continue; }
+		const uint64_t tiles = (uint64_t) ((g.M + tm - 1) / tm) * (g.N / tn);
+		// how evenly the tiles fall on the CUs (the tiles of a CU share its matrix pipes,
+		// so the CU with the most tiles sets the time); wider tiles read B less often
+		const uint64_t cus = (uint64_t) ctx->num_cus;
+		const uint64_t most = (tiles + cus - 1) / cus;
+		// (a tile as wide as the result copies the stretch of the image once, not once per column of tiles:
+		// 51200 x 64 x 800 took 59.5 us with tiles of 112 x 64 and 66.5 us with 144 x 32)
+		double score = (double) tiles / (double) (most * cus) * (1.0 + tm / 2048.0) * (tn == g.N ? 1.15 : 1.0);
+		if (const char* force = getenv("TCG_CONV_PATCH_SHAPE")) { score = atoi(force) == which ? 10.0 : score * 0.01; } // for measurements
+		if (score > best)
+		{
+			best = score;
+			pp.shape = which;
+			pp.patch_floats = floats;
+		}
+	}
+	if (pp.shape < 0) { return none; }
+	pp.smin = (int32_t) smin;
+	pp.smax = (int32_t) smax;
+	pp.vlo = (int32_t) vlo;
+	pp.vhi = (int32_t) vhi;
+	pp.pad_shift = pad_shift;
+	return pp;
+}
+
 template <typename T>
 int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img, const T* ker, T* out)
 {
@@ -750,6 +865,7 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 	if (rc == TCG_OK && false == direct_c) { rc = tcg_alloc(ctx, c_bytes, &C); }
 	// the tables depend on the plan alone: kept with the context, filled once
 	bool kept_tables = false, fill_tables = tables;
+	tcg_ctx::ConvTables* kept_entry = nullptr;
 	if (rc == TCG_OK && tables)
 	{
 		std::string key((const char*) &g, sizeof(g));
@@ -760,6 +876,7 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			ST = it->second.sums;
 			kept_tables = true;
 			fill_tables = false;
+			kept_entry = &it->second;
 		}
 		else if (ctx->conv_table_bytes + rt_bytes + st_bytes <= tcg_ctx::conv_table_limit)
 		{
@@ -769,7 +886,7 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 				RT = kept.rows;
 				ST = kept.sums;
 				kept_tables = true;
-				ctx->conv_tables.emplace(key, kept);
+				kept_entry = &ctx->conv_tables.emplace(key, kept).first->second;
 				ctx->conv_table_bytes += rt_bytes + st_bytes;
 			}
 			else
@@ -811,6 +928,31 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 			// with 25 rows, whichever index ran along the lanes)
 			implicit = operand.vec4;
 		}
+		// the image's patch in LDS where that pays (TCG_CONV_PATCH=0: never, for tests)
+		tcg_conv_patch patch;
+		const char* patch_env = getenv("TCG_CONV_PATCH");
+		if (implicit && chunk == g.M && !(patch_env && patch_env[0] == '0'))
+		{
+			if (kept_entry && kept_entry->patch_known)
+			{
+				patch.shape = kept_entry->patch_shape;
+				patch.smin = kept_entry->patch_smin; patch.smax = kept_entry->patch_smax;
+				patch.vlo = kept_entry->patch_vlo; patch.vhi = kept_entry->patch_vhi;
+				patch.pad_shift = kept_entry->patch_pad_shift; patch.patch_floats = kept_entry->patch_floats;
+			}
+			else
+			{
+				patch = conv_patch_prepare(ctx, g, operand);
+				if (kept_entry)
+				{
+					kept_entry->patch_known = true;
+					kept_entry->patch_shape = patch.shape;
+					kept_entry->patch_smin = patch.smin; kept_entry->patch_smax = patch.smax;
+					kept_entry->patch_vlo = patch.vlo; kept_entry->patch_vhi = patch.vhi;
+					kept_entry->patch_pad_shift = patch.pad_shift; kept_entry->patch_floats = patch.patch_floats;
+				}
+			}
+		}
 		// the kernel laid out as B: by a launch of its own, or by the workgroups that the
 		// launch which lays out the first rows of A has left over
 		bool gather_b = false == direct_b;
@@ -831,8 +973,17 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 					operand.rows = (const ConvTabEntry*) RT + m0;
 					operand.sums = (const ConvTabEntry*) ST;
 					bool handled = false;
-					rc = tcg_gemm_f32_mfma_conv(ctx, rows, g.Np, g.S, img, operand, (const float*) Bmat, ldb,
-						(float*) Cmat, ldc, &handled);
+					if (patch.shape >= 0 && rows == g.M)
+					{
+						rc = tcg_conv_patch_f32(ctx, rows, g.Np, g.S, img, operand, patch, (const float*) Bmat, ldb,
+							(float*) Cmat, ldc, &handled);
+						if (rc != TCG_OK) { break; }
+					}
+					if (false == handled)
+					{
+						rc = tcg_gemm_f32_mfma_conv(ctx, rows, g.Np, g.S, img, operand, (const float*) Bmat, ldb,
+							(float*) Cmat, ldc, &handled);
+					}
 					if (rc != TCG_OK) { break; }
 					if (handled)
 					{

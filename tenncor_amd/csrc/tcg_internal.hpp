@@ -71,9 +71,19 @@ struct tcg_ctx
 	// again instead of launching the kernel that fills them.  Never evicted
 	// (recorded launches keep their addresses); new plans stop being kept at
 	// conv_table_limit bytes.
-	struct ConvTables { void* rows = nullptr; void* sums = nullptr; };
+	struct ConvTables
+	{
+		void* rows = nullptr;
+		void* sums = nullptr;
+		// what conv_patch.hip needs to know about the plan (worked out on the host, once)
+		bool patch_known = false;
+		int patch_shape = -1;
+		int32_t patch_smin = 0, patch_smax = 0, patch_vlo = 0, patch_vhi = 0;
+		uint32_t patch_pad_shift = 0, patch_floats = 0;
+	};
 	std::map<std::string,ConvTables> conv_tables;
 	size_t conv_table_bytes = 0;
+	uint64_t conv_patch_launches = 0; // products that read the image out of a patch in LDS (conv_patch.hip)
 	// tables first met while launches are being recorded are filled at once on
 	// this stream, so that the recording does not fill them again at every replay
 	hipStream_t side_stream = nullptr;
@@ -208,6 +218,25 @@ struct tcg_conv_operand
 	bool along_m = false;
 	bool vec4 = false;
 };
+
+// The same product with the stretch of the image that the rows of a tile can
+// touch copied into LDS once per workgroup (conv_patch.hip): which of its tile
+// shapes to use (-1: none), the least and greatest offset of the summed index
+// over the multiples of four, the image elements [vlo, vhi) that exist, the
+// distance between neighbouring rows as a shift, and the floats of LDS the
+// padded stretch of the widest tile takes
+struct tcg_conv_patch
+{
+	int shape = -1;
+	int32_t smin = 0, smax = 0, vlo = 0, vhi = 0;
+	uint32_t pad_shift = 31, patch_floats = 0;
+};
+constexpr size_t TCG_CONV_PATCH_LDS = 80 * 1024; // per workgroup: two of them fit a CU
+int tcg_conv_patch_shapes (void);
+void tcg_conv_patch_shape (int which, uint32_t* rows, uint32_t* cols, uint32_t* threads);
+size_t tcg_conv_patch_lds (int which, uint32_t patch_floats, uint64_t S, int ncheck);
+int tcg_conv_patch_f32 (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S, const float* image,
+	const tcg_conv_operand& op, const tcg_conv_patch& pp, const float* B, uint64_t ldb, float* C, uint64_t ldc, bool* handled);
 
 // C[m][n] = sum_s A[m][s] B[s][n] with A read through `op` (never materialised);
 // *handled = false when the shapes do not fit the matrix-core kernel
