@@ -629,14 +629,19 @@ int tcg_conv_views (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const void* box, const int64_t box_stride[8],
 	const void* kernel, const int64_t kernel_stride[8],
 	void* out, const int64_t out_stride[8]);
-/* How many of the context's convolutions so far ran as a matrix product that
- * reads the image out of a patch held in LDS (fp32, the summed index along
- * memory in multiples of 32, 32 or 64 and more result columns, large enough:
- * the forward pass and the image gradient of a conv2d layer over 32 and more
- * channels).  No counterpart in the reference; for tests and for callers who
- * want to know which route their shapes take.  TCG_CONV_PATCH=0 in the
- * environment keeps every convolution off that route. */
-int tcg_conv_patch_launches (const tcg_ctx* ctx, uint64_t* launches);
+/* How many of the context's convolutions so far took one of the two special
+ * routes of the matrix-product lowering (fp32 only):
+ *   patch      the product reads the image out of a patch held in LDS (the summed
+ *              index along memory in multiples of 32, 32 or 64 and more result
+ *              columns, large enough: the forward pass and the image gradient of
+ *              a conv2d layer over 32 and more channels; TCG_CONV_PATCH=0 in the
+ *              environment keeps every convolution off it);
+ *   short_sum  gather, product and the kernel's layout in one launch (at most 32
+ *              summed indices, 16, 32, 48 or 64 columns: a first layer over one
+ *              channel; TCG_CONV_SHORT=0 keeps every convolution off it).
+ * No counterpart in the reference; for tests and for callers who want to know
+ * which route their shapes take. */
+int tcg_conv_route_counts (const tcg_ctx* ctx, uint64_t* patch, uint64_t* short_sum);
 
 #ifdef __cplusplus
 }

@@ -44,7 +44,7 @@ EXPORTS = [
     "tcg_ew_unary", "tcg_ew_binary", "tcg_ew_nary", "tcg_ew_select", "tcg_cast",
     "tcg_assign", "tcg_ew_fused", "tcg_ew_fusedx", "tcg_reduce", "tcg_reduce_noalloc", "tcg_argmax", "tcg_extend", "tcg_permute", "tcg_slice",
     "tcg_pad", "tcg_pad_interior", "tcg_reverse", "tcg_stride", "tcg_scatter", "tcg_concat", "tcg_matmul", "tcg_contract", "tcg_contract_sum",
-    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_jit_stats", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_conv_patch_launches", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort", "tcg_batch_begin", "tcg_batch_end", "tcg_fork", "tcg_fork_end", "tcg_join",
+    "tcg_gemm", "tcg_gemm_terms", "tcg_gemm_terms_ranges", "tcg_gemm_terms_grid", "tcg_gemm_terms_fx", "tcg_jit_stats", "tcg_conv", "tcg_conv_boxed", "tcg_conv_dense_box", "tcg_conv_views", "tcg_conv_route_counts", "tcg_capture_begin", "tcg_capture_begin_small", "tcg_capture_feed", "tcg_graph_feed", "tcg_capture_end", "tcg_capture_abort", "tcg_batch_begin", "tcg_batch_end", "tcg_fork", "tcg_fork_end", "tcg_join",
     "tcg_graph_launch", "tcg_graph_claim", "tcg_graph_stats", "tcg_graph_destroy",
     "tcg_rand_seed", "tcg_rand_state", "tcg_rand_uniform",
 ]
@@ -151,7 +151,7 @@ def load():
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_views": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, i64p, vp, i64p, vp, i64p],
-        "tcg_conv_patch_launches": [vp, u64p],
+        "tcg_conv_route_counts": [vp, u64p, u64p],
         "tcg_capture_begin": [vp],
         "tcg_capture_end": [vp, ctypes.POINTER(vp)],
         "tcg_capture_abort": [vp],
@@ -532,11 +532,12 @@ class Context:
                                             olo, ohi, box, i64(box_stride), kernel, i64(kernel_stride),
                                             dst, i64(out_stride)))
 
-    def conv_patch_launches(self):
-        """Convolutions of this context that ran as a product reading the image out of a patch in LDS."""
-        n = ctypes.c_uint64()
-        self._check(self.lib.tcg_conv_patch_launches(self.handle, ctypes.byref(n)))
-        return n.value
+    def conv_route_counts(self):
+        """Convolutions of this context that ran (a) as a product reading the image out of a patch
+        in LDS, (b) as one launch for a short summed index."""
+        a, b = ctypes.c_uint64(), ctypes.c_uint64()
+        self._check(self.lib.tcg_conv_route_counts(self.handle, ctypes.byref(a), ctypes.byref(b)))
+        return {"patch": a.value, "short_sum": b.value}
 
     def jit_stats(self):
         """Kernels compiled at run time by this process, kernels loaded from the

@@ -280,6 +280,8 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_gather_image_k (ConvGemmPlan p,
 	}
 }
 
+constexpr int64_t CONV_NO_KERNEL = INT64_MIN;
+
 // rows: entry m describes output row m; sums: entry s describes summed index s
 __global__ __launch_bounds__(CG_BLOCK) void conv_tables_k (ConvGemmPlan p, ConvTabEntry* __restrict__ rows,
 	ConvTabEntry* __restrict__ sums)
@@ -329,6 +331,45 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_tables_k (ConvGemmPlan p, ConvT
 		// padding columns of A: a coordinate no row can complete into the box
 		if (i >= p.S) { e.c[0] = INT32_MIN / 2; }
 		sums[i] = e;
+	}
+	// behind the sums: where B[s][n] lies in the kernel, as a part that follows from s
+	// and a part that follows from n (CONV_NO_KERNEL: no such element, B[s][n] = 0)
+	int64_t* ktab = (int64_t*) (sums + p.Sp);
+	if (i < p.Sp)
+	{
+		uint32_t rs = i;
+		int64_t off = 0;
+		bool valid = i < p.S;
+		for (int j = 0; j < 8; ++j)
+		{
+			const uint32_t d = p.sord[j];
+			uint32_t qs = conv_div(rs, p.sdiv[d]);
+			int32_t w = (int32_t) (rs - qs * p.ssize[d]) + p.slo[d];
+			rs = qs;
+			if (p.is_col[d]) { continue; }
+			valid = valid && w >= 0 && w < (int32_t) p.ksize[d];
+			off += (int64_t) w * p.kstr[d];
+		}
+		ktab[i] = valid ? off : CONV_NO_KERNEL;
+	}
+	if (i < p.Np)
+	{
+		uint32_t rn = i;
+		int64_t off = 0;
+		bool valid = i < p.N;
+		for (int j = 0; j < 8; ++j)
+		{
+			const uint32_t d = p.nord[j];
+			uint32_t qn = conv_div(rn, p.ndiv[d]);
+			uint32_t xq = rn - qn * p.nsize[d];
+			rn = qn;
+			if (0 == p.is_col[d]) { continue; }
+			if (p.nflip[d]) { xq = p.nsize[d] - 1 - xq; }
+			int32_t w = p.ilo[d] - (p.xlo[d] + (int32_t) xq);
+			valid = valid && w >= 0 && w < (int32_t) p.ksize[d];
+			off += (int64_t) w * p.kstr[d];
+		}
+		ktab[p.Sp + i] = valid ? off : CONV_NO_KERNEL;
 	}
 }
 
@@ -449,6 +490,118 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_gather_tab_k (ConvGemmPlan p, u
 		T v = 0;
 		if (inside) { v = img[row.off + col.off]; }
 		A[(uint64_t) r * p.Sp + s] = v;
+	}
+}
+
+// The whole product for a short summed index (a 5x5 window over one channel: 25
+// terms) and few columns, in one launch: B is small enough for every wave to hold
+// its share of it in registers for good (v_mfma_f32_16x16x4_f32: SP4 x CB values per
+// lane), gathered from the kernel itself through the offsets kept behind the sum
+// table (`ker`) or read from the matrix (`Bmat`); a wave then gathers the rows of A
+// that belong to 64 output rows straight into the lanes that multiply them.  A is
+// never written to memory, B needs no launch of its own, nothing goes through LDS.
+typedef float conv_f4 __attribute__((ext_vector_type(4)));
+constexpr int CS_MAX_S = 32, CS_MAX_N = 64, CS_RB = 4;
+
+template <int SP4, int CB>
+__global__ __launch_bounds__(CG_BLOCK) void conv_short_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
+	const ConvTabEntry* __restrict__ rowtab, const ConvTabEntry* __restrict__ sumtab, const float* __restrict__ img,
+	const float* __restrict__ ker, const float* __restrict__ Bmat, int64_t ldb, float* __restrict__ C, int64_t ldc, int64_t safe)
+{
+	const uint32_t lane = threadIdx.x & 63u, r16 = lane & 15u, q = lane >> 4;
+	const uint32_t wave = blockIdx.x * (CG_BLOCK / 64) + (threadIdx.x >> 6);
+	const uint32_t first = wave * (16 * CS_RB);
+	if (first >= rows) { return; }
+	// checks beyond the plan's own pass everything (their table entries are zero)
+	uint32_t ext[4];
+#pragma unroll
+	for (int j = 0; j < 4; ++j) { ext[j] = j < p.ncheck ? p.check_ext[j] : 0xffffffffu; }
+	// this lane's summed indices 4 j + q and its share of B
+	ConvTabEntry col[SP4];
+	float b[SP4][CB];
+	const int64_t* ktab = (const int64_t*) (sumtab + p.Sp);
+#pragma unroll
+	for (int j = 0; j < SP4; ++j)
+	{
+		const uint32_t s = 4 * j + q;
+		col[j] = sumtab[s];
+		const int64_t ks = ker ? ktab[s] : 0;
+#pragma unroll
+		for (int cb = 0; cb < CB; ++cb)
+		{
+			const uint32_t n = 16 * cb + r16;
+			if (ker)
+			{
+				const int64_t kn = ktab[p.Sp + n];
+				const bool there = ks != CONV_NO_KERNEL && kn != CONV_NO_KERNEL;
+				const float v = ker[there ? ks + kn : 0];
+				b[j][cb] = there ? v : 0.f;
+			}
+			else { b[j][cb] = Bmat[(int64_t) s * ldb + n]; }
+		}
+	}
+	conv_f4 acc[CS_RB][CB];
+	float a[CS_RB][SP4];
+#pragma unroll
+	for (int rb = 0; rb < CS_RB; ++rb)
+	{
+		const uint32_t r = first + 16 * rb + r16;
+		const bool real = r < rows;
+		const ConvTabEntry row = rowtab[m0 + (real ? r : first)];
+#pragma unroll
+		for (int j = 0; j < SP4; ++j)
+		{
+			bool inside = real & (4 * j + q < p.S);
+#pragma unroll
+			for (int k = 0; k < 4; ++k) { inside = inside & ((uint32_t) (row.c[k] + col[j].c[k]) < ext[k]); }
+			// (every lane loads, from an element that exists when its own lies in the zero border)
+			const float v = img[inside ? row.off + col[j].off : safe];
+			a[rb][j] = inside ? v : 0.f;
+		}
+	}
+#pragma unroll
+	for (int rb = 0; rb < CS_RB; ++rb)
+	{
+#pragma unroll
+		for (int cb = 0; cb < CB; ++cb)
+		{
+			acc[rb][cb] = conv_f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+			for (int j = 0; j < SP4; ++j) { acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[rb][j], b[j][cb], acc[rb][cb], 0, 0, 0); }
+		}
+	}
+	// a lane holds rows 4 q .. 4 q + 3 of column r16 of each block
+#pragma unroll
+	for (int rb = 0; rb < CS_RB; ++rb)
+	{
+		const uint32_t r = first + 16 * rb + 4 * q;
+		float* to = C + (int64_t) r * ldc + r16;
+#pragma unroll
+		for (int cb = 0; cb < CB; ++cb)
+		{
+			if (r < rows) { to[16 * cb] = acc[rb][cb].x; }
+			if (r + 1 < rows) { to[ldc + 16 * cb] = acc[rb][cb].y; }
+			if (r + 2 < rows) { to[2 * ldc + 16 * cb] = acc[rb][cb].z; }
+			if (r + 3 < rows) { to[3 * ldc + 16 * cb] = acc[rb][cb].w; }
+		}
+	}
+}
+
+template <int SP4>
+void conv_short_launch (tcg_ctx* ctx, const ConvGemmPlan& g, uint32_t m0, uint32_t rows, const ConvTabEntry* rt, const ConvTabEntry* st,
+	const float* img, const float* ker, const float* Bmat, int64_t ldb, float* C, int64_t ldc)
+{
+	// an element of the image that exists: the first of its box
+	int64_t safe = 0;
+	for (int d = 0; d < 8; ++d) { safe += (int64_t) g.ilo[d] * g.istr[d]; }
+	const uint32_t per_group = 16 * CS_RB * (CG_BLOCK / 64);
+	const uint32_t groups = (rows + per_group - 1) / per_group;
+	switch (g.Np / 16)
+	{
+		case 1: conv_short_k<SP4,1><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, ker, Bmat, ldb, C, ldc, safe); break;
+		case 2: conv_short_k<SP4,2><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, ker, Bmat, ldb, C, ldc, safe); break;
+		case 3: conv_short_k<SP4,3><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, ker, Bmat, ldb, C, ldc, safe); break;
+		default: conv_short_k<SP4,4><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, rt, st, img, ker, Bmat, ldb, C, ldc, safe); break;
 	}
 }
 
@@ -855,7 +1008,8 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 	size_t a_bytes = sizeof(T) * (size_t) chunk * g.Sp;
 	size_t b_bytes = sizeof(T) * (size_t) g.Sp * g.Np;
 	size_t c_bytes = sizeof(T) * (size_t) chunk * g.Np;
-	size_t rt_bytes = sizeof(ConvTabEntry) * (size_t) g.M, st_bytes = sizeof(ConvTabEntry) * (size_t) g.Sp;
+	size_t rt_bytes = sizeof(ConvTabEntry) * (size_t) g.M;
+	size_t st_bytes = sizeof(ConvTabEntry) * (size_t) g.Sp + sizeof(int64_t) * ((size_t) g.Sp + g.Np); // sums, then kernel offsets
 	void *A = nullptr, *B = nullptr, *C = nullptr, *RT = nullptr, *ST = nullptr;
 	// fp32: the product reads A through the tables, nothing is gathered
 	const char* impl_env = getenv("TCG_CONV_IMPLICIT"); // "0": always materialise A (the parity reference)
@@ -907,6 +1061,7 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 		if (fill_tables)
 		{
 			uint32_t longest = g.M > g.Sp ? g.M : g.Sp;
+			if (g.Np > longest) { longest = g.Np; }
 			hipStream_t where = ctx->stream;
 			if (kept_tables && ctx->capturing)
 			{
@@ -995,6 +1150,36 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 						continue;
 					}
 					implicit = false; // shapes the matrix-core kernel does not take: gather as below
+				}
+			}
+			if constexpr (std::is_same<T,float>::value)
+			{
+				// a short summed index and few columns: gather, product and the kernel's layout in one launch
+				const char* short_env = getenv("TCG_CONV_SHORT"); // "0": gather and multiply (for tests)
+				if (tables && g.Sp <= (uint32_t) CS_MAX_S && g.Np <= (uint32_t) CS_MAX_N && g.Np % 16 == 0 &&
+					!(short_env && short_env[0] == '0'))
+				{
+					const ConvTabEntry* rt = (const ConvTabEntry*) RT;
+					const ConvTabEntry* st = (const ConvTabEntry*) ST;
+					const float* kb = gather_b ? (const float*) ker : nullptr;
+					switch (g.Sp / 4)
+					{
+						case 1: conv_short_launch<1>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						case 2: conv_short_launch<2>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						case 3: conv_short_launch<3>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						case 4: conv_short_launch<4>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						case 5: conv_short_launch<5>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						case 6: conv_short_launch<6>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						case 7: conv_short_launch<7>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+						default: conv_short_launch<8>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
+					}
+					++ctx->conv_short_launches;
+					if (false == direct_c)
+					{
+						grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
+						conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+					}
+					continue;
 				}
 			}
 			if (nullptr == A)

@@ -7,7 +7,8 @@ Checked against the direct kernels (which tests/test_gpu_ops.py ties to the
 oracle) at 1e-4, and against the product that reads the image through its
 tables (TCG_CONV_PATCH=0) -- the two products sum in different orders.  The
 counter of the route says which one ran; shapes the route does not take (a
-summed index that is no multiple of 32) must leave it alone.
+summed index that is no multiple of 32) must leave it alone.  Also here: the
+one-launch route for a short summed index (the CNN's first layer).
 """
 import os
 
@@ -76,11 +77,11 @@ CASES = [
 
 @pytest.mark.parametrize("which,dims", CASES, ids=["%s-%s" % (w, "x".join(str(v) for v in d.values())) for w, d in CASES])
 def test_product_over_a_patch_in_lds_equals_the_direct_kernels(ctx, oracle, which, dims):
-    before = ctx.conv_patch_launches()
+    before = ctx.conv_route_counts()["patch"]
     got = run_views(ctx, oracle, which, dims, {})
-    assert ctx.conv_patch_launches() == before + 1, "the route under test was not taken"
+    assert ctx.conv_route_counts()["patch"] == before + 1, "the route under test was not taken"
     tables = run_views(ctx, oracle, which, dims, {"TCG_CONV_PATCH": "0"})
-    assert ctx.conv_patch_launches() == before + 1
+    assert ctx.conv_route_counts()["patch"] == before + 1
     direct = run_views(ctx, oracle, which, dims, {"TCG_CONV_GEMM": "0"})
     assert_acc_close(got, direct, ACC_RTOL)
     assert_acc_close(got, tables, ACC_RTOL)
@@ -89,9 +90,26 @@ def test_product_over_a_patch_in_lds_equals_the_direct_kernels(ctx, oracle, whic
 
 
 def test_shapes_the_route_does_not_take_leave_it_alone(ctx, oracle):
-    before = ctx.conv_patch_launches()
+    before = ctx.conv_route_counts()["patch"]
     # 16 channels: the summed index (5 x 5 x 16 = 400) is no multiple of 32
     dims = dict(C=16, W=24, H=24, B=32, O=64, KW=5, KH=5)
     got = run_views(ctx, oracle, "forward", dims, {})
-    assert ctx.conv_patch_launches() == before
+    assert ctx.conv_route_counts()["patch"] == before
     assert_acc_close(got, run_views(ctx, oracle, "forward", dims, {"TCG_CONV_GEMM": "0"}), ACC_RTOL)
+
+
+@pytest.mark.parametrize("dims", [dict(C=1, W=28, H=28, B=32, O=32, KW=5, KH=5), dict(C=2, W=17, H=23, B=37, O=64, KW=4, KH=3),
+                                  dict(C=1, W=20, H=20, B=50, O=16, KW=5, KH=5)],
+                         ids=["cnn_first_layer", "two_channels_64_filters", "16_filters"])
+def test_short_summed_index_in_one_launch_equals_the_direct_kernels(ctx, oracle, dims):
+    """The first layer of the reference's CNN (one channel, a 5x5 window: 25 summed indices): gather, product and the
+    layout of the kernel as one launch, against the direct kernels and against gather + product."""
+    before = ctx.conv_route_counts()["short_sum"]
+    got = run_views(ctx, oracle, "forward", dims, {})
+    assert ctx.conv_route_counts()["short_sum"] == before + 1, "the route under test was not taken"
+    two = run_views(ctx, oracle, "forward", dims, {"TCG_CONV_SHORT": "0"})
+    assert ctx.conv_route_counts()["short_sum"] == before + 1
+    direct = run_views(ctx, oracle, "forward", dims, {"TCG_CONV_GEMM": "0"})
+    assert_acc_close(got, direct, ACC_RTOL)
+    assert_acc_close(got, two, ACC_RTOL)
+    np.testing.assert_array_equal(run_views(ctx, oracle, "forward", dims, {}), got)
