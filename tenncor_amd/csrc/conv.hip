@@ -1110,8 +1110,12 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 		}
 		// the kernel laid out as B: by a launch of its own, or by the workgroups that the
 		// launch which lays out the first rows of A has left over
+		// (the latter only for a small kernel behind a launch one workgroup wide: the extra
+		// workgroups are counted along y, and a launch many workgroups wide would start that
+		// many idle ones for each of them -- 498 us for a kernel of 73728 x 32 elements)
 		bool gather_b = false == direct_b;
-		if (gather_b && (implicit || false == tables))
+		const bool fold_b = tables && g.Sp <= (uint32_t) CG_BLOCK && (uint64_t) g.Sp * g.Np <= ((uint64_t) 1 << 16);
+		if (gather_b && (implicit || false == fold_b))
 		{
 			grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
 			conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
