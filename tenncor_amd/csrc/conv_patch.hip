@@ -259,6 +259,9 @@ struct Shape
 };
 
 // the tiles there are kernels for: rows x columns = 16 rbt x 16 cbt
+// (tiles twice as tall, one workgroup and so one wave per SIMD on every CU, were measured on the
+// second layer of the reference's CNN: 208 x 64 forwards 59.6 against 57-59 us, 288 x 32 for the
+// image gradient 93 against 77 us)
 constexpr Shape SHAPES[] = {
 	{9, 2}, // 144 x 32
 	{6, 2}, //  96 x 32
