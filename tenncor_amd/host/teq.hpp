@@ -26,7 +26,14 @@ namespace teq
 // ---- shape (internal/teq/shape.hpp) ----------------------------------------
 
 using RankT = uint8_t;
-using DimT = uint16_t; // SDIM_BYTES default, internal/teq/shape.hpp:27-33
+// the width of a dimension is a build option, as in internal/teq/shape.hpp:27-33
+#if !defined(SDIM_BYTES) || SDIM_BYTES <= 2
+using DimT = uint16_t;
+#elif SDIM_BYTES <= 4
+using DimT = uint32_t;
+#else
+using DimT = uint64_t;
+#endif
 using RanksT = std::vector<RankT>;
 using DimsT = std::vector<DimT>;
 using NElemT = uint64_t;

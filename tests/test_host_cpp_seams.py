@@ -46,3 +46,35 @@ def test_pool_and_arena_lifetimes_on_the_host(tmp_path):
     ran = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert ran.returncode == 0, ran.stdout[-4000:] + ran.stderr[-2000:]
     assert "0 failure(s)" in ran.stdout
+
+
+@pytest.mark.skipif(shutil.which("g++") is None, reason="no host C++ compiler")
+def test_the_build_with_wide_dimensions(tmp_path):
+    """SDIM_BYTES (internal/teq/shape.hpp:27-33) is a build option here as well: the host layer compiled with
+    -DSDIM_BYTES=4 (every source, warnings on) carries a dimension of 70000 through a small graph
+    (tests/cpp/wide_dims.cpp); with -DSDIM_BYTES=8 the headers still compile."""
+    import glob
+    from concurrent.futures import ThreadPoolExecutor
+    if not os.path.exists(os.path.join(PKG, "libtcg.so")):
+        from tenncor_amd import build
+        build.build_all()
+    flags = ["-std=c++17", "-O0", "-Wall", "-Wextra", "-Werror", "-I" + os.path.join(PKG, "host"), "-I" + os.path.join(ROOT, "include")]
+    sources = sorted(glob.glob(os.path.join(PKG, "host", "src", "*.cpp"))) + [os.path.join(ROOT, "tests", "cpp", "wide_dims.cpp")]
+
+    def compile_one(src):
+        obj = str(tmp_path / (os.path.basename(src)[:-4] + ".o"))
+        done = subprocess.run(["g++"] + flags + ["-DSDIM_BYTES=4", "-c", src, "-o", obj], capture_output=True, text=True)
+        assert done.returncode == 0, done.stderr[-4000:]
+        return obj
+
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        objs = list(pool.map(compile_one, sources))
+    exe = str(tmp_path / "wide_dims")
+    linked = subprocess.run(["g++", "-o", exe] + objs + ["-L" + PKG, "-ltcg", "-Wl,-rpath," + PKG], capture_output=True, text=True)
+    assert linked.returncode == 0, linked.stderr[-4000:]
+    ran = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert ran.returncode == 0, ran.stdout[-4000:] + ran.stderr[-2000:]
+    assert "0 failure(s)" in ran.stdout
+    eight = subprocess.run(["g++"] + flags + ["-DSDIM_BYTES=8", "-fsyntax-only", os.path.join(PKG, "host", "src", "teq.cpp"),
+                            os.path.join(PKG, "host", "src", "oprules.cpp")], capture_output=True, text=True)
+    assert eight.returncode == 0, eight.stderr[-4000:]
