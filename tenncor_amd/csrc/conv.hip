@@ -968,7 +968,7 @@ tcg_conv_patch conv_patch_prepare (const tcg_ctx* ctx, const ConvGemmPlan& g, co
 		// (a tile as wide as the result copies the stretch of the image once, not once per column of tiles:
 		// 51200 x 64 x 800 took 59.5 us with tiles of 112 x 64 and 66.5 us with 144 x 32)
 		double score = (double) tiles / (double) (most * cus) * (1.0 + tm / 2048.0) * (tn == g.N ? 1.15 : 1.0);
-		if (const char* force = getenv("TCG_CONV_PATCH_SHAPE")) { score = atoi(force) == which ? 10.0 : score * 0.01; } // for measurements
+		if (const char* force = getenv("TCG_CONV_PATCH_SHAPE")) { score = atoi(force) == which ? 10.0 : score * 0.01; } // for measurements and tests
 		if (score > best)
 		{
 			best = score;

@@ -75,6 +75,16 @@ CASES = [
 ]
 
 
+def test_a_patch_of_more_than_64_kib(ctx, oracle):
+    """Ten rows of 26 pixels x 64 channels under a tile of 144 rows: 78 KiB of LDS, which a kernel has to ask for.
+    (The tile is forced: left alone, this size takes the tile of 96 rows, which fills more CUs.)"""
+    dims = dict(C=32, W=30, H=20, B=16, O=64, KW=5, KH=5)
+    before = ctx.conv_route_counts()["patch"]
+    got = run_views(ctx, oracle, "image_gradient", dims, {"TCG_CONV_PATCH_SHAPE": "0"})
+    assert ctx.conv_route_counts()["patch"] == before + 1, "the route under test was not taken"
+    assert_acc_close(got, run_views(ctx, oracle, "image_gradient", dims, {"TCG_CONV_GEMM": "0"}), ACC_RTOL)
+
+
 @pytest.mark.parametrize("which,dims", CASES, ids=["%s-%s" % (w, "x".join(str(v) for v in d.values())) for w, d in CASES])
 def test_product_over_a_patch_in_lds_equals_the_direct_kernels(ctx, oracle, which, dims):
     before = ctx.conv_route_counts()["patch"]
