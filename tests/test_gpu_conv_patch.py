@@ -72,6 +72,8 @@ CASES = [
     ("image_gradient", dict(C=32, W=22, H=26, B=11, O=64, KW=5, KH=5)),
     ("forward", dict(C=64, W=19, H=17, B=24, O=128, KW=3, KH=4)),
     ("image_gradient", dict(C=64, W=19, H=17, B=36, O=32, KW=3, KH=4)),
+    # a window one row high: only one dim of the image gradient meets a zero border
+    ("image_gradient", dict(C=32, W=40, H=12, B=64, O=64, KW=5, KH=1)),
 ]
 
 
