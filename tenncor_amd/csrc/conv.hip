@@ -880,7 +880,7 @@ tcg_conv_patch conv_patch_prepare (const tcg_ctx* ctx, const ConvGemmPlan& g, co
 {
 	tcg_conv_patch none, pp;
 	if (op.along_m || false == op.vec4 || g.ncheck < 0 || g.ncheck > 2 || g.S != g.Sp || g.S % 32 != 0 || g.S < 128 || g.S > 8192 ||
-		g.N % 32 != 0 || g.N != g.Np || (uint64_t) g.M * g.N * g.S < (1ull << 28))
+		g.N % 32 != 0 || g.N != g.Np || (uint64_t) g.M * g.N * g.S < (1ull << 28) || g.M > (1u << 22)) // (the row offsets are worked out here, once per plan)
 	{
 		return none;
 	}
