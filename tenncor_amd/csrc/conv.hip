@@ -426,6 +426,22 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_k (ConvGemmPlan p
 	conv_gather_kernel_part<T>(p, ker, B, (uint64_t) blockIdx.x * CG_BLOCK + threadIdx.x, (uint64_t) gridDim.x * CG_BLOCK);
 }
 
+// the same from the offsets kept behind the sum table (conv_tables_k): two table reads and one of the kernel per element
+template <typename T>
+__global__ __launch_bounds__(CG_BLOCK) void conv_gather_kernel_tab_k (uint32_t Sp, uint32_t Np, const int64_t* __restrict__ ktab,
+	const T* __restrict__ ker, T* __restrict__ B)
+{
+	const uint32_t total = Sp * Np;
+	for (uint32_t i = blockIdx.x * CG_BLOCK + threadIdx.x; i < total; i += gridDim.x * CG_BLOCK)
+	{
+		const uint32_t s = i / Np, n = i - s * Np;
+		const int64_t ks = ktab[s], kn = ktab[Sp + n];
+		T v = 0;
+		if (ks != CONV_NO_KERNEL && kn != CONV_NO_KERNEL) { v = ker[ks + kn]; }
+		B[i] = v;
+	}
+}
+
 constexpr int CG_ROWS = 16;
 constexpr int CG_NARROW_ROWS = 128; // rows per workgroup when the summed index is at most CG_BLOCK / 2 long
 
@@ -1118,7 +1134,12 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 		if (gather_b && (implicit || false == fold_b))
 		{
 			grid = tcg_grid(ctx, (uint64_t) g.Sp * g.Np, CG_BLOCK, 16);
-			conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B);
+			if (tables && (uint64_t) g.Sp * g.Np < (1ull << 32))
+			{
+				const int64_t* ktab = (const int64_t*) ((const ConvTabEntry*) ST + g.Sp);
+				conv_gather_kernel_tab_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g.Sp, g.Np, ktab, ker, (T*) B);
+			}
+			else { conv_gather_kernel_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, ker, (T*) B); }
 			gather_b = false;
 		}
 		for (uint32_t m0 = 0; m0 < g.M && rc == TCG_OK; m0 += chunk)
