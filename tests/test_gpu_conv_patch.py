@@ -125,3 +125,28 @@ def test_short_summed_index_in_one_launch_equals_the_direct_kernels(ctx, oracle,
     assert_acc_close(got, direct, ACC_RTOL)
     assert_acc_close(got, two, ACC_RTOL)
     np.testing.assert_array_equal(run_views(ctx, oracle, "forward", dims, {}), got)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_seeded_layers_on_the_patch_route(ctx, oracle, seed):
+    """Random conv2d layers whose forward pass or image gradient is large enough for the route: channel counts that make
+    32, 64, 96 or 128 columns (one, two or three columns of tiles), windows of 1..5 x 1..5, images that are not square,
+    batches that leave the last tile ragged."""
+    rng = np.random.default_rng(seed_of("convpatch-random", seed))
+    which = "forward" if seed % 2 == 0 else "image_gradient"
+    KW, KH = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    if KW * KH < 4:
+        KW, KH = 3, 3
+    W, H = int(rng.integers(KW + 8, 31)), int(rng.integers(KH + 8, 31))
+    if which == "forward":
+        C, O = 32 * int(rng.integers(1, 3)), 32 * int(rng.integers(1, 5))      # summed: KW KH C, columns: O
+        rows_per_image, cols, sums = (W - KW + 1) * (H - KH + 1), O, KW * KH * C
+    else:
+        C, O = 32 * int(rng.integers(1, 5)), 32 * int(rng.integers(1, 3))      # summed: KW KH O, columns: C
+        rows_per_image, cols, sums = W * H, C, KW * KH * O
+    B = int(-(-(1 << 28) // (rows_per_image * cols * sums))) + int(rng.integers(0, 3))
+    dims = dict(C=C, W=W, H=H, B=B, O=O, KW=KW, KH=KH)
+    before = ctx.conv_route_counts()["patch"]
+    got = run_views(ctx, oracle, which, dims, {})
+    assert ctx.conv_route_counts()["patch"] == before + 1, "the route under test was not taken: %r" % (dims,)
+    assert_acc_close(got, run_views(ctx, oracle, which, dims, {"TCG_CONV_GEMM": "0"}), ACC_RTOL)
