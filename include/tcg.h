@@ -629,7 +629,7 @@ int tcg_conv_views (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
 	const void* box, const int64_t box_stride[8],
 	const void* kernel, const int64_t kernel_stride[8],
 	void* out, const int64_t out_stride[8]);
-/* How many of the context's convolutions so far took one of the two special
+/* How many of the context's convolutions so far took one of the three special
  * routes of the matrix-product lowering (fp32 only):
  *   patch      the product reads the image out of a patch held in LDS (the summed
  *              index along memory in multiples of 32, 32 or 64 and more result
@@ -638,10 +638,15 @@ int tcg_conv_views (tcg_ctx* ctx, int dtype, const uint64_t imgshape[8],
  *              environment keeps every convolution off it);
  *   short_sum  gather, product and the kernel's layout in one launch (at most 32
  *              summed indices, 16, 32, 48 or 64 columns: a first layer over one
- *              channel; TCG_CONV_SHORT=0 keeps every convolution off it).
+ *              channel; TCG_CONV_SHORT=0 keeps every convolution off it);
+ *   few_rows   at most 32 rows under a summed index of 4096 and more (the kernel
+ *              gradient of such a first layer): A is gathered while it is
+ *              multiplied, stretch by stretch of the summed index, and the
+ *              stretches are added up by a second launch (TCG_CONV_FEWROWS=0
+ *              keeps every convolution off it).
  * No counterpart in the reference; for tests and for callers who want to know
  * which route their shapes take. */
-int tcg_conv_route_counts (const tcg_ctx* ctx, uint64_t* patch, uint64_t* short_sum);
+int tcg_conv_route_counts (const tcg_ctx* ctx, uint64_t* patch, uint64_t* short_sum, uint64_t* few_rows);
 
 #ifdef __cplusplus
 }

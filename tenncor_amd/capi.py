@@ -151,7 +151,7 @@ def load():
         "tcg_conv_boxed": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_dense_box": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, vp, vp],
         "tcg_conv_views": [vp, i32, u64p, u64p, i32, u64p, u64p, u64p, u64p, u64p, vp, i64p, vp, i64p, vp, i64p],
-        "tcg_conv_route_counts": [vp, u64p, u64p],
+        "tcg_conv_route_counts": [vp, u64p, u64p, u64p],
         "tcg_capture_begin": [vp],
         "tcg_capture_end": [vp, ctypes.POINTER(vp)],
         "tcg_capture_abort": [vp],
@@ -534,10 +534,10 @@ class Context:
 
     def conv_route_counts(self):
         """Convolutions of this context that ran (a) as a product reading the image out of a patch
-        in LDS, (b) as one launch for a short summed index."""
-        a, b = ctypes.c_uint64(), ctypes.c_uint64()
-        self._check(self.lib.tcg_conv_route_counts(self.handle, ctypes.byref(a), ctypes.byref(b)))
-        return {"patch": a.value, "short_sum": b.value}
+        in LDS, (b) as one launch for a short summed index, (c) as few rows under a long summed index."""
+        a, b, c = ctypes.c_uint64(), ctypes.c_uint64(), ctypes.c_uint64()
+        self._check(self.lib.tcg_conv_route_counts(self.handle, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+        return {"patch": a.value, "short_sum": b.value, "few_rows": c.value}
 
     def jit_stats(self):
         """Kernels compiled at run time by this process, kernels loaded from the

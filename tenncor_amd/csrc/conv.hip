@@ -621,6 +621,144 @@ void conv_short_launch (tcg_ctx* ctx, const ConvGemmPlan& g, uint32_t m0, uint32
 	}
 }
 
+// Few rows under a very long summed index (the kernel gradient of a first layer:
+// 25 x 32 results, each a sum over 73728 pixels): a workgroup takes a stretch of the
+// summed index, its four waves a quarter each; a lane gathers A[m][s] for its row
+// and its summed index of the step and reads B[s][n] beside it, nothing is laid out
+// in memory first.  The waves' sums meet in LDS in wave order; the workgroups' sums
+// go side by side into `partial` ([workgroup][m][Np]) for conv_ranges_sum_k.
+constexpr int CF_MAX_M = 32, CF_STRETCH = 256;
+
+template <int RB, int CB>
+__global__ __launch_bounds__(CG_BLOCK) void conv_fewrows_k (ConvGemmPlan p,
+	const ConvTabEntry* __restrict__ rowtab, const ConvTabEntry* __restrict__ sumtab, const float* __restrict__ img,
+	const float* __restrict__ Bmat, int64_t ldb, float* __restrict__ partial, int64_t safe)
+{
+	__shared__ conv_f4 meet[3][RB * CB][64];
+	const uint32_t lane = threadIdx.x & 63u, r16 = lane & 15u, q = lane >> 4, wave = threadIdx.x >> 6;
+	uint32_t ext[4];
+#pragma unroll
+	for (int j = 0; j < 4; ++j) { ext[j] = j < p.ncheck ? p.check_ext[j] : 0xffffffffu; }
+	ConvTabEntry row[RB];
+	bool real[RB];
+#pragma unroll
+	for (int rb = 0; rb < RB; ++rb)
+	{
+		const uint32_t m = 16 * rb + r16;
+		real[rb] = m < p.M;
+		row[rb] = rowtab[real[rb] ? m : 0];
+	}
+	conv_f4 acc[RB][CB];
+#pragma unroll
+	for (int rb = 0; rb < RB; ++rb)
+	{
+#pragma unroll
+		for (int cb = 0; cb < CB; ++cb) { acc[rb][cb] = conv_f4{0.f, 0.f, 0.f, 0.f}; }
+	}
+	// a wave's sixteen steps in three sweeps, so that it waits for memory twice, not
+	// twice per step: the table entries of its summed indices, then every element of A
+	// and B, then the matrix instructions
+	constexpr int STEPS = CF_STRETCH / 4 / 4;
+	const uint32_t begin = blockIdx.x * CF_STRETCH + wave * (CF_STRETCH / 4);
+	ConvTabEntry col[STEPS];
+#pragma unroll
+	for (int j = 0; j < STEPS; ++j)
+	{
+		const uint32_t s = begin + 4 * j + q;
+		col[j] = sumtab[s < p.S ? s : 0];
+	}
+	float a[STEPS][RB], b[STEPS][CB];
+#pragma unroll
+	for (int j = 0; j < STEPS; ++j)
+	{
+		const uint32_t s = begin + 4 * j + q;
+		const bool there = s < p.S;
+#pragma unroll
+		for (int rb = 0; rb < RB; ++rb)
+		{
+			bool inside = real[rb] & there;
+#pragma unroll
+			for (int k = 0; k < 4; ++k) { inside = inside & ((uint32_t) (row[rb].c[k] + col[j].c[k]) < ext[k]); }
+			const float v = img[inside ? row[rb].off + col[j].off : safe];
+			a[j][rb] = inside ? v : 0.f;
+		}
+#pragma unroll
+		for (int cb = 0; cb < CB; ++cb)
+		{
+			const float v = Bmat[(int64_t) (there ? s : 0) * ldb + 16 * cb + r16];
+			b[j][cb] = there ? v : 0.f;
+		}
+	}
+#pragma unroll
+	for (int j = 0; j < STEPS; ++j)
+	{
+#pragma unroll
+		for (int rb = 0; rb < RB; ++rb)
+		{
+#pragma unroll
+			for (int cb = 0; cb < CB; ++cb) { acc[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][rb], b[j][cb], acc[rb][cb], 0, 0, 0); }
+		}
+	}
+	if (wave > 0)
+	{
+#pragma unroll
+		for (int rb = 0; rb < RB; ++rb)
+		{
+#pragma unroll
+			for (int cb = 0; cb < CB; ++cb) { meet[wave - 1][rb * CB + cb][lane] = acc[rb][cb]; }
+		}
+	}
+	__syncthreads();
+	if (wave > 0) { return; }
+	float* to = partial + (uint64_t) blockIdx.x * p.M * p.Np;
+#pragma unroll
+	for (int rb = 0; rb < RB; ++rb)
+	{
+#pragma unroll
+		for (int cb = 0; cb < CB; ++cb)
+		{
+			conv_f4 sum = acc[rb][cb];
+#pragma unroll
+			for (int w = 0; w < 3; ++w) { sum += meet[w][rb * CB + cb][lane]; }
+			// a lane holds rows 4 q .. 4 q + 3 of column r16 of the block
+			const uint32_t m = 16 * rb + 4 * q, n = 16 * cb + r16;
+			if (m < p.M) { to[m * p.Np + n] = sum.x; }
+			if (m + 1 < p.M) { to[(m + 1) * p.Np + n] = sum.y; }
+			if (m + 2 < p.M) { to[(m + 2) * p.Np + n] = sum.z; }
+			if (m + 3 < p.M) { to[(m + 3) * p.Np + n] = sum.w; }
+		}
+	}
+}
+
+// C[m][n] = the sum of partial[g][m][n] over g: a wave per result; lane l adds the
+// workgroups l, l + 64, ... in that order, then the 64 lane sums meet in a fixed tree
+__global__ __launch_bounds__(CG_BLOCK) void conv_ranges_sum_k (const float* __restrict__ partial, uint32_t groups, uint32_t M, uint32_t Np,
+	float* __restrict__ C, int64_t ldc)
+{
+	const uint32_t i = blockIdx.x * (CG_BLOCK / 64) + (threadIdx.x >> 6), lane = threadIdx.x & 63u;
+	if (i >= M * Np) { return; }
+	float acc = 0.f;
+	for (uint32_t g = lane; g < groups; g += 64) { acc += partial[(uint64_t) g * M * Np + i]; }
+#pragma unroll
+	for (int w = 32; w >= 1; w >>= 1) { acc += __shfl_xor(acc, w, 64); }
+	if (lane == 0) { C[(int64_t) (i / Np) * ldc + i % Np] = acc; }
+}
+
+template <int RB>
+void conv_fewrows_launch (tcg_ctx* ctx, const ConvGemmPlan& g, uint32_t groups, const ConvTabEntry* rt, const ConvTabEntry* st,
+	const float* img, const float* Bmat, int64_t ldb, float* partial)
+{
+	int64_t safe = 0;
+	for (int d = 0; d < 8; ++d) { safe += (int64_t) g.ilo[d] * g.istr[d]; }
+	switch (g.Np / 16)
+	{
+		case 1: conv_fewrows_k<RB,1><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, rt, st, img, Bmat, ldb, partial, safe); break;
+		case 2: conv_fewrows_k<RB,2><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, rt, st, img, Bmat, ldb, partial, safe); break;
+		case 3: conv_fewrows_k<RB,3><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, rt, st, img, Bmat, ldb, partial, safe); break;
+		default: conv_fewrows_k<RB,4><<<groups, CG_BLOCK, 0, ctx->stream>>>(g, rt, st, img, Bmat, ldb, partial, safe); break;
+	}
+}
+
 // out[window coordinate of (m, n)] = C[m - m0][n]
 template <typename T>
 __global__ __launch_bounds__(CG_BLOCK) void conv_scatter_k (ConvGemmPlan p, uint32_t m0, uint32_t rows,
@@ -1199,6 +1337,35 @@ int conv_gemm_run (tcg_ctx* ctx, int dtype, const ConvGemmPlan& g, const T* img,
 						default: conv_short_launch<8>(ctx, g, m0, rows, rt, st, img, kb, (const float*) Bmat, (int64_t) ldb, (float*) Cmat, (int64_t) ldc); break;
 					}
 					++ctx->conv_short_launches;
+					if (false == direct_c)
+					{
+						grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);
+						conv_scatter_k<T><<<grid, CG_BLOCK, 0, ctx->stream>>>(g, m0, rows, (const T*) C, out);
+					}
+					continue;
+				}
+			}
+			if constexpr (std::is_same<T,float>::value)
+			{
+				// few rows under a very long summed index: gathered and multiplied stretch by stretch, then summed
+				const char* few_env = getenv("TCG_CONV_FEWROWS"); // "0": gather and multiply (for tests)
+				if (tables && rows == g.M && g.M <= (uint32_t) CF_MAX_M && g.Np <= (uint32_t) CS_MAX_N && g.Np % 16 == 0 &&
+					g.S >= 4096 && false == gather_b && !(few_env && few_env[0] == '0'))
+				{
+					const uint32_t groups = (g.S + CF_STRETCH - 1) / CF_STRETCH;
+					const size_t partial_bytes = sizeof(float) * (size_t) groups * g.M * g.Np;
+					void* partial = nullptr;
+					rc = tcg_alloc(ctx, partial_bytes, &partial);
+					if (rc != TCG_OK) { break; }
+					const ConvTabEntry* rt = (const ConvTabEntry*) RT;
+					const ConvTabEntry* st = (const ConvTabEntry*) ST;
+					if (g.M <= 16) { conv_fewrows_launch<1>(ctx, g, groups, rt, st, img, (const float*) Bmat, (int64_t) ldb, (float*) partial); }
+					else { conv_fewrows_launch<2>(ctx, g, groups, rt, st, img, (const float*) Bmat, (int64_t) ldb, (float*) partial); }
+					const uint32_t results = g.M * g.Np;
+					conv_ranges_sum_k<<<(results + CG_BLOCK / 64 - 1) / (CG_BLOCK / 64), CG_BLOCK, 0, ctx->stream>>>((const float*) partial, groups,
+						g.M, g.Np, (float*) Cmat, (int64_t) ldc);
+					tcg_free(ctx, partial, partial_bytes);
+					++ctx->conv_fewrows_launches;
 					if (false == direct_c)
 					{
 						grid = tcg_grid(ctx, (uint64_t) rows * g.N, CG_BLOCK, 16);

@@ -361,10 +361,11 @@ int tcg_conv_patch_f32 (tcg_ctx* ctx, uint64_t M, uint64_t N, uint64_t S, const 
 	return TCG_OK;
 }
 
-extern "C" int tcg_conv_route_counts (const tcg_ctx* ctx, uint64_t* patch, uint64_t* short_sum)
+extern "C" int tcg_conv_route_counts (const tcg_ctx* ctx, uint64_t* patch, uint64_t* short_sum, uint64_t* few_rows)
 {
-	if (!ctx || !patch || !short_sum) { return TCG_ERR_ARG; }
+	if (!ctx || !patch || !short_sum || !few_rows) { return TCG_ERR_ARG; }
 	*patch = ctx->conv_patch_launches;
 	*short_sum = ctx->conv_short_launches;
+	*few_rows = ctx->conv_fewrows_launches;
 	return TCG_OK;
 }

@@ -85,6 +85,7 @@ struct tcg_ctx
 	size_t conv_table_bytes = 0;
 	uint64_t conv_patch_launches = 0; // products that read the image out of a patch in LDS (conv_patch.hip)
 	uint64_t conv_short_launches = 0; // convolutions with a short summed index done in one launch (conv.hip)
+	uint64_t conv_fewrows_launches = 0; // convolutions with few rows under a long summed index, gathered while multiplied (conv.hip)
 	// tables first met while launches are being recorded are filled at once on
 	// this stream, so that the recording does not fill them again at every replay
 	hipStream_t side_stream = nullptr;

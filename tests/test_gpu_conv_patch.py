@@ -8,7 +8,8 @@ oracle) at 1e-4, and against the product that reads the image through its
 tables (TCG_CONV_PATCH=0) -- the two products sum in different orders.  The
 counter of the route says which one ran; shapes the route does not take (a
 summed index that is no multiple of 32) must leave it alone.  Also here: the
-one-launch route for a short summed index (the CNN's first layer).
+one-launch route for a short summed index (the CNN's first layer) and the
+route for few rows under a long summed index (that layer's kernel gradient).
 """
 import os
 
@@ -150,3 +151,21 @@ def test_seeded_layers_on_the_patch_route(ctx, oracle, seed):
     got = run_views(ctx, oracle, which, dims, {})
     assert ctx.conv_route_counts()["patch"] == before + 1, "the route under test was not taken: %r" % (dims,)
     assert_acc_close(got, run_views(ctx, oracle, which, dims, {"TCG_CONV_GEMM": "0"}), ACC_RTOL)
+
+
+@pytest.mark.parametrize("dims", [dict(C=1, W=28, H=28, B=32, O=32, KW=5, KH=5), dict(C=2, W=17, H=23, B=40, O=64, KW=4, KH=3),
+                                  dict(C=1, W=20, H=21, B=90, O=16, KW=3, KH=3)],
+                         ids=["cnn_first_layer", "two_channels_64_filters", "nine_rows_16_filters"])
+def test_few_rows_under_a_long_summed_index_equal_the_direct_kernels(ctx, oracle, dims):
+    """The kernel gradient of the reference's first CNN layer (25 x 32 results, each a sum over every pixel of the batch):
+    A gathered while it is multiplied, stretches of the summed index added up by a second launch, against the direct
+    kernels and against gather + product."""
+    before = ctx.conv_route_counts()["few_rows"]
+    got = run_views(ctx, oracle, "kernel_gradient", dims, {})
+    assert ctx.conv_route_counts()["few_rows"] == before + 1, "the route under test was not taken"
+    two = run_views(ctx, oracle, "kernel_gradient", dims, {"TCG_CONV_FEWROWS": "0"})
+    assert ctx.conv_route_counts()["few_rows"] == before + 1
+    direct = run_views(ctx, oracle, "kernel_gradient", dims, {"TCG_CONV_GEMM": "0"})
+    assert_acc_close(got, direct, ACC_RTOL)
+    assert_acc_close(got, two, ACC_RTOL)
+    np.testing.assert_array_equal(run_views(ctx, oracle, "kernel_gradient", dims, {}), got)
