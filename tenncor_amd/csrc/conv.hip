@@ -532,28 +532,37 @@ __global__ __launch_bounds__(CG_BLOCK) void conv_short_k (ConvGemmPlan p, uint32
 	uint32_t ext[4];
 #pragma unroll
 	for (int j = 0; j < 4; ++j) { ext[j] = j < p.ncheck ? p.check_ext[j] : 0xffffffffu; }
-	// this lane's summed indices 4 j + q and its share of B
+	// this lane's summed indices 4 j + q and its share of B: every offset first, then
+	// every element (no load waits for another of its kind)
 	ConvTabEntry col[SP4];
 	float b[SP4][CB];
-	const int64_t* ktab = (const int64_t*) (sumtab + p.Sp);
-#pragma unroll
-	for (int j = 0; j < SP4; ++j)
 	{
-		const uint32_t s = 4 * j + q;
-		col[j] = sumtab[s];
-		const int64_t ks = ker ? ktab[s] : 0;
+		const int64_t* ktab = (const int64_t*) (sumtab + p.Sp);
+		const float* from = ker ? ker : Bmat;
+		int64_t ks[SP4], kn[CB];
+#pragma unroll
+		for (int j = 0; j < SP4; ++j)
+		{
+			const uint32_t s = 4 * j + q;
+			col[j] = sumtab[s];
+			ks[j] = ker ? ktab[s] : (int64_t) s * ldb;
+		}
 #pragma unroll
 		for (int cb = 0; cb < CB; ++cb)
 		{
 			const uint32_t n = 16 * cb + r16;
-			if (ker)
+			kn[cb] = ker ? ktab[p.Sp + n] : (int64_t) n;
+		}
+#pragma unroll
+		for (int j = 0; j < SP4; ++j)
+		{
+#pragma unroll
+			for (int cb = 0; cb < CB; ++cb)
 			{
-				const int64_t kn = ktab[p.Sp + n];
-				const bool there = ks != CONV_NO_KERNEL && kn != CONV_NO_KERNEL;
-				const float v = ker[there ? ks + kn : 0];
+				const bool there = nullptr == ker || (ks[j] != CONV_NO_KERNEL && kn[cb] != CONV_NO_KERNEL);
+				const float v = from[there ? ks[j] + kn[cb] : 0];
 				b[j][cb] = there ? v : 0.f;
 			}
-			else { b[j][cb] = Bmat[(int64_t) s * ldb + n]; }
 		}
 	}
 	conv_f4 acc[CS_RB][CB];
