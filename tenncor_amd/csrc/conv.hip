@@ -1092,22 +1092,15 @@ tcg_conv_patch conv_patch_prepare (const tcg_ctx* ctx, const ConvGemmPlan& g, co
 	}
 	if (smin < -limit || smax > limit) { return none; }
 	// neighbouring rows a power of two apart: padding behind every such stretch keeps
-	// the sixteen rows of a matrix instruction in different banks.  Only when every row
-	// lies a whole number of such distances from every other: the kernel adds the padded
-	// row part and the padded summed part of an address instead of padding their sum.
+	// the sixteen rows of a matrix instruction in different banks
 	uint32_t pad_shift = 31;
 	if (g.M > 1)
 	{
 		const int64_t step = rowoff[1] > rowoff[0] ? rowoff[1] - rowoff[0] : rowoff[0] - rowoff[1];
 		if (step >= 16 && step <= 4096 && (step & (step - 1)) == 0)
 		{
-			bool whole = true;
-			for (uint32_t m = 1; m < g.M && whole; ++m) { whole = ((rowoff[m] - rowoff[0]) & (step - 1)) == 0; }
-			if (whole)
-			{
-				pad_shift = 0;
-				while (((int64_t) 1 << pad_shift) < step) { ++pad_shift; }
-			}
+			pad_shift = 0;
+			while (((int64_t) 1 << pad_shift) < step) { ++pad_shift; }
 		}
 	}
 	double best = 0;

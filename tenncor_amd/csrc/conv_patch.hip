@@ -115,8 +115,7 @@ __global__ __launch_bounds__(64 * NW) void conv_patch_k (PatchArgs a)
 	for (uint32_t f = (uint32_t) tid; f < S4; f += NT)
 	{
 		const tcg_conv_tab e = a.sums[4 * f];
-		// (where the summed index's part of the address lies behind the least one, padding included)
-		stab[f] = padded((int) e.off - a.smin, a.pad_shift);
+		stab[f] = (int) e.off;
 #pragma unroll
 		for (int k = 0; k < NCHECK; ++k) { stab[(k + 1) * S4 + f] = e.c[k]; }
 	}
@@ -133,15 +132,8 @@ __global__ __launch_bounds__(64 * NW) void conv_patch_k (PatchArgs a)
 			*(f4*) (patch + padded(p - lo, a.pad_shift)) = v;
 		}
 	}
-	// The row's part of an address, padding included: the rows of a tile lie whole
-	// multiples of the padded distance behind the first (the host has seen to that, or
-	// set the distance so large that nothing is padded), so the padded position of
-	// row part + summed part is the sum of the two padded parts
 #pragma unroll
-	for (int rb = 0; rb < RBT; ++rb) { rbase[rb] = padded(rbase[rb] - range[0], a.pad_shift); }
-	// the last four floats of the patch's room are never part of the stretch
-	const int zeros_at = (int) a.patch_floats - 4;
-	if (tid == 0) { *(f4*) (patch + zeros_at) = f4{0.f, 0.f, 0.f, 0.f}; }
+	for (int rb = 0; rb < RBT; ++rb) { rbase[rb] -= lo; }
 	__syncthreads();
 	f4 acc[RBT][CBT];
 #pragma unroll
@@ -170,10 +162,8 @@ __global__ __launch_bounds__(64 * NW) void conv_patch_k (PatchArgs a)
 			bool ok = rok[rb];
 #pragma unroll
 			for (int k = 0; k < NCHECK; ++k) { ok = ok & ((uint32_t) (rc[rb][k] + sc[k]) < a.check_ext[k]); }
-			// (an element of the zero border is read from four zeros behind the patch: one
-			// select on the address instead of four on the values)
-			const int at = rbase[rb] + so;
-			av[rb] = *(const f4*) (patch + (NCHECK == 0 || ok ? at : zeros_at));
+			const f4 v = *(const f4*) (patch + padded(rbase[rb] + so, a.pad_shift));
+			av[rb] = ok ? v : f4{0.f, 0.f, 0.f, 0.f};
 		}
 	};
 	// (Leaving out the sixteen-row blocks that lie wholly in the zero border for a step --
